@@ -1,0 +1,422 @@
+"""Python plumbing over libffk.so, the gfx950 operator-kernel library.
+
+This module only loads the C-ABI library (``include/ffk.h``) with ctypes and
+offers thin helpers that pass ``torch`` tensors' device pointers and the
+current HIP stream to it.  PyTorch is used for device memory and streams only;
+no arithmetic here is done by torch.  If ``libffk.so`` is missing the import of
+any entry point fails loudly -- there is no fallback path.
+
+The directory name contains a hyphen, so load it with
+``importlib.util.spec_from_file_location('flexflow_train_amd', .../__init__.py)``
+(see ``tests/conftest.py``).
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libffk.so")
+
+c_int = ctypes.c_int
+c_i64 = ctypes.c_int64
+c_u64 = ctypes.c_uint64
+c_f = ctypes.c_float
+c_p = ctypes.c_void_p
+c_sz = ctypes.c_size_t
+
+# DataType ordinals of include/ffk.h
+BOOL, INT32, INT64, HALF, FLOAT, DOUBLE, BF16 = range(7)
+ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH, ACT_GELU = -1, 0, 1, 2, 3
+AGGR_NONE, AGGR_SUM, AGGR_AVG = -1, 0, 1
+OP = dict(
+    SCALAR_MULTIPLY=8, SCALAR_ADD=9, SCALAR_TRUE_DIV=11, SCALAR_SUB=12, RELU=13,
+    IDENTITY=14, SIGMOID=15, TANH=16, ELU=17, EW_ADD=28, EW_MUL=29, EW_SUB=35,
+    EW_DIV=36, EW_MAX=40, EW_MIN=41, EXP=56, SIN=61, COS=62, GELU=67, RSQRT=70,
+    POW=71, GELU_REFERENCE_GRAD=1067,
+)
+
+
+class FFKError(RuntimeError):
+    """A non-zero status from the C ABI (the reference aborts in its place)."""
+
+
+class AttentionDesc(ctypes.Structure):
+    _fields_ = [
+        ("batch", c_i64), ("heads", c_i64), ("seq_q", c_i64), ("seq_kv", c_i64),
+        ("head_dim", c_i64),
+        ("q_batch_stride", c_i64), ("q_seq_stride", c_i64),
+        ("k_batch_stride", c_i64), ("k_seq_stride", c_i64),
+        ("v_batch_stride", c_i64), ("v_seq_stride", c_i64),
+        ("o_batch_stride", c_i64), ("o_seq_stride", c_i64),
+        ("scale", c_f), ("causal", c_int),
+    ]
+
+
+class MHADesc(ctypes.Structure):
+    _fields_ = [
+        ("num_samples", c_i64), ("num_heads", c_i64),
+        ("q_size", c_i64), ("k_size", c_i64), ("v_size", c_i64),
+        ("q_proj_size", c_i64), ("k_proj_size", c_i64), ("v_proj_size", c_i64),
+        ("o_proj_size", c_i64),
+        ("qo_seq_length", c_i64), ("kv_seq_length", c_i64),
+        ("scale", c_f), ("causal", c_int),
+    ]
+
+
+# name -> (restype, argtypes); must list every symbol include/ffk.h declares.
+SIGNATURES = {
+    "ffk_last_error": (ctypes.c_char_p, []),
+    "ffk_device_count": (c_int, [ctypes.POINTER(c_int)]),
+    "ffk_set_device": (c_int, [c_int]),
+    "ffk_malloc": (c_int, [ctypes.POINTER(c_p), c_sz]),
+    "ffk_free": (c_int, [c_p]),
+    "ffk_host_malloc": (c_int, [ctypes.POINTER(c_p), c_sz]),
+    "ffk_host_free": (c_int, [c_p]),
+    "ffk_memcpy": (c_int, [c_p, c_p, c_sz, c_int, c_p]),
+    "ffk_fill_zero": (c_int, [c_p, c_sz, c_p]),
+    "ffk_stream_create": (c_int, [ctypes.POINTER(c_p)]),
+    "ffk_stream_destroy": (c_int, [c_p]),
+    "ffk_stream_synchronize": (c_int, [c_p]),
+    "ffk_event_create": (c_int, [ctypes.POINTER(c_p)]),
+    "ffk_event_destroy": (c_int, [c_p]),
+    "ffk_event_record": (c_int, [c_p, c_p]),
+    "ffk_event_synchronize": (c_int, [c_p]),
+    "ffk_event_elapsed_ms": (c_int, [c_p, c_p, ctypes.POINTER(c_f)]),
+    "ffk_linear_forward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_p, c_i64, c_i64, c_i64]),
+    "ffk_linear_backward_workspace_bytes": (c_sz, [c_int, c_int, c_int, c_i64, c_i64]),
+    "ffk_linear_backward": (c_int, [c_p, c_int, c_int, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
+                                    c_i64, c_i64, c_i64, c_p, c_sz, c_int]),
+    "ffk_gemm": (c_int, [c_p, c_int, c_int, c_int, c_i64, c_i64, c_i64, c_p, c_p, c_p, c_int]),
+    "ffk_element_unary_forward": (c_int, [c_p, c_int, c_int, c_f, c_p, c_p, c_i64]),
+    "ffk_element_unary_backward": (c_int, [c_p, c_int, c_int, c_f, c_p, c_p, c_p, c_p, c_i64,
+                                           c_int]),
+    "ffk_element_binary_forward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_i64, c_i64,
+                                           c_i64]),
+    "ffk_element_binary_backward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_p, c_p, c_i64,
+                                            c_int]),
+    "ffk_layer_norm_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_i64, c_i64,
+                                       c_f]),
+    "ffk_layer_norm_backward_workspace_bytes": (c_sz, [c_i64, c_i64]),
+    "ffk_layer_norm_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
+                                        c_i64, c_i64, c_p, c_sz, c_int]),
+    "ffk_softmax_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_i64, c_i64]),
+    "ffk_softmax_backward_copy": (c_int, [c_p, c_int, c_p, c_p, c_sz]),
+    "ffk_softmax_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_i64, c_i64]),
+    "ffk_dropout_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
+    "ffk_dropout_backward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64, c_int]),
+    "ffk_dropout_mask": (c_int, [c_p, c_p, c_i64, c_f, c_u64, c_u64]),
+    "ffk_embedding_forward": (c_int, [c_p, c_int, c_int, c_int, c_p, c_p, c_p, c_int, c_i64,
+                                      c_i64, c_i64, c_i64]),
+    "ffk_embedding_backward_workspace_bytes": (c_sz, [c_i64, c_i64]),
+    "ffk_embedding_backward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_int, c_i64, c_i64,
+                                       c_i64, c_i64, c_int, c_p, c_sz]),
+    "ffk_attention_forward": (c_int, [c_p, c_int, ctypes.POINTER(AttentionDesc), c_p, c_p, c_p,
+                                      c_p, c_p]),
+    "ffk_attention_backward": (c_int, [c_p, c_int, ctypes.POINTER(AttentionDesc), c_p, c_p, c_p,
+                                       c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
+    "ffk_mha_weight_elements": (c_sz, [ctypes.POINTER(MHADesc)]),
+    "ffk_mha_reserve_bytes": (c_sz, [ctypes.POINTER(MHADesc), c_int]),
+    "ffk_mha_forward": (c_int, [c_p, c_int, ctypes.POINTER(MHADesc), c_p, c_p, c_p, c_p, c_p,
+                                c_p, c_sz]),
+    "ffk_mha_backward": (c_int, [c_p, c_int, ctypes.POINTER(MHADesc), c_p, c_p, c_p, c_p, c_p,
+                                 c_p, c_p, c_p, c_p, c_p, c_sz, c_int]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded libffk.so with argtypes set; raises if it was never built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FFKError(
+                "libffk.so is missing at %s: build it with "
+                "`python flexflow-train_amd/build.py` (there is no fallback path)" % LIB_PATH
+            )
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise FFKError("ffk error %d: %s" % (rc, lib().ffk_last_error().decode()))
+
+
+# --------------------------------------------------------------------------
+# torch-tensor helpers
+# --------------------------------------------------------------------------
+
+def _torch():
+    import torch
+    return torch
+
+
+def dtype_of(t):
+    torch = _torch()
+    table = {torch.float32: FLOAT, torch.bfloat16: BF16, torch.int32: INT32,
+             torch.int64: INT64, torch.float16: HALF, torch.float64: DOUBLE,
+             torch.bool: BOOL}
+    return table[t.dtype]
+
+
+def ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensor required"
+    return t.data_ptr()
+
+
+def current_stream():
+    return _torch().cuda.current_stream().cuda_stream
+
+
+def linear_forward(x, w, b=None, activation=ACT_NONE, out=None):
+    torch = _torch()
+    batch, in_dim = x.shape
+    out_dim = w.shape[0]
+    if out is None:
+        out = torch.empty((batch, out_dim), dtype=x.dtype, device=x.device)
+    check(lib().ffk_linear_forward(current_stream(), dtype_of(x), activation, ptr(x), ptr(out),
+                                   ptr(w), ptr(b), batch, in_dim, out_dim))
+    return out
+
+
+def linear_backward(y, dy, x, w, dx=None, dw=None, db=None, activation=ACT_NONE,
+                    relu_grad_mode=0, accumulate=False, workspace=None):
+    torch = _torch()
+    batch, in_dim = x.shape
+    out_dim = w.shape[0]
+    if workspace is None:
+        need = lib().ffk_linear_backward_workspace_bytes(dtype_of(x), activation,
+                                                         int(db is not None), batch, out_dim)
+        if need:
+            workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(lib().ffk_linear_backward(current_stream(), dtype_of(x), activation, relu_grad_mode,
+                                    ptr(y), ptr(dy), ptr(x), ptr(dx), ptr(w), ptr(dw), ptr(db),
+                                    batch, in_dim, out_dim, ptr(workspace), ws_bytes,
+                                    int(accumulate)))
+    return dx, dw, db
+
+
+def gemm(A, B, C, trans_a=False, trans_b=False, accumulate=False):
+    M, N = C.shape
+    K = A.shape[0] if trans_a else A.shape[1]
+    check(lib().ffk_gemm(current_stream(), dtype_of(A), int(trans_a), int(trans_b), M, N, K,
+                         ptr(A), ptr(B), ptr(C), int(accumulate)))
+    return C
+
+
+def element_unary_forward(op, x, scalar=0.0, out=None):
+    torch = _torch()
+    if out is None:
+        out = torch.empty_like(x)
+    check(lib().ffk_element_unary_forward(current_stream(), dtype_of(x), op, scalar, ptr(x),
+                                          ptr(out), x.numel()))
+    return out
+
+
+def element_unary_backward(op, y, dy, x, dx, scalar=0.0, accumulate=-1):
+    check(lib().ffk_element_unary_backward(current_stream(), dtype_of(x), op, scalar, ptr(y),
+                                           ptr(dy), ptr(x), ptr(dx), x.numel(), accumulate))
+    return dx
+
+
+def element_binary_forward(op, l, r, out=None):
+    torch = _torch()
+    if out is None:
+        out = torch.empty_like(l if l.numel() >= r.numel() else r)
+    check(lib().ffk_element_binary_forward(current_stream(), dtype_of(out), op, ptr(l), ptr(r),
+                                           ptr(out), out.numel(), l.numel(), r.numel()))
+    return out
+
+
+def element_binary_backward(op, g, l, r, dl, dr, accumulate=False):
+    check(lib().ffk_element_binary_backward(current_stream(), dtype_of(g), op, ptr(g), ptr(l),
+                                            ptr(r), ptr(dl), ptr(dr), g.numel(),
+                                            int(accumulate)))
+    return dl, dr
+
+
+def layer_norm_forward(x, gamma, beta, eps, out=None, mean=None, rstd=None):
+    torch = _torch()
+    M, N = x.shape
+    if out is None:
+        out = torch.empty_like(x)
+    if mean is None:
+        mean = torch.empty((M,), dtype=torch.float32, device=x.device)
+    if rstd is None:
+        rstd = torch.empty((M,), dtype=torch.float32, device=x.device)
+    check(lib().ffk_layer_norm_forward(current_stream(), dtype_of(x), ptr(x), ptr(out),
+                                       ptr(gamma), ptr(beta), ptr(mean), ptr(rstd), M, N, eps))
+    return out, mean, rstd
+
+
+def layer_norm_backward(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, accumulate=False,
+                        workspace=None):
+    torch = _torch()
+    M, N = x.shape
+    need = lib().ffk_layer_norm_backward_workspace_bytes(M, N)
+    if workspace is None:
+        workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)
+    check(lib().ffk_layer_norm_backward(current_stream(), dtype_of(x), ptr(dy), ptr(x),
+                                        ptr(mean), ptr(rstd), ptr(gamma), ptr(dx), ptr(dgamma),
+                                        ptr(dbeta), M, N, ptr(workspace), workspace.numel(),
+                                        int(accumulate)))
+    return dx, dgamma, dbeta
+
+
+def softmax_forward(x, outer, dim, inner, out=None):
+    torch = _torch()
+    if out is None:
+        out = torch.empty_like(x)
+    check(lib().ffk_softmax_forward(current_stream(), dtype_of(x), ptr(x), ptr(out), outer, dim,
+                                    inner))
+    return out
+
+
+def softmax_backward(y, dy, outer, dim, inner, dx=None):
+    torch = _torch()
+    if dx is None:
+        dx = torch.empty_like(y)
+    check(lib().ffk_softmax_backward(current_stream(), dtype_of(y), ptr(y), ptr(dy), ptr(dx),
+                                     outer, dim, inner))
+    return dx
+
+
+def softmax_backward_copy(dy, dx=None):
+    torch = _torch()
+    if dx is None:
+        dx = torch.empty_like(dy)
+    check(lib().ffk_softmax_backward_copy(current_stream(), dtype_of(dy), ptr(dy), ptr(dx),
+                                          dy.numel()))
+    return dx
+
+
+def dropout_forward(x, rate, seed, offset=0, out=None):
+    torch = _torch()
+    if out is None:
+        out = torch.empty_like(x)
+    check(lib().ffk_dropout_forward(current_stream(), dtype_of(x), ptr(x), ptr(out), x.numel(),
+                                    rate, seed, offset))
+    return out
+
+
+def dropout_backward(dy, rate, seed, offset=0, dx=None, accumulate=False):
+    torch = _torch()
+    if dx is None:
+        dx = torch.empty_like(dy)
+    check(lib().ffk_dropout_backward(current_stream(), dtype_of(dy), ptr(dy), ptr(dx),
+                                     dy.numel(), rate, seed, offset, int(accumulate)))
+    return dx
+
+
+def dropout_mask(n, rate, seed, offset=0, device="cuda"):
+    torch = _torch()
+    m = torch.empty((n,), dtype=torch.uint8, device=device)
+    check(lib().ffk_dropout_mask(current_stream(), ptr(m), n, rate, seed, offset))
+    return m
+
+
+def embedding_forward(indices, weight, aggr=AGGR_NONE, out_dtype=None):
+    torch = _torch()
+    V, D = weight.shape
+    if aggr == AGGR_NONE:
+        num_bags, bag = indices.numel(), 1
+    else:
+        bag = indices.shape[-1]
+        num_bags = indices.numel() // bag
+    out_dtype = out_dtype or weight.dtype
+    out = torch.empty((num_bags, D), dtype=out_dtype, device=weight.device)
+    check(lib().ffk_embedding_forward(current_stream(), dtype_of(indices), dtype_of(weight),
+                                      dtype_of(out), ptr(indices), ptr(out), ptr(weight), aggr,
+                                      num_bags, bag, D, V))
+    return out
+
+
+def embedding_backward(indices, out_grad, weight_grad, aggr=AGGR_NONE, deterministic=False):
+    torch = _torch()
+    V, D = weight_grad.shape
+    if aggr == AGGR_NONE:
+        num_bags, bag = indices.numel(), 1
+    else:
+        bag = indices.shape[-1]
+        num_bags = indices.numel() // bag
+    ws = None
+    ws_bytes = 0
+    if deterministic:
+        ws_bytes = lib().ffk_embedding_backward_workspace_bytes(num_bags * bag, V)
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=weight_grad.device)
+    check(lib().ffk_embedding_backward(current_stream(), dtype_of(indices), dtype_of(out_grad),
+                                       ptr(indices), ptr(out_grad), ptr(weight_grad), aggr,
+                                       num_bags, bag, D, V, int(deterministic), ptr(ws),
+                                       ws_bytes))
+    return weight_grad
+
+
+def attention_desc_bshd(q, k, scale, causal):
+    """Descriptor for dense [B, S, H, D] tensors."""
+    B, Sq, H, D = q.shape
+    Skv = k.shape[1]
+    return AttentionDesc(B, H, Sq, Skv, D, Sq * H * D, H * D, Skv * H * D, H * D,
+                         Skv * H * D, H * D, Sq * H * D, H * D, scale, int(causal))
+
+
+def attention_forward(q, k, v, scale, causal, desc=None):
+    torch = _torch()
+    desc = desc or attention_desc_bshd(q, k, scale, causal)
+    o = torch.empty_like(q)
+    lse = torch.empty((desc.batch, desc.heads, desc.seq_q), dtype=torch.float32, device=q.device)
+    check(lib().ffk_attention_forward(current_stream(), dtype_of(q), ctypes.byref(desc), ptr(q),
+                                      ptr(k), ptr(v), ptr(o), ptr(lse)))
+    return o, lse
+
+
+def attention_backward(q, k, v, o, d_o, lse, scale, causal, desc=None):
+    torch = _torch()
+    desc = desc or attention_desc_bshd(q, k, scale, causal)
+    dq = torch.empty_like(q)
+    dk = torch.empty_like(k)
+    dv = torch.empty_like(v)
+    delta = torch.empty_like(lse)
+    check(lib().ffk_attention_backward(current_stream(), dtype_of(q), ctypes.byref(desc), ptr(q),
+                                       ptr(k), ptr(v), ptr(o), ptr(d_o), ptr(lse), ptr(delta),
+                                       ptr(dq), ptr(dk), ptr(dv)))
+    return dq, dk, dv
+
+
+def mha_desc(num_samples, num_heads, q_size, k_size, v_size, q_proj, k_proj, v_proj, o_proj,
+             sq, skv, scale=1.0, causal=False):
+    return MHADesc(num_samples, num_heads, q_size, k_size, v_size, q_proj, k_proj, v_proj, o_proj,
+                   sq, skv, scale, int(causal))
+
+
+def mha_reserve(desc, dtype, device="cuda"):
+    torch = _torch()
+    n = lib().ffk_mha_reserve_bytes(ctypes.byref(desc), dtype)
+    return torch.empty((n,), dtype=torch.uint8, device=device)
+
+
+def mha_forward(desc, query, key, value, weight, reserve, out=None):
+    torch = _torch()
+    if out is None:
+        out = torch.empty((desc.num_samples, desc.qo_seq_length, desc.o_proj_size),
+                          dtype=query.dtype, device=query.device)
+    check(lib().ffk_mha_forward(current_stream(), dtype_of(query), ctypes.byref(desc), ptr(query),
+                                ptr(key), ptr(value), ptr(weight), ptr(out), ptr(reserve),
+                                reserve.numel()))
+    return out
+
+
+def mha_backward(desc, query, dquery, key, dkey, value, dvalue, weight, dweight, out_grad,
+                 reserve, accumulate=False):
+    check(lib().ffk_mha_backward(current_stream(), dtype_of(query), ctypes.byref(desc),
+                                 ptr(query), ptr(dquery), ptr(key), ptr(dkey), ptr(value),
+                                 ptr(dvalue), ptr(weight), ptr(dweight), ptr(out_grad),
+                                 ptr(reserve), reserve.numel(), int(accumulate)))
+    return dquery, dkey, dvalue, dweight

@@ -1,0 +1,206 @@
+// Dropout forward/backward for gfx950 with a counter-based mask.
+//
+// The reference delegates to cudnnDropoutForward/Backward, whose generator
+// state and reserve space are opaque (lib/kernels/src/cuda/ops/
+// dropout_kernels.cu:24-95).  Here the keep mask is a pure function of
+// (seed, element index): Philox4x32-10, key = (seed lo, seed hi), counter =
+// (block lo, block hi, 0, 0) with block = (offset + i) / 4, and element
+// (offset + i) uses word (offset + i) % 4; it is kept iff
+// word >= ceil(rate * 2^32).  Nothing is stored between forward and backward:
+// backward regenerates the mask, so both directions move 2 tensors only.
+#include "ffk_common.h"
+#include <math.h>
+
+namespace ffk {
+
+struct PhiloxKey {
+  uint32_t k0, k1;
+};
+
+__device__ __forceinline__ void philox4x32_10(uint64_t block, PhiloxKey key,
+                                              uint32_t (&out)[4]) {
+  uint32_t c0 = (uint32_t)block, c1 = (uint32_t)(block >> 32), c2 = 0u, c3 = 0u;
+  uint32_t k0 = key.k0, k1 = key.k1;
+#pragma unroll
+  for (int r = 0; r < 10; r++) {
+    uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    uint32_t n1 = (uint32_t)p1;
+    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+struct DropoutParams {
+  PhiloxKey key;
+  uint64_t offset;
+  uint32_t threshold;  // keep iff word >= threshold ...
+  int drop_all;        // ... unless rate rounds to 2^32 (everything dropped)
+  float scale;         // 1 / (1 - rate)
+};
+
+__device__ __forceinline__ bool keep(uint32_t word, DropoutParams const &p) {
+  return !p.drop_all && word >= p.threshold;
+}
+
+constexpr int kDropThreads = 256;
+
+// offset % 4 == 0, 16-byte aligned pointers: each lane owns whole Philox blocks.
+template <typename T, bool ACC>
+__global__ __launch_bounds__(kDropThreads) void dropout_vec_kernel(
+    T const *__restrict__ X, T *Y, int64_t n, DropoutParams p) {
+  constexpr int V = VecIO<T>::kVec;
+  int64_t const nvec = n / V;
+  int64_t const stride = (int64_t)gridDim.x * kDropThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kDropThreads + threadIdx.x; i < nvec; i += stride) {
+    float x[V], y[V];
+    VecIO<T>::load(X + i * V, x);
+    if (ACC) VecIO<T>::load(Y + i * V, y);
+    uint64_t const blk0 = (p.offset + (uint64_t)i * V) >> 2;
+#pragma unroll
+    for (int b = 0; b < V / 4; b++) {
+      uint32_t w[4];
+      philox4x32_10(blk0 + b, p.key, w);
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        float v = keep(w[e], p) ? x[4 * b + e] * p.scale : 0.0f;
+        y[4 * b + e] = ACC ? y[4 * b + e] + v : v;
+      }
+    }
+    VecIO<T>::store(Y + i * V, y);
+  }
+}
+
+// Any offset / alignment / tail: one element per thread.
+template <typename T, bool ACC>
+__global__ __launch_bounds__(kDropThreads) void dropout_scalar_kernel(
+    T const *__restrict__ X, T *Y, int64_t first, int64_t n, DropoutParams p) {
+  int64_t const stride = (int64_t)gridDim.x * kDropThreads;
+  for (int64_t i = first + (int64_t)blockIdx.x * kDropThreads + threadIdx.x; i < n; i += stride) {
+    uint64_t const e = p.offset + (uint64_t)i;
+    uint32_t w[4];
+    philox4x32_10(e >> 2, p.key, w);
+    uint32_t word = w[0];
+    if ((e & 3) == 1) word = w[1];
+    if ((e & 3) == 2) word = w[2];
+    if ((e & 3) == 3) word = w[3];
+    float v = keep(word, p) ? VecIO<T>::load1(X + i) * p.scale : 0.0f;
+    if (ACC) v += VecIO<T>::load1(Y + i);
+    VecIO<T>::store1(Y + i, v);
+  }
+}
+
+__global__ __launch_bounds__(kDropThreads) void dropout_mask_kernel(
+    uint8_t *mask, int64_t n, DropoutParams p) {
+  int64_t const stride = (int64_t)gridDim.x * kDropThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kDropThreads + threadIdx.x; i < n; i += stride) {
+    uint64_t const e = p.offset + (uint64_t)i;
+    uint32_t w[4];
+    philox4x32_10(e >> 2, p.key, w);
+    uint32_t word = w[0];
+    if ((e & 3) == 1) word = w[1];
+    if ((e & 3) == 2) word = w[2];
+    if ((e & 3) == 3) word = w[3];
+    mask[i] = keep(word, p) ? 1 : 0;
+  }
+}
+
+static int make_params(char const *who, float rate, uint64_t seed,
+                       uint64_t offset, DropoutParams &p) {
+  FFK_REQUIRE(rate >= 0.0f && rate <= 1.0f, "%s: rate %f outside [0, 1]", who, (double)rate);
+  double t = ceil((double)rate * 4294967296.0);
+  p.drop_all = t >= 4294967296.0;
+  p.threshold = p.drop_all ? 0xffffffffu : (uint32_t)t;
+  p.key.k0 = (uint32_t)seed;
+  p.key.k1 = (uint32_t)(seed >> 32);
+  p.offset = offset;
+  p.scale = 1.0f / (1.0f - rate);
+  return FFK_OK;
+}
+
+static int grid_for(int64_t items) {
+  int64_t b = ceil_div(items > 0 ? items : 1, kDropThreads);
+  int64_t const cap = (int64_t)kNumCU * 16;
+  return (int)(b < cap ? b : cap);
+}
+
+template <typename T, bool ACC>
+static int dropout_run(hipStream_t st, void const *x, void *y, int64_t n,
+                       DropoutParams const &p) {
+  constexpr int V = VecIO<T>::kVec;
+  T const *X = static_cast<T const *>(x);
+  T *Y = static_cast<T *>(y);
+  int64_t done = 0;
+  if ((p.offset & 3) == 0 && aligned16(x) && aligned16(y) && n >= V) {
+    int64_t nvec = n / V;
+    dropout_vec_kernel<T, ACC><<<grid_for(nvec), kDropThreads, 0, st>>>(X, Y, n, p);
+    FFK_CHECK_LAUNCH();
+    done = nvec * V;
+  }
+  if (done < n) {
+    dropout_scalar_kernel<T, ACC><<<grid_for(n - done), kDropThreads, 0, st>>>(X, Y, done, n, p);
+    FFK_CHECK_LAUNCH();
+  }
+  return FFK_OK;
+}
+
+}  // namespace ffk
+
+using namespace ffk;
+
+extern "C" int ffk_dropout_forward(ffk_stream_t stream, int dtype,
+                                   void const *input, void *output,
+                                   int64_t num_elements, float rate,
+                                   uint64_t seed, uint64_t offset) {
+  FFK_REQUIRE(num_elements >= 0, "dropout_forward: negative size");
+  DropoutParams p;
+  int rc = make_params("dropout_forward", rate, seed, offset, p);
+  if (rc != FFK_OK) return rc;
+  if (num_elements == 0) return FFK_OK;
+  FFK_REQUIRE(input && output, "dropout_forward: NULL tensor");
+  if (dtype == FFK_FLOAT) return dropout_run<float, false>(as_stream(stream), input, output, num_elements, p);
+  if (dtype == FFK_BF16) return dropout_run<bf16, false>(as_stream(stream), input, output, num_elements, p);
+  return fail(FFK_ERR_UNSUPPORTED, "dropout_forward: dtype %d not supported", dtype);
+}
+
+extern "C" int ffk_dropout_backward(ffk_stream_t stream, int dtype,
+                                    void const *output_grad, void *input_grad,
+                                    int64_t num_elements, float rate,
+                                    uint64_t seed, uint64_t offset,
+                                    int accumulate) {
+  FFK_REQUIRE(num_elements >= 0, "dropout_backward: negative size");
+  DropoutParams p;
+  int rc = make_params("dropout_backward", rate, seed, offset, p);
+  if (rc != FFK_OK) return rc;
+  if (num_elements == 0) return FFK_OK;
+  FFK_REQUIRE(output_grad && input_grad, "dropout_backward: NULL tensor");
+  hipStream_t st = as_stream(stream);
+  if (dtype == FFK_FLOAT) {
+    return accumulate ? dropout_run<float, true>(st, output_grad, input_grad, num_elements, p)
+                      : dropout_run<float, false>(st, output_grad, input_grad, num_elements, p);
+  }
+  if (dtype == FFK_BF16) {
+    return accumulate ? dropout_run<bf16, true>(st, output_grad, input_grad, num_elements, p)
+                      : dropout_run<bf16, false>(st, output_grad, input_grad, num_elements, p);
+  }
+  return fail(FFK_ERR_UNSUPPORTED, "dropout_backward: dtype %d not supported", dtype);
+}
+
+extern "C" int ffk_dropout_mask(ffk_stream_t stream, uint8_t *mask,
+                                int64_t num_elements, float rate, uint64_t seed,
+                                uint64_t offset) {
+  FFK_REQUIRE(num_elements >= 0, "dropout_mask: negative size");
+  DropoutParams p;
+  int rc = make_params("dropout_mask", rate, seed, offset, p);
+  if (rc != FFK_OK) return rc;
+  if (num_elements == 0) return FFK_OK;
+  FFK_REQUIRE(mask != nullptr, "dropout_mask: NULL mask");
+  dropout_mask_kernel<<<grid_for(num_elements), kDropThreads, 0, as_stream(stream)>>>(mask, num_elements, p);
+  FFK_CHECK_LAUNCH();
+  return FFK_OK;
+}

@@ -1,0 +1,155 @@
+// Shared device/host helpers for the gfx950 operator kernels: error reporting
+// across the C ABI, bf16 <-> fp32 conversion, 16-byte vector access and
+// wavefront (64-lane) reductions. Everything here is written for CDNA4 only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include "../../include/ffk.h"
+
+namespace ffk {
+
+// ---- error plumbing -------------------------------------------------------
+// Each entry point returns FFK_OK or an error code; the text is kept per
+// thread and read back through ffk_last_error().
+void set_error(char const *fmt, ...);
+int fail(int code, char const *fmt, ...);
+
+#define FFK_HIP(expr)                                                          \
+  do {                                                                         \
+    hipError_t e__ = (expr);                                                   \
+    if (e__ != hipSuccess) {                                                   \
+      return ::ffk::fail(FFK_ERR_HIP, "%s failed: %s (%s:%d)", #expr,          \
+                         hipGetErrorString(e__), __FILE__, __LINE__);          \
+    }                                                                          \
+  } while (0)
+
+#define FFK_REQUIRE(cond, ...)                                                 \
+  do {                                                                         \
+    if (!(cond)) {                                                             \
+      return ::ffk::fail(FFK_ERR_INVALID, __VA_ARGS__);                        \
+    }                                                                          \
+  } while (0)
+
+#define FFK_CHECK_LAUNCH() FFK_HIP(hipGetLastError())
+
+static inline hipStream_t as_stream(ffk_stream_t s) {
+  return reinterpret_cast<hipStream_t>(s);
+}
+
+static inline size_t dtype_size(int dt) {
+  switch (dt) {
+    case FFK_BOOL: return 1;
+    case FFK_INT32: return 4;
+    case FFK_INT64: return 8;
+    case FFK_HALF: return 2;
+    case FFK_FLOAT: return 4;
+    case FFK_DOUBLE: return 8;
+    case FFK_BF16: return 2;
+    default: return 0;
+  }
+}
+
+constexpr int kWave = 64;     // CDNA wavefront width
+constexpr int kNumCU = 256;   // MI355X compute units (8 XCDs x 32)
+constexpr int kNumXCD = 8;
+
+// ---- bf16 -----------------------------------------------------------------
+typedef __bf16 bf16;
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) {
+  return __uint_as_float(bits16 << 16);
+}
+// Round-to-nearest-even fp32 -> bf16 (the single rounding point of every
+// bf16 kernel: inputs bf16 -> fp32 arithmetic -> one rounding at the store).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    return (u >> 16) | 0x40u;  // quiet NaN
+  }
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// ---- typed vector access: N elements of T <-> N floats --------------------
+// VecIO<T>::kVec elements make one 16-byte access.
+template <typename T>
+struct VecIO;
+
+template <>
+struct VecIO<float> {
+  static constexpr int kVec = 4;
+  __device__ __forceinline__ static void load(float const *p, float (&v)[4]) {
+    f32x4 r = *reinterpret_cast<f32x4 const *>(p);
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  __device__ __forceinline__ static void store(float *p, float const (&v)[4]) {
+    f32x4 r = {v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<f32x4 *>(p) = r;
+  }
+  __device__ __forceinline__ static float load1(float const *p) { return *p; }
+  __device__ __forceinline__ static void store1(float *p, float v) { *p = v; }
+};
+
+template <>
+struct VecIO<bf16> {
+  static constexpr int kVec = 8;
+  __device__ __forceinline__ static void load(bf16 const *p, float (&v)[8]) {
+    u32x4 r = *reinterpret_cast<u32x4 const *>(p);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[2 * i] = __uint_as_float(r[i] << 16);
+      v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+    }
+  }
+  __device__ __forceinline__ static void store(bf16 *p, float const (&v)[8]) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      r[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+    }
+    *reinterpret_cast<u32x4 *>(p) = r;
+  }
+  __device__ __forceinline__ static float load1(bf16 const *p) {
+    return bf16_bits_to_f32(*reinterpret_cast<uint16_t const *>(p));
+  }
+  __device__ __forceinline__ static void store1(bf16 *p, float v) {
+    *reinterpret_cast<uint16_t *>(p) = (uint16_t)f32_to_bf16_bits(v);
+  }
+};
+
+// ---- wavefront reductions (64 lanes, DPP/shuffle based) -------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    v += __shfl_xor(v, off, 64);
+  }
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    v = fmaxf(v, __shfl_xor(v, off, 64));
+  }
+  return v;
+}
+
+static inline bool aligned16(void const *p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+__host__ __device__ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace ffk

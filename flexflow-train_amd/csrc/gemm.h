@@ -1,0 +1,31 @@
+// Internal GEMM interface shared by Linear, the attention projections and the
+// public ffk_gemm entry point.
+#pragma once
+#include "ffk_common.h"
+
+namespace ffk {
+
+struct GemmEpilogue {
+  void const *bias = nullptr;  // [N] in the GEMM dtype, added to every row
+  int activation = FFK_ACT_NONE;
+  bool accumulate = false;     // C += result instead of C = result
+};
+
+// C[M,N] (+)= op(A) . op(B), fp32 accumulation.
+//   trans_a == false: A is [M,K] row-major (lda = K); true: A is [K,M] (lda = M)
+//   trans_b == false: B is [K,N] row-major (ldb = N); true: B is [N,K] (ldb = K)
+// lda/ldb/ldc are row strides in elements (>= the dense value), so strided
+// views (column slices of a fused buffer) can be used directly.
+int gemm_dispatch(hipStream_t stream, int dtype, bool trans_a, bool trans_b,
+                  int64_t M, int64_t N, int64_t K, void const *A, int64_t lda,
+                  void const *B, int64_t ldb, void *C, int64_t ldc,
+                  GemmEpilogue const &ep);
+
+// out[N] (+)= sum over the M rows of X[M,N] (ldx row stride); `partials` is
+// fp32 scratch of colsum_partials_elems(M, N) floats.
+int64_t colsum_partials_elems(int64_t M, int64_t N);
+int colsum_dispatch(hipStream_t stream, int dtype, void const *X, int64_t ldx,
+                    int64_t M, int64_t N, void *out, bool accumulate,
+                    float *partials);
+
+}  // namespace ffk

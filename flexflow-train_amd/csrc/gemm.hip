@@ -1,0 +1,579 @@
+// GEMM kernels for gfx950 behind Linear and the attention projections.
+//
+//  * bf16: LDS-tiled, double-buffered MFMA kernel (v_mfma_f32_32x32x16_bf16,
+//    fp32 accumulators, one rounding at the store).  Operands whose reduction
+//    dimension is not contiguous in memory are staged into LDS as they lie in
+//    memory and read back with the transposing LDS load (ds_read_b64_tr_b16),
+//    so all four transpose variants run on the same pipeline.
+//  * fp32: MFMA v_mfma_f32_32x32x2f32 kernel with bounds-checked loads, used
+//    for the fp32 Linear (small, latency-bound shapes).
+//  * a plain one-thread-per-output kernel for shapes the tiled bf16 kernel
+//    cannot take (K or leading dimensions not a multiple of 8 elements).
+//
+// These replace the cublasGemmEx calls of the reference
+// (lib/kernels/src/cuda/ops/linear_kernels.cu:143,163,249,298,321).
+#include "gemm.h"
+
+namespace ffk {
+
+__device__ __forceinline__ float apply_activation(float v, int act) {
+  switch (act) {
+    case FFK_ACT_RELU:
+      // tensor_accessor_relu keeps x >= 0 (tensor_accessor_unary_ops.cc:32-38);
+      // identical to x > 0 ? x : 0 on every input except -0.0f.
+      return v >= 0.0f ? v : 0.0f;
+    case FFK_ACT_SIGMOID:
+      return 1.0f / (1.0f + expf(-v));
+    case FFK_ACT_TANH:
+      return tanhf(v);
+    case FFK_ACT_GELU:
+      return v * 0.5f * erfcf(-v * 0.70710678118654752440f);
+    default:
+      return v;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Block -> tile mapping.  Workgroups are dealt round-robin to the 8 XCDs, each
+// with its own L2; regroup ids so that one XCD works on a compact patch of the
+// output (tiles that share A rows / B columns), then walk the patch in groups
+// of kGroupM tile rows.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void tile_coords(int pid, int nbm, int nbn, int &tm,
+                                            int &tn) {
+  int const total = nbm * nbn;
+  if (total % kNumXCD == 0) {
+    int const xcd = pid % kNumXCD;
+    int const local = pid / kNumXCD;
+    pid = xcd * (total / kNumXCD) + local;
+  }
+  constexpr int kGroupM = 8;
+  int const group_size = kGroupM * nbn;
+  int const group = pid / group_size;
+  int const first_m = group * kGroupM;
+  int const rows = min(nbm - first_m, kGroupM);
+  int const in_group = pid % group_size;
+  tm = first_m + in_group % rows;
+  tn = in_group / rows;
+}
+
+// ---------------------------------------------------------------------------
+// bf16 MFMA kernel
+// ---------------------------------------------------------------------------
+constexpr int kBK = 64;        // K extent of one LDS tile
+constexpr int kPadK = 8;       // row padding (elements) of a K-contiguous tile
+constexpr int kPadMN = 32;     // row padding of an M/N-contiguous tile
+
+template <int ROWS, bool TRANS>
+struct TileGeom {
+  // TRANS == false: tile held as [ROWS][kBK] (reduction dim contiguous)
+  // TRANS == true : tile held as [kBK][ROWS] (as it lies in memory)
+  static constexpr int kStride = TRANS ? (ROWS + kPadMN) : (kBK + kPadK);
+  static constexpr int kElems = TRANS ? kBK * kStride : ROWS * kStride;
+};
+
+template <int BM, int BN, int WM, int WN, bool TA, bool TB, bool EDGE>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
+    bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
+    int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+    bf16 const *__restrict__ bias, int act, int accumulate) {
+  constexpr int NW = (BM / WM) * (BN / WN);
+  constexpr int NT = NW * 64;
+  constexpr int TM = WM / 32;  // MFMA tiles per wave along M
+  constexpr int TN = WN / 32;
+  using GA = TileGeom<BM, TA>;
+  using GB = TileGeom<BN, TB == false>;  // B is "transposed" when it is [K,N]
+  constexpr bool TBL = (TB == false);    // B tile lies as [kBK][BN]
+  constexpr int A_CHUNKS = BM * kBK / 8 / NT;  // 16-byte chunks per thread
+  constexpr int B_CHUNKS = BN * kBK / 8 / NT;
+  static_assert(BM * kBK / 8 % NT == 0 && BN * kBK / 8 % NT == 0, "tile/threads");
+
+  __shared__ __attribute__((aligned(16))) bf16 As[2][GA::kElems];
+  __shared__ __attribute__((aligned(16))) bf16 Bs[2][GB::kElems];
+
+  int const t = threadIdx.x;
+  int const lane = t & 63;
+  int const wave = t >> 6;
+  int const wm0 = (wave / (BN / WN)) * WM;
+  int const wn0 = (wave % (BN / WN)) * WN;
+
+  int tm, tn;
+  tile_coords(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+  int const m0 = tm * BM;
+  int const n0 = tn * BN;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  u32x4 ra[A_CHUNKS], rb[B_CHUNKS];
+
+  auto gload = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; i++) {
+      int c = t + i * NT;
+      int64_t off;
+      bool ok = true;
+      if (!TA) {
+        int row = c >> 3, kc = c & 7;
+        int gm = m0 + row, gk = k0 + kc * 8;
+        if (EDGE) {
+          gm = min(gm, M - 1);
+          ok = gk < K;
+          gk = ok ? gk : 0;
+        }
+        off = (int64_t)gm * lda + gk;
+      } else {
+        int krow = c / (BM / 8), mc = c % (BM / 8);
+        int gk = k0 + krow, gm = m0 + mc * 8;
+        if (EDGE) {
+          ok = gk < K && gm < M;  // M % 8 == 0 is required, so chunks are whole
+          gk = ok ? gk : 0;
+          gm = ok ? gm : 0;
+        }
+        off = (int64_t)gk * lda + gm;
+      }
+      u32x4 v = *reinterpret_cast<u32x4 const *>(A + off);
+      if (EDGE && !ok) v = u32x4{0u, 0u, 0u, 0u};
+      ra[i] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; i++) {
+      int c = t + i * NT;
+      int64_t off;
+      bool ok = true;
+      if (!TBL) {
+        int row = c >> 3, kc = c & 7;
+        int gn = n0 + row, gk = k0 + kc * 8;
+        if (EDGE) {
+          gn = min(gn, N - 1);
+          ok = gk < K;
+          gk = ok ? gk : 0;
+        }
+        off = (int64_t)gn * ldb + gk;
+      } else {
+        int krow = c / (BN / 8), nc = c % (BN / 8);
+        int gk = k0 + krow, gn = n0 + nc * 8;
+        if (EDGE) {
+          ok = gk < K && gn < N;
+          gk = ok ? gk : 0;
+          gn = ok ? gn : 0;
+        }
+        off = (int64_t)gk * ldb + gn;
+      }
+      u32x4 v = *reinterpret_cast<u32x4 const *>(B + off);
+      if (EDGE && !ok) v = u32x4{0u, 0u, 0u, 0u};
+      rb[i] = v;
+    }
+  };
+
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; i++) {
+      int c = t + i * NT;
+      int idx;
+      if (!TA) {
+        idx = (c >> 3) * GA::kStride + (c & 7) * 8;
+      } else {
+        idx = (c / (BM / 8)) * GA::kStride + (c % (BM / 8)) * 8;
+      }
+      *reinterpret_cast<u32x4 *>(&As[buf][idx]) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; i++) {
+      int c = t + i * NT;
+      int idx;
+      if (!TBL) {
+        idx = (c >> 3) * GB::kStride + (c & 7) * 8;
+      } else {
+        idx = (c / (BN / 8)) * GB::kStride + (c % (BN / 8)) * 8;
+      }
+      *reinterpret_cast<u32x4 *>(&Bs[buf][idx]) = rb[i];
+    }
+  };
+
+  // Operand fragment for one 32-row MFMA tile and one 16-wide k step.
+  // Lane l supplies row (l % 32), k = 8 * (l / 32) .. + 7.
+  auto frag = [&](bf16 const *tile, int stride, bool trans, int row0,
+                  int kk) -> bf16x8 {
+    if (!trans) {
+      bf16 const *p = tile + (row0 + (lane & 31)) * stride + kk * 16 + (lane >> 5) * 8;
+      return *reinterpret_cast<bf16x8 const *>(p);
+    }
+    // Transposing load: within each 16-lane group, lane i points at 4 elements
+    // of row k_(i/4), columns 4*(i%4)..+3, and receives column i of the four
+    // rows.  Two loads give 8 consecutive k for this lane's row.
+    int const i16 = lane & 15;
+    int const col = row0 + ((lane >> 4) & 1) * 16 + (i16 & 3) * 4;
+    int const kbase = kk * 16 + (lane >> 5) * 8 + (i16 >> 2);
+    typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (lds_s16x4_ptr)(tile + kbase * stride + col));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (lds_s16x4_ptr)(tile + (kbase + 4) * stride + col));
+    union {
+      s16x4 h[2];
+      bf16x8 v;
+    } u;
+    u.h[0] = lo;
+    u.h[1] = hi;
+    return u.v;
+  };
+
+  int const KT = (K + kBK - 1) / kBK;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  int cur = 0;
+  for (int kt = 0; kt < KT; kt++) {
+    bool const more = kt + 1 < KT;
+    if (more) {
+      gload((kt + 1) * kBK);
+    }
+#pragma unroll
+    for (int kk = 0; kk < kBK / 16; kk++) {
+      bf16x8 af[TM], bfr[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        af[i] = frag(As[cur], GA::kStride, TA, wm0 + i * 32, kk);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        bfr[j] = frag(Bs[cur], GB::kStride, TBL, wn0 + j * 32, kk);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j],
+                                                             acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      lstore(cur ^ 1);
+    }
+    __syncthreads();
+    cur ^= 1;
+  }
+
+  // Epilogue: accumulator element r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
+  // column l % 32 of its 32x32 tile.
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    int const n = n0 + wn0 + j * 32 + (lane & 31);
+    bool const n_ok = !EDGE || n < N;
+    float bv = 0.0f;
+    if (bias != nullptr && n_ok) {
+      bv = VecIO<bf16>::load1(bias + n);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        int const m = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (n_ok && (!EDGE || m < M)) {
+          float v = acc[i][j][r] + bv;
+          v = apply_activation(v, act);
+          bf16 *dst = C + (int64_t)m * ldc + n;
+          if (accumulate) {
+            v += VecIO<bf16>::load1(dst);
+          }
+          VecIO<bf16>::store1(dst, v);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// fp32 MFMA kernel (32x32x2), 64x64 block tile, bounds-checked everywhere.
+// ---------------------------------------------------------------------------
+template <bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(
+    float const *__restrict__ A, float const *__restrict__ B, float *C, int M,
+    int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+    float const *__restrict__ bias, int act, int accumulate) {
+  constexpr int BM = 64, BN = 64, BKF = 16, LD = 68;
+  __shared__ float As[BKF][LD];  // [k][m]
+  __shared__ float Bs[BKF][LD];  // [k][n]
+  int const t = threadIdx.x;
+  int const lane = t & 63;
+  int const wave = t >> 6;
+  int const wm0 = (wave >> 1) * 32;
+  int const wn0 = (wave & 1) * 32;
+  int const nbn = (N + BN - 1) / BN;
+  int const m0 = (blockIdx.x / nbn) * BM;
+  int const n0 = (blockIdx.x % nbn) * BN;
+
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+  for (int k0 = 0; k0 < K; k0 += BKF) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      int m, k;
+      if (!TA) {  // A[M,K]: k fastest across lanes
+        k = t & 15;
+        m = (t >> 4) + 16 * i;
+      } else {  // A[K,M]: m fastest
+        m = t & 63;
+        k = (t >> 6) + 4 * i;
+      }
+      int gm = m0 + m, gk = k0 + k;
+      float v = 0.0f;
+      if (gm < M && gk < K) {
+        v = TA ? A[(int64_t)gk * lda + gm] : A[(int64_t)gm * lda + gk];
+      }
+      As[k][m] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      int n, k;
+      if (TB) {  // B[N,K]: k fastest
+        k = t & 15;
+        n = (t >> 4) + 16 * i;
+      } else {  // B[K,N]: n fastest
+        n = t & 63;
+        k = (t >> 6) + 4 * i;
+      }
+      int gn = n0 + n, gk = k0 + k;
+      float v = 0.0f;
+      if (gn < N && gk < K) {
+        v = TB ? B[(int64_t)gn * ldb + gk] : B[(int64_t)gk * ldb + gn];
+      }
+      Bs[k][n] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BKF / 2; kk++) {
+      float a = As[2 * kk + (lane >> 5)][wm0 + (lane & 31)];
+      float b = Bs[2 * kk + (lane >> 5)][wn0 + (lane & 31)];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  int const n = n0 + wn0 + (lane & 31);
+  if (n < N) {
+    float bv = bias != nullptr ? bias[n] : 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      int const m = m0 + wm0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+      if (m < M) {
+        float v = apply_activation(acc[r] + bv, act);
+        float *dst = C + (int64_t)m * ldc + n;
+        if (accumulate) {
+          v += *dst;
+        }
+        *dst = v;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Plain kernel for bf16 shapes the tiled kernel cannot take.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gemm_bf16_plain_kernel(
+    bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
+    int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int ta, int tb,
+    bf16 const *__restrict__ bias, int act, int accumulate) {
+  int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * N) return;
+  int m = (int)(idx / N), n = (int)(idx % N);
+  float acc = 0.0f;
+  for (int k = 0; k < K; k++) {
+    float a = VecIO<bf16>::load1(ta ? A + (int64_t)k * lda + m : A + (int64_t)m * lda + k);
+    float b = VecIO<bf16>::load1(tb ? B + (int64_t)n * ldb + k : B + (int64_t)k * ldb + n);
+    acc += a * b;
+  }
+  if (bias != nullptr) acc += VecIO<bf16>::load1(bias + n);
+  acc = apply_activation(acc, act);
+  bf16 *dst = C + (int64_t)m * ldc + n;
+  if (accumulate) acc += VecIO<bf16>::load1(dst);
+  VecIO<bf16>::store1(dst, acc);
+}
+
+template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+static hipError_t launch_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
+                              bf16 *C, int M, int N, int K, int64_t lda,
+                              int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
+  int const blocks = (int)(ceil_div(M, BM) * ceil_div(N, BN));
+  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  bool const edge = (M % BM) || (N % BN) || (K % kBK);
+  bf16 const *bias = static_cast<bf16 const *>(ep.bias);
+  if (edge) {
+    gemm_bf16_kernel<BM, BN, WM, WN, TA, TB, true><<<blocks, NT, 0, st>>>(
+        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate);
+  } else {
+    gemm_bf16_kernel<BM, BN, WM, WN, TA, TB, false><<<blocks, NT, 0, st>>>(
+        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate);
+  }
+  return hipGetLastError();
+}
+
+template <bool TA, bool TB>
+static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
+                            bf16 *C, int M, int N, int K, int64_t lda,
+                            int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
+  // Largest tile that still gives every CU a workgroup.
+  int64_t const b128 = ceil_div(M, 128) * ceil_div(N, 128);
+  if (b128 >= kNumCU) {
+    return launch_bf16<128, 128, 64, 64, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+  }
+  return launch_bf16<64, 64, 32, 32, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+}
+
+// ---------------------------------------------------------------------------
+// Column sums (bias gradient): out[n] (+)= sum_m X[m,n]
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_partial_kernel(
+    T const *__restrict__ X, int64_t ldx, int M, int N, int rows_per_split,
+    float *__restrict__ partials) {
+  __shared__ float red[4][64];
+  int const cx = threadIdx.x & 63;
+  int const ry = threadIdx.x >> 6;
+  int const n = blockIdx.x * 64 + cx;
+  int const r0 = blockIdx.y * rows_per_split;
+  int const r1 = min(M, r0 + rows_per_split);
+  float s = 0.0f;
+  if (n < N) {
+    for (int m = r0 + ry; m < r1; m += 4) {
+      s += VecIO<T>::load1(X + (int64_t)m * ldx + n);
+    }
+  }
+  red[ry][cx] = s;
+  __syncthreads();
+  if (ry == 0 && n < N) {
+    partials[(int64_t)blockIdx.y * N + n] =
+        red[0][cx] + red[1][cx] + red[2][cx] + red[3][cx];
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_final_kernel(
+    float const *__restrict__ partials, int splits, int N, T *out,
+    int accumulate) {
+  int const n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  float s = 0.0f;
+  for (int r = 0; r < splits; r++) {
+    s += partials[(int64_t)r * N + n];
+  }
+  if (accumulate) {
+    s += VecIO<T>::load1(out + n);
+  }
+  VecIO<T>::store1(out + n, s);
+}
+
+static int colsum_splits(int64_t M) {
+  int64_t s = ceil_div(M, 128);
+  return (int)(s < 1 ? 1 : (s > 64 ? 64 : s));
+}
+
+int64_t colsum_partials_elems(int64_t M, int64_t N) {
+  return (int64_t)colsum_splits(M) * N;
+}
+
+int colsum_dispatch(hipStream_t st, int dtype, void const *X, int64_t ldx,
+                    int64_t M, int64_t N, void *out, bool accumulate,
+                    float *partials) {
+  FFK_REQUIRE(partials != nullptr, "colsum: partials scratch is NULL");
+  int const splits = colsum_splits(M);
+  int const rows_per_split = (int)ceil_div(M, splits);
+  dim3 grid((unsigned)ceil_div(N, 64), (unsigned)splits);
+  if (dtype == FFK_FLOAT) {
+    colsum_partial_kernel<float><<<grid, 256, 0, st>>>(
+        static_cast<float const *>(X), ldx, (int)M, (int)N, rows_per_split, partials);
+    FFK_CHECK_LAUNCH();
+    colsum_final_kernel<float><<<(unsigned)ceil_div(N, 256), 256, 0, st>>>(
+        partials, splits, (int)N, static_cast<float *>(out), accumulate);
+  } else if (dtype == FFK_BF16) {
+    colsum_partial_kernel<bf16><<<grid, 256, 0, st>>>(
+        static_cast<bf16 const *>(X), ldx, (int)M, (int)N, rows_per_split, partials);
+    FFK_CHECK_LAUNCH();
+    colsum_final_kernel<bf16><<<(unsigned)ceil_div(N, 256), 256, 0, st>>>(
+        partials, splits, (int)N, static_cast<bf16 *>(out), accumulate);
+  } else {
+    return fail(FFK_ERR_UNSUPPORTED, "colsum: dtype %d not supported", dtype);
+  }
+  FFK_CHECK_LAUNCH();
+  return FFK_OK;
+}
+
+int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
+                  int64_t N, int64_t K, void const *A, int64_t lda,
+                  void const *B, int64_t ldb, void *C, int64_t ldc,
+                  GemmEpilogue const &ep) {
+  FFK_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm: negative dimension");
+  if (M == 0 || N == 0) return FFK_OK;
+  FFK_REQUIRE(A && B && C, "gemm: NULL operand");
+  FFK_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31),
+              "gemm: dimension exceeds 2^31");
+  FFK_REQUIRE(lda >= (ta ? M : K) && ldb >= (tb ? K : N) && ldc >= N,
+              "gemm: leading dimension smaller than the row length");
+  hipError_t e;
+  if (dtype == FFK_FLOAT) {
+    float const *a = static_cast<float const *>(A);
+    float const *b = static_cast<float const *>(B);
+    float *c = static_cast<float *>(C);
+    float const *bias = static_cast<float const *>(ep.bias);
+    int const blocks = (int)(ceil_div(M, 64) * ceil_div(N, 64));
+#define FFK_LAUNCH_F32(TA_, TB_)                                               \
+  gemm_f32_kernel<TA_, TB_><<<blocks, 256, 0, st>>>(                           \
+      a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, bias, ep.activation,     \
+      ep.accumulate)
+    if (!ta && !tb) FFK_LAUNCH_F32(false, false);
+    else if (!ta && tb) FFK_LAUNCH_F32(false, true);
+    else if (ta && !tb) FFK_LAUNCH_F32(true, false);
+    else FFK_LAUNCH_F32(true, true);
+#undef FFK_LAUNCH_F32
+    e = hipGetLastError();
+  } else if (dtype == FFK_BF16) {
+    bf16 const *a = static_cast<bf16 const *>(A);
+    bf16 const *b = static_cast<bf16 const *>(B);
+    bf16 *c = static_cast<bf16 *>(C);
+    // 16-byte chunks: K and any contiguous non-reduction extent must be a
+    // multiple of 8 elements, rows 16-byte aligned.
+    bool vec_ok = (K % 8 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
+                  aligned16(A) && aligned16(B) && (!ta || M % 8 == 0) &&
+                  (tb || N % 8 == 0) && K > 0;
+    if (!vec_ok) {
+      int64_t total = M * N;
+      gemm_bf16_plain_kernel<<<(unsigned)ceil_div(total, 256), 256, 0, st>>>(
+          a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ta, tb,
+          static_cast<bf16 const *>(ep.bias), ep.activation, ep.accumulate);
+      e = hipGetLastError();
+    } else if (!ta && !tb) {
+      e = pick_bf16<false, false>(st, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ep);
+    } else if (!ta && tb) {
+      e = pick_bf16<false, true>(st, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ep);
+    } else if (ta && !tb) {
+      e = pick_bf16<true, false>(st, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ep);
+    } else {
+      e = pick_bf16<true, true>(st, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ep);
+    }
+  } else {
+    return fail(FFK_ERR_UNSUPPORTED, "gemm: dtype %d not supported", dtype);
+  }
+  FFK_HIP(e);
+  return FFK_OK;
+}
+
+}  // namespace ffk
+
+using namespace ffk;
+
+extern "C" int ffk_gemm(ffk_stream_t stream, int dtype, int trans_a,
+                        int trans_b, int64_t M, int64_t N, int64_t K,
+                        void const *A, void const *B, void *C, int accumulate) {
+  GemmEpilogue ep;
+  ep.accumulate = accumulate != 0;
+  return gemm_dispatch(as_stream(stream), dtype, trans_a != 0, trans_b != 0, M,
+                       N, K, A, trans_a ? M : K, B, trans_b ? K : N, C, N, ep);
+}

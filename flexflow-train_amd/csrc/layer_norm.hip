@@ -1,0 +1,468 @@
+// LayerNorm forward/backward for gfx950: one pass over the data.
+//
+// forward : a row lives in the registers of one wavefront (or one workgroup
+//           for long rows); mean and variance are reduced with wave shuffles,
+//           the normalised row is written once.  (Reference: two kernels and
+//           three reads of X, lib/kernels/src/cuda/ops/layer_norm_kernels.cu:
+//           69-112,328-352.)
+// backward: one pass over dY and X produces dX (the formula of
+//           LayerNormBackwardCUDAKenrel, layer_norm_kernels.cu:163-181, which
+//           the reference never launches) and per-workgroup partial column
+//           sums for dgamma/dbeta, reduced by a second small kernel
+//           (reference: ComputeInternalGradients + GammaBetaBackward, two more
+//           passes, :115-290,354-410).
+#include "rowwise.h"
+
+namespace ffk {
+
+template <typename T, int EPT, int WPR>
+__global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_kernel(
+    T const *__restrict__ X, T *__restrict__ Y, T const *__restrict__ gamma,
+    T const *__restrict__ beta, float *__restrict__ mean,
+    float *__restrict__ rstd, int64_t M, int N, float eps) {
+  constexpr int V = VecIO<T>::kVec;
+  constexpr int RPB = 4 / WPR;  // rows per workgroup
+  constexpr int LANES = 64 * WPR;
+  __shared__ float smem[2][4][2];
+  RowReducer<WPR> red(smem);
+  int const nvec = N / V;
+  int const lane = WPR == 1 ? (threadIdx.x & 63) : threadIdx.x;
+  int64_t const row = (int64_t)blockIdx.x * RPB + (WPR == 1 ? (threadIdx.x >> 6) : 0);
+  bool const row_ok = row < M;
+  T const *xr = X + (row_ok ? row : 0) * (int64_t)N;
+
+  float x[EPT][V];
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < EPT; j++) {
+    int v = lane + j * LANES;
+    if (v < nvec) {
+      VecIO<T>::load(xr + (int64_t)v * V, x[j]);
+#pragma unroll
+      for (int e = 0; e < V; e++) s += x[j][e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; e++) x[j][e] = 0.0f;
+    }
+  }
+  float const inv_n = 1.0f / (float)N;
+  float const mu = red.sum(s) * inv_n;
+  float q = 0.0f;
+#pragma unroll
+  for (int j = 0; j < EPT; j++) {
+    int v = lane + j * LANES;
+    if (v < nvec) {
+#pragma unroll
+      for (int e = 0; e < V; e++) {
+        float d = x[j][e] - mu;
+        q += d * d;
+      }
+    }
+  }
+  float const var = red.sum(q) * inv_n;
+  float const rs = 1.0f / sqrtf(var + eps);
+  if (!row_ok) return;
+  if (lane == 0) {
+    mean[row] = mu;
+    rstd[row] = rs;
+  }
+  T *yr = Y + row * (int64_t)N;
+#pragma unroll
+  for (int j = 0; j < EPT; j++) {
+    int v = lane + j * LANES;
+    if (v < nvec) {
+      float g[V], b[V], y[V];
+      if (gamma != nullptr) {
+        VecIO<T>::load(gamma + (int64_t)v * V, g);
+      }
+      if (beta != nullptr) {
+        VecIO<T>::load(beta + (int64_t)v * V, b);
+      }
+#pragma unroll
+      for (int e = 0; e < V; e++) {
+        float xh = (x[j][e] - mu) * rs;
+        float gv = gamma != nullptr ? g[e] : 1.0f;
+        float bv = beta != nullptr ? b[e] : 0.0f;
+        y[e] = xh * gv + bv;
+      }
+      VecIO<T>::store(yr + (int64_t)v * V, y);
+    }
+  }
+}
+
+// Generic forward: any N, one workgroup per row, scalar accesses.
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_generic_kernel(
+    T const *__restrict__ X, T *__restrict__ Y, T const *__restrict__ gamma,
+    T const *__restrict__ beta, float *__restrict__ mean,
+    float *__restrict__ rstd, int64_t M, int N, float eps) {
+  __shared__ float smem[2][4][2];
+  RowReducer<4> red(smem);
+  int64_t const row = blockIdx.x;
+  T const *xr = X + row * (int64_t)N;
+  float s = 0.0f;
+  for (int j = threadIdx.x; j < N; j += kRowThreads) s += VecIO<T>::load1(xr + j);
+  float const mu = red.sum(s) / (float)N;
+  float q = 0.0f;
+  for (int j = threadIdx.x; j < N; j += kRowThreads) {
+    float d = VecIO<T>::load1(xr + j) - mu;
+    q += d * d;
+  }
+  float const rs = 1.0f / sqrtf(red.sum(q) / (float)N + eps);
+  if (threadIdx.x == 0) {
+    mean[row] = mu;
+    rstd[row] = rs;
+  }
+  T *yr = Y + row * (int64_t)N;
+  for (int j = threadIdx.x; j < N; j += kRowThreads) {
+    float gv = gamma != nullptr ? VecIO<T>::load1(gamma + j) : 1.0f;
+    float bv = beta != nullptr ? VecIO<T>::load1(beta + j) : 0.0f;
+    VecIO<T>::store1(yr + j, (VecIO<T>::load1(xr + j) - mu) * rs * gv + bv);
+  }
+}
+
+// Backward, persistent over rows so that the dgamma/dbeta partial sums stay
+// in registers until the workgroup is done.
+template <typename T, int EPT, int WPR, bool ACC>
+__global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
+    T const *__restrict__ dY, T const *__restrict__ X,
+    float const *__restrict__ mean, float const *__restrict__ rstd,
+    T const *__restrict__ gamma, T *dX, float *__restrict__ partials,
+    int64_t M, int N) {
+  constexpr int V = VecIO<T>::kVec;
+  constexpr int RPB = 4 / WPR;
+  constexpr int LANES = 64 * WPR;
+  __shared__ float smem[2][4][2];
+  RowReducer<WPR> red(smem);
+  int const nvec = N / V;
+  int const lane = WPR == 1 ? (threadIdx.x & 63) : threadIdx.x;
+  int const sub = WPR == 1 ? (threadIdx.x >> 6) : 0;
+  float const inv_n = 1.0f / (float)N;
+
+  float g[EPT][V], dg[EPT][V], db[EPT][V];
+#pragma unroll
+  for (int j = 0; j < EPT; j++) {
+    int v = lane + j * LANES;
+#pragma unroll
+    for (int e = 0; e < V; e++) {
+      g[j][e] = 1.0f;
+      dg[j][e] = 0.0f;
+      db[j][e] = 0.0f;
+    }
+    if (gamma != nullptr && v < nvec) {
+      VecIO<T>::load(gamma + (int64_t)v * V, g[j]);
+    }
+  }
+
+  int64_t const row_step = (int64_t)gridDim.x * RPB;
+  // Every wave of a workgroup runs the same number of iterations so the
+  // barriers inside the reducer stay aligned.
+  for (int64_t base = (int64_t)blockIdx.x * RPB; base < M; base += row_step) {
+    int64_t const row = base + sub;
+    bool const row_ok = row < M;
+    int64_t const r = row_ok ? row : 0;
+    float x[EPT][V], dy[EPT][V];
+    float const mu = mean[r], rs = rstd[r];
+    float s1 = 0.0f, s2 = 0.0f;  // sum dy*g, sum dy*g*xhat
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+      int v = lane + j * LANES;
+      if (v < nvec) {
+        VecIO<T>::load(X + r * (int64_t)N + (int64_t)v * V, x[j]);
+        VecIO<T>::load(dY + r * (int64_t)N + (int64_t)v * V, dy[j]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; e++) {
+          x[j][e] = 0.0f;
+          dy[j][e] = 0.0f;
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+#pragma unroll
+      for (int e = 0; e < V; e++) {
+        float xh = (x[j][e] - mu) * rs;
+        float dyg = dy[j][e] * g[j][e];
+        s1 += dyg;
+        s2 += dyg * xh;
+        x[j][e] = xh;
+        if (row_ok) {
+          dg[j][e] += dy[j][e] * xh;
+          db[j][e] += dy[j][e];
+        }
+      }
+    }
+    red.sum2(s1, s2);
+    float const m1 = s1 * inv_n, m2 = s2 * inv_n;
+    if (row_ok && dX != nullptr) {
+#pragma unroll
+      for (int j = 0; j < EPT; j++) {
+        int v = lane + j * LANES;
+        if (v < nvec) {
+          float o[V];
+          T *dst = dX + row * (int64_t)N + (int64_t)v * V;
+          if (ACC) {
+            VecIO<T>::load(dst, o);
+          }
+#pragma unroll
+          for (int e = 0; e < V; e++) {
+            float val = rs * (dy[j][e] * g[j][e] - m1 - x[j][e] * m2);
+            o[e] = ACC ? o[e] + val : val;
+          }
+          VecIO<T>::store(dst, o);
+        }
+      }
+    }
+  }
+
+  // Workgroup partial: with WPR == 1 the four waves hold different rows of the
+  // same columns; fold them through LDS first.
+  float *pg = partials + (int64_t)blockIdx.x * 2 * N;
+  float *pb = pg + N;
+  if (WPR == 1) {
+    __shared__ float fold[3][64][V + 1];
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+      int v = lane + j * LANES;
+      for (int pass = 0; pass < 2; pass++) {
+        __syncthreads();
+        if (sub > 0) {
+#pragma unroll
+          for (int e = 0; e < V; e++) {
+            fold[sub - 1][lane][e] = pass == 0 ? dg[j][e] : db[j][e];
+          }
+        }
+        __syncthreads();
+        if (sub == 0 && v < nvec) {
+#pragma unroll
+          for (int e = 0; e < V; e++) {
+            float tot = (pass == 0 ? dg[j][e] : db[j][e]) + fold[0][lane][e] +
+                        fold[1][lane][e] + fold[2][lane][e];
+            (pass == 0 ? pg : pb)[(int64_t)v * V + e] = tot;
+          }
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+      int v = lane + j * LANES;
+      if (v < nvec) {
+#pragma unroll
+        for (int e = 0; e < V; e++) {
+          pg[(int64_t)v * V + e] = dg[j][e];
+          pb[(int64_t)v * V + e] = db[j][e];
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void layer_norm_param_grad_final_kernel(
+    float const *__restrict__ partials, int nparts, int N, T *dgamma,
+    T *dbeta) {
+  int const j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= N) return;
+  float sg = 0.0f, sb = 0.0f;
+  for (int p = 0; p < nparts; p++) {
+    sg += partials[(int64_t)p * 2 * N + j];
+    sb += partials[(int64_t)p * 2 * N + N + j];
+  }
+  if (dgamma != nullptr) VecIO<T>::store1(dgamma + j, sg);
+  if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, sb);
+}
+
+// Generic backward: any N; one workgroup per row for dX, then a column kernel
+// for dgamma/dbeta that walks all rows (GammaBetaBackwardSimpleCUDAKernel
+// style, layer_norm_kernels.cu:184-214).
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_generic_dx_kernel(
+    T const *__restrict__ dY, T const *__restrict__ X,
+    float const *__restrict__ mean, float const *__restrict__ rstd,
+    T const *__restrict__ gamma, T *dX, int64_t M, int N, int acc) {
+  __shared__ float smem[2][4][2];
+  RowReducer<4> red(smem);
+  int64_t const row = blockIdx.x;
+  float const mu = mean[row], rs = rstd[row];
+  float s1 = 0.0f, s2 = 0.0f;
+  for (int j = threadIdx.x; j < N; j += kRowThreads) {
+    float gv = gamma != nullptr ? VecIO<T>::load1(gamma + j) : 1.0f;
+    float dyg = VecIO<T>::load1(dY + row * (int64_t)N + j) * gv;
+    float xh = (VecIO<T>::load1(X + row * (int64_t)N + j) - mu) * rs;
+    s1 += dyg;
+    s2 += dyg * xh;
+  }
+  red.sum2(s1, s2);
+  float const m1 = s1 / (float)N, m2 = s2 / (float)N;
+  for (int j = threadIdx.x; j < N; j += kRowThreads) {
+    float gv = gamma != nullptr ? VecIO<T>::load1(gamma + j) : 1.0f;
+    float dyg = VecIO<T>::load1(dY + row * (int64_t)N + j) * gv;
+    float xh = (VecIO<T>::load1(X + row * (int64_t)N + j) - mu) * rs;
+    float val = rs * (dyg - m1 - xh * m2);
+    T *dst = dX + row * (int64_t)N + j;
+    if (acc) val += VecIO<T>::load1(dst);
+    VecIO<T>::store1(dst, val);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void layer_norm_bwd_generic_param_kernel(
+    T const *__restrict__ dY, T const *__restrict__ X,
+    float const *__restrict__ mean, float const *__restrict__ rstd, T *dgamma,
+    T *dbeta, int64_t M, int N) {
+  int const j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= N) return;
+  float sg = 0.0f, sb = 0.0f;
+  for (int64_t i = 0; i < M; i++) {
+    float d = VecIO<T>::load1(dY + i * (int64_t)N + j);
+    float xh = (VecIO<T>::load1(X + i * (int64_t)N + j) - mean[i]) * rstd[i];
+    sg += d * xh;
+    sb += d;
+  }
+  if (dgamma != nullptr) VecIO<T>::store1(dgamma + j, sg);
+  if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, sb);
+}
+
+constexpr int kLnBwdMaxBlocks = 2 * kNumCU;
+
+static int ln_bwd_blocks(int64_t M, int wpr) {
+  int64_t rpb = 4 / wpr;
+  int64_t b = ceil_div(M, rpb);
+  return (int)(b < kLnBwdMaxBlocks ? b : kLnBwdMaxBlocks);
+}
+
+template <typename T>
+static int ln_forward(hipStream_t st, void const *x, void *y, void const *gamma,
+                      void const *beta, float *mean, float *rstd, int64_t M,
+                      int64_t N, float eps) {
+  constexpr int V = VecIO<T>::kVec;
+  T const *X = static_cast<T const *>(x);
+  T *Y = static_cast<T *>(y);
+  T const *G = static_cast<T const *>(gamma);
+  T const *Bt = static_cast<T const *>(beta);
+  int ept = 0, wpr = 0;
+  bool vec = (N % V == 0) && aligned16(x) && aligned16(y) &&
+             (gamma == nullptr || aligned16(gamma)) &&
+             (beta == nullptr || aligned16(beta)) && pick_row_config(N / V, ept, wpr);
+  if (vec) {
+    int64_t blocks = ceil_div(M, 4 / wpr);
+#define CALL(E, W)                                                             \
+  layer_norm_fwd_kernel<T, E, W><<<(unsigned)blocks, kRowThreads, 0, st>>>(    \
+      X, Y, G, Bt, mean, rstd, M, (int)N, eps)
+    FFK_ROW_DISPATCH(ept, wpr, CALL);
+#undef CALL
+  } else {
+    layer_norm_fwd_generic_kernel<T><<<(unsigned)M, kRowThreads, 0, st>>>(
+        X, Y, G, Bt, mean, rstd, M, (int)N, eps);
+  }
+  FFK_CHECK_LAUNCH();
+  return FFK_OK;
+}
+
+template <typename T>
+static int ln_backward(hipStream_t st, void const *dy, void const *x,
+                       float const *mean, float const *rstd, void const *gamma,
+                       void *dx, void *dgamma, void *dbeta, int64_t M, int64_t N,
+                       void *workspace, size_t workspace_bytes, bool acc) {
+  constexpr int V = VecIO<T>::kVec;
+  T const *DY = static_cast<T const *>(dy);
+  T const *X = static_cast<T const *>(x);
+  T const *G = static_cast<T const *>(gamma);
+  T *DX = static_cast<T *>(dx);
+  int ept = 0, wpr = 0;
+  bool vec = (N % V == 0) && aligned16(dy) && aligned16(x) &&
+             (dx == nullptr || aligned16(dx)) &&
+             (gamma == nullptr || aligned16(gamma)) && pick_row_config(N / V, ept, wpr);
+  if (vec) {
+    int const blocks = ln_bwd_blocks(M, wpr);
+    size_t need = (size_t)blocks * 2 * (size_t)N * sizeof(float);
+    if (workspace == nullptr || workspace_bytes < need) {
+      return fail(FFK_ERR_WORKSPACE,
+                  "layer_norm_backward: workspace of %zu bytes needed, %zu given",
+                  need, workspace_bytes);
+    }
+    float *partials = static_cast<float *>(workspace);
+#define CALL(E, W)                                                             \
+  do {                                                                         \
+    if (acc)                                                                   \
+      layer_norm_bwd_kernel<T, E, W, true><<<blocks, kRowThreads, 0, st>>>(    \
+          DY, X, mean, rstd, G, DX, partials, M, (int)N);                      \
+    else                                                                       \
+      layer_norm_bwd_kernel<T, E, W, false><<<blocks, kRowThreads, 0, st>>>(   \
+          DY, X, mean, rstd, G, DX, partials, M, (int)N);                      \
+  } while (0)
+    FFK_ROW_DISPATCH(ept, wpr, CALL);
+#undef CALL
+    FFK_CHECK_LAUNCH();
+    if (dgamma != nullptr || dbeta != nullptr) {
+      layer_norm_param_grad_final_kernel<T>
+          <<<(unsigned)ceil_div(N, 256), 256, 0, st>>>(
+              partials, blocks, (int)N, static_cast<T *>(dgamma),
+              static_cast<T *>(dbeta));
+      FFK_CHECK_LAUNCH();
+    }
+  } else {
+    if (dx != nullptr) {
+      layer_norm_bwd_generic_dx_kernel<T><<<(unsigned)M, kRowThreads, 0, st>>>(
+          DY, X, mean, rstd, G, DX, M, (int)N, acc);
+      FFK_CHECK_LAUNCH();
+    }
+    if (dgamma != nullptr || dbeta != nullptr) {
+      layer_norm_bwd_generic_param_kernel<T>
+          <<<(unsigned)ceil_div(N, 256), 256, 0, st>>>(
+              DY, X, mean, rstd, static_cast<T *>(dgamma),
+              static_cast<T *>(dbeta), M, (int)N);
+      FFK_CHECK_LAUNCH();
+    }
+  }
+  return FFK_OK;
+}
+
+}  // namespace ffk
+
+using namespace ffk;
+
+extern "C" int ffk_layer_norm_forward(ffk_stream_t stream, int dtype,
+                                      void const *input, void *output,
+                                      void const *gamma, void const *beta,
+                                      float *mean, float *rstd, int64_t M,
+                                      int64_t N, float eps) {
+  FFK_REQUIRE(M >= 0 && N > 0 && N < (1ll << 31), "layer_norm_forward: bad shape");
+  if (M == 0) return FFK_OK;
+  FFK_REQUIRE(M < (1ll << 31), "layer_norm_forward: too many rows");
+  FFK_REQUIRE(input && output && mean && rstd, "layer_norm_forward: NULL tensor");
+  if (dtype == FFK_FLOAT)
+    return ln_forward<float>(as_stream(stream), input, output, gamma, beta, mean, rstd, M, N, eps);
+  if (dtype == FFK_BF16)
+    return ln_forward<bf16>(as_stream(stream), input, output, gamma, beta, mean, rstd, M, N, eps);
+  return fail(FFK_ERR_UNSUPPORTED, "layer_norm_forward: dtype %d not supported", dtype);
+}
+
+extern "C" size_t ffk_layer_norm_backward_workspace_bytes(int64_t M, int64_t N) {
+  int64_t blocks = M < kLnBwdMaxBlocks ? M : kLnBwdMaxBlocks;
+  if (blocks < 1) blocks = 1;
+  return (size_t)blocks * 2 * (size_t)N * sizeof(float);
+}
+
+extern "C" int ffk_layer_norm_backward(
+    ffk_stream_t stream, int dtype, void const *output_grad, void const *input,
+    float const *mean, float const *rstd, void const *gamma, void *input_grad,
+    void *gamma_grad, void *beta_grad, int64_t M, int64_t N, void *workspace,
+    size_t workspace_bytes, int accumulate_input_grad) {
+  FFK_REQUIRE(M >= 0 && N > 0 && N < (1ll << 31), "layer_norm_backward: bad shape");
+  if (M == 0) return FFK_OK;
+  FFK_REQUIRE(M < (1ll << 31), "layer_norm_backward: too many rows");
+  FFK_REQUIRE(output_grad && input && mean && rstd, "layer_norm_backward: NULL tensor");
+  bool acc = accumulate_input_grad != 0;
+  if (dtype == FFK_FLOAT)
+    return ln_backward<float>(as_stream(stream), output_grad, input, mean, rstd, gamma,
+                              input_grad, gamma_grad, beta_grad, M, N, workspace,
+                              workspace_bytes, acc);
+  if (dtype == FFK_BF16)
+    return ln_backward<bf16>(as_stream(stream), output_grad, input, mean, rstd, gamma,
+                             input_grad, gamma_grad, beta_grad, M, N, workspace,
+                             workspace_bytes, acc);
+  return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: dtype %d not supported", dtype);
+}

@@ -1,0 +1,152 @@
+// Linear forward/backward for gfx950.
+//
+// forward : output = act(input . weight^T + bias), bias and activation fused
+//           into the GEMM epilogue (the reference runs a second rank-1 GEMM for
+//           the bias, lib/kernels/src/cuda/ops/linear_kernels.cu:163, and never
+//           applies the activation on the GPU, :183-200; its CPU path does,
+//           lib/kernels/src/kernels/linear_kernels_cpu.cc:33-42).
+// backward: g = act'(.) * output_grad into the caller's workspace (the
+//           reference cudaMallocs a copy of output_grad per call,
+//           lib/kernels/src/kernels/linear_kernels.cc:104-106), then three
+//           products: input_grad (+)= g . W, weight_grad (+)= g^T . X,
+//           bias_grad (+)= column sums of g (linear_kernels.cu:249-334).
+#include "elementwise.h"
+#include "gemm.h"
+
+namespace ffk {
+
+// in = (output, output_grad); out = g
+template <int ACT, int MODE>
+struct ActGrad {
+  __device__ __forceinline__ void operator()(float const (&in)[2],
+                                             float (&out)[1]) const {
+    float y = in[0], dy = in[1];
+    float g;
+    if (ACT == FFK_ACT_RELU) {
+      if (MODE == 1) {
+        g = dy > 0.0f ? 1.0f : 0.0f;  // linear_kernels_cpu.cc:46-52,69-71
+      } else {
+        g = y > 0.0f ? dy : 0.0f;     // cuda_helper.cu:60-64
+      }
+    } else if (ACT == FFK_ACT_SIGMOID) {
+      g = dy * y * (1.0f - y);        // cuda_helper.cu:87-91
+    } else {
+      g = dy * (1.0f - y * y);        // tanh
+    }
+    out[0] = g;
+  }
+};
+
+template <typename T>
+static hipError_t act_grad(hipStream_t st, int act, int mode, void const *y,
+                           void const *dy, void *g, int64_t n) {
+  EwArgs<T, 2, 1> a;
+  a.in[0] = static_cast<T const *>(y);
+  a.in[1] = static_cast<T const *>(dy);
+  a.in_elems[0] = n;
+  a.in_elems[1] = n;
+  a.out[0] = static_cast<T *>(g);
+  a.n = n;
+  if (act == FFK_ACT_RELU && mode == 1) return ew_launch<T, 2, 1>(st, a, ActGrad<FFK_ACT_RELU, 1>{});
+  if (act == FFK_ACT_RELU) return ew_launch<T, 2, 1>(st, a, ActGrad<FFK_ACT_RELU, 0>{});
+  if (act == FFK_ACT_SIGMOID) return ew_launch<T, 2, 1>(st, a, ActGrad<FFK_ACT_SIGMOID, 0>{});
+  return ew_launch<T, 2, 1>(st, a, ActGrad<FFK_ACT_TANH, 0>{});
+}
+
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+}  // namespace ffk
+
+using namespace ffk;
+
+extern "C" size_t ffk_linear_backward_workspace_bytes(int dtype, int activation,
+                                                      int use_bias,
+                                                      int64_t batch,
+                                                      int64_t out_dim) {
+  size_t bytes = 0;
+  if (activation != FFK_ACT_NONE) {
+    bytes += align256((size_t)batch * (size_t)out_dim * dtype_size(dtype));
+  }
+  if (use_bias) {
+    bytes += align256((size_t)colsum_partials_elems(batch, out_dim) * sizeof(float));
+  }
+  return bytes;
+}
+
+extern "C" int ffk_linear_forward(ffk_stream_t stream, int dtype,
+                                  int activation, void const *input,
+                                  void *output, void const *weight,
+                                  void const *bias, int64_t batch,
+                                  int64_t in_dim, int64_t out_dim) {
+  FFK_REQUIRE(dtype == FFK_FLOAT || dtype == FFK_BF16,
+              "linear_forward: dtype %d not supported", dtype);
+  FFK_REQUIRE(activation >= FFK_ACT_NONE && activation <= FFK_ACT_GELU,
+              "linear_forward: Unhandled activation function %d", activation);
+  FFK_REQUIRE(batch > 0 && in_dim > 0 && out_dim > 0,
+              "linear_forward: non-positive dimension");
+  FFK_REQUIRE(input && output && weight, "linear_forward: NULL tensor");
+  GemmEpilogue ep;
+  ep.bias = bias;
+  ep.activation = activation;
+  // output[batch,out] = input[batch,in] . weight[out,in]^T
+  return gemm_dispatch(as_stream(stream), dtype, false, true, batch, out_dim,
+                       in_dim, input, in_dim, weight, in_dim, output, out_dim, ep);
+}
+
+extern "C" int ffk_linear_backward(
+    ffk_stream_t stream, int dtype, int activation, int relu_grad_mode,
+    void const *output, void const *output_grad, void const *input,
+    void *input_grad, void const *weight, void *weight_grad, void *bias_grad,
+    int64_t batch, int64_t in_dim, int64_t out_dim, void *workspace,
+    size_t workspace_bytes, int accumulate) {
+  FFK_REQUIRE(dtype == FFK_FLOAT || dtype == FFK_BF16,
+              "linear_backward: dtype %d not supported", dtype);
+  FFK_REQUIRE(activation >= FFK_ACT_NONE && activation <= FFK_ACT_TANH,
+              "linear_backward: Unhandled activation function %d (GELU needs "
+              "the pre-activation; use an ElementUnary GELU op)",
+              activation);
+  FFK_REQUIRE(batch > 0 && in_dim > 0 && out_dim > 0,
+              "linear_backward: non-positive dimension");
+  FFK_REQUIRE(output_grad && weight && input, "linear_backward: NULL tensor");
+  hipStream_t st = as_stream(stream);
+  size_t need = ffk_linear_backward_workspace_bytes(dtype, activation,
+                                                    bias_grad != nullptr, batch, out_dim);
+  if (need > 0 && (workspace == nullptr || workspace_bytes < need)) {
+    return fail(FFK_ERR_WORKSPACE,
+                "linear_backward: workspace of %zu bytes needed, %zu given", need,
+                workspace_bytes);
+  }
+  uint8_t *ws = static_cast<uint8_t *>(workspace);
+  void const *g = output_grad;
+  if (activation != FFK_ACT_NONE) {
+    FFK_REQUIRE(output != nullptr, "linear_backward: output needed for activation");
+    int64_t n = batch * out_dim;
+    hipError_t e = dtype == FFK_FLOAT
+                       ? act_grad<float>(st, activation, relu_grad_mode, output, output_grad, ws, n)
+                       : act_grad<bf16>(st, activation, relu_grad_mode, output, output_grad, ws, n);
+    FFK_HIP(e);
+    g = ws;
+    ws += align256((size_t)n * dtype_size(dtype));
+  }
+  GemmEpilogue ep;
+  ep.accumulate = accumulate != 0;
+  int rc;
+  if (input_grad != nullptr) {
+    // input_grad[batch,in] = g[batch,out] . weight[out,in]
+    rc = gemm_dispatch(st, dtype, false, false, batch, in_dim, out_dim, g, out_dim,
+                       weight, in_dim, input_grad, in_dim, ep);
+    if (rc != FFK_OK) return rc;
+  }
+  if (weight_grad != nullptr) {
+    // weight_grad[out,in] = g[batch,out]^T . input[batch,in]
+    rc = gemm_dispatch(st, dtype, true, false, out_dim, in_dim, batch, g, out_dim,
+                       input, in_dim, weight_grad, in_dim, ep);
+    if (rc != FFK_OK) return rc;
+  }
+  if (bias_grad != nullptr) {
+    rc = colsum_dispatch(st, dtype, g, out_dim, batch, out_dim, bias_grad,
+                         accumulate != 0, reinterpret_cast<float *>(ws));
+    if (rc != FFK_OK) return rc;
+  }
+  return FFK_OK;
+}

@@ -1,0 +1,375 @@
+/*
+ * ffk.h -- C ABI of the gfx950 (MI355X) operator-kernel library libffk.so.
+ *
+ * Every function is what the reference's `Kernels::<Op>::gpu_*_kernel`
+ * (lib/kernels/include/kernels/<op>_kernels_gpu.h) does for one operator on one
+ * device, with the C++ value types flattened to plain pointers, sizes and
+ * enum ordinals so it can be bound from any host language.
+ *
+ * Conventions
+ *  - All tensor pointers are DEVICE pointers to dense row-major data (FF dim
+ *    order: dim 0 outermost, last dim contiguous; reference
+ *    lib/kernels/src/kernels/accessor.cc:15-33).
+ *  - Every call is asynchronous on `stream` (a hipStream_t passed as void*)
+ *    and never synchronises (reference: only profiling_wrapper syncs,
+ *    lib/kernels/include/kernels/profiling.h:78-106).
+ *  - Return value: FFK_OK (0) or an FFK_ERR_* code; ffk_last_error() returns
+ *    the calling thread's message. No C++ exception crosses the boundary.
+ *  - `accumulate` != 0 means the gradient output is added to (the reference
+ *    GPU path's beta = 1), 0 means it is overwritten.
+ *  - dtype arguments use the ordinals of the reference's DataType enum
+ *    (lib/op-attrs/include/op-attrs/datatype.dtg.toml:11-27) plus BF16.
+ *  - There is no CPU fallback inside this library.
+ */
+#ifndef FFK_H
+#define FFK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *ffk_stream_t; /* hipStream_t; NULL = the null stream */
+typedef void *ffk_event_t;  /* hipEvent_t */
+
+enum {
+  FFK_OK = 0,
+  FFK_ERR_INVALID = 1,     /* precondition on shapes/dtypes/pointers failed */
+  FFK_ERR_HIP = 2,         /* a HIP runtime call failed */
+  FFK_ERR_UNSUPPORTED = 3, /* combination not implemented */
+  FFK_ERR_WORKSPACE = 4    /* caller-provided workspace too small */
+};
+
+/* DataType ordinals (datatype.dtg.toml:11-27); BF16 is appended. */
+enum {
+  FFK_BOOL = 0,
+  FFK_INT32 = 1,
+  FFK_INT64 = 2,
+  FFK_HALF = 3,
+  FFK_FLOAT = 4,
+  FFK_DOUBLE = 5,
+  FFK_BF16 = 6
+};
+
+/* Activation ordinals (lib/op-attrs/include/op-attrs/activation.dtg.toml). */
+enum {
+  FFK_ACT_NONE = -1,
+  FFK_ACT_RELU = 0,
+  FFK_ACT_SIGMOID = 1,
+  FFK_ACT_TANH = 2,
+  FFK_ACT_GELU = 3
+};
+
+/* OperatorType ordinals used by the element-wise kernels
+ * (lib/op-attrs/include/op-attrs/operator_type.dtg.toml:12-94). */
+enum {
+  FFK_OP_SCALAR_MULTIPLY = 8,
+  FFK_OP_SCALAR_ADD = 9,
+  FFK_OP_SCALAR_TRUE_DIV = 11,
+  FFK_OP_SCALAR_SUB = 12,
+  FFK_OP_RELU = 13,
+  FFK_OP_IDENTITY = 14,
+  FFK_OP_SIGMOID = 15,
+  FFK_OP_TANH = 16,
+  FFK_OP_ELU = 17,
+  FFK_OP_EW_ADD = 28,
+  FFK_OP_EW_MUL = 29,
+  FFK_OP_EW_SUB = 35,
+  FFK_OP_EW_DIV = 36,
+  FFK_OP_EW_MAX = 40,
+  FFK_OP_EW_MIN = 41,
+  FFK_OP_EXP = 56,
+  FFK_OP_SIN = 61,
+  FFK_OP_COS = 62,
+  FFK_OP_GELU = 67,
+  FFK_OP_RSQRT = 70,
+  FFK_OP_POW = 71,
+  /* not a reference ordinal: GELU whose backward is the literal formula of
+   * element_unary_kernels.cu:226-231 (0.5 erfc(-x/sqrt2) - 0.5/sqrt2 x exp(-x^2/2))
+   * instead of the true derivative Phi(x) + x phi(x) */
+  FFK_OP_GELU_REFERENCE_GRAD = 1067
+};
+
+/* AggregateOp (lib/op-attrs/include/op-attrs/aggregate_op.dtg.toml). */
+enum { FFK_AGGR_NONE = -1, FFK_AGGR_SUM = 0, FFK_AGGR_AVG = 1 };
+
+/* ------------------------------------------------------------------------ */
+/* Runtime shim: the only way host C++ reaches HIP (no hip headers above it).
+ * Replaces the cudaMalloc/cudaMemcpy/cudaStreamCreate/cudaEvent* calls of
+ * lib/kernels/src/kernels/local_cuda_allocator.cc, accessor.cc:45-74,
+ * managed_ff_stream.cc and include/kernels/profiling.h:78-106.              */
+/* ------------------------------------------------------------------------ */
+char const *ffk_last_error(void);
+int ffk_device_count(int *count);
+int ffk_set_device(int device);
+int ffk_malloc(void **ptr, size_t bytes);
+int ffk_free(void *ptr);
+int ffk_host_malloc(void **ptr, size_t bytes); /* pinned host memory */
+int ffk_host_free(void *ptr);
+enum { FFK_H2D = 1, FFK_D2H = 2, FFK_D2D = 3 };
+int ffk_memcpy(void *dst, void const *src, size_t bytes, int kind,
+               ffk_stream_t stream); /* blocking when stream == NULL */
+int ffk_fill_zero(void *ptr, size_t bytes, ffk_stream_t stream);
+int ffk_stream_create(ffk_stream_t *stream);
+int ffk_stream_destroy(ffk_stream_t stream);
+int ffk_stream_synchronize(ffk_stream_t stream);
+int ffk_event_create(ffk_event_t *ev);
+int ffk_event_destroy(ffk_event_t ev);
+int ffk_event_record(ffk_event_t ev, ffk_stream_t stream);
+int ffk_event_synchronize(ffk_event_t ev);
+int ffk_event_elapsed_ms(ffk_event_t start, ffk_event_t stop, float *ms);
+
+/* ------------------------------------------------------------------------ */
+/* Linear -- replaces Kernels::Linear::gpu_forward_kernel / gpu_backward_kernel
+ * (lib/kernels/include/kernels/linear_kernels_gpu.h:22-43; CUDA body
+ * lib/kernels/src/cuda/ops/linear_kernels.cu:121-341) and computes what
+ * linear_cpu_forward_kernel / linear_cpu_backward_kernel do
+ * (lib/kernels/src/kernels/linear_kernels_cpu.cc:12-94).
+ *   input [batch,in], weight [out,in] (lib/op-attrs/src/op-attrs/ops/linear.cc:43-55),
+ *   bias [out] or NULL, output [batch,out].  dtype: FFK_FLOAT or FFK_BF16
+ *   (bf16 operands, fp32 accumulate, one rounding at the store).
+ * forward:  output = act(input . weight^T + bias)
+ * backward: g = act'(output) * output_grad; input_grad (+)= g . weight;
+ *           weight_grad (+)= g^T . input; bias_grad (+)= sum_batch g.
+ *   relu_grad_mode selects the activation gradient for RELU:
+ *     0 = g = output_grad * [output > 0]  (reference GPU, cuda_helper.cu:60-64)
+ *     1 = g = [output_grad > 0] ? 1 : 0   (reference CPU, linear_kernels_cpu.cc:46-52,65-71)
+ *   Any of input_grad / weight_grad / bias_grad may be NULL (skipped).
+ *   workspace: device scratch of ffk_linear_backward_workspace_bytes(...)
+ *   bytes (holds g when there is an activation, and the partial column sums
+ *   of the bias gradient); may be NULL when that size is 0.                  */
+/* ------------------------------------------------------------------------ */
+int ffk_linear_forward(ffk_stream_t stream, int dtype, int activation,
+                       void const *input, void *output, void const *weight,
+                       void const *bias, int64_t batch, int64_t in_dim,
+                       int64_t out_dim);
+size_t ffk_linear_backward_workspace_bytes(int dtype, int activation,
+                                           int use_bias, int64_t batch,
+                                           int64_t out_dim);
+int ffk_linear_backward(ffk_stream_t stream, int dtype, int activation,
+                        int relu_grad_mode, void const *output,
+                        void const *output_grad, void const *input,
+                        void *input_grad, void const *weight, void *weight_grad,
+                        void *bias_grad, int64_t batch, int64_t in_dim,
+                        int64_t out_dim, void *workspace,
+                        size_t workspace_bytes, int accumulate);
+
+/* General GEMM behind Linear and the attention projections:
+ *   C[M,N] (+)= op(A) . op(B)   with fp32 accumulation.
+ *   trans_a == 0: A is [M,K] row-major; 1: A is [K,M] row-major.
+ *   trans_b == 0: B is [K,N] row-major; 1: B is [N,K] row-major.
+ * Replaces the cublasGemmEx calls of linear_kernels.cu:143,249,321.          */
+int ffk_gemm(ffk_stream_t stream, int dtype, int trans_a, int trans_b,
+             int64_t M, int64_t N, int64_t K, void const *A, void const *B,
+             void *C, int accumulate);
+
+/* ------------------------------------------------------------------------ */
+/* ElementUnary -- Kernels::ElementUnary::gpu_forward_kernel/gpu_backward_kernel
+ * (element_unary_kernels_gpu.h:16-30; lib/kernels/src/cuda/ops/
+ * element_unary_kernels.cu:104-250,255-380).  `scalar` is used by the
+ * SCALAR_* / POW ops and as the ELU coefficient.
+ * backward: reference semantics per op (`+=` for most ops, `=` for GELU, POW,
+ * RSQRT) when accumulate == -1; 0/1 force overwrite/accumulate uniformly.    */
+/* ------------------------------------------------------------------------ */
+int ffk_element_unary_forward(ffk_stream_t stream, int dtype, int op_type,
+                              float scalar, void const *input, void *output,
+                              int64_t num_elements);
+int ffk_element_unary_backward(ffk_stream_t stream, int dtype, int op_type,
+                               float scalar, void const *output,
+                               void const *output_grad, void const *input,
+                               void *input_grad, int64_t num_elements,
+                               int accumulate);
+
+/* ------------------------------------------------------------------------ */
+/* ElementBinary -- Kernels::ElementBinary::gpu_forward_kernel/gpu_backward_kernel
+ * (element_binary_kernels_gpu.h:18-37; lib/kernels/src/cuda/ops/
+ * element_binary_kernels.cu:27-81,150-427).  ops: EW_ADD/SUB/MUL/DIV/MAX/MIN.
+ * lhs_elems / rhs_elems: element counts of the operands; an operand with fewer
+ * elements than the output is broadcast as a trailing-dims tensor (index
+ * i % operand_elems), which covers the bias-style broadcast the reference
+ * builds with cudnnOpTensor (element_binary_kernels.cu:171-234).             */
+/* ------------------------------------------------------------------------ */
+int ffk_element_binary_forward(ffk_stream_t stream, int dtype, int op_type,
+                               void const *lhs, void const *rhs, void *out,
+                               int64_t out_elems, int64_t lhs_elems,
+                               int64_t rhs_elems);
+int ffk_element_binary_backward(ffk_stream_t stream, int dtype, int op_type,
+                                void const *out_grad, void const *lhs,
+                                void const *rhs, void *lhs_grad, void *rhs_grad,
+                                int64_t out_elems, int accumulate);
+
+/* ------------------------------------------------------------------------ */
+/* LayerNorm -- Kernels::LayerNorm::gpu_forward_kernel / gpu_backward_kernel
+ * (layer_norm_kernels_gpu.h:19-33; lib/kernels/src/cuda/ops/
+ * layer_norm_kernels.cu:69-181,328-410).  X,Y [M,N]; gamma,beta [N] (NULL =
+ * no affine); mean,rstd [M] fp32 written by forward and read by backward
+ * (LayerNormPerDeviceState.mean/.rstd).  backward also writes dX -- the
+ * formula of LayerNormBackwardCUDAKenrel (layer_norm_kernels.cu:163-181)
+ * which the reference defines but never launches.
+ * workspace: ffk_layer_norm_backward_workspace_bytes(M, N) bytes (partial
+ * column sums for dgamma/dbeta); dgamma/dbeta are always overwritten.        */
+/* ------------------------------------------------------------------------ */
+int ffk_layer_norm_forward(ffk_stream_t stream, int dtype, void const *input,
+                           void *output, void const *gamma, void const *beta,
+                           float *mean, float *rstd, int64_t M, int64_t N,
+                           float eps);
+size_t ffk_layer_norm_backward_workspace_bytes(int64_t M, int64_t N);
+int ffk_layer_norm_backward(ffk_stream_t stream, int dtype,
+                            void const *output_grad, void const *input,
+                            float const *mean, float const *rstd,
+                            void const *gamma, void *input_grad,
+                            void *gamma_grad, void *beta_grad, int64_t M,
+                            int64_t N, void *workspace, size_t workspace_bytes,
+                            int accumulate_input_grad);
+
+/* ------------------------------------------------------------------------ */
+/* Softmax -- Kernels::Softmax::gpu_forward_kernel / gpu_backward_kernel
+ * (softmax_kernels_gpu.h:18-26; lib/kernels/src/cuda/ops/softmax_kernels.cu:
+ * 45-78).  The tensor is viewed as [outer, dim_size, inner]; softmax is taken
+ * over dim_size (cudnnSoftmaxForward ACCURATE/MODE_CHANNEL is outer = n,
+ * dim_size = c, inner = h*w).
+ * ffk_softmax_backward_copy is the reference's backward (a device copy,
+ * softmax_kernels.cu:68-78); ffk_softmax_backward is the true gradient
+ * dx = y * (dy - sum(y * dy)).                                               */
+/* ------------------------------------------------------------------------ */
+int ffk_softmax_forward(ffk_stream_t stream, int dtype, void const *input,
+                        void *output, int64_t outer, int64_t dim_size,
+                        int64_t inner);
+int ffk_softmax_backward_copy(ffk_stream_t stream, int dtype,
+                              void const *output_grad, void *input_grad,
+                              size_t num_elements);
+int ffk_softmax_backward(ffk_stream_t stream, int dtype, void const *output,
+                         void const *output_grad, void *input_grad,
+                         int64_t outer, int64_t dim_size, int64_t inner);
+
+/* ------------------------------------------------------------------------ */
+/* Dropout -- Kernels::Dropout::gpu_forward_kernel / gpu_backward_kernel
+ * (dropout_kernels_gpu.h:18-26; lib/kernels/src/cuda/ops/dropout_kernels.cu:
+ * 60-95, where the mask comes from cuDNN's opaque generator).  Here the mask
+ * is a pure function of (seed, offset + element index): Philox4x32-10 with
+ * key = (seed low 32, seed high 32), counter = ((offset+i)/4 low, high, 0, 0),
+ * word (offset+i) % 4; element i is kept iff word >= ceil(rate * 2^32);
+ * kept elements are scaled by 1/(1-rate).  No mask is stored: backward
+ * regenerates it.                                                            */
+/* ------------------------------------------------------------------------ */
+int ffk_dropout_forward(ffk_stream_t stream, int dtype, void const *input,
+                        void *output, int64_t num_elements, float rate,
+                        uint64_t seed, uint64_t offset);
+int ffk_dropout_backward(ffk_stream_t stream, int dtype,
+                         void const *output_grad, void *input_grad,
+                         int64_t num_elements, float rate, uint64_t seed,
+                         uint64_t offset, int accumulate);
+/* The keep mask itself (1 byte per element), for bit-exact checks. */
+int ffk_dropout_mask(ffk_stream_t stream, uint8_t *mask, int64_t num_elements,
+                     float rate, uint64_t seed, uint64_t offset);
+
+/* ------------------------------------------------------------------------ */
+/* Embedding -- Kernels::Embedding::gpu_forward_kernel / gpu_backward_kernel
+ * (embedding_kernels_gpu.h:10-28; lib/kernels/src/cuda/embedding_kernels.cu:
+ * 48-317,811-853).  indices [num_bags, bag] (bag == 1 with FFK_AGGR_NONE),
+ * index_dtype FFK_INT32 or FFK_INT64; weight [num_entries, dim]; output
+ * [num_bags, dim].  AVG divides the bag sum by `bag` (not the reference's
+ * scale-inside-the-loop, embedding_kernels.cu:85-98).
+ * forward:  output[b,:] = sum_j weight[indices[b,j],:]
+ * backward: weight_grad[indices[b,j],:] += output_grad[b,:] (* 1/bag for AVG),
+ *   fp32 accumulators; weight_grad is always accumulated into.
+ *   deterministic == 0: hardware fp32 atomics (order varies run to run);
+ *   deterministic == 1: rows are summed in ascending position order (bit-
+ *   reproducible); needs workspace of
+ *   ffk_embedding_backward_workspace_bytes(num_bags*bag, num_entries) bytes. */
+/* ------------------------------------------------------------------------ */
+int ffk_embedding_forward(ffk_stream_t stream, int index_dtype,
+                          int weight_dtype, int output_dtype,
+                          void const *indices, void *output,
+                          void const *weight, int aggr, int64_t num_bags,
+                          int64_t bag, int64_t dim, int64_t num_entries);
+size_t ffk_embedding_backward_workspace_bytes(int64_t num_indices,
+                                              int64_t num_entries);
+int ffk_embedding_backward(ffk_stream_t stream, int index_dtype,
+                           int output_grad_dtype, void const *indices,
+                           void const *output_grad, float *weight_grad,
+                           int aggr, int64_t num_bags, int64_t bag, int64_t dim,
+                           int64_t num_entries, int deterministic,
+                           void *workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------ */
+/* Fused (flash-style) scaled-dot-product attention core: the QK^T / softmax /
+ * PV contraction that cudnnMultiHeadAttnForward/BackwardData perform inside
+ * lib/kernels/src/cuda/ops/attention_kernels.cu:224,261, without the S x S
+ * score matrix ever reaching HBM.  dtype FFK_BF16.
+ *   q,k,v,o: element (b, s, h, d) at  b*batch_stride + s*seq_stride +
+ *   h*head_dim + d  (strides in elements), so the same kernel reads the
+ *   [batch, seq, heads*head_dim] projections and a fused QKV buffer.
+ *   lse [batch, heads, seq_q] fp32: log-sum-exp of the scaled scores, written
+ *   by forward and read by backward.  scale multiplies QK^T (the reference
+ *   uses 1.0, attention_kernels.cu:76); causal != 0 masks k > q.
+ * backward needs delta [batch, heads, seq_q] fp32 scratch (written inside).  */
+/* ------------------------------------------------------------------------ */
+typedef struct {
+  int64_t batch, heads, seq_q, seq_kv, head_dim;
+  int64_t q_batch_stride, q_seq_stride;
+  int64_t k_batch_stride, k_seq_stride;
+  int64_t v_batch_stride, v_seq_stride;
+  int64_t o_batch_stride, o_seq_stride;
+  float scale;
+  int causal;
+} ffk_attention_desc_t;
+
+int ffk_attention_forward(ffk_stream_t stream, int dtype,
+                          ffk_attention_desc_t const *desc, void const *q,
+                          void const *k, void const *v, void *o, float *lse);
+int ffk_attention_backward(ffk_stream_t stream, int dtype,
+                           ffk_attention_desc_t const *desc, void const *q,
+                           void const *k, void const *v, void const *o,
+                           void const *d_o, float const *lse, float *delta,
+                           void *dq, void *dk, void *dv);
+
+/* ------------------------------------------------------------------------ */
+/* MultiHeadAttention -- Kernels::MultiHeadAttention::gpu_forward_kernel /
+ * gpu_backward_kernel (attention_kernels_gpu.h:27-45; CUDA body
+ * lib/kernels/src/cuda/ops/attention_kernels.cu:215-303).
+ *   query [B,Sq,qSize], key [B,Skv,kSize], value [B,Skv,vSize],
+ *   output [B,Sq,oProjSize].  No bias, no dropout (attention_kernels.cu:73-92).
+ *   weight blob (defined by this library; the reference never indexes it):
+ *     [ W_Q | W_K | W_V | W_O ], W_Q = [heads*qProj, qSize] row-major with
+ *     head-major rows (likewise W_K [heads*kProj, kSize], W_V [heads*vProj,
+ *     vSize]), W_O = [oProjSize, heads*vProj] row-major.  Total element count
+ *     equals the reference's weight tensor (lib/op-attrs/src/op-attrs/ops/
+ *     attention.cc:165-185).
+ *   The reserve space (ffk_mha_reserve_bytes) holds the projected Q,K,V, the
+ *   pre-projection context and the log-sum-exp between forward and backward
+ *   plus backward scratch, like MHAPerDeviceState.reserveSpace.
+ * backward: query_grad/key_grad/value_grad are overwritten unless accumulate;
+ *   key_grad/value_grad may be NULL when key/value alias query (their
+ *   gradients are then folded into query_grad, as the reference's task impl
+ *   expects, lib/task-spec/src/task-spec/ops/impl/attention.cc:129-133);
+ *   weight_grad is accumulated into (CUDNN_WGRAD_MODE_ADD).                  */
+/* ------------------------------------------------------------------------ */
+typedef struct {
+  int64_t num_samples, num_heads;
+  int64_t q_size, k_size, v_size;
+  int64_t q_proj_size, k_proj_size, v_proj_size, o_proj_size;
+  int64_t qo_seq_length, kv_seq_length;
+  float scale; /* reference: 1.0 */
+  int causal;  /* reference: 0   */
+} ffk_mha_desc_t;
+
+size_t ffk_mha_weight_elements(ffk_mha_desc_t const *desc);
+size_t ffk_mha_reserve_bytes(ffk_mha_desc_t const *desc, int dtype);
+int ffk_mha_forward(ffk_stream_t stream, int dtype, ffk_mha_desc_t const *desc,
+                    void const *query, void const *key, void const *value,
+                    void const *weight, void *output, void *reserve,
+                    size_t reserve_bytes);
+int ffk_mha_backward(ffk_stream_t stream, int dtype, ffk_mha_desc_t const *desc,
+                     void const *query, void *query_grad, void const *key,
+                     void *key_grad, void const *value, void *value_grad,
+                     void const *weight, void *weight_grad,
+                     void const *output_grad, void *reserve,
+                     size_t reserve_bytes, int accumulate);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FFK_H */

@@ -1,0 +1,353 @@
+"""ctypes binding of the CPU oracle (oracle/libffk_oracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the
+CPU-baseline leg of bench.py.  The product package never imports this module.
+Arrays are numpy float32 (C-contiguous) unless stated.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libffk_oracle.so")
+_lib = None
+
+c_i64 = ctypes.c_int64
+c_f = ctypes.c_float
+c_int = ctypes.c_int
+c_u64 = ctypes.c_uint64
+c_p = ctypes.c_void_p
+
+
+def build():
+    subprocess.run(["make", "-C", _HERE, "-B"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+class MHADesc(ctypes.Structure):
+    _fields_ = [
+        ("num_samples", c_i64), ("num_heads", c_i64),
+        ("q_size", c_i64), ("k_size", c_i64), ("v_size", c_i64),
+        ("q_proj_size", c_i64), ("k_proj_size", c_i64), ("v_proj_size", c_i64),
+        ("o_proj_size", c_i64),
+        ("qo_seq_length", c_i64), ("kv_seq_length", c_i64),
+        ("scale", c_f), ("causal", c_int),
+    ]
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.orc_round_bf16.restype = c_f
+        _lib.orc_round_bf16.argtypes = [c_f]
+        _lib.orc_offset.restype = c_i64
+    return _lib
+
+
+def _f32(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(c_p)
+
+
+def round_bf16(a):
+    a = _f32(a).copy()
+    lib().orc_round_bf16_array(_p(a), c_i64(a.size))
+    return a
+
+
+def offset(dims, coord):
+    d = np.asarray(dims, dtype=np.int64)
+    c = np.asarray(coord, dtype=np.int64)
+    return int(lib().orc_offset(_p(d), c_int(len(d)), _p(c)))
+
+
+def matmul(lhs, rhs):
+    lhs, rhs = _f32(lhs), _f32(rhs)
+    M, K = lhs.shape
+    K2, N = rhs.shape
+    assert K == K2
+    out = np.empty((M, N), np.float32)
+    lib().orc_matmul(_p(lhs), _p(rhs), _p(out), c_i64(M), c_i64(K), c_i64(N))
+    return out
+
+
+def transpose(a):
+    a = _f32(a)
+    out = np.empty((a.shape[1], a.shape[0]), np.float32)
+    lib().orc_transpose(_p(a), _p(out), c_i64(a.shape[0]), c_i64(a.shape[1]))
+    return out
+
+
+def broadcast(a, out_dims):
+    a = _f32(a)
+    ind = np.asarray(a.shape, dtype=np.int64)
+    outd = np.asarray(out_dims, dtype=np.int64)
+    out = np.empty(tuple(out_dims), np.float32)
+    lib().orc_broadcast(_p(a), _p(ind), c_int(a.ndim), _p(out), _p(outd), c_int(len(outd)))
+    return out
+
+
+def reduce_dim(a, dim):
+    a = _f32(a)
+    d = np.asarray(a.shape, dtype=np.int64)
+    out_shape = a.shape[:dim] + a.shape[dim + 1:]
+    out = np.empty(out_shape, np.float32)
+    lib().orc_reduce_dim(_p(a), _p(d), c_int(a.ndim), c_int(dim), _p(out))
+    return out
+
+
+def relu(a):
+    a = _f32(a)
+    out = np.empty_like(a)
+    lib().orc_relu(_p(a), _p(out), c_i64(a.size))
+    return out
+
+
+def scale(a, c):
+    a = _f32(a)
+    out = np.empty_like(a)
+    lib().orc_scale(_p(a), c_f(c), _p(out), c_i64(a.size))
+    return out
+
+
+def linear_forward(x, w, b=None, activation=-1):
+    x, w = _f32(x), _f32(w)
+    b = None if b is None else _f32(b)
+    batch, in_dim = x.shape
+    out_dim = w.shape[0]
+    y = np.empty((batch, out_dim), np.float32)
+    rc = lib().orc_linear_forward(c_int(activation), _p(x), _p(y), _p(w), _p(b),
+                                  c_i64(batch), c_i64(in_dim), c_i64(out_dim))
+    if rc:
+        raise ValueError("Unhandled activation function")
+    return y
+
+
+def linear_backward(y, dy, x, w, activation=-1, relu_grad_mode=0, use_bias=True):
+    y, dy, x, w = _f32(y), _f32(dy), _f32(x), _f32(w)
+    batch, in_dim = x.shape
+    out_dim = w.shape[0]
+    dx = np.empty_like(x)
+    dw = np.empty_like(w)
+    db = np.empty((out_dim,), np.float32) if use_bias else None
+    rc = lib().orc_linear_backward(c_int(activation), c_int(relu_grad_mode), _p(y), _p(dy),
+                                   _p(x), _p(dx), _p(w), _p(dw), _p(db),
+                                   c_i64(batch), c_i64(in_dim), c_i64(out_dim))
+    if rc:
+        raise ValueError("Unhandled activation function")
+    return dx, dw, db
+
+
+def gemm_f64(A, B, trans_a=False, trans_b=False):
+    A, B = _f32(A), _f32(B)
+    M = A.shape[1] if trans_a else A.shape[0]
+    K = A.shape[0] if trans_a else A.shape[1]
+    N = B.shape[0] if trans_b else B.shape[1]
+    C = np.empty((M, N), np.float32)
+    lib().orc_gemm_f64(c_int(int(trans_a)), c_int(int(trans_b)), c_i64(M), c_i64(N), c_i64(K),
+                       _p(A), _p(B), _p(C))
+    return C
+
+
+def element_unary_forward(op, x, scalar=0.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    rc = lib().orc_element_unary_forward(c_int(op), c_f(scalar), _p(x), _p(y), c_i64(x.size))
+    if rc:
+        raise ValueError("unhandled unary op %d" % op)
+    return y
+
+
+def element_unary_backward(op, y, dy, x, dx_init=None, scalar=0.0, accumulate=-1):
+    y, dy, x = _f32(y), _f32(dy), _f32(x)
+    dx = np.zeros_like(x) if dx_init is None else _f32(dx_init).copy()
+    rc = lib().orc_element_unary_backward(c_int(op), c_f(scalar), _p(y), _p(dy), _p(x), _p(dx),
+                                          c_i64(x.size), c_int(accumulate))
+    if rc:
+        raise ValueError("unhandled unary op %d" % op)
+    return dx
+
+
+def element_binary_forward(op, l, r, out_shape=None):
+    l, r = _f32(l), _f32(r)
+    shape = out_shape if out_shape is not None else (l.shape if l.size >= r.size else r.shape)
+    out = np.empty(shape, np.float32)
+    rc = lib().orc_element_binary_forward(c_int(op), _p(l), _p(r), _p(out), c_i64(out.size),
+                                          c_i64(l.size), c_i64(r.size))
+    if rc:
+        raise ValueError("unhandled binary op %d" % op)
+    return out
+
+
+def element_binary_backward(op, g, l, r, dl_init=None, dr_init=None, accumulate=0):
+    g, l, r = _f32(g), _f32(l), _f32(r)
+    dl = np.zeros_like(g) if dl_init is None else _f32(dl_init).copy()
+    dr = np.zeros_like(g) if dr_init is None else _f32(dr_init).copy()
+    rc = lib().orc_element_binary_backward(c_int(op), _p(g), _p(l), _p(r), _p(dl), _p(dr),
+                                           c_i64(g.size), c_int(accumulate))
+    if rc:
+        raise ValueError("unhandled binary op %d" % op)
+    return dl, dr
+
+
+def layer_norm_forward(x, gamma, beta, eps):
+    x = _f32(x)
+    M, N = x.shape
+    gamma = None if gamma is None else _f32(gamma)
+    beta = None if beta is None else _f32(beta)
+    y = np.empty_like(x)
+    mean = np.empty((M,), np.float32)
+    rstd = np.empty((M,), np.float32)
+    lib().orc_layer_norm_forward(_p(x), _p(y), _p(gamma), _p(beta), _p(mean), _p(rstd),
+                                 c_i64(M), c_i64(N), c_f(eps))
+    return y, mean, rstd
+
+
+def layer_norm_backward(dy, x, mean, rstd, gamma, dx_init=None):
+    dy, x, mean, rstd = _f32(dy), _f32(x), _f32(mean), _f32(rstd)
+    M, N = x.shape
+    gamma = None if gamma is None else _f32(gamma)
+    dx = np.zeros_like(x) if dx_init is None else _f32(dx_init).copy()
+    dg = np.empty((N,), np.float32)
+    db = np.empty((N,), np.float32)
+    lib().orc_layer_norm_backward(_p(dy), _p(x), _p(mean), _p(rstd), _p(gamma), _p(dx), _p(dg),
+                                  _p(db), c_i64(M), c_i64(N), c_int(0 if dx_init is None else 1))
+    return dx, dg, db
+
+
+def softmax_forward(x, outer, dim, inner):
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().orc_softmax_forward(_p(x), _p(y), c_i64(outer), c_i64(dim), c_i64(inner))
+    return y
+
+
+def softmax_backward(y, dy, outer, dim, inner):
+    y, dy = _f32(y), _f32(dy)
+    dx = np.empty_like(y)
+    lib().orc_softmax_backward(_p(y), _p(dy), _p(dx), c_i64(outer), c_i64(dim), c_i64(inner))
+    return dx
+
+
+def philox4x32_10(ctr, key):
+    c = np.asarray(ctr, dtype=np.uint32)
+    k = np.asarray(key, dtype=np.uint32)
+    out = np.empty((4,), np.uint32)
+    lib().orc_philox4x32_10(_p(c), _p(k), _p(out))
+    return out
+
+
+def dropout_mask(n, rate, seed, offset=0):
+    m = np.empty((n,), np.uint8)
+    lib().orc_dropout_mask(_p(m), c_i64(n), c_f(rate), c_u64(seed), c_u64(offset))
+    return m
+
+
+def dropout_forward(x, rate, seed, offset=0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().orc_dropout_forward(_p(x), _p(y), c_i64(x.size), c_f(rate), c_u64(seed), c_u64(offset))
+    return y
+
+
+def dropout_backward(dy, rate, seed, offset=0, dx_init=None):
+    dy = _f32(dy)
+    dx = np.zeros_like(dy) if dx_init is None else _f32(dx_init).copy()
+    lib().orc_dropout_backward(_p(dy), _p(dx), c_i64(dy.size), c_f(rate), c_u64(seed),
+                               c_u64(offset), c_int(0 if dx_init is None else 1))
+    return dx
+
+
+def embedding_forward(indices, weight, aggr=-1):
+    idx = np.ascontiguousarray(indices, dtype=np.int64)
+    weight = _f32(weight)
+    if idx.ndim == 1:
+        idx2 = idx.reshape(-1, 1)
+    else:
+        idx2 = idx.reshape(-1, idx.shape[-1]) if aggr >= 0 else idx.reshape(-1, 1)
+    num_bags, bag = idx2.shape
+    V, D = weight.shape
+    out = np.empty((num_bags, D), np.float32)
+    rc = lib().orc_embedding_forward(_p(idx2), _p(out), _p(weight), c_int(aggr), c_i64(num_bags),
+                                     c_i64(bag), c_i64(D), c_i64(V))
+    if rc:
+        raise ValueError("embedding_forward failed rc=%d" % rc)
+    return out
+
+
+def embedding_backward(indices, out_grad, num_entries, aggr=-1, f64=False, dw_init=None):
+    idx = np.ascontiguousarray(indices, dtype=np.int64)
+    g = _f32(out_grad)
+    if idx.ndim == 1 or aggr < 0:
+        idx2 = idx.reshape(-1, 1)
+    else:
+        idx2 = idx.reshape(-1, idx.shape[-1])
+    num_bags, bag = idx2.shape
+    D = g.shape[-1]
+    dw = np.zeros((num_entries, D), np.float32) if dw_init is None else _f32(dw_init).copy()
+    fn = lib().orc_embedding_backward_f64 if f64 else lib().orc_embedding_backward
+    rc = fn(_p(idx2), _p(g), _p(dw), c_int(aggr), c_i64(num_bags), c_i64(bag), c_i64(D),
+            c_i64(num_entries))
+    if rc:
+        raise ValueError("embedding_backward failed rc=%d" % rc)
+    return dw
+
+
+def attention_forward(q, k, v, scale, causal, bf16_mode=False):
+    """q [B,Sq,H,D], k/v [B,Skv,H,D] -> o [B,Sq,H,D], lse [B,H,Sq]."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    B, Sq, H, D = q.shape
+    Skv = k.shape[1]
+    o = np.empty_like(q)
+    lse = np.empty((B, H, Sq), np.float32)
+    lib().orc_attention_forward(_p(q), _p(k), _p(v), _p(o), _p(lse), c_i64(B), c_i64(H),
+                                c_i64(Sq), c_i64(Skv), c_i64(D), c_f(scale), c_int(int(causal)),
+                                c_int(int(bf16_mode)))
+    return o, lse
+
+
+def attention_backward(q, k, v, d_o, scale, causal):
+    q, k, v, d_o = _f32(q), _f32(k), _f32(v), _f32(d_o)
+    B, Sq, H, D = q.shape
+    Skv = k.shape[1]
+    dq = np.empty_like(q)
+    dk = np.empty_like(k)
+    dv = np.empty_like(v)
+    lib().orc_attention_backward(_p(q), _p(k), _p(v), _p(d_o), _p(dq), _p(dk), _p(dv), c_i64(B),
+                                 c_i64(H), c_i64(Sq), c_i64(Skv), c_i64(D), c_f(scale),
+                                 c_int(int(causal)))
+    return dq, dk, dv
+
+
+def mha_desc(num_samples, num_heads, q_size, k_size, v_size, q_proj, k_proj, v_proj, o_proj,
+             sq, skv, scale=1.0, causal=False):
+    return MHADesc(num_samples, num_heads, q_size, k_size, v_size, q_proj, k_proj, v_proj, o_proj,
+                   sq, skv, scale, int(causal))
+
+
+def mha_forward(desc, query, key, value, weight, bf16_mode=False):
+    query, key, value, weight = _f32(query), _f32(key), _f32(value), _f32(weight)
+    out = np.empty((desc.num_samples, desc.qo_seq_length, desc.o_proj_size), np.float32)
+    lib().orc_mha_forward(ctypes.byref(desc), _p(query), _p(key), _p(value), _p(weight), _p(out),
+                          c_int(int(bf16_mode)))
+    return out
+
+
+def mha_backward(desc, query, key, value, weight, out_grad, bf16_mode=False):
+    query, key, value, weight, out_grad = map(_f32, (query, key, value, weight, out_grad))
+    dq = np.empty_like(query)
+    dk = np.empty_like(key)
+    dv = np.empty_like(value)
+    dw = np.zeros_like(weight)
+    lib().orc_mha_backward(ctypes.byref(desc), _p(query), _p(key), _p(value), _p(weight),
+                           _p(out_grad), _p(dq), _p(dk), _p(dv), _p(dw), c_int(int(bf16_mode)))
+    return dq, dk, dv, dw

@@ -1,0 +1,100 @@
+"""Embedding gather / scatter-add parity against the oracle."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from util import BF16_RTOL, FP32_RTOL, assert_close, bf16_round, rng, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def zipf_ids(g, n, vocab, s=1.1):
+    """Zipf(s) over [0, vocab) by inverse CDF."""
+    p = 1.0 / np.arange(1, vocab + 1) ** s
+    cdf = np.cumsum(p / p.sum())
+    return np.minimum(np.searchsorted(cdf, g.random(n)), vocab - 1)
+
+
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+@pytest.mark.parametrize("wdt,odt", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                     (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("V,D,n", [(10, 4, 7), (1000, 128, 513), (50257, 1024, 4096), (97, 33, 50)])
+def test_gather_bit_exact(ffk, oracle, idt, wdt, odt, V, D, n):
+    say("embedding gather", idt, wdt, odt, (V, D, n))
+    g = rng(V + D)
+    w = (g.standard_normal((V, D)) * 0.02).astype(np.float32)
+    if wdt == torch.bfloat16:
+        w = bf16_round(w)
+    ids = zipf_ids(g, n, V)
+    want = oracle.embedding_forward(ids, w)
+    if odt == torch.bfloat16:
+        want = bf16_round(want)
+    out = ffk.embedding_forward(to_dev(ids, torch, idt), to_dev(w, torch, wdt), out_dtype=odt)
+    assert np.array_equal(to_np(out), want)   # a gather is a copy: bit-exact
+
+
+@pytest.mark.parametrize("aggr", [0, 1])
+@pytest.mark.parametrize("V,D,B,bag", [(1000, 128, 64, 32), (100, 16, 9, 5), (5000, 128, 1024, 32), (50, 7, 3, 1)])
+def test_bag_forward(ffk, oracle, aggr, V, D, B, bag):
+    say("embedding bag fwd", aggr, (V, D, B, bag))
+    g = rng(B + bag)
+    w = g.standard_normal((V, D)).astype(np.float32)
+    ids = zipf_ids(g, B * bag, V).reshape(B, bag)
+    want = oracle.embedding_forward(ids, w, aggr=aggr)
+    out = ffk.embedding_forward(to_dev(ids, torch, torch.int64), to_dev(w, torch), aggr=aggr)
+    # same left-to-right fp32 summation order as the oracle: bit-exact
+    assert np.array_equal(to_np(out), want)
+
+
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V,D,n", [(10, 4, 7), (1000, 128, 2000), (50257, 1024, 2048), (97, 33, 50)])
+def test_scatter_add(ffk, oracle, gdt, V, D, n):
+    say("embedding scatter-add", gdt, (V, D, n))
+    g = rng(V * 3 + n)
+    ids = zipf_ids(g, n, V)
+    dy = g.standard_normal((n, D)).astype(np.float32)
+    if gdt == torch.bfloat16:
+        dy = bf16_round(dy)
+    dw0 = g.standard_normal((V, D)).astype(np.float32)
+    want = oracle.embedding_backward(ids, dy, V, f64=True, dw_init=dw0)
+    dw = to_dev(dw0, torch)
+    ffk.embedding_backward(to_dev(ids, torch, torch.int32), to_dev(dy, torch, gdt), dw)
+    # fp32 atomics: order-dependent rounding, checked against the fp64 sum
+    assert_close(to_np(dw), want, FP32_RTOL, "dW")
+
+
+@pytest.mark.parametrize("aggr", [0, 1])
+def test_bag_backward(ffk, oracle, aggr):
+    V, D, B, bag = 2000, 128, 256, 32
+    say("embedding bag bwd", aggr)
+    g = rng(5)
+    ids = zipf_ids(g, B * bag, V).reshape(B, bag)
+    dy = g.standard_normal((B, D)).astype(np.float32)
+    want = oracle.embedding_backward(ids, dy, V, aggr=aggr, f64=True)
+    dw = torch.zeros((V, D), device="cuda")
+    ffk.embedding_backward(to_dev(ids, torch, torch.int64), to_dev(dy, torch), dw, aggr=aggr)
+    assert_close(to_np(dw), want, FP32_RTOL, "dW")
+
+
+def test_out_of_range_ids_are_skipped_and_errors(ffk):
+    say("embedding invalid ids")
+    w = torch.ones((10, 8), device="cuda")
+    ids = torch.tensor([1, 10, -1, 3], dtype=torch.int64, device="cuda")
+    out = ffk.embedding_forward(ids, w)
+    assert out[0].sum() == 8 and out[1].sum() == 0 and out[2].sum() == 0 and out[3].sum() == 8
+    dw = torch.zeros((10, 8), device="cuda")
+    ffk.embedding_backward(ids, torch.ones((4, 8), device="cuda"), dw)
+    assert dw.sum() == 16
+    with pytest.raises(ffk.FFKError, match="bag must be 1"):
+        ffk.check(ffk.lib().ffk_embedding_forward(0, ffk.INT64, ffk.FLOAT, ffk.FLOAT, ids.data_ptr(),
+                                                  out.data_ptr(), w.data_ptr(), ffk.AGGR_NONE, 2, 2, 8, 10))
+    # empty input is a no-op
+    ffk.check(ffk.lib().ffk_embedding_forward(0, ffk.INT64, ffk.FLOAT, ffk.FLOAT, None, None, None,
+                                              ffk.AGGR_NONE, 0, 1, 8, 10))

@@ -1,0 +1,168 @@
+"""Linear / GEMM parity: HIP kernels through the C ABI against the oracle."""
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from util import BF16_RTOL, FP32_RTOL, assert_close, bf16_round, rng, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def test_linear_reference_kat_fp32(ffk, golden_dir):
+    k = json.load(open(os.path.join(golden_dir, "linear_kat.json")))
+    say("linear KAT 4x3 . 3x2 fp32")
+    x = to_dev(np.array(k["input"], np.float32), torch)
+    w = to_dev(np.array(k["projection"], np.float32), torch)
+    b = to_dev(np.array(k["bias"], np.float32), torch)
+    y = ffk.linear_forward(x, w, b)
+    assert np.array_equal(to_np(y), np.array(k["output"], np.float32))
+    dy = to_dev(np.array(k["output_grad"], np.float32), torch)
+    dx, dw, db = torch.zeros_like(x), torch.zeros_like(w), torch.zeros_like(b)
+    ffk.linear_backward(y, dy, x, w, dx, dw, db)
+    assert np.array_equal(to_np(dx), np.array(k["input_grad"], np.float32))
+    assert np.array_equal(to_np(dw), np.array(k["projection_grad"], np.float32))
+    assert np.array_equal(to_np(db), np.array(k["bias_grad"], np.float32))
+
+
+def _cfg1_inputs(seed=0, batch=32, in_dim=64, out_dim=128):
+    g = rng(seed)
+    x = g.uniform(-1, 1, (batch, in_dim)).astype(np.float32)
+    w = (g.standard_normal((out_dim, in_dim)) * 0.02).astype(np.float32)
+    b = (g.standard_normal((out_dim,)) * 0.02).astype(np.float32)
+    dy = g.standard_normal((batch, out_dim)).astype(np.float32)
+    return x, w, b, dy
+
+
+@pytest.mark.parametrize("relu_grad_mode", [0, 1])
+def test_linear_config1_fp32_relu(ffk, oracle, relu_grad_mode):
+    """BASELINE config 1: fp32 [32,64] . [128,64]^T + bias, ReLU; both readings
+    of the ReLU gradient (reference GPU helper / reference CPU text)."""
+    x, w, b, dy = _cfg1_inputs()
+    say("linear cfg1 fp32 relu mode", relu_grad_mode)
+    y_ref = oracle.linear_forward(x, w, b, activation=0)
+    dx_ref, dw_ref, db_ref = oracle.linear_backward(y_ref, dy, x, w, activation=0,
+                                                    relu_grad_mode=relu_grad_mode)
+    xd, wd, bd, dyd = (to_dev(a, torch) for a in (x, w, b, dy))
+    y = ffk.linear_forward(xd, wd, bd, activation=ffk.ACT_RELU)
+    assert_close(to_np(y), y_ref, FP32_RTOL, "y")
+    dx, dw, db = torch.zeros_like(xd), torch.zeros_like(wd), torch.zeros_like(bd)
+    ffk.linear_backward(y, dyd, xd, wd, dx, dw, db, activation=ffk.ACT_RELU,
+                        relu_grad_mode=relu_grad_mode)
+    assert_close(to_np(dx), dx_ref, FP32_RTOL, "dx")
+    assert_close(to_np(dw), dw_ref, FP32_RTOL, "dw")
+    assert_close(to_np(db), db_ref, FP32_RTOL, "db")
+    # accumulate (reference GPU beta = 1): a second call doubles the gradients
+    ffk.linear_backward(y, dyd, xd, wd, dx, dw, db, activation=ffk.ACT_RELU,
+                        relu_grad_mode=relu_grad_mode, accumulate=True)
+    assert_close(to_np(dx), 2 * dx_ref, FP32_RTOL, "dx acc")
+    assert_close(to_np(dw), 2 * dw_ref, FP32_RTOL, "dw acc")
+    assert_close(to_np(db), 2 * db_ref, FP32_RTOL, "db acc")
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 3, 7), (33, 65, 129), (70, 17, 64), (128, 256, 96)])
+@pytest.mark.parametrize("act", [-1, 0, 1, 2])
+def test_linear_fp32_ragged(ffk, oracle, shape, act):
+    batch, in_dim, out_dim = shape
+    say("linear fp32 ragged", shape, "act", act)
+    x, w, b, dy = _cfg1_inputs(seed=batch * 1000 + in_dim, batch=batch, in_dim=in_dim, out_dim=out_dim)
+    w = w * 20
+    y_ref = oracle.linear_forward(x, w, b, activation=act)
+    dx_ref, dw_ref, db_ref = oracle.linear_backward(y_ref, dy, x, w, activation=act)
+    xd, wd, bd, dyd = (to_dev(a, torch) for a in (x, w, b, dy))
+    y = ffk.linear_forward(xd, wd, bd, activation=act)
+    assert_close(to_np(y), y_ref, FP32_RTOL, "y")
+    dx, dw, db = torch.zeros_like(xd), torch.zeros_like(wd), torch.zeros_like(bd)
+    ffk.linear_backward(to_dev(y_ref, torch), dyd, xd, wd, dx, dw, db, activation=act)
+    assert_close(to_np(dx), dx_ref, FP32_RTOL, "dx")
+    assert_close(to_np(dw), dw_ref, FP32_RTOL, "dw")
+    assert_close(to_np(db), db_ref, FP32_RTOL, "db")
+
+
+def test_linear_no_bias_and_skipped_grads(ffk, oracle):
+    x, w, b, dy = _cfg1_inputs(seed=5, batch=16, in_dim=24, out_dim=40)
+    say("linear fp32 no bias / NULL grads")
+    y_ref = oracle.linear_forward(x, w, None)
+    xd, wd, dyd = (to_dev(a, torch) for a in (x, w, dy))
+    y = ffk.linear_forward(xd, wd, None)
+    assert_close(to_np(y), y_ref, FP32_RTOL, "y")
+    dx_ref, dw_ref, _ = oracle.linear_backward(y_ref, dy, x, w, use_bias=False)
+    dw = torch.zeros_like(wd)
+    ffk.linear_backward(y, dyd, xd, wd, None, dw, None)
+    assert_close(to_np(dw), dw_ref, FP32_RTOL, "dw")
+    dx = torch.zeros_like(xd)
+    ffk.linear_backward(y, dyd, xd, wd, dx, None, None)
+    assert_close(to_np(dx), dx_ref, FP32_RTOL, "dx")
+
+
+def test_linear_errors(ffk):
+    x = torch.zeros((4, 4), device="cuda")
+    with pytest.raises(ffk.FFKError, match="Unhandled activation"):
+        ffk.linear_forward(x, x, None, activation=9)
+    with pytest.raises(ffk.FFKError, match="workspace"):
+        ffk.check(ffk.lib().ffk_linear_backward(0, ffk.FLOAT, ffk.ACT_RELU, 0, x.data_ptr(), x.data_ptr(),
+                                                x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), None,
+                                                4, 4, 4, None, 0, 0))
+
+
+@pytest.mark.parametrize("trans_a,trans_b", [(False, True), (False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("mnk", [(128, 128, 64), (256, 384, 192), (64, 64, 64), (200, 72, 40), (8, 8, 8),
+                                 (130, 258, 136), (512, 1024, 256)])
+def test_gemm_bf16(ffk, oracle, trans_a, trans_b, mnk):
+    M, N, K = mnk
+    say("gemm bf16", mnk, "ta", trans_a, "tb", trans_b)
+    g = rng(M * 7 + N * 3 + K)
+    A = bf16_round(g.standard_normal((K, M) if trans_a else (M, K)))
+    B = bf16_round(g.standard_normal((N, K) if trans_b else (K, N)))
+    want = oracle.gemm_f64(A, B, trans_a, trans_b)
+    Ad, Bd = to_dev(A, torch, torch.bfloat16), to_dev(B, torch, torch.bfloat16)
+    C = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    ffk.gemm(Ad, Bd, C, trans_a, trans_b)
+    # exact products, fp32 accumulation, one bf16 rounding at the store
+    assert_close(to_np(C), want, 2.0 ** -8, "C")
+    C0 = bf16_round(g.standard_normal((M, N)))
+    Cd = to_dev(C0, torch, torch.bfloat16)
+    ffk.gemm(Ad, Bd, Cd, trans_a, trans_b, accumulate=True)
+    assert_close(to_np(Cd), want + C0, 2.0 ** -7, "C accumulate")
+
+
+@pytest.mark.parametrize("mnk", [(7, 5, 3), (33, 9, 12), (16, 24, 20)])
+def test_gemm_bf16_unaligned_shapes_take_the_plain_kernel(ffk, oracle, mnk):
+    M, N, K = mnk
+    say("gemm bf16 unaligned", mnk)
+    g = rng(99)
+    A = bf16_round(g.standard_normal((M, K)))
+    B = bf16_round(g.standard_normal((N, K)))
+    want = oracle.gemm_f64(A, B, False, True)
+    C = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    ffk.gemm(to_dev(A, torch, torch.bfloat16), to_dev(B, torch, torch.bfloat16), C, False, True)
+    assert_close(to_np(C), want, 2.0 ** -8, "C")
+
+
+@pytest.mark.parametrize("act", [-1, 0])
+def test_linear_bf16(ffk, oracle, act):
+    batch, in_dim, out_dim = 256, 192, 384
+    say("linear bf16", (batch, in_dim, out_dim), "act", act)
+    g = rng(21)
+    x = bf16_round(g.standard_normal((batch, in_dim)))
+    w = bf16_round(g.standard_normal((out_dim, in_dim)) * 0.05)
+    b = bf16_round(g.standard_normal((out_dim,)) * 0.05)
+    dy = bf16_round(g.standard_normal((batch, out_dim)))
+    y_ref = bf16_round(oracle.linear_forward(x, w, b, activation=act))
+    xd, wd, bd, dyd = (to_dev(a, torch, torch.bfloat16) for a in (x, w, b, dy))
+    y = ffk.linear_forward(xd, wd, bd, activation=act)
+    assert_close(to_np(y), y_ref, BF16_RTOL, "y")
+    dx_ref, dw_ref, db_ref = oracle.linear_backward(to_np(y), dy, x, w, activation=act)
+    dx, dw, db = torch.zeros_like(xd), torch.zeros_like(wd), torch.zeros_like(bd)
+    ffk.linear_backward(y, dyd, xd, wd, dx, dw, db, activation=act)
+    assert_close(to_np(dx), dx_ref, BF16_RTOL, "dx")
+    assert_close(to_np(dw), dw_ref, BF16_RTOL, "dw")
+    assert_close(to_np(db), db_ref, BF16_RTOL, "db")
