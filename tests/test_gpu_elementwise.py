@@ -103,7 +103,7 @@ def test_binary_broadcast_rhs(ffk, oracle, dtype):
         l, r = bf16_round(l), bf16_round(r)
     out = ffk.element_binary_forward(ffk.OP["EW_ADD"], to_dev(l, torch, tdt), to_dev(r, torch, tdt))
     assert_close(to_np(out), oracle.element_binary_forward(ffk.OP["EW_ADD"], l, r, l.shape), rtol, "bcast")
-    r5 = r[:5].copy()  # 48 % 5 != 0: not broadcastable
+    r5 = r[:7].copy()  # 65 * 48 is not a multiple of 7: not broadcastable
     with pytest.raises(ffk.FFKError, match="broadcast"):
         ffk.element_binary_forward(ffk.OP["EW_ADD"], to_dev(l, torch, tdt), to_dev(r5, torch, tdt),
                                    out=torch.empty((65, 48), dtype=tdt, device="cuda"))
