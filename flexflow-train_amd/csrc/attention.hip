@@ -1,0 +1,676 @@
+// Fused (flash-style) attention for gfx950, bf16 operands / fp32 accumulation.
+//
+// The reference hands Q, K, V to cudnnMultiHeadAttnForward / BackwardData
+// (lib/kernels/src/cuda/ops/attention_kernels.cu:224,261), which materialise
+// the seq x seq score matrix.  Here scores never leave the CU:
+//
+//  forward   one workgroup = 128 query rows of one (batch, head); each of its
+//            4 wavefronts owns 32 rows.  Scores are computed transposed,
+//            S^T = K Q^T, so that a lane owns one query row's column of the
+//            MFMA accumulator: the running max / sum are lane-local and the
+//            probabilities feed the P V product straight from registers.
+//            V is staged in LDS as it lies in memory and read with the
+//            transposing LDS load.
+//  backward  two kernels, no atomics, deterministic:
+//            (A) one workgroup = 128 key/value rows, loops over query tiles and
+//                accumulates dK, dV in registers;
+//            (B) one workgroup = 128 query rows, loops over key tiles and
+//                accumulates dQ in registers.
+//            Both recompute P from the saved log-sum-exp.
+//
+// MFMA 32x32x16 bf16 register layouts used throughout (l = lane):
+//   A operand: row l%32, k = 8*(l/32) .. +7      B operand: column l%32, same k
+//   accumulator element r: row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+// When an accumulator tile is re-used as an operand of the next product, its
+// 8 values r = 8s .. 8s+7 are taken as the k-slots of step s; the other operand
+// is then loaded with the same permutation of the reduction index, which the
+// transposing load does for free.
+#include "ffk_common.h"
+
+namespace ffk {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+
+struct AttnParams {
+  bf16 const *q, *k, *v;
+  bf16 *o;
+  float *lse;
+  int B, H, Sq, Skv;
+  int64_t q_bs, q_ss, k_bs, k_ss, v_bs, v_ss, o_bs, o_ss;
+  float scale_log2;  // scale * log2(e)
+  int causal;
+};
+
+__device__ __forceinline__ bf16x8 pack8(float const *v) {
+  union {
+    uint32_t u[4];
+    bf16x8 b;
+  } x;
+#pragma unroll
+  for (int i = 0; i < 4; i++) x.u[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+  return x.b;
+}
+
+// B- or A-operand fragment from a row-major LDS tile whose rows are the
+// operand's rows/columns and whose contiguous dim is the reduction dim.
+__device__ __forceinline__ bf16x8 frag_k(bf16 const *tile, int stride, int row0,
+                                         int k0, int lane) {
+  return *reinterpret_cast<bf16x8 const *>(tile + (row0 + (lane & 31)) * stride +
+                                           k0 + (lane >> 5) * 8);
+}
+
+// Fragment from an LDS tile stored [reduction index][row/column index]
+// (contiguous along the operand's non-reduction dim), using the reduction
+// order of an accumulator re-used as the other operand: k-slot (h, j) of step
+// s is tile row  r0 + 16 s + 8 (j / 4) + 4 h + j % 4.
+__device__ __forceinline__ bf16x8 frag_tr_acc(bf16 const *tile, int stride,
+                                              int r0, int s, int col0, int lane) {
+  int const i16 = lane & 15;
+  int const h = lane >> 5;
+  int const col = col0 + ((lane >> 4) & 1) * 16 + (i16 & 3) * 4;
+  int const row = r0 + 16 * s + 4 * h + (i16 >> 2);
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(tile + row * stride + col));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(tile + (row + 8) * stride + col));
+  union {
+    s16x4 h2[2];
+    bf16x8 v;
+  } u;
+  u.h2[0] = lo;
+  u.h2[1] = hi;
+  return u.v;
+}
+
+template <int D>
+struct AttnCfg {
+  static constexpr int kBQ = 128;          // query rows per workgroup (forward, dQ)
+  static constexpr int kBKV = 64;          // key rows per LDS tile (forward, dQ)
+  static constexpr int kKStride = D + 8;   // K tile row stride (b128 reads)
+  static constexpr int kVStride = D + 32;  // V tile row stride (transposing reads)
+  static constexpr int kChunks = kBKV * D / 8 / 256;  // 16-byte chunks per thread
+};
+
+// --------------------------------------------------------------------------
+// forward
+// --------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
+  using C = AttnCfg<D>;
+  __shared__ __attribute__((aligned(16))) bf16 Ks[2][C::kBKV * C::kKStride];
+  __shared__ __attribute__((aligned(16))) bf16 Vs[2][C::kBKV * C::kVStride];
+  int const t = threadIdx.x, lane = t & 63, wave = t >> 6, h32 = lane >> 5;
+  int const nqb = (p.Sq + C::kBQ - 1) / C::kBQ;
+  int const qb = nqb - 1 - blockIdx.x;  // heavy (late) causal blocks first
+  int const head = blockIdx.y, b = blockIdx.z;
+  int const q0 = qb * C::kBQ;
+  int const qrow = q0 + wave * 32 + (lane & 31);  // this lane's query row
+  bf16 const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * D;
+  bf16 const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * D;
+  bf16 const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * D;
+
+  // Q as the B operand of S^T = K Q^T: column = query row, k = d.
+  bf16x8 qf[D / 16];
+  {
+    int const r = min(qrow, p.Sq - 1);
+#pragma unroll
+    for (int kk = 0; kk < D / 16; kk++) {
+      qf[kk] = *reinterpret_cast<bf16x8 const *>(qp + (int64_t)r * p.q_ss + kk * 16 + h32 * 8);
+    }
+  }
+
+  int kv_end = p.Skv;
+  if (p.causal) kv_end = min(p.Skv, q0 + C::kBQ);
+  int const ntiles = (kv_end + C::kBKV - 1) / C::kBKV;
+
+  u32x4 rk[C::kChunks], rv[C::kChunks];
+  auto gload = [&](int kv0) {
+#pragma unroll
+    for (int i = 0; i < C::kChunks; i++) {
+      int c = t + i * 256;
+      int row = c / (D / 8), ch = c % (D / 8);
+      int gr = min(kv0 + row, p.Skv - 1);
+      rk[i] = *reinterpret_cast<u32x4 const *>(kp + (int64_t)gr * p.k_ss + ch * 8);
+      rv[i] = *reinterpret_cast<u32x4 const *>(vp + (int64_t)gr * p.v_ss + ch * 8);
+    }
+  };
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < C::kChunks; i++) {
+      int c = t + i * 256;
+      int row = c / (D / 8), ch = c % (D / 8);
+      *reinterpret_cast<u32x4 *>(&Ks[buf][row * C::kKStride + ch * 8]) = rk[i];
+      *reinterpret_cast<u32x4 *>(&Vs[buf][row * C::kVStride + ch * 8]) = rv[i];
+    }
+  };
+
+  f32x16 oacc[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) oacc[i][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  int cur = 0;
+  for (int it = 0; it < ntiles; it++) {
+    int const kv0 = it * C::kBKV;
+    bool const more = it + 1 < ntiles;
+    if (more) gload(kv0 + C::kBKV);
+
+    // A wave whose rows all lie before this tile (causal) has nothing to add.
+    bool const active = !p.causal || kv0 <= q0 + wave * 32 + 31;
+    if (active) {
+      // S^T tiles: rows = keys (32 per tile), columns = this wave's queries.
+      f32x16 s[C::kBKV / 32];
+#pragma unroll
+      for (int j = 0; j < C::kBKV / 32; j++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[j][r] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < D / 16; kk++) {
+          bf16x8 kf = frag_k(Ks[cur], C::kKStride, j * 32, kk * 16, lane);
+          s[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[j], 0, 0, 0);
+        }
+      }
+      // scale, mask, running max
+      bool const need_mask = (kv0 + C::kBKV > p.Skv) || (p.causal && kv0 + C::kBKV - 1 > q0 + wave * 32);
+      float mx = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < C::kBKV / 32; j++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float v = s[j][r] * p.scale_log2;
+          if (need_mask) {
+            int kv = kv0 + j * 32 + 8 * (r >> 2) + 4 * h32 + (r & 3);
+            if (kv >= p.Skv || (p.causal && kv > qrow)) v = -INFINITY;
+          }
+          s[j][r] = v;
+          mx = fmaxf(mx, v);
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      float const m_new = fmaxf(m_run, mx);
+      // m_new is finite: key 0 is visible to every query and tile 0 comes first.
+      float const alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      float sum = 0.0f;
+      bf16x8 pf[C::kBKV / 16];
+#pragma unroll
+      for (int j = 0; j < C::kBKV / 32; j++) {
+        float pv[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          // Round to bf16 first so that the row sum is the sum of the values
+          // that actually enter the P V product.
+          float e = __builtin_amdgcn_exp2f(s[j][r] - m_new);
+          e = bf16_bits_to_f32(f32_to_bf16_bits(e));
+          pv[r] = e;
+          sum += e;
+        }
+        pf[2 * j] = pack8(pv);
+        pf[2 * j + 1] = pack8(pv + 8);
+      }
+      sum += __shfl_xor(sum, 32, 64);
+      l_run = l_run * alpha + sum;
+      m_run = m_new;
+      // O^T += V^T P^T : A = V^T (rows d) via transposing loads, B = P^T.
+#pragma unroll
+      for (int i = 0; i < D / 32; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+#pragma unroll
+        for (int j = 0; j < C::kBKV / 32; j++) {
+#pragma unroll
+          for (int s2 = 0; s2 < 2; s2++) {
+            bf16x8 vf = frag_tr_acc(Vs[cur], C::kVStride, j * 32, s2, i * 32, lane);
+            oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[2 * j + s2], oacc[i], 0, 0, 0);
+          }
+        }
+      }
+    }
+    if (more) lstore(cur ^ 1);
+    __syncthreads();
+    cur ^= 1;
+  }
+
+  if (qrow < p.Sq) {
+    float const inv = 1.0f / l_run;
+    bf16 *op = p.o + (int64_t)b * p.o_bs + (int64_t)qrow * p.o_ss + (int64_t)head * D;
+#pragma unroll
+    for (int i = 0; i < D / 32; i++) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        int d = i * 32 + 8 * g + 4 * h32;
+        u32x2 w = {pack_bf16x2(oacc[i][4 * g] * inv, oacc[i][4 * g + 1] * inv),
+                   pack_bf16x2(oacc[i][4 * g + 2] * inv, oacc[i][4 * g + 3] * inv)};
+        *reinterpret_cast<u32x2 *>(op + d) = w;
+      }
+    }
+    if (h32 == 0 && p.lse != nullptr) {
+      p.lse[((int64_t)b * p.H + head) * p.Sq + qrow] = (m_run + __log2f(l_run)) * kLn2;
+    }
+  }
+}
+
+// --------------------------------------------------------------------------
+// backward
+// --------------------------------------------------------------------------
+struct AttnBwdParams {
+  bf16 const *q, *k, *v, *o, *d_o;
+  float const *lse;
+  float *delta;
+  bf16 *dq, *dk, *dv;
+  int B, H, Sq, Skv;
+  int64_t q_bs, q_ss, k_bs, k_ss, v_bs, v_ss, o_bs, o_ss;
+  float scale, scale_log2;
+  int causal;
+};
+
+// delta[b,h,q] = sum_d O * dO  (one wave per row)
+template <int D>
+__global__ __launch_bounds__(256) void attn_delta_kernel(AttnBwdParams p) {
+  int const lane = threadIdx.x & 63;
+  int64_t const row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  int64_t const total = (int64_t)p.B * p.H * p.Sq;
+  if (row >= total) return;
+  int const q = (int)(row % p.Sq);
+  int const head = (int)((row / p.Sq) % p.H);
+  int const b = (int)(row / ((int64_t)p.Sq * p.H));
+  int64_t off = (int64_t)b * p.o_bs + (int64_t)q * p.o_ss + (int64_t)head * D;
+  float s = 0.0f;
+  for (int d = lane; d < D; d += 64) {
+    s += VecIO<bf16>::load1(p.o + off + d) * VecIO<bf16>::load1(p.d_o + off + d);
+  }
+  s = wave_sum(s);
+  if (lane == 0) p.delta[row] = s;
+}
+
+template <int D>
+struct AttnBwdCfg {
+  static constexpr int kBlk = 128;         // rows owned by a workgroup
+  static constexpr int kTile = 32;         // rows of the streamed operand per step
+  static constexpr int kStride = D + 40;   // serves b128 and transposing reads
+  static constexpr int kChunks = kTile * D / 8 / 256;
+  static_assert(kTile * D / 8 % 256 == 0, "tile chunks");
+};
+
+// (A) dK, dV: workgroup owns 128 key rows (32 per wave), streams query tiles.
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
+  using C = AttnBwdCfg<D>;
+  __shared__ __attribute__((aligned(16))) bf16 Qs[2][C::kTile * C::kStride];
+  __shared__ __attribute__((aligned(16))) bf16 Gs[2][C::kTile * C::kStride];  // dO
+  __shared__ float Ls[2][C::kTile], Ds[2][C::kTile];
+  int const t = threadIdx.x, lane = t & 63, wave = t >> 6, h32 = lane >> 5;
+  int const head = blockIdx.y, b = blockIdx.z;
+  int const kv0 = blockIdx.x * C::kBlk;
+  int const kvrow = kv0 + wave * 32 + (lane & 31);
+  bf16 const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * D;
+  bf16 const *gp = p.d_o + (int64_t)b * p.o_bs + (int64_t)head * D;
+  bf16 const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * D;
+  bf16 const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * D;
+  float const *lsep = p.lse + ((int64_t)b * p.H + head) * p.Sq;
+  float const *delp = p.delta + ((int64_t)b * p.H + head) * p.Sq;
+
+  // K and V rows of this lane as B operands (column = key row, k = d).
+  bf16x8 kf[D / 16], vf[D / 16];
+  {
+    int const r = min(kvrow, p.Skv - 1);
+#pragma unroll
+    for (int kk = 0; kk < D / 16; kk++) {
+      kf[kk] = *reinterpret_cast<bf16x8 const *>(kp + (int64_t)r * p.k_ss + kk * 16 + h32 * 8);
+      vf[kk] = *reinterpret_cast<bf16x8 const *>(vp + (int64_t)r * p.v_ss + kk * 16 + h32 * 8);
+    }
+  }
+  f32x16 dk[D / 32], dv[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      dk[i][r] = 0.0f;
+      dv[i][r] = 0.0f;
+    }
+
+  int const q_begin = p.causal ? (kv0 / C::kTile) * C::kTile : 0;
+  int const ntiles = (p.Sq - q_begin + C::kTile - 1) / C::kTile;
+
+  u32x4 rq[C::kChunks], rg[C::kChunks];
+  float rl = 0.0f, rd = 0.0f;
+  auto gload = [&](int qt0) {
+#pragma unroll
+    for (int i = 0; i < C::kChunks; i++) {
+      int c = t + i * 256;
+      int row = c / (D / 8), ch = c % (D / 8);
+      int gr = min(qt0 + row, p.Sq - 1);
+      rq[i] = *reinterpret_cast<u32x4 const *>(qp + (int64_t)gr * p.q_ss + ch * 8);
+      rg[i] = *reinterpret_cast<u32x4 const *>(gp + (int64_t)gr * p.o_ss + ch * 8);
+    }
+    if (t < C::kTile) {
+      int gr = min(qt0 + t, p.Sq - 1);
+      rl = lsep[gr] * kLog2e;
+      rd = delp[gr];
+    }
+  };
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < C::kChunks; i++) {
+      int c = t + i * 256;
+      int row = c / (D / 8), ch = c % (D / 8);
+      *reinterpret_cast<u32x4 *>(&Qs[buf][row * C::kStride + ch * 8]) = rq[i];
+      *reinterpret_cast<u32x4 *>(&Gs[buf][row * C::kStride + ch * 8]) = rg[i];
+    }
+    if (t < C::kTile) {
+      Ls[buf][t] = rl;
+      Ds[buf][t] = rd;
+    }
+  };
+
+  if (ntiles > 0) {
+    gload(q_begin);
+    lstore(0);
+  }
+  __syncthreads();
+  int cur = 0;
+  for (int it = 0; it < ntiles; it++) {
+    int const qt0 = q_begin + it * C::kTile;
+    bool const more = it + 1 < ntiles;
+    if (more) gload(qt0 + C::kTile);
+    // A wave whose keys all lie after this query tile (causal) contributes 0.
+    bool const active = !p.causal || kv0 + wave * 32 <= qt0 + C::kTile - 1;
+    if (active) {
+      // S = Q K^T and dP = dO V^T: rows = queries of the tile, column = key.
+      f32x16 s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        s[r] = 0.0f;
+        dp[r] = 0.0f;
+      }
+#pragma unroll
+      for (int kk = 0; kk < D / 16; kk++) {
+        bf16x8 qa = frag_k(Qs[cur], C::kStride, 0, kk * 16, lane);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s, 0, 0, 0);
+        bf16x8 ga = frag_k(Gs[cur], C::kStride, 0, kk * 16, lane);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[kk], dp, 0, 0, 0);
+      }
+      float pv[16], dsv[16];
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        int const qi = 8 * (r >> 2) + 4 * h32 + (r & 3);
+        int const qg = qt0 + qi;
+        float e = __builtin_amdgcn_exp2f(s[r] * p.scale_log2 - Ls[cur][qi]);
+        bool const masked = qg >= p.Sq || kvrow >= p.Skv || (p.causal && kvrow > qg);
+        e = masked ? 0.0f : e;
+        pv[r] = e;
+        dsv[r] = e * (dp[r] - Ds[cur][qi]) * p.scale;
+      }
+      // dV += P^T dO ; dK += dS^T Q.  A = accumulator re-used (row = key),
+      // B = dO / Q read with the matching reduction order (k = query).
+#pragma unroll
+      for (int s2 = 0; s2 < 2; s2++) {
+        bf16x8 pa = pack8(pv + 8 * s2);
+        bf16x8 da = pack8(dsv + 8 * s2);
+#pragma unroll
+        for (int i = 0; i < D / 32; i++) {
+          bf16x8 gb = frag_tr_acc(Gs[cur], C::kStride, 0, s2, i * 32, lane);
+          dv[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa, gb, dv[i], 0, 0, 0);
+          bf16x8 qb = frag_tr_acc(Qs[cur], C::kStride, 0, s2, i * 32, lane);
+          dk[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, qb, dk[i], 0, 0, 0);
+        }
+      }
+    }
+    if (more) lstore(cur ^ 1);
+    __syncthreads();
+    cur ^= 1;
+  }
+
+  // dK / dV accumulators: row = key (32 per wave, 8*(r/4)+4*h+r%4), column = d.
+  bf16 *dkp = p.dk + (int64_t)b * p.k_bs + (int64_t)head * D;
+  bf16 *dvp = p.dv + (int64_t)b * p.v_bs + (int64_t)head * D;
+#pragma unroll
+  for (int i = 0; i < D / 32; i++) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      int const row = kv0 + wave * 32 + 8 * (r >> 2) + 4 * h32 + (r & 3);
+      int const d = i * 32 + (lane & 31);
+      if (row < p.Skv) {
+        VecIO<bf16>::store1(dkp + (int64_t)row * p.k_ss + d, dk[i][r]);
+        VecIO<bf16>::store1(dvp + (int64_t)row * p.v_ss + d, dv[i][r]);
+      }
+    }
+  }
+}
+
+// (B) dQ: workgroup owns 128 query rows (32 per wave), streams key tiles.
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
+  using C = AttnBwdCfg<D>;
+  __shared__ __attribute__((aligned(16))) bf16 Ks[2][C::kTile * C::kStride];
+  __shared__ __attribute__((aligned(16))) bf16 Vs[2][C::kTile * C::kStride];
+  int const t = threadIdx.x, lane = t & 63, wave = t >> 6, h32 = lane >> 5;
+  int const nqb = (p.Sq + C::kBlk - 1) / C::kBlk;
+  int const qb = nqb - 1 - blockIdx.x;
+  int const head = blockIdx.y, b = blockIdx.z;
+  int const q0 = qb * C::kBlk;
+  int const qrow = q0 + wave * 32 + (lane & 31);
+  bf16 const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * D;
+  bf16 const *gp = p.d_o + (int64_t)b * p.o_bs + (int64_t)head * D;
+  bf16 const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * D;
+  bf16 const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * D;
+
+  bf16x8 qf[D / 16], gf[D / 16];
+  float lse2, delta;
+  {
+    int const r = min(qrow, p.Sq - 1);
+#pragma unroll
+    for (int kk = 0; kk < D / 16; kk++) {
+      qf[kk] = *reinterpret_cast<bf16x8 const *>(qp + (int64_t)r * p.q_ss + kk * 16 + h32 * 8);
+      gf[kk] = *reinterpret_cast<bf16x8 const *>(gp + (int64_t)r * p.o_ss + kk * 16 + h32 * 8);
+    }
+    lse2 = p.lse[((int64_t)b * p.H + head) * p.Sq + r] * kLog2e;
+    delta = p.delta[((int64_t)b * p.H + head) * p.Sq + r];
+  }
+  f32x16 dq[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dq[i][r] = 0.0f;
+
+  int kv_end = p.Skv;
+  if (p.causal) kv_end = min(p.Skv, q0 + C::kBlk);
+  int const ntiles = (kv_end + C::kTile - 1) / C::kTile;
+
+  u32x4 rk[C::kChunks], rv[C::kChunks];
+  auto gload = [&](int kt0) {
+#pragma unroll
+    for (int i = 0; i < C::kChunks; i++) {
+      int c = t + i * 256;
+      int row = c / (D / 8), ch = c % (D / 8);
+      int gr = min(kt0 + row, p.Skv - 1);
+      rk[i] = *reinterpret_cast<u32x4 const *>(kp + (int64_t)gr * p.k_ss + ch * 8);
+      rv[i] = *reinterpret_cast<u32x4 const *>(vp + (int64_t)gr * p.v_ss + ch * 8);
+    }
+  };
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < C::kChunks; i++) {
+      int c = t + i * 256;
+      int row = c / (D / 8), ch = c % (D / 8);
+      *reinterpret_cast<u32x4 *>(&Ks[buf][row * C::kStride + ch * 8]) = rk[i];
+      *reinterpret_cast<u32x4 *>(&Vs[buf][row * C::kStride + ch * 8]) = rv[i];
+    }
+  };
+
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  int cur = 0;
+  for (int it = 0; it < ntiles; it++) {
+    int const kt0 = it * C::kTile;
+    bool const more = it + 1 < ntiles;
+    if (more) gload(kt0 + C::kTile);
+    bool const active = !p.causal || kt0 <= q0 + wave * 32 + 31;
+    if (active) {
+      // S^T = K Q^T, dP^T = V dO^T: rows = keys of the tile, column = query.
+      f32x16 s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        s[r] = 0.0f;
+        dp[r] = 0.0f;
+      }
+#pragma unroll
+      for (int kk = 0; kk < D / 16; kk++) {
+        bf16x8 ka = frag_k(Ks[cur], C::kStride, 0, kk * 16, lane);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], s, 0, 0, 0);
+        bf16x8 va = frag_k(Vs[cur], C::kStride, 0, kk * 16, lane);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, gf[kk], dp, 0, 0, 0);
+      }
+      float dsv[16];
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        int const kv = kt0 + 8 * (r >> 2) + 4 * h32 + (r & 3);
+        float e = __builtin_amdgcn_exp2f(s[r] * p.scale_log2 - lse2);
+        bool const masked = kv >= p.Skv || (p.causal && kv > qrow);
+        e = masked ? 0.0f : e;
+        dsv[r] = e * (dp[r] - delta) * p.scale;
+      }
+      // dQ^T += K^T dS^T : A = K^T (rows d) via transposing loads, B = dS^T.
+#pragma unroll
+      for (int s2 = 0; s2 < 2; s2++) {
+        bf16x8 db = pack8(dsv + 8 * s2);
+#pragma unroll
+        for (int i = 0; i < D / 32; i++) {
+          bf16x8 ka = frag_tr_acc(Ks[cur], C::kStride, 0, s2, i * 32, lane);
+          dq[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, db, dq[i], 0, 0, 0);
+        }
+      }
+    }
+    if (more) lstore(cur ^ 1);
+    __syncthreads();
+    cur ^= 1;
+  }
+
+  if (qrow < p.Sq) {
+    bf16 *dqp = p.dq + (int64_t)b * p.q_bs + (int64_t)qrow * p.q_ss + (int64_t)head * D;
+#pragma unroll
+    for (int i = 0; i < D / 32; i++) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        int d = i * 32 + 8 * g + 4 * h32;
+        u32x2 w = {pack_bf16x2(dq[i][4 * g], dq[i][4 * g + 1]),
+                   pack_bf16x2(dq[i][4 * g + 2], dq[i][4 * g + 3])};
+        *reinterpret_cast<u32x2 *>(dqp + d) = w;
+      }
+    }
+  }
+}
+
+static int check_desc(char const *who, int dtype, ffk_attention_desc_t const *d) {
+  FFK_REQUIRE(d != nullptr, "%s: NULL descriptor", who);
+  FFK_REQUIRE(dtype == FFK_BF16, "%s: dtype %d not supported (bf16 only)", who, dtype);
+  FFK_REQUIRE(d->head_dim == 64 || d->head_dim == 128,
+              "%s: head_dim %lld not supported (64 or 128)", who, (long long)d->head_dim);
+  FFK_REQUIRE(d->batch > 0 && d->heads > 0 && d->seq_q > 0 && d->seq_kv > 0, "%s: bad shape", who);
+  FFK_REQUIRE(d->batch < 65536 && d->heads < 65536, "%s: batch/heads exceed the grid limit", who);
+  FFK_REQUIRE(d->seq_q < (1ll << 30) && d->seq_kv < (1ll << 30), "%s: sequence too long", who);
+  FFK_REQUIRE(d->q_seq_stride % 8 == 0 && d->k_seq_stride % 8 == 0 && d->v_seq_stride % 8 == 0 &&
+                  d->o_seq_stride % 8 == 0 && d->q_batch_stride % 8 == 0 && d->k_batch_stride % 8 == 0 &&
+                  d->v_batch_stride % 8 == 0 && d->o_batch_stride % 8 == 0,
+              "%s: strides must be multiples of 8 elements", who);
+  FFK_REQUIRE(d->q_seq_stride >= d->heads * d->head_dim && d->k_seq_stride >= d->heads * d->head_dim &&
+                  d->v_seq_stride >= d->heads * d->head_dim && d->o_seq_stride >= d->heads * d->head_dim,
+              "%s: sequence stride smaller than heads * head_dim", who);
+  return FFK_OK;
+}
+
+}  // namespace ffk
+
+using namespace ffk;
+
+extern "C" int ffk_attention_forward(ffk_stream_t stream, int dtype,
+                                     ffk_attention_desc_t const *d,
+                                     void const *q, void const *k,
+                                     void const *v, void *o, float *lse) {
+  int rc = check_desc("attention_forward", dtype, d);
+  if (rc != FFK_OK) return rc;
+  FFK_REQUIRE(q && k && v && o, "attention_forward: NULL tensor");
+  FFK_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o),
+              "attention_forward: tensors must be 16-byte aligned");
+  AttnParams p;
+  p.q = static_cast<bf16 const *>(q);
+  p.k = static_cast<bf16 const *>(k);
+  p.v = static_cast<bf16 const *>(v);
+  p.o = static_cast<bf16 *>(o);
+  p.lse = lse;
+  p.B = (int)d->batch; p.H = (int)d->heads; p.Sq = (int)d->seq_q; p.Skv = (int)d->seq_kv;
+  p.q_bs = d->q_batch_stride; p.q_ss = d->q_seq_stride;
+  p.k_bs = d->k_batch_stride; p.k_ss = d->k_seq_stride;
+  p.v_bs = d->v_batch_stride; p.v_ss = d->v_seq_stride;
+  p.o_bs = d->o_batch_stride; p.o_ss = d->o_seq_stride;
+  p.scale_log2 = d->scale * kLog2e;
+  p.causal = d->causal;
+  dim3 grid((unsigned)ceil_div(p.Sq, 128), (unsigned)p.H, (unsigned)p.B);
+  if (d->head_dim == 64) {
+    attn_fwd_kernel<64><<<grid, 256, 0, as_stream(stream)>>>(p);
+  } else {
+    attn_fwd_kernel<128><<<grid, 256, 0, as_stream(stream)>>>(p);
+  }
+  FFK_CHECK_LAUNCH();
+  return FFK_OK;
+}
+
+extern "C" int ffk_attention_backward(ffk_stream_t stream, int dtype,
+                                      ffk_attention_desc_t const *d,
+                                      void const *q, void const *k,
+                                      void const *v, void const *o,
+                                      void const *d_o, float const *lse,
+                                      float *delta, void *dq, void *dk,
+                                      void *dv) {
+  int rc = check_desc("attention_backward", dtype, d);
+  if (rc != FFK_OK) return rc;
+  FFK_REQUIRE(q && k && v && o && d_o && lse && delta && dq && dk && dv,
+              "attention_backward: NULL tensor");
+  FFK_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) && aligned16(d_o) &&
+                  aligned16(dq) && aligned16(dk) && aligned16(dv),
+              "attention_backward: tensors must be 16-byte aligned");
+  AttnBwdParams p;
+  p.q = static_cast<bf16 const *>(q);
+  p.k = static_cast<bf16 const *>(k);
+  p.v = static_cast<bf16 const *>(v);
+  p.o = static_cast<bf16 const *>(o);
+  p.d_o = static_cast<bf16 const *>(d_o);
+  p.lse = lse;
+  p.delta = delta;
+  p.dq = static_cast<bf16 *>(dq);
+  p.dk = static_cast<bf16 *>(dk);
+  p.dv = static_cast<bf16 *>(dv);
+  p.B = (int)d->batch; p.H = (int)d->heads; p.Sq = (int)d->seq_q; p.Skv = (int)d->seq_kv;
+  p.q_bs = d->q_batch_stride; p.q_ss = d->q_seq_stride;
+  p.k_bs = d->k_batch_stride; p.k_ss = d->k_seq_stride;
+  p.v_bs = d->v_batch_stride; p.v_ss = d->v_seq_stride;
+  p.o_bs = d->o_batch_stride; p.o_ss = d->o_seq_stride;
+  p.scale = d->scale;
+  p.scale_log2 = d->scale * kLog2e;
+  p.causal = d->causal;
+  hipStream_t st = as_stream(stream);
+  int64_t rows = (int64_t)p.B * p.H * p.Sq;
+  dim3 gkv((unsigned)ceil_div(p.Skv, 128), (unsigned)p.H, (unsigned)p.B);
+  dim3 gq((unsigned)ceil_div(p.Sq, 128), (unsigned)p.H, (unsigned)p.B);
+  if (d->head_dim == 64) {
+    attn_delta_kernel<64><<<(unsigned)ceil_div(rows, 4), 256, 0, st>>>(p);
+    FFK_CHECK_LAUNCH();
+    attn_bwd_dkdv_kernel<64><<<gkv, 256, 0, st>>>(p);
+    FFK_CHECK_LAUNCH();
+    attn_bwd_dq_kernel<64><<<gq, 256, 0, st>>>(p);
+  } else {
+    attn_delta_kernel<128><<<(unsigned)ceil_div(rows, 4), 256, 0, st>>>(p);
+    FFK_CHECK_LAUNCH();
+    attn_bwd_dkdv_kernel<128><<<gkv, 256, 0, st>>>(p);
+    FFK_CHECK_LAUNCH();
+    attn_bwd_dq_kernel<128><<<gq, 256, 0, st>>>(p);
+  }
+  FFK_CHECK_LAUNCH();
+  return FFK_OK;
+}

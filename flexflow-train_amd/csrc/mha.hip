@@ -1,0 +1,250 @@
+// MultiHeadAttention forward/backward for gfx950: projection GEMMs around the
+// fused attention core (reference: one cudnnMultiHeadAttnForward /
+// BackwardData / BackwardWeights call each, lib/kernels/src/cuda/ops/
+// attention_kernels.cu:215-303).
+//
+// Weight blob: [ W_Q | W_K | W_V | W_O ] with W_Q = [heads*qProj, qSize]
+// (head-major rows), W_K = [heads*kProj, kSize], W_V = [heads*vProj, vSize],
+// W_O = [oProj, heads*vProj], all row-major.  When query, key and value are
+// the same tensor the three input projections run as one GEMM against the
+// contiguous [3*heads*proj, size] block and the core reads the fused buffer
+// through strides.
+//
+// Reserve space layout (bytes, each region 256-byte aligned):
+//   QKV projections | context | lse | delta | d(context) | d(QKV projections)
+#include "gemm.h"
+
+namespace ffk {
+
+struct MhaLayout {
+  int64_t TQ, TK;                 // tokens: B*Sq, B*Skv
+  int64_t nQ, nK, nV, nC;         // elements of each projected tensor / context
+  size_t off_qkv, off_ctx, off_lse, off_delta, off_dctx, off_dqkv, total;
+  int64_t wq, wk, wv, wo;         // weight offsets (elements)
+};
+
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static MhaLayout make_layout(ffk_mha_desc_t const *d, size_t es) {
+  MhaLayout L;
+  L.TQ = d->num_samples * d->qo_seq_length;
+  L.TK = d->num_samples * d->kv_seq_length;
+  L.nQ = L.TQ * d->num_heads * d->q_proj_size;
+  L.nK = L.TK * d->num_heads * d->k_proj_size;
+  L.nV = L.TK * d->num_heads * d->v_proj_size;
+  L.nC = L.TQ * d->num_heads * d->v_proj_size;
+  size_t off = 0;
+  L.off_qkv = off;   off += align256((size_t)(L.nQ + L.nK + L.nV) * es);
+  L.off_ctx = off;   off += align256((size_t)L.nC * es);
+  L.off_lse = off;   off += align256((size_t)(d->num_samples * d->num_heads * d->qo_seq_length) * 4);
+  L.off_delta = off; off += align256((size_t)(d->num_samples * d->num_heads * d->qo_seq_length) * 4);
+  L.off_dctx = off;  off += align256((size_t)L.nC * es);
+  L.off_dqkv = off;  off += align256((size_t)(L.nQ + L.nK + L.nV) * es);
+  L.total = off;
+  L.wq = 0;
+  L.wk = L.wq + d->num_heads * d->q_proj_size * d->q_size;
+  L.wv = L.wk + d->num_heads * d->k_proj_size * d->k_size;
+  L.wo = L.wv + d->num_heads * d->v_proj_size * d->v_size;
+  return L;
+}
+
+static int check_mha(char const *who, int dtype, ffk_mha_desc_t const *d) {
+  FFK_REQUIRE(d != nullptr, "%s: NULL descriptor", who);
+  FFK_REQUIRE(dtype == FFK_BF16, "%s: dtype %d not supported (bf16 only)", who, dtype);
+  FFK_REQUIRE(d->num_samples > 0 && d->num_heads > 0 && d->q_size > 0 && d->k_size > 0 &&
+                  d->v_size > 0 && d->o_proj_size > 0 && d->qo_seq_length > 0 && d->kv_seq_length > 0,
+              "%s: non-positive size", who);
+  FFK_REQUIRE(d->q_proj_size == d->k_proj_size, "%s: qProjSize must equal kProjSize", who);
+  FFK_REQUIRE(d->v_proj_size == d->q_proj_size,
+              "%s: vProjSize != qProjSize is not supported by the fused core", who);
+  FFK_REQUIRE(d->q_proj_size == 64 || d->q_proj_size == 128,
+              "%s: projection size %lld not supported (64 or 128)", who, (long long)d->q_proj_size);
+  return FFK_OK;
+}
+
+static bool is_fused(ffk_mha_desc_t const *d, void const *q, void const *k, void const *v) {
+  return q == k && k == v && d->q_size == d->k_size && d->k_size == d->v_size &&
+         d->qo_seq_length == d->kv_seq_length;
+}
+
+static ffk_attention_desc_t core_desc(ffk_mha_desc_t const *d, bool fused) {
+  int64_t const H = d->num_heads, D = d->q_proj_size;
+  ffk_attention_desc_t a;
+  a.batch = d->num_samples;
+  a.heads = H;
+  a.seq_q = d->qo_seq_length;
+  a.seq_kv = d->kv_seq_length;
+  a.head_dim = D;
+  int64_t const row = fused ? 3 * H * D : H * D;
+  a.q_seq_stride = a.k_seq_stride = a.v_seq_stride = row;
+  a.q_batch_stride = d->qo_seq_length * row;
+  a.k_batch_stride = a.v_batch_stride = d->kv_seq_length * row;
+  a.o_seq_stride = H * D;
+  a.o_batch_stride = d->qo_seq_length * H * D;
+  a.scale = d->scale;
+  a.causal = d->causal;
+  return a;
+}
+
+}  // namespace ffk
+
+using namespace ffk;
+
+extern "C" size_t ffk_mha_weight_elements(ffk_mha_desc_t const *d) {
+  if (d == nullptr) return 0;
+  return (size_t)(d->num_heads * (d->q_proj_size * d->q_size + d->k_proj_size * d->k_size +
+                                  d->v_proj_size * d->v_size + d->v_proj_size * d->o_proj_size));
+}
+
+extern "C" size_t ffk_mha_reserve_bytes(ffk_mha_desc_t const *d, int dtype) {
+  if (d == nullptr || dtype_size(dtype) == 0) return 0;
+  return make_layout(d, dtype_size(dtype)).total;
+}
+
+extern "C" int ffk_mha_forward(ffk_stream_t stream, int dtype,
+                               ffk_mha_desc_t const *d, void const *query,
+                               void const *key, void const *value,
+                               void const *weight, void *output, void *reserve,
+                               size_t reserve_bytes) {
+  int rc = check_mha("mha_forward", dtype, d);
+  if (rc != FFK_OK) return rc;
+  FFK_REQUIRE(query && key && value && weight && output, "mha_forward: NULL tensor");
+  size_t const es = dtype_size(dtype);
+  MhaLayout L = make_layout(d, es);
+  if (reserve == nullptr || reserve_bytes < L.total) {
+    return fail(FFK_ERR_WORKSPACE, "mha_forward: reserve space of %zu bytes needed, %zu given",
+                L.total, reserve_bytes);
+  }
+  hipStream_t st = as_stream(stream);
+  uint8_t *rs = static_cast<uint8_t *>(reserve);
+  uint8_t const *w = static_cast<uint8_t const *>(weight);
+  int64_t const H = d->num_heads, D = d->q_proj_size, HD = H * D;
+  bool const fused = is_fused(d, query, key, value);
+  uint8_t *qkv = rs + L.off_qkv;
+  GemmEpilogue ep;
+  void const *qp, *kp, *vp;
+  if (fused) {
+    // [T, 3HD] = X . [W_Q; W_K; W_V]^T
+    rc = gemm_dispatch(st, dtype, false, true, L.TQ, 3 * HD, d->q_size, query, d->q_size,
+                       w + L.wq * es, d->q_size, qkv, 3 * HD, ep);
+    if (rc != FFK_OK) return rc;
+    qp = qkv;
+    kp = qkv + HD * es;
+    vp = qkv + 2 * HD * es;
+  } else {
+    uint8_t *Q = qkv, *K = qkv + L.nQ * es, *V = K + L.nK * es;
+    rc = gemm_dispatch(st, dtype, false, true, L.TQ, HD, d->q_size, query, d->q_size,
+                       w + L.wq * es, d->q_size, Q, HD, ep);
+    if (rc != FFK_OK) return rc;
+    rc = gemm_dispatch(st, dtype, false, true, L.TK, HD, d->k_size, key, d->k_size,
+                       w + L.wk * es, d->k_size, K, HD, ep);
+    if (rc != FFK_OK) return rc;
+    rc = gemm_dispatch(st, dtype, false, true, L.TK, HD, d->v_size, value, d->v_size,
+                       w + L.wv * es, d->v_size, V, HD, ep);
+    if (rc != FFK_OK) return rc;
+    qp = Q; kp = K; vp = V;
+  }
+  ffk_attention_desc_t a = core_desc(d, fused);
+  rc = ffk_attention_forward(stream, dtype, &a, qp, kp, vp, rs + L.off_ctx,
+                             reinterpret_cast<float *>(rs + L.off_lse));
+  if (rc != FFK_OK) return rc;
+  // output[T, oProj] = context[T, HD] . W_O[oProj, HD]^T
+  return gemm_dispatch(st, dtype, false, true, L.TQ, d->o_proj_size, HD, rs + L.off_ctx, HD,
+                       w + L.wo * es, HD, output, d->o_proj_size, ep);
+}
+
+extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
+                                ffk_mha_desc_t const *d, void const *query,
+                                void *query_grad, void const *key,
+                                void *key_grad, void const *value,
+                                void *value_grad, void const *weight,
+                                void *weight_grad, void const *output_grad,
+                                void *reserve, size_t reserve_bytes,
+                                int accumulate) {
+  int rc = check_mha("mha_backward", dtype, d);
+  if (rc != FFK_OK) return rc;
+  FFK_REQUIRE(query && key && value && weight && output_grad, "mha_backward: NULL tensor");
+  size_t const es = dtype_size(dtype);
+  MhaLayout L = make_layout(d, es);
+  if (reserve == nullptr || reserve_bytes < L.total) {
+    return fail(FFK_ERR_WORKSPACE, "mha_backward: reserve space of %zu bytes needed, %zu given",
+                L.total, reserve_bytes);
+  }
+  hipStream_t st = as_stream(stream);
+  uint8_t *rs = static_cast<uint8_t *>(reserve);
+  uint8_t const *w = static_cast<uint8_t const *>(weight);
+  uint8_t *dw = static_cast<uint8_t *>(weight_grad);
+  int64_t const H = d->num_heads, D = d->q_proj_size, HD = H * D;
+  bool const fused = is_fused(d, query, key, value);
+  uint8_t *qkv = rs + L.off_qkv, *dqkv = rs + L.off_dqkv;
+  uint8_t *ctx = rs + L.off_ctx, *dctx = rs + L.off_dctx;
+  GemmEpilogue over, acc, in_ep;
+  acc.accumulate = true;
+  in_ep.accumulate = accumulate != 0;
+
+  // d(context) = dOut . W_O ; dW_O += dOut^T . context
+  rc = gemm_dispatch(st, dtype, false, false, L.TQ, HD, d->o_proj_size, output_grad,
+                     d->o_proj_size, w + L.wo * es, HD, dctx, HD, over);
+  if (rc != FFK_OK) return rc;
+  if (dw != nullptr) {
+    rc = gemm_dispatch(st, dtype, true, false, d->o_proj_size, HD, L.TQ, output_grad,
+                       d->o_proj_size, ctx, HD, dw + L.wo * es, HD, acc);
+    if (rc != FFK_OK) return rc;
+  }
+
+  ffk_attention_desc_t a = core_desc(d, fused);
+  void const *qp, *kp, *vp;
+  void *dqp, *dkp, *dvp;
+  int64_t ld;
+  if (fused) {
+    qp = qkv; kp = qkv + HD * es; vp = qkv + 2 * HD * es;
+    dqp = dqkv; dkp = dqkv + HD * es; dvp = dqkv + 2 * HD * es;
+    ld = 3 * HD;
+  } else {
+    qp = qkv; kp = qkv + L.nQ * es; vp = qkv + (L.nQ + L.nK) * es;
+    dqp = dqkv; dkp = dqkv + L.nQ * es; dvp = dqkv + (L.nQ + L.nK) * es;
+    ld = HD;
+  }
+  // The core writes dQ/dK/dV with the same strides it reads Q/K/V with.
+  rc = ffk_attention_backward(stream, dtype, &a, qp, kp, vp, ctx, dctx,
+                              reinterpret_cast<float const *>(rs + L.off_lse),
+                              reinterpret_cast<float *>(rs + L.off_delta), dqp, dkp, dvp);
+  if (rc != FFK_OK) return rc;
+
+  bool const folded = fused && key_grad == nullptr && value_grad == nullptr;
+  if (folded) {
+    // dX (+)= dQKV[T,3HD] . [W_Q; W_K; W_V]  and  dW_QKV += dQKV^T . X
+    if (query_grad != nullptr) {
+      rc = gemm_dispatch(st, dtype, false, false, L.TQ, d->q_size, 3 * HD, dqkv, 3 * HD,
+                         w + L.wq * es, d->q_size, query_grad, d->q_size, in_ep);
+      if (rc != FFK_OK) return rc;
+    }
+    if (dw != nullptr) {
+      rc = gemm_dispatch(st, dtype, true, false, 3 * HD, d->q_size, L.TQ, dqkv, 3 * HD, query,
+                         d->q_size, dw + L.wq * es, d->q_size, acc);
+      if (rc != FFK_OK) return rc;
+    }
+    return FFK_OK;
+  }
+  struct Part {
+    void const *x; void *dx; void const *dp; int64_t T, size, woff;
+  } parts[3] = {
+      {query, query_grad, dqp, L.TQ, d->q_size, L.wq},
+      {key, key_grad, dkp, L.TK, d->k_size, L.wk},
+      {value, value_grad, dvp, L.TK, d->v_size, L.wv},
+  };
+  for (int i = 0; i < 3; i++) {
+    Part const &pt = parts[i];
+    if (pt.dx != nullptr) {
+      rc = gemm_dispatch(st, dtype, false, false, pt.T, pt.size, HD, pt.dp, ld,
+                         w + pt.woff * es, pt.size, pt.dx, pt.size, in_ep);
+      if (rc != FFK_OK) return rc;
+    }
+    if (dw != nullptr) {
+      rc = gemm_dispatch(st, dtype, true, false, HD, pt.size, pt.T, pt.dp, ld, pt.x, pt.size,
+                         dw + pt.woff * es, pt.size, acc);
+      if (rc != FFK_OK) return rc;
+    }
+  }
+  return FFK_OK;
+}

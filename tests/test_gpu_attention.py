@@ -1,0 +1,241 @@
+"""Fused attention core and MultiHeadAttention parity against the oracle."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from util import BF16_RTOL, assert_close, bf16_round, rng, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+BT = torch.bfloat16
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+SHAPES = [  # B, H, Sq, Skv, D
+    (1, 1, 8, 8, 64), (2, 3, 11, 11, 64), (1, 2, 100, 100, 128), (2, 2, 129, 129, 64),
+    (1, 4, 256, 256, 128), (1, 2, 300, 300, 64), (1, 1, 64, 200, 64), (2, 1, 160, 96, 128),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_core(ffk, oracle, shape, causal):
+    B, H, Sq, Skv, D = shape
+    if causal and Sq != Skv:
+        pytest.skip("causal is defined for self-attention (Sq == Skv) here")
+    say("attention core", shape, "causal", causal)
+    g = rng(Sq * 7 + D + int(causal))
+    q = bf16_round(g.standard_normal((B, Sq, H, D)))
+    k = bf16_round(g.standard_normal((B, Skv, H, D)))
+    v = bf16_round(g.standard_normal((B, Skv, H, D)))
+    do = bf16_round(g.standard_normal((B, Sq, H, D)))
+    scale = 1.0 / np.sqrt(D)
+    o_ref, lse_ref = oracle.attention_forward(q, k, v, scale, causal, bf16_mode=True)
+    qd, kd, vd, dod = (to_dev(a, torch, BT) for a in (q, k, v, do))
+    o, lse = ffk.attention_forward(qd, kd, vd, scale, causal)
+    assert_close(to_np(o), o_ref, BF16_RTOL, "O")
+    assert_close(to_np(lse), lse_ref, 1e-3, "lse")
+    dq_ref, dk_ref, dv_ref = oracle.attention_backward(q, k, v, do, scale, causal)
+    dq, dk, dv = ffk.attention_backward(qd, kd, vd, o, dod, lse, scale, causal)
+    assert_close(to_np(dq), dq_ref, BF16_RTOL, "dQ")
+    assert_close(to_np(dk), dk_ref, BF16_RTOL, "dK")
+    assert_close(to_np(dv), dv_ref, BF16_RTOL, "dV")
+
+
+def test_attention_reference_scale_one(ffk, oracle):
+    """The reference configures cuDNN with smScalar = 1.0 (attention_kernels.cu:76)."""
+    say("attention scale 1.0")
+    g = rng(3)
+    B, H, S, D = 1, 2, 40, 64
+    q = bf16_round(g.standard_normal((B, S, H, D)) * 0.3)
+    k = bf16_round(g.standard_normal((B, S, H, D)) * 0.3)
+    v = bf16_round(g.standard_normal((B, S, H, D)))
+    o_ref, _ = oracle.attention_forward(q, k, v, 1.0, False, bf16_mode=True)
+    o, _ = ffk.attention_forward(*(to_dev(a, torch, BT) for a in (q, k, v)), 1.0, False)
+    assert_close(to_np(o), o_ref, BF16_RTOL, "O")
+
+
+def test_attention_strided_views(ffk, oracle):
+    """q/k/v interleaved in one [B, S, 3*H*D] buffer, addressed through strides."""
+    say("attention strided")
+    g = rng(4)
+    B, H, S, D = 2, 2, 70, 64
+    qkv = bf16_round(g.standard_normal((B, S, 3, H, D)))
+    do = bf16_round(g.standard_normal((B, S, H, D)))
+    q, k, v = (np.ascontiguousarray(qkv[:, :, i]) for i in range(3))
+    scale = 0.125
+    o_ref, _ = oracle.attention_forward(q, k, v, scale, True, bf16_mode=True)
+    dq_ref, dk_ref, dv_ref = oracle.attention_backward(q, k, v, do, scale, True)
+    buf = to_dev(qkv, torch, BT)
+    row = 3 * H * D
+    desc = ffk.AttentionDesc(B, H, S, S, D, S * row, row, S * row, row, S * row, row, S * H * D, H * D,
+                             scale, 1)
+    es = 2
+    o = torch.empty((B, S, H, D), dtype=BT, device="cuda")
+    lse = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
+    base = buf.data_ptr()
+    st = ffk.current_stream()
+    ffk.check(ffk.lib().ffk_attention_forward(st, ffk.BF16, desc, base, base + H * D * es, base + 2 * H * D * es,
+                                              o.data_ptr(), lse.data_ptr()))
+    assert_close(to_np(o), o_ref, BF16_RTOL, "O")
+    dbuf = torch.zeros_like(buf)
+    delta = torch.empty_like(lse)
+    dod = to_dev(do, torch, BT)
+    db = dbuf.data_ptr()
+    ffk.check(ffk.lib().ffk_attention_backward(st, ffk.BF16, desc, base, base + H * D * es, base + 2 * H * D * es,
+                                               o.data_ptr(), dod.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                                               db, db + H * D * es, db + 2 * H * D * es))
+    d = to_np(dbuf)
+    assert_close(d[:, :, 0], dq_ref, BF16_RTOL, "dQ")
+    assert_close(d[:, :, 1], dk_ref, BF16_RTOL, "dK")
+    assert_close(d[:, :, 2], dv_ref, BF16_RTOL, "dV")
+
+
+def test_attention_errors(ffk):
+    q = torch.zeros((1, 8, 1, 32), dtype=BT, device="cuda")
+    with pytest.raises(ffk.FFKError, match="head_dim"):
+        ffk.attention_forward(q, q, q, 1.0, False)
+    q32 = torch.zeros((1, 8, 1, 64), dtype=torch.float32, device="cuda")
+    with pytest.raises(ffk.FFKError, match="dtype"):
+        ffk.attention_forward(q32, q32, q32, 1.0, False)
+
+
+def test_attention_config5_causal_prefix(ffk, oracle):
+    """BASELINE config 5 (B 4, S 4096, H 32, hd 128, causal) at full size.
+    Causality makes the first P queries a function of the first P keys only,
+    so the oracle on that prefix is the exact expectation for the full run;
+    dK/dV of the LAST keys depend only on the last queries likewise."""
+    B, H, S, D = 4, 32, 4096, 128
+    say("attention cfg5 full size")
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v, do = (torch.randn((B, S, H, D), device="cuda", generator=gen).to(BT) for _ in range(4))
+    scale = 1.0 / np.sqrt(D)
+    o, lse = ffk.attention_forward(q, k, v, scale, True)
+    P = 192
+    for (b, h) in ((0, 0), (3, 31)):
+        qs, ks, vs = (to_np(t[b:b + 1, :P, h:h + 1]) for t in (q, k, v))
+        o_ref, lse_ref = oracle.attention_forward(qs, ks, vs, scale, True, bf16_mode=True)
+        assert_close(to_np(o[b:b + 1, :P, h:h + 1]), o_ref, BF16_RTOL, "O prefix")
+        assert_close(to_np(lse[b, h, :P]), lse_ref[0, 0], 1e-3, "lse prefix")
+    assert torch.isfinite(o.float()).all()
+    dq, dk, dv = ffk.attention_backward(q, k, v, o, do, lse, scale, True)
+    assert torch.isfinite(dq.float()).all() and torch.isfinite(dk.float()).all()
+    # dQ of the first P queries depends on the first P keys only
+    b, h = 1, 7
+    qs, ks, vs, dos = (to_np(t[b:b + 1, :P, h:h + 1]) for t in (q, k, v, do))
+    dq_ref, _, _ = oracle.attention_backward(qs, ks, vs, dos, scale, True)
+    assert_close(to_np(dq[b:b + 1, :P, h:h + 1]), dq_ref, BF16_RTOL, "dQ prefix")
+    # dV/dK of the last T keys: only queries >= S-T see them, but those queries
+    # attend to all keys; check with the oracle on the last-T queries x all keys
+    T = 8
+    qs = to_np(q[b:b + 1, S - T:, h:h + 1])
+    dos = to_np(do[b:b + 1, S - T:, h:h + 1])
+    ks, vs = to_np(k[b:b + 1, :, h:h + 1]), to_np(v[b:b + 1, :, h:h + 1])
+    # causal mask for a suffix of queries = explicit per-row limits: emulate by
+    # running non-causal on each row's visible keys
+    dv_ref = np.zeros((T, D), np.float64)
+    dk_ref = np.zeros((T, D), np.float64)
+    for i in range(T):
+        lim = S - T + i + 1
+        _, dkr, dvr = oracle.attention_backward(qs[:, i:i + 1], ks[:, :lim], vs[:, :lim], dos[:, i:i + 1],
+                                                scale, False)
+        dk_ref[: i + 1] += dkr[0, S - T:lim, 0]
+        dv_ref[: i + 1] += dvr[0, S - T:lim, 0]
+    assert_close(to_np(dk[b, S - T:, h]), dk_ref, BF16_RTOL, "dK suffix")
+    assert_close(to_np(dv[b, S - T:, h]), dv_ref, BF16_RTOL, "dV suffix")
+
+
+MHA_CASES = [  # B, Sq, Skv, H, E(q), Ek, Ev, Dh, oProj, self-attention?
+    (2, 20, 20, 4, 64, 64, 64, 64, 64, True),
+    (2, 33, 33, 2, 128, 128, 128, 64, 96, True),
+    (1, 24, 40, 2, 64, 72, 80, 64, 64, False),
+    (2, 64, 64, 2, 256, 256, 256, 128, 256, True),
+]
+
+
+@pytest.mark.parametrize("case", MHA_CASES)
+@pytest.mark.parametrize("causal", [False, True])
+def test_mha(ffk, oracle, case, causal):
+    B, Sq, Skv, H, E, Ek, Ev, Dh, oP, self_attn = case
+    if causal and Sq != Skv:
+        pytest.skip("causal needs Sq == Skv")
+    say("mha", case, "causal", causal)
+    g = rng(Sq + E + int(causal))
+    scale = 1.0 / np.sqrt(Dh)
+    query = bf16_round(g.standard_normal((B, Sq, E)))
+    key = query if self_attn else bf16_round(g.standard_normal((B, Skv, Ek)))
+    value = query if self_attn else bf16_round(g.standard_normal((B, Skv, Ev)))
+    odesc = oracle.mha_desc(B, H, E, Ek, Ev, Dh, Dh, Dh, oP, Sq, Skv, scale, causal)
+    desc = ffk.mha_desc(B, H, E, Ek, Ev, Dh, Dh, Dh, oP, Sq, Skv, scale, causal)
+    nw = ffk.lib().ffk_mha_weight_elements(desc)
+    assert nw == H * Dh * (E + Ek + Ev) + oP * H * Dh
+    w = bf16_round(g.standard_normal((nw,)) * (2.0 / np.sqrt(E)))
+    dout = bf16_round(g.standard_normal((B, Sq, oP)))
+    out_ref = oracle.mha_forward(odesc, query, key, value, w, bf16_mode=True)
+    dq_ref, dk_ref, dv_ref, dw_ref = oracle.mha_backward(odesc, query, key, value, w, dout, bf16_mode=True)
+
+    qd = to_dev(query, torch, BT)
+    kd = qd if self_attn else to_dev(key, torch, BT)
+    vd = qd if self_attn else to_dev(value, torch, BT)
+    wd, doutd = to_dev(w, torch, BT), to_dev(dout, torch, BT)
+    reserve = ffk.mha_reserve(desc, ffk.BF16)
+    out = ffk.mha_forward(desc, qd, kd, vd, wd, reserve)
+    assert_close(to_np(out), out_ref, BF16_RTOL, "out")
+    dw = torch.zeros_like(wd)
+    dq = torch.zeros_like(qd)
+    if self_attn:
+        # key/value alias query: their gradients fold into query_grad
+        ffk.mha_backward(desc, qd, dq, kd, None, vd, None, wd, dw, doutd, reserve)
+        assert_close(to_np(dq), dq_ref + dk_ref + dv_ref, BF16_RTOL, "dquery (folded)")
+    else:
+        dk, dv = torch.zeros_like(kd), torch.zeros_like(vd)
+        ffk.mha_backward(desc, qd, dq, kd, dk, vd, dv, wd, dw, doutd, reserve)
+        assert_close(to_np(dq), dq_ref, BF16_RTOL, "dquery")
+        assert_close(to_np(dk), dk_ref, BF16_RTOL, "dkey")
+        assert_close(to_np(dv), dv_ref, BF16_RTOL, "dvalue")
+    assert_close(to_np(dw), dw_ref, BF16_RTOL, "dweight")
+    # weight_grad accumulates (CUDNN_WGRAD_MODE_ADD): a second call doubles it
+    dq2 = torch.zeros_like(qd)
+    if self_attn:
+        ffk.mha_backward(desc, qd, dq2, kd, None, vd, None, wd, dw, doutd, reserve)
+    else:
+        ffk.mha_backward(desc, qd, dq2, kd, torch.zeros_like(kd), vd, torch.zeros_like(vd), wd, dw, doutd, reserve)
+    assert_close(to_np(dw), 2 * dw_ref, BF16_RTOL * 1.5, "dweight accumulated")
+
+
+def test_mha_separate_grads_when_aliased(ffk, oracle):
+    say("mha aliased, separate grads")
+    B, S, H, E, Dh = 1, 16, 2, 64, 64
+    g = rng(8)
+    x = bf16_round(g.standard_normal((B, S, E)))
+    odesc = oracle.mha_desc(B, H, E, E, E, Dh, Dh, Dh, E, S, S, 0.125, False)
+    desc = ffk.mha_desc(B, H, E, E, E, Dh, Dh, Dh, E, S, S, 0.125, False)
+    w = bf16_round(g.standard_normal((ffk.lib().ffk_mha_weight_elements(desc),)) * 0.2)
+    dout = bf16_round(g.standard_normal((B, S, E)))
+    dq_ref, dk_ref, dv_ref, _ = oracle.mha_backward(odesc, x, x, x, w, dout, bf16_mode=True)
+    xd, wd, dd = to_dev(x, torch, BT), to_dev(w, torch, BT), to_dev(dout, torch, BT)
+    reserve = ffk.mha_reserve(desc, ffk.BF16)
+    ffk.mha_forward(desc, xd, xd, xd, wd, reserve)
+    dq, dk, dv = (torch.zeros_like(xd) for _ in range(3))
+    dw = torch.zeros_like(wd)
+    ffk.mha_backward(desc, xd, dq, xd, dk, xd, dv, wd, dw, dd, reserve)
+    assert_close(to_np(dq), dq_ref, BF16_RTOL, "dq")
+    assert_close(to_np(dk), dk_ref, BF16_RTOL, "dk")
+    assert_close(to_np(dv), dv_ref, BF16_RTOL, "dv")
+
+
+def test_mha_errors(ffk):
+    desc = ffk.mha_desc(1, 2, 64, 64, 64, 64, 64, 64, 64, 8, 8)
+    x = torch.zeros((1, 8, 64), dtype=BT, device="cuda")
+    w = torch.zeros((ffk.lib().ffk_mha_weight_elements(desc),), dtype=BT, device="cuda")
+    small = torch.zeros((16,), dtype=torch.uint8, device="cuda")
+    with pytest.raises(ffk.FFKError, match="reserve"):
+        ffk.mha_forward(desc, x, x, x, w, small)
+    bad = ffk.mha_desc(1, 2, 64, 64, 64, 48, 48, 48, 64, 8, 8)
+    with pytest.raises(ffk.FFKError, match="projection size"):
+        ffk.mha_forward(bad, x, x, x, w, ffk.mha_reserve(desc, ffk.BF16))
