@@ -62,6 +62,19 @@ class MHADesc(ctypes.Structure):
     ]
 
 
+class EncoderLayerDesc(ctypes.Structure):
+    _fields_ = [
+        ("batch", c_i64), ("seq", c_i64), ("d_model", c_i64), ("heads", c_i64), ("d_ff", c_i64),
+        ("dropout_rate", c_f), ("seed", c_u64), ("ln_eps", c_f), ("attn_scale", c_f),
+        ("causal", c_int), ("pre_layer_norm", c_int), ("activation", c_int),
+    ]
+
+
+class EncoderLayerParams(ctypes.Structure):
+    _fields_ = [(n, c_p) for n in ("ln1_gamma", "ln1_beta", "attn_weight", "ln2_gamma", "ln2_beta",
+                                   "w1", "b1", "w2", "b2")]
+
+
 # name -> (restype, argtypes); must list every symbol include/ffk.h declares.
 SIGNATURES = {
     "ffk_last_error": (ctypes.c_char_p, []),
@@ -119,6 +132,13 @@ SIGNATURES = {
                                 c_p, c_sz]),
     "ffk_mha_backward": (c_int, [c_p, c_int, ctypes.POINTER(MHADesc), c_p, c_p, c_p, c_p, c_p,
                                  c_p, c_p, c_p, c_p, c_p, c_sz, c_int]),
+    "ffk_encoder_layer_workspace_bytes": (c_sz, [ctypes.POINTER(EncoderLayerDesc), c_int]),
+    "ffk_encoder_layer_forward": (c_int, [c_p, c_int, ctypes.POINTER(EncoderLayerDesc),
+                                          ctypes.POINTER(EncoderLayerParams), c_p, c_p, c_p, c_sz]),
+    "ffk_encoder_layer_backward": (c_int, [c_p, c_int, ctypes.POINTER(EncoderLayerDesc),
+                                           ctypes.POINTER(EncoderLayerParams),
+                                           ctypes.POINTER(EncoderLayerParams), c_p, c_p, c_p, c_p,
+                                           c_sz]),
 }
 
 _lib = None
@@ -200,7 +220,7 @@ def linear_backward(y, dy, x, w, dx=None, dw=None, db=None, activation=ACT_NONE,
     check(lib().ffk_linear_backward(current_stream(), dtype_of(x), activation, relu_grad_mode,
                                     ptr(y), ptr(dy), ptr(x), ptr(dx), ptr(w), ptr(dw), ptr(db),
                                     batch, in_dim, out_dim, ptr(workspace), ws_bytes,
-                                    int(accumulate)))
+                                    7 if accumulate is True else int(accumulate)))
     return dx, dw, db
 
 
@@ -420,3 +440,40 @@ def mha_backward(desc, query, dquery, key, dkey, value, dvalue, weight, dweight,
                                  ptr(dvalue), ptr(weight), ptr(dweight), ptr(out_grad),
                                  ptr(reserve), reserve.numel(), int(accumulate)))
     return dquery, dkey, dvalue, dweight
+
+
+PARAM_NAMES = ("ln1_gamma", "ln1_beta", "attn_weight", "ln2_gamma", "ln2_beta", "w1", "b1", "w2", "b2")
+
+
+def encoder_layer_param_shapes(desc):
+    """name -> shape of every weight tensor of one encoder layer."""
+    E, F, H = desc.d_model, desc.d_ff, desc.heads
+    hd = E // H
+    return {
+        "ln1_gamma": (E,), "ln1_beta": (E,), "attn_weight": (H * hd * 3 * E + E * H * hd,),
+        "ln2_gamma": (E,), "ln2_beta": (E,), "w1": (F, E), "b1": (F,), "w2": (E, F), "b2": (E,),
+    }
+
+
+def encoder_layer_params(tensors):
+    return EncoderLayerParams(*[ptr(tensors[n]) for n in PARAM_NAMES])
+
+
+def encoder_layer_workspace(desc, dtype, device="cuda"):
+    torch = _torch()
+    n = lib().ffk_encoder_layer_workspace_bytes(ctypes.byref(desc), dtype)
+    return torch.empty((n,), dtype=torch.uint8, device=device)
+
+
+def encoder_layer_forward(desc, weights, x, y, workspace):
+    check(lib().ffk_encoder_layer_forward(current_stream(), dtype_of(x), ctypes.byref(desc),
+                                          ctypes.byref(weights), ptr(x), ptr(y), ptr(workspace),
+                                          workspace.numel()))
+    return y
+
+
+def encoder_layer_backward(desc, weights, grads, x, dy, dx, workspace):
+    check(lib().ffk_encoder_layer_backward(current_stream(), dtype_of(x), ctypes.byref(desc),
+                                           ctypes.byref(weights), ctypes.byref(grads), ptr(x),
+                                           ptr(dy), ptr(dx), ptr(workspace), workspace.numel()))
+    return dx

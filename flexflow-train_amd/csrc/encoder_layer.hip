@@ -1,0 +1,223 @@
+// One transformer encoder layer (forward + backward) as a sequence of the
+// operator entry points, in the order the reference's local executor would
+// run the layer's ops (forward in topological order, backward in reverse).
+// Host code only: every arithmetic step is one of the ffk_* kernels.
+#include "ffk_common.h"
+
+namespace ffk {
+
+struct LayerWs {
+  // forward activations kept for backward
+  size_t h1, mean1, rstd1, attn_out, attn_drop, x1, h2, mean2, rstd2;
+  size_t f1, act1, act1_drop, f2, f2_drop, pre2;
+  // backward scratch
+  size_t g_f2, g_act1_drop, g_act1, g_f1, g_h2, g_x1, g_attn, g_h1, g_tmp;
+  size_t mha_reserve, ln_ws, lin_ws;
+  size_t total;
+};
+
+static size_t a256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static ffk_mha_desc_t mha_desc(ffk_encoder_layer_desc_t const *d) {
+  ffk_mha_desc_t m;
+  int64_t const hd = d->d_model / d->heads;
+  m.num_samples = d->batch;
+  m.num_heads = d->heads;
+  m.q_size = m.k_size = m.v_size = d->d_model;
+  m.q_proj_size = m.k_proj_size = m.v_proj_size = hd;
+  m.o_proj_size = d->d_model;
+  m.qo_seq_length = m.kv_seq_length = d->seq;
+  m.scale = d->attn_scale;
+  m.causal = d->causal;
+  return m;
+}
+
+static LayerWs layout(ffk_encoder_layer_desc_t const *d, int dtype) {
+  LayerWs L;
+  size_t const es = dtype_size(dtype);
+  size_t const T = (size_t)(d->batch * d->seq);
+  size_t const td = a256(T * (size_t)d->d_model * es);
+  size_t const tf = a256(T * (size_t)d->d_ff * es);
+  size_t const tr = a256(T * sizeof(float));
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off += bytes; return o; };
+  L.h1 = take(td); L.mean1 = take(tr); L.rstd1 = take(tr);
+  L.attn_out = take(td); L.attn_drop = take(td); L.x1 = take(td);
+  L.h2 = take(td); L.mean2 = take(tr); L.rstd2 = take(tr);
+  L.f1 = take(tf); L.act1 = take(tf); L.act1_drop = take(tf);
+  L.f2 = take(td); L.f2_drop = take(td); L.pre2 = take(td);
+  L.g_f2 = take(td); L.g_act1_drop = take(tf); L.g_act1 = take(tf); L.g_f1 = take(tf);
+  L.g_h2 = take(td); L.g_x1 = take(td); L.g_attn = take(td); L.g_h1 = take(td); L.g_tmp = take(td);
+  ffk_mha_desc_t m = mha_desc(d);
+  L.mha_reserve = take(a256(ffk_mha_reserve_bytes(&m, dtype)));
+  L.ln_ws = take(a256(ffk_layer_norm_backward_workspace_bytes((int64_t)T, d->d_model)));
+  size_t l1 = ffk_linear_backward_workspace_bytes(dtype, FFK_ACT_RELU, 1, (int64_t)T, d->d_ff);
+  size_t l2 = ffk_linear_backward_workspace_bytes(dtype, FFK_ACT_NONE, 1, (int64_t)T, d->d_model);
+  L.lin_ws = take(a256(l1 > l2 ? l1 : l2));
+  L.total = off;
+  return L;
+}
+
+static int check_layer(char const *who, int dtype, ffk_encoder_layer_desc_t const *d) {
+  FFK_REQUIRE(d != nullptr, "%s: NULL descriptor", who);
+  FFK_REQUIRE(dtype == FFK_BF16, "%s: dtype %d not supported (bf16 only)", who, dtype);
+  FFK_REQUIRE(d->batch > 0 && d->seq > 0 && d->d_model > 0 && d->heads > 0 && d->d_ff > 0,
+              "%s: non-positive size", who);
+  FFK_REQUIRE(d->d_model % d->heads == 0, "%s: d_model not divisible by heads", who);
+  FFK_REQUIRE(d->activation == FFK_ACT_RELU || d->activation == FFK_ACT_GELU,
+              "%s: Unhandled activation function %d", who, d->activation);
+  return FFK_OK;
+}
+
+#define FFK_TRY(expr)                                                          \
+  do {                                                                         \
+    int rc__ = (expr);                                                         \
+    if (rc__ != FFK_OK) return rc__;                                           \
+  } while (0)
+
+}  // namespace ffk
+
+using namespace ffk;
+
+extern "C" size_t ffk_encoder_layer_workspace_bytes(ffk_encoder_layer_desc_t const *d, int dtype) {
+  if (d == nullptr || dtype_size(dtype) == 0) return 0;
+  return layout(d, dtype).total;
+}
+
+extern "C" int ffk_encoder_layer_forward(ffk_stream_t st, int dtype,
+                                         ffk_encoder_layer_desc_t const *d,
+                                         ffk_encoder_layer_params_t const *w,
+                                         void const *x, void *y, void *workspace,
+                                         size_t workspace_bytes) {
+  FFK_TRY(check_layer("encoder_layer_forward", dtype, d));
+  FFK_REQUIRE(w && x && y, "encoder_layer_forward: NULL argument");
+  LayerWs L = layout(d, dtype);
+  if (workspace == nullptr || workspace_bytes < L.total) {
+    return fail(FFK_ERR_WORKSPACE, "encoder_layer_forward: workspace of %zu bytes needed, %zu given",
+                L.total, workspace_bytes);
+  }
+  uint8_t *ws = static_cast<uint8_t *>(workspace);
+  int64_t const T = d->batch * d->seq, E = d->d_model, F = d->d_ff;
+  ffk_mha_desc_t m = mha_desc(d);
+  float const p = d->dropout_rate;
+  bool const gelu = d->activation == FFK_ACT_GELU;
+  auto mean = [&](size_t o) { return reinterpret_cast<float *>(ws + o); };
+
+  void const *attn_in = x;
+  if (d->pre_layer_norm) {
+    FFK_TRY(ffk_layer_norm_forward(st, dtype, x, ws + L.h1, w->ln1_gamma, w->ln1_beta,
+                                   mean(L.mean1), mean(L.rstd1), T, E, d->ln_eps));
+    attn_in = ws + L.h1;
+  }
+  FFK_TRY(ffk_mha_forward(st, dtype, &m, attn_in, attn_in, attn_in, w->attn_weight, ws + L.attn_out,
+                          ws + L.mha_reserve, L.ln_ws - L.mha_reserve));
+  void const *attn_res = ws + L.attn_out;
+  if (d->pre_layer_norm) {  // the reference applies no dropout after attention
+    FFK_TRY(ffk_dropout_forward(st, dtype, ws + L.attn_out, ws + L.attn_drop, T * E, p, d->seed + 0, 0));
+    attn_res = ws + L.attn_drop;
+  }
+  void *ffn_in;
+  if (d->pre_layer_norm) {
+    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, attn_res, x, ws + L.x1, T * E, T * E, T * E));
+    FFK_TRY(ffk_layer_norm_forward(st, dtype, ws + L.x1, ws + L.h2, w->ln2_gamma, w->ln2_beta,
+                                   mean(L.mean2), mean(L.rstd2), T, E, d->ln_eps));
+    ffn_in = ws + L.h2;
+  } else {
+    // h1 = attn + x ; x1 = LN1(h1)
+    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, attn_res, x, ws + L.h1, T * E, T * E, T * E));
+    FFK_TRY(ffk_layer_norm_forward(st, dtype, ws + L.h1, ws + L.x1, w->ln1_gamma, w->ln1_beta,
+                                   mean(L.mean1), mean(L.rstd1), T, E, d->ln_eps));
+    ffn_in = ws + L.x1;
+  }
+  // dense(d_ff, activation) -> dropout -> dense(d_model) -> dropout
+  if (gelu) {
+    FFK_TRY(ffk_linear_forward(st, dtype, FFK_ACT_NONE, ffn_in, ws + L.f1, w->w1, w->b1, T, E, F));
+    FFK_TRY(ffk_element_unary_forward(st, dtype, FFK_OP_GELU, 0.0f, ws + L.f1, ws + L.act1, T * F));
+  } else {
+    FFK_TRY(ffk_linear_forward(st, dtype, FFK_ACT_RELU, ffn_in, ws + L.act1, w->w1, w->b1, T, E, F));
+  }
+  FFK_TRY(ffk_dropout_forward(st, dtype, ws + L.act1, ws + L.act1_drop, T * F, p, d->seed + 1, 0));
+  FFK_TRY(ffk_linear_forward(st, dtype, FFK_ACT_NONE, ws + L.act1_drop, ws + L.f2, w->w2, w->b2, T, F, E));
+  FFK_TRY(ffk_dropout_forward(st, dtype, ws + L.f2, ws + L.f2_drop, T * E, p, d->seed + 2, 0));
+  if (d->pre_layer_norm) {
+    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.x1, ws + L.f2_drop, y, T * E, T * E, T * E));
+  } else {
+    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.x1, ws + L.f2_drop, ws + L.pre2, T * E, T * E, T * E));
+    FFK_TRY(ffk_layer_norm_forward(st, dtype, ws + L.pre2, y, w->ln2_gamma, w->ln2_beta,
+                                   mean(L.mean2), mean(L.rstd2), T, E, d->ln_eps));
+  }
+  return FFK_OK;
+}
+
+extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
+                                          ffk_encoder_layer_desc_t const *d,
+                                          ffk_encoder_layer_params_t const *w,
+                                          ffk_encoder_layer_params_t const *g,
+                                          void const *x, void const *dy, void *dx,
+                                          void *workspace, size_t workspace_bytes) {
+  FFK_TRY(check_layer("encoder_layer_backward", dtype, d));
+  FFK_REQUIRE(w && g && x && dy && dx, "encoder_layer_backward: NULL argument");
+  LayerWs L = layout(d, dtype);
+  if (workspace == nullptr || workspace_bytes < L.total) {
+    return fail(FFK_ERR_WORKSPACE, "encoder_layer_backward: workspace of %zu bytes needed, %zu given",
+                L.total, workspace_bytes);
+  }
+  uint8_t *ws = static_cast<uint8_t *>(workspace);
+  int64_t const T = d->batch * d->seq, E = d->d_model, F = d->d_ff;
+  ffk_mha_desc_t m = mha_desc(d);
+  float const p = d->dropout_rate;
+  bool const gelu = d->activation == FFK_ACT_GELU;
+  auto mean = [&](size_t o) { return reinterpret_cast<float *>(ws + o); };
+  size_t const ln_ws_bytes = L.lin_ws - L.ln_ws, lin_ws_bytes = L.total - L.lin_ws;
+
+  // ---- tail: y = x1 + f2_drop (pre-LN) or y = LN2(x1 + f2_drop) (post-LN)
+  void const *g_sum = dy;  // gradient of (x1 + f2_drop)
+  if (!d->pre_layer_norm) {
+    FFK_TRY(ffk_layer_norm_backward(st, dtype, dy, ws + L.pre2, mean(L.mean2), mean(L.rstd2), w->ln2_gamma,
+                                    ws + L.g_tmp, g->ln2_gamma, g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+    g_sum = ws + L.g_tmp;
+  }
+  // ---- FFN backward
+  FFK_TRY(ffk_dropout_backward(st, dtype, g_sum, ws + L.g_f2, T * E, p, d->seed + 2, 0, 0));
+  FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_NONE, 0, ws + L.f2, ws + L.g_f2, ws + L.act1_drop,
+                              ws + L.g_act1_drop, w->w2, g->w2, g->b2, T, F, E, ws + L.lin_ws, lin_ws_bytes, FFK_ACC_WEIGHT | FFK_ACC_BIAS));
+  FFK_TRY(ffk_dropout_backward(st, dtype, ws + L.g_act1_drop, ws + L.g_act1, T * F, p, d->seed + 1, 0, 0));
+  void const *ffn_in = d->pre_layer_norm ? ws + L.h2 : ws + L.x1;
+  if (gelu) {
+    FFK_TRY(ffk_element_unary_backward(st, dtype, FFK_OP_GELU, 0.0f, ws + L.act1, ws + L.g_act1, ws + L.f1,
+                                       ws + L.g_f1, T * F, 0));
+    FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_NONE, 0, ws + L.f1, ws + L.g_f1, ffn_in, ws + L.g_h2,
+                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws, lin_ws_bytes, FFK_ACC_WEIGHT | FFK_ACC_BIAS));
+  } else {
+    FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_RELU, 0, ws + L.act1, ws + L.g_act1, ffn_in, ws + L.g_h2,
+                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws, lin_ws_bytes, FFK_ACC_WEIGHT | FFK_ACC_BIAS));
+  }
+  // ---- gradient reaching x1
+  if (d->pre_layer_norm) {
+    FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h2, ws + L.x1, mean(L.mean2), mean(L.rstd2), w->ln2_gamma,
+                                    ws + L.g_x1, g->ln2_gamma, g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.g_x1, dy, ws + L.g_x1, T * E, T * E, T * E));
+  } else {
+    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.g_h2, g_sum, ws + L.g_x1, T * E, T * E, T * E));
+  }
+  // ---- attention block backward
+  void const *g_attn_res;  // gradient of (attn (+dropout) + x)
+  if (d->pre_layer_norm) {
+    g_attn_res = ws + L.g_x1;
+    FFK_TRY(ffk_dropout_backward(st, dtype, g_attn_res, ws + L.g_attn, T * E, p, d->seed + 0, 0, 0));
+    FFK_TRY(ffk_mha_backward(st, dtype, &m, ws + L.h1, ws + L.g_h1, ws + L.h1, nullptr, ws + L.h1, nullptr,
+                             w->attn_weight, g->attn_weight, ws + L.g_attn, ws + L.mha_reserve,
+                             L.ln_ws - L.mha_reserve, 0));
+    FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h1, x, mean(L.mean1), mean(L.rstd1), w->ln1_gamma, dx,
+                                    g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, dx, g_attn_res, dx, T * E, T * E, T * E));
+  } else {
+    FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_x1, ws + L.h1, mean(L.mean1), mean(L.rstd1), w->ln1_gamma,
+                                    ws + L.g_attn, g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+    g_attn_res = ws + L.g_attn;
+    FFK_TRY(ffk_mha_backward(st, dtype, &m, x, dx, x, nullptr, x, nullptr, w->attn_weight, g->attn_weight,
+                             g_attn_res, ws + L.mha_reserve, L.ln_ws - L.mha_reserve, 0));
+    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, dx, g_attn_res, dx, T * E, T * E, T * E));
+  }
+  return FFK_OK;
+}

@@ -129,15 +129,16 @@ extern "C" int ffk_linear_backward(
     ws += align256((size_t)n * dtype_size(dtype));
   }
   GemmEpilogue ep;
-  ep.accumulate = accumulate != 0;
   int rc;
   if (input_grad != nullptr) {
+    ep.accumulate = (accumulate & FFK_ACC_INPUT) != 0;
     // input_grad[batch,in] = g[batch,out] . weight[out,in]
     rc = gemm_dispatch(st, dtype, false, false, batch, in_dim, out_dim, g, out_dim,
                        weight, in_dim, input_grad, in_dim, ep);
     if (rc != FFK_OK) return rc;
   }
   if (weight_grad != nullptr) {
+    ep.accumulate = (accumulate & FFK_ACC_WEIGHT) != 0;
     // weight_grad[out,in] = g[batch,out]^T . input[batch,in]
     rc = gemm_dispatch(st, dtype, true, false, out_dim, in_dim, batch, g, out_dim,
                        input, in_dim, weight_grad, in_dim, ep);
@@ -145,7 +146,7 @@ extern "C" int ffk_linear_backward(
   }
   if (bias_grad != nullptr) {
     rc = colsum_dispatch(st, dtype, g, out_dim, batch, out_dim, bias_grad,
-                         accumulate != 0, reinterpret_cast<float *>(ws));
+                         (accumulate & FFK_ACC_BIAS) != 0, reinterpret_cast<float *>(ws));
     if (rc != FFK_OK) return rc;
   }
   return FFK_OK;

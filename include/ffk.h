@@ -137,6 +137,10 @@ int ffk_event_elapsed_ms(ffk_event_t start, ffk_event_t stop, float *ms);
  *     0 = g = output_grad * [output > 0]  (reference GPU, cuda_helper.cu:60-64)
  *     1 = g = [output_grad > 0] ? 1 : 0   (reference CPU, linear_kernels_cpu.cc:46-52,65-71)
  *   Any of input_grad / weight_grad / bias_grad may be NULL (skipped).
+ *   accumulate is a bit mask of FFK_ACC_INPUT / FFK_ACC_WEIGHT / FFK_ACC_BIAS
+ *   (FFK_ACC_ALL = the reference GPU path, beta = 1 on all three products,
+ *   linear_kernels.cu:262,311,334; 0 = the reference CPU path, which
+ *   overwrites, linear_kernels_cpu.cc:80-93).
  *   workspace: device scratch of ffk_linear_backward_workspace_bytes(...)
  *   bytes (holds g when there is an activation, and the partial column sums
  *   of the bias gradient); may be NULL when that size is 0.                  */
@@ -145,6 +149,7 @@ int ffk_linear_forward(ffk_stream_t stream, int dtype, int activation,
                        void const *input, void *output, void const *weight,
                        void const *bias, int64_t batch, int64_t in_dim,
                        int64_t out_dim);
+enum { FFK_ACC_INPUT = 1, FFK_ACC_WEIGHT = 2, FFK_ACC_BIAS = 4, FFK_ACC_ALL = 7 };
 size_t ffk_linear_backward_workspace_bytes(int dtype, int activation,
                                            int use_bias, int64_t batch,
                                            int64_t out_dim);
@@ -368,6 +373,59 @@ int ffk_mha_backward(ffk_stream_t stream, int dtype, ffk_mha_desc_t const *desc,
                      void const *weight, void *weight_grad,
                      void const *output_grad, void *reserve,
                      size_t reserve_bytes, int accumulate);
+
+/* ------------------------------------------------------------------------ */
+/* One transformer encoder layer, forward and backward, sequenced over the
+ * operator entry points above in the order lib/local-execution runs them
+ * (topological FWD pass, then BWD pass in reverse;
+ * lib/local-execution/src/local-execution/computation_graph_instance.cc:104-137)
+ * for the op list of create_transformer_encoder_layer
+ * (lib/models/src/models/transformer/transformer.cc:19-67).
+ *   pre_layer_norm == 0: the reference's order
+ *       y = LN2(x1 + FFN(x1)),  x1 = LN1(x + MHA(x,x,x))
+ *   pre_layer_norm == 1:
+ *       x1 = x + drop(MHA(LN1(x)));  y = x1 + drop(W2 drop(act(W1 LN2(x1) + b1)) + b2)
+ *   FFN = dense(d_ff, activation, bias) -> dropout -> dense(d_model, bias) -> dropout;
+ *   activation: FFK_ACT_RELU (reference) or FFK_ACT_GELU (exact erf GELU as an
+ *   ElementUnary op).  MHA: heads x (d_model/heads), no bias, `attn_scale`,
+ *   `causal`.  Dropout op i uses seed + i.
+ * Tensors: x, y, dy, dx [batch*seq, d_model]; weights as named.  Weight
+ * gradients are accumulated into (zero them for a fresh step); dx is
+ * overwritten.  The workspace keeps every saved activation between the two
+ * calls.                                                                     */
+/* ------------------------------------------------------------------------ */
+typedef struct {
+  int64_t batch, seq, d_model, heads, d_ff;
+  float dropout_rate;
+  uint64_t seed;
+  float ln_eps;
+  float attn_scale;
+  int causal;
+  int pre_layer_norm;
+  int activation;
+} ffk_encoder_layer_desc_t;
+
+typedef struct {
+  void *ln1_gamma, *ln1_beta; /* [d_model] */
+  void *attn_weight;          /* ffk_mha_weight_elements() */
+  void *ln2_gamma, *ln2_beta; /* [d_model] */
+  void *w1, *b1;              /* [d_ff, d_model], [d_ff] */
+  void *w2, *b2;              /* [d_model, d_ff], [d_model] */
+} ffk_encoder_layer_params_t;
+
+size_t ffk_encoder_layer_workspace_bytes(ffk_encoder_layer_desc_t const *desc,
+                                         int dtype);
+int ffk_encoder_layer_forward(ffk_stream_t stream, int dtype,
+                              ffk_encoder_layer_desc_t const *desc,
+                              ffk_encoder_layer_params_t const *weights,
+                              void const *x, void *y, void *workspace,
+                              size_t workspace_bytes);
+int ffk_encoder_layer_backward(ffk_stream_t stream, int dtype,
+                               ffk_encoder_layer_desc_t const *desc,
+                               ffk_encoder_layer_params_t const *weights,
+                               ffk_encoder_layer_params_t const *weight_grads,
+                               void const *x, void const *dy, void *dx,
+                               void *workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

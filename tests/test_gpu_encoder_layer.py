@@ -1,0 +1,82 @@
+"""Transformer encoder layer forward+backward (BASELINE config 2 structure)
+against the layer composed from oracle operators."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from layer_oracle import layer_forward_backward, make_params
+from util import assert_close, bf16_round, rng, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+BT = torch.bfloat16
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def run_device(ffk, cfg, params, x, dy):
+    desc = ffk.EncoderLayerDesc(cfg["batch"], cfg["seq"], cfg["d_model"], cfg["heads"], cfg["d_ff"],
+                                cfg["p"], cfg["seed"], cfg["eps"], cfg["scale"], int(cfg["causal"]),
+                                int(cfg["pre_ln"]), ffk.ACT_GELU if cfg["gelu"] else ffk.ACT_RELU)
+    wt = {k: to_dev(v, torch, BT) for k, v in params.items()}
+    gt = {k: torch.zeros_like(v) for k, v in wt.items()}
+    xd, dyd = to_dev(x, torch, BT), to_dev(dy, torch, BT)
+    y, dx = torch.empty_like(xd), torch.empty_like(xd)
+    ws = ffk.encoder_layer_workspace(desc, ffk.BF16)
+    W, G = ffk.encoder_layer_params(wt), ffk.encoder_layer_params(gt)
+    ffk.encoder_layer_forward(desc, W, xd, y, ws)
+    ffk.encoder_layer_backward(desc, W, G, xd, dyd, dx, ws)
+    torch.cuda.synchronize()
+    return to_np(y), to_np(dx), {k: to_np(v) for k, v in gt.items()}
+
+
+@pytest.mark.parametrize("pre_ln,gelu", [(True, True), (False, False)])
+@pytest.mark.parametrize("p", [0.0, 0.1])
+def test_encoder_layer_small(ffk, oracle, pre_ln, gelu, p):
+    cfg = dict(batch=2, seq=48, d_model=128, heads=2, d_ff=256, p=p, seed=1234, eps=1e-5,
+               scale=1.0 / 8.0, causal=False, pre_ln=pre_ln, gelu=gelu)
+    say("encoder layer", cfg)
+    g = rng(17)
+    params = make_params(g, cfg, bf16_round)
+    # larger weights than N(0, 0.02) so that every branch contributes visibly
+    for k in ("attn_weight", "w1", "w2"):
+        params[k] = bf16_round(params[k] * 4)
+    x = bf16_round(g.standard_normal((cfg["batch"], cfg["seq"], cfg["d_model"])))
+    dy = bf16_round(g.standard_normal(x.shape))
+    y_ref, dx_ref, g_ref = layer_forward_backward(oracle, cfg, params, x, dy)
+    y, dx, grads = run_device(ffk, cfg, params, x, dy)
+    # bf16 tolerance with headroom for a dozen chained bf16 roundings.  ReLU's
+    # gradient is discontinuous: a pre-activation that rounds to +-tiny on one
+    # side and to the other sign on the other flips one mask bit and moves a
+    # handful of gradient elements, so the ReLU variant tolerates 1% outliers.
+    frac = 0.0 if gelu else 1e-2
+    assert_close(y, y_ref, 2e-2, "y")
+    assert_close(dx, dx_ref, 3e-2, "dx", frac)
+    for k in g_ref:
+        assert_close(grads[k].reshape(g_ref[k].shape), g_ref[k], 3e-2, "grad " + k, frac)
+
+
+def test_encoder_layer_config2_shape_runs_and_is_deterministic(ffk):
+    """BASELINE config 2 at full size: B 8, S 512, d 1024, H 16, FFN 4096,
+    pre-LN, GELU, dropout 0.1.  Size-independent checks: finite outputs,
+    bit-identical repeat (no atomics on this path), dropout really drops."""
+    cfg = dict(batch=8, seq=512, d_model=1024, heads=16, d_ff=4096, p=0.1, seed=7, eps=1e-5,
+               scale=0.125, causal=False, pre_ln=True, gelu=True)
+    say("encoder layer cfg2 full size")
+    g = rng(2)
+    params = make_params(g, cfg, bf16_round)
+    x = bf16_round(g.standard_normal((8, 512, 1024)))
+    dy = bf16_round(g.standard_normal(x.shape))
+    y1, dx1, g1 = run_device(ffk, cfg, params, x, dy)
+    y2, dx2, g2 = run_device(ffk, cfg, params, x, dy)
+    assert np.isfinite(y1).all() and np.isfinite(dx1).all()
+    assert np.array_equal(y1, y2) and np.array_equal(dx1, dx2)
+    for k in g1:
+        assert np.isfinite(g1[k]).all() and np.array_equal(g1[k], g2[k]), k
+    cfg0 = dict(cfg, p=0.0)
+    y0, _, _ = run_device(ffk, cfg0, params, x, dy)
+    assert not np.array_equal(y0, y1)
