@@ -52,21 +52,28 @@ def make_device_state(ffk, torch, cfg):
         if name.endswith("gamma"):
             t = t + 1.0
         wt[name] = t.to(bt)
-    gt = {k: torch.zeros_like(v) for k, v in wt.items()}
+    # all weight gradients live in one flat buffer (16-byte aligned slices) so a
+    # training step clears them with a single fill
+    sizes = {k: (v.numel() + 7) // 8 * 8 for k, v in wt.items()}
+    flat = torch.zeros((sum(sizes.values()),), dtype=bt, device="cuda")
+    gt, off = {}, 0
+    for k, v in wt.items():
+        gt[k] = flat[off:off + v.numel()].view(v.shape)
+        off += sizes[k]
     T = cfg["batch"] * cfg["seq"]
     x = torch.randn((T, cfg["d_model"]), device="cuda", generator=gen).to(bt)
     dy = torch.randn((T, cfg["d_model"]), device="cuda", generator=gen).to(bt)
     y, dx = torch.empty_like(x), torch.empty_like(x)
     ws = ffk.encoder_layer_workspace(desc, ffk.BF16)
-    return dict(desc=desc, wt=wt, gt=gt, x=x, dy=dy, y=y, dx=dx, ws=ws,
+    return dict(desc=desc, wt=wt, gt=gt, grad_flat=flat, x=x, dy=dy, y=y, dx=dx, ws=ws,
                 W=ffk.encoder_layer_params(wt), G=ffk.encoder_layer_params(gt))
 
 
 def step(ffk, st):
     # one training step of the layer: fresh weight gradients, forward, backward
-    for g in st["gt"].values():
-        ffk.check(ffk.lib().ffk_fill_zero(g.data_ptr(), g.numel() * g.element_size(),
-                                          ffk.current_stream()))
+    g = st["grad_flat"]
+    ffk.check(ffk.lib().ffk_fill_zero(g.data_ptr(), g.numel() * g.element_size(),
+                                      ffk.current_stream()))
     ffk.encoder_layer_forward(st["desc"], st["W"], st["x"], st["y"], st["ws"])
     ffk.encoder_layer_backward(st["desc"], st["W"], st["G"], st["x"], st["dy"], st["dx"], st["ws"])
 

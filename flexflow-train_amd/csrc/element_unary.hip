@@ -23,7 +23,7 @@ struct UnaryFwd {
     else if (OP == FFK_OP_POW) r = powf(v, s);
     else if (OP == FFK_OP_EXP) r = expf(v);
     else if (OP == FFK_OP_IDENTITY) r = v;
-    else if (OP == FFK_OP_GELU) r = v * 0.5f * erfcf(-v * FFK_SQRT1_2);
+    else if (OP == FFK_OP_GELU) r = v * (0.5f + 0.5f * erff(v * FFK_SQRT1_2));  // = x/2 erfc(-x/sqrt2)
     else if (OP == FFK_OP_RSQRT) r = 1.0f / sqrtf(v);
     else if (OP == FFK_OP_SIN) r = sinf(v);
     else if (OP == FFK_OP_COS) r = cosf(v);
@@ -53,8 +53,8 @@ struct UnaryBwd {
     else if (OP == FFK_OP_IDENTITY) g = dy;
     else if (OP == FFK_OP_GELU)
       // d/dx [x Phi(x)] = Phi(x) + x phi(x)
-      g = dy * (0.5f * erfcf(-x * FFK_SQRT1_2) +
-                x * FFK_INV_SQRT_2PI * expf(-0.5f * x * x));
+      g = dy * (0.5f + 0.5f * erff(x * FFK_SQRT1_2) +
+                x * FFK_INV_SQRT_2PI * __expf(-0.5f * x * x));
     else if (OP == FFK_OP_GELU_REFERENCE_GRAD)
       // literal text of element_unary_kernels.cu:226-231
       g = dy * (0.5f * erfcf(-x * FFK_SQRT1_2) -

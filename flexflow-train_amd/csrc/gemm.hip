@@ -13,6 +13,7 @@
 // These replace the cublasGemmEx calls of the reference
 // (lib/kernels/src/cuda/ops/linear_kernels.cu:143,163,249,298,321).
 #include "gemm.h"
+#include <stdlib.h>
 
 namespace ffk {
 
@@ -289,6 +290,257 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// bf16 MFMA kernel, pipelined variant for shapes that tile exactly:
+//  * operand tiles go global -> LDS directly (global_load_lds_dwordx4, no VGPR
+//    staging, no LDS write instructions) into a ring of STAGES buffers, so the
+//    loads of the next STAGES-1 k-tiles are in flight while one is consumed --
+//    this is what hides HBM/L2 latency when only one workgroup fits a CU;
+//  * a direct load writes 64 lanes x 16 B contiguously, so bank conflicts are
+//    avoided by permuting which 16-byte chunk each lane FETCHES (an XOR
+//    swizzle) instead of padding rows;
+//  * the accumulator tile is computed transposed (B as the first MFMA operand)
+//    so that a lane holds 4 consecutive output columns, staged through LDS and
+//    written to HBM as full 16-byte chunks with bias/activation/accumulate
+//    applied on the way.
+// ---------------------------------------------------------------------------
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+typedef void const __attribute__((address_space(1))) * gptr_t;
+typedef void __attribute__((address_space(3))) * lptr_t;
+
+template <int BM, int BN, int WM, int WN, int BK, int STAGES, bool TA, bool TB>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_kernel(
+    bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
+    int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+    bf16 const *__restrict__ bias, int act, int accumulate) {
+  constexpr int NW = (BM / WM) * (BN / WN);
+  constexpr int NT = NW * 64;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr bool TBL = (TB == false);  // B tile lies as [BK][BN]
+  constexpr int A_ELEMS = BM * BK, B_ELEMS = BN * BK;
+  constexpr int A_LOADS = A_ELEMS / 8 / NT, B_LOADS = B_ELEMS / 8 / NT;
+  constexpr int LPT = A_LOADS + B_LOADS;  // direct loads per thread per k-tile
+  constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
+  constexpr int CPRK = BK / 8;             // 16-byte chunks per K-contiguous row
+  constexpr int RPW = 256 / (BK * 2);      // K-contiguous rows per 256-byte bank window
+  constexpr int CS = WN + 8;               // row stride of a wave's staged output tile
+  static_assert(A_ELEMS / 8 % NT == 0 && B_ELEMS / 8 % NT == 0, "tile/threads");
+  static_assert((STAGES - 2) * LPT <= 63, "vmcnt range");
+
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
+
+  int const t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  int const wm0 = (wave / (BN / WN)) * WM;
+  int const wn0 = (wave % (BN / WN)) * WN;
+  int tm, tn;
+  tile_coords(blockIdx.x, M / BM, N / BN, tm, tn);
+  int const m0 = tm * BM, n0 = tn * BN;
+
+  // Per-lane global offsets of its chunks (constant over k except for k0).
+  // K-contiguous tile [rows][BK]: physical chunk pc of a row holds logical
+  // chunk pc ^ ((row / RPW) % CPRK).  Tile lying as [BK][cols]: the 64-byte
+  // segment s of row k sits at segment s ^ (k % 4).
+  int64_t goff_a[A_LOADS], goff_b[B_LOADS];
+#pragma unroll
+  for (int i = 0; i < A_LOADS; i++) {
+    int c = (i * NW + wave) * 64 + lane;
+    if (!TA) {
+      int row = c / CPRK, pc = c % CPRK;
+      int lc = pc ^ ((row / RPW) & (CPRK - 1));
+      goff_a[i] = (int64_t)(m0 + row) * lda + lc * 8;
+    } else {
+      constexpr int CPR = BM / 8;
+      int krow = c / CPR, pc = c % CPR;
+      int lc = ((((pc >> 2) ^ (krow & 3)) << 2) | (pc & 3));
+      goff_a[i] = (int64_t)krow * lda + m0 + lc * 8;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < B_LOADS; i++) {
+    int c = (i * NW + wave) * 64 + lane;
+    if (!TBL) {
+      int row = c / CPRK, pc = c % CPRK;
+      int lc = pc ^ ((row / RPW) & (CPRK - 1));
+      goff_b[i] = (int64_t)(n0 + row) * ldb + lc * 8;
+    } else {
+      constexpr int CPR = BN / 8;
+      int krow = c / CPR, pc = c % CPR;
+      int lc = ((((pc >> 2) ^ (krow & 3)) << 2) | (pc & 3));
+      goff_b[i] = (int64_t)krow * ldb + n0 + lc * 8;
+    }
+  }
+
+  auto issue = [&](int kt, int stage) {
+    bf16 *sa = smem + stage * STAGE_ELEMS;
+    bf16 *sb = sa + A_ELEMS;
+    int64_t const ka = TA ? (int64_t)kt * BK * lda : (int64_t)kt * BK;
+    int64_t const kb = TBL ? (int64_t)kt * BK * ldb : (int64_t)kt * BK;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; i++) {
+      __builtin_amdgcn_global_load_lds((gptr_t)(A + goff_a[i] + ka),
+                                       (lptr_t)(sa + (i * NW + wave) * 512), 16, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; i++) {
+      __builtin_amdgcn_global_load_lds((gptr_t)(B + goff_b[i] + kb),
+                                       (lptr_t)(sb + (i * NW + wave) * 512), 16, 0, 0);
+    }
+  };
+
+  // Fragment readers (see the layouts above).
+  auto frag_kc = [&](bf16 const *tile, int row0, int kk) -> bf16x8 {
+    int const row = row0 + (lane & 31);
+    int const pc = (2 * kk + (lane >> 5)) ^ ((row / RPW) & (CPRK - 1));
+    return *reinterpret_cast<bf16x8 const *>(tile + row * BK + pc * 8);
+  };
+  auto frag_tr = [&](bf16 const *tile, int rowlen, int col0, int kk) -> bf16x8 {
+    int const i16 = lane & 15;
+    int const col = col0 + ((lane >> 4) & 1) * 16 + (i16 & 3) * 4;
+    int const krow = kk * 16 + (lane >> 5) * 8 + (i16 >> 2);
+    int const pcol = ((((col >> 5) ^ (krow & 3)) << 5) | (col & 31));
+    typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(tile + krow * rowlen + pcol));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(tile + (krow + 4) * rowlen + pcol));
+    union {
+      s16x4 h[2];
+      bf16x8 v;
+    } u;
+    u.h[0] = lo;
+    u.h[1] = hi;
+    return u.v;
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  int const KT = K / BK;
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; s++) {
+    if (s < KT) issue(s, s);
+  }
+  for (int kt = 0; kt < KT; kt++) {
+    int const stage = kt % STAGES;
+    // Tile kt must have landed; up to STAGES-2 younger tiles may be in flight.
+    // (Near the end fewer tiles are outstanding, so wait for everything.)
+    if (kt + STAGES - 2 < KT) {
+      wait_vmcnt<(STAGES - 2) * LPT>();
+    } else {
+      wait_vmcnt<0>();
+    }
+    // Barrier without a memory fence: a fence would wait for every direct load
+    // still in flight; the vmcnt wait above already covers the tile needed.
+    asm volatile("s_barrier" ::: "memory");
+    // Every wave has finished reading the stage consumed last iteration.
+    if (kt + STAGES - 1 < KT) issue(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+    bf16 const *sa = smem + stage * STAGE_ELEMS;
+    bf16 const *sb = sa + A_ELEMS;
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; kk++) {
+      bf16x8 af[TM], bfr[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        af[i] = TA ? frag_tr(sa, BM, wm0 + i * 32, kk) : frag_kc(sa, wm0 + i * 32, kk);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        bfr[j] = TBL ? frag_tr(sb, BN, wn0 + j * 32, kk) : frag_kc(sb, wn0 + j * 32, kk);
+      }
+      // Transposed accumulation: rows of the MFMA result = output columns.
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+    }
+  }
+  __syncthreads();  // all stages are free now: reuse them for the output tile
+
+  // acc[i][j][r]: output row m = wm0 + 32 i + lane % 32,
+  //               column n = wn0 + 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4.
+  // Each wave stages its own WM x WN tile and writes it out in 16-byte chunks.
+  bf16 *cs = smem + wave * (WM * CS);
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    int const m = i * 32 + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        int const n = j * 32 + 8 * g + 4 * (lane >> 5);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e];
+        if (bias != nullptr) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] += VecIO<bf16>::load1(bias + n0 + wn0 + n + e);
+        }
+        if (act != FFK_ACT_NONE) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = apply_activation(v[e], act);
+        }
+        if (accumulate) {
+          // add the old value in fp32 before the single rounding
+          u32x2 old = *reinterpret_cast<u32x2 const *>(C + (int64_t)(m0 + wm0 + m) * ldc + n0 + wn0 + n);
+          v[0] += __uint_as_float(old[0] << 16);
+          v[1] += __uint_as_float(old[0] & 0xffff0000u);
+          v[2] += __uint_as_float(old[1] << 16);
+          v[3] += __uint_as_float(old[1] & 0xffff0000u);
+        }
+        u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        *reinterpret_cast<u32x2 *>(cs + m * CS + n) = w;
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int CCH = WM * WN / 8 / 64;  // 16-byte chunks per lane
+#pragma unroll
+  for (int i = 0; i < CCH; i++) {
+    int c = lane + i * 64;
+    int row = c / (WN / 8), ch = c % (WN / 8);
+    u32x4 v = *reinterpret_cast<u32x4 const *>(cs + row * CS + ch * 8);
+    *reinterpret_cast<u32x4 *>(C + (int64_t)(m0 + wm0 + row) * ldc + n0 + wn0 + ch * 8) = v;
+  }
+}
+
+template <int BM, int BN, int WM, int WN, int BK, int STAGES>
+struct PipeCfg {
+  static constexpr int NW = (BM / WM) * (BN / WN);
+  static constexpr size_t kStageBytes = (size_t)STAGES * (BM + BN) * BK * sizeof(bf16);
+  static constexpr size_t kOutBytes = (size_t)NW * WM * (WN + 8) * sizeof(bf16);
+  static constexpr size_t kLds = kStageBytes > kOutBytes ? kStageBytes : kOutBytes;
+  static_assert(kLds <= 160 * 1024, "LDS budget");
+};
+
+template <int BM, int BN, int WM, int WN, int BK, int STAGES, bool TA, bool TB>
+static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
+                              bf16 *C, int M, int N, int K, int64_t lda,
+                              int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
+  using Cfg = PipeCfg<BM, BN, WM, WN, BK, STAGES>;
+  constexpr int NT = Cfg::NW * 64;
+  auto kern = gemm_bf16_pipe_kernel<BM, BN, WM, WN, BK, STAGES, TA, TB>;
+  static bool configured = false;  // per template instance
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg::kLds);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  int const blocks = (M / BM) * (N / BN);
+  kern<<<blocks, NT, Cfg::kLds, st>>>(A, B, C, M, N, K, lda, ldb, ldc,
+                                     static_cast<bf16 const *>(ep.bias), ep.activation,
+                                     ep.accumulate);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
 // fp32 MFMA kernel (32x32x2), 64x64 block tile, bounds-checked everywhere.
 // ---------------------------------------------------------------------------
 template <bool TA, bool TB>
@@ -416,10 +668,44 @@ static hipError_t launch_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
   return hipGetLastError();
 }
 
+// FFK_GEMM_VARIANT=128|256|1 forces a tile configuration (1 = the register-
+// staged kernel); unset or 0 = the heuristic.  For tuning runs only.
+static int gemm_variant_override() {
+  static int v = -1;
+  if (v < 0) {
+    char const *e = getenv("FFK_GEMM_VARIANT");
+    v = e ? atoi(e) : 0;
+  }
+  return v;
+}
+
 template <bool TA, bool TB>
 static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
                             bf16 *C, int M, int N, int K, int64_t lda,
                             int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
+  bool const c_vec = (ldc % 8 == 0) && aligned16(C);
+  int const variant = gemm_variant_override();
+  if (c_vec && K % 64 == 0) {
+    bool const fits256 = M % 256 == 0 && N % 256 == 0;
+    bool const fits128 = M % 128 == 0 && N % 128 == 0;
+    int64_t const t256 = fits256 ? (int64_t)(M / 256) * (N / 256) : 0;
+    int64_t const t128 = fits128 ? (int64_t)(M / 128) * (N / 128) : 0;
+    if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) {
+      return launch_pipe<256, 256, 128, 64, 32, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+    }
+    if (variant == 2565 && fits256) {
+      return launch_pipe<256, 256, 128, 64, 32, 5, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+    }
+    if (variant == 2563 && fits256) {
+      return launch_pipe<256, 256, 128, 64, 32, 3, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+    }
+    if (variant == 2564 && fits256) {
+      return launch_pipe<256, 256, 128, 128, 32, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+    }
+    if ((variant == 0 && t128 >= kNumCU / 2) || (variant == 128 && fits128)) {
+      return launch_pipe<128, 128, 64, 64, 64, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+    }
+  }
   // Largest tile that still gives every CU a workgroup.
   int64_t const b128 = ceil_div(M, 128) * ceil_div(N, 128);
   if (b128 >= kNumCU) {

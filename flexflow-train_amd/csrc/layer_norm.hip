@@ -259,19 +259,36 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
   }
 }
 
+// Sums the per-workgroup partials: 32 columns x 8 row groups per workgroup so
+// that even N = 1024 spreads over 32 workgroups and every access is a 128-byte
+// row segment.
 template <typename T>
 __global__ __launch_bounds__(256) void layer_norm_param_grad_final_kernel(
     float const *__restrict__ partials, int nparts, int N, T *dgamma,
     T *dbeta) {
-  int const j = blockIdx.x * 256 + threadIdx.x;
-  if (j >= N) return;
+  __shared__ float red[2][8][33];
+  int const cx = threadIdx.x & 31, ry = threadIdx.x >> 5;
+  int const j = blockIdx.x * 32 + cx;
   float sg = 0.0f, sb = 0.0f;
-  for (int p = 0; p < nparts; p++) {
-    sg += partials[(int64_t)p * 2 * N + j];
-    sb += partials[(int64_t)p * 2 * N + N + j];
+  if (j < N) {
+    for (int p = ry; p < nparts; p += 8) {
+      sg += partials[(int64_t)p * 2 * N + j];
+      sb += partials[(int64_t)p * 2 * N + N + j];
+    }
   }
-  if (dgamma != nullptr) VecIO<T>::store1(dgamma + j, sg);
-  if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, sb);
+  red[0][ry][cx] = sg;
+  red[1][ry][cx] = sb;
+  __syncthreads();
+  if (ry == 0 && j < N) {
+    float tg = 0.0f, tb = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 8; r++) {
+      tg += red[0][r][cx];
+      tb += red[1][r][cx];
+    }
+    if (dgamma != nullptr) VecIO<T>::store1(dgamma + j, tg);
+    if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, tb);
+  }
 }
 
 // Generic backward: any N; one workgroup per row for dX, then a column kernel
@@ -398,7 +415,7 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
     FFK_CHECK_LAUNCH();
     if (dgamma != nullptr || dbeta != nullptr) {
       layer_norm_param_grad_final_kernel<T>
-          <<<(unsigned)ceil_div(N, 256), 256, 0, st>>>(
+          <<<(unsigned)ceil_div(N, 32), 256, 0, st>>>(
               partials, blocks, (int)N, static_cast<T *>(dgamma),
               static_cast<T *>(dbeta));
       FFK_CHECK_LAUNCH();
