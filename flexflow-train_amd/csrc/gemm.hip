@@ -14,6 +14,7 @@
 // (lib/kernels/src/cuda/ops/linear_kernels.cu:143,163,249,298,321).
 #include "gemm.h"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace ffk {
 
@@ -422,44 +423,87 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
   int const KT = K / BK;
+  constexpr int KS = BK / 16;  // MFMA k-steps per tile
+  static_assert(KS % 2 == 0, "fragment double buffering assumes an even step count");
+  static_assert(STAGES >= 3, "need a stage in flight besides the two in use");
 #pragma unroll
   for (int s = 0; s < STAGES - 1; s++) {
     if (s < KT) issue(s, s);
   }
-  for (int kt = 0; kt < KT; kt++) {
-    int const stage = kt % STAGES;
-    // Tile kt must have landed; up to STAGES-2 younger tiles may be in flight.
-    // (Near the end fewer tiles are outstanding, so wait for everything.)
-    if (kt + STAGES - 2 < KT) {
-      wait_vmcnt<(STAGES - 2) * LPT>();
-    } else {
-      wait_vmcnt<0>();
-    }
-    // Barrier without a memory fence: a fence would wait for every direct load
-    // still in flight; the vmcnt wait above already covers the tile needed.
-    asm volatile("s_barrier" ::: "memory");
-    // Every wave has finished reading the stage consumed last iteration.
-    if (kt + STAGES - 1 < KT) issue(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+  // Fragments are double-buffered in registers: while the MFMAs of one k-step
+  // run, the LDS reads of the next step (of the next tile, at a tile's last
+  // step) are already in flight.
+  bf16x8 af[2][TM], bfr[2][TN];
+  auto read_frags = [&](int buf, int stage, int kk) {
     bf16 const *sa = smem + stage * STAGE_ELEMS;
     bf16 const *sb = sa + A_ELEMS;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; kk++) {
-      bf16x8 af[TM], bfr[TN];
+    for (int i = 0; i < TM; i++) {
+      af[buf][i] = TA ? frag_tr(sa, BM, wm0 + i * 32, kk) : frag_kc(sa, wm0 + i * 32, kk);
+    }
 #pragma unroll
-      for (int i = 0; i < TM; i++) {
-        af[i] = TA ? frag_tr(sa, BM, wm0 + i * 32, kk) : frag_kc(sa, wm0 + i * 32, kk);
-      }
+    for (int j = 0; j < TN; j++) {
+      bfr[buf][j] = TBL ? frag_tr(sb, BN, wn0 + j * 32, kk) : frag_kc(sb, wn0 + j * 32, kk);
+    }
+  };
+  // Tile 0 must have landed (STAGES-2 younger tiles may still be in flight).
+  if (STAGES - 2 < KT) {
+    wait_vmcnt<(STAGES - 2) * LPT>();
+  } else {
+    wait_vmcnt<0>();
+  }
+  // Barrier without a memory fence: a fence would wait for every direct load
+  // still in flight; the vmcnt waits already cover the tile that is needed.
+  asm volatile("s_barrier" ::: "memory");
+  read_frags(0, 0, 0);
+  // One k-tile.  STEADY: every condition of the generic body is known true
+  // (next tile exists, a refill is due, STAGES-3 younger tiles in flight), so
+  // the steady-state loop is branch-free.
+  auto tile_step = [&](int kt, auto steady_tag) {
+    constexpr bool STEADY = decltype(steady_tag)::value;
+    int const stage = kt % STAGES;
 #pragma unroll
-      for (int j = 0; j < TN; j++) {
-        bfr[j] = TBL ? frag_tr(sb, BN, wn0 + j * 32, kk) : frag_kc(sb, wn0 + j * 32, kk);
+    for (int kk = 0; kk < KS; kk++) {
+      int const cur = kk & 1;
+      // The first MFMA of the step is issued before the prefetch below so that
+      // the wait for this step's fragments is the only LDS wait outstanding at
+      // that point (the hardware counter is in order; a wait placed after the
+      // prefetch would also wait for the prefetched data).
+      __builtin_amdgcn_sched_barrier(0);
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0], af[cur][0], acc[0][0], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (kk + 1 < KS) {
+        read_frags(cur ^ 1, stage, kk + 1);
+      } else if (STEADY || kt + 1 < KT) {
+        // Last step of the tile: make tile kt+1 visible, refill the stage that
+        // was consumed one iteration ago, and start reading tile kt+1 -- all
+        // under this step's MFMAs, which cover those latencies.
+        if (STEADY || kt + STAGES - 2 < KT) {
+          wait_vmcnt<(STAGES - 3) * LPT>();
+        } else {
+          wait_vmcnt<0>();
+        }
+        asm volatile("s_barrier" ::: "memory");
+        if (STEADY || kt + STAGES - 1 < KT) issue(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+        read_frags(cur ^ 1, (kt + 1) % STAGES, 0);
       }
+      __builtin_amdgcn_sched_barrier(0);
       // Transposed accumulation: rows of the MFMA result = output columns.
 #pragma unroll
       for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+          if (i + j > 0)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
+  };
+  int kt = 0;
+  for (; kt + STAGES - 1 < KT; kt++) {
+    tile_step(kt, std::true_type{});
+  }
+  for (; kt < KT; kt++) {
+    tile_step(kt, std::false_type{});
   }
   __syncthreads();  // all stages are free now: reuse them for the output tile
 
@@ -685,25 +729,19 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
                             int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
   bool const c_vec = (ldc % 8 == 0) && aligned16(C);
   int const variant = gemm_variant_override();
-  if (c_vec && K % 64 == 0) {
+  if (c_vec && K % 64 == 0 && variant != 1) {
     bool const fits256 = M % 256 == 0 && N % 256 == 0;
     bool const fits128 = M % 128 == 0 && N % 128 == 0;
     int64_t const t256 = fits256 ? (int64_t)(M / 256) * (N / 256) : 0;
     int64_t const t128 = fits128 ? (int64_t)(M / 128) * (N / 128) : 0;
+    // 256x256 tiles (8 waves of 128x64) halve the L2->LDS traffic per flop and
+    // win whenever they still occupy most CUs; otherwise 128x128 tiles with 8
+    // waves of 64x32 keep two waves per SIMD on every CU.
     if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) {
       return launch_pipe<256, 256, 128, 64, 32, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
-    if (variant == 2565 && fits256) {
-      return launch_pipe<256, 256, 128, 64, 32, 5, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
-    }
-    if (variant == 2563 && fits256) {
-      return launch_pipe<256, 256, 128, 64, 32, 3, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
-    }
-    if (variant == 2564 && fits256) {
-      return launch_pipe<256, 256, 128, 128, 32, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
-    }
     if ((variant == 0 && t128 >= kNumCU / 2) || (variant == 128 && fits128)) {
-      return launch_pipe<128, 128, 64, 64, 64, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+      return launch_pipe<128, 128, 64, 32, 64, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
   }
   // Largest tile that still gives every CU a workgroup.

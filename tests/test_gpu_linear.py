@@ -166,3 +166,69 @@ def test_linear_bf16(ffk, oracle, act):
     assert_close(to_np(dx), dx_ref, BF16_RTOL, "dx")
     assert_close(to_np(dw), dw_ref, BF16_RTOL, "dw")
     assert_close(to_np(db), db_ref, BF16_RTOL, "db")
+
+
+# Shapes that tile exactly take the pipelined direct-to-LDS kernels: 128x128
+# tiles when that yields >= 128 workgroups, 256x256 tiles from 192 workgroups.
+PIPE_SHAPES = [(2048, 2048, 512), (1024, 2048, 320), (4096, 3072, 256), (3072, 4096, 192)]
+
+
+@pytest.mark.parametrize("trans_a,trans_b", [(False, True), (False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("mnk", PIPE_SHAPES)
+def test_gemm_bf16_pipelined_tiles(ffk, oracle, trans_a, trans_b, mnk):
+    M, N, K = mnk
+    say("gemm bf16 pipelined", mnk, "ta", trans_a, "tb", trans_b)
+    g = rng(M + 3 * N + 7 * K)
+    A = bf16_round(g.standard_normal((K, M) if trans_a else (M, K)))
+    B = bf16_round(g.standard_normal((N, K) if trans_b else (K, N)))
+    Ad, Bd = to_dev(A, torch, torch.bfloat16), to_dev(B, torch, torch.bfloat16)
+    C = torch.full((M, N), 3.0, dtype=torch.bfloat16, device="cuda")
+    ffk.gemm(Ad, Bd, C, trans_a, trans_b)
+    Cn = to_np(C)
+    # (1) the oracle on a sample of rows and on a sample of columns
+    rows = np.sort(g.choice(M, 40, replace=False))
+    cols = np.sort(g.choice(N, 40, replace=False))
+    A_rows = np.ascontiguousarray(A[:, rows] if trans_a else A[rows])
+    B_cols = np.ascontiguousarray(B[cols] if trans_b else B[:, cols])
+    assert_close(Cn[rows], oracle.gemm_f64(A_rows, B, trans_a, trans_b), 2.0 ** -8, "C rows")
+    assert_close(Cn[:, cols], oracle.gemm_f64(A, B_cols, trans_a, trans_b), 2.0 ** -8, "C cols")
+    # (2) every element, through linearity: C v = A (B v)
+    v = g.standard_normal((N,))
+    A64 = (A.T if trans_a else A).astype(np.float64)
+    B64 = (B.T if trans_b else B).astype(np.float64)
+    want = A64 @ (B64 @ v)
+    got = Cn.astype(np.float64) @ v
+    bound = 2.0 ** -8 * (np.abs(A64) @ (np.abs(B64) @ np.abs(v)))
+    assert np.all(np.abs(got - want) <= bound + 1e-6)
+    # (3) accumulate adds to the old contents with a single rounding
+    C0 = bf16_round(g.standard_normal((M, N)))
+    Cd = to_dev(C0, torch, torch.bfloat16)
+    ffk.gemm(Ad, Bd, Cd, trans_a, trans_b, accumulate=True)
+    assert_close(to_np(Cd)[rows], oracle.gemm_f64(A_rows, B, trans_a, trans_b) + C0[rows], 2.0 ** -7, "C acc")
+
+
+@pytest.mark.parametrize("act", [-1, 0])
+def test_linear_bf16_pipelined(ffk, oracle, act):
+    """Linear at a size whose three products all take the pipelined kernels
+    (NT forward with bias/activation epilogue, NN and TN backward)."""
+    batch, in_dim, out_dim = 2048, 1024, 2048
+    say("linear bf16 pipelined", (batch, in_dim, out_dim), "act", act)
+    g = rng(23)
+    x = bf16_round(g.standard_normal((batch, in_dim)))
+    w = bf16_round(g.standard_normal((out_dim, in_dim)) * 0.03)
+    b = bf16_round(g.standard_normal((out_dim,)) * 0.5)
+    dy = bf16_round(g.standard_normal((batch, out_dim)))
+    xd, wd, bd, dyd = (to_dev(a, torch, torch.bfloat16) for a in (x, w, b, dy))
+    y = ffk.linear_forward(xd, wd, bd, activation=act)
+    rows = np.sort(g.choice(batch, 32, replace=False))
+    y_ref = oracle.linear_forward(x[rows], w, b, activation=act)
+    assert_close(to_np(y)[rows], y_ref, BF16_RTOL, "y rows")
+    yn = to_np(y)
+    dx, dw, db = torch.zeros_like(xd), torch.zeros_like(wd), torch.zeros_like(bd)
+    ffk.linear_backward(y, dyd, xd, wd, dx, dw, db, activation=act)
+    gmat = dy * (yn > 0) if act == 0 else dy
+    assert_close(to_np(dx)[rows], oracle.gemm_f64(np.ascontiguousarray(gmat[rows]), w), BF16_RTOL, "dx rows")
+    orows = np.sort(g.choice(out_dim, 32, replace=False))
+    dw_ref = oracle.gemm_f64(np.ascontiguousarray(gmat[:, orows]), x, trans_a=True)
+    assert_close(to_np(dw)[orows], dw_ref, BF16_RTOL, "dw rows")
+    assert_close(to_np(db), gmat.astype(np.float64).sum(0), BF16_RTOL, "db")
