@@ -1,0 +1,475 @@
+// The reference's operator entry points (namespace FlexFlow / Kernels::<Op>),
+// each unpacking accessors and per-device state into one C-ABI call.  The CPU
+// device branch raises: this library executes on the GPU only.
+#include "ffk.h"
+#include "kernels/attention_kernels.h"
+#include "kernels/dropout_kernels.h"
+#include "kernels/element_kernels.h"
+#include "kernels/embedding_kernels.h"
+#include "kernels/layer_norm_kernels.h"
+#include "kernels/linear_kernels.h"
+#include "kernels/softmax_kernels.h"
+
+namespace FlexFlow {
+
+[[noreturn]] static void no_cpu(char const *who) {
+  throw std::runtime_error(std::string(who) + ": NOT_IMPLEMENTED for the CPU device type in this library");
+}
+
+static int dt(DataType d) { return static_cast<int>(d); }
+static int act_code(std::optional<Activation> const &a) { return a.has_value() ? static_cast<int>(*a) : FFK_ACT_NONE; }
+
+static void require_gpu(GenericTensorAccessorR const &a, char const *who) {
+  if (a.device_type != DeviceType::GPU) throw std::runtime_error(std::string(who) + ": accessor is not device-resident");
+}
+
+// ---- Linear ---------------------------------------------------------------
+
+std::optional<LinearPerDeviceState> linear_init_kernel(
+    DeviceType device_type, device_handle_t const &handle, std::optional<Activation> activation,
+    std::optional<RegularizerAttrs> regularizer, bool use_bias, DataType input_type,
+    DataType weight_type, DataType output_type, int batch_size, int output_num_channels) {
+  if (device_type != DeviceType::GPU) return std::nullopt;
+  LinearPerDeviceState s;
+  s.handle = handle.require_for_gpu();
+  // ReLU sizes the scratch for any activation (same bytes for all of them)
+  s.workspace_bytes = ffk_linear_backward_workspace_bytes(
+      dt(output_type), activation.has_value() ? FFK_ACT_RELU : FFK_ACT_NONE, use_bias, batch_size, output_num_channels);
+  s.workspace = nullptr;
+  if (s.workspace_bytes > 0) check_ffk(ffk_malloc(&s.workspace, s.workspace_bytes), "linear_init_kernel");
+  s.activation = activation;
+  s.regularizer = regularizer;
+  s.use_bias = use_bias;
+  s.input_type = input_type;
+  s.weight_type = weight_type;
+  s.output_type = output_type;
+  return s;
+}
+
+void linear_forward_kernel(device_stream_t const &stream, std::optional<LinearPerDeviceState> const &state,
+                           LinearAttrs const &attrs, GenericTensorAccessorR const &input,
+                           GenericTensorAccessorW const &output, GenericTensorAccessorR const &projection,
+                           std::optional<GenericTensorAccessorR> const &bias) {
+  if (!stream.is_gpu()) no_cpu("linear_forward_kernel");
+  if (attrs.use_bias != bias.has_value()) throw std::runtime_error("linear_forward_kernel: use_bias does not match bias");
+  require_gpu(input, "linear_forward_kernel");
+  (void)state;
+  int64_t in_dim = dim_at_idx(input.shape.dims, -1);
+  int64_t batch = get_num_elements(input.shape.dims) / in_dim;
+  int64_t out_dim = dim_at_idx(projection.shape.dims, 0);
+  check_ffk(ffk_linear_forward(stream.require_gpu(), dt(input.shape.data_type), act_code(attrs.activation),
+                               input.ptr, output.ptr, projection.ptr, bias ? bias->ptr : nullptr, batch,
+                               in_dim, out_dim),
+            "linear_forward_kernel");
+}
+
+void linear_backward_kernel(device_stream_t const &stream, std::optional<LinearPerDeviceState> const &state,
+                            LinearAttrs const &attrs, GenericTensorAccessorR const &output,
+                            GenericTensorAccessorR const &output_grad, GenericTensorAccessorR const &input,
+                            GenericTensorAccessorW const &input_grad, GenericTensorAccessorR const &projection,
+                            GenericTensorAccessorW const &projection_grad,
+                            std::optional<GenericTensorAccessorW> const &bias_grad) {
+  if (!stream.is_gpu()) no_cpu("linear_backward_kernel");
+  if (!state.has_value()) throw std::runtime_error("linear_backward_kernel: per-device state required on the GPU");
+  int64_t in_dim = dim_at_idx(input.shape.dims, -1);
+  int64_t batch = get_num_elements(input.shape.dims) / in_dim;
+  int64_t out_dim = dim_at_idx(projection.shape.dims, 0);
+  // Reference GPU semantics: all three gradients accumulate (beta = 1).
+  check_ffk(ffk_linear_backward(stream.require_gpu(), dt(input.shape.data_type), act_code(attrs.activation), 0,
+                                output.ptr, output_grad.ptr, input.ptr, input_grad.ptr, projection.ptr,
+                                projection_grad.ptr, bias_grad ? bias_grad->ptr : nullptr, batch, in_dim, out_dim,
+                                state->workspace, state->workspace_bytes, FFK_ACC_ALL),
+            "linear_backward_kernel");
+}
+
+void linear_cleanup_kernel(DeviceType device_type, std::optional<LinearPerDeviceState> &state) {
+  if (device_type == DeviceType::GPU && state.has_value() && state->workspace != nullptr) {
+    check_ffk(ffk_free(state->workspace), "linear_cleanup_kernel");
+    state->workspace = nullptr;
+  }
+}
+
+// ---- MultiHeadAttention -----------------------------------------------------
+
+namespace Kernels::MultiHeadAttention {
+
+static ffk_mha_desc_t make_desc(MHAPerDeviceState const &s) {
+  ffk_mha_desc_t d;
+  d.num_samples = s.num_samples; d.num_heads = s.num_heads;
+  d.q_size = s.qSize; d.k_size = s.kSize; d.v_size = s.vSize;
+  d.q_proj_size = s.qProjSize; d.k_proj_size = s.kProjSize; d.v_proj_size = s.vProjSize;
+  d.o_proj_size = s.oProjSize;
+  d.qo_seq_length = s.qoSeqLength; d.kv_seq_length = s.kvSeqLength;
+  d.scale = s.scale; d.causal = s.causal ? 1 : 0;
+  return d;
+}
+
+std::optional<MHAPerDeviceState> init_kernel(DeviceType device_type, device_handle_t const &handle,
+                                             Allocator &allocator, int num_samples, int num_heads, int qSize,
+                                             int kSize, int vSize, int qProjSize, int kProjSize, int vProjSize,
+                                             int oProjSize, int qoSeqLength, int kvSeqLength, bool add_bias_kv,
+                                             DataType data_type, float scale, bool causal) {
+  if (device_type != DeviceType::GPU) return std::nullopt;
+  if (add_bias_kv) throw std::runtime_error("MultiHeadAttention: add_bias_kv is not supported");
+  MHAPerDeviceState s{handle.require_for_gpu(), 0, 0, num_samples, num_heads, qSize, kSize, vSize, qProjSize,
+                      kProjSize, vProjSize, oProjSize, qoSeqLength, kvSeqLength, scale, causal, data_type,
+                      nullptr, allocator};
+  ffk_mha_desc_t d = make_desc(s);
+  s.weightSize = ffk_mha_weight_elements(&d) * size_of_datatype(data_type);
+  s.reserveSpaceSize = ffk_mha_reserve_bytes(&d, dt(data_type));
+  s.reserveSpace = allocator.allocate(s.reserveSpaceSize);
+  return s;
+}
+
+std::optional<MHAPerDeviceState> init_kernel(DeviceType device_type, device_handle_t const &handle,
+                                             Allocator &allocator, int num_samples, int num_heads, int qSize,
+                                             int kSize, int vSize, int qProjSize, int kProjSize, int vProjSize,
+                                             int oProjSize, int qoSeqLength, int kvSeqLength, bool add_bias_kv) {
+  // reference configuration: fp32 tensors, smScalar = 1.0, full window
+  // (src/cuda/ops/attention_kernels.cu:73-92,188-193)
+  return init_kernel(device_type, handle, allocator, num_samples, num_heads, qSize, kSize, vSize, qProjSize,
+                     kProjSize, vProjSize, oProjSize, qoSeqLength, kvSeqLength, add_bias_kv, DataType::FLOAT,
+                     1.0f, false);
+}
+
+static void run_forward(device_stream_t const &stream, MHAPerDeviceState const &s, void const *q, void const *k,
+                        void const *v, void const *w, void *out) {
+  ffk_mha_desc_t d = make_desc(s);
+  check_ffk(ffk_mha_forward(stream.require_gpu(), dt(s.data_type), &d, q, k, v, w, out, s.reserveSpace,
+                            s.reserveSpaceSize),
+            "MultiHeadAttention::forward_kernel");
+}
+
+void forward_kernel(device_stream_t const &stream, std::optional<MHAPerDeviceState> const &state,
+                    float const *q, float const *k, float const *v, float const *w, float *out) {
+  if (!stream.is_gpu()) no_cpu("MultiHeadAttention::forward_kernel");
+  run_forward(stream, state.value(), q, k, v, w, out);  // fp32 state: the C ABI reports "bf16 only"
+}
+
+void forward_kernel(device_stream_t const &stream, std::optional<MHAPerDeviceState> const &state,
+                    GenericTensorAccessorR const &q, GenericTensorAccessorR const &k,
+                    GenericTensorAccessorR const &v, GenericTensorAccessorR const &w,
+                    GenericTensorAccessorW const &out) {
+  if (!stream.is_gpu()) no_cpu("MultiHeadAttention::forward_kernel");
+  if (q.shape.data_type != state.value().data_type) throw std::runtime_error("MultiHeadAttention: dtype differs from the state's");
+  run_forward(stream, *state, q.ptr, k.ptr, v.ptr, w.ptr, out.ptr);
+}
+
+static void run_backward(device_stream_t const &stream, MHAPerDeviceState const &s, void const *q, void *dq,
+                         void const *k, void *dk, void const *v, void *dv, void const *w, void *dw,
+                         void const *dout) {
+  ffk_mha_desc_t d = make_desc(s);
+  // input gradients accumulate like every reference GPU backward (callers zero them first)
+  check_ffk(ffk_mha_backward(stream.require_gpu(), dt(s.data_type), &d, q, dq, k, dk, v, dv, w, dw, dout,
+                             s.reserveSpace, s.reserveSpaceSize, 1),
+            "MultiHeadAttention::backward_kernel");
+}
+
+void backward_kernel(device_stream_t const &stream, std::optional<MHAPerDeviceState> const &state,
+                     float const *q, float *dq, float const *k, float *dk, float const *v, float *dv,
+                     float const *w, float *dw, float const *dout) {
+  if (!stream.is_gpu()) no_cpu("MultiHeadAttention::backward_kernel");
+  run_backward(stream, state.value(), q, dq, k, dk, v, dv, w, dw, dout);
+}
+
+void backward_kernel(device_stream_t const &stream, std::optional<MHAPerDeviceState> const &state,
+                     GenericTensorAccessorR const &q, GenericTensorAccessorW const &dq,
+                     GenericTensorAccessorR const &k, std::optional<GenericTensorAccessorW> const &dk,
+                     GenericTensorAccessorR const &v, std::optional<GenericTensorAccessorW> const &dv,
+                     GenericTensorAccessorR const &w, GenericTensorAccessorW const &dw,
+                     GenericTensorAccessorR const &dout) {
+  if (!stream.is_gpu()) no_cpu("MultiHeadAttention::backward_kernel");
+  run_backward(stream, state.value(), q.ptr, dq.ptr, k.ptr, dk ? dk->ptr : nullptr, v.ptr,
+               dv ? dv->ptr : nullptr, w.ptr, dw.ptr, dout.ptr);
+}
+
+void cleanup_kernel(DeviceType device_type, Allocator &allocator, std::optional<MHAPerDeviceState> const &state) {
+  if (device_type == DeviceType::GPU && state.has_value() && state->reserveSpace != nullptr) {
+    allocator.deallocate(state->reserveSpace);
+  }
+}
+
+}  // namespace Kernels::MultiHeadAttention
+
+// ---- LayerNorm --------------------------------------------------------------
+
+namespace Kernels::LayerNorm {
+
+std::optional<LayerNormPerDeviceState> init_kernel(DeviceType device_type, device_handle_t const &handle,
+                                                   Allocator &allocator, bool elementwise_affine,
+                                                   int64_t effective_batch_size, int64_t effective_num_elements,
+                                                   float eps) {
+  if (device_type != DeviceType::GPU) return std::nullopt;
+  LayerNormPerDeviceState s;
+  s.handle = handle.require_for_gpu();
+  s.elementwise_affine = elementwise_affine;
+  s.effective_batch_size = effective_batch_size;
+  s.effective_num_elements = effective_num_elements;
+  s.eps = eps;
+  s.mean = static_cast<float *>(allocator.allocate(sizeof(float) * effective_batch_size));
+  s.rstd = static_cast<float *>(allocator.allocate(sizeof(float) * effective_batch_size));
+  s.workspace_bytes = ffk_layer_norm_backward_workspace_bytes(effective_batch_size, effective_num_elements);
+  s.workspace = allocator.allocate(s.workspace_bytes);
+  s.data_type = DataType::FLOAT;
+  return s;
+}
+
+void forward_kernel(device_stream_t const &stream, std::optional<LayerNormPerDeviceState> const &state,
+                    GenericTensorAccessorR const &input, GenericTensorAccessorW const &output,
+                    GenericTensorAccessorW const &gamma, GenericTensorAccessorW const &beta) {
+  if (!stream.is_gpu()) no_cpu("LayerNorm::forward_kernel");
+  LayerNormPerDeviceState const &s = state.value();
+  bool affine = s.elementwise_affine;
+  check_ffk(ffk_layer_norm_forward(stream.require_gpu(), dt(input.shape.data_type), input.ptr, output.ptr,
+                                   affine ? gamma.ptr : nullptr, affine ? beta.ptr : nullptr, s.mean, s.rstd,
+                                   s.effective_batch_size, s.effective_num_elements, s.eps),
+            "LayerNorm::forward_kernel");
+}
+
+void backward_kernel(device_stream_t const &stream, std::optional<LayerNormPerDeviceState> const &state,
+                     GenericTensorAccessorR const &output_grad, GenericTensorAccessorR const &input,
+                     GenericTensorAccessorW const &input_grad, GenericTensorAccessorR const &gamma,
+                     GenericTensorAccessorW const &gamma_grad, GenericTensorAccessorW const &beta_grad) {
+  if (!stream.is_gpu()) no_cpu("LayerNorm::backward_kernel");
+  LayerNormPerDeviceState const &s = state.value();
+  bool affine = s.elementwise_affine;
+  check_ffk(ffk_layer_norm_backward(stream.require_gpu(), dt(input.shape.data_type), output_grad.ptr, input.ptr,
+                                    s.mean, s.rstd, affine ? gamma.ptr : nullptr, input_grad.ptr,
+                                    affine ? gamma_grad.ptr : nullptr, affine ? beta_grad.ptr : nullptr,
+                                    s.effective_batch_size, s.effective_num_elements, s.workspace,
+                                    s.workspace_bytes, 1),
+            "LayerNorm::backward_kernel");
+}
+
+void cleanup_kernel(DeviceType, std::optional<LayerNormPerDeviceState> const &) {
+  // mean/rstd/workspace belong to the Allocator given to init_kernel
+}
+
+}  // namespace Kernels::LayerNorm
+
+// ---- Softmax ----------------------------------------------------------------
+
+namespace Kernels::Softmax {
+
+std::optional<SoftmaxPerDeviceState> init_kernel(DeviceType device_type, device_handle_t const &handle,
+                                                 ff_dim_t dim, int n, int c, int h, int w) {
+  if (device_type != DeviceType::GPU) return std::nullopt;
+  return SoftmaxPerDeviceState{handle.require_for_gpu(), n, c, h, w, dim, DataType::FLOAT};
+}
+
+static void run_forward(device_stream_t const &stream, SoftmaxPerDeviceState const &s, int dtype, void const *in,
+                        void *out) {
+  // cudnnSoftmaxForward(ACCURATE, MODE_CHANNEL) on an (n, c, h, w) view
+  check_ffk(ffk_softmax_forward(stream.require_gpu(), dtype, in, out, s.n, s.c, (int64_t)s.h * s.w),
+            "Softmax::forward_kernel");
+}
+
+void forward_kernel(device_stream_t const &stream, std::optional<SoftmaxPerDeviceState> const &state,
+                    float const *in, float *out) {
+  if (!stream.is_gpu()) no_cpu("Softmax::forward_kernel");
+  run_forward(stream, state.value(), FFK_FLOAT, in, out);
+}
+void forward_kernel(device_stream_t const &stream, std::optional<SoftmaxPerDeviceState> const &state,
+                    GenericTensorAccessorR const &in, GenericTensorAccessorW const &out) {
+  if (!stream.is_gpu()) no_cpu("Softmax::forward_kernel");
+  run_forward(stream, state.value(), dt(in.shape.data_type), in.ptr, out.ptr);
+}
+void backward_kernel(device_stream_t const &stream, float const *dout, float *din, size_t n) {
+  if (!stream.is_gpu()) no_cpu("Softmax::backward_kernel");
+  check_ffk(ffk_softmax_backward_copy(stream.require_gpu(), FFK_FLOAT, dout, din, n), "Softmax::backward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, std::optional<SoftmaxPerDeviceState> const &state,
+                     GenericTensorAccessorR const &output, GenericTensorAccessorR const &output_grad,
+                     GenericTensorAccessorW const &input_grad) {
+  if (!stream.is_gpu()) no_cpu("Softmax::backward_kernel");
+  SoftmaxPerDeviceState const &s = state.value();
+  check_ffk(ffk_softmax_backward(stream.require_gpu(), dt(output.shape.data_type), output.ptr, output_grad.ptr,
+                                 input_grad.ptr, s.n, s.c, (int64_t)s.h * s.w),
+            "Softmax::backward_kernel");
+}
+void cleanup_kernel(DeviceType, std::optional<SoftmaxPerDeviceState> &) {}
+
+}  // namespace Kernels::Softmax
+
+// ---- Dropout ----------------------------------------------------------------
+
+namespace Kernels::Dropout {
+
+std::optional<DropoutPerDeviceState> init_kernel(DeviceType device_type, device_handle_t const &handle,
+                                                 float rate, unsigned long long seed,
+                                                 TensorShape const &output_shape, Allocator &) {
+  if (device_type != DeviceType::GPU) return std::nullopt;
+  return DropoutPerDeviceState{handle.require_for_gpu(), rate, seed, output_shape};
+}
+void forward_kernel(device_stream_t const &stream, std::optional<DropoutPerDeviceState> const &state,
+                    float const *in, float *out) {
+  if (!stream.is_gpu()) no_cpu("Dropout::forward_kernel");
+  DropoutPerDeviceState const &s = state.value();
+  check_ffk(ffk_dropout_forward(stream.require_gpu(), FFK_FLOAT, in, out, get_num_elements(s.output_shape.dims),
+                                s.rate, s.seed, 0),
+            "Dropout::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, std::optional<DropoutPerDeviceState> const &state,
+                     float const *dout, float *din) {
+  if (!stream.is_gpu()) no_cpu("Dropout::backward_kernel");
+  DropoutPerDeviceState const &s = state.value();
+  // cudnnDropoutBackward overwrites dx
+  check_ffk(ffk_dropout_backward(stream.require_gpu(), FFK_FLOAT, dout, din,
+                                 get_num_elements(s.output_shape.dims), s.rate, s.seed, 0, 0),
+            "Dropout::backward_kernel");
+}
+void forward_kernel(device_stream_t const &stream, std::optional<DropoutPerDeviceState> const &state,
+                    GenericTensorAccessorR const &in, GenericTensorAccessorW const &out) {
+  if (!stream.is_gpu()) no_cpu("Dropout::forward_kernel");
+  DropoutPerDeviceState const &s = state.value();
+  check_ffk(ffk_dropout_forward(stream.require_gpu(), dt(in.shape.data_type), in.ptr, out.ptr,
+                                get_num_elements(in.shape.dims), s.rate, s.seed, 0),
+            "Dropout::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, std::optional<DropoutPerDeviceState> const &state,
+                     GenericTensorAccessorR const &dout, GenericTensorAccessorW const &din) {
+  if (!stream.is_gpu()) no_cpu("Dropout::backward_kernel");
+  DropoutPerDeviceState const &s = state.value();
+  check_ffk(ffk_dropout_backward(stream.require_gpu(), dt(dout.shape.data_type), dout.ptr, din.ptr,
+                                 get_num_elements(dout.shape.dims), s.rate, s.seed, 0, 0),
+            "Dropout::backward_kernel");
+}
+void cleanup_kernel(DeviceType, Allocator &, std::optional<DropoutPerDeviceState> &) {}
+
+}  // namespace Kernels::Dropout
+
+// ---- ElementUnary / ElementBinary -------------------------------------------
+
+namespace Kernels::ElementUnary {
+
+std::optional<ElementUnaryPerDeviceState> init_kernel(DeviceType device_type, TensorShape const &in,
+                                                      TensorShape const &out, ElementUnaryAttrs const &attrs) {
+  if (device_type != DeviceType::GPU) return std::nullopt;
+  return ElementUnaryPerDeviceState{in, out, attrs.op_type};
+}
+void forward_kernel(device_stream_t const &stream, std::optional<ElementUnaryPerDeviceState> const &,
+                    ElementUnaryAttrs const &attrs, device_handle_t const &, GenericTensorAccessorR const &input,
+                    GenericTensorAccessorW const &output) {
+  if (!stream.is_gpu()) no_cpu("ElementUnary::forward_kernel");
+  check_ffk(ffk_element_unary_forward(stream.require_gpu(), dt(input.shape.data_type),
+                                      static_cast<int>(attrs.op_type), attrs.scalar.value_or(0.0f), input.ptr,
+                                      output.ptr, get_num_elements(input.shape.dims)),
+            "ElementUnary::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, std::optional<ElementUnaryPerDeviceState> const &,
+                     ElementUnaryAttrs const &attrs, device_handle_t const &, GenericTensorAccessorR const &output,
+                     GenericTensorAccessorR const &output_grad, GenericTensorAccessorR const &input,
+                     GenericTensorAccessorW const &input_grad) {
+  if (!stream.is_gpu()) no_cpu("ElementUnary::backward_kernel");
+  // -1: the reference's per-op `=` / `+=` behaviour
+  check_ffk(ffk_element_unary_backward(stream.require_gpu(), dt(input.shape.data_type),
+                                       static_cast<int>(attrs.op_type), attrs.scalar.value_or(0.0f), output.ptr,
+                                       output_grad.ptr, input.ptr, input_grad.ptr,
+                                       get_num_elements(input.shape.dims), -1),
+            "ElementUnary::backward_kernel");
+}
+void cleanup_kernel(DeviceType, std::optional<ElementUnaryPerDeviceState> &) {}
+
+}  // namespace Kernels::ElementUnary
+
+namespace Kernels::ElementBinary {
+
+std::optional<ElementBinaryPerDeviceState> init_kernel(DeviceType device_type, device_handle_t const &handle,
+                                                       OperatorType op_type, bool bl, bool br,
+                                                       TensorShape const &lhs, TensorShape const &rhs,
+                                                       TensorShape const &out) {
+  if (device_type != DeviceType::GPU) return std::nullopt;
+  return ElementBinaryPerDeviceState{handle.require_for_gpu(), op_type, bl, br, lhs, rhs, out};
+}
+void forward_kernel(device_stream_t const &stream, std::optional<ElementBinaryPerDeviceState> const &state,
+                    float const *lhs, float const *rhs, float *out, OperatorType op_type, bool,
+                    device_handle_t const &) {
+  if (!stream.is_gpu()) no_cpu("ElementBinary::forward_kernel");
+  ElementBinaryPerDeviceState const &s = state.value();
+  check_ffk(ffk_element_binary_forward(stream.require_gpu(), FFK_FLOAT, static_cast<int>(op_type), lhs, rhs, out,
+                                       get_num_elements(s.output_shape.dims), get_num_elements(s.lhs_shape.dims),
+                                       get_num_elements(s.rhs_shape.dims)),
+            "ElementBinary::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, std::optional<ElementBinaryPerDeviceState> const &state,
+                     float const *dout, float const *lhs, float const *rhs, float *dl, float *dr,
+                     OperatorType op_type, bool bl, bool br, device_handle_t const &) {
+  if (!stream.is_gpu()) no_cpu("ElementBinary::backward_kernel");
+  if (bl || br) throw std::runtime_error("ElementBinary::backward_kernel: broadcast gradients are not supported "
+                                         "(shape inference rejects broadcasting, op-attrs/ops/element_binary.cc:5-21)");
+  check_ffk(ffk_element_binary_backward(stream.require_gpu(), FFK_FLOAT, static_cast<int>(op_type), dout, lhs, rhs,
+                                        dl, dr, get_num_elements(state.value().output_shape.dims), 1),
+            "ElementBinary::backward_kernel");
+}
+void forward_kernel(device_stream_t const &stream, std::optional<ElementBinaryPerDeviceState> const &state,
+                    GenericTensorAccessorR const &lhs, GenericTensorAccessorR const &rhs,
+                    GenericTensorAccessorW const &out) {
+  if (!stream.is_gpu()) no_cpu("ElementBinary::forward_kernel");
+  check_ffk(ffk_element_binary_forward(stream.require_gpu(), dt(out.shape.data_type),
+                                       static_cast<int>(state.value().op_type), lhs.ptr, rhs.ptr, out.ptr,
+                                       get_num_elements(out.shape.dims), get_num_elements(lhs.shape.dims),
+                                       get_num_elements(rhs.shape.dims)),
+            "ElementBinary::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, std::optional<ElementBinaryPerDeviceState> const &state,
+                     GenericTensorAccessorR const &dout, GenericTensorAccessorR const &lhs,
+                     GenericTensorAccessorR const &rhs, GenericTensorAccessorW const &dl,
+                     GenericTensorAccessorW const &dr) {
+  if (!stream.is_gpu()) no_cpu("ElementBinary::backward_kernel");
+  check_ffk(ffk_element_binary_backward(stream.require_gpu(), dt(dout.shape.data_type),
+                                        static_cast<int>(state.value().op_type), dout.ptr, lhs.ptr, rhs.ptr,
+                                        dl.ptr, dr.ptr, get_num_elements(dout.shape.dims), 1),
+            "ElementBinary::backward_kernel");
+}
+void cleanup_kernel(DeviceType, std::optional<ElementBinaryPerDeviceState> const &) {}
+
+}  // namespace Kernels::ElementBinary
+
+// ---- Embedding --------------------------------------------------------------
+
+namespace Kernels::Embedding {
+
+static void bag_geometry(GenericTensorAccessorR const &input, std::optional<AggregateOp> const &aggr,
+                         int64_t &num_bags, int64_t &bag) {
+  int64_t n = get_num_elements(input.shape.dims);
+  bag = aggr.has_value() ? dim_at_idx(input.shape.dims, -1) : 1;
+  num_bags = n / bag;
+}
+
+void forward_kernel(device_stream_t const &stream, GenericTensorAccessorR const &input,
+                    GenericTensorAccessorW const &output, GenericTensorAccessorR const &weight,
+                    DataType input_data_type, DataType output_data_type, std::optional<AggregateOp> aggr,
+                    num_tensor_dims_t, num_tensor_dims_t, int) {
+  if (!stream.is_gpu()) no_cpu("Embedding::forward_kernel");
+  if (input.shape.data_type != input_data_type || output.shape.data_type != output_data_type) {
+    throw std::runtime_error("Embedding::forward_kernel: data types differ from the accessors'");
+  }
+  int64_t num_bags, bag;
+  bag_geometry(input, aggr, num_bags, bag);
+  check_ffk(ffk_embedding_forward(stream.require_gpu(), dt(input_data_type), dt(weight.shape.data_type),
+                                  dt(output_data_type), input.ptr, output.ptr, weight.ptr,
+                                  aggr.has_value() ? static_cast<int>(*aggr) : FFK_AGGR_NONE, num_bags, bag,
+                                  dim_at_idx(weight.shape.dims, 1), dim_at_idx(weight.shape.dims, 0)),
+            "Embedding::forward_kernel");
+}
+
+void backward_kernel(device_stream_t const &stream, GenericTensorAccessorR const &output,
+                     GenericTensorAccessorR const &input, GenericTensorAccessorW const &weight_grad,
+                     DataType output_data_type, DataType input_data_type, std::optional<AggregateOp> aggr,
+                     num_tensor_dims_t, num_tensor_dims_t, int) {
+  if (!stream.is_gpu()) no_cpu("Embedding::backward_kernel");
+  if (weight_grad.shape.data_type != DataType::FLOAT) {
+    throw std::runtime_error("Embedding::backward_kernel: weight_grad must be FLOAT (fp32 accumulators)");
+  }
+  int64_t num_bags, bag;
+  bag_geometry(input, aggr, num_bags, bag);
+  check_ffk(ffk_embedding_backward(stream.require_gpu(), dt(input_data_type), dt(output_data_type), input.ptr,
+                                   output.ptr, static_cast<float *>(weight_grad.ptr),
+                                   aggr.has_value() ? static_cast<int>(*aggr) : FFK_AGGR_NONE, num_bags, bag,
+                                   dim_at_idx(weight_grad.shape.dims, 1), dim_at_idx(weight_grad.shape.dims, 0), 0,
+                                   nullptr, 0),
+            "Embedding::backward_kernel");
+}
+
+}  // namespace Kernels::Embedding
+}  // namespace FlexFlow

@@ -1,0 +1,387 @@
+// Tests of the host mirror, written the way the reference's kernel tests are
+// (lib/kernels/test/src: allocate through an Allocator, fill accessors, call
+// the entry point, copy back, compare).  The CPU oracle is the checker.
+//   test_host --cpu   host-only checks (no device needed)
+//   test_host --gpu   every operator entry point on the device
+#include "ffk_oracle.h"
+#include "kernels/allocation.h"
+#include "kernels/attention_kernels.h"
+#include "kernels/dropout_kernels.h"
+#include "kernels/element_kernels.h"
+#include "kernels/embedding_kernels.h"
+#include "kernels/layer_norm_kernels.h"
+#include "kernels/linear_kernels.h"
+#include "kernels/profiling.h"
+#include "kernels/softmax_kernels.h"
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <random>
+#include <string>
+
+using namespace FlexFlow;
+
+static int g_failed = 0, g_checks = 0;
+#define CHECK(cond)                                                            \
+  do {                                                                         \
+    g_checks++;                                                                \
+    if (!(cond)) {                                                             \
+      g_failed++;                                                              \
+      printf("  CHECK failed: %s (%s:%d)\n", #cond, __FILE__, __LINE__);       \
+    }                                                                          \
+  } while (0)
+#define CHECK_THROWS(expr)                                                     \
+  do {                                                                         \
+    g_checks++;                                                                \
+    bool threw__ = false;                                                      \
+    try { (void)(expr); } catch (std::exception const &) { threw__ = true; }   \
+    if (!threw__) {                                                            \
+      g_failed++;                                                              \
+      printf("  CHECK_THROWS failed: %s (%s:%d)\n", #expr, __FILE__, __LINE__);\
+    }                                                                          \
+  } while (0)
+
+static void run(char const *name, std::function<void()> const &f) {
+  printf("TEST_CASE %s\n", name);
+  fflush(stdout);
+  try {
+    f();
+  } catch (std::exception const &e) {
+    g_failed++;
+    printf("  exception: %s\n", e.what());
+  }
+}
+
+static TensorShape shape(std::vector<int64_t> dims, DataType dtype) { return TensorShape{TensorDims{dims}, dtype}; }
+
+static std::vector<float> random_vec(size_t n, unsigned seed, float lo = -1.0f, float hi = 1.0f) {
+  std::mt19937 gen(seed);  // the reference's tests use std::mt19937(0) and U(-1, 1)
+  std::uniform_real_distribution<float> dist(lo, hi);
+  std::vector<float> v(n);
+  for (auto &x : v) x = dist(gen);
+  return v;
+}
+
+// device accessor filled from host floats (converted to the accessor's dtype)
+static GenericTensorAccessorW device_accessor(Allocator &gpu, TensorShape const &s, std::vector<float> const &host) {
+  Allocator cpu = create_local_cpu_memory_allocator();
+  GenericTensorAccessorW h = cpu.allocate_tensor(s);
+  size_t n = (size_t)get_num_elements(s.dims);
+  if (s.data_type == DataType::FLOAT) {
+    memcpy(h.ptr, host.data(), n * 4);
+  } else if (s.data_type == DataType::BF16) {
+    uint16_t *p = static_cast<uint16_t *>(h.ptr);
+    for (size_t i = 0; i < n; i++) {
+      float r = orc_round_bf16(host[i]);
+      uint32_t u;
+      memcpy(&u, &r, 4);
+      p[i] = (uint16_t)(u >> 16);
+    }
+  } else {
+    throw std::runtime_error("device_accessor: dtype");
+  }
+  GenericTensorAccessorW d = gpu.allocate_tensor(s);
+  copy_accessor_data_to_l_from_r(d, h);
+  return d;
+}
+
+static std::vector<float> to_host(GenericTensorAccessorW const &d) {
+  Allocator cpu = create_local_cpu_memory_allocator();
+  GenericTensorAccessorW h = copy_tensor_accessor_w(d, cpu);
+  size_t n = (size_t)get_num_elements(d.shape.dims);
+  std::vector<float> out(n);
+  if (d.shape.data_type == DataType::FLOAT) {
+    memcpy(out.data(), h.ptr, n * 4);
+  } else {
+    uint16_t const *p = static_cast<uint16_t const *>(h.ptr);
+    for (size_t i = 0; i < n; i++) {
+      uint32_t u = (uint32_t)p[i] << 16;
+      memcpy(&out[i], &u, 4);
+    }
+  }
+  return out;
+}
+
+static bool close(std::vector<float> const &a, std::vector<float> const &b, double rtol) {
+  if (a.size() != b.size()) return false;
+  double scale = 0;
+  for (float v : b) scale = std::max(scale, (double)std::fabs(v));
+  for (size_t i = 0; i < a.size(); i++) {
+    if (std::fabs((double)a[i] - b[i]) > rtol * scale + rtol * std::fabs(b[i])) {
+      printf("  mismatch at %zu: got %g want %g\n", i, a[i], b[i]);
+      return false;
+    }
+  }
+  return true;
+}
+
+static bool contains_non_zero(std::vector<float> const &v) {
+  for (float x : v) if (x != 0.0f) return true;
+  return false;
+}
+
+// ---------------------------------------------------------------------------
+static void cpu_tests() {
+  run("calculate_accessor_offset", [] {
+    CHECK(calculate_accessor_offset({4}, TensorDims{{13}}) == 4);
+    CHECK(calculate_accessor_offset({0, 0}, TensorDims{{5, 6}}) == 0);
+    CHECK(calculate_accessor_offset({1, 0}, TensorDims{{5, 6}}) == 6);
+    CHECK(calculate_accessor_offset({0, 1}, TensorDims{{5, 6}}) == 1);
+    CHECK(calculate_accessor_offset({2, 4}, TensorDims{{5, 6}}) == 2 * 6 + 4);
+    CHECK(calculate_accessor_offset({}, TensorDims{{}}) == 0);
+    CHECK_THROWS(calculate_accessor_offset({1, 2, 4}, TensorDims{{5, 6}}));
+    CHECK_THROWS(calculate_accessor_offset({2, 6}, TensorDims{{5, 6}}));
+  });
+  run("LocalCPUAllocator and accessors", [] {
+    Allocator cpu = create_local_cpu_memory_allocator();
+    CHECK(cpu.get_allocation_device_type() == DeviceType::CPU);
+    GenericTensorAccessorW a = cpu.allocate_tensor(shape({2, 3}, DataType::FLOAT));
+    fill_with_zeros(a);
+    a.at<float>({1, 2}) = 12.0f;
+    GenericTensorAccessorR r = read_only_accessor_from_write_accessor(a);
+    CHECK(r.at<float>({1, 2}) == 12.0f);
+    CHECK(r.get_float_ptr()[5] == 12.0f);
+    CHECK_THROWS(r.get_int32_ptr());
+    CHECK_THROWS(r.at<double>({0, 0}));
+    GenericTensorAccessorW b = copy_tensor_accessor_w(a, cpu);
+    CHECK(b.at<float>({1, 2}) == 12.0f && b.at<float>({0, 0}) == 0.0f);
+    cpu.deallocate_tensor(b);
+    CHECK_THROWS(cpu.deallocate_tensor(b));  // double free is an error
+    CHECK(size_of_datatype(DataType::BF16) == 2 && size_of_datatype(DataType::DOUBLE) == 8);
+  });
+  run("CPU device type is not executed", [] {
+    Allocator cpu = create_local_cpu_memory_allocator();
+    LinearAttrs attrs{2, false, DataType::FLOAT, std::nullopt, std::nullopt};
+    GenericTensorAccessorW x = cpu.allocate_tensor(shape({4, 3}, DataType::FLOAT));
+    GenericTensorAccessorW w = cpu.allocate_tensor(shape({2, 3}, DataType::FLOAT));
+    GenericTensorAccessorW y = cpu.allocate_tensor(shape({4, 2}, DataType::FLOAT));
+    CHECK(!linear_init_kernel(DeviceType::CPU, device_handle_t::for_cpu(), std::nullopt, std::nullopt, false,
+                              DataType::FLOAT, DataType::FLOAT, DataType::FLOAT, 4, 2)
+               .has_value());
+    CHECK_THROWS(linear_forward_kernel(get_cpu_device_stream(), std::nullopt, attrs, x, y, w, std::nullopt));
+  });
+}
+
+// ---------------------------------------------------------------------------
+static void gpu_tests() {
+  ManagedPerDeviceFFHandle managed_handle = initialize_single_gpu_handle(1024 * 1024, true);
+  device_handle_t handle = device_handle_t_from_managed_ff_handle(managed_handle);
+  device_stream_t stream = get_gpu_device_stream();
+  Allocator gpu = create_local_cuda_memory_allocator();
+
+  run("linear_forward_kernel / linear_backward_kernel (reference KAT, exact)", [&] {
+    std::vector<float> x = {3, 3, 6, 2, 1, 5, 1, 2, -2, 8, 0.5, -3}, w = {1, 2, 1.5, 0.5, 4, -1}, b = {3, -1};
+    std::vector<float> dy = {1, -0.5, 2, -2, 1, 9, -3.5, 1};
+    LinearAttrs attrs{2, true, DataType::FLOAT, std::nullopt, std::nullopt};
+    auto state = linear_init_kernel(DeviceType::GPU, handle, std::nullopt, std::nullopt, true, DataType::FLOAT,
+                                    DataType::FLOAT, DataType::FLOAT, 4, 2);
+    auto X = device_accessor(gpu, shape({4, 3}, DataType::FLOAT), x);
+    auto W = device_accessor(gpu, shape({2, 3}, DataType::FLOAT), w);
+    auto B = device_accessor(gpu, shape({2}, DataType::FLOAT), b);
+    auto Y = gpu.allocate_tensor(shape({4, 2}, DataType::FLOAT));
+    linear_forward_kernel(stream, state, attrs, X, Y, W, GenericTensorAccessorR(B));
+    CHECK(to_host(Y) == (std::vector<float>{21, 6.5, 14.5, -1, 5, 9.5, 7.5, 8}));
+    auto DY = device_accessor(gpu, shape({4, 2}, DataType::FLOAT), dy);
+    auto DX = gpu.allocate_tensor(X.shape);
+    auto DW = gpu.allocate_tensor(W.shape);
+    auto DB = gpu.allocate_tensor(B.shape);
+    fill_with_zeros(DX); fill_with_zeros(DW); fill_with_zeros(DB);
+    linear_backward_kernel(stream, state, attrs, Y, DY, X, DX, W, DW, DB);
+    CHECK(to_host(DX) == (std::vector<float>{0.75, 0, 2, 1, -4, 5, 5.5, 38, -7.5, -3, -3, -6.25}));
+    CHECK(to_host(DW) == (std::vector<float>{-20, 5.25, 24.5, 11.5, 15, -34}));
+    CHECK(to_host(DB) == (std::vector<float>{0.5, 7.5}));
+    // gradients accumulate on the GPU path (beta = 1)
+    linear_backward_kernel(stream, state, attrs, Y, DY, X, DX, W, DW, DB);
+    CHECK(to_host(DB) == (std::vector<float>{1.0, 15.0}));
+    linear_cleanup_kernel(DeviceType::GPU, state);
+  });
+
+  run("linear with ReLU vs oracle (config-1 shape)", [&] {
+    int batch = 32, in = 64, out = 128;
+    auto x = random_vec(batch * in, 1), w = random_vec(out * in, 2, -0.05f, 0.05f), b = random_vec(out, 3, -0.05f, 0.05f);
+    auto dy = random_vec(batch * out, 4);
+    std::vector<float> y(batch * out), dx(batch * in), dw(out * in), db(out);
+    orc_linear_forward(0, x.data(), y.data(), w.data(), b.data(), batch, in, out);
+    orc_linear_backward(0, 0, y.data(), dy.data(), x.data(), dx.data(), w.data(), dw.data(), db.data(), batch, in, out);
+    LinearAttrs attrs{out, true, DataType::FLOAT, Activation::RELU, std::nullopt};
+    auto state = linear_init_kernel(DeviceType::GPU, handle, Activation::RELU, std::nullopt, true, DataType::FLOAT,
+                                    DataType::FLOAT, DataType::FLOAT, batch, out);
+    auto X = device_accessor(gpu, shape({batch, in}, DataType::FLOAT), x);
+    auto W = device_accessor(gpu, shape({out, in}, DataType::FLOAT), w);
+    auto B = device_accessor(gpu, shape({out}, DataType::FLOAT), b);
+    auto DY = device_accessor(gpu, shape({batch, out}, DataType::FLOAT), dy);
+    auto Y = gpu.allocate_tensor(shape({batch, out}, DataType::FLOAT));
+    auto DX = gpu.allocate_tensor(X.shape), DW = gpu.allocate_tensor(W.shape), DB = gpu.allocate_tensor(B.shape);
+    fill_with_zeros(DX); fill_with_zeros(DW); fill_with_zeros(DB);
+    auto ms = profiling_wrapper(linear_forward_kernel, ProfilingSettings{1, 3}, DeviceType::GPU, state, attrs,
+                                GenericTensorAccessorR(X), Y, GenericTensorAccessorR(W),
+                                std::optional<GenericTensorAccessorR>(B));
+    CHECK(ms.has_value() && ms->value > 0.0f);
+    CHECK(close(to_host(Y), y, 1e-5));
+    linear_backward_kernel(stream, state, attrs, Y, DY, X, DX, W, DW, DB);
+    CHECK(close(to_host(DX), dx, 1e-5) && close(to_host(DW), dw, 1e-5) && close(to_host(DB), db, 1e-5));
+    // {0, 0}: runs once, reports nothing
+    fill_with_zeros(Y);
+    auto none = profiling_wrapper(linear_forward_kernel, ProfilingSettings{0, 0}, DeviceType::GPU, state, attrs,
+                                  GenericTensorAccessorR(X), Y, GenericTensorAccessorR(W),
+                                  std::optional<GenericTensorAccessorR>(B));
+    CHECK(!none.has_value() && contains_non_zero(to_host(Y)));
+    linear_cleanup_kernel(DeviceType::GPU, state);
+  });
+
+  run("LayerNorm forward/backward vs oracle", [&] {
+    int64_t M = 37, N = 96;
+    auto x = random_vec(M * N, 5, -2, 2), g = random_vec(N, 6, 0.5f, 1.5f), b = random_vec(N, 7), dy = random_vec(M * N, 8);
+    std::vector<float> y(M * N), mean(M), rstd(M), dx(M * N), dg(N), db(N);
+    orc_layer_norm_forward(x.data(), y.data(), g.data(), b.data(), mean.data(), rstd.data(), M, N, 1e-5f);
+    orc_layer_norm_backward(dy.data(), x.data(), mean.data(), rstd.data(), g.data(), dx.data(), dg.data(), db.data(), M, N, 0);
+    auto state = Kernels::LayerNorm::init_kernel(DeviceType::GPU, handle, gpu, true, M, N, 1e-5f);
+    auto X = device_accessor(gpu, shape({M, N}, DataType::FLOAT), x);
+    auto G = device_accessor(gpu, shape({N}, DataType::FLOAT), g);
+    auto Bt = device_accessor(gpu, shape({N}, DataType::FLOAT), b);
+    auto DY = device_accessor(gpu, shape({M, N}, DataType::FLOAT), dy);
+    auto Y = gpu.allocate_tensor(X.shape), DX = gpu.allocate_tensor(X.shape);
+    auto DG = gpu.allocate_tensor(G.shape), DB = gpu.allocate_tensor(G.shape);
+    fill_with_zeros(DX);
+    Kernels::LayerNorm::forward_kernel(stream, state, X, Y, G, Bt);
+    CHECK(close(to_host(Y), y, 2e-5));
+    Kernels::LayerNorm::backward_kernel(stream, state, DY, X, DX, G, DG, DB);
+    CHECK(close(to_host(DX), dx, 5e-5) && close(to_host(DG), dg, 5e-5) && close(to_host(DB), db, 5e-5));
+    Kernels::LayerNorm::cleanup_kernel(DeviceType::GPU, state);
+  });
+
+  run("Softmax over the channel of (n,c,h,w); reference backward is a copy", [&] {
+    int n = 2, c = 5, h = 3, w = 4;
+    auto x = random_vec(n * c * h * w, 9, -4, 4), dy = random_vec(n * c * h * w, 10);
+    std::vector<float> y(x.size()), dx(x.size());
+    orc_softmax_forward(x.data(), y.data(), n, c, h * w);
+    auto state = Kernels::Softmax::init_kernel(DeviceType::GPU, handle, ff_dim_t{1}, n, c, h, w);
+    auto X = device_accessor(gpu, shape({n, c, h, w}, DataType::FLOAT), x);
+    auto DY = device_accessor(gpu, X.shape, dy);
+    auto Y = gpu.allocate_tensor(X.shape), DX = gpu.allocate_tensor(X.shape);
+    Kernels::Softmax::forward_kernel(stream, state, X.get_float_ptr(), Y.get_float_ptr());
+    CHECK(close(to_host(Y), y, 2e-5));
+    Kernels::Softmax::backward_kernel(stream, DY.get_float_ptr(), DX.get_float_ptr(), x.size());
+    CHECK(to_host(DX) == dy);
+    orc_softmax_backward(to_host(Y).data(), dy.data(), dx.data(), n, c, h * w);
+    Kernels::Softmax::backward_kernel(stream, state, Y, DY, DX);
+    CHECK(close(to_host(DX), dx, 5e-5));
+  });
+
+  run("Dropout mask equals the oracle's stream bit for bit", [&] {
+    size_t n = 10 * 1000 + 3;
+    auto x = random_vec(n, 11);
+    std::vector<float> y(n), dx(n);
+    orc_dropout_forward(x.data(), y.data(), n, 0.1f, 12345ull, 0);
+    orc_dropout_backward(x.data(), dx.data(), n, 0.1f, 12345ull, 0, 0);
+    TensorShape s = shape({(int64_t)n}, DataType::FLOAT);
+    auto state = Kernels::Dropout::init_kernel(DeviceType::GPU, handle, 0.1f, 12345ull, s, gpu);
+    auto X = device_accessor(gpu, s, x);
+    auto Y = gpu.allocate_tensor(s), DX = gpu.allocate_tensor(s);
+    Kernels::Dropout::forward_kernel(stream, state, X.get_float_ptr(), Y.get_float_ptr());
+    CHECK(to_host(Y) == y);
+    CHECK(contains_non_zero(to_host(Y)));
+    Kernels::Dropout::backward_kernel(stream, state, X.get_float_ptr(), DX.get_float_ptr());
+    CHECK(to_host(DX) == dx);
+  });
+
+  run("ElementUnary GELU and ElementBinary add/mul vs oracle", [&] {
+    size_t n = 5000;
+    auto x = random_vec(n, 12, -3, 3), r = random_vec(n, 13, 0.5f, 2.0f), dy = random_vec(n, 14);
+    TensorShape s = shape({50, 100}, DataType::FLOAT);
+    ElementUnaryAttrs gelu{OperatorType::GELU, std::nullopt};
+    auto ustate = Kernels::ElementUnary::init_kernel(DeviceType::GPU, s, s, gelu);
+    std::vector<float> y(n), dx(n, 0.0f);
+    orc_element_unary_forward(67, 0.0f, x.data(), y.data(), n);
+    orc_element_unary_backward(67, 0.0f, y.data(), dy.data(), x.data(), dx.data(), n, -1);
+    auto X = device_accessor(gpu, s, x), R = device_accessor(gpu, s, r), DY = device_accessor(gpu, s, dy);
+    auto Y = gpu.allocate_tensor(s), DX = gpu.allocate_tensor(s), DR = gpu.allocate_tensor(s);
+    fill_with_zeros(DX);
+    Kernels::ElementUnary::forward_kernel(stream, ustate, gelu, handle, X, Y);
+    CHECK(close(to_host(Y), y, 2e-5));
+    Kernels::ElementUnary::backward_kernel(stream, ustate, gelu, handle, Y, DY, X, DX);
+    CHECK(close(to_host(DX), dx, 2e-5));
+    for (OperatorType op : {OperatorType::EW_ADD, OperatorType::EW_MUL}) {
+      auto bstate = Kernels::ElementBinary::init_kernel(DeviceType::GPU, handle, op, false, false, s, s, s);
+      std::vector<float> o(n), dl(n, 0.0f), dr(n, 0.0f);
+      orc_element_binary_forward(static_cast<int>(op), x.data(), r.data(), o.data(), n, n, n);
+      orc_element_binary_backward(static_cast<int>(op), dy.data(), x.data(), r.data(), dl.data(), dr.data(), n, 1);
+      Kernels::ElementBinary::forward_kernel(stream, bstate, X.get_float_ptr(), R.get_float_ptr(), Y.get_float_ptr(),
+                                             op, false, handle);
+      CHECK(close(to_host(Y), o, 1e-6));
+      fill_with_zeros(DX); fill_with_zeros(DR);
+      Kernels::ElementBinary::backward_kernel(stream, bstate, DY.get_float_ptr(), X.get_float_ptr(), R.get_float_ptr(),
+                                              DX.get_float_ptr(), DR.get_float_ptr(), op, false, false, handle);
+      CHECK(close(to_host(DX), dl, 1e-6) && close(to_host(DR), dr, 1e-6));
+    }
+  });
+
+  run("Embedding gather (exact) and scatter-add vs oracle", [&] {
+    int64_t V = 97, D = 32, B = 40, bag = 4;
+    auto w = random_vec(V * D, 15), dy = random_vec(B * D, 16);
+    std::vector<int64_t> idx(B * bag);
+    std::mt19937 gen(0);
+    for (auto &i : idx) i = gen() % V;
+    std::vector<int32_t> idx32(idx.begin(), idx.end());
+    std::vector<float> out(B * D), dw(V * D, 0.0f);
+    orc_embedding_forward(idx.data(), out.data(), w.data(), 0, B, bag, D, V);
+    orc_embedding_backward_f64(idx.data(), dy.data(), dw.data(), 0, B, bag, D, V);
+    Allocator cpu = create_local_cpu_memory_allocator();
+    GenericTensorAccessorW hidx = cpu.allocate_tensor(shape({B, bag}, DataType::INT32));
+    memcpy(hidx.ptr, idx32.data(), idx32.size() * 4);
+    GenericTensorAccessorW I = copy_tensor_accessor_w(hidx, gpu);
+    auto W = device_accessor(gpu, shape({V, D}, DataType::FLOAT), w);
+    auto DYa = device_accessor(gpu, shape({B, D}, DataType::FLOAT), dy);
+    auto O = gpu.allocate_tensor(shape({B, D}, DataType::FLOAT)), DW = gpu.allocate_tensor(W.shape);
+    fill_with_zeros(DW);
+    Kernels::Embedding::forward_kernel(stream, I, O, W, DataType::INT32, DataType::FLOAT, AggregateOp::SUM, 2, 2, (int)B);
+    CHECK(to_host(O) == out);
+    Kernels::Embedding::backward_kernel(stream, DYa, I, DW, DataType::FLOAT, DataType::INT32, AggregateOp::SUM, 2, 2, (int)B);
+    CHECK(close(to_host(DW), dw, 1e-5));
+  });
+
+  run("MultiHeadAttention (bf16 accessors) vs oracle; fp32 pointers are refused", [&] {
+    int B = 2, H = 4, E = 64, D = 64, S = 20;  // the reference test's sizes, [batch, seq, size]
+    auto q = random_vec(B * S * E, 17), dout = random_vec(B * S * E, 18);
+    size_t nw = (size_t)H * D * 3 * E + (size_t)E * H * D;
+    auto w = random_vec(nw, 19, -0.2f, 0.2f);
+    for (auto *v : {&q, &dout, &w}) orc_round_bf16_array(v->data(), v->size());
+    orc_mha_desc_t od{B, H, E, E, E, D, D, D, E, S, S, 1.0f, 0};
+    std::vector<float> out(B * S * E), dq(q.size()), dk(q.size()), dv(q.size()), dw(nw, 0.0f);
+    orc_mha_forward(&od, q.data(), q.data(), q.data(), w.data(), out.data(), 1);
+    orc_mha_backward(&od, q.data(), q.data(), q.data(), w.data(), dout.data(), dq.data(), dk.data(), dv.data(), dw.data(), 1);
+    for (size_t i = 0; i < dq.size(); i++) dq[i] += dk[i] + dv[i];
+    auto state = Kernels::MultiHeadAttention::init_kernel(DeviceType::GPU, handle, gpu, B, H, E, E, E, D, D, D, E, S, S,
+                                                          false, DataType::BF16, 1.0f, false);
+    CHECK(state->weightSize == nw * 2);
+    auto Q = device_accessor(gpu, shape({B, S, E}, DataType::BF16), q);
+    auto W = device_accessor(gpu, shape({(int64_t)nw}, DataType::BF16), w);
+    auto DO = device_accessor(gpu, Q.shape, dout);
+    auto O = gpu.allocate_tensor(Q.shape), DQ = gpu.allocate_tensor(Q.shape), DW = gpu.allocate_tensor(W.shape);
+    fill_with_zeros(DQ); fill_with_zeros(DW);
+    Kernels::MultiHeadAttention::forward_kernel(stream, state, Q, Q, Q, W, O);
+    CHECK(contains_non_zero(to_host(O)));
+    CHECK(close(to_host(O), out, 2e-2));
+    Kernels::MultiHeadAttention::backward_kernel(stream, state, Q, DQ, Q, std::nullopt, Q, std::nullopt, W, DW, DO);
+    CHECK(close(to_host(DQ), dq, 2e-2) && close(to_host(DW), dw, 2e-2));
+    Kernels::MultiHeadAttention::cleanup_kernel(DeviceType::GPU, gpu, state);
+    auto fstate = Kernels::MultiHeadAttention::init_kernel(DeviceType::GPU, handle, gpu, B, H, E, E, E, D, D, D, E, S, S, false);
+    CHECK_THROWS(Kernels::MultiHeadAttention::forward_kernel(stream, fstate, (float const *)Q.ptr, (float const *)Q.ptr,
+                                                             (float const *)Q.ptr, (float const *)W.ptr, (float *)O.ptr));
+  });
+}
+
+int main(int argc, char **argv) {
+  std::string mode = argc > 1 ? argv[1] : "--cpu";
+  if (mode == "--cpu") {
+    cpu_tests();
+  } else if (mode == "--gpu") {
+    gpu_tests();
+  } else {
+    printf("usage: test_host --cpu | --gpu\n");
+    return 2;
+  }
+  printf("%d checks, %d failed\n", g_checks, g_failed);
+  return g_failed == 0 ? 0 : 1;
+}
