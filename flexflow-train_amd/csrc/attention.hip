@@ -56,24 +56,30 @@ __device__ __forceinline__ bf16x8 pack8(float const *v) {
 
 // B- or A-operand fragment from a row-major LDS tile whose rows are the
 // operand's rows/columns and whose contiguous dim is the reduction dim.
-__device__ __forceinline__ bf16x8 frag_k(bf16 const *tile, int stride, int row0,
-                                         int k0, int lane) {
-  return *reinterpret_cast<bf16x8 const *>(tile + (row0 + (lane & 31)) * stride +
-                                           k0 + (lane >> 5) * 8);
+// The lane-dependent part of the address (lane_k_off) is computed once per
+// kernel; row0 / k0 are compile-time after unrolling and fold into the
+// instruction's offset field.
+__device__ __forceinline__ int lane_k_off(int stride, int lane) {
+  return (lane & 31) * stride + (lane >> 5) * 8;
+}
+__device__ __forceinline__ bf16x8 frag_k(bf16 const *tile_plus_lane, int stride,
+                                         int row0, int k0) {
+  return *reinterpret_cast<bf16x8 const *>(tile_plus_lane + row0 * stride + k0);
 }
 
 // Fragment from an LDS tile stored [reduction index][row/column index]
 // (contiguous along the operand's non-reduction dim), using the reduction
 // order of an accumulator re-used as the other operand: k-slot (h, j) of step
 // s is tile row  r0 + 16 s + 8 (j / 4) + 4 h + j % 4.
-__device__ __forceinline__ bf16x8 frag_tr_acc(bf16 const *tile, int stride,
-                                              int r0, int s, int col0, int lane) {
+__device__ __forceinline__ int lane_tr_off(int stride, int lane) {
   int const i16 = lane & 15;
-  int const h = lane >> 5;
-  int const col = col0 + ((lane >> 4) & 1) * 16 + (i16 & 3) * 4;
-  int const row = r0 + 16 * s + 4 * h + (i16 >> 2);
-  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(tile + row * stride + col));
-  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(tile + (row + 8) * stride + col));
+  return (4 * (lane >> 5) + (i16 >> 2)) * stride + ((lane >> 4) & 1) * 16 + (i16 & 3) * 4;
+}
+__device__ __forceinline__ bf16x8 frag_tr_acc(bf16 const *tile_plus_lane, int stride,
+                                              int r0, int s, int col0) {
+  bf16 const *p = tile_plus_lane + (r0 + 16 * s) * stride + col0;
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 8 * stride));
   union {
     s16x4 h2[2];
     bf16x8 v;
@@ -96,14 +102,17 @@ struct AttnCfg {
 // forward
 // --------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
   using C = AttnCfg<D>;
   __shared__ __attribute__((aligned(16))) bf16 Ks[2][C::kBKV * C::kKStride];
   __shared__ __attribute__((aligned(16))) bf16 Vs[2][C::kBKV * C::kVStride];
   int const t = threadIdx.x, lane = t & 63, wave = t >> 6, h32 = lane >> 5;
+  // 1-D grid ordered so that, under a causal mask, the heaviest (latest) query
+  // blocks of every (batch, head) are dispatched first and light ones fill the tail.
   int const nqb = (p.Sq + C::kBQ - 1) / C::kBQ;
-  int const qb = nqb - 1 - blockIdx.x;  // heavy (late) causal blocks first
-  int const head = blockIdx.y, b = blockIdx.z;
+  int const hb = blockIdx.x % (p.H * p.B);
+  int const qb = nqb - 1 - blockIdx.x / (p.H * p.B);
+  int const head = hb % p.H, b = hb / p.H;
   int const q0 = qb * C::kBQ;
   int const qrow = q0 + wave * 32 + (lane & 31);  // this lane's query row
   bf16 const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * D;
@@ -152,6 +161,8 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
     for (int r = 0; r < 16; r++) oacc[i][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
 
+  int const koff = lane_k_off(C::kKStride, lane);
+  int const voff = lane_tr_off(C::kVStride, lane);
   gload(0);
   lstore(0);
   __syncthreads();
@@ -164,6 +175,8 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
     // A wave whose rows all lie before this tile (causal) has nothing to add.
     bool const active = !p.causal || kv0 <= q0 + wave * 32 + 31;
     if (active) {
+      bf16 const *kt = Ks[cur] + koff;
+      bf16 const *vt = Vs[cur] + voff;
       // S^T tiles: rows = keys (32 per tile), columns = this wave's queries.
       f32x16 s[C::kBKV / 32];
 #pragma unroll
@@ -172,7 +185,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
         for (int r = 0; r < 16; r++) s[j][r] = 0.0f;
 #pragma unroll
         for (int kk = 0; kk < D / 16; kk++) {
-          bf16x8 kf = frag_k(Ks[cur], C::kKStride, j * 32, kk * 16, lane);
+          bf16x8 kf = frag_k(kt, C::kKStride, j * 32, kk * 16);
           s[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[j], 0, 0, 0);
         }
       }
@@ -203,10 +216,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
         float pv[16];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          // Round to bf16 first so that the row sum is the sum of the values
-          // that actually enter the P V product.
           float e = __builtin_amdgcn_exp2f(s[j][r] - m_new);
-          e = bf16_bits_to_f32(f32_to_bf16_bits(e));
           pv[r] = e;
           sum += e;
         }
@@ -216,16 +226,21 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
       sum += __shfl_xor(sum, 32, 64);
       l_run = l_run * alpha + sum;
       m_run = m_new;
+      // Rescale the running output only when some row's maximum moved.
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int i = 0; i < D / 32; i++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+      }
       // O^T += V^T P^T : A = V^T (rows d) via transposing loads, B = P^T.
 #pragma unroll
       for (int i = 0; i < D / 32; i++) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
-#pragma unroll
         for (int j = 0; j < C::kBKV / 32; j++) {
 #pragma unroll
           for (int s2 = 0; s2 < 2; s2++) {
-            bf16x8 vf = frag_tr_acc(Vs[cur], C::kVStride, j * 32, s2, i * 32, lane);
+            bf16x8 vf = frag_tr_acc(vt, C::kVStride, j * 32, s2, i * 32);
             oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[2 * j + s2], oacc[i], 0, 0, 0);
           }
         }
@@ -303,10 +318,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
   using C = AttnBwdCfg<D>;
   __shared__ __attribute__((aligned(16))) bf16 Qs[2][C::kTile * C::kStride];
   __shared__ __attribute__((aligned(16))) bf16 Gs[2][C::kTile * C::kStride];  // dO
-  __shared__ float Ls[2][C::kTile], Ds[2][C::kTile];
+  __shared__ __attribute__((aligned(16))) float Ls[2][C::kTile], Ds[2][C::kTile];
   int const t = threadIdx.x, lane = t & 63, wave = t >> 6, h32 = lane >> 5;
-  int const head = blockIdx.y, b = blockIdx.z;
-  int const kv0 = blockIdx.x * C::kBlk;
+  // key block 0 sees every query under a causal mask: heaviest first for all heads
+  int const hb = blockIdx.x % (p.H * p.B);
+  int const head = hb % p.H, b = hb / p.H;
+  int const kv0 = (blockIdx.x / (p.H * p.B)) * C::kBlk;
   int const kvrow = kv0 + wave * 32 + (lane & 31);
   bf16 const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * D;
   bf16 const *gp = p.d_o + (int64_t)b * p.o_bs + (int64_t)head * D;
@@ -368,6 +385,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
     }
   };
 
+  int const koff = lane_k_off(C::kStride, lane);
+  int const toff = lane_tr_off(C::kStride, lane);
   if (ntiles > 0) {
     gload(q_begin);
     lstore(0);
@@ -381,6 +400,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
     // A wave whose keys all lie after this query tile (causal) contributes 0.
     bool const active = !p.causal || kv0 + wave * 32 <= qt0 + C::kTile - 1;
     if (active) {
+      bf16 const *qk = Qs[cur] + koff, *gk = Gs[cur] + koff;
+      bf16 const *qtr = Qs[cur] + toff, *gtr = Gs[cur] + toff;
       // S = Q K^T and dP = dO V^T: rows = queries of the tile, column = key.
       f32x16 s, dp;
 #pragma unroll
@@ -390,21 +411,30 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
       }
 #pragma unroll
       for (int kk = 0; kk < D / 16; kk++) {
-        bf16x8 qa = frag_k(Qs[cur], C::kStride, 0, kk * 16, lane);
+        bf16x8 qa = frag_k(qk, C::kStride, 0, kk * 16);
         s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s, 0, 0, 0);
-        bf16x8 ga = frag_k(Gs[cur], C::kStride, 0, kk * 16, lane);
+        bf16x8 ga = frag_k(gk, C::kStride, 0, kk * 16);
         dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[kk], dp, 0, 0, 0);
       }
       float pv[16], dsv[16];
+      bool const edge = qt0 + C::kTile > p.Sq || kvrow >= p.Skv || (p.causal && kv0 + wave * 32 + 31 > qt0);
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        int const qi = 8 * (r >> 2) + 4 * h32 + (r & 3);
-        int const qg = qt0 + qi;
-        float e = __builtin_amdgcn_exp2f(s[r] * p.scale_log2 - Ls[cur][qi]);
-        bool const masked = qg >= p.Sq || kvrow >= p.Skv || (p.causal && kvrow > qg);
-        e = masked ? 0.0f : e;
-        pv[r] = e;
-        dsv[r] = e * (dp[r] - Ds[cur][qi]) * p.scale;
+      for (int g = 0; g < 4; g++) {
+        // rows 8 g + 4 h + 0..3 of the tile: one 16-byte read each
+        f32x4 const lrow = *reinterpret_cast<f32x4 const *>(&Ls[cur][8 * g + 4 * h32]);
+        f32x4 const drow = *reinterpret_cast<f32x4 const *>(&Ds[cur][8 * g + 4 * h32]);
+#pragma unroll
+        for (int e4 = 0; e4 < 4; e4++) {
+          int const r = 4 * g + e4;
+          float e = __builtin_amdgcn_exp2f(s[r] * p.scale_log2 - lrow[e4]);
+          if (edge) {
+            int const qg = qt0 + 8 * g + 4 * h32 + e4;
+            bool const masked = qg >= p.Sq || kvrow >= p.Skv || (p.causal && kvrow > qg);
+            e = masked ? 0.0f : e;
+          }
+          pv[r] = e;
+          dsv[r] = e * (dp[r] - drow[e4]) * p.scale;
+        }
       }
       // dV += P^T dO ; dK += dS^T Q.  A = accumulator re-used (row = key),
       // B = dO / Q read with the matching reduction order (k = query).
@@ -414,9 +444,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
         bf16x8 da = pack8(dsv + 8 * s2);
 #pragma unroll
         for (int i = 0; i < D / 32; i++) {
-          bf16x8 gb = frag_tr_acc(Gs[cur], C::kStride, 0, s2, i * 32, lane);
+          bf16x8 gb = frag_tr_acc(gtr, C::kStride, 0, s2, i * 32);
           dv[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa, gb, dv[i], 0, 0, 0);
-          bf16x8 qb = frag_tr_acc(Qs[cur], C::kStride, 0, s2, i * 32, lane);
+          bf16x8 qb = frag_tr_acc(qtr, C::kStride, 0, s2, i * 32);
           dk[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, qb, dk[i], 0, 0, 0);
         }
       }
@@ -451,8 +481,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
   __shared__ __attribute__((aligned(16))) bf16 Vs[2][C::kTile * C::kStride];
   int const t = threadIdx.x, lane = t & 63, wave = t >> 6, h32 = lane >> 5;
   int const nqb = (p.Sq + C::kBlk - 1) / C::kBlk;
-  int const qb = nqb - 1 - blockIdx.x;
-  int const head = blockIdx.y, b = blockIdx.z;
+  int const hb = blockIdx.x % (p.H * p.B);
+  int const qb = nqb - 1 - blockIdx.x / (p.H * p.B);
+  int const head = hb % p.H, b = hb / p.H;
   int const q0 = qb * C::kBlk;
   int const qrow = q0 + wave * 32 + (lane & 31);
   bf16 const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * D;
@@ -503,6 +534,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
     }
   };
 
+  int const koff = lane_k_off(C::kStride, lane);
+  int const toff = lane_tr_off(C::kStride, lane);
   gload(0);
   lstore(0);
   __syncthreads();
@@ -513,6 +546,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
     if (more) gload(kt0 + C::kTile);
     bool const active = !p.causal || kt0 <= q0 + wave * 32 + 31;
     if (active) {
+      bf16 const *kk_ = Ks[cur] + koff, *vk_ = Vs[cur] + koff, *ktr = Ks[cur] + toff;
       // S^T = K Q^T, dP^T = V dO^T: rows = keys of the tile, column = query.
       f32x16 s, dp;
 #pragma unroll
@@ -522,18 +556,21 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
       }
 #pragma unroll
       for (int kk = 0; kk < D / 16; kk++) {
-        bf16x8 ka = frag_k(Ks[cur], C::kStride, 0, kk * 16, lane);
+        bf16x8 ka = frag_k(kk_, C::kStride, 0, kk * 16);
         s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], s, 0, 0, 0);
-        bf16x8 va = frag_k(Vs[cur], C::kStride, 0, kk * 16, lane);
+        bf16x8 va = frag_k(vk_, C::kStride, 0, kk * 16);
         dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, gf[kk], dp, 0, 0, 0);
       }
       float dsv[16];
+      bool const edge = kt0 + C::kTile > p.Skv || (p.causal && kt0 + C::kTile - 1 > q0 + wave * 32);
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        int const kv = kt0 + 8 * (r >> 2) + 4 * h32 + (r & 3);
         float e = __builtin_amdgcn_exp2f(s[r] * p.scale_log2 - lse2);
-        bool const masked = kv >= p.Skv || (p.causal && kv > qrow);
-        e = masked ? 0.0f : e;
+        if (edge) {
+          int const kv = kt0 + 8 * (r >> 2) + 4 * h32 + (r & 3);
+          bool const masked = kv >= p.Skv || (p.causal && kv > qrow);
+          e = masked ? 0.0f : e;
+        }
         dsv[r] = e * (dp[r] - delta) * p.scale;
       }
       // dQ^T += K^T dS^T : A = K^T (rows d) via transposing loads, B = dS^T.
@@ -542,7 +579,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
         bf16x8 db = pack8(dsv + 8 * s2);
 #pragma unroll
         for (int i = 0; i < D / 32; i++) {
-          bf16x8 ka = frag_tr_acc(Ks[cur], C::kStride, 0, s2, i * 32, lane);
+          bf16x8 ka = frag_tr_acc(ktr, C::kStride, 0, s2, i * 32);
           dq[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, db, dq[i], 0, 0, 0);
         }
       }
@@ -573,7 +610,8 @@ static int check_desc(char const *who, int dtype, ffk_attention_desc_t const *d)
   FFK_REQUIRE(d->head_dim == 64 || d->head_dim == 128,
               "%s: head_dim %lld not supported (64 or 128)", who, (long long)d->head_dim);
   FFK_REQUIRE(d->batch > 0 && d->heads > 0 && d->seq_q > 0 && d->seq_kv > 0, "%s: bad shape", who);
-  FFK_REQUIRE(d->batch < 65536 && d->heads < 65536, "%s: batch/heads exceed the grid limit", who);
+  FFK_REQUIRE(d->batch * d->heads * ((d->seq_q > d->seq_kv ? d->seq_q : d->seq_kv) / 128 + 1) < (1ll << 31),
+              "%s: too many workgroups", who);
   FFK_REQUIRE(d->seq_q < (1ll << 30) && d->seq_kv < (1ll << 30), "%s: sequence too long", who);
   FFK_REQUIRE(d->q_seq_stride % 8 == 0 && d->k_seq_stride % 8 == 0 && d->v_seq_stride % 8 == 0 &&
                   d->o_seq_stride % 8 == 0 && d->q_batch_stride % 8 == 0 && d->k_batch_stride % 8 == 0 &&
@@ -611,7 +649,7 @@ extern "C" int ffk_attention_forward(ffk_stream_t stream, int dtype,
   p.o_bs = d->o_batch_stride; p.o_ss = d->o_seq_stride;
   p.scale_log2 = d->scale * kLog2e;
   p.causal = d->causal;
-  dim3 grid((unsigned)ceil_div(p.Sq, 128), (unsigned)p.H, (unsigned)p.B);
+  dim3 grid((unsigned)(ceil_div(p.Sq, 128) * p.H * p.B));
   if (d->head_dim == 64) {
     attn_fwd_kernel<64><<<grid, 256, 0, as_stream(stream)>>>(p);
   } else {
@@ -656,8 +694,8 @@ extern "C" int ffk_attention_backward(ffk_stream_t stream, int dtype,
   p.causal = d->causal;
   hipStream_t st = as_stream(stream);
   int64_t rows = (int64_t)p.B * p.H * p.Sq;
-  dim3 gkv((unsigned)ceil_div(p.Skv, 128), (unsigned)p.H, (unsigned)p.B);
-  dim3 gq((unsigned)ceil_div(p.Sq, 128), (unsigned)p.H, (unsigned)p.B);
+  dim3 gkv((unsigned)(ceil_div(p.Skv, 128) * p.H * p.B));
+  dim3 gq((unsigned)(ceil_div(p.Sq, 128) * p.H * p.B));
   if (d->head_dim == 64) {
     attn_delta_kernel<64><<<(unsigned)ceil_div(rows, 4), 256, 0, st>>>(p);
     FFK_CHECK_LAUNCH();

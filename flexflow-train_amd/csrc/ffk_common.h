@@ -79,8 +79,11 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);
   return u >> 16;
 }
+// Two fp32 -> packed bf16x2 in one instruction (v_cvt_pk_bf16_f32, RNE).
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  f32x2 v = {lo, hi};
+  bf16x2 b = __builtin_convertvector(v, bf16x2);
+  return __builtin_bit_cast(uint32_t, b);
 }
 
 // ---- typed vector access: N elements of T <-> N floats --------------------

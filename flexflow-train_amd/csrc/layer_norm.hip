@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256) void layer_norm_bwd_generic_param_kernel(
   if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, sb);
 }
 
-constexpr int kLnBwdMaxBlocks = 2 * kNumCU;
+constexpr int kLnBwdMaxBlocks = kNumCU;
 
 static int ln_bwd_blocks(int64_t M, int wpr) {
   int64_t rpb = 4 / wpr;
@@ -391,7 +391,7 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
   int ept = 0, wpr = 0;
   bool vec = (N % V == 0) && aligned16(dy) && aligned16(x) &&
              (dx == nullptr || aligned16(dx)) &&
-             (gamma == nullptr || aligned16(gamma)) && pick_row_config(N / V, ept, wpr);
+             (gamma == nullptr || aligned16(gamma)) && pick_row_config_small(N / V, ept, wpr);
   if (vec) {
     int const blocks = ln_bwd_blocks(M, wpr);
     size_t need = (size_t)blocks * 2 * (size_t)N * sizeof(float);
@@ -410,7 +410,7 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
       layer_norm_bwd_kernel<T, E, W, false><<<blocks, kRowThreads, 0, st>>>(   \
           DY, X, mean, rstd, G, DX, partials, M, (int)N);                      \
   } while (0)
-    FFK_ROW_DISPATCH(ept, wpr, CALL);
+    FFK_ROW_DISPATCH_SMALL(ept, wpr, CALL);
 #undef CALL
     FFK_CHECK_LAUNCH();
     if (dgamma != nullptr || dbeta != nullptr) {

@@ -70,6 +70,36 @@ static inline bool pick_row_config(int64_t nvec, int &ept, int &wpr) {
   return false;
 }
 
+// Backward kernels keep several row-sized arrays in registers, so they switch
+// to one workgroup per row much earlier (at most 2 vectors per lane per array
+// while the row fits 256 x 2 vectors).
+static inline bool pick_row_config_small(int64_t nvec, int &ept, int &wpr) {
+  if (nvec <= 128) {
+    wpr = 1;
+    ept = nvec <= 64 ? 1 : 2;
+    return true;
+  }
+  if (nvec <= 256 * 8) {
+    wpr = 4;
+    ept = nvec <= 256 ? 1 : nvec <= 512 ? 2 : nvec <= 1024 ? 4 : 8;
+    return true;
+  }
+  return false;
+}
+
+#define FFK_ROW_DISPATCH_SMALL(EPT_, WPR_, CALL)                               \
+  do {                                                                         \
+    if ((WPR_) == 1) {                                                         \
+      if ((EPT_) == 1) { CALL(1, 1); }                                         \
+      else { CALL(2, 1); }                                                     \
+    } else {                                                                   \
+      if ((EPT_) == 1) { CALL(1, 4); }                                         \
+      else if ((EPT_) == 2) { CALL(2, 4); }                                    \
+      else if ((EPT_) == 4) { CALL(4, 4); }                                    \
+      else { CALL(8, 4); }                                                     \
+    }                                                                          \
+  } while (0)
+
 #define FFK_ROW_DISPATCH(EPT_, WPR_, CALL)                                     \
   do {                                                                         \
     if ((WPR_) == 1) {                                                         \
