@@ -9,6 +9,20 @@ namespace ffk {
 #define FFK_SQRT1_2 0.70710678118654752440f
 #define FFK_INV_SQRT_2PI 0.39894228040143267794f
 
+// erf by Abramowitz & Stegun 7.1.26 (|error| <= 1.5e-7), sharing exp(-z^2)
+// with the caller: returns erf(z) given e = exp(-z*z).
+__device__ __forceinline__ float erf_from_exp(float z, float e) {
+  float const az = fabsf(z);
+  float const t = __frcp_rn(1.0f + 0.3275911f * az);
+  float poly = 1.061405429f;
+  poly = poly * t - 1.453152027f;
+  poly = poly * t + 1.421413741f;
+  poly = poly * t - 0.284496736f;
+  poly = poly * t + 0.254829592f;
+  float const r = 1.0f - poly * t * e;
+  return copysignf(r, z);
+}
+
 template <int OP>
 struct UnaryFwd {
   float s;
@@ -23,7 +37,11 @@ struct UnaryFwd {
     else if (OP == FFK_OP_POW) r = powf(v, s);
     else if (OP == FFK_OP_EXP) r = expf(v);
     else if (OP == FFK_OP_IDENTITY) r = v;
-    else if (OP == FFK_OP_GELU) r = v * (0.5f + 0.5f * erff(v * FFK_SQRT1_2));  // = x/2 erfc(-x/sqrt2)
+    else if (OP == FFK_OP_GELU) {
+      // x/2 erfc(-x/sqrt2) = x (1/2 + 1/2 erf(x/sqrt2))
+      float const z = v * FFK_SQRT1_2;
+      r = v * (0.5f + 0.5f * erf_from_exp(z, __expf(-z * z)));
+    }
     else if (OP == FFK_OP_RSQRT) r = 1.0f / sqrtf(v);
     else if (OP == FFK_OP_SIN) r = sinf(v);
     else if (OP == FFK_OP_COS) r = cosf(v);
@@ -53,8 +71,11 @@ struct UnaryBwd {
     else if (OP == FFK_OP_IDENTITY) g = dy;
     else if (OP == FFK_OP_GELU)
       // d/dx [x Phi(x)] = Phi(x) + x phi(x)
-      g = dy * (0.5f + 0.5f * erff(x * FFK_SQRT1_2) +
-                x * FFK_INV_SQRT_2PI * __expf(-0.5f * x * x));
+    {
+      float const z = x * FFK_SQRT1_2;
+      float const e = __expf(-z * z);  // = exp(-x^2 / 2), shared by Phi and phi
+      g = dy * (0.5f + 0.5f * erf_from_exp(z, e) + x * FFK_INV_SQRT_2PI * e);
+    }
     else if (OP == FFK_OP_GELU_REFERENCE_GRAD)
       // literal text of element_unary_kernels.cu:226-231
       g = dy * (0.5f * erfcf(-x * FFK_SQRT1_2) -

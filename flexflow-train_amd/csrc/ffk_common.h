@@ -102,6 +102,15 @@ struct VecIO<float> {
     f32x4 r = {v[0], v[1], v[2], v[3]};
     *reinterpret_cast<f32x4 *>(p) = r;
   }
+  // streaming variants: data touched once, do not keep it in the caches
+  __device__ __forceinline__ static void load_stream(float const *p, float (&v)[4]) {
+    f32x4 r = __builtin_nontemporal_load(reinterpret_cast<f32x4 const *>(p));
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  __device__ __forceinline__ static void store_stream(float *p, float const (&v)[4]) {
+    f32x4 r = {v[0], v[1], v[2], v[3]};
+    __builtin_nontemporal_store(r, reinterpret_cast<f32x4 *>(p));
+  }
   __device__ __forceinline__ static float load1(float const *p) { return *p; }
   __device__ __forceinline__ static void store1(float *p, float v) { *p = v; }
 };
@@ -125,6 +134,22 @@ struct VecIO<bf16> {
     }
     *reinterpret_cast<u32x4 *>(p) = r;
   }
+  __device__ __forceinline__ static void load_stream(bf16 const *p, float (&v)[8]) {
+    u32x4 r = __builtin_nontemporal_load(reinterpret_cast<u32x4 const *>(p));
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[2 * i] = __uint_as_float(r[i] << 16);
+      v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+    }
+  }
+  __device__ __forceinline__ static void store_stream(bf16 *p, float const (&v)[8]) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      r[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+    }
+    __builtin_nontemporal_store(r, reinterpret_cast<u32x4 *>(p));
+  }
   __device__ __forceinline__ static float load1(bf16 const *p) {
     return bf16_bits_to_f32(*reinterpret_cast<uint16_t const *>(p));
   }
@@ -132,6 +157,23 @@ struct VecIO<bf16> {
     *reinterpret_cast<uint16_t *>(p) = (uint16_t)f32_to_bf16_bits(v);
   }
 };
+
+// Raw 16-byte streaming load, unpacked later: lets a kernel issue the loads of
+// its next row before it works on the current one.
+__device__ __forceinline__ u32x4 load_raw_stream(void const *p) {
+  return __builtin_nontemporal_load(reinterpret_cast<u32x4 const *>(p));
+}
+__device__ __forceinline__ void unpack_raw(u32x4 r, float (&v)[4], float const *) {
+  v[0] = __uint_as_float(r[0]); v[1] = __uint_as_float(r[1]);
+  v[2] = __uint_as_float(r[2]); v[3] = __uint_as_float(r[3]);
+}
+__device__ __forceinline__ void unpack_raw(u32x4 r, float (&v)[8], bf16 const *) {
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    v[2 * i] = __uint_as_float(r[i] << 16);
+    v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+  }
+}
 
 // ---- wavefront reductions (64 lanes, DPP/shuffle based) -------------------
 __device__ __forceinline__ float wave_sum(float v) {

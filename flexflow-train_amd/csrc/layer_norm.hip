@@ -155,12 +155,28 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
   }
 
   int64_t const row_step = (int64_t)gridDim.x * RPB;
+  // The loads of the next row are issued before the current row is reduced, so
+  // two rows of dY and X are in flight per wave.
+  u32x4 rx[EPT], rdy[EPT];
+  auto issue_row = [&](int64_t base) {
+    int64_t const r = min(base + sub, M - 1);
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+      int v = lane + j * LANES;
+      if (v < nvec) {
+        rx[j] = load_raw_stream(X + r * (int64_t)N + (int64_t)v * V);
+        rdy[j] = load_raw_stream(dY + r * (int64_t)N + (int64_t)v * V);
+      }
+    }
+  };
+  int64_t base = (int64_t)blockIdx.x * RPB;
+  if (base < M) issue_row(base);
   // Every wave of a workgroup runs the same number of iterations so the
   // barriers inside the reducer stay aligned.
-  for (int64_t base = (int64_t)blockIdx.x * RPB; base < M; base += row_step) {
+  for (; base < M; base += row_step) {
     int64_t const row = base + sub;
     bool const row_ok = row < M;
-    int64_t const r = row_ok ? row : 0;
+    int64_t const r = row_ok ? row : M - 1;
     float x[EPT][V], dy[EPT][V];
     float const mu = mean[r], rs = rstd[r];
     float s1 = 0.0f, s2 = 0.0f;  // sum dy*g, sum dy*g*xhat
@@ -168,8 +184,8 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
     for (int j = 0; j < EPT; j++) {
       int v = lane + j * LANES;
       if (v < nvec) {
-        VecIO<T>::load(X + r * (int64_t)N + (int64_t)v * V, x[j]);
-        VecIO<T>::load(dY + r * (int64_t)N + (int64_t)v * V, dy[j]);
+        unpack_raw(rx[j], x[j], (T const *)nullptr);
+        unpack_raw(rdy[j], dy[j], (T const *)nullptr);
       } else {
 #pragma unroll
         for (int e = 0; e < V; e++) {
@@ -178,6 +194,7 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
         }
       }
     }
+    if (base + row_step < M) issue_row(base + row_step);
 #pragma unroll
     for (int j = 0; j < EPT; j++) {
 #pragma unroll
@@ -342,7 +359,7 @@ __global__ __launch_bounds__(256) void layer_norm_bwd_generic_param_kernel(
   if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, sb);
 }
 
-constexpr int kLnBwdMaxBlocks = kNumCU;
+constexpr int kLnBwdMaxBlocks = 2 * kNumCU;
 
 static int ln_bwd_blocks(int64_t M, int wpr) {
   int64_t rpb = 4 / wpr;
@@ -362,13 +379,14 @@ static int ln_forward(hipStream_t st, void const *x, void *y, void const *gamma,
   int ept = 0, wpr = 0;
   bool vec = (N % V == 0) && aligned16(x) && aligned16(y) &&
              (gamma == nullptr || aligned16(gamma)) &&
-             (beta == nullptr || aligned16(beta)) && pick_row_config(N / V, ept, wpr);
+             (beta == nullptr || aligned16(beta)) &&
+             pick_row_config_small(N / V, ept, wpr);
   if (vec) {
     int64_t blocks = ceil_div(M, 4 / wpr);
 #define CALL(E, W)                                                             \
   layer_norm_fwd_kernel<T, E, W><<<(unsigned)blocks, kRowThreads, 0, st>>>(    \
       X, Y, G, Bt, mean, rstd, M, (int)N, eps)
-    FFK_ROW_DISPATCH(ept, wpr, CALL);
+    FFK_ROW_DISPATCH_SMALL(ept, wpr, CALL);
 #undef CALL
   } else {
     layer_norm_fwd_generic_kernel<T><<<(unsigned)M, kRowThreads, 0, st>>>(

@@ -85,8 +85,9 @@ __global__ __launch_bounds__(kRowThreads) void softmax_bwd_kernel(
   for (int j = 0; j < EPT; j++) {
     int v = lane + j * LANES;
     if (v < nvec) {
-      VecIO<T>::load(Y + r * (int64_t)N + (int64_t)v * V, y[j]);
-      VecIO<T>::load(dY + r * (int64_t)N + (int64_t)v * V, dy[j]);
+      // two input streams read once: cache-bypassing loads
+      VecIO<T>::load_stream(Y + r * (int64_t)N + (int64_t)v * V, y[j]);
+      VecIO<T>::load_stream(dY + r * (int64_t)N + (int64_t)v * V, dy[j]);
 #pragma unroll
       for (int e = 0; e < V; e++) dot += y[j][e] * dy[j][e];
     }
