@@ -391,20 +391,45 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
     }
   };
 
-  // Fragment readers (see the layouts above).
+  // Fragment readers (see the layouts above).  Everything lane-dependent in
+  // an LDS address is tabulated once here; inside the loop an address is
+  // stage base + table entry + a compile-time constant that folds into the
+  // instruction's offset field, so the k-loop carries almost no address math.
+  constexpr int KS = BK / 16;  // MFMA k-steps per tile
+  // K-contiguous tile: lane l reads row (row0 + l%32), logical chunk 2 kk + l/32.
+  // row0 is a multiple of 32, so the swizzle term depends on the lane only.
+  int kc_off[KS];
+  {
+    int const sw = ((lane & 31) / RPW) & (CPRK - 1);
+#pragma unroll
+    for (int kk = 0; kk < KS; kk++) {
+      kc_off[kk] = (lane & 31) * BK + (((2 * kk + (lane >> 5)) ^ sw) << 3);
+    }
+  }
   auto frag_kc = [&](bf16 const *tile, int row0, int kk) -> bf16x8 {
-    int const row = row0 + (lane & 31);
-    int const pc = (2 * kk + (lane >> 5)) ^ ((row / RPW) & (CPRK - 1));
-    return *reinterpret_cast<bf16x8 const *>(tile + row * BK + pc * 8);
+    return *reinterpret_cast<bf16x8 const *>(tile + kc_off[kk] + row0 * BK);
   };
-  auto frag_tr = [&](bf16 const *tile, int rowlen, int col0, int kk) -> bf16x8 {
+  // Tile lying as [BK][cols]: lane reads rows kk*16 + 8 (l/32) + (l%16)/4 (+4),
+  // columns col0 + 16 ((l/16)%2) + 4 (l%4); the 64-byte segment index is
+  // XOR-ed with (row % 4), which touches only its two low bits.
+  int tr_tab_a[4], tr_tab_b[4];
+  {
     int const i16 = lane & 15;
-    int const col = col0 + ((lane >> 4) & 1) * 16 + (i16 & 3) * 4;
-    int const krow = kk * 16 + (lane >> 5) * 8 + (i16 >> 2);
-    int const pcol = ((((col >> 5) ^ (krow & 3)) << 5) | (col & 31));
+    int const q = i16 >> 2;
+    int const inseg = ((lane >> 4) & 1) * 16 + (i16 & 3) * 4;
+    int const krow = (lane >> 5) * 8 + q;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      tr_tab_a[c] = krow * BM + ((c ^ q) << 5) + inseg;
+      tr_tab_b[c] = krow * BN + ((c ^ q) << 5) + inseg;
+    }
+  }
+  auto frag_tr = [&](bf16 const *tile, int rowlen, int const (&tab)[4], int col0, int kk) -> bf16x8 {
+    int const seg = col0 >> 5;
+    bf16 const *p = tile + tab[seg & 3] + ((seg & ~3) << 5) + kk * 16 * rowlen;
     typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(tile + krow * rowlen + pcol));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(tile + (krow + 4) * rowlen + pcol));
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * rowlen));
     union {
       s16x4 h[2];
       bf16x8 v;
@@ -423,7 +448,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
   int const KT = K / BK;
-  constexpr int KS = BK / 16;  // MFMA k-steps per tile
   static_assert(KS % 2 == 0, "fragment double buffering assumes an even step count");
   static_assert(STAGES >= 3, "need a stage in flight besides the two in use");
 #pragma unroll
@@ -439,11 +463,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
     bf16 const *sb = sa + A_ELEMS;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-      af[buf][i] = TA ? frag_tr(sa, BM, wm0 + i * 32, kk) : frag_kc(sa, wm0 + i * 32, kk);
+      af[buf][i] = TA ? frag_tr(sa, BM, tr_tab_a, wm0 + i * 32, kk) : frag_kc(sa, wm0 + i * 32, kk);
     }
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      bfr[buf][j] = TBL ? frag_tr(sb, BN, wn0 + j * 32, kk) : frag_kc(sb, wn0 + j * 32, kk);
+      bfr[buf][j] = TBL ? frag_tr(sb, BN, tr_tab_b, wn0 + j * 32, kk) : frag_kc(sb, wn0 + j * 32, kk);
     }
   };
   // Tile 0 must have landed (STAGES-2 younger tiles may still be in flight).
