@@ -9,6 +9,7 @@
 // word >= ceil(rate * 2^32).  Nothing is stored between forward and backward:
 // backward regenerates the mask, so both directions move 2 tensors only.
 #include "ffk_common.h"
+#include "fused_ops.h"
 #include <math.h>
 
 namespace ffk {
@@ -50,16 +51,29 @@ __device__ __forceinline__ bool keep(uint32_t word, DropoutParams const &p) {
 
 constexpr int kDropThreads = 256;
 
+// What a fused pass does with the dropped-out value d (rounded to the storage
+// type first, as if a separate dropout op had stored it):
+//   kDropPlain        y = d
+//   kDropAddResidual  y = aux + d            (dropout feeding a residual add)
+//   kDropGeluGrad     y = d * GELU'(aux)     (dropout backward feeding the
+//                                             backward of a GELU whose input was aux)
+enum DropMode { kDropPlain = 0, kDropAddResidual = 1, kDropGeluGrad = 2 };
+
 // offset % 4 == 0, 16-byte aligned pointers: each lane owns whole Philox blocks.
-template <typename T, bool ACC>
+template <typename T, bool ACC, int MODE>
 __global__ __launch_bounds__(kDropThreads) void dropout_vec_kernel(
-    T const *__restrict__ X, T *Y, int64_t n, DropoutParams p) {
+    T const *__restrict__ X, T const *__restrict__ AUX, T *Y, int64_t n, DropoutParams p) {
   constexpr int V = VecIO<T>::kVec;
   int64_t const nvec = n / V;
   int64_t const stride = (int64_t)gridDim.x * kDropThreads;
   for (int64_t i = (int64_t)blockIdx.x * kDropThreads + threadIdx.x; i < nvec; i += stride) {
-    float x[V], y[V];
-    VecIO<T>::load(X + i * V, x);
+    float x[V], y[V], aux[V];
+    if (MODE == kDropPlain) {
+      VecIO<T>::load(X + i * V, x);
+    } else {
+      VecIO<T>::load_stream(X + i * V, x);
+      VecIO<T>::load_stream(AUX + i * V, aux);
+    }
     if (ACC) VecIO<T>::load(Y + i * V, y);
     uint64_t const blk0 = (p.offset + (uint64_t)i * V) >> 2;
 #pragma unroll
@@ -69,6 +83,8 @@ __global__ __launch_bounds__(kDropThreads) void dropout_vec_kernel(
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         float v = keep(w[e], p) ? x[4 * b + e] * p.scale : 0.0f;
+        if (MODE == kDropAddResidual) v = storage_round<T>(v) + aux[4 * b + e];
+        if (MODE == kDropGeluGrad) v = storage_round<T>(v) * gelu_derivative(aux[4 * b + e]);
         y[4 * b + e] = ACC ? y[4 * b + e] + v : v;
       }
     }
@@ -139,7 +155,7 @@ static int dropout_run(hipStream_t st, void const *x, void *y, int64_t n,
   int64_t done = 0;
   if ((p.offset & 3) == 0 && aligned16(x) && aligned16(y) && n >= V) {
     int64_t nvec = n / V;
-    dropout_vec_kernel<T, ACC><<<grid_for(nvec), kDropThreads, 0, st>>>(X, Y, n, p);
+    dropout_vec_kernel<T, ACC, kDropPlain><<<grid_for(nvec), kDropThreads, 0, st>>>(X, nullptr, Y, n, p);
     FFK_CHECK_LAUNCH();
     done = nvec * V;
   }
@@ -148,6 +164,53 @@ static int dropout_run(hipStream_t st, void const *x, void *y, int64_t n,
     FFK_CHECK_LAUNCH();
   }
   return FFK_OK;
+}
+
+// Fused passes used by the encoder-layer sequence; they exist only in the
+// vector form and report "not fusable" otherwise so the caller can run the
+// separate ops instead.
+template <typename T, int MODE>
+static int dropout_fused_typed(hipStream_t st, void const *x, void const *aux,
+                               void *y, int64_t n, DropoutParams const &p) {
+  constexpr int V = VecIO<T>::kVec;
+  dropout_vec_kernel<T, false, MODE><<<grid_for(n / V), kDropThreads, 0, st>>>(
+      static_cast<T const *>(x), static_cast<T const *>(aux), static_cast<T *>(y), n, p);
+  FFK_CHECK_LAUNCH();
+  return FFK_OK;
+}
+
+bool dropout_fusable(int dtype, void const *x, void const *aux, void const *y,
+                     int64_t n, uint64_t offset) {
+  int64_t const V = dtype == FFK_BF16 ? 8 : 4;
+  return (dtype == FFK_BF16 || dtype == FFK_FLOAT) && n > 0 && n % V == 0 &&
+         (offset & 3) == 0 && aligned16(x) && aligned16(aux) && aligned16(y);
+}
+
+static int dropout_fused(char const *who, int mode, hipStream_t st, int dtype,
+                         void const *x, void const *aux, void *y, int64_t n,
+                         float rate, uint64_t seed, uint64_t offset) {
+  FFK_REQUIRE(dropout_fusable(dtype, x, aux, y, n, offset), "%s: operands not fusable", who);
+  DropoutParams p;
+  int rc = make_params(who, rate, seed, offset, p);
+  if (rc != FFK_OK) return rc;
+  if (dtype == FFK_FLOAT) {
+    return mode == kDropAddResidual ? dropout_fused_typed<float, kDropAddResidual>(st, x, aux, y, n, p)
+                                    : dropout_fused_typed<float, kDropGeluGrad>(st, x, aux, y, n, p);
+  }
+  return mode == kDropAddResidual ? dropout_fused_typed<bf16, kDropAddResidual>(st, x, aux, y, n, p)
+                                  : dropout_fused_typed<bf16, kDropGeluGrad>(st, x, aux, y, n, p);
+}
+
+int dropout_add_residual(hipStream_t st, int dtype, void const *x,
+                         void const *residual, void *y, int64_t n, float rate,
+                         uint64_t seed, uint64_t offset) {
+  return dropout_fused("dropout_add_residual", kDropAddResidual, st, dtype, x, residual, y, n, rate, seed, offset);
+}
+
+int dropout_backward_gelu_backward(hipStream_t st, int dtype, void const *dy,
+                                   void const *gelu_input, void *dx, int64_t n,
+                                   float rate, uint64_t seed, uint64_t offset) {
+  return dropout_fused("dropout_backward_gelu_backward", kDropGeluGrad, st, dtype, dy, gelu_input, dx, n, rate, seed, offset);
 }
 
 }  // namespace ffk

@@ -9,20 +9,6 @@ namespace ffk {
 #define FFK_SQRT1_2 0.70710678118654752440f
 #define FFK_INV_SQRT_2PI 0.39894228040143267794f
 
-// erf by Abramowitz & Stegun 7.1.26 (|error| <= 1.5e-7), sharing exp(-z^2)
-// with the caller: returns erf(z) given e = exp(-z*z).
-__device__ __forceinline__ float erf_from_exp(float z, float e) {
-  float const az = fabsf(z);
-  float const t = __frcp_rn(1.0f + 0.3275911f * az);
-  float poly = 1.061405429f;
-  poly = poly * t - 1.453152027f;
-  poly = poly * t + 1.421413741f;
-  poly = poly * t - 0.284496736f;
-  poly = poly * t + 0.254829592f;
-  float const r = 1.0f - poly * t * e;
-  return copysignf(r, z);
-}
-
 template <int OP>
 struct UnaryFwd {
   float s;
@@ -37,11 +23,7 @@ struct UnaryFwd {
     else if (OP == FFK_OP_POW) r = powf(v, s);
     else if (OP == FFK_OP_EXP) r = expf(v);
     else if (OP == FFK_OP_IDENTITY) r = v;
-    else if (OP == FFK_OP_GELU) {
-      // x/2 erfc(-x/sqrt2) = x (1/2 + 1/2 erf(x/sqrt2))
-      float const z = v * FFK_SQRT1_2;
-      r = v * (0.5f + 0.5f * erf_from_exp(z, __expf(-z * z)));
-    }
+    else if (OP == FFK_OP_GELU) r = gelu_forward(v);
     else if (OP == FFK_OP_RSQRT) r = 1.0f / sqrtf(v);
     else if (OP == FFK_OP_SIN) r = sinf(v);
     else if (OP == FFK_OP_COS) r = cosf(v);
@@ -54,13 +36,30 @@ struct UnaryFwd {
   }
 };
 
-// Backward: inputs are (output, output_grad, input[, old input_grad]).
+// Which saved tensors an op's gradient reads; the others are never loaded.
+template <int OP>
+struct UnaryBwdNeeds {
+  static constexpr bool kY = OP == FFK_OP_RSQRT || OP == FFK_OP_SIGMOID ||
+                             OP == FFK_OP_TANH || OP == FFK_OP_ELU;
+  static constexpr bool kX = OP == FFK_OP_POW || OP == FFK_OP_EXP ||
+                             OP == FFK_OP_GELU || OP == FFK_OP_GELU_REFERENCE_GRAD ||
+                             OP == FFK_OP_SIN || OP == FFK_OP_COS ||
+                             OP == FFK_OP_RELU || OP == FFK_OP_ELU;
+  static constexpr int kInputs = 1 + (kY ? 1 : 0) + (kX ? 1 : 0);
+};
+
+// Backward: inputs are (output_grad[, output][, input][, old input_grad]),
+// the optional ones present when UnaryBwdNeeds / ACC say so.
 template <int OP, bool ACC>
 struct UnaryBwd {
+  using Needs = UnaryBwdNeeds<OP>;
+  static constexpr int kIn = Needs::kInputs + (ACC ? 1 : 0);
   float s;
-  __device__ __forceinline__ void operator()(float const (&in)[ACC ? 4 : 3],
+  __device__ __forceinline__ void operator()(float const (&in)[kIn],
                                              float (&out)[1]) const {
-    float y = in[0], dy = in[1], x = in[2];
+    float const dy = in[0];
+    float const y = Needs::kY ? in[1] : 0.0f;
+    float const x = Needs::kX ? in[Needs::kY ? 2 : 1] : 0.0f;
     float g;
     if (OP == FFK_OP_SCALAR_MULTIPLY) g = dy * s;
     else if (OP == FFK_OP_SCALAR_ADD) g = dy;
@@ -71,11 +70,7 @@ struct UnaryBwd {
     else if (OP == FFK_OP_IDENTITY) g = dy;
     else if (OP == FFK_OP_GELU)
       // d/dx [x Phi(x)] = Phi(x) + x phi(x)
-    {
-      float const z = x * FFK_SQRT1_2;
-      float const e = __expf(-z * z);  // = exp(-x^2 / 2), shared by Phi and phi
-      g = dy * (0.5f + 0.5f * erf_from_exp(z, e) + x * FFK_INV_SQRT_2PI * e);
-    }
+      g = dy * gelu_derivative(x);
     else if (OP == FFK_OP_GELU_REFERENCE_GRAD)
       // literal text of element_unary_kernels.cu:226-231
       g = dy * (0.5f * erfcf(-x * FFK_SQRT1_2) -
@@ -88,7 +83,7 @@ struct UnaryBwd {
     else if (OP == FFK_OP_TANH) g = dy * (1.0f - y * y);
     else if (OP == FFK_OP_ELU) g = x > 0.0f ? dy : dy * (y + s);
     else g = dy;
-    out[0] = ACC ? in[3] + g : g;
+    out[0] = ACC ? in[kIn - 1] + g : g;
   }
 };
 
@@ -103,29 +98,30 @@ static hipError_t unary_fwd(hipStream_t st, float s, void const *in, void *out,
   return ew_launch<T, 1, 1>(st, a, UnaryFwd<OP>{s});
 }
 
+template <typename T, int OP, bool ACC>
+static hipError_t unary_bwd_acc(hipStream_t st, float s, void const *y,
+                                void const *dy, void const *x, void *dx,
+                                int64_t n) {
+  using Needs = UnaryBwdNeeds<OP>;
+  constexpr int NIN = UnaryBwd<OP, ACC>::kIn;
+  EwArgs<T, NIN, 1> a;
+  int k = 0;
+  a.in[k++] = static_cast<T const *>(dy);
+  if (Needs::kY) a.in[k++] = static_cast<T const *>(y);
+  if (Needs::kX) a.in[k++] = static_cast<T const *>(x);
+  if (ACC) a.in[k++] = static_cast<T const *>(dx);
+  for (int i = 0; i < NIN; i++) a.in_elems[i] = n;
+  a.out[0] = static_cast<T *>(dx);
+  a.n = n;
+  return ew_launch<T, NIN, 1>(st, a, UnaryBwd<OP, ACC>{s});
+}
+
 template <typename T, int OP>
 static hipError_t unary_bwd(hipStream_t st, float s, void const *y,
                             void const *dy, void const *x, void *dx, int64_t n,
                             bool acc) {
-  if (acc) {
-    EwArgs<T, 4, 1> a;
-    a.in[0] = static_cast<T const *>(y);
-    a.in[1] = static_cast<T const *>(dy);
-    a.in[2] = static_cast<T const *>(x);
-    a.in[3] = static_cast<T const *>(dx);
-    for (int k = 0; k < 4; k++) a.in_elems[k] = n;
-    a.out[0] = static_cast<T *>(dx);
-    a.n = n;
-    return ew_launch<T, 4, 1>(st, a, UnaryBwd<OP, true>{s});
-  }
-  EwArgs<T, 3, 1> a;
-  a.in[0] = static_cast<T const *>(y);
-  a.in[1] = static_cast<T const *>(dy);
-  a.in[2] = static_cast<T const *>(x);
-  for (int k = 0; k < 3; k++) a.in_elems[k] = n;
-  a.out[0] = static_cast<T *>(dx);
-  a.n = n;
-  return ew_launch<T, 3, 1>(st, a, UnaryBwd<OP, false>{s});
+  if (acc) return unary_bwd_acc<T, OP, true>(st, s, y, dy, x, dx, n);
+  return unary_bwd_acc<T, OP, false>(st, s, y, dy, x, dx, n);
 }
 
 // Reference accumulate behaviour per op (element_unary_kernels.cu:172-250:

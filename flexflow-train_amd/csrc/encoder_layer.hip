@@ -3,6 +3,8 @@
 // run the layer's ops (forward in topological order, backward in reverse).
 // Host code only: every arithmetic step is one of the ffk_* kernels.
 #include "ffk_common.h"
+#include "fused_ops.h"
+#include <stdlib.h>
 
 namespace ffk {
 
@@ -69,6 +71,27 @@ static int check_layer(char const *who, int dtype, ffk_encoder_layer_desc_t cons
   return FFK_OK;
 }
 
+// FFK_LAYER_UNFUSED=1 runs every op of the layer as its own kernel (the plain
+// operator sequence); the default fuses neighbours where the result is
+// bit-identical.  For tests that compare the two.
+static bool layer_fusion_enabled() {
+  char const *e = getenv("FFK_LAYER_UNFUSED");  // read per call: tests toggle it
+  return !(e != nullptr && atoi(e) != 0);
+}
+
+// out = residual + dropout(in): one fused pass when possible, else dropout
+// into `scratch` followed by the element-wise add.
+static int dropout_then_add(ffk_stream_t st, int dtype, void const *in, void *scratch,
+                            void const *residual, void *out, int64_t n, float rate,
+                            uint64_t seed) {
+  if (layer_fusion_enabled() && dropout_fusable(dtype, in, residual, out, n, 0)) {
+    return dropout_add_residual(as_stream(st), dtype, in, residual, out, n, rate, seed, 0);
+  }
+  int rc = ffk_dropout_forward(st, dtype, in, scratch, n, rate, seed, 0);
+  if (rc != FFK_OK) return rc;
+  return ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, scratch, residual, out, n, n, n);
+}
+
 #define FFK_TRY(expr)                                                          \
   do {                                                                         \
     int rc__ = (expr);                                                         \
@@ -112,13 +135,10 @@ extern "C" int ffk_encoder_layer_forward(ffk_stream_t st, int dtype,
   FFK_TRY(ffk_mha_forward(st, dtype, &m, attn_in, attn_in, attn_in, w->attn_weight, ws + L.attn_out,
                           ws + L.mha_reserve, L.ln_ws - L.mha_reserve));
   void const *attn_res = ws + L.attn_out;
-  if (d->pre_layer_norm) {  // the reference applies no dropout after attention
-    FFK_TRY(ffk_dropout_forward(st, dtype, ws + L.attn_out, ws + L.attn_drop, T * E, p, d->seed + 0, 0));
-    attn_res = ws + L.attn_drop;
-  }
   void *ffn_in;
   if (d->pre_layer_norm) {
-    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, attn_res, x, ws + L.x1, T * E, T * E, T * E));
+    // x1 = dropout(attn) + x (the reference's encoder applies no dropout here)
+    FFK_TRY(dropout_then_add(st, dtype, ws + L.attn_out, ws + L.attn_drop, x, ws + L.x1, T * E, p, d->seed + 0));
     FFK_TRY(ffk_layer_norm_forward(st, dtype, ws + L.x1, ws + L.h2, w->ln2_gamma, w->ln2_beta,
                                    mean(L.mean2), mean(L.rstd2), T, E, d->ln_eps));
     ffn_in = ws + L.h2;
@@ -130,7 +150,10 @@ extern "C" int ffk_encoder_layer_forward(ffk_stream_t st, int dtype,
     ffn_in = ws + L.x1;
   }
   // dense(d_ff, activation) -> dropout -> dense(d_model) -> dropout
-  if (gelu) {
+  if (gelu && layer_fusion_enabled()) {
+    FFK_TRY(linear_forward_keep_preactivation(as_stream(st), dtype, FFK_ACT_GELU, ffn_in, ws + L.f1,
+                                              ws + L.act1, w->w1, w->b1, T, E, F));
+  } else if (gelu) {
     FFK_TRY(ffk_linear_forward(st, dtype, FFK_ACT_NONE, ffn_in, ws + L.f1, w->w1, w->b1, T, E, F));
     FFK_TRY(ffk_element_unary_forward(st, dtype, FFK_OP_GELU, 0.0f, ws + L.f1, ws + L.act1, T * F));
   } else {
@@ -138,11 +161,10 @@ extern "C" int ffk_encoder_layer_forward(ffk_stream_t st, int dtype,
   }
   FFK_TRY(ffk_dropout_forward(st, dtype, ws + L.act1, ws + L.act1_drop, T * F, p, d->seed + 1, 0));
   FFK_TRY(ffk_linear_forward(st, dtype, FFK_ACT_NONE, ws + L.act1_drop, ws + L.f2, w->w2, w->b2, T, F, E));
-  FFK_TRY(ffk_dropout_forward(st, dtype, ws + L.f2, ws + L.f2_drop, T * E, p, d->seed + 2, 0));
   if (d->pre_layer_norm) {
-    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.x1, ws + L.f2_drop, y, T * E, T * E, T * E));
+    FFK_TRY(dropout_then_add(st, dtype, ws + L.f2, ws + L.f2_drop, ws + L.x1, y, T * E, p, d->seed + 2));
   } else {
-    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.x1, ws + L.f2_drop, ws + L.pre2, T * E, T * E, T * E));
+    FFK_TRY(dropout_then_add(st, dtype, ws + L.f2, ws + L.f2_drop, ws + L.x1, ws + L.pre2, T * E, p, d->seed + 2));
     FFK_TRY(ffk_layer_norm_forward(st, dtype, ws + L.pre2, y, w->ln2_gamma, w->ln2_beta,
                                    mean(L.mean2), mean(L.rstd2), T, E, d->ln_eps));
   }
@@ -181,11 +203,20 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   FFK_TRY(ffk_dropout_backward(st, dtype, g_sum, ws + L.g_f2, T * E, p, d->seed + 2, 0, 0));
   FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_NONE, 0, ws + L.f2, ws + L.g_f2, ws + L.act1_drop,
                               ws + L.g_act1_drop, w->w2, g->w2, g->b2, T, F, E, ws + L.lin_ws, lin_ws_bytes, FFK_ACC_WEIGHT | FFK_ACC_BIAS));
-  FFK_TRY(ffk_dropout_backward(st, dtype, ws + L.g_act1_drop, ws + L.g_act1, T * F, p, d->seed + 1, 0, 0));
   void const *ffn_in = d->pre_layer_norm ? ws + L.h2 : ws + L.x1;
+  bool const fuse_gelu_bwd = gelu && layer_fusion_enabled() &&
+                             dropout_fusable(dtype, ws + L.g_act1_drop, ws + L.f1, ws + L.g_f1, T * F, 0);
+  if (fuse_gelu_bwd) {
+    FFK_TRY(dropout_backward_gelu_backward(as_stream(st), dtype, ws + L.g_act1_drop, ws + L.f1, ws + L.g_f1,
+                                           T * F, p, d->seed + 1, 0));
+  } else {
+    FFK_TRY(ffk_dropout_backward(st, dtype, ws + L.g_act1_drop, ws + L.g_act1, T * F, p, d->seed + 1, 0, 0));
+  }
   if (gelu) {
-    FFK_TRY(ffk_element_unary_backward(st, dtype, FFK_OP_GELU, 0.0f, ws + L.act1, ws + L.g_act1, ws + L.f1,
-                                       ws + L.g_f1, T * F, 0));
+    if (!fuse_gelu_bwd) {
+      FFK_TRY(ffk_element_unary_backward(st, dtype, FFK_OP_GELU, 0.0f, ws + L.act1, ws + L.g_act1, ws + L.f1,
+                                         ws + L.g_f1, T * F, 0));
+    }
     FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_NONE, 0, ws + L.f1, ws + L.g_f1, ffn_in, ws + L.g_h2,
                                 w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws, lin_ws_bytes, FFK_ACC_WEIGHT | FFK_ACC_BIAS));
   } else {
@@ -194,9 +225,19 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   }
   // ---- gradient reaching x1
   if (d->pre_layer_norm) {
-    FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h2, ws + L.x1, mean(L.mean2), mean(L.rstd2), w->ln2_gamma,
-                                    ws + L.g_x1, g->ln2_gamma, g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
-    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.g_x1, dy, ws + L.g_x1, T * E, T * E, T * E));
+    // g_x1 = LN2_backward(g_h2) + dy
+    int rc = FFK_ERR_UNSUPPORTED;
+    if (layer_fusion_enabled()) {
+      rc = layer_norm_backward_add_residual(as_stream(st), dtype, ws + L.g_h2, ws + L.x1, mean(L.mean2),
+                                            mean(L.rstd2), w->ln2_gamma, dy, ws + L.g_x1, g->ln2_gamma,
+                                            g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes);
+      if (rc != FFK_OK && rc != FFK_ERR_UNSUPPORTED) return rc;
+    }
+    if (rc == FFK_ERR_UNSUPPORTED) {
+      FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h2, ws + L.x1, mean(L.mean2), mean(L.rstd2), w->ln2_gamma,
+                                      ws + L.g_x1, g->ln2_gamma, g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+      FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.g_x1, dy, ws + L.g_x1, T * E, T * E, T * E));
+    }
   } else {
     FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.g_h2, g_sum, ws + L.g_x1, T * E, T * E, T * E));
   }
@@ -208,9 +249,19 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
     FFK_TRY(ffk_mha_backward(st, dtype, &m, ws + L.h1, ws + L.g_h1, ws + L.h1, nullptr, ws + L.h1, nullptr,
                              w->attn_weight, g->attn_weight, ws + L.g_attn, ws + L.mha_reserve,
                              L.ln_ws - L.mha_reserve, 0));
-    FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h1, x, mean(L.mean1), mean(L.rstd1), w->ln1_gamma, dx,
-                                    g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
-    FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, dx, g_attn_res, dx, T * E, T * E, T * E));
+    // dx = LN1_backward(g_h1) + g_x1
+    int rc = FFK_ERR_UNSUPPORTED;
+    if (layer_fusion_enabled()) {
+      rc = layer_norm_backward_add_residual(as_stream(st), dtype, ws + L.g_h1, x, mean(L.mean1), mean(L.rstd1),
+                                            w->ln1_gamma, g_attn_res, dx, g->ln1_gamma, g->ln1_beta, T, E,
+                                            ws + L.ln_ws, ln_ws_bytes);
+      if (rc != FFK_OK && rc != FFK_ERR_UNSUPPORTED) return rc;
+    }
+    if (rc == FFK_ERR_UNSUPPORTED) {
+      FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h1, x, mean(L.mean1), mean(L.rstd1), w->ln1_gamma, dx,
+                                      g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+      FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, dx, g_attn_res, dx, T * E, T * E, T * E));
+    }
   } else {
     FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_x1, ws + L.h1, mean(L.mean1), mean(L.rstd1), w->ln1_gamma,
                                     ws + L.g_attn, g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));

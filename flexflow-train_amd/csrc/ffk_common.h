@@ -175,6 +175,44 @@ __device__ __forceinline__ void unpack_raw(u32x4 r, float (&v)[8], bf16 const *)
   }
 }
 
+// ---- GELU (exact erf form) shared by ElementUnary and the GEMM epilogue ----
+// erf by Abramowitz & Stegun 7.1.26 (|error| <= 1.5e-7), sharing exp(-z^2)
+// with the caller: returns erf(z) given e = exp(-z*z).
+__device__ __forceinline__ float erf_from_exp(float z, float e) {
+  float const az = fabsf(z);
+  float const t = __frcp_rn(1.0f + 0.3275911f * az);
+  float poly = 1.061405429f;
+  poly = poly * t - 1.453152027f;
+  poly = poly * t + 1.421413741f;
+  poly = poly * t - 0.284496736f;
+  poly = poly * t + 0.254829592f;
+  float const r = 1.0f - poly * t * e;
+  return copysignf(r, z);
+}
+// x/2 erfc(-x/sqrt2) = x (1/2 + 1/2 erf(x/sqrt2))
+__device__ __forceinline__ float gelu_forward(float v) {
+  float const z = v * 0.70710678118654752440f;
+  return v * (0.5f + 0.5f * erf_from_exp(z, __expf(-z * z)));
+}
+
+// d/dx [x Phi(x)] = Phi(x) + x phi(x)
+__device__ __forceinline__ float gelu_derivative(float x) {
+  float const z = x * 0.70710678118654752440f;
+  float const e = __expf(-z * z);  // = exp(-x^2 / 2), shared by Phi and phi
+  return 0.5f + 0.5f * erf_from_exp(z, e) + x * 0.39894228040143267794f * e;
+}
+
+// Value a float takes after a round trip through the storage type: what a
+// following op would read had this value been stored in between.
+template <typename T>
+__device__ __forceinline__ float storage_round(float v);
+template <>
+__device__ __forceinline__ float storage_round<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float storage_round<bf16>(float v) {
+  return bf16_bits_to_f32(f32_to_bf16_bits(v));
+}
+
 // ---- wavefront reductions (64 lanes, DPP/shuffle based) -------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -1,0 +1,45 @@
+// Fused passes behind the encoder-layer entry points.  Each one produces
+// exactly the bits the corresponding sequence of separate operator kernels
+// would (intermediate values are rounded to the storage type where the
+// separate ops would have stored them), and saves the intermediate tensor's
+// trip through HBM.  Internal: the C ABI exposes only the separate ops and the
+// layer entry points.
+#pragma once
+#include "ffk_common.h"
+
+namespace ffk {
+
+// True when the operands allow the vector kernels below (whole 16-byte
+// chunks, aligned pointers, offset a multiple of 4).
+bool dropout_fusable(int dtype, void const *x, void const *aux, void const *y,
+                     int64_t n, uint64_t offset);
+
+// y = residual + dropout(x)
+int dropout_add_residual(hipStream_t st, int dtype, void const *x,
+                         void const *residual, void *y, int64_t n, float rate,
+                         uint64_t seed, uint64_t offset);
+
+// dx = dropout_backward(dy) * GELU'(gelu_input)
+int dropout_backward_gelu_backward(hipStream_t st, int dtype, void const *dy,
+                                   void const *gelu_input, void *dx, int64_t n,
+                                   float rate, uint64_t seed, uint64_t offset);
+
+// output = act(pre_activation), pre_activation = input . weight^T + bias, both
+// stored; equals Linear without activation followed by the ElementUnary op.
+int linear_forward_keep_preactivation(hipStream_t st, int dtype, int activation,
+                                      void const *input, void *pre_activation,
+                                      void *output, void const *weight,
+                                      void const *bias, int64_t batch,
+                                      int64_t in_dim, int64_t out_dim);
+
+// dx = residual + LayerNorm_backward(dy) (dgamma/dbeta as the separate op);
+// FFK_ERR_UNSUPPORTED when the row length has no vector kernel.
+int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
+                                     void const *x, float const *mean,
+                                     float const *rstd, void const *gamma,
+                                     void const *residual, void *dx,
+                                     void *dgamma, void *dbeta, int64_t M,
+                                     int64_t N, void *workspace,
+                                     size_t workspace_bytes);
+
+}  // namespace ffk

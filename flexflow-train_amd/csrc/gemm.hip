@@ -13,6 +13,7 @@
 // These replace the cublasGemmEx calls of the reference
 // (lib/kernels/src/cuda/ops/linear_kernels.cu:143,163,249,298,321).
 #include "gemm.h"
+#include "colreduce.h"
 #include <stdlib.h>
 #include <type_traits>
 
@@ -29,7 +30,7 @@ __device__ __forceinline__ float apply_activation(float v, int act) {
     case FFK_ACT_TANH:
       return tanhf(v);
     case FFK_ACT_GELU:
-      return v * 0.5f * erfcf(-v * 0.70710678118654752440f);
+      return gelu_forward(v);
     default:
       return v;
   }
@@ -78,7 +79,7 @@ template <int BM, int BN, int WM, int WN, bool TA, bool TB, bool EDGE>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-    bf16 const *__restrict__ bias, int act, int accumulate) {
+    bf16 const *__restrict__ bias, int act, int accumulate, bf16 *pre_act) {
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int NT = NW * 64;
   constexpr int TM = WM / 32;  // MFMA tiles per wave along M
@@ -278,6 +279,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
         int const m = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (n_ok && (!EDGE || m < M)) {
           float v = acc[i][j][r] + bv;
+          if (pre_act != nullptr) {
+            VecIO<bf16>::store1(pre_act + (int64_t)m * ldc + n, v);
+            v = bf16_bits_to_f32(f32_to_bf16_bits(v));
+          }
           v = apply_activation(v, act);
           bf16 *dst = C + (int64_t)m * ldc + n;
           if (accumulate) {
@@ -316,7 +321,7 @@ template <int BM, int BN, int WM, int WN, int BK, int STAGES, bool TA, bool TB>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-    bf16 const *__restrict__ bias, int act, int accumulate) {
+    bf16 const *__restrict__ bias, int act, int accumulate, bf16 *pre_act) {
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int NT = NW * 64;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -329,7 +334,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   constexpr int RPW = 256 / (BK * 2);      // K-contiguous rows per 256-byte bank window
   constexpr int CS = WN + 8;               // row stride of a wave's staged output tile
   static_assert(A_ELEMS / 8 % NT == 0 && B_ELEMS / 8 % NT == 0, "tile/threads");
-  static_assert((STAGES - 2) * LPT <= 63, "vmcnt range");
+  static_assert((STAGES - 1) * LPT <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
 
@@ -340,53 +345,58 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   tile_coords(blockIdx.x, M / BM, N / BN, tm, tn);
   int const m0 = tm * BM, n0 = tn * BN;
 
-  // Per-lane global offsets of its chunks (constant over k except for k0).
+  // Per-lane offset of its first chunk inside the block's operand panel; the
+  // chunk of load i lies a uniform number of rows further on, and the k-tile
+  // advances a uniform base, so a load address is a scalar base plus one
+  // 32-bit lane offset that never changes.
   // K-contiguous tile [rows][BK]: physical chunk pc of a row holds logical
   // chunk pc ^ ((row / RPW) % CPRK).  Tile lying as [BK][cols]: the 64-byte
   // segment s of row k sits at segment s ^ (k % 4).
-  int64_t goff_a[A_LOADS], goff_b[B_LOADS];
-#pragma unroll
-  for (int i = 0; i < A_LOADS; i++) {
-    int c = (i * NW + wave) * 64 + lane;
+  constexpr int ROWS_PER_LOAD_KC = NT / CPRK;     // rows covered by one load of all threads
+  static_assert((ROWS_PER_LOAD_KC / RPW) % CPRK == 0, "swizzle must repeat per load");
+  static_assert((NT * 8 / BM) % 4 == 0 && (NT * 8 / BN) % 4 == 0, "swizzle must repeat per load");
+  unsigned voff_a, voff_b;
+  {
+    int c = wave * 64 + lane;
     if (!TA) {
       int row = c / CPRK, pc = c % CPRK;
       int lc = pc ^ ((row / RPW) & (CPRK - 1));
-      goff_a[i] = (int64_t)(m0 + row) * lda + lc * 8;
+      voff_a = (unsigned)(row * lda + lc * 8);
     } else {
       constexpr int CPR = BM / 8;
       int krow = c / CPR, pc = c % CPR;
       int lc = ((((pc >> 2) ^ (krow & 3)) << 2) | (pc & 3));
-      goff_a[i] = (int64_t)krow * lda + m0 + lc * 8;
+      voff_a = (unsigned)(krow * lda + lc * 8);
     }
-  }
-#pragma unroll
-  for (int i = 0; i < B_LOADS; i++) {
-    int c = (i * NW + wave) * 64 + lane;
     if (!TBL) {
       int row = c / CPRK, pc = c % CPRK;
       int lc = pc ^ ((row / RPW) & (CPRK - 1));
-      goff_b[i] = (int64_t)(n0 + row) * ldb + lc * 8;
+      voff_b = (unsigned)(row * ldb + lc * 8);
     } else {
       constexpr int CPR = BN / 8;
       int krow = c / CPR, pc = c % CPR;
       int lc = ((((pc >> 2) ^ (krow & 3)) << 2) | (pc & 3));
-      goff_b[i] = (int64_t)krow * ldb + n0 + lc * 8;
+      voff_b = (unsigned)(krow * ldb + lc * 8);
     }
   }
+  int64_t const step_a = TA ? (int64_t)(NT * 8 / BM) * lda : (int64_t)ROWS_PER_LOAD_KC * lda;
+  int64_t const step_b = TBL ? (int64_t)(NT * 8 / BN) * ldb : (int64_t)ROWS_PER_LOAD_KC * ldb;
+  bf16 const *const panel_a = TA ? A + m0 : A + (int64_t)m0 * lda;
+  bf16 const *const panel_b = TBL ? B + n0 : B + (int64_t)n0 * ldb;
 
   auto issue = [&](int kt, int stage) {
     bf16 *sa = smem + stage * STAGE_ELEMS;
     bf16 *sb = sa + A_ELEMS;
-    int64_t const ka = TA ? (int64_t)kt * BK * lda : (int64_t)kt * BK;
-    int64_t const kb = TBL ? (int64_t)kt * BK * ldb : (int64_t)kt * BK;
+    bf16 const *ga = panel_a + (TA ? (int64_t)kt * BK * lda : (int64_t)kt * BK);
+    bf16 const *gb = panel_b + (TBL ? (int64_t)kt * BK * ldb : (int64_t)kt * BK);
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
-      __builtin_amdgcn_global_load_lds((gptr_t)(A + goff_a[i] + ka),
+      __builtin_amdgcn_global_load_lds((gptr_t)(ga + i * step_a + voff_a),
                                        (lptr_t)(sa + (i * NW + wave) * 512), 16, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
-      __builtin_amdgcn_global_load_lds((gptr_t)(B + goff_b[i] + kb),
+      __builtin_amdgcn_global_load_lds((gptr_t)(gb + i * step_b + voff_b),
                                        (lptr_t)(sb + (i * NW + wave) * 512), 16, 0, 0);
     }
   };
@@ -449,9 +459,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
 
   int const KT = K / BK;
   static_assert(KS % 2 == 0, "fragment double buffering assumes an even step count");
-  static_assert(STAGES >= 3, "need a stage in flight besides the two in use");
+  static_assert(STAGES >= 2, "one stage in use, at least one in flight");
 #pragma unroll
-  for (int s = 0; s < STAGES - 1; s++) {
+  for (int s = 0; s < STAGES; s++) {
     if (s < KT) issue(s, s);
   }
   // Fragments are double-buffered in registers: while the MFMAs of one k-step
@@ -470,9 +480,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       bfr[buf][j] = TBL ? frag_tr(sb, BN, tr_tab_b, wn0 + j * 32, kk) : frag_kc(sb, wn0 + j * 32, kk);
     }
   };
-  // Tile 0 must have landed (STAGES-2 younger tiles may still be in flight).
-  if (STAGES - 2 < KT) {
-    wait_vmcnt<(STAGES - 2) * LPT>();
+  // Tile 0 must have landed (STAGES-1 younger tiles may still be in flight).
+  if (STAGES - 1 < KT) {
+    wait_vmcnt<(STAGES - 1) * LPT>();
   } else {
     wait_vmcnt<0>();
   }
@@ -481,7 +491,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   asm volatile("s_barrier" ::: "memory");
   read_frags(0, 0, 0);
   // One k-tile.  STEADY: every condition of the generic body is known true
-  // (next tile exists, a refill is due, STAGES-3 younger tiles in flight), so
+  // (next tile exists, a refill is due, STAGES-2 younger tiles in flight), so
   // the steady-state loop is branch-free.
   auto tile_step = [&](int kt, auto steady_tag) {
     constexpr bool STEADY = decltype(steady_tag)::value;
@@ -499,16 +509,18 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       if (kk + 1 < KS) {
         read_frags(cur ^ 1, stage, kk + 1);
       } else if (STEADY || kt + 1 < KT) {
-        // Last step of the tile: make tile kt+1 visible, refill the stage that
-        // was consumed one iteration ago, and start reading tile kt+1 -- all
-        // under this step's MFMAs, which cover those latencies.
-        if (STEADY || kt + STAGES - 2 < KT) {
-          wait_vmcnt<(STAGES - 3) * LPT>();
+        // Last step of the tile: make tile kt+1 visible, refill this tile's own
+        // stage, and start reading tile kt+1 -- all under this step's MFMAs,
+        // which cover those latencies.  Every wave has its last fragments of
+        // tile kt in registers once its LDS counter drains, so after the
+        // barrier the stage is free.
+        if (STEADY || kt + STAGES - 1 < KT) {
+          wait_vmcnt<(STAGES - 2) * LPT>();
         } else {
           wait_vmcnt<0>();
         }
-        asm volatile("s_barrier" ::: "memory");
-        if (STEADY || kt + STAGES - 1 < KT) issue(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (STEADY || kt + STAGES < KT) issue(kt + STAGES, stage);
         read_frags(cur ^ 1, (kt + 1) % STAGES, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -523,7 +535,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
     }
   };
   int kt = 0;
-  for (; kt + STAGES - 1 < KT; kt++) {
+  for (; kt + STAGES < KT; kt++) {
     tile_step(kt, std::true_type{});
   }
   for (; kt < KT; kt++) {
@@ -534,47 +546,64 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // acc[i][j][r]: output row m = wm0 + 32 i + lane % 32,
   //               column n = wn0 + 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4.
   // Each wave stages its own WM x WN tile and writes it out in 16-byte chunks.
+  // With pre_act set there are two such passes: bias-added values rounded to
+  // the storage type go to pre_act, and the activation is applied to those
+  // rounded values, so C equals what a separate activation op would produce
+  // from the stored pre-activation.
   bf16 *cs = smem + wave * (WM * CS);
+  constexpr int CCH = WM * WN / 8 / 64;  // 16-byte chunks per lane
+  auto emit = [&](bf16 *dst, bool with_act, bool round_first, bool add_old) __attribute__((always_inline)) {
 #pragma unroll
-  for (int i = 0; i < TM; i++) {
-    int const m = i * 32 + (lane & 31);
+    for (int i = 0; i < TM; i++) {
+      int const m = i * 32 + (lane & 31);
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
+      for (int j = 0; j < TN; j++) {
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        int const n = j * 32 + 8 * g + 4 * (lane >> 5);
-        float v[4];
+        for (int g = 0; g < 4; g++) {
+          int const n = j * 32 + 8 * g + 4 * (lane >> 5);
+          float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e];
-        if (bias != nullptr) {
+          for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e];
+          if (bias != nullptr) {
 #pragma unroll
-          for (int e = 0; e < 4; e++) v[e] += VecIO<bf16>::load1(bias + n0 + wn0 + n + e);
+            for (int e = 0; e < 4; e++) v[e] += VecIO<bf16>::load1(bias + n0 + wn0 + n + e);
+          }
+          if (round_first) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = bf16_bits_to_f32(f32_to_bf16_bits(v[e]));
+          }
+          if (with_act && act != FFK_ACT_NONE) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = apply_activation(v[e], act);
+          }
+          if (add_old) {
+            // add the old value in fp32 before the single rounding
+            u32x2 old = *reinterpret_cast<u32x2 const *>(dst + (int64_t)(m0 + wm0 + m) * ldc + n0 + wn0 + n);
+            v[0] += __uint_as_float(old[0] << 16);
+            v[1] += __uint_as_float(old[0] & 0xffff0000u);
+            v[2] += __uint_as_float(old[1] << 16);
+            v[3] += __uint_as_float(old[1] & 0xffff0000u);
+          }
+          u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          *reinterpret_cast<u32x2 *>(cs + m * CS + n) = w;
         }
-        if (act != FFK_ACT_NONE) {
-#pragma unroll
-          for (int e = 0; e < 4; e++) v[e] = apply_activation(v[e], act);
-        }
-        if (accumulate) {
-          // add the old value in fp32 before the single rounding
-          u32x2 old = *reinterpret_cast<u32x2 const *>(C + (int64_t)(m0 + wm0 + m) * ldc + n0 + wn0 + n);
-          v[0] += __uint_as_float(old[0] << 16);
-          v[1] += __uint_as_float(old[0] & 0xffff0000u);
-          v[2] += __uint_as_float(old[1] << 16);
-          v[3] += __uint_as_float(old[1] & 0xffff0000u);
-        }
-        u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        *reinterpret_cast<u32x2 *>(cs + m * CS + n) = w;
       }
     }
-  }
-  __syncthreads();
-  constexpr int CCH = WM * WN / 8 / 64;  // 16-byte chunks per lane
+    __syncthreads();
 #pragma unroll
-  for (int i = 0; i < CCH; i++) {
-    int c = lane + i * 64;
-    int row = c / (WN / 8), ch = c % (WN / 8);
-    u32x4 v = *reinterpret_cast<u32x4 const *>(cs + row * CS + ch * 8);
-    *reinterpret_cast<u32x4 *>(C + (int64_t)(m0 + wm0 + row) * ldc + n0 + wn0 + ch * 8) = v;
+    for (int i = 0; i < CCH; i++) {
+      int c = lane + i * 64;
+      int row = c / (WN / 8), ch = c % (WN / 8);
+      u32x4 v = *reinterpret_cast<u32x4 const *>(cs + row * CS + ch * 8);
+      *reinterpret_cast<u32x4 *>(dst + (int64_t)(m0 + wm0 + row) * ldc + n0 + wn0 + ch * 8) = v;
+    }
+  };
+  if (pre_act != nullptr) {
+    emit(pre_act, false, false, false);
+    __syncthreads();
+    emit(C, true, true, accumulate != 0);
+  } else {
+    emit(C, true, false, accumulate != 0);
   }
 }
 
@@ -604,7 +633,7 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
   int const blocks = (M / BM) * (N / BN);
   kern<<<blocks, NT, Cfg::kLds, st>>>(A, B, C, M, N, K, lda, ldb, ldc,
                                      static_cast<bf16 const *>(ep.bias), ep.activation,
-                                     ep.accumulate);
+                                     ep.accumulate, static_cast<bf16 *>(ep.pre_activation_out));
   return hipGetLastError();
 }
 
@@ -615,7 +644,7 @@ template <bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(
     float const *__restrict__ A, float const *__restrict__ B, float *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-    float const *__restrict__ bias, int act, int accumulate) {
+    float const *__restrict__ bias, int act, int accumulate, float *pre_act) {
   constexpr int BM = 64, BN = 64, BKF = 16, LD = 68;
   __shared__ float As[BKF][LD];  // [k][m]
   __shared__ float Bs[BKF][LD];  // [k][n]
@@ -684,7 +713,9 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
     for (int r = 0; r < 16; r++) {
       int const m = m0 + wm0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
       if (m < M) {
-        float v = apply_activation(acc[r] + bv, act);
+        float v = acc[r] + bv;
+        if (pre_act != nullptr) pre_act[(int64_t)m * ldc + n] = v;
+        v = apply_activation(v, act);
         float *dst = C + (int64_t)m * ldc + n;
         if (accumulate) {
           v += *dst;
@@ -701,7 +732,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 __global__ __launch_bounds__(256) void gemm_bf16_plain_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int ta, int tb,
-    bf16 const *__restrict__ bias, int act, int accumulate) {
+    bf16 const *__restrict__ bias, int act, int accumulate, bf16 *pre_act) {
   int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (int64_t)M * N) return;
   int m = (int)(idx / N), n = (int)(idx % N);
@@ -712,6 +743,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_plain_kernel(
     acc += a * b;
   }
   if (bias != nullptr) acc += VecIO<bf16>::load1(bias + n);
+  if (pre_act != nullptr) {
+    VecIO<bf16>::store1(pre_act + (int64_t)m * ldc + n, acc);
+    acc = bf16_bits_to_f32(f32_to_bf16_bits(acc));
+  }
   acc = apply_activation(acc, act);
   bf16 *dst = C + (int64_t)m * ldc + n;
   if (accumulate) acc += VecIO<bf16>::load1(dst);
@@ -728,10 +763,12 @@ static hipError_t launch_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
   bf16 const *bias = static_cast<bf16 const *>(ep.bias);
   if (edge) {
     gemm_bf16_kernel<BM, BN, WM, WN, TA, TB, true><<<blocks, NT, 0, st>>>(
-        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate);
+        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate,
+        static_cast<bf16 *>(ep.pre_activation_out));
   } else {
     gemm_bf16_kernel<BM, BN, WM, WN, TA, TB, false><<<blocks, NT, 0, st>>>(
-        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate);
+        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate,
+        static_cast<bf16 *>(ep.pre_activation_out));
   }
   return hipGetLastError();
 }
@@ -758,11 +795,12 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
     bool const fits128 = M % 128 == 0 && N % 128 == 0;
     int64_t const t256 = fits256 ? (int64_t)(M / 256) * (N / 256) : 0;
     int64_t const t128 = fits128 ? (int64_t)(M / 128) * (N / 128) : 0;
-    // 256x256 tiles (8 waves of 128x64) halve the L2->LDS traffic per flop and
-    // win whenever they still occupy most CUs; otherwise 128x128 tiles with 8
-    // waves of 64x32 keep two waves per SIMD on every CU.
+    // 256x256x64 tiles (8 waves of 128x64, two 64 KB stages) halve the L2->LDS
+    // traffic per flop and fetch whole 128-byte lines; they win whenever they
+    // still occupy most CUs.  Otherwise 128x128x64 tiles with 8 waves of 64x32
+    // keep two waves per SIMD on every CU.
     if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) {
-      return launch_pipe<256, 256, 128, 64, 32, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+      return launch_pipe<256, 256, 128, 64, 64, 2, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
     if ((variant == 0 && t128 >= kNumCU / 2) || (variant == 128 && fits128)) {
       return launch_pipe<128, 128, 64, 32, 64, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
@@ -803,55 +841,101 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(
   }
 }
 
+// Vectorised first pass: a thread reads 16 bytes (8 bf16 / 4 fp32 columns) of
+// kColsumRowsPerLane rows, all loads independent; 64 threads span the columns,
+// the 4 row lanes of the workgroup meet in LDS.
+constexpr int kColsumRowsPerLane = 8;
+constexpr int kColsumRowsPerBlock = 4 * kColsumRowsPerLane;
+
 template <typename T>
-__global__ __launch_bounds__(256) void colsum_final_kernel(
-    float const *__restrict__ partials, int splits, int N, T *out,
-    int accumulate) {
-  int const n = blockIdx.x * 256 + threadIdx.x;
-  if (n >= N) return;
-  float s = 0.0f;
-  for (int r = 0; r < splits; r++) {
-    s += partials[(int64_t)r * N + n];
+__global__ __launch_bounds__(256) void colsum_partial_vec_kernel(
+    T const *__restrict__ X, int64_t ldx, int M, int N, int rows_per_split,
+    float *__restrict__ partials) {
+  constexpr int V = VecIO<T>::kVec;
+  __shared__ float red[4][64][V + 1];
+  int const cx = threadIdx.x & 63;
+  int const ry = threadIdx.x >> 6;
+  int const n = (blockIdx.x * 64 + cx) * V;
+  int const r0 = blockIdx.y * rows_per_split;
+  int const r1 = min(M, r0 + rows_per_split);
+  float s[V];
+#pragma unroll
+  for (int e = 0; e < V; e++) s[e] = 0.0f;
+  if (n < N) {
+    for (int m0 = r0 + ry * kColsumRowsPerLane; m0 < r1; m0 += kColsumRowsPerBlock) {
+      float v[kColsumRowsPerLane][V];
+#pragma unroll
+      for (int i = 0; i < kColsumRowsPerLane; i++) {
+        int const m = min(m0 + i, r1 - 1);  // clamped rows are masked below
+        VecIO<T>::load_stream(X + (int64_t)m * ldx + n, v[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < kColsumRowsPerLane; i++) {
+        if (m0 + i < r1) {
+#pragma unroll
+          for (int e = 0; e < V; e++) s[e] += v[i][e];
+        }
+      }
+    }
   }
-  if (accumulate) {
-    s += VecIO<T>::load1(out + n);
+#pragma unroll
+  for (int e = 0; e < V; e++) red[ry][cx][e] = s[e];
+  __syncthreads();
+  if (ry == 0 && n < N) {
+#pragma unroll
+    for (int e = 0; e < V; e++) {
+      partials[(int64_t)blockIdx.y * N + n + e] =
+          (red[0][cx][e] + red[1][cx][e]) + (red[2][cx][e] + red[3][cx][e]);
+    }
   }
-  VecIO<T>::store1(out + n, s);
 }
 
 static int colsum_splits(int64_t M) {
-  int64_t s = ceil_div(M, 128);
-  return (int)(s < 1 ? 1 : (s > 64 ? 64 : s));
+  int64_t s = ceil_div(M, kColsumRowsPerBlock);
+  return (int)(s < 1 ? 1 : (s > 256 ? 256 : s));
 }
 
 int64_t colsum_partials_elems(int64_t M, int64_t N) {
   return (int64_t)colsum_splits(M) * N;
 }
 
+template <typename T>
+static int colsum_typed(hipStream_t st, T const *X, int64_t ldx, int64_t M,
+                        int64_t N, T *out, bool accumulate, float *partials) {
+  constexpr int V = VecIO<T>::kVec;
+  int const splits = colsum_splits(M);
+  int rows_per_split = (int)ceil_div(M, splits);
+  bool const vec = (N % V == 0) && (ldx % V == 0) && aligned16(X);
+  if (vec) {
+    // whole row blocks per split so that only the last split has a ragged end
+    rows_per_split = (int)(ceil_div(rows_per_split, kColsumRowsPerBlock) * kColsumRowsPerBlock);
+    int const used = (int)ceil_div(M, rows_per_split);
+    dim3 grid((unsigned)ceil_div(N, 64 * V), (unsigned)used);
+    colsum_partial_vec_kernel<T><<<grid, 256, 0, st>>>(X, ldx, (int)M, (int)N, rows_per_split, partials);
+    FFK_CHECK_LAUNCH();
+    FFK_HIP(colreduce_launch<T>(st, partials, used, (int)N, (int)N, out, nullptr, accumulate));
+    return FFK_OK;
+  }
+  dim3 grid((unsigned)ceil_div(N, 64), (unsigned)splits);
+  colsum_partial_kernel<T><<<grid, 256, 0, st>>>(X, ldx, (int)M, (int)N, rows_per_split, partials);
+  FFK_CHECK_LAUNCH();
+  FFK_HIP(colreduce_launch<T>(st, partials, splits, (int)N, (int)N, out, nullptr, accumulate));
+  return FFK_OK;
+}
+
 int colsum_dispatch(hipStream_t st, int dtype, void const *X, int64_t ldx,
                     int64_t M, int64_t N, void *out, bool accumulate,
                     float *partials) {
   FFK_REQUIRE(partials != nullptr, "colsum: partials scratch is NULL");
-  int const splits = colsum_splits(M);
-  int const rows_per_split = (int)ceil_div(M, splits);
-  dim3 grid((unsigned)ceil_div(N, 64), (unsigned)splits);
   if (dtype == FFK_FLOAT) {
-    colsum_partial_kernel<float><<<grid, 256, 0, st>>>(
-        static_cast<float const *>(X), ldx, (int)M, (int)N, rows_per_split, partials);
-    FFK_CHECK_LAUNCH();
-    colsum_final_kernel<float><<<(unsigned)ceil_div(N, 256), 256, 0, st>>>(
-        partials, splits, (int)N, static_cast<float *>(out), accumulate);
-  } else if (dtype == FFK_BF16) {
-    colsum_partial_kernel<bf16><<<grid, 256, 0, st>>>(
-        static_cast<bf16 const *>(X), ldx, (int)M, (int)N, rows_per_split, partials);
-    FFK_CHECK_LAUNCH();
-    colsum_final_kernel<bf16><<<(unsigned)ceil_div(N, 256), 256, 0, st>>>(
-        partials, splits, (int)N, static_cast<bf16 *>(out), accumulate);
-  } else {
-    return fail(FFK_ERR_UNSUPPORTED, "colsum: dtype %d not supported", dtype);
+    return colsum_typed<float>(st, static_cast<float const *>(X), ldx, M, N,
+                               static_cast<float *>(out), accumulate, partials);
   }
-  FFK_CHECK_LAUNCH();
-  return FFK_OK;
+  if (dtype == FFK_BF16) {
+    return colsum_typed<bf16>(st, static_cast<bf16 const *>(X), ldx, M, N,
+                              static_cast<bf16 *>(out), accumulate, partials);
+  }
+  return fail(FFK_ERR_UNSUPPORTED, "colsum: dtype %d not supported", dtype);
 }
 
 int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
@@ -875,7 +959,7 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
 #define FFK_LAUNCH_F32(TA_, TB_)                                               \
   gemm_f32_kernel<TA_, TB_><<<blocks, 256, 0, st>>>(                           \
       a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, bias, ep.activation,     \
-      ep.accumulate)
+      ep.accumulate, static_cast<float *>(ep.pre_activation_out))
     if (!ta && !tb) FFK_LAUNCH_F32(false, false);
     else if (!ta && tb) FFK_LAUNCH_F32(false, true);
     else if (ta && !tb) FFK_LAUNCH_F32(true, false);
@@ -895,7 +979,8 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
       int64_t total = M * N;
       gemm_bf16_plain_kernel<<<(unsigned)ceil_div(total, 256), 256, 0, st>>>(
           a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ta, tb,
-          static_cast<bf16 const *>(ep.bias), ep.activation, ep.accumulate);
+          static_cast<bf16 const *>(ep.bias), ep.activation, ep.accumulate,
+          static_cast<bf16 *>(ep.pre_activation_out));
       e = hipGetLastError();
     } else if (!ta && !tb) {
       e = pick_bf16<false, false>(st, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ep);

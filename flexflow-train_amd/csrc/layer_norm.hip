@@ -12,6 +12,8 @@
 //           (reference: ComputeInternalGradients + GammaBetaBackward, two more
 //           passes, :115-290,354-410).
 #include "rowwise.h"
+#include "colreduce.h"
+#include "fused_ops.h"
 
 namespace ffk {
 
@@ -128,7 +130,10 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
     T const *__restrict__ dY, T const *__restrict__ X,
     float const *__restrict__ mean, float const *__restrict__ rstd,
     T const *__restrict__ gamma, T *dX, float *__restrict__ partials,
-    int64_t M, int N) {
+    int64_t M, int N, T const *res) {
+  // ACC with res == nullptr: dX += gradient (one rounding).  ACC with res set:
+  // dX = res + gradient rounded to the storage type, i.e. what a separate
+  // element-wise add of res to the stored gradient would give.
   constexpr int V = VecIO<T>::kVec;
   constexpr int RPB = 4 / WPR;
   constexpr int LANES = 64 * WPR;
@@ -220,11 +225,12 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
           float o[V];
           T *dst = dX + row * (int64_t)N + (int64_t)v * V;
           if (ACC) {
-            VecIO<T>::load(dst, o);
+            VecIO<T>::load(res != nullptr ? res + row * (int64_t)N + (int64_t)v * V : dst, o);
           }
 #pragma unroll
           for (int e = 0; e < V; e++) {
             float val = rs * (dy[j][e] * g[j][e] - m1 - x[j][e] * m2);
+            if (ACC && res != nullptr) val = storage_round<T>(val);
             o[e] = ACC ? o[e] + val : val;
           }
           VecIO<T>::store(dst, o);
@@ -273,38 +279,6 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
         }
       }
     }
-  }
-}
-
-// Sums the per-workgroup partials: 32 columns x 8 row groups per workgroup so
-// that even N = 1024 spreads over 32 workgroups and every access is a 128-byte
-// row segment.
-template <typename T>
-__global__ __launch_bounds__(256) void layer_norm_param_grad_final_kernel(
-    float const *__restrict__ partials, int nparts, int N, T *dgamma,
-    T *dbeta) {
-  __shared__ float red[2][8][33];
-  int const cx = threadIdx.x & 31, ry = threadIdx.x >> 5;
-  int const j = blockIdx.x * 32 + cx;
-  float sg = 0.0f, sb = 0.0f;
-  if (j < N) {
-    for (int p = ry; p < nparts; p += 8) {
-      sg += partials[(int64_t)p * 2 * N + j];
-      sb += partials[(int64_t)p * 2 * N + N + j];
-    }
-  }
-  red[0][ry][cx] = sg;
-  red[1][ry][cx] = sb;
-  __syncthreads();
-  if (ry == 0 && j < N) {
-    float tg = 0.0f, tb = 0.0f;
-#pragma unroll
-    for (int r = 0; r < 8; r++) {
-      tg += red[0][r][cx];
-      tb += red[1][r][cx];
-    }
-    if (dgamma != nullptr) VecIO<T>::store1(dgamma + j, tg);
-    if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, tb);
   }
 }
 
@@ -400,16 +374,22 @@ template <typename T>
 static int ln_backward(hipStream_t st, void const *dy, void const *x,
                        float const *mean, float const *rstd, void const *gamma,
                        void *dx, void *dgamma, void *dbeta, int64_t M, int64_t N,
-                       void *workspace, size_t workspace_bytes, bool acc) {
+                       void *workspace, size_t workspace_bytes, bool acc,
+                       void const *residual = nullptr) {
   constexpr int V = VecIO<T>::kVec;
+  T const *RES = static_cast<T const *>(residual);
+  if (RES != nullptr) acc = true;
   T const *DY = static_cast<T const *>(dy);
   T const *X = static_cast<T const *>(x);
   T const *G = static_cast<T const *>(gamma);
   T *DX = static_cast<T *>(dx);
   int ept = 0, wpr = 0;
   bool vec = (N % V == 0) && aligned16(dy) && aligned16(x) &&
-             (dx == nullptr || aligned16(dx)) &&
+             (dx == nullptr || aligned16(dx)) && aligned16(residual) &&
              (gamma == nullptr || aligned16(gamma)) && pick_row_config_small(N / V, ept, wpr);
+  if (!vec && RES != nullptr) {
+    return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: residual form needs the vector kernel");
+  }
   if (vec) {
     int const blocks = ln_bwd_blocks(M, wpr);
     size_t need = (size_t)blocks * 2 * (size_t)N * sizeof(float);
@@ -423,19 +403,18 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
   do {                                                                         \
     if (acc)                                                                   \
       layer_norm_bwd_kernel<T, E, W, true><<<blocks, kRowThreads, 0, st>>>(    \
-          DY, X, mean, rstd, G, DX, partials, M, (int)N);                      \
+          DY, X, mean, rstd, G, DX, partials, M, (int)N, RES);                 \
     else                                                                       \
       layer_norm_bwd_kernel<T, E, W, false><<<blocks, kRowThreads, 0, st>>>(   \
-          DY, X, mean, rstd, G, DX, partials, M, (int)N);                      \
+          DY, X, mean, rstd, G, DX, partials, M, (int)N, nullptr);             \
   } while (0)
     FFK_ROW_DISPATCH_SMALL(ept, wpr, CALL);
 #undef CALL
     FFK_CHECK_LAUNCH();
     if (dgamma != nullptr || dbeta != nullptr) {
-      layer_norm_param_grad_final_kernel<T>
-          <<<(unsigned)ceil_div(N, 32), 256, 0, st>>>(
-              partials, blocks, (int)N, static_cast<T *>(dgamma),
-              static_cast<T *>(dbeta));
+      // partials are [blocks][2][N]: gamma sums in columns [0, N), beta after
+      FFK_HIP(colreduce_launch<T>(st, partials, blocks, (int)(2 * N), (int)N,
+                                  static_cast<T *>(dgamma), static_cast<T *>(dbeta), false));
       FFK_CHECK_LAUNCH();
     }
   } else {
@@ -453,6 +432,25 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
     }
   }
   return FFK_OK;
+}
+
+int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
+                                     void const *x, float const *mean,
+                                     float const *rstd, void const *gamma,
+                                     void const *residual, void *dx,
+                                     void *dgamma, void *dbeta, int64_t M,
+                                     int64_t N, void *workspace,
+                                     size_t workspace_bytes) {
+  FFK_REQUIRE(M > 0 && N > 0 && M < (1ll << 31) && N < (1ll << 31),
+              "layer_norm_backward: bad shape");
+  FFK_REQUIRE(dy && x && mean && rstd && residual && dx, "layer_norm_backward: NULL tensor");
+  if (dtype == FFK_FLOAT)
+    return ln_backward<float>(st, dy, x, mean, rstd, gamma, dx, dgamma, dbeta, M, N,
+                              workspace, workspace_bytes, true, residual);
+  if (dtype == FFK_BF16)
+    return ln_backward<bf16>(st, dy, x, mean, rstd, gamma, dx, dgamma, dbeta, M, N,
+                             workspace, workspace_bytes, true, residual);
+  return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: dtype %d not supported", dtype);
 }
 
 }  // namespace ffk

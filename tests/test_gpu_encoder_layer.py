@@ -80,3 +80,31 @@ def test_encoder_layer_config2_shape_runs_and_is_deterministic(ffk):
     cfg0 = dict(cfg, p=0.0)
     y0, _, _ = run_device(ffk, cfg0, params, x, dy)
     assert not np.array_equal(y0, y1)
+
+
+@pytest.mark.parametrize("shape", ["small", "config2"])
+@pytest.mark.parametrize("pre_ln,gelu", [(True, True), (False, True), (False, False)])
+def test_fused_layer_equals_operator_sequence(ffk, shape, pre_ln, gelu, monkeypatch):
+    """The layer entry points fuse neighbouring ops (GELU into the GEMM
+    epilogue, dropout into the residual add, dropout backward into GELU
+    backward, the residual add into LayerNorm backward).  With
+    FFK_LAYER_UNFUSED=1 the same entry points run one kernel per operator;
+    both must give the same bits."""
+    if shape == "small":
+        cfg = dict(batch=2, seq=64, d_model=128, heads=2, d_ff=256)
+    else:
+        cfg = dict(batch=8, seq=512, d_model=1024, heads=16, d_ff=4096)
+    cfg.update(p=0.1, seed=99, eps=1e-5, scale=0.125, causal=False, pre_ln=pre_ln, gelu=gelu)
+    say("fused vs operator sequence", cfg)
+    g = rng(5)
+    params = make_params(g, cfg, bf16_round)
+    x = bf16_round(g.standard_normal((cfg["batch"], cfg["seq"], cfg["d_model"])))
+    dy = bf16_round(g.standard_normal(x.shape))
+    monkeypatch.setenv("FFK_LAYER_UNFUSED", "1")
+    y_u, dx_u, g_u = run_device(ffk, cfg, params, x, dy)
+    monkeypatch.setenv("FFK_LAYER_UNFUSED", "0")
+    y_f, dx_f, g_f = run_device(ffk, cfg, params, x, dy)
+    assert np.array_equal(y_u, y_f)
+    assert np.array_equal(dx_u, dx_f)
+    for k in g_u:
+        assert np.array_equal(g_u[k], g_f[k]), k
