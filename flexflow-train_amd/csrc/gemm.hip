@@ -314,10 +314,31 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-typedef void const __attribute__((address_space(1))) * gptr_t;
-typedef void __attribute__((address_space(3))) * lptr_t;
+// One direct global->LDS load: lane l's 16 bytes at `g` land at LDS address
+// lds_base + 16 l (M0 carries the wave-uniform base).  Issued as inline
+// assembly on purpose: the compiler then does not know that LDS is being
+// written asynchronously, and therefore does not put a full `vmcnt(0)` wait in
+// front of later LDS reads it cannot prove disjoint (it did so in front of
+// every transposing read, which serialised load and compute).  The kernel
+// orders these loads against its LDS reads itself, with wait_vmcnt and the
+// barrier.  Loads the compiler does know about stay correct: its vmcnt waits
+// count these extra, younger loads too, which only makes them stricter.
+__device__ __forceinline__ void lds_dma16(void const *g, void *lds_base) {
+  // wave-uniform by construction; readfirstlane moves it to a scalar register
+  unsigned const base = __builtin_amdgcn_readfirstlane(
+      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(base), "v"(g)
+               : "memory");  // M0 is not in the clobber list (the compiler rejects
+                             // reserved registers there); nothing else in these
+                             // kernels uses M0 (no GDS, message or relative-move ops)
+}
 
-template <int BM, int BN, int WM, int WN, int BK, int STAGES, bool TA, bool TB>
+// PF = how many k-steps ahead of its use a fragment is read from LDS (PF + 1
+// register buffers).  PF = 1 is what both tile configurations use; PF = 3 was
+// measured on the 128x128 tile (2 MFMAs per k-step per wave) and gained nothing.
+template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, bool TB>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
@@ -391,13 +412,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
     bf16 const *gb = panel_b + (TBL ? (int64_t)kt * BK * ldb : (int64_t)kt * BK);
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
-      __builtin_amdgcn_global_load_lds((gptr_t)(ga + i * step_a + voff_a),
-                                       (lptr_t)(sa + (i * NW + wave) * 512), 16, 0, 0);
+      lds_dma16(ga + i * step_a + voff_a, sa + (i * NW + wave) * 512);
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
-      __builtin_amdgcn_global_load_lds((gptr_t)(gb + i * step_b + voff_b),
-                                       (lptr_t)(sb + (i * NW + wave) * 512), 16, 0, 0);
+      lds_dma16(gb + i * step_b + voff_b, sb + (i * NW + wave) * 512);
     }
   };
 
@@ -458,7 +477,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
   int const KT = K / BK;
-  static_assert(KS % 2 == 0, "fragment double buffering assumes an even step count");
+  constexpr int NB = PF + 1;  // fragment buffers
+  static_assert(KS % NB == 0, "buffer index must not depend on the tile");
   static_assert(STAGES >= 2, "one stage in use, at least one in flight");
 #pragma unroll
   for (int s = 0; s < STAGES; s++) {
@@ -467,7 +487,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // Fragments are double-buffered in registers: while the MFMAs of one k-step
   // run, the LDS reads of the next step (of the next tile, at a tile's last
   // step) are already in flight.
-  bf16x8 af[2][TM], bfr[2][TN];
+  bf16x8 af[NB][TM], bfr[NB][TN];
   auto read_frags = [&](int buf, int stage, int kk) {
     bf16 const *sa = smem + stage * STAGE_ELEMS;
     bf16 const *sb = sa + A_ELEMS;
@@ -489,7 +509,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // Barrier without a memory fence: a fence would wait for every direct load
   // still in flight; the vmcnt waits already cover the tile that is needed.
   asm volatile("s_barrier" ::: "memory");
-  read_frags(0, 0, 0);
+#pragma unroll
+  for (int kk = 0; kk < PF; kk++) read_frags(kk, 0, kk);
   // One k-tile.  STEADY: every condition of the generic body is known true
   // (next tile exists, a refill is due, STAGES-2 younger tiles in flight), so
   // the steady-state loop is branch-free.
@@ -498,30 +519,31 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
     int const stage = kt % STAGES;
 #pragma unroll
     for (int kk = 0; kk < KS; kk++) {
-      int const cur = kk & 1;
+      int const cur = kk % NB;
+      int const nxt = (kk + PF) % NB;  // buffer of the step read now
       // The first MFMA of the step is issued before the prefetch below so that
-      // the wait for this step's fragments is the only LDS wait outstanding at
-      // that point (the hardware counter is in order; a wait placed after the
-      // prefetch would also wait for the prefetched data).
+      // the wait for this step's fragments does not also cover the reads
+      // issued now (the hardware counter is in order).
       __builtin_amdgcn_sched_barrier(0);
       acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0], af[cur][0], acc[0][0], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-      if (kk + 1 < KS) {
-        read_frags(cur ^ 1, stage, kk + 1);
+      if (kk + PF < KS) {
+        read_frags(nxt, stage, kk + PF);
       } else if (STEADY || kt + 1 < KT) {
-        // Last step of the tile: make tile kt+1 visible, refill this tile's own
-        // stage, and start reading tile kt+1 -- all under this step's MFMAs,
-        // which cover those latencies.  Every wave has its last fragments of
-        // tile kt in registers once its LDS counter drains, so after the
-        // barrier the stage is free.
-        if (STEADY || kt + STAGES - 1 < KT) {
-          wait_vmcnt<(STAGES - 2) * LPT>();
-        } else {
-          wait_vmcnt<0>();
+        if (kk + PF == KS) {
+          // First read of tile kt+1: make it visible and refill this tile's own
+          // stage -- under this step's MFMAs, which cover those latencies.
+          // Every wave has all fragments of tile kt in registers once its LDS
+          // counter drains, so after the barrier the stage is free.
+          if (STEADY || kt + STAGES - 1 < KT) {
+            wait_vmcnt<(STAGES - 2) * LPT>();
+          } else {
+            wait_vmcnt<0>();
+          }
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          if (STEADY || kt + STAGES < KT) issue(kt + STAGES, stage);
         }
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        if (STEADY || kt + STAGES < KT) issue(kt + STAGES, stage);
-        read_frags(cur ^ 1, (kt + 1) % STAGES, 0);
+        read_frags(nxt, (kt + 1) % STAGES, kk + PF - KS);
       }
       __builtin_amdgcn_sched_barrier(0);
       // Transposed accumulation: rows of the MFMA result = output columns.
@@ -616,13 +638,13 @@ struct PipeCfg {
   static_assert(kLds <= 160 * 1024, "LDS budget");
 };
 
-template <int BM, int BN, int WM, int WN, int BK, int STAGES, bool TA, bool TB>
+template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, bool TB>
 static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
                               bf16 *C, int M, int N, int K, int64_t lda,
                               int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
   using Cfg = PipeCfg<BM, BN, WM, WN, BK, STAGES>;
   constexpr int NT = Cfg::NW * 64;
-  auto kern = gemm_bf16_pipe_kernel<BM, BN, WM, WN, BK, STAGES, TA, TB>;
+  auto kern = gemm_bf16_pipe_kernel<BM, BN, WM, WN, BK, STAGES, PF, TA, TB>;
   static bool configured = false;  // per template instance
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const *>(kern),
@@ -800,10 +822,10 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
     // still occupy most CUs.  Otherwise 128x128x64 tiles with 8 waves of 64x32
     // keep two waves per SIMD on every CU.
     if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) {
-      return launch_pipe<256, 256, 128, 64, 64, 2, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+      return launch_pipe<256, 256, 128, 64, 64, 2, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
     if ((variant == 0 && t128 >= kNumCU / 2) || (variant == 128 && fits128)) {
-      return launch_pipe<128, 128, 64, 32, 64, 4, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+      return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
   }
   // Largest tile that still gives every CU a workgroup.
