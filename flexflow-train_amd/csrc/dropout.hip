@@ -57,7 +57,9 @@ constexpr int kDropThreads = 256;
 //   kDropAddResidual  y = aux + d            (dropout feeding a residual add)
 //   kDropGeluGrad     y = d * GELU'(aux)     (dropout backward feeding the
 //                                             backward of a GELU whose input was aux)
-enum DropMode { kDropPlain = 0, kDropAddResidual = 1, kDropGeluGrad = 2 };
+//   kDropAfterGelu    y = dropout(GELU(x))   (x is replaced by GELU(x), rounded,
+//                                             before the mask is applied)
+enum DropMode { kDropPlain = 0, kDropAddResidual = 1, kDropGeluGrad = 2, kDropAfterGelu = 3 };
 
 // offset % 4 == 0, 16-byte aligned pointers: each lane owns whole Philox blocks.
 template <typename T, bool ACC, int MODE>
@@ -68,8 +70,12 @@ __global__ __launch_bounds__(kDropThreads) void dropout_vec_kernel(
   int64_t const stride = (int64_t)gridDim.x * kDropThreads;
   for (int64_t i = (int64_t)blockIdx.x * kDropThreads + threadIdx.x; i < nvec; i += stride) {
     float x[V], y[V], aux[V];
-    if (MODE == kDropPlain) {
+    if (MODE == kDropPlain || MODE == kDropAfterGelu) {
       VecIO<T>::load(X + i * V, x);
+      if (MODE == kDropAfterGelu) {
+#pragma unroll
+        for (int e = 0; e < V; e++) x[e] = storage_round<T>(gelu_forward(x[e]));
+      }
     } else {
       VecIO<T>::load_stream(X + i * V, x);
       VecIO<T>::load_stream(AUX + i * V, aux);
@@ -194,11 +200,18 @@ static int dropout_fused(char const *who, int mode, hipStream_t st, int dtype,
   int rc = make_params(who, rate, seed, offset, p);
   if (rc != FFK_OK) return rc;
   if (dtype == FFK_FLOAT) {
+    if (mode == kDropAfterGelu) return dropout_fused_typed<float, kDropAfterGelu>(st, x, aux, y, n, p);
     return mode == kDropAddResidual ? dropout_fused_typed<float, kDropAddResidual>(st, x, aux, y, n, p)
                                     : dropout_fused_typed<float, kDropGeluGrad>(st, x, aux, y, n, p);
   }
+  if (mode == kDropAfterGelu) return dropout_fused_typed<bf16, kDropAfterGelu>(st, x, aux, y, n, p);
   return mode == kDropAddResidual ? dropout_fused_typed<bf16, kDropAddResidual>(st, x, aux, y, n, p)
                                   : dropout_fused_typed<bf16, kDropGeluGrad>(st, x, aux, y, n, p);
+}
+
+int gelu_dropout_forward(hipStream_t st, int dtype, void const *x, void *y,
+                         int64_t n, float rate, uint64_t seed, uint64_t offset) {
+  return dropout_fused("gelu_dropout_forward", kDropAfterGelu, st, dtype, x, nullptr, y, n, rate, seed, offset);
 }
 
 int dropout_add_residual(hipStream_t st, int dtype, void const *x,

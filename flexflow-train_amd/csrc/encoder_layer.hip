@@ -150,16 +150,19 @@ extern "C" int ffk_encoder_layer_forward(ffk_stream_t st, int dtype,
     ffn_in = ws + L.x1;
   }
   // dense(d_ff, activation) -> dropout -> dense(d_model) -> dropout
-  if (gelu && layer_fusion_enabled()) {
-    FFK_TRY(linear_forward_keep_preactivation(as_stream(st), dtype, FFK_ACT_GELU, ffn_in, ws + L.f1,
-                                              ws + L.act1, w->w1, w->b1, T, E, F));
-  } else if (gelu) {
+  if (gelu) {
     FFK_TRY(ffk_linear_forward(st, dtype, FFK_ACT_NONE, ffn_in, ws + L.f1, w->w1, w->b1, T, E, F));
-    FFK_TRY(ffk_element_unary_forward(st, dtype, FFK_OP_GELU, 0.0f, ws + L.f1, ws + L.act1, T * F));
   } else {
     FFK_TRY(ffk_linear_forward(st, dtype, FFK_ACT_RELU, ffn_in, ws + L.act1, w->w1, w->b1, T, E, F));
   }
-  FFK_TRY(ffk_dropout_forward(st, dtype, ws + L.act1, ws + L.act1_drop, T * F, p, d->seed + 1, 0));
+  if (gelu && layer_fusion_enabled() &&
+      dropout_fusable(dtype, ws + L.f1, nullptr, ws + L.act1_drop, T * F, 0)) {
+    // GELU's own output is not needed again: backward reads the pre-activation
+    FFK_TRY(gelu_dropout_forward(as_stream(st), dtype, ws + L.f1, ws + L.act1_drop, T * F, p, d->seed + 1, 0));
+  } else {
+    if (gelu) FFK_TRY(ffk_element_unary_forward(st, dtype, FFK_OP_GELU, 0.0f, ws + L.f1, ws + L.act1, T * F));
+    FFK_TRY(ffk_dropout_forward(st, dtype, ws + L.act1, ws + L.act1_drop, T * F, p, d->seed + 1, 0));
+  }
   FFK_TRY(ffk_linear_forward(st, dtype, FFK_ACT_NONE, ws + L.act1_drop, ws + L.f2, w->w2, w->b2, T, F, E));
   if (d->pre_layer_norm) {
     FFK_TRY(dropout_then_add(st, dtype, ws + L.f2, ws + L.f2_drop, ws + L.x1, y, T * E, p, d->seed + 2));

@@ -24,13 +24,9 @@ int dropout_backward_gelu_backward(hipStream_t st, int dtype, void const *dy,
                                    void const *gelu_input, void *dx, int64_t n,
                                    float rate, uint64_t seed, uint64_t offset);
 
-// output = act(pre_activation), pre_activation = input . weight^T + bias, both
-// stored; equals Linear without activation followed by the ElementUnary op.
-int linear_forward_keep_preactivation(hipStream_t st, int dtype, int activation,
-                                      void const *input, void *pre_activation,
-                                      void *output, void const *weight,
-                                      void const *bias, int64_t batch,
-                                      int64_t in_dim, int64_t out_dim);
+// y = dropout(GELU(x)) with GELU's output rounded to the storage type first
+int gelu_dropout_forward(hipStream_t st, int dtype, void const *x, void *y,
+                         int64_t n, float rate, uint64_t seed, uint64_t offset);
 
 // dx = residual + LayerNorm_backward(dy) (dgamma/dbeta as the separate op);
 // FFK_ERR_UNSUPPORTED when the row length has no vector kernel.

@@ -9,10 +9,6 @@ struct GemmEpilogue {
   void const *bias = nullptr;  // [N] in the GEMM dtype, added to every row
   int activation = FFK_ACT_NONE;
   bool accumulate = false;     // C += result instead of C = result
-  // Optional second output with C's shape and row stride: the bias-added value
-  // before the activation, rounded to the storage type.  When set, the
-  // activation is applied to that rounded value.
-  void *pre_activation_out = nullptr;
 };
 
 // C[M,N] (+)= op(A) . op(B), fp32 accumulation.

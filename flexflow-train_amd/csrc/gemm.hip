@@ -79,7 +79,7 @@ template <int BM, int BN, int WM, int WN, bool TA, bool TB, bool EDGE>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-    bf16 const *__restrict__ bias, int act, int accumulate, bf16 *pre_act) {
+    bf16 const *__restrict__ bias, int act, int accumulate) {
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int NT = NW * 64;
   constexpr int TM = WM / 32;  // MFMA tiles per wave along M
@@ -279,10 +279,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
         int const m = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (n_ok && (!EDGE || m < M)) {
           float v = acc[i][j][r] + bv;
-          if (pre_act != nullptr) {
-            VecIO<bf16>::store1(pre_act + (int64_t)m * ldc + n, v);
-            v = bf16_bits_to_f32(f32_to_bf16_bits(v));
-          }
           v = apply_activation(v, act);
           bf16 *dst = C + (int64_t)m * ldc + n;
           if (accumulate) {
@@ -342,7 +338,7 @@ template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, b
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-    bf16 const *__restrict__ bias, int act, int accumulate, bf16 *pre_act) {
+    bf16 const *__restrict__ bias, int act, int accumulate) {
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int NT = NW * 64;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -568,13 +564,29 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // acc[i][j][r]: output row m = wm0 + 32 i + lane % 32,
   //               column n = wn0 + 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4.
   // Each wave stages its own WM x WN tile and writes it out in 16-byte chunks.
-  // With pre_act set there are two such passes: bias-added values rounded to
-  // the storage type go to pre_act, and the activation is applied to those
-  // rounded values, so C equals what a separate activation op would produce
-  // from the stored pre-activation.
   bf16 *cs = smem + wave * (WM * CS);
   constexpr int CCH = WM * WN / 8 / 64;  // 16-byte chunks per lane
-  auto emit = [&](bf16 *dst, bool with_act, bool round_first, bool add_old) __attribute__((always_inline)) {
+  // The lane's bias values depend on (j, g, lane / 32) only: fetch them once.
+  float bv[TN][4][4];
+#pragma unroll
+  for (int j = 0; j < TN; j++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      u32x2 raw = {0u, 0u};
+      if (bias != nullptr) {
+        raw = *reinterpret_cast<u32x2 const *>(bias + n0 + wn0 + j * 32 + 8 * g + 4 * (lane >> 5));
+      }
+      bv[j][g][0] = __uint_as_float(raw[0] << 16);
+      bv[j][g][1] = __uint_as_float(raw[0] & 0xffff0000u);
+      bv[j][g][2] = __uint_as_float(raw[1] << 16);
+      bv[j][g][3] = __uint_as_float(raw[1] & 0xffff0000u);
+    }
+  // The activation is a compile-time functor here: a per-element switch inside
+  // the unrolled loops made the epilogue several times longer than the GEMM's
+  // own store traffic.
+  auto finish = [&](auto actf) __attribute__((always_inline)) {
+    bf16 *const dst = C;
+    bool const add_old = accumulate != 0;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       int const m = i * 32 + (lane & 31);
@@ -585,19 +597,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
           int const n = j * 32 + 8 * g + 4 * (lane >> 5);
           float v[4];
 #pragma unroll
-          for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e];
-          if (bias != nullptr) {
+          for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + bv[j][g][e];
 #pragma unroll
-            for (int e = 0; e < 4; e++) v[e] += VecIO<bf16>::load1(bias + n0 + wn0 + n + e);
-          }
-          if (round_first) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = bf16_bits_to_f32(f32_to_bf16_bits(v[e]));
-          }
-          if (with_act && act != FFK_ACT_NONE) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = apply_activation(v[e], act);
-          }
+          for (int e = 0; e < 4; e++) v[e] = actf(v[e]);
           if (add_old) {
             // add the old value in fp32 before the single rounding
             u32x2 old = *reinterpret_cast<u32x2 const *>(dst + (int64_t)(m0 + wm0 + m) * ldc + n0 + wn0 + n);
@@ -620,12 +622,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       *reinterpret_cast<u32x4 *>(dst + (int64_t)(m0 + wm0 + row) * ldc + n0 + wn0 + ch * 8) = v;
     }
   };
-  if (pre_act != nullptr) {
-    emit(pre_act, false, false, false);
-    __syncthreads();
-    emit(C, true, true, accumulate != 0);
+  if (act == FFK_ACT_NONE) {
+    finish([](float v) { return v; });
+  } else if (act == FFK_ACT_GELU) {
+    finish([](float v) { return gelu_forward(v); });
+  } else if (act == FFK_ACT_RELU) {
+    finish([](float v) { return v >= 0.0f ? v : 0.0f; });
   } else {
-    emit(C, true, false, accumulate != 0);
+    finish([act](float v) { return apply_activation(v, act); });
   }
 }
 
@@ -655,7 +659,7 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
   int const blocks = (M / BM) * (N / BN);
   kern<<<blocks, NT, Cfg::kLds, st>>>(A, B, C, M, N, K, lda, ldb, ldc,
                                      static_cast<bf16 const *>(ep.bias), ep.activation,
-                                     ep.accumulate, static_cast<bf16 *>(ep.pre_activation_out));
+                                     ep.accumulate);
   return hipGetLastError();
 }
 
@@ -666,7 +670,7 @@ template <bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(
     float const *__restrict__ A, float const *__restrict__ B, float *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-    float const *__restrict__ bias, int act, int accumulate, float *pre_act) {
+    float const *__restrict__ bias, int act, int accumulate) {
   constexpr int BM = 64, BN = 64, BKF = 16, LD = 68;
   __shared__ float As[BKF][LD];  // [k][m]
   __shared__ float Bs[BKF][LD];  // [k][n]
@@ -735,9 +739,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
     for (int r = 0; r < 16; r++) {
       int const m = m0 + wm0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
       if (m < M) {
-        float v = acc[r] + bv;
-        if (pre_act != nullptr) pre_act[(int64_t)m * ldc + n] = v;
-        v = apply_activation(v, act);
+        float v = apply_activation(acc[r] + bv, act);
         float *dst = C + (int64_t)m * ldc + n;
         if (accumulate) {
           v += *dst;
@@ -754,7 +756,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 __global__ __launch_bounds__(256) void gemm_bf16_plain_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int ta, int tb,
-    bf16 const *__restrict__ bias, int act, int accumulate, bf16 *pre_act) {
+    bf16 const *__restrict__ bias, int act, int accumulate) {
   int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (int64_t)M * N) return;
   int m = (int)(idx / N), n = (int)(idx % N);
@@ -765,10 +767,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_plain_kernel(
     acc += a * b;
   }
   if (bias != nullptr) acc += VecIO<bf16>::load1(bias + n);
-  if (pre_act != nullptr) {
-    VecIO<bf16>::store1(pre_act + (int64_t)m * ldc + n, acc);
-    acc = bf16_bits_to_f32(f32_to_bf16_bits(acc));
-  }
   acc = apply_activation(acc, act);
   bf16 *dst = C + (int64_t)m * ldc + n;
   if (accumulate) acc += VecIO<bf16>::load1(dst);
@@ -785,12 +783,10 @@ static hipError_t launch_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
   bf16 const *bias = static_cast<bf16 const *>(ep.bias);
   if (edge) {
     gemm_bf16_kernel<BM, BN, WM, WN, TA, TB, true><<<blocks, NT, 0, st>>>(
-        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate,
-        static_cast<bf16 *>(ep.pre_activation_out));
+        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate);
   } else {
     gemm_bf16_kernel<BM, BN, WM, WN, TA, TB, false><<<blocks, NT, 0, st>>>(
-        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate,
-        static_cast<bf16 *>(ep.pre_activation_out));
+        A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate);
   }
   return hipGetLastError();
 }
@@ -812,7 +808,9 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
                             int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
   bool const c_vec = (ldc % 8 == 0) && aligned16(C);
   int const variant = gemm_variant_override();
-  if (c_vec && K % 64 == 0 && variant != 1) {
+  // the pipelined kernels fetch the bias in 8-byte pieces
+  bool const aux_ok = reinterpret_cast<uintptr_t>(ep.bias) % 8 == 0;
+  if (c_vec && aux_ok && K % 64 == 0 && variant != 1) {
     bool const fits256 = M % 256 == 0 && N % 256 == 0;
     bool const fits128 = M % 128 == 0 && N % 128 == 0;
     int64_t const t256 = fits256 ? (int64_t)(M / 256) * (N / 256) : 0;
@@ -981,7 +979,7 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
 #define FFK_LAUNCH_F32(TA_, TB_)                                               \
   gemm_f32_kernel<TA_, TB_><<<blocks, 256, 0, st>>>(                           \
       a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, bias, ep.activation,     \
-      ep.accumulate, static_cast<float *>(ep.pre_activation_out))
+      ep.accumulate)
     if (!ta && !tb) FFK_LAUNCH_F32(false, false);
     else if (!ta && tb) FFK_LAUNCH_F32(false, true);
     else if (ta && !tb) FFK_LAUNCH_F32(true, false);
@@ -1001,8 +999,7 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
       int64_t total = M * N;
       gemm_bf16_plain_kernel<<<(unsigned)ceil_div(total, 256), 256, 0, st>>>(
           a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ta, tb,
-          static_cast<bf16 const *>(ep.bias), ep.activation, ep.accumulate,
-          static_cast<bf16 *>(ep.pre_activation_out));
+          static_cast<bf16 const *>(ep.bias), ep.activation, ep.accumulate);
       e = hipGetLastError();
     } else if (!ta && !tb) {
       e = pick_bf16<false, false>(st, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ep);

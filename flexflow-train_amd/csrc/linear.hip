@@ -12,7 +12,6 @@
 //           bias_grad (+)= column sums of g (linear_kernels.cu:249-334).
 #include "elementwise.h"
 #include "gemm.h"
-#include "fused_ops.h"
 
 namespace ffk {
 
@@ -55,27 +54,6 @@ static hipError_t act_grad(hipStream_t st, int act, int mode, void const *y,
 }
 
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-
-}  // namespace ffk
-
-namespace ffk {
-
-int linear_forward_keep_preactivation(hipStream_t st, int dtype, int activation,
-                                      void const *input, void *pre_activation,
-                                      void *output, void const *weight,
-                                      void const *bias, int64_t batch,
-                                      int64_t in_dim, int64_t out_dim) {
-  FFK_REQUIRE(dtype == FFK_FLOAT || dtype == FFK_BF16,
-              "linear_forward: dtype %d not supported", dtype);
-  FFK_REQUIRE(batch > 0 && in_dim > 0 && out_dim > 0, "linear_forward: non-positive dimension");
-  FFK_REQUIRE(input && output && weight && pre_activation, "linear_forward: NULL tensor");
-  GemmEpilogue ep;
-  ep.bias = bias;
-  ep.activation = activation;
-  ep.pre_activation_out = pre_activation;
-  return gemm_dispatch(st, dtype, false, true, batch, out_dim, in_dim, input,
-                       in_dim, weight, in_dim, output, out_dim, ep);
-}
 
 }  // namespace ffk
 
