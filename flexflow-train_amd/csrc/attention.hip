@@ -284,23 +284,35 @@ struct AttnBwdParams {
   int causal;
 };
 
-// delta[b,h,q] = sum_d O * dO  (one wave per row)
+// delta[b,h,q] = sum_d O * dO.  D/8 lanes share a row (16 bytes each), so a
+// wave covers 64 / (D/8) rows and every access is a whole 128/256-byte row.
 template <int D>
 __global__ __launch_bounds__(256) void attn_delta_kernel(AttnBwdParams p) {
+  constexpr int LPR = D / 8;        // lanes per row
+  constexpr int RPW = 64 / LPR;     // rows per wave
   int const lane = threadIdx.x & 63;
-  int64_t const row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  int64_t const row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / LPR;
   int64_t const total = (int64_t)p.B * p.H * p.Sq;
-  if (row >= total) return;
-  int const q = (int)(row % p.Sq);
-  int const head = (int)((row / p.Sq) % p.H);
-  int const b = (int)(row / ((int64_t)p.Sq * p.H));
-  int64_t off = (int64_t)b * p.o_bs + (int64_t)q * p.o_ss + (int64_t)head * D;
   float s = 0.0f;
-  for (int d = lane; d < D; d += 64) {
-    s += VecIO<bf16>::load1(p.o + off + d) * VecIO<bf16>::load1(p.d_o + off + d);
+  if (row < total) {
+    // rows are numbered (b, q, h) so that neighbouring rows are neighbours in memory
+    int const head = (int)(row % p.H);
+    int const q = (int)((row / p.H) % p.Sq);
+    int const b = (int)(row / ((int64_t)p.Sq * p.H));
+    int64_t const off = (int64_t)b * p.o_bs + (int64_t)q * p.o_ss + (int64_t)head * D + (lane % LPR) * 8;
+    float o[8], g[8];
+    VecIO<bf16>::load(p.o + off, o);
+    VecIO<bf16>::load(p.d_o + off, g);
+#pragma unroll
+    for (int e = 0; e < 8; e++) s += o[e] * g[e];
+#pragma unroll
+    for (int m = 1; m < LPR; m <<= 1) s += __shfl_xor(s, m, 64);
+    if (lane % LPR == 0) p.delta[((int64_t)b * p.H + head) * p.Sq + q] = s;
+  } else {
+    // keep the shuffles convergent for the tail wave
+#pragma unroll
+    for (int m = 1; m < LPR; m <<= 1) s += __shfl_xor(s, m, 64);
   }
-  s = wave_sum(s);
-  if (lane == 0) p.delta[row] = s;
 }
 
 template <int D>
@@ -697,13 +709,13 @@ extern "C" int ffk_attention_backward(ffk_stream_t stream, int dtype,
   dim3 gkv((unsigned)(ceil_div(p.Skv, 128) * p.H * p.B));
   dim3 gq((unsigned)(ceil_div(p.Sq, 128) * p.H * p.B));
   if (d->head_dim == 64) {
-    attn_delta_kernel<64><<<(unsigned)ceil_div(rows, 4), 256, 0, st>>>(p);
+    attn_delta_kernel<64><<<(unsigned)ceil_div(rows, 4 * 8), 256, 0, st>>>(p);
     FFK_CHECK_LAUNCH();
     attn_bwd_dkdv_kernel<64><<<gkv, 256, 0, st>>>(p);
     FFK_CHECK_LAUNCH();
     attn_bwd_dq_kernel<64><<<gq, 256, 0, st>>>(p);
   } else {
-    attn_delta_kernel<128><<<(unsigned)ceil_div(rows, 4), 256, 0, st>>>(p);
+    attn_delta_kernel<128><<<(unsigned)ceil_div(rows, 4 * 4), 256, 0, st>>>(p);
     FFK_CHECK_LAUNCH();
     attn_bwd_dkdv_kernel<128><<<gkv, 256, 0, st>>>(p);
     FFK_CHECK_LAUNCH();

@@ -9,6 +9,10 @@ struct GemmEpilogue {
   void const *bias = nullptr;  // [N] in the GEMM dtype, added to every row
   int activation = FFK_ACT_NONE;
   bool accumulate = false;     // C += result instead of C = result
+  // Optional fp32 scratch for split-K (used when the output has too few tiles
+  // to occupy the chip); gemm_splitk_workspace_bytes() says how much helps.
+  void *splitk_ws = nullptr;
+  size_t splitk_ws_bytes = 0;
 };
 
 // C[M,N] (+)= op(A) . op(B), fp32 accumulation.
@@ -20,6 +24,10 @@ int gemm_dispatch(hipStream_t stream, int dtype, bool trans_a, bool trans_b,
                   int64_t M, int64_t N, int64_t K, void const *A, int64_t lda,
                   void const *B, int64_t ldb, void *C, int64_t ldc,
                   GemmEpilogue const &ep);
+
+// Scratch bytes with which a bf16 GEMM of this shape would split its reduction
+// (0: it would not).
+size_t gemm_splitk_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K);
 
 // out[N] (+)= sum over the M rows of X[M,N] (ldx row stride); `partials` is
 // fp32 scratch of colsum_partials_elems(M, N) floats.

@@ -338,7 +338,12 @@ template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, b
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-    bf16 const *__restrict__ bias, int act, int accumulate) {
+    bf16 const *__restrict__ bias, int act, int accumulate,
+    float *__restrict__ partial, int k_tiles_per_split) {
+  // partial != nullptr: split-K.  Workgroup (tile, split) reduces k-tiles
+  // [split * k_tiles_per_split, +k_tiles_per_split) and stores its fp32
+  // accumulators to partial[split][M][N]; a second kernel sums the splits and
+  // applies the epilogue.
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int NT = NW * 64;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -359,8 +364,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   int const wm0 = (wave / (BN / WN)) * WM;
   int const wn0 = (wave % (BN / WN)) * WN;
   int tm, tn;
-  tile_coords(blockIdx.x, M / BM, N / BN, tm, tn);
+  int const tiles = (M / BM) * (N / BN);
+  int const split = partial != nullptr ? blockIdx.x / tiles : 0;
+  tile_coords(partial != nullptr ? blockIdx.x % tiles : blockIdx.x, M / BM, N / BN, tm, tn);
   int const m0 = tm * BM, n0 = tn * BN;
+  int const kt0 = split * k_tiles_per_split;  // first k-tile of this workgroup
 
   // Per-lane offset of its first chunk inside the block's operand panel; the
   // chunk of load i lies a uniform number of rows further on, and the k-tile
@@ -404,8 +412,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   auto issue = [&](int kt, int stage) {
     bf16 *sa = smem + stage * STAGE_ELEMS;
     bf16 *sb = sa + A_ELEMS;
-    bf16 const *ga = panel_a + (TA ? (int64_t)kt * BK * lda : (int64_t)kt * BK);
-    bf16 const *gb = panel_b + (TBL ? (int64_t)kt * BK * ldb : (int64_t)kt * BK);
+    bf16 const *ga = panel_a + (TA ? (int64_t)(kt0 + kt) * BK * lda : (int64_t)(kt0 + kt) * BK);
+    bf16 const *gb = panel_b + (TBL ? (int64_t)(kt0 + kt) * BK * ldb : (int64_t)(kt0 + kt) * BK);
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
       lds_dma16(ga + i * step_a + voff_a, sa + (i * NW + wave) * 512);
@@ -472,7 +480,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-  int const KT = K / BK;
+  int const KT = partial != nullptr ? k_tiles_per_split : K / BK;
   constexpr int NB = PF + 1;  // fragment buffers
   static_assert(KS % NB == 0, "buffer index must not depend on the tile");
   static_assert(STAGES >= 2, "one stage in use, at least one in flight");
@@ -622,6 +630,24 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       *reinterpret_cast<u32x4 *>(dst + (int64_t)(m0 + wm0 + row) * ldc + n0 + wn0 + ch * 8) = v;
     }
   };
+  if (partial != nullptr) {
+    // raw accumulators, 16 bytes (4 consecutive columns) per store
+    float *dst = partial + (int64_t)split * M * N;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      int64_t const m = m0 + wm0 + i * 32 + (lane & 31);
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          int const n = n0 + wn0 + j * 32 + 8 * g + 4 * (lane >> 5);
+          f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          *reinterpret_cast<f32x4 *>(dst + m * N + n) = v;
+        }
+      }
+    }
+    return;
+  }
   if (act == FFK_ACT_NONE) {
     finish([](float v) { return v; });
   } else if (act == FFK_ACT_GELU) {
@@ -631,6 +657,38 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   } else {
     finish([act](float v) { return apply_activation(v, act); });
   }
+}
+
+// Second pass of split-K: C = epilogue(sum over splits of partial[s][M][N]).
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(
+    float const *__restrict__ partial, int splits, int M, int N, bf16 *C,
+    int64_t ldc, bf16 const *__restrict__ bias, int act, int accumulate) {
+  int64_t const q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  int64_t const total = (int64_t)M * N;
+  if (q * 4 >= total) return;
+  int64_t const m = (q * 4) / N;
+  int const n = (int)((q * 4) % N);
+  f32x4 s = *reinterpret_cast<f32x4 const *>(partial + q * 4);
+  for (int k = 1; k < splits; k++) {
+    f32x4 v = *reinterpret_cast<f32x4 const *>(partial + k * total + q * 4);
+    s += v;
+  }
+  bf16 *dst = C + m * ldc + n;
+  float v[4] = {s[0], s[1], s[2], s[3]};
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    if (bias != nullptr) v[e] += VecIO<bf16>::load1(bias + n + e);
+    v[e] = apply_activation(v[e], act);
+  }
+  if (accumulate) {
+    u32x2 old = *reinterpret_cast<u32x2 const *>(dst);
+    v[0] += __uint_as_float(old[0] << 16);
+    v[1] += __uint_as_float(old[0] & 0xffff0000u);
+    v[2] += __uint_as_float(old[1] << 16);
+    v[3] += __uint_as_float(old[1] & 0xffff0000u);
+  }
+  u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+  *reinterpret_cast<u32x2 *>(dst) = w;
 }
 
 template <int BM, int BN, int WM, int WN, int BK, int STAGES>
@@ -645,7 +703,8 @@ struct PipeCfg {
 template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, bool TB>
 static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
                               bf16 *C, int M, int N, int K, int64_t lda,
-                              int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
+                              int64_t ldb, int64_t ldc, GemmEpilogue const &ep,
+                              int splits = 1) {
   using Cfg = PipeCfg<BM, BN, WM, WN, BK, STAGES>;
   constexpr int NT = Cfg::NW * 64;
   auto kern = gemm_bf16_pipe_kernel<BM, BN, WM, WN, BK, STAGES, PF, TA, TB>;
@@ -657,9 +716,21 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
     configured = true;
   }
   int const blocks = (M / BM) * (N / BN);
+  if (splits > 1) {
+    float *partial = static_cast<float *>(ep.splitk_ws);
+    kern<<<blocks * splits, NT, Cfg::kLds, st>>>(A, B, C, M, N, K, lda, ldb, ldc, nullptr,
+                                                FFK_ACT_NONE, 0, partial, K / BK / splits);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    int64_t const quads = (int64_t)M * N / 4;
+    splitk_reduce_kernel<<<(unsigned)ceil_div(quads, 256), 256, 0, st>>>(
+        partial, splits, M, N, C, ldc, static_cast<bf16 const *>(ep.bias), ep.activation,
+        ep.accumulate);
+    return hipGetLastError();
+  }
   kern<<<blocks, NT, Cfg::kLds, st>>>(A, B, C, M, N, K, lda, ldb, ldc,
                                      static_cast<bf16 const *>(ep.bias), ep.activation,
-                                     ep.accumulate);
+                                     ep.accumulate, nullptr, 0);
   return hipGetLastError();
 }
 
@@ -794,12 +865,28 @@ static hipError_t launch_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
 // FFK_GEMM_VARIANT=128|256|1 forces a tile configuration (1 = the register-
 // staged kernel); unset or 0 = the heuristic.  For tuning runs only.
 static int gemm_variant_override() {
-  static int v = -1;
-  if (v < 0) {
-    char const *e = getenv("FFK_GEMM_VARIANT");
-    v = e ? atoi(e) : 0;
+  char const *e = getenv("FFK_GEMM_VARIANT");  // read per call: tests toggle it
+  return e ? atoi(e) : 0;
+}
+
+// Number of K splits for an M x N output of 128x128 tiles: enough to give
+// every CU a workgroup, each split at least 8 k-tiles of 64 long, and no more
+// than the caller's scratch (splits * M * N floats) allows.
+static int splitk_splits(int64_t M, int64_t N, int64_t K, size_t ws_bytes) {
+  int64_t const tiles = (M / 128) * (N / 128);
+  if (tiles <= 0 || tiles >= kNumCU / 2 || K % 64 != 0) return 1;
+  int s = 1;
+  while (s * 2 * tiles <= kNumCU && s < 8 && (K / 64) % (s * 2) == 0 && K / (s * 2) >= 512 &&
+         (size_t)(s * 2) * (size_t)(M * N) * sizeof(float) <= ws_bytes) {
+    s *= 2;
   }
-  return v;
+  return s;
+}
+
+size_t gemm_splitk_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K) {
+  if (dtype != FFK_BF16 || M % 128 != 0 || N % 128 != 0) return 0;
+  int const s = splitk_splits(M, N, K, ~(size_t)0);
+  return s > 1 ? (size_t)s * (size_t)(M * N) * sizeof(float) : 0;
 }
 
 template <bool TA, bool TB>
@@ -824,6 +911,11 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
     }
     if ((variant == 0 && t128 >= kNumCU / 2) || (variant == 128 && fits128)) {
       return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+    }
+    // Few output tiles and a long reduction: split K so every CU has a tile.
+    int const splits = fits128 ? splitk_splits(M, N, K, ep.splitk_ws_bytes) : 1;
+    if (variant == 0 && splits > 1 && ep.splitk_ws != nullptr && aligned16(ep.splitk_ws)) {
+      return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep, splits);
     }
   }
   // Largest tile that still gives every CU a workgroup.

@@ -187,8 +187,13 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
                      d->o_proj_size, w + L.wo * es, HD, dctx, HD, over);
   if (rc != FFK_OK) return rc;
   if (dw != nullptr) {
+    // d(QKV projections) is not written before the core's backward: until
+    // then it serves as split-K scratch for this small-output, long-K GEMM.
+    GemmEpilogue acc_o = acc;
+    acc_o.splitk_ws = dqkv;
+    acc_o.splitk_ws_bytes = L.total - L.off_dqkv;
     rc = gemm_dispatch(st, dtype, true, false, d->o_proj_size, HD, L.TQ, output_grad,
-                       d->o_proj_size, ctx, HD, dw + L.wo * es, HD, acc);
+                       d->o_proj_size, ctx, HD, dw + L.wo * es, HD, acc_o);
     if (rc != FFK_OK) return rc;
   }
 

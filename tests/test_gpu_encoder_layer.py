@@ -108,3 +108,27 @@ def test_fused_layer_equals_operator_sequence(ffk, shape, pre_ln, gelu, monkeypa
     assert np.array_equal(dx_u, dx_f)
     for k in g_u:
         assert np.array_equal(g_u[k], g_f[k]), k
+
+
+def test_split_k_weight_gradient_matches_unsplit(ffk, monkeypatch):
+    """At config 2 the attention output projection's weight gradient
+    ([1024 x 1024] output, reduction over 4096 tokens) runs as a split-K GEMM
+    with fp32 partial sums.  FFK_GEMM_VARIANT=128 forces the same tile
+    configuration without the split; the two differ only in fp32 summation
+    order, so the bf16 results agree to a rounding step."""
+    cfg = dict(batch=8, seq=512, d_model=1024, heads=16, d_ff=4096, p=0.1, seed=3, eps=1e-5,
+               scale=0.125, causal=False, pre_ln=True, gelu=True)
+    say("split-K vs unsplit", cfg)
+    g = rng(8)
+    params = make_params(g, cfg, bf16_round)
+    x = bf16_round(g.standard_normal((8, 512, 1024)))
+    dy = bf16_round(g.standard_normal(x.shape))
+    monkeypatch.setenv("FFK_GEMM_VARIANT", "128")
+    _, _, g_plain = run_device(ffk, cfg, params, x, dy)
+    monkeypatch.delenv("FFK_GEMM_VARIANT")
+    _, _, g_split = run_device(ffk, cfg, params, x, dy)
+    E = 1024
+    wo_plain = g_plain["attn_weight"][3 * E * E:]
+    wo_split = g_split["attn_weight"][3 * E * E:]
+    assert np.abs(wo_plain).max() > 0
+    assert_close(wo_split, wo_plain, 1e-2, "dW_O split-K vs unsplit")
