@@ -78,25 +78,39 @@ def step(ffk, st):
     ffk.encoder_layer_backward(st["desc"], st["W"], st["G"], st["x"], st["dy"], st["dx"], st["ws"])
 
 
-def time_dominant_kernel(ffk, torch, cfg, iters=50):
-    """The FFN up-projection GEMM at its real shape, HIP events on the stream
-    the kernel is launched on."""
+# HBM bytes one launch of the dominant kernel moves, from `rocprofv3 --pmc
+# FETCH_SIZE` and `--pmc WRITE_SIZE` runs of `bench.py --roofline-only`, each
+# counter scaled by what it reads for the 256 MiB copy kernel that the same run
+# launches (profiles/ffn_up_gemm_hbm_traffic.md holds the runs and the factors).
+DOMINANT_KERNEL_TRAFFIC_BYTES = 84188160  # 48.3 MiB fetched + 32 MiB written; 48 MiB algorithmic
+
+
+def time_dominant_kernel(ffk, torch, cfg, iters=50, calibration_copy=False):
+    """The FFN up-projection (Linear forward with bias, [4096,1024] x
+    [4096,1024]^T) at its real shape, HIP events on the stream the kernel is
+    launched on.  calibration_copy also launches one element-wise copy of
+    256 MiB (read 256 MiB, write 256 MiB) for scaling HBM traffic counters."""
     import ctypes
     T, E, F = cfg["batch"] * cfg["seq"], cfg["d_model"], cfg["d_ff"]
     bt = torch.bfloat16
     A = torch.randn((T, E), device="cuda").to(bt)
     B = (torch.randn((F, E), device="cuda") * 0.02).to(bt)
+    bias = (torch.randn((F,), device="cuda") * 0.02).to(bt)
     C = torch.empty((T, F), device="cuda", dtype=bt)
+    if calibration_copy:
+        src = torch.randn((128 << 20,), device="cuda").to(bt)  # 256 MiB of bf16
+        dst = torch.empty_like(src)
+        ffk.element_unary_forward(ffk.OP["IDENTITY"], src, out=dst)
     lib = ffk.lib()
     stream = ffk.current_stream()
     e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
     ffk.check(lib.ffk_event_create(ctypes.byref(e0)))
     ffk.check(lib.ffk_event_create(ctypes.byref(e1)))
     for _ in range(5):
-        ffk.gemm(A, B, C, False, True)
+        ffk.linear_forward(A, B, bias, ffk.ACT_NONE, C)
     ffk.check(lib.ffk_event_record(e0, stream))
     for _ in range(iters):
-        ffk.gemm(A, B, C, False, True)
+        ffk.linear_forward(A, B, bias, ffk.ACT_NONE, C)
     ffk.check(lib.ffk_event_record(e1, stream))
     ffk.check(lib.ffk_event_synchronize(e1))
     ms = ctypes.c_float()
@@ -106,8 +120,10 @@ def time_dominant_kernel(ffk, torch, cfg, iters=50):
     sec = ms.value / iters * 1e-3
     flops = 2.0 * T * F * E
     return dict(bound="mfma", achieved=flops / sec / 1e12, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
-                frac=flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS, traffic=None,
-                kernel="gemm_bf16_kernel (FFN up-projection, M%d N%d K%d)" % (T, F, E),
+                frac=flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                traffic=DOMINANT_KERNEL_TRAFFIC_BYTES,
+                kernel="gemm_bf16_pipe_kernel<256,256,128,64,64,2,1,false,true> "
+                       "(FFN up-projection, M%d N%d K%d, bias)" % (T, F, E),
                 us_per_launch=sec * 1e6)
 
 
@@ -138,6 +154,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="run only the dominant kernel's timing loop and a 256 MiB calibration "
+                         "copy (for rocprofv3 counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every kernel here runs on a single MI355X and no "
@@ -147,6 +166,9 @@ def main():
     ffk.lib()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    if args.roofline_only:
+        print(json.dumps({"roofline": time_dominant_kernel(ffk, torch, CFG, calibration_copy=True)}))
+        return
     st = make_device_state(ffk, torch, CFG)
     for _ in range(args.warmup):
         step(ffk, st)
