@@ -359,7 +359,10 @@ def embedding_forward(indices, weight, aggr=AGGR_NONE, out_dtype=None):
     return out
 
 
-def embedding_backward(indices, out_grad, weight_grad, aggr=AGGR_NONE, deterministic=False):
+def embedding_backward(indices, out_grad, weight_grad, aggr=AGGR_NONE, deterministic=False,
+                       workspace=True):
+    """workspace=True allocates the sort scratch (sorted scatter-add);
+    workspace=False passes none (plain atomics, what a caller without scratch gets)."""
     torch = _torch()
     V, D = weight_grad.shape
     if aggr == AGGR_NONE:
@@ -369,9 +372,10 @@ def embedding_backward(indices, out_grad, weight_grad, aggr=AGGR_NONE, determini
         num_bags = indices.numel() // bag
     ws = None
     ws_bytes = 0
-    if deterministic:
+    if workspace or deterministic:
         ws_bytes = lib().ffk_embedding_backward_workspace_bytes(num_bags * bag, V)
-        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=weight_grad.device)
+        if ws_bytes:
+            ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=weight_grad.device)
     check(lib().ffk_embedding_backward(current_stream(), dtype_of(indices), dtype_of(out_grad),
                                        ptr(indices), ptr(out_grad), ptr(weight_grad), aggr,
                                        num_bags, bag, D, V, int(deterministic), ptr(ws),

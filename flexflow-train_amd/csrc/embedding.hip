@@ -11,6 +11,8 @@
 // Indices outside [0, num_entries) are skipped (the reference reads or writes
 // out of bounds for them).
 #include "ffk_common.h"
+#include <cstring>
+#include <rocprim/device/device_radix_sort.hpp>
 
 namespace ffk {
 
@@ -137,6 +139,317 @@ __global__ __launch_bounds__(kEmbThreads) void embedding_bwd_atomic_kernel(
   }
 }
 
+// Sorted scatter-add.  The atomic kernel above is bound by the rate at which
+// the memory side retires fp32 atomics (about 0.7 TB/s of payload measured on
+// MI355X, far below HBM).  With scratch from the caller the lookups are sorted
+// by row id first (stable radix sort of (id, lookup) pairs); equal ids then
+// form runs, a walker sums the gradient rows of a run in registers and adds the
+// sum to the weight-gradient row with ordinary loads and stores, because a run
+// that lies inside one walker's chunk is touched by nobody else.  Only runs
+// that cross a chunk border (at most two per walker) go through atomics.
+constexpr int kEmbChunk = 16;  // sorted positions per walker
+
+template <typename IT>
+__global__ __launch_bounds__(256) void embedding_sort_keys_kernel(
+    IT const *__restrict__ idx, uint32_t *keys, uint32_t *vals, int64_t n,
+    int64_t num_entries) {
+  int64_t const i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  int64_t const r = (int64_t)idx[i];
+  // invalid ids get the key num_entries: they sort behind every valid row
+  keys[i] = (uint64_t)r < (uint64_t)num_entries ? (uint32_t)r : (uint32_t)num_entries;
+  vals[i] = (uint32_t)i;
+}
+
+template <typename GT>
+__device__ __forceinline__ void load_grad4(GT const *p, float (&v)[4]);
+template <>
+__device__ __forceinline__ void load_grad4<float>(float const *p, float (&v)[4]) {
+  f32x4 r = __builtin_nontemporal_load(reinterpret_cast<f32x4 const *>(p));
+  v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+}
+template <>
+__device__ __forceinline__ void load_grad4<bf16>(bf16 const *p, float (&v)[4]) {
+  u32x2 r = __builtin_nontemporal_load(reinterpret_cast<u32x2 const *>(p));
+  v[0] = __uint_as_float(r[0] << 16);
+  v[1] = __uint_as_float(r[0] & 0xffff0000u);
+  v[2] = __uint_as_float(r[1] << 16);
+  v[3] = __uint_as_float(r[1] & 0xffff0000u);
+}
+
+// LPR lanes share a row, 4 columns per lane and CPL such chunks per lane in
+// one pass (columns c = ((k * LPR) + lane) * 4, k < CPL).
+// DET: a walker owns every run that STARTS in its chunk and follows it to its
+// end, however far; no run is shared, nothing is atomic, and every row is
+// summed in ascending lookup order, so the result is bit-reproducible (a very
+// popular row is then summed by a single walker, which is slow).
+template <typename GT, int LPR, int CPL, bool DET>
+__global__ __launch_bounds__(256) void embedding_bwd_sorted_kernel(
+    uint32_t const *__restrict__ keys, uint32_t const *__restrict__ vals,
+    GT const *__restrict__ dY, float *dW, int64_t n, int bag, int64_t dim,
+    uint32_t invalid_key, float scale) {
+  int64_t const walker = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
+  int const wl = threadIdx.x % LPR;
+  int64_t const p0 = walker * kEmbChunk;
+  if (p0 >= n) return;
+  int64_t const p1 = min(p0 + (int64_t)kEmbChunk, n);
+  int64_t start = p0;
+  if (DET) {
+    while (start < p1 && start > 0 && keys[start - 1] == keys[start]) start++;
+    if (start >= p1) return;
+  }
+  // is position p part of this walker's work?
+  auto mine = [&](int64_t p) {
+    return p < p1 || (DET && p < n && keys[p] == keys[p - 1]);
+  };
+  for (int64_t cbase = 0; cbase < dim; cbase += (int64_t)LPR * 4 * CPL) {
+    float acc[CPL][4], cur[CPL][4], nxt[CPL][4];
+    auto fetch = [&](int64_t p, float (&v)[CPL][4]) {
+      int64_t const l = (int64_t)vals[p];
+      GT const *row = dY + (l / bag) * dim;
+#pragma unroll
+      for (int k = 0; k < CPL; k++) {
+        int64_t const c = cbase + ((int64_t)k * LPR + wl) * 4;
+        if (c < dim) {
+          load_grad4<GT>(row + c, v[k]);
+        } else {
+          v[k][0] = v[k][1] = v[k][2] = v[k][3] = 0.0f;
+        }
+      }
+    };
+#pragma unroll
+    for (int k = 0; k < CPL; k++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) acc[k][e] = 0.0f;
+    // a run that began in the previous chunk is shared with that walker
+    bool shared_run = !DET && p0 > 0 && keys[p0 - 1] == keys[p0];
+    fetch(start, cur);
+    for (int64_t p = start; mine(p); p++) {
+      bool const more = mine(p + 1);
+      if (more) fetch(p + 1, nxt);  // next row in flight while this one is added
+      uint32_t const id = keys[p];
+#pragma unroll
+      for (int k = 0; k < CPL; k++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[k][e] += cur[k][e];
+      bool const run_end = !more || keys[p + 1] != id;
+      if (run_end) {
+        if (!DET && !more && p + 1 < n && keys[p + 1] == id) shared_run = true;  // continues next door
+        if (id != invalid_key) {
+#pragma unroll
+          for (int k = 0; k < CPL; k++) {
+            int64_t const c = cbase + ((int64_t)k * LPR + wl) * 4;
+            if (c < dim) {
+              float *dst = dW + (int64_t)id * dim + c;
+              if (shared_run) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) atomicAdd(dst + e, acc[k][e] * scale);
+              } else {
+                f32x4 old = *reinterpret_cast<f32x4 const *>(dst);
+                f32x4 upd = {old[0] + acc[k][0] * scale, old[1] + acc[k][1] * scale,
+                             old[2] + acc[k][2] * scale, old[3] + acc[k][3] * scale};
+                *reinterpret_cast<f32x4 *>(dst) = upd;
+              }
+            }
+          }
+        }
+        shared_run = false;
+#pragma unroll
+        for (int k = 0; k < CPL; k++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) acc[k][e] = 0.0f;
+      }
+#pragma unroll
+      for (int k = 0; k < CPL; k++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) cur[k][e] = nxt[k][e];
+    }
+  }
+}
+
+// The non-deterministic sorted path: a workgroup of 1024 threads owns
+// (1024 / LPR) * kEmbChunk consecutive sorted positions.  Walkers add runs that
+// lie inside their chunk straight to memory; the partial sums of runs that
+// cross a walker border meet in LDS and are merged by the workgroup, so only
+// runs that cross a WORKGROUP border reach memory as atomics.  A row looked up
+// thousands of times (Zipf-distributed tokens) then costs one atomic per
+// element per workgroup instead of one per walker, which matters because
+// atomics to one address are retired one after the other.
+constexpr int kEmbBlockThreads = 1024;
+
+// CPL column chunks of 4 per lane and pass (more bytes in flight per walker
+// step: the walk is latency-bound otherwise).  LDS: 2 * WPB border partials of
+// LPR * 4 * CPL floats, passed as dynamic shared memory.
+template <typename GT, int LPR, int CPL>
+__global__ __launch_bounds__(kEmbBlockThreads) void embedding_bwd_sorted_block_kernel(
+    uint32_t const *__restrict__ keys, uint32_t const *__restrict__ vals,
+    GT const *__restrict__ dY, float *dW, int64_t n, int bag, int64_t dim,
+    uint32_t invalid_key, float scale) {
+  constexpr int WPB = kEmbBlockThreads / LPR;  // walkers per workgroup
+  constexpr int PW = LPR * 4 * CPL;            // columns per pass
+  extern __shared__ __attribute__((aligned(16))) float emb_part[];  // [2 * WPB][PW]
+  __shared__ uint32_t part_id[2 * WPB];
+  __shared__ int part_valid[2 * WPB];
+  int const w = threadIdx.x / LPR, wl = threadIdx.x % LPR;
+  int64_t const block0 = (int64_t)blockIdx.x * WPB * kEmbChunk;
+  int64_t const block1 = min(block0 + (int64_t)WPB * kEmbChunk, n);
+  int64_t const p0 = block0 + (int64_t)w * kEmbChunk;
+  int64_t const p1 = min(p0 + (int64_t)kEmbChunk, n);
+  bool const active = p0 < n;
+  bool const head_shared = active && p0 > 0 && keys[p0 - 1] == keys[p0];
+  auto add_row = [&](uint32_t id, int64_t cbase, float const (&acc)[CPL][4], bool atomic) {
+#pragma unroll
+    for (int k = 0; k < CPL; k++) {
+      int64_t const c = cbase + ((int64_t)k * LPR + wl) * 4;
+      if (c < dim) {
+        float *dst = dW + (int64_t)id * dim + c;
+        if (atomic) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) atomicAdd(dst + e, acc[k][e] * scale);
+        } else {
+          f32x4 old = *reinterpret_cast<f32x4 const *>(dst);
+          f32x4 upd = {old[0] + acc[k][0] * scale, old[1] + acc[k][1] * scale,
+                       old[2] + acc[k][2] * scale, old[3] + acc[k][3] * scale};
+          *reinterpret_cast<f32x4 *>(dst) = upd;
+        }
+      }
+    }
+  };
+  for (int64_t cbase = 0; cbase < dim; cbase += PW) {
+    if (wl == 0) {
+      part_valid[2 * w] = 0;
+      part_valid[2 * w + 1] = 0;
+    }
+    if (active) {
+      float acc[CPL][4], cur[CPL][4], nxt[CPL][4];
+      auto fetch = [&](int64_t p, float (&v)[CPL][4]) {
+        int64_t const l = (int64_t)vals[p];
+        GT const *row = dY + (l / bag) * dim;
+#pragma unroll
+        for (int k = 0; k < CPL; k++) {
+          int64_t const c = cbase + ((int64_t)k * LPR + wl) * 4;
+          if (c < dim) {
+            load_grad4<GT>(row + c, v[k]);
+          } else {
+            v[k][0] = v[k][1] = v[k][2] = v[k][3] = 0.0f;
+          }
+        }
+      };
+#pragma unroll
+      for (int k = 0; k < CPL; k++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[k][e] = 0.0f;
+      bool shared_run = head_shared;
+      fetch(p0, cur);
+      for (int64_t p = p0; p < p1; p++) {
+        bool const more = p + 1 < p1;
+        if (more) fetch(p + 1, nxt);
+        uint32_t const id = keys[p];
+#pragma unroll
+        for (int k = 0; k < CPL; k++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) acc[k][e] += cur[k][e];
+        if (!more || keys[p + 1] != id) {
+          bool const tail_shared = !more && p + 1 < n && keys[p + 1] == id;
+          if (id != invalid_key) {
+            if (shared_run || tail_shared) {
+              // slot 2w: run shared with the previous walker (or both sides);
+              // slot 2w+1: run shared with the next walker only
+              int const slot = shared_run ? 2 * w : 2 * w + 1;
+#pragma unroll
+              for (int k = 0; k < CPL; k++) {
+                f32x4 v = {acc[k][0], acc[k][1], acc[k][2], acc[k][3]};
+                *reinterpret_cast<f32x4 *>(emb_part + slot * PW + (k * LPR + wl) * 4) = v;
+              }
+              if (wl == 0) {
+                part_id[slot] = id;
+                // 1: a border partial; 2 / 4: its run also extends before /
+                // beyond the workgroup's positions
+                part_valid[slot] = 1 | ((shared_run && p0 == block0) ? 2 : 0) |
+                                   ((tail_shared && p1 == block1) ? 4 : 0);
+              }
+            } else {
+              add_row(id, cbase, acc, false);
+            }
+          }
+          shared_run = false;
+#pragma unroll
+          for (int k = 0; k < CPL; k++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[k][e] = 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < CPL; k++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) cur[k][e] = nxt[k][e];
+      }
+    }
+    __syncthreads();
+    // merge the border partials in position order (first LPR threads, their column chunks)
+    if (threadIdx.x < LPR) {
+      float acc[CPL][4];
+#pragma unroll
+      for (int k = 0; k < CPL; k++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[k][e] = 0.0f;
+      uint32_t cur_id = invalid_key;
+      int flags = 0;
+      for (int sidx = 0; sidx < 2 * WPB; sidx++) {
+        int const v = part_valid[sidx];
+        if (v == 0) continue;
+        uint32_t const id = part_id[sidx];
+        if (id != cur_id) {
+          if (cur_id != invalid_key) add_row(cur_id, cbase, acc, (flags & 6) != 0);
+          cur_id = id;
+          flags = 0;
+#pragma unroll
+          for (int k = 0; k < CPL; k++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[k][e] = 0.0f;
+        }
+        flags |= v;
+#pragma unroll
+        for (int k = 0; k < CPL; k++) {
+          f32x4 pv = *reinterpret_cast<f32x4 const *>(emb_part + sidx * PW + (k * LPR + wl) * 4);
+#pragma unroll
+          for (int e = 0; e < 4; e++) acc[k][e] += pv[e];
+        }
+      }
+      if (cur_id != invalid_key) add_row(cur_id, cbase, acc, (flags & 6) != 0);
+    }
+    __syncthreads();
+  }
+}
+
+// Scratch layout: keys in | keys out | lookups in | lookups out | sort scratch
+struct EmbSortLayout {
+  size_t keys_in, keys_out, vals_in, vals_out, temp, temp_bytes, total;
+};
+
+static unsigned key_bits(int64_t num_entries) {
+  unsigned b = 1;
+  while (b < 32 && ((int64_t)1 << b) <= num_entries) b++;
+  return b;
+}
+
+static bool emb_sort_layout(int64_t n, int64_t num_entries, EmbSortLayout &L) {
+  if (n <= 0 || n >= (1ll << 31) || num_entries >= 0xffffffffll) return false;
+  size_t temp = 0;
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, (uint32_t *)nullptr, (uint32_t *)nullptr,
+                                           (uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n, 0u,
+                                           key_bits(num_entries), (hipStream_t)0);
+  if (e != hipSuccess) return false;
+  size_t const arr = ((size_t)n * 4 + 255) & ~(size_t)255;
+  L.keys_in = 0;
+  L.keys_out = arr;
+  L.vals_in = 2 * arr;
+  L.vals_out = 3 * arr;
+  L.temp = 4 * arr;
+  L.temp_bytes = temp;
+  L.total = 4 * arr + ((temp + 255) & ~(size_t)255);
+  return true;
+}
+
 static int emb_grid(int64_t threads_needed) {
   int64_t b = ceil_div(threads_needed > 0 ? threads_needed : 1, kEmbThreads);
   int64_t const cap = (int64_t)kNumCU * 32;
@@ -166,7 +479,59 @@ static int emb_forward(hipStream_t st, void const *indices, void *output,
 template <typename IT, typename GT>
 static int emb_backward(hipStream_t st, void const *indices, void const *dy,
                         float *dw, int64_t num_bags, int64_t bag, int64_t dim,
-                        int64_t num_entries, float scale) {
+                        int64_t num_entries, float scale, void *workspace,
+                        size_t workspace_bytes, bool deterministic) {
+  int64_t const lookups = num_bags * bag;
+  EmbSortLayout L;
+  bool const sorted = workspace != nullptr && dim % 4 == 0 &&
+                      reinterpret_cast<uintptr_t>(dy) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(dw) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(workspace) % 256 == 0 &&
+                      emb_sort_layout(lookups, num_entries, L) && L.total <= workspace_bytes;
+  if (sorted) {
+    uint8_t *ws = static_cast<uint8_t *>(workspace);
+    uint32_t *keys_in = reinterpret_cast<uint32_t *>(ws + L.keys_in);
+    uint32_t *keys_out = reinterpret_cast<uint32_t *>(ws + L.keys_out);
+    uint32_t *vals_in = reinterpret_cast<uint32_t *>(ws + L.vals_in);
+    uint32_t *vals_out = reinterpret_cast<uint32_t *>(ws + L.vals_out);
+    embedding_sort_keys_kernel<IT><<<(unsigned)ceil_div(lookups, 256), 256, 0, st>>>(
+        static_cast<IT const *>(indices), keys_in, vals_in, lookups, num_entries);
+    FFK_CHECK_LAUNCH();
+    size_t temp = L.temp_bytes;
+    FFK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp, keys_in, keys_out, vals_in, vals_out,
+                                      (size_t)lookups, 0u, key_bits(num_entries), st));
+    GT const *G = static_cast<GT const *>(dy);
+    int64_t const walkers = ceil_div(lookups, kEmbChunk);
+#define FFK_EMB_SORTED(LPR_, CPL_)                                             \
+  do {                                                                         \
+    if (deterministic) {                                                       \
+      unsigned const blocks = (unsigned)ceil_div(walkers * LPR_, 256);         \
+      embedding_bwd_sorted_kernel<GT, LPR_, CPL_, true><<<blocks, 256, 0, st>>>( \
+          keys_out, vals_out, G, dw, lookups, (int)bag, dim, (uint32_t)num_entries, scale); \
+    } else {                                                                   \
+      unsigned const blocks = (unsigned)ceil_div(walkers * LPR_, kEmbBlockThreads); \
+      auto kern = embedding_bwd_sorted_block_kernel<GT, LPR_, CPL_>;           \
+      int const lds = 2 * (kEmbBlockThreads / LPR_) * LPR_ * 4 * CPL_ * (int)sizeof(float); \
+      FFK_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(kern),        \
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds)); \
+      kern<<<blocks, kEmbBlockThreads, lds, st>>>(                             \
+          keys_out, vals_out, G, dw, lookups, (int)bag, dim, (uint32_t)num_entries, scale); \
+    }                                                                          \
+  } while (0)
+    if (dim > 512) FFK_EMB_SORTED(64, 4);
+    else if (dim > 256) FFK_EMB_SORTED(64, 2);
+    else if (dim > 128) FFK_EMB_SORTED(64, 1);
+    else if (dim > 64) FFK_EMB_SORTED(32, 1);
+    else FFK_EMB_SORTED(16, 1);
+#undef FFK_EMB_SORTED
+    FFK_CHECK_LAUNCH();
+    return FFK_OK;
+  }
+  if (deterministic) {
+    return fail(FFK_ERR_WORKSPACE,
+                "embedding_backward: deterministic mode needs the sort workspace "
+                "(ffk_embedding_backward_workspace_bytes), 256-byte aligned, and dim %% 4 == 0");
+  }
   int64_t waves = num_bags * ceil_div(dim, 64);
   embedding_bwd_atomic_kernel<IT, GT><<<emb_grid(waves * 64), kEmbThreads, 0, st>>>(
       static_cast<IT const *>(indices), static_cast<GT const *>(dy), dw, num_bags,
@@ -221,9 +586,9 @@ extern "C" int ffk_embedding_forward(ffk_stream_t stream, int index_dtype,
 
 extern "C" size_t ffk_embedding_backward_workspace_bytes(int64_t num_indices,
                                                          int64_t num_entries) {
-  (void)num_entries;
-  // keys + positions, double-buffered, plus per-pass digit histograms
-  return (size_t)num_indices * 16 + ((size_t)1 << 20);
+  EmbSortLayout L;
+  if (!emb_sort_layout(num_indices, num_entries, L)) return 0;
+  return L.total;
 }
 
 extern "C" int ffk_embedding_backward(ffk_stream_t stream, int index_dtype,
@@ -239,15 +604,11 @@ extern "C" int ffk_embedding_backward(ffk_stream_t stream, int index_dtype,
   if (rc != FFK_OK) return rc;
   if (num_bags == 0) return FFK_OK;
   FFK_REQUIRE(indices && output_grad && weight_grad, "embedding_backward: NULL tensor");
-  (void)workspace;
-  (void)workspace_bytes;
-  if (deterministic) {
-    return fail(FFK_ERR_UNSUPPORTED, "embedding_backward: deterministic mode not built yet");
-  }
   float scale = aggr == FFK_AGGR_AVG ? 1.0f / (float)bag : 1.0f;
   hipStream_t st = as_stream(stream);
 #define FFK_EMB_BWD(IT, GT)                                                    \
-  return emb_backward<IT, GT>(st, indices, output_grad, weight_grad, num_bags, bag, dim, num_entries, scale)
+  return emb_backward<IT, GT>(st, indices, output_grad, weight_grad, num_bags, bag, dim, num_entries, scale, \
+                              workspace, workspace_bytes, deterministic != 0)
   if (index_dtype == FFK_INT32) {
     if (output_grad_dtype == FFK_FLOAT) FFK_EMB_BWD(int32_t, float);
     if (output_grad_dtype == FFK_BF16) FFK_EMB_BWD(int32_t, bf16);

@@ -280,10 +280,14 @@ int ffk_dropout_mask(ffk_stream_t stream, uint8_t *mask, int64_t num_elements,
  * forward:  output[b,:] = sum_j weight[indices[b,j],:]
  * backward: weight_grad[indices[b,j],:] += output_grad[b,:] (* 1/bag for AVG),
  *   fp32 accumulators; weight_grad is always accumulated into.
- *   deterministic == 0: hardware fp32 atomics (order varies run to run);
- *   deterministic == 1: rows are summed in ascending position order (bit-
- *   reproducible); needs workspace of
- *   ffk_embedding_backward_workspace_bytes(num_bags*bag, num_entries) bytes. */
+ *   Without workspace: hardware fp32 atomics, one wave instruction per 64
+ *   consecutive floats of a row (order, hence rounding, varies run to run).
+ *   With workspace of ffk_embedding_backward_workspace_bytes(num_bags*bag,
+ *   num_entries) bytes (256-byte aligned) and dim % 4 == 0: lookups are sorted
+ *   by row first and runs of equal rows are summed in registers; only runs
+ *   that straddle two walkers' chunks still use atomics.
+ *   deterministic == 1 (needs the workspace): every row is summed by one
+ *   walker in ascending lookup order, no atomics, bit-reproducible.          */
 /* ------------------------------------------------------------------------ */
 int ffk_embedding_forward(ffk_stream_t stream, int index_dtype,
                           int weight_dtype, int output_dtype,

@@ -98,3 +98,48 @@ def test_out_of_range_ids_are_skipped_and_errors(ffk):
     # empty input is a no-op
     ffk.check(ffk.lib().ffk_embedding_forward(0, ffk.INT64, ffk.FLOAT, ffk.FLOAT, None, None, None,
                                               ffk.AGGR_NONE, 0, 1, 8, 10))
+
+
+@pytest.mark.parametrize("mode", ["atomic", "sorted", "deterministic"])
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V,D,B,bag", [(300, 1024, 5000, 1), (50, 64, 2300, 3), (1000, 100, 700, 4),
+                                       (4000, 192, 2049, 2), (7, 256, 4096, 1), (20, 8, 5, 1)])
+def test_scatter_add_modes(ffk, oracle, mode, idt, gdt, V, D, B, bag):
+    """The three backward paths on the same inputs: plain atomics (no scratch),
+    sorted runs summed in registers (scratch given), and the deterministic
+    variant.  Ragged ends, row widths below and above one wave, heavy
+    duplication (runs far longer than a walker's chunk), ids outside the table."""
+    say("embedding scatter-add", mode, idt, gdt, (V, D, B, bag))
+    g = rng(V + D + B)
+    ids = zipf_ids(g, B * bag, V).reshape(B, bag)
+    bad = g.random(ids.shape) < 0.01
+    ids_dev = np.where(bad, np.where(g.random(ids.shape) < 0.5, -1, V + 5), ids)
+    dy = g.standard_normal((B, D)).astype(np.float32)
+    if gdt == torch.bfloat16:
+        dy = bf16_round(dy)
+    aggr = 0 if bag > 1 else -1
+    # expected: invalid lookups contribute nothing (checked against the oracle
+    # on the all-valid ids, then used with the invalid ones masked out)
+    rows = np.repeat(np.arange(B), bag).reshape(B, bag)
+    all_valid = np.zeros((V, D), dtype=np.float64)
+    np.add.at(all_valid, ids.reshape(-1), dy[rows.reshape(-1)].astype(np.float64))
+    assert_close(all_valid, oracle.embedding_backward(ids, dy, V, aggr=aggr, f64=True), 1e-6,
+                 "test-side expectation vs oracle")
+    want = np.zeros((V, D), dtype=np.float64)
+    ok = ~bad
+    np.add.at(want, ids[ok], dy[rows[ok]].astype(np.float64))
+    kw = dict(atomic=dict(workspace=False), sorted=dict(workspace=True),
+              deterministic=dict(deterministic=True))[mode]
+    dw = torch.zeros((V, D), device="cuda")
+    ffk.embedding_backward(to_dev(ids_dev, torch, idt), to_dev(dy, torch, gdt), dw, aggr=aggr, **kw)
+    assert_close(to_np(dw), want, FP32_RTOL, "dW")
+    if mode == "deterministic":
+        # every row summed in ascending lookup order from zero: the oracle's
+        # fp32 loop does the same additions in the same order -> same bits
+        ids_masked = np.where(bad, V, ids)   # the oracle skips out-of-range ids
+        same = oracle.embedding_backward(ids_masked, dy, V + 1, aggr=aggr)[:V]
+        assert np.array_equal(to_np(dw), same)
+        dw2 = torch.zeros((V, D), device="cuda")
+        ffk.embedding_backward(to_dev(ids_dev, torch, idt), to_dev(dy, torch, gdt), dw2, aggr=aggr, **kw)
+        assert torch.equal(dw, dw2)
