@@ -30,6 +30,16 @@ HIP_FLAGS = [
 ]
 
 
+# Per-file additions.  attention.hip: its backward kernels keep 128-160
+# accumulator registers live across the loop; by default the compiler selects
+# the MFMA form whose accumulators sit in accumulation registers and then
+# copies every accumulator in and out of them around each step (several hundred
+# moves per step).  Forcing the ordinary-register form removes the copies.
+EXTRA_FLAGS = {
+    "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
 def _sources():
     return sorted(
         os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip")
@@ -53,7 +63,7 @@ def _compile_one(src, force):
         and os.path.getmtime(obj) > max(os.path.getmtime(src), _headers_mtime())
     ):
         return obj, ""
-    cmd = [HIPCC] + HIP_FLAGS + ["-c", src, "-o", obj]
+    cmd = [HIPCC] + HIP_FLAGS + EXTRA_FLAGS.get(os.path.basename(src), []) + ["-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     log = "\n".join(
         ln for ln in (proc.stdout + proc.stderr).splitlines()

@@ -1,0 +1,172 @@
+"""Per-kernel measurements at the shapes of the baseline configurations.
+
+    python flexflow-train_amd/kernel_bench.py [group ...]
+
+Groups: gemm (config 2 and config 5 projection GEMMs), bandwidth (config 3:
+LayerNorm, Softmax, ElementBinary, Dropout, plus GELU), embedding (config 4:
+token gather / scatter-add, DLRM bags), attention (config 5 and the config 2
+core).  Every line gives the mean launch time over the timed iterations
+(HIP events on torch's current stream, which is the stream the entry points are
+given) and the ALGORITHMIC bytes or flops of the op divided by that time,
+against 8 TB/s HBM or the 2.5 PFLOP/s dense bf16 MFMA peak.  Inputs are
+synthetic (seeded normal / Zipf) and already resident in HBM.
+"""
+import importlib.util
+import math
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_spec = importlib.util.spec_from_file_location("flexflow_train_amd", os.path.join(HERE, "__init__.py"))
+ffk = importlib.util.module_from_spec(_spec)
+sys.modules["flexflow_train_amd"] = ffk
+_spec.loader.exec_module(ffk)
+BT = torch.bfloat16
+HBM_PEAK = 8e12
+MFMA_PEAK = 2.5e15
+
+
+def timeit(fn, iters=20, warm=5):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    s = torch.cuda.Event(enable_timing=True)
+    e = torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters * 1e-3
+
+
+def report(name, t, bytes_=None, flops=None):
+    msg = "%-46s %9.1f us" % (name, t * 1e6)
+    if bytes_:
+        msg += "  %8.1f GB/s    (%5.1f%% of 8 TB/s)" % (bytes_ / t / 1e9, bytes_ / t / HBM_PEAK * 100)
+    if flops:
+        msg += "  %8.1f TFLOP/s (%5.1f%% of 2.5 PFLOP/s)" % (flops / t / 1e12, flops / t / MFMA_PEAK * 100)
+    print(msg, flush=True)
+
+
+def zipf(n, vocab, s=1.1, seed=0):
+    p = 1.0 / np.arange(1, vocab + 1) ** s
+    cdf = np.cumsum(p / p.sum())
+    return np.minimum(np.searchsorted(cdf, np.random.default_rng(seed).random(n)), vocab - 1)
+
+
+def bench_gemm():
+    # (M, N, K, trans_a, trans_b): forward (NT), input-gradient (NN) and
+    # weight-gradient (TN) GEMMs of the config 2 layer, then config 5's projections
+    shapes = [(4096, 3072, 1024, 0, 1), (4096, 1024, 1024, 0, 1), (4096, 4096, 1024, 0, 1), (4096, 1024, 4096, 0, 1),
+              (4096, 4096, 1024, 0, 0), (4096, 1024, 4096, 0, 0), (4096, 1024, 3072, 0, 0), (4096, 1024, 1024, 0, 0),
+              (1024, 4096, 4096, 1, 0), (4096, 1024, 4096, 1, 0), (3072, 1024, 4096, 1, 0), (1024, 1024, 4096, 1, 0),
+              (16384, 4096, 4096, 0, 1), (16384, 4096, 4096, 0, 0), (4096, 4096, 16384, 1, 0)]
+    for (M, N, K, ta, tb) in shapes:
+        A = torch.randn((K, M) if ta else (M, K), device="cuda").to(BT)
+        B = torch.randn((N, K) if tb else (K, N), device="cuda").to(BT)
+        C = torch.empty((M, N), device="cuda", dtype=BT)
+        t = timeit(lambda: ffk.gemm(A, B, C, bool(ta), bool(tb)))
+        report("gemm bf16 M%d N%d K%d %s%s" % (M, N, K, "T" if ta else "N", "T" if tb else "N"), t,
+               flops=2.0 * M * N * K)
+
+
+def bench_bandwidth():
+    n = 16384 * 4096
+    a = torch.randn(n, device="cuda").to(BT)
+    b = torch.randn(n, device="cuda").to(BT)
+    o = torch.empty_like(a)
+    da, db = torch.zeros_like(a), torch.zeros_like(a)
+    t = timeit(lambda: o.copy_(a))
+    report("device copy (torch) [16384,4096] bf16", t, bytes_=4 * n)
+    t = timeit(lambda: ffk.element_binary_forward(ffk.OP["EW_ADD"], a, b, out=o))
+    report("ElementBinary add fwd", t, bytes_=6 * n)
+    t = timeit(lambda: ffk.element_binary_forward(ffk.OP["EW_MUL"], a, b, out=o))
+    report("ElementBinary mul fwd", t, bytes_=6 * n)
+    t = timeit(lambda: ffk.element_binary_backward(ffk.OP["EW_ADD"], o, a, b, da, db))
+    report("ElementBinary add bwd", t, bytes_=6 * n)
+    t = timeit(lambda: ffk.element_binary_backward(ffk.OP["EW_MUL"], o, a, b, da, db))
+    report("ElementBinary mul bwd", t, bytes_=10 * n)
+    t = timeit(lambda: ffk.element_unary_forward(ffk.OP["GELU"], a, out=o))
+    report("ElementUnary GELU fwd", t, bytes_=4 * n)
+    t = timeit(lambda: ffk.element_unary_backward(ffk.OP["GELU"], o, b, a, da))
+    report("ElementUnary GELU bwd", t, bytes_=6 * n)
+    t = timeit(lambda: ffk.dropout_forward(a, 0.1, 12345, out=o))
+    report("Dropout p=0.1 fwd", t, bytes_=4 * n)
+    t = timeit(lambda: ffk.dropout_backward(a, 0.1, 12345, dx=o))
+    report("Dropout p=0.1 bwd", t, bytes_=4 * n)
+    for (M, N) in [(16384, 4096), (4096, 1024)]:
+        x = torch.randn((M, N), device="cuda").to(BT)
+        dy = torch.randn((M, N), device="cuda").to(BT)
+        g = torch.ones(N, device="cuda", dtype=BT)
+        beta = torch.zeros(N, device="cuda", dtype=BT)
+        y = torch.empty_like(x)
+        mean, rstd = torch.empty(M, device="cuda"), torch.empty(M, device="cuda")
+        dx, dg, dbeta = torch.empty_like(x), torch.empty_like(g), torch.empty_like(beta)
+        ws = torch.empty(ffk.lib().ffk_layer_norm_backward_workspace_bytes(M, N), dtype=torch.uint8, device="cuda")
+        t = timeit(lambda: ffk.layer_norm_forward(x, g, beta, 1e-5, y, mean, rstd))
+        report("LayerNorm fwd [%d,%d]" % (M, N), t, bytes_=4 * M * N)
+        t = timeit(lambda: ffk.layer_norm_backward(dy, x, mean, rstd, g, dx, dg, dbeta, workspace=ws))
+        report("LayerNorm bwd [%d,%d]" % (M, N), t, bytes_=6 * M * N)
+    outer, dim = 128 * 2048, 2048
+    x = (torch.randn((outer, dim), device="cuda") * 4).to(BT)
+    y = torch.empty_like(x)
+    dy = torch.randn((outer, dim), device="cuda").to(BT)
+    dx = torch.empty_like(x)
+    t = timeit(lambda: ffk.softmax_forward(x, outer, dim, 1, out=y), iters=10)
+    report("Softmax fwd [128,2048,2048]", t, bytes_=4 * outer * dim)
+    t = timeit(lambda: ffk.softmax_backward(y, dy, outer, dim, 1, dx=dx), iters=10)
+    report("Softmax bwd [128,2048,2048]", t, bytes_=6 * outer * dim)
+
+
+def bench_embedding():
+    V, D, n = 50257, 1024, 65536
+    w = torch.randn((V, D), device="cuda") * 0.02
+    ids = torch.from_numpy(zipf(n, V)).to(torch.int32).cuda()
+    dy = torch.randn((n, D), device="cuda").to(BT)
+    dw = torch.zeros((V, D), device="cuda")
+    uniq = int(torch.unique(ids).numel())
+    t = timeit(lambda: ffk.embedding_forward(ids, w, out_dtype=BT))
+    report("Embedding gather 65536 ids (fp32 -> bf16)", t, bytes_=n * 4 + uniq * D * 4 + n * D * 2)
+    scatter_bytes = n * 4 + n * D * 2 + uniq * D * 8
+    t = timeit(lambda: ffk.embedding_backward(ids, dy, dw, workspace=True))
+    report("Embedding scatter-add, sorted (with sort)", t, bytes_=scatter_bytes)
+    t = timeit(lambda: ffk.embedding_backward(ids, dy, dw, workspace=False))
+    report("Embedding scatter-add, atomics only", t, bytes_=scatter_bytes)
+    V, D, B, bag = 1000000, 128, 16384, 32
+    w = torch.randn((V, D), device="cuda")
+    ids = torch.from_numpy(zipf(B * bag, V)).to(torch.int64).cuda().view(B, bag)
+    uniq = int(torch.unique(ids).numel())
+    t = timeit(lambda: ffk.embedding_forward(ids, w, aggr=0))
+    report("DLRM bag fwd 1M x 128, 16384 bags of 32", t, bytes_=B * bag * 8 + uniq * D * 4 + B * D * 4)
+    dy = torch.randn((B, D), device="cuda")
+    dw = torch.zeros((V, D), device="cuda")
+    bag_bytes = B * bag * 8 + B * D * 4 + uniq * D * 8
+    t = timeit(lambda: ffk.embedding_backward(ids, dy, dw, aggr=0, workspace=True))
+    report("DLRM bag bwd, sorted (with sort)", t, bytes_=bag_bytes)
+    t = timeit(lambda: ffk.embedding_backward(ids, dy, dw, aggr=0, workspace=False))
+    report("DLRM bag bwd, atomics only", t, bytes_=bag_bytes)
+
+
+def bench_attention():
+    for (B, H, S, D, causal) in [(4, 32, 4096, 128, True), (4, 32, 4096, 128, False), (8, 16, 512, 64, False)]:
+        q, k, v, do = (torch.randn((B, S, H, D), device="cuda").to(BT) for _ in range(4))
+        scale = 1.0 / math.sqrt(D)
+        o, lse = ffk.attention_forward(q, k, v, scale, causal)
+        f = 4.0 * B * H * S * S * D * (0.5 if causal else 1.0)
+        t = timeit(lambda: ffk.attention_forward(q, k, v, scale, causal), iters=10)
+        report("attention fwd B%d H%d S%d D%d causal=%d" % (B, H, S, D, causal), t, flops=f)
+        t = timeit(lambda: ffk.attention_backward(q, k, v, o, do, lse, scale, causal), iters=10)
+        report("attention bwd B%d H%d S%d D%d causal=%d" % (B, H, S, D, causal), t, flops=2.5 * f)
+
+
+GROUPS = dict(gemm=bench_gemm, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention)
+
+if __name__ == "__main__":
+    ffk.lib()
+    assert torch.cuda.is_available(), "kernel_bench.py needs a GPU"
+    for name in sys.argv[1:] or list(GROUPS):
+        GROUPS[name]()
