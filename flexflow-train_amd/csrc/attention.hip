@@ -26,6 +26,7 @@
 // is then loaded with the same permutation of the reduction index, which the
 // transposing load does for free.
 #include "ffk_common.h"
+#include <type_traits>
 
 namespace ffk {
 
@@ -366,49 +367,58 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
   int const q_begin = p.causal ? (kv0 / C::kTile) * C::kTile : 0;
   int const ntiles = (p.Sq - q_begin + C::kTile - 1) / C::kTile;
 
-  u32x4 rq[C::kChunks], rg[C::kChunks];
-  float rl = 0.0f, rd = 0.0f;
-  auto gload = [&](int qt0) {
+  // Tiles travel global -> registers -> LDS.  Two register sets: the loads of
+  // tile it + 2 are issued at the start of step it and stored to LDS at the end
+  // of step it + 1, so a load has two steps to arrive (with one wave per SIMD
+  // nothing else covers the latency; one step was measured not to be enough).
+  // Tile n uses register set n % 2 and LDS buffer n % 2.
+  u32x4 rq[2][C::kChunks], rg[2][C::kChunks];
+  float rl[2] = {0.0f, 0.0f}, rd[2] = {0.0f, 0.0f};
+  auto gload = [&](int qt0, auto set_tag) {
+    constexpr int R = decltype(set_tag)::value;
 #pragma unroll
     for (int i = 0; i < C::kChunks; i++) {
       int c = t + i * 256;
       int row = c / (D / 8), ch = c % (D / 8);
       int gr = min(qt0 + row, p.Sq - 1);
-      rq[i] = *reinterpret_cast<u32x4 const *>(qp + (int64_t)gr * p.q_ss + ch * 8);
-      rg[i] = *reinterpret_cast<u32x4 const *>(gp + (int64_t)gr * p.o_ss + ch * 8);
+      rq[R][i] = *reinterpret_cast<u32x4 const *>(qp + (int64_t)gr * p.q_ss + ch * 8);
+      rg[R][i] = *reinterpret_cast<u32x4 const *>(gp + (int64_t)gr * p.o_ss + ch * 8);
     }
     if (t < C::kTile) {
       int gr = min(qt0 + t, p.Sq - 1);
-      rl = lsep[gr] * kLog2e;
-      rd = delp[gr];
+      rl[R] = lsep[gr] * kLog2e;
+      rd[R] = delp[gr];
     }
   };
-  auto lstore = [&](int buf) {
+  auto lstore = [&](auto set_tag) {
+    constexpr int R = decltype(set_tag)::value;
 #pragma unroll
     for (int i = 0; i < C::kChunks; i++) {
       int c = t + i * 256;
       int row = c / (D / 8), ch = c % (D / 8);
-      *reinterpret_cast<u32x4 *>(&Qs[buf][row * C::kStride + ch * 8]) = rq[i];
-      *reinterpret_cast<u32x4 *>(&Gs[buf][row * C::kStride + ch * 8]) = rg[i];
+      *reinterpret_cast<u32x4 *>(&Qs[R][row * C::kStride + ch * 8]) = rq[R][i];
+      *reinterpret_cast<u32x4 *>(&Gs[R][row * C::kStride + ch * 8]) = rg[R][i];
     }
     if (t < C::kTile) {
-      Ls[buf][t] = rl;
-      Ds[buf][t] = rd;
+      Ls[R][t] = rl[R];
+      Ds[R][t] = rd[R];
     }
   };
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
 
   int const koff = lane_k_off(C::kStride, lane);
   int const toff = lane_tr_off(C::kStride, lane);
   if (ntiles > 0) {
-    gload(q_begin);
-    lstore(0);
+    gload(q_begin, Set0{});
+    lstore(Set0{});
   }
+  if (ntiles > 1) gload(q_begin + C::kTile, Set1{});
   __syncthreads();
-  int cur = 0;
-  for (int it = 0; it < ntiles; it++) {
+  auto step = [&](int it, auto parity) {
+    constexpr int cur = decltype(parity)::value;  // == it % 2
     int const qt0 = q_begin + it * C::kTile;
-    bool const more = it + 1 < ntiles;
-    if (more) gload(qt0 + C::kTile);
+    if (it + 2 < ntiles) gload(qt0 + 2 * C::kTile, parity);
     // A wave whose keys all lie after this query tile (causal) contributes 0.
     bool const active = !p.causal || kv0 + wave * 32 <= qt0 + C::kTile - 1;
     if (active) {
@@ -463,9 +473,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
         }
       }
     }
-    if (more) lstore(cur ^ 1);
+    if (it + 1 < ntiles) lstore(std::integral_constant<int, cur ^ 1>{});
     __syncthreads();
-    cur ^= 1;
+  };
+  for (int it = 0; it < ntiles; it += 2) {
+    step(it, Set0{});
+    if (it + 1 < ntiles) step(it + 1, Set1{});
   }
 
   // dK / dV accumulators: row = key (32 per wave, 8*(r/4)+4*h+r%4), column = d.
@@ -525,37 +538,42 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
   if (p.causal) kv_end = min(p.Skv, q0 + C::kBlk);
   int const ntiles = (kv_end + C::kTile - 1) / C::kTile;
 
-  u32x4 rk[C::kChunks], rv[C::kChunks];
-  auto gload = [&](int kt0) {
+  // Two register sets, loads two steps ahead of their use (see the dK/dV kernel).
+  u32x4 rk[2][C::kChunks], rv[2][C::kChunks];
+  auto gload = [&](int kt0, auto set_tag) {
+    constexpr int R = decltype(set_tag)::value;
 #pragma unroll
     for (int i = 0; i < C::kChunks; i++) {
       int c = t + i * 256;
       int row = c / (D / 8), ch = c % (D / 8);
       int gr = min(kt0 + row, p.Skv - 1);
-      rk[i] = *reinterpret_cast<u32x4 const *>(kp + (int64_t)gr * p.k_ss + ch * 8);
-      rv[i] = *reinterpret_cast<u32x4 const *>(vp + (int64_t)gr * p.v_ss + ch * 8);
+      rk[R][i] = *reinterpret_cast<u32x4 const *>(kp + (int64_t)gr * p.k_ss + ch * 8);
+      rv[R][i] = *reinterpret_cast<u32x4 const *>(vp + (int64_t)gr * p.v_ss + ch * 8);
     }
   };
-  auto lstore = [&](int buf) {
+  auto lstore = [&](auto set_tag) {
+    constexpr int R = decltype(set_tag)::value;
 #pragma unroll
     for (int i = 0; i < C::kChunks; i++) {
       int c = t + i * 256;
       int row = c / (D / 8), ch = c % (D / 8);
-      *reinterpret_cast<u32x4 *>(&Ks[buf][row * C::kStride + ch * 8]) = rk[i];
-      *reinterpret_cast<u32x4 *>(&Vs[buf][row * C::kStride + ch * 8]) = rv[i];
+      *reinterpret_cast<u32x4 *>(&Ks[R][row * C::kStride + ch * 8]) = rk[R][i];
+      *reinterpret_cast<u32x4 *>(&Vs[R][row * C::kStride + ch * 8]) = rv[R][i];
     }
   };
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
 
   int const koff = lane_k_off(C::kStride, lane);
   int const toff = lane_tr_off(C::kStride, lane);
-  gload(0);
-  lstore(0);
+  gload(0, Set0{});
+  lstore(Set0{});
+  if (ntiles > 1) gload(C::kTile, Set1{});
   __syncthreads();
-  int cur = 0;
-  for (int it = 0; it < ntiles; it++) {
+  auto step = [&](int it, auto parity) {
+    constexpr int cur = decltype(parity)::value;  // == it % 2
     int const kt0 = it * C::kTile;
-    bool const more = it + 1 < ntiles;
-    if (more) gload(kt0 + C::kTile);
+    if (it + 2 < ntiles) gload(kt0 + 2 * C::kTile, parity);
     bool const active = !p.causal || kt0 <= q0 + wave * 32 + 31;
     if (active) {
       bf16 const *kk_ = Ks[cur] + koff, *vk_ = Vs[cur] + koff, *ktr = Ks[cur] + toff;
@@ -596,9 +614,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
         }
       }
     }
-    if (more) lstore(cur ^ 1);
+    if (it + 1 < ntiles) lstore(std::integral_constant<int, cur ^ 1>{});
     __syncthreads();
-    cur ^= 1;
+  };
+  for (int it = 0; it < ntiles; it += 2) {
+    step(it, Set0{});
+    if (it + 1 < ntiles) step(it + 1, Set1{});
   }
 
   if (qrow < p.Sq) {
