@@ -117,6 +117,16 @@ SIGNATURES = {
     "ffk_dropout_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
     "ffk_dropout_backward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64, c_int]),
     "ffk_dropout_mask": (c_int, [c_p, c_p, c_i64, c_f, c_u64, c_u64]),
+    "ffk_sgd_update": (c_int, [c_p, c_int, c_f, c_f, c_int, c_f, c_p, c_i64, c_int, c_p, c_p, c_p]),
+    "ffk_adam_update": (c_int, [c_p, c_int, c_f, c_f, c_f, c_f, c_f, c_p, c_i64, c_int, c_p, c_p,
+                                c_p, c_p]),
+    "ffk_sparse_categorical_crossentropy_loss_backward": (
+        c_int, [c_p, c_p, c_p, c_p, c_i64, c_i64, c_int, c_int, c_int, c_f]),
+    "ffk_categorical_crossentropy_loss_backward": (c_int, [c_p, c_p, c_p, c_p, c_i64, c_i64, c_f]),
+    "ffk_mean_squared_error_avg_loss_backward": (c_int, [c_p, c_p, c_p, c_p, c_i64, c_i64, c_f]),
+    "ffk_identity_loss_backward": (c_int, [c_p, c_p, c_p, c_i64, c_i64, c_f]),
+    "ffk_cast_forward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_i64]),
+    "ffk_cast_backward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_i64]),
     "ffk_embedding_forward": (c_int, [c_p, c_int, c_int, c_int, c_p, c_p, c_p, c_int, c_i64,
                                       c_i64, c_i64, c_i64]),
     "ffk_embedding_backward_workspace_bytes": (c_sz, [c_i64, c_i64]),
@@ -341,6 +351,68 @@ def dropout_mask(n, rate, seed, offset=0, device="cuda"):
     m = torch.empty((n,), dtype=torch.uint8, device=device)
     check(lib().ffk_dropout_mask(current_stream(), ptr(m), n, rate, seed, offset))
     return m
+
+
+def sgd_update(weight, grad, lr, momentum=0.0, nesterov=False, weight_decay=0.0, sgd_v=None,
+               num_replicas=1, weight_lowp=None):
+    """In-place SGD step on fp32 `weight` (and `sgd_v`); grad is [num_replicas * n] fp32 or bf16."""
+    n = weight.numel()
+    check(lib().ffk_sgd_update(current_stream(), dtype_of(grad), lr, momentum, int(nesterov),
+                               weight_decay, ptr(grad), n, num_replicas, ptr(weight), ptr(sgd_v),
+                               ptr(weight_lowp)))
+    return weight
+
+
+def adam_update(weight, grad, adam_m, adam_v, alpha_t, beta1=0.9, beta2=0.999, weight_decay=0.0,
+                epsilon=1e-8, num_replicas=1, weight_lowp=None):
+    n = weight.numel()
+    check(lib().ffk_adam_update(current_stream(), dtype_of(grad), alpha_t, beta1, beta2, weight_decay,
+                                epsilon, ptr(grad), n, num_replicas, ptr(weight), ptr(adam_v),
+                                ptr(adam_m), ptr(weight_lowp)))
+    return weight
+
+
+def sparse_categorical_crossentropy_loss_backward(logit, label, num_samples, num_classes, k,
+                                                  scale_factor, out=None):
+    torch = _torch()
+    if out is None:
+        out = torch.empty_like(logit)
+    check(lib().ffk_sparse_categorical_crossentropy_loss_backward(
+        current_stream(), ptr(out), ptr(logit), ptr(label), logit.numel(), out.numel(), num_samples,
+        num_classes, k, scale_factor))
+    return out
+
+
+def difference_loss_backward(kind, logit, label, scale_factor, out=None):
+    """kind: 'categorical_crossentropy' or 'mean_squared_error_avg'."""
+    torch = _torch()
+    if out is None:
+        out = torch.empty_like(logit)
+    fn = getattr(lib(), "ffk_%s_loss_backward" % kind)
+    check(fn(current_stream(), ptr(out), ptr(logit), ptr(label), logit.numel(), out.numel(),
+             scale_factor))
+    return out
+
+
+def identity_loss_backward(loss, scale_factor, out=None):
+    torch = _torch()
+    if out is None:
+        out = torch.empty_like(loss)
+    check(lib().ffk_identity_loss_backward(current_stream(), ptr(out), ptr(loss), loss.numel(),
+                                           out.numel(), scale_factor))
+    return out
+
+
+def cast_forward(x, out):
+    check(lib().ffk_cast_forward(current_stream(), dtype_of(x), dtype_of(out), ptr(x), ptr(out),
+                                 x.numel()))
+    return out
+
+
+def cast_backward(out_grad, in_grad):
+    check(lib().ffk_cast_backward(current_stream(), dtype_of(out_grad), dtype_of(in_grad),
+                                  ptr(out_grad), ptr(in_grad), out_grad.numel()))
+    return in_grad
 
 
 def embedding_forward(indices, weight, aggr=AGGR_NONE, out_dtype=None):

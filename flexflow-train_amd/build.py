@@ -35,8 +35,13 @@ HIP_FLAGS = [
 # the MFMA form whose accumulators sit in accumulation registers and then
 # copies every accumulator in and out of them around each step (several hundred
 # moves per step).  Forcing the ordinary-register form removes the copies.
+# optimizer.hip, loss.hip: these kernels promise the bits of the reference's CPU
+# evaluation, where every fp32 operation is rounded on its own; the device
+# compiler's default contracts a * b + c into one fused operation.
 EXTRA_FLAGS = {
     "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "optimizer.hip": ["-ffp-contract=off"],
+    "loss.hip": ["-ffp-contract=off"],
 }
 
 

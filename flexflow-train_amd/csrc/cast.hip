@@ -1,0 +1,134 @@
+// Cast forward/backward for gfx950 (reference: lib/kernels/src/cuda/ops/
+// cast_kernels.cu:25-37, CPU lib/kernels/src/kernels/cast_kernels_cpu.cc).
+//   forward : output[i] = (ODT) input[i]
+//   backward: input_grad[i] = (ODT) output_grad[i] + 1 * input_grad[i]
+// Any pair of {bool, int32, int64, half, float, double, bf16}; conversions follow
+// C++ static_cast except float -> bf16/half, which round to nearest even.
+#include "ffk_common.h"
+
+namespace ffk {
+
+constexpr int kCastThreads = 256;
+
+template <typename T> struct IsBf16 { static constexpr bool value = false; };
+template <> struct IsBf16<bf16> { static constexpr bool value = true; };
+template <typename T> struct IsBool { static constexpr bool value = false; };
+template <> struct IsBool<bool> { static constexpr bool value = true; };
+template <typename T> struct IsHalf { static constexpr bool value = false; };
+template <> struct IsHalf<_Float16> { static constexpr bool value = true; };
+
+// static_cast<ODT>(x) with bf16 handled through its fp32 value (round to
+// nearest even on the way in) and bool as "non-zero".
+template <typename ODT, typename IDT>
+__device__ __forceinline__ ODT convert(IDT x) {
+  if constexpr (IsBf16<IDT>::value) {
+    float const f = bf16_bits_to_f32(*reinterpret_cast<uint16_t const *>(&x));
+    return convert<ODT, float>(f);
+  } else if constexpr (IsBf16<ODT>::value) {
+    float f;
+    if constexpr (IsBool<IDT>::value) f = x ? 1.0f : 0.0f;
+    else f = static_cast<float>(x);
+    uint16_t const bits = (uint16_t)f32_to_bf16_bits(f);
+    return *reinterpret_cast<bf16 const *>(&bits);
+  } else if constexpr (IsBool<ODT>::value) {
+    return x != static_cast<IDT>(0);
+  } else if constexpr (IsBool<IDT>::value) {
+    return static_cast<ODT>(x ? 1 : 0);
+  } else if constexpr (IsHalf<IDT>::value || IsHalf<ODT>::value) {
+    return static_cast<ODT>(static_cast<float>(x));
+  } else {
+    return static_cast<ODT>(x);
+  }
+}
+
+// a + b in the type's own arithmetic (bf16/half: add in fp32, round once;
+// bool: logical or, as `bool + 1 * bool` converts back to bool)
+template <typename T>
+__device__ __forceinline__ T add_in_type(T a, T b) {
+  if constexpr (IsBf16<T>::value) {
+    return convert<T, float>(convert<float, T>(a) + convert<float, T>(b));
+  } else if constexpr (IsHalf<T>::value) {
+    return static_cast<T>(static_cast<float>(a) + static_cast<float>(b));
+  } else if constexpr (IsBool<T>::value) {
+    return a || b;
+  } else {
+    return static_cast<T>(a + b);
+  }
+}
+
+template <typename IDT, typename ODT, bool BACKWARD>
+__global__ __launch_bounds__(kCastThreads) void cast_kernel(IDT const *__restrict__ in, ODT *out, int64_t n) {
+  int64_t const stride = (int64_t)gridDim.x * kCastThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kCastThreads + threadIdx.x; i < n; i += stride) {
+    ODT c = convert<ODT, IDT>(in[i]);
+    if (BACKWARD) c = add_in_type<ODT>(c, out[i]);
+    out[i] = c;
+  }
+}
+
+template <typename IDT, typename ODT>
+static hipError_t cast_launch(hipStream_t st, void const *in, void *out, int64_t n, bool backward) {
+  int64_t b = ceil_div(n, kCastThreads);
+  int64_t const cap = (int64_t)kNumCU * 64;
+  unsigned const blocks = (unsigned)(b < cap ? b : cap);
+  if (backward) {
+    cast_kernel<IDT, ODT, true><<<blocks, kCastThreads, 0, st>>>(static_cast<IDT const *>(in),
+                                                                static_cast<ODT *>(out), n);
+  } else {
+    cast_kernel<IDT, ODT, false><<<blocks, kCastThreads, 0, st>>>(static_cast<IDT const *>(in),
+                                                                 static_cast<ODT *>(out), n);
+  }
+  return hipGetLastError();
+}
+
+template <typename IDT>
+static int cast_out(char const *who, hipStream_t st, int out_dtype, void const *in, void *out,
+                    int64_t n, bool backward) {
+  hipError_t e;
+  switch (out_dtype) {
+    case FFK_BOOL: e = cast_launch<IDT, bool>(st, in, out, n, backward); break;
+    case FFK_INT32: e = cast_launch<IDT, int32_t>(st, in, out, n, backward); break;
+    case FFK_INT64: e = cast_launch<IDT, int64_t>(st, in, out, n, backward); break;
+    case FFK_HALF: e = cast_launch<IDT, _Float16>(st, in, out, n, backward); break;
+    case FFK_FLOAT: e = cast_launch<IDT, float>(st, in, out, n, backward); break;
+    case FFK_DOUBLE: e = cast_launch<IDT, double>(st, in, out, n, backward); break;
+    case FFK_BF16: e = cast_launch<IDT, bf16>(st, in, out, n, backward); break;
+    default: return fail(FFK_ERR_UNSUPPORTED, "%s: output dtype %d not supported", who, out_dtype);
+  }
+  FFK_HIP(e);
+  return FFK_OK;
+}
+
+static int cast_any(char const *who, ffk_stream_t stream, int in_dtype, int out_dtype,
+                    void const *in, void *out, int64_t n, bool backward) {
+  FFK_REQUIRE(n >= 0, "%s: negative size", who);
+  if (n == 0) return FFK_OK;
+  FFK_REQUIRE(in && out, "%s: NULL tensor", who);
+  hipStream_t st = as_stream(stream);
+  switch (in_dtype) {
+    case FFK_BOOL: return cast_out<bool>(who, st, out_dtype, in, out, n, backward);
+    case FFK_INT32: return cast_out<int32_t>(who, st, out_dtype, in, out, n, backward);
+    case FFK_INT64: return cast_out<int64_t>(who, st, out_dtype, in, out, n, backward);
+    case FFK_HALF: return cast_out<_Float16>(who, st, out_dtype, in, out, n, backward);
+    case FFK_FLOAT: return cast_out<float>(who, st, out_dtype, in, out, n, backward);
+    case FFK_DOUBLE: return cast_out<double>(who, st, out_dtype, in, out, n, backward);
+    case FFK_BF16: return cast_out<bf16>(who, st, out_dtype, in, out, n, backward);
+    default: return fail(FFK_ERR_UNSUPPORTED, "%s: input dtype %d not supported", who, in_dtype);
+  }
+}
+
+}  // namespace ffk
+
+using namespace ffk;
+
+extern "C" int ffk_cast_forward(ffk_stream_t stream, int input_dtype, int output_dtype,
+                                void const *input, void *output, int64_t num_elements) {
+  return cast_any("cast_forward", stream, input_dtype, output_dtype, input, output, num_elements, false);
+}
+
+extern "C" int ffk_cast_backward(ffk_stream_t stream, int output_grad_dtype,
+                                 int input_grad_dtype, void const *output_grad,
+                                 void *input_grad, int64_t num_elements) {
+  return cast_any("cast_backward", stream, output_grad_dtype, input_grad_dtype, output_grad,
+                  input_grad, num_elements, true);
+}

@@ -6,6 +6,9 @@
 #include "kernels/dropout_kernels.h"
 #include "kernels/element_kernels.h"
 #include "kernels/embedding_kernels.h"
+#include "kernels/cast_kernels.h"
+#include "kernels/loss_function_kernels.h"
+#include "kernels/optimizer_kernels.h"
 #include "kernels/layer_norm_kernels.h"
 #include "kernels/linear_kernels.h"
 #include "kernels/softmax_kernels.h"
@@ -472,4 +475,103 @@ void backward_kernel(device_stream_t const &stream, GenericTensorAccessorR const
 }
 
 }  // namespace Kernels::Embedding
+// ---- Optimizer, loss, cast --------------------------------------------------
+
+void sgd_update_task(device_stream_t const &stream, device_handle_t const &, float lr, float momentum,
+                     bool nesterov, float weight_decay, GenericTensorAccessorR const &weight_grad,
+                     int num_replicas, GenericTensorAccessorW const &weight,
+                     std::optional<GenericTensorAccessorW> const &sgd_v) {
+  if (sgd_v.has_value() != (momentum > 0.0f)) {
+    throw std::runtime_error("sgd_update_task: sgd_v must be given exactly when momentum > 0");
+  }
+  if (!stream.is_gpu()) no_cpu("sgd_update_task");
+  if (weight.shape.data_type != DataType::FLOAT) {
+    throw std::runtime_error("sgd_update_task: weights must be FLOAT");
+  }
+  check_ffk(ffk_sgd_update(stream.require_gpu(), dt(weight_grad.shape.data_type), lr, momentum, nesterov,
+                           weight_decay, weight_grad.ptr, get_num_elements(weight.shape.dims), num_replicas,
+                           static_cast<float *>(weight.ptr),
+                           sgd_v.has_value() ? static_cast<float *>(sgd_v->ptr) : nullptr, nullptr),
+            "sgd_update_task");
+}
+
+void adam_update_task(device_stream_t const &stream, device_handle_t const &, float alpha_t, float beta1,
+                      float beta2, float weight_decay, float epsilon, float const *weight_grad_ptr,
+                      size_t size, int num_replicas, float *weight_ptr, float *adam_v_ptr,
+                      float *adam_m_ptr) {
+  if (!stream.is_gpu()) no_cpu("adam_update_task");
+  check_ffk(ffk_adam_update(stream.require_gpu(), FFK_FLOAT, alpha_t, beta1, beta2, weight_decay, epsilon,
+                            weight_grad_ptr, (int64_t)size, num_replicas, weight_ptr, adam_v_ptr, adam_m_ptr,
+                            nullptr),
+            "adam_update_task");
+}
+
+void sparse_categorical_crossentropy_loss_backward_kernel(device_stream_t const &stream, float *logit_grad_ptr,
+                                                          float const *logit_ptr, int const *label_ptr,
+                                                          size_t logit_volume, size_t logit_grad_volume,
+                                                          int num_samples, int num_classes, int k,
+                                                          float scale_factor) {
+  if (!stream.is_gpu()) no_cpu("sparse_categorical_crossentropy_loss_backward_kernel");
+  check_ffk(ffk_sparse_categorical_crossentropy_loss_backward(stream.require_gpu(), logit_grad_ptr, logit_ptr,
+                                                              label_ptr, (int64_t)logit_volume,
+                                                              (int64_t)logit_grad_volume, num_samples,
+                                                              num_classes, k, scale_factor),
+            "sparse_categorical_crossentropy_loss_backward_kernel");
+}
+
+void categorical_crossentropy_loss_backward_kernel(device_stream_t const &stream,
+                                                   GenericTensorAccessorW const &logit_grad,
+                                                   GenericTensorAccessorR const &logit,
+                                                   GenericTensorAccessorR const &label, float scale_factor) {
+  if (!stream.is_gpu()) no_cpu("categorical_crossentropy_loss_backward_kernel");
+  if (logit.shape.data_type != DataType::FLOAT || label.shape.data_type != DataType::FLOAT ||
+      logit_grad.shape.data_type != DataType::FLOAT) {
+    throw std::runtime_error("categorical_crossentropy_loss_backward_kernel: tensors must be FLOAT");
+  }
+  check_ffk(ffk_categorical_crossentropy_loss_backward(
+                stream.require_gpu(), static_cast<float *>(logit_grad.ptr),
+                static_cast<float const *>(logit.ptr), static_cast<float const *>(label.ptr),
+                get_num_elements(logit.shape.dims), get_num_elements(logit_grad.shape.dims), scale_factor),
+            "categorical_crossentropy_loss_backward_kernel");
+}
+
+void mean_squared_error_avg_loss_backward_kernel(device_stream_t const &stream, float *logit_grad_ptr,
+                                                 float const *logit_ptr, float const *label_ptr,
+                                                 size_t logit_volume, size_t logit_grad_volume,
+                                                 float scale_factor) {
+  if (!stream.is_gpu()) no_cpu("mean_squared_error_avg_loss_backward_kernel");
+  check_ffk(ffk_mean_squared_error_avg_loss_backward(stream.require_gpu(), logit_grad_ptr, logit_ptr, label_ptr,
+                                                     (int64_t)logit_volume, (int64_t)logit_grad_volume,
+                                                     scale_factor),
+            "mean_squared_error_avg_loss_backward_kernel");
+}
+
+void identity_loss_backward_kernel(device_stream_t const &stream, float *loss_grad_ptr, float const *loss_ptr,
+                                   size_t loss_volume, size_t loss_grad_volume, float scale_factor) {
+  if (!stream.is_gpu()) no_cpu("identity_loss_backward_kernel");
+  check_ffk(ffk_identity_loss_backward(stream.require_gpu(), loss_grad_ptr, loss_ptr, (int64_t)loss_volume,
+                                       (int64_t)loss_grad_volume, scale_factor),
+            "identity_loss_backward_kernel");
+}
+
+namespace Kernels::Cast {
+
+void forward_kernel(device_stream_t const &stream, GenericTensorAccessorR const &input,
+                    GenericTensorAccessorW const &output) {
+  if (!stream.is_gpu()) no_cpu("Cast::forward_kernel");
+  check_ffk(ffk_cast_forward(stream.require_gpu(), dt(input.shape.data_type), dt(output.shape.data_type),
+                             input.ptr, output.ptr, get_num_elements(input.shape.dims)),
+            "Cast::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, GenericTensorAccessorR const &output_grad,
+                     GenericTensorAccessorW const &input_grad) {
+  if (!stream.is_gpu()) no_cpu("Cast::backward_kernel");
+  check_ffk(ffk_cast_backward(stream.require_gpu(), dt(output_grad.shape.data_type),
+                              dt(input_grad.shape.data_type), output_grad.ptr, input_grad.ptr,
+                              get_num_elements(output_grad.shape.dims)),
+            "Cast::backward_kernel");
+}
+
+}  // namespace Kernels::Cast
+
 }  // namespace FlexFlow

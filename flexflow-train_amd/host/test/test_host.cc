@@ -6,11 +6,14 @@
 #include "ffk_oracle.h"
 #include "kernels/allocation.h"
 #include "kernels/attention_kernels.h"
+#include "kernels/cast_kernels.h"
 #include "kernels/dropout_kernels.h"
 #include "kernels/element_kernels.h"
 #include "kernels/embedding_kernels.h"
 #include "kernels/layer_norm_kernels.h"
 #include "kernels/linear_kernels.h"
+#include "kernels/loss_function_kernels.h"
+#include "kernels/optimizer_kernels.h"
 #include "kernels/profiling.h"
 #include "kernels/softmax_kernels.h"
 #include <cmath>
@@ -369,6 +372,74 @@ static void gpu_tests() {
     auto fstate = Kernels::MultiHeadAttention::init_kernel(DeviceType::GPU, handle, gpu, B, H, E, E, E, D, D, D, E, S, S, false);
     CHECK_THROWS(Kernels::MultiHeadAttention::forward_kernel(stream, fstate, (float const *)Q.ptr, (float const *)Q.ptr,
                                                              (float const *)Q.ptr, (float const *)W.ptr, (float *)O.ptr));
+  });
+  run("sgd_update_task / adam_update_task equal the oracle bit for bit", [&] {
+    int64_t n = 10007;
+    auto w = random_vec(n, 20), g = random_vec(n, 21), v = random_vec(n, 22, 0.0f, 1.0f), m = random_vec(n, 23);
+    TensorShape s = shape({n}, DataType::FLOAT);
+    auto W = device_accessor(gpu, s, w), G = device_accessor(gpu, s, g), V = device_accessor(gpu, s, v);
+    std::vector<float> w1 = w, v1 = v;
+    orc_sgd_update(0.01f, 0.9f, 1, 1e-4f, g.data(), n, 1, w1.data(), v1.data());
+    sgd_update_task(stream, handle, 0.01f, 0.9f, true, 1e-4f, read_only_accessor_from_write_accessor(G), 1, W, V);
+    CHECK(to_host(W) == w1 && to_host(V) == v1);
+    CHECK_THROWS(sgd_update_task(stream, handle, 0.01f, 0.9f, true, 1e-4f, read_only_accessor_from_write_accessor(G), 1,
+                                 W, std::nullopt));
+    // a fresh second moment: the SGD velocity above may be negative
+    auto M = device_accessor(gpu, s, m);
+    V = device_accessor(gpu, s, v);
+    std::vector<float> w2 = w1, v2 = v, m2 = m;
+    orc_adam_update(1e-3f, 0.9f, 0.999f, 1e-2f, 1e-8f, g.data(), n, 1, w2.data(), v2.data(), m2.data());
+    adam_update_task(stream, handle, 1e-3f, 0.9f, 0.999f, 1e-2f, 1e-8f, G.get_float_ptr(), (size_t)n, 1,
+                     W.get_float_ptr(), V.get_float_ptr(), M.get_float_ptr());
+    CHECK(to_host(W) == w2 && to_host(V) == v2 && to_host(M) == m2);
+  });
+
+  run("loss backward kernels equal the oracle bit for bit", [&] {
+    int samples = 33, classes = 17;
+    int64_t n = (int64_t)samples * classes;
+    auto logit = random_vec(n, 24, 0.0f, 1.0f), label = random_vec(n, 25, 0.0f, 1.0f);
+    std::vector<int> sparse(samples);
+    std::mt19937 gen(1);
+    for (auto &l : sparse) l = (int)(gen() % classes);
+    TensorShape s = shape({samples, classes}, DataType::FLOAT);
+    auto L = device_accessor(gpu, s, logit), T = device_accessor(gpu, s, label);
+    auto DL = gpu.allocate_tensor(s);
+    Allocator cpu = create_local_cpu_memory_allocator();
+    GenericTensorAccessorW hl = cpu.allocate_tensor(shape({samples}, DataType::INT32));
+    memcpy(hl.ptr, sparse.data(), sparse.size() * 4);
+    GenericTensorAccessorW SL = copy_tensor_accessor_w(hl, gpu);
+    float scale = 1.0f / samples;
+    std::vector<float> want(n);
+    orc_sparse_cce_loss_backward(want.data(), logit.data(), sparse.data(), n, samples, classes, 1, scale);
+    sparse_categorical_crossentropy_loss_backward_kernel(stream, DL.get_float_ptr(), L.get_float_ptr(),
+                                                         static_cast<int const *>(SL.ptr), n, n, samples, classes, 1,
+                                                         scale);
+    CHECK(to_host(DL) == want);
+    orc_difference_loss_backward(want.data(), logit.data(), label.data(), n, scale);
+    categorical_crossentropy_loss_backward_kernel(stream, DL, read_only_accessor_from_write_accessor(L),
+                                                  read_only_accessor_from_write_accessor(T), scale);
+    CHECK(to_host(DL) == want);
+    mean_squared_error_avg_loss_backward_kernel(stream, DL.get_float_ptr(), L.get_float_ptr(), T.get_float_ptr(), n, n,
+                                                scale);
+    CHECK(to_host(DL) == want);
+    orc_identity_loss_backward(want.data(), n, scale);
+    identity_loss_backward_kernel(stream, DL.get_float_ptr(), L.get_float_ptr(), n, n, scale);
+    CHECK(to_host(DL) == want);
+  });
+
+  run("Cast float -> bf16 -> float rounds to nearest even; backward accumulates", [&] {
+    int64_t n = 4099;
+    auto x = random_vec(n, 26, -100.0f, 100.0f);
+    auto X = device_accessor(gpu, shape({n}, DataType::FLOAT), x);
+    auto Y = gpu.allocate_tensor(shape({n}, DataType::BF16));
+    Kernels::Cast::forward_kernel(stream, read_only_accessor_from_write_accessor(X), Y);
+    std::vector<float> want = x;
+    orc_round_bf16_array(want.data(), want.size());
+    CHECK(to_host(Y) == want);
+    auto DX = device_accessor(gpu, shape({n}, DataType::FLOAT), x);
+    Kernels::Cast::backward_kernel(stream, read_only_accessor_from_write_accessor(Y), DX);
+    for (int64_t i = 0; i < n; i++) want[i] += x[i];
+    CHECK(to_host(DX) == want);
   });
 }
 

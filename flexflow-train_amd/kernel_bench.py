@@ -5,7 +5,8 @@
 Groups: gemm (config 2 and config 5 projection GEMMs), bandwidth (config 3:
 LayerNorm, Softmax, ElementBinary, Dropout, plus GELU), embedding (config 4:
 token gather / scatter-add, DLRM bags), attention (config 5 and the config 2
-core).  Every line gives the mean launch time over the timed iterations
+core), update (optimizer steps, Cast and loss backward over a parameter-sized
+buffer).  Every line gives the mean launch time over the timed iterations
 (HIP events on torch's current stream, which is the stream the entry points are
 given) and the ALGORITHMIC bytes or flops of the op divided by that time,
 against 8 TB/s HBM or the 2.5 PFLOP/s dense bf16 MFMA peak.  Inputs are
@@ -163,7 +164,41 @@ def bench_attention():
         report("attention bwd B%d H%d S%d D%d causal=%d" % (B, H, S, D, causal), t, flops=2.5 * f)
 
 
-GROUPS = dict(gemm=bench_gemm, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention)
+def bench_update():
+    # 64 Mi parameters: a few encoder layers' worth; the config 2 layer alone (12.6 M)
+    # is over in a handful of microseconds
+    n = 64 << 20
+    w = torch.randn(n, device="cuda")
+    g = torch.randn(n, device="cuda")
+    gb = g.to(BT)
+    v = torch.zeros(n, device="cuda")
+    m = torch.zeros(n, device="cuda")
+    wl = torch.empty(n, device="cuda", dtype=BT)
+    t = timeit(lambda: ffk.sgd_update(w, g, 0.01))
+    report("SGD plain, fp32 grad", t, bytes_=12 * n)
+    t = timeit(lambda: ffk.sgd_update(w, g, 0.01, 0.9, True, 1e-4, sgd_v=v))
+    report("SGD momentum+nesterov, fp32 grad", t, bytes_=20 * n)
+    t = timeit(lambda: ffk.sgd_update(w, gb, 0.01, 0.9, True, 1e-4, sgd_v=v, weight_lowp=wl))
+    report("SGD momentum, bf16 grad, bf16 weight copy out", t, bytes_=20 * n)
+    t = timeit(lambda: ffk.adam_update(w, g, m, v, 1e-3, weight_decay=1e-2))
+    report("Adam, fp32 grad", t, bytes_=28 * n)
+    t = timeit(lambda: ffk.adam_update(w, gb, m, v, 1e-3, weight_decay=1e-2, weight_lowp=wl))
+    report("Adam, bf16 grad, bf16 weight copy out", t, bytes_=28 * n)
+    t = timeit(lambda: ffk.cast_forward(w, wl))
+    report("Cast fp32 -> bf16", t, bytes_=6 * n)
+    t = timeit(lambda: ffk.cast_backward(wl, g))
+    report("Cast backward bf16 -> fp32 (accumulating)", t, bytes_=10 * n)
+    samples, classes = 4096, 50257
+    logit = torch.rand((samples, classes), device="cuda")
+    label = torch.randint(0, classes, (samples,), device="cuda", dtype=torch.int32)
+    out = torch.empty_like(logit)
+    t = timeit(lambda: ffk.sparse_categorical_crossentropy_loss_backward(logit, label, samples, classes, 1,
+                                                                         1.0 / samples, out=out))
+    report("sparse CCE loss backward [4096, 50257]", t, bytes_=8 * samples * classes)
+
+
+GROUPS = dict(gemm=bench_gemm, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention,
+              update=bench_update)
 
 if __name__ == "__main__":
     ffk.lib()

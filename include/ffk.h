@@ -431,6 +431,72 @@ int ffk_encoder_layer_backward(ffk_stream_t stream, int dtype,
                                void const *x, void const *dy, void *dx,
                                void *workspace, size_t workspace_bytes);
 
+/* ------------------------------------------------------------------------ */
+/* Optimizer updates -- sgd_update_task / adam_update_task
+ * (lib/kernels/include/kernels/optimizer_kernels.h:11-36; CUDA bodies
+ * lib/kernels/src/cuda/optimizer_kernels.cu:23-44,111-133; CPU SGD
+ * lib/kernels/src/kernels/optimizer_kernels_cpu.cc:10-60).
+ *   SGD : gt = g + wd*W; if momentum > 0 { V = V*momentum + gt;
+ *         gt = nesterov ? gt + momentum*V : V }; W -= lr*gt
+ *   Adam: gt = g + wd*W; M = b1*M + (1-b1)*gt; V = b2*V + (1-b2)*gt*gt;
+ *         W -= alpha_t * M / (sqrt(V) + epsilon)    (alpha_t is the caller's
+ *         bias-corrected step, as in the reference)
+ * Every step is a separately rounded fp32 operation, matching the reference's
+ * CPU evaluation.  weight, sgd_v, adam_v, adam_m: fp32 [num_elements].
+ * weight_grad: grad_dtype FFK_FLOAT or FFK_BF16, [num_replicas][num_elements];
+ * replicas are summed in order (the parameter-server launcher's first step;
+ * unlike it, the sum is not written back into replica 0).  sgd_v must be given
+ * exactly when momentum > 0.  weight_lowp: optional bf16 copy of the updated
+ * weights written in the same pass (NULL: none); no reference counterpart.    */
+int ffk_sgd_update(ffk_stream_t stream, int grad_dtype, float lr, float momentum,
+                   int nesterov, float weight_decay, void const *weight_grad,
+                   int64_t num_elements, int num_replicas, float *weight,
+                   float *sgd_v, void *weight_lowp);
+int ffk_adam_update(ffk_stream_t stream, int grad_dtype, float alpha_t,
+                    float beta1, float beta2, float weight_decay, float epsilon,
+                    void const *weight_grad, int64_t num_elements,
+                    int num_replicas, float *weight, float *adam_v,
+                    float *adam_m, void *weight_lowp);
+
+/* ------------------------------------------------------------------------ */
+/* Loss-function backward -- *_loss_backward_kernel
+ * (lib/kernels/include/kernels/loss_function_kernels.h:9-45; CUDA bodies
+ * lib/kernels/src/cuda/loss_function_kernels.cu:21-139).  fp32; the volumes
+ * are element counts and must be equal.
+ *   sparse categorical CE: logit_grad[s,c] = (logit[s,c] - [c == label[s/k]])
+ *                          * (scale_factor * k) for the first num_samples rows
+ *                          of num_classes, plain logit * scale beyond them;
+ *                          labels outside [0, num_classes) subtract nothing
+ *                          (the reference writes out of bounds for them)
+ *   categorical CE, MSE  : logit_grad = (logit - label) * scale_factor
+ *   identity             : loss_grad = 1 * scale_factor                      */
+int ffk_sparse_categorical_crossentropy_loss_backward(
+    ffk_stream_t stream, float *logit_grad, float const *logit, int const *label,
+    int64_t logit_volume, int64_t logit_grad_volume, int num_samples,
+    int num_classes, int k, float scale_factor);
+int ffk_categorical_crossentropy_loss_backward(
+    ffk_stream_t stream, float *logit_grad, float const *logit, float const *label,
+    int64_t logit_volume, int64_t logit_grad_volume, float scale_factor);
+int ffk_mean_squared_error_avg_loss_backward(
+    ffk_stream_t stream, float *logit_grad, float const *logit, float const *label,
+    int64_t logit_volume, int64_t logit_grad_volume, float scale_factor);
+int ffk_identity_loss_backward(ffk_stream_t stream, float *loss_grad,
+                               float const *loss, int64_t loss_volume,
+                               int64_t loss_grad_volume, float scale_factor);
+
+/* ------------------------------------------------------------------------ */
+/* Cast -- Kernels::Cast::gpu_forward_kernel / gpu_backward_kernel
+ * (cast_kernels_gpu.h; lib/kernels/src/cuda/ops/cast_kernels.cu:25-37).
+ *   forward : output[i] = (ODT) input[i]
+ *   backward: input_grad[i] = (ODT) output_grad[i] + input_grad[i]
+ * Any pair of FFK_BOOL, FFK_INT32, FFK_INT64, FFK_HALF, FFK_FLOAT, FFK_DOUBLE,
+ * FFK_BF16; static_cast semantics, float -> bf16/half rounds to nearest even. */
+int ffk_cast_forward(ffk_stream_t stream, int input_dtype, int output_dtype,
+                     void const *input, void *output, int64_t num_elements);
+int ffk_cast_backward(ffk_stream_t stream, int output_grad_dtype,
+                      int input_grad_dtype, void const *output_grad,
+                      void *input_grad, int64_t num_elements);
+
 #ifdef __cplusplus
 }
 #endif

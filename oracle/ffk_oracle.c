@@ -45,6 +45,24 @@
  *      "non-zero": PARITY UNPINNED by the reference.  Pinned here by the
  *      textbook definition: torch scaled_dot_product_attention in fp64,
  *      softmax row sums, causal independence, finite differences.
+ *  orc_sgd_update             src/cuda/optimizer_kernels.cu:23-44 and the CPU
+ *      composition src/kernels/optimizer_kernels_cpu.cc:10-60 (every tensor op
+ *      separately rounded, which is what -ffp-contract=off gives here).  The
+ *      reference has no test for it (PARITY UNPINNED there); pinned by
+ *      torch.optim.SGD (the kernel cites it) in fp64 and by special cases
+ *      (lr = 0, momentum = 0, weight_decay = 0 reduce to textbook steps).
+ *  orc_adam_update            src/cuda/optimizer_kernels.cu:111-133 (the CPU
+ *      version is NOT_IMPLEMENTED in the reference; no test: PARITY UNPINNED
+ *      there).  Pinned by the closed form in fp64 and by the first step from
+ *      zero state, where W moves by alpha_t*(1-b1)*g / (sqrt((1-b2) g^2)+eps).
+ *  orc_*_loss_backward        src/cuda/loss_function_kernels.cu:21-139
+ *      no reference test (PARITY UNPINNED there); pinned by the closed forms
+ *      (gradient of mean softmax-cross-entropy w.r.t. the softmax output path
+ *      the reference uses: logit - onehot, times the scale).
+ *  orc_cast_*                 src/kernels/cast_kernels_cpu.cc:6-20
+ *      the reference tests only compare its GPU and CPU kernels on random
+ *      data; pinned by numpy astype on exactly representable values and on
+ *      rounding boundaries.
  */
 #include "ffk_oracle.h"
 #include <math.h>
@@ -939,4 +957,95 @@ void orc_mha_backward(orc_mha_desc_t const *d, float const *query,
   }
   free(tmp);
   free(Q); free(K); free(V); free(C); free(dC); free(dQ); free(dK); free(dV);
+}
+
+/* ------------------------------------------------------- optimizer updates */
+
+void orc_sgd_update(float lr, float momentum, int nesterov, float weight_decay,
+                    float const *grad, int64_t n, int replicas, float *w,
+                    float *v) {
+  for (int64_t i = 0; i < n; i++) {
+    float g = grad[i];
+    for (int r = 1; r < replicas; r++) {
+      g = g + grad[(int64_t)r * n + i];
+    }
+    float t = weight_decay * w[i];
+    float gt = g + t;
+    if (momentum > 0.0f) {
+      float vm = v[i] * momentum;
+      float vn = vm + gt;
+      v[i] = vn;
+      if (nesterov) {
+        float mv = momentum * vn;
+        gt = gt + mv;
+      } else {
+        gt = vn;
+      }
+    }
+    float step = lr * gt;
+    w[i] = w[i] - step;
+  }
+}
+
+void orc_adam_update(float alpha_t, float beta1, float beta2, float weight_decay,
+                     float epsilon, float const *grad, int64_t n, int replicas,
+                     float *w, float *vv, float *mm) {
+  for (int64_t i = 0; i < n; i++) {
+    float g = grad[i];
+    for (int r = 1; r < replicas; r++) {
+      g = g + grad[(int64_t)r * n + i];
+    }
+    float t = weight_decay * w[i];
+    float gt = g + t;
+    float a = beta1 * mm[i];
+    float c1 = 1.0f - beta1;
+    float b = c1 * gt;
+    float mt = a + b;
+    float c = beta2 * vv[i];
+    float c2 = 1.0f - beta2;
+    float d = c2 * gt;
+    float e = d * gt;
+    float vt = c + e;
+    mm[i] = mt;
+    vv[i] = vt;
+    float num = alpha_t * mt;
+    float den = sqrtf(vt) + epsilon;
+    float q = num / den;
+    w[i] = w[i] - q;
+  }
+}
+
+/* ------------------------------------------------------------ loss backward */
+
+void orc_sparse_cce_loss_backward(float *dlogit, float const *logit,
+                                  int const *label, int64_t volume,
+                                  int64_t num_samples, int64_t num_classes,
+                                  int k, float scale_factor) {
+  /* copy, subtract 1 at the label, scale by scale_factor * k */
+  memcpy(dlogit, logit, sizeof(float) * (size_t)volume);
+  for (int64_t i = 0; i < num_samples; i++) {
+    int64_t l = label[i / k];
+    if (l >= 0 && l < num_classes) {
+      dlogit[i * num_classes + l] -= 1.0f;
+    }
+  }
+  float s = scale_factor * (float)k;
+  for (int64_t i = 0; i < volume; i++) {
+    dlogit[i] = dlogit[i] * s;
+  }
+}
+
+void orc_difference_loss_backward(float *dlogit, float const *logit,
+                                  float const *label, int64_t volume,
+                                  float scale_factor) {
+  for (int64_t i = 0; i < volume; i++) {
+    float d = logit[i] - label[i];
+    dlogit[i] = d * scale_factor;
+  }
+}
+
+void orc_identity_loss_backward(float *dloss, int64_t volume, float scale_factor) {
+  for (int64_t i = 0; i < volume; i++) {
+    dloss[i] = 1.0f * scale_factor;
+  }
 }

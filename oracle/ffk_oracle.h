@@ -138,6 +138,21 @@ void orc_mha_backward(orc_mha_desc_t const *d, float const *query,
                       float *dquery, float *dkey, float *dvalue,
                       float *dweight, int bf16_mode);
 
+void orc_sgd_update(float lr, float momentum, int nesterov, float weight_decay,
+                    float const *grad, int64_t n, int replicas, float *w,
+                    float *v);
+void orc_adam_update(float alpha_t, float beta1, float beta2, float weight_decay,
+                     float epsilon, float const *grad, int64_t n, int replicas,
+                     float *w, float *vv, float *mm);
+void orc_sparse_cce_loss_backward(float *dlogit, float const *logit,
+                                  int const *label, int64_t volume,
+                                  int64_t num_samples, int64_t num_classes,
+                                  int k, float scale_factor);
+void orc_difference_loss_backward(float *dlogit, float const *logit,
+                                  float const *label, int64_t volume,
+                                  float scale_factor);
+void orc_identity_loss_backward(float *dloss, int64_t volume, float scale_factor);
+
 #ifdef __cplusplus
 }
 #endif

@@ -351,3 +351,53 @@ def mha_backward(desc, query, key, value, weight, out_grad, bf16_mode=False):
     lib().orc_mha_backward(ctypes.byref(desc), _p(query), _p(key), _p(value), _p(weight),
                            _p(out_grad), _p(dq), _p(dk), _p(dv), _p(dw), c_int(int(bf16_mode)))
     return dq, dk, dv, dw
+
+
+def sgd_update(w, grad, lr, momentum=0.0, nesterov=False, weight_decay=0.0, v=None, replicas=1):
+    """Returns (w_new, v_new); grad holds `replicas` copies of length w.size back to back."""
+    w = _f32(w).copy()
+    g = _f32(grad)
+    vv = None if v is None else _f32(v).copy()
+    lib().orc_sgd_update(c_f(lr), c_f(momentum), c_int(int(nesterov)), c_f(weight_decay), _p(g),
+                         c_i64(w.size), c_int(replicas), _p(w), _p(vv))
+    return w, vv
+
+
+def adam_update(w, grad, m, v, alpha_t, beta1=0.9, beta2=0.999, weight_decay=0.0, epsilon=1e-8,
+                replicas=1):
+    """Returns (w_new, m_new, v_new)."""
+    w, m, v = _f32(w).copy(), _f32(m).copy(), _f32(v).copy()
+    g = _f32(grad)
+    lib().orc_adam_update(c_f(alpha_t), c_f(beta1), c_f(beta2), c_f(weight_decay), c_f(epsilon),
+                          _p(g), c_i64(w.size), c_int(replicas), _p(w), _p(v), _p(m))
+    return w, m, v
+
+
+def sparse_cce_loss_backward(logit, label, num_samples, num_classes, k, scale_factor):
+    logit = _f32(logit)
+    label = np.ascontiguousarray(label, dtype=np.int32)
+    out = np.empty_like(logit)
+    lib().orc_sparse_cce_loss_backward(_p(out), _p(logit), _p(label), c_i64(logit.size),
+                                       c_i64(num_samples), c_i64(num_classes), c_int(k),
+                                       c_f(scale_factor))
+    return out
+
+
+def difference_loss_backward(logit, label, scale_factor):
+    logit, label = _f32(logit), _f32(label)
+    out = np.empty_like(logit)
+    lib().orc_difference_loss_backward(_p(out), _p(logit), _p(label), c_i64(logit.size),
+                                       c_f(scale_factor))
+    return out
+
+
+def identity_loss_backward(shape, scale_factor):
+    out = np.empty(shape, np.float32)
+    lib().orc_identity_loss_backward(_p(out), c_i64(out.size), c_f(scale_factor))
+    return out
+
+
+def cast(x, out_dtype):
+    """static_cast element by element (cast_kernels_cpu.cc:6-11); numpy's astype
+    is the same conversion for the type pairs used here."""
+    return np.ascontiguousarray(x).astype(out_dtype)
