@@ -66,17 +66,60 @@ __global__ __launch_bounds__(kCastThreads) void cast_kernel(IDT const *__restric
   }
 }
 
+// V consecutive elements moved as one naturally aligned object, so a lane's
+// loads and stores are 16-byte (or, for the narrower side, 8- or 4-byte) accesses
+template <typename T, int V>
+struct alignas(sizeof(T) * V > 16 ? 16 : sizeof(T) * V) CastPack {
+  T v[V];
+};
+
+template <typename IDT, typename ODT>
+constexpr int cast_pack_width() {
+  return (sizeof(IDT) > 4 || sizeof(ODT) > 4) ? 4 : 8;
+}
+
+template <typename IDT, typename ODT, bool BACKWARD>
+__global__ __launch_bounds__(kCastThreads) void cast_vec_kernel(IDT const *__restrict__ in, ODT *out, int64_t n) {
+  constexpr int V = cast_pack_width<IDT, ODT>();
+  int64_t const packs = n / V;
+  int64_t const stride = (int64_t)gridDim.x * kCastThreads;
+  int64_t const tid = (int64_t)blockIdx.x * kCastThreads + threadIdx.x;
+  for (int64_t p = tid; p < packs; p += stride) {
+    CastPack<IDT, V> const a = reinterpret_cast<CastPack<IDT, V> const *>(in)[p];
+    CastPack<ODT, V> o;
+    if (BACKWARD) o = reinterpret_cast<CastPack<ODT, V> const *>(out)[p];
+#pragma unroll
+    for (int e = 0; e < V; e++) {
+      ODT c = convert<ODT, IDT>(a.v[e]);
+      if (BACKWARD) c = add_in_type<ODT>(c, o.v[e]);
+      o.v[e] = c;
+    }
+    reinterpret_cast<CastPack<ODT, V> *>(out)[p] = o;
+  }
+  int64_t const j = packs * V + tid;
+  if (j < n) {
+    ODT c = convert<ODT, IDT>(in[j]);
+    if (BACKWARD) c = add_in_type<ODT>(c, out[j]);
+    out[j] = c;
+  }
+}
+
 template <typename IDT, typename ODT>
 static hipError_t cast_launch(hipStream_t st, void const *in, void *out, int64_t n, bool backward) {
-  int64_t b = ceil_div(n, kCastThreads);
+  constexpr int V = cast_pack_width<IDT, ODT>();
+  bool const vec = n >= V && reinterpret_cast<uintptr_t>(in) % alignof(CastPack<IDT, V>) == 0 &&
+                   reinterpret_cast<uintptr_t>(out) % alignof(CastPack<ODT, V>) == 0;
+  int64_t b = ceil_div(vec ? n / V : n, kCastThreads);
   int64_t const cap = (int64_t)kNumCU * 64;
   unsigned const blocks = (unsigned)(b < cap ? b : cap);
-  if (backward) {
-    cast_kernel<IDT, ODT, true><<<blocks, kCastThreads, 0, st>>>(static_cast<IDT const *>(in),
-                                                                static_cast<ODT *>(out), n);
+  IDT const *ip = static_cast<IDT const *>(in);
+  ODT *op = static_cast<ODT *>(out);
+  if (vec) {
+    if (backward) cast_vec_kernel<IDT, ODT, true><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
+    else cast_vec_kernel<IDT, ODT, false><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
   } else {
-    cast_kernel<IDT, ODT, false><<<blocks, kCastThreads, 0, st>>>(static_cast<IDT const *>(in),
-                                                                 static_cast<ODT *>(out), n);
+    if (backward) cast_kernel<IDT, ODT, true><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
+    else cast_kernel<IDT, ODT, false><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
   }
   return hipGetLastError();
 }

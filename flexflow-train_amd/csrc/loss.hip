@@ -9,30 +9,75 @@ namespace ffk {
 
 constexpr int kLossThreads = 256;
 
+// Each lane handles four consecutive elements with 16-byte accesses when the
+// tensors are 16-byte aligned (`vec`), one element otherwise.
+
 // logit_grad[s, c] = (logit[s, c] - [c == label[s / k]]) * (scale * k)
 // (copy, then `logit_grad[i * num_classes + label[i / k]] -= 1`, then
 // scale_kernel(.., 0, scale_factor * k): loss_function_kernels.cu:21-31,59-84)
+template <bool VEC>
 __global__ __launch_bounds__(kLossThreads) void sparse_cce_backward_kernel(
     float *__restrict__ dlogit, float const *__restrict__ logit,
     int const *__restrict__ label, int64_t num_samples, int64_t num_classes,
     int k, int64_t volume, float scale) {
-  int64_t const i = (int64_t)blockIdx.x * kLossThreads + threadIdx.x;
+  constexpr int V = VEC ? 4 : 1;
+  int64_t const i = ((int64_t)blockIdx.x * kLossThreads + threadIdx.x) * V;
   if (i >= volume) return;
-  int64_t const s = i / num_classes;
-  int64_t const c = i % num_classes;
-  float v = logit[i];
-  if (s < num_samples && (int64_t)label[s / k] == c) v = __fsub_rn(v, 1.0f);
-  dlogit[i] = __fmul_rn(v, scale);
+  int64_t s = i / num_classes;
+  int64_t c = i - s * num_classes;
+  if (VEC && i + 4 <= volume) {
+    f32x4 v = *reinterpret_cast<f32x4 const *>(logit + i);
+    // the row's label is looked up once per row the lane touches (-1: no such sample)
+    int64_t hot = s < num_samples ? (int64_t)label[s / k] : -1;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      if (hot == c) v[e] = __fsub_rn(v[e], 1.0f);
+      v[e] = __fmul_rn(v[e], scale);
+      if (++c == num_classes) {
+        c = 0;
+        s++;
+        hot = s < num_samples ? (int64_t)label[s / k] : -1;
+      }
+    }
+    *reinterpret_cast<f32x4 *>(dlogit + i) = v;
+  } else {
+    for (int64_t j = i; j < i + V && j < volume; j++) {
+      float v = logit[j];
+      if (s < num_samples && (int64_t)label[s / k] == c) v = __fsub_rn(v, 1.0f);
+      dlogit[j] = __fmul_rn(v, scale);
+      if (++c == num_classes) {
+        c = 0;
+        s++;
+      }
+    }
+  }
 }
 
 // (logit - label) * scale: categorical cross-entropy and mean-squared-error
 // (loss_function_kernels.cu:33-49)
+template <bool VEC>
 __global__ __launch_bounds__(kLossThreads) void difference_loss_backward_kernel(
     float *__restrict__ dlogit, float const *__restrict__ logit,
     float const *__restrict__ label, int64_t volume, float scale) {
-  int64_t const i = (int64_t)blockIdx.x * kLossThreads + threadIdx.x;
+  constexpr int V = VEC ? 4 : 1;
+  int64_t const i = ((int64_t)blockIdx.x * kLossThreads + threadIdx.x) * V;
   if (i >= volume) return;
-  dlogit[i] = __fmul_rn(__fsub_rn(logit[i], label[i]), scale);
+  if (VEC && i + 4 <= volume) {
+    f32x4 const a = *reinterpret_cast<f32x4 const *>(logit + i);
+    f32x4 const b = *reinterpret_cast<f32x4 const *>(label + i);
+    f32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) o[e] = __fmul_rn(__fsub_rn(a[e], b[e]), scale);
+    *reinterpret_cast<f32x4 *>(dlogit + i) = o;
+  } else {
+    for (int64_t j = i; j < i + V && j < volume; j++) {
+      dlogit[j] = __fmul_rn(__fsub_rn(logit[j], label[j]), scale);
+    }
+  }
+}
+
+static bool aligned16(void const *a, void const *b, void const *c) {
+  return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15) == 0;
 }
 
 // 1 * scale (loss_function_kernels.cu:51-57)
@@ -60,9 +105,13 @@ extern "C" int ffk_sparse_categorical_crossentropy_loss_backward(
               "sparse_categorical_crossentropy_loss_backward: num_samples * num_classes exceeds the logits");
   if (logit_volume == 0) return FFK_OK;
   FFK_REQUIRE(logit_grad && logit && label, "sparse_categorical_crossentropy_loss_backward: NULL tensor");
-  sparse_cce_backward_kernel<<<loss_blocks(logit_volume), kLossThreads, 0, as_stream(stream)>>>(
-      logit_grad, logit, label, num_samples, num_classes, k, logit_volume,
-      scale_factor * (float)k);
+  if (aligned16(logit_grad, logit, nullptr)) {
+    sparse_cce_backward_kernel<true><<<loss_blocks(ceil_div(logit_volume, 4)), kLossThreads, 0, as_stream(stream)>>>(
+        logit_grad, logit, label, num_samples, num_classes, k, logit_volume, scale_factor * (float)k);
+  } else {
+    sparse_cce_backward_kernel<false><<<loss_blocks(logit_volume), kLossThreads, 0, as_stream(stream)>>>(
+        logit_grad, logit, label, num_samples, num_classes, k, logit_volume, scale_factor * (float)k);
+  }
   FFK_CHECK_LAUNCH();
   return FFK_OK;
 }
@@ -73,8 +122,13 @@ static int difference_loss(char const *who, ffk_stream_t stream, float *logit_gr
   FFK_REQUIRE(logit_volume >= 0 && logit_grad_volume == logit_volume, "%s: bad sizes", who);
   if (logit_volume == 0) return FFK_OK;
   FFK_REQUIRE(logit_grad && logit && label, "%s: NULL tensor", who);
-  difference_loss_backward_kernel<<<loss_blocks(logit_volume), kLossThreads, 0, as_stream(stream)>>>(
-      logit_grad, logit, label, logit_volume, scale_factor);
+  if (aligned16(logit_grad, logit, label)) {
+    difference_loss_backward_kernel<true><<<loss_blocks(ceil_div(logit_volume, 4)), kLossThreads, 0, as_stream(stream)>>>(
+        logit_grad, logit, label, logit_volume, scale_factor);
+  } else {
+    difference_loss_backward_kernel<false><<<loss_blocks(logit_volume), kLossThreads, 0, as_stream(stream)>>>(
+        logit_grad, logit, label, logit_volume, scale_factor);
+  }
   FFK_CHECK_LAUNCH();
   return FFK_OK;
 }

@@ -80,10 +80,11 @@ def test_adam_update_bit_exact(ffk, oracle, n, gdt):
     assert np.array_equal(to_np(w), w_ref)
 
 
-def test_loss_backward_bit_exact(ffk, oracle):
-    say("loss backward")
+@pytest.mark.parametrize("C", [1000, 1003, 3, 1])
+def test_loss_backward_bit_exact(ffk, oracle, C):
+    say("loss backward", C)
     g = rng(9)
-    B, C = 96, 1000
+    B = 96
     logit = g.random((B, C)).astype(np.float32)
     label = g.integers(0, C, size=B).astype(np.int32)
     scale = 1.0 / B
@@ -119,7 +120,7 @@ NP = {torch.bool: np.bool_, torch.int32: np.int32, torch.int64: np.int64, torch.
 def test_cast_forward_backward(ffk, oracle, idt, odt):
     say("cast", idt, odt)
     g = rng(3)
-    n = 1000
+    n = 1003
     # small integers and halves: exactly representable in every type, so the
     # conversion itself (not a rounding choice) is what is checked ...
     vals = g.integers(-64, 64, size=n).astype(np.float64) / (1.0 if idt in (torch.int32, torch.int64, torch.bool) else 2.0)
@@ -160,3 +161,30 @@ def test_cast_rounding_to_bf16_and_half(ffk, oracle):
     outd = torch.empty(4096, dtype=torch.float64, device="cuda")
     ffk.cast_forward(to_dev(x, torch), outd)
     assert np.array_equal(outd.cpu().numpy(), oracle.cast(x, np.float64))
+
+
+def test_cast_and_loss_on_unaligned_views(ffk, oracle):
+    say("cast / loss, pointers off the 16-byte grid")
+    g = rng(12)
+    n = 777
+    x = g.standard_normal(n + 1).astype(np.float32)
+    xd = to_dev(x, torch)[1:]                       # 4 bytes past a 16-byte boundary
+    out = torch.empty(n + 3, dtype=torch.bfloat16, device="cuda")[3:]
+    ffk.cast_forward(xd, out)
+    assert np.array_equal(to_np(out), bf16_round(x[1:]))
+    acc = to_dev(x, torch)[1:].clone()
+    accv = torch.zeros(n + 1, device="cuda")[1:]
+    accv.copy_(acc)
+    ffk.cast_backward(out, accv)
+    assert np.array_equal(to_np(accv), bf16_round(x[1:]) + x[1:])
+    B, C = 7, 111
+    logit = g.random(B * C + 1).astype(np.float32)
+    lab = g.random(B * C).astype(np.float32)
+    label = g.integers(0, C, size=B).astype(np.int32)
+    ld = to_dev(logit, torch)[1:]
+    want = oracle.sparse_cce_loss_backward(logit[1:].reshape(B, C), label, B, C, 1, 0.25)
+    got = ffk.sparse_categorical_crossentropy_loss_backward(ld, to_dev(label, torch, torch.int32), B, C, 1, 0.25)
+    assert np.array_equal(to_np(got).reshape(B, C), want)
+    want = oracle.difference_loss_backward(logit[1:], lab, 0.25)
+    got = ffk.difference_loss_backward("categorical_crossentropy", ld, to_dev(lab, torch), 0.25)
+    assert np.array_equal(to_np(got), want)
