@@ -1,0 +1,654 @@
+// The training-step driver (reference: lib/local-execution/src/local-execution/
+// computation_graph_instance.cc:61-260, task_execution.cc:84-125,
+// tensor_allocation.cc, per_device_op_state_initialization.cc:21-56; the task
+// bodies it dispatches to are lib/task-spec/src/task-spec/ops/impl/*.cc,
+// loss_functions.cc:24-150 and optimizer.cc:10-108).
+//
+// Everything a step needs is decided once, here: one device allocation holds
+// every tensor the caller did not bring (gradients that are added into first,
+// so a single fill clears them), the saved operator state and a scratch region
+// the backward kernels share; each invocation is a closure over final device
+// pointers that makes one C-ABI call.
+#include "ffk.h"
+#include "local-execution/computation_graph_instance.h"
+#include <cmath>
+#include <cstring>
+
+namespace FlexFlow {
+
+[[noreturn]] static void bad(std::string const &msg) { throw std::runtime_error("computation graph instance: " + msg); }
+
+static int dt(DataType d) { return static_cast<int>(d); }
+static bool is_float_type(DataType d) {
+  return d == DataType::FLOAT || d == DataType::BF16 || d == DataType::HALF || d == DataType::DOUBLE;
+}
+static size_t align_up(size_t n) { return (n + 255) & ~(size_t)255; }
+
+LossFunction get_loss_function(LossAttrs const &a) {
+  if (std::holds_alternative<SparseCategoricalCrossEntropyLossAttrs>(a)) {
+    return LossFunction::SPARSE_CATEGORICAL_CROSSENTROPY;
+  }
+  return std::get<NonconfigurableLossAttrs>(a).loss_type;
+}
+
+OptimizerAttrs get_optimizer_attrs_for_next_iter(OptimizerAttrs const &old_attrs) {
+  if (auto const *old = std::get_if<AdamOptimizerAttrs>(&old_attrs)) {
+    double new_beta1_t = old->beta_t * old->beta1;
+    double new_beta2_t = old->beta2_t * old->beta2;
+    double new_alpha_t = old->alpha * std::sqrt(1 - new_beta2_t) / (1 - new_beta1_t);
+    return AdamOptimizerAttrs{old->alpha,  old->beta1,  old->beta2,  old->weight_decay,
+                              new_alpha_t, new_beta1_t, new_beta2_t, old->epsilon};
+  }
+  return old_attrs;
+}
+
+// ---- state --------------------------------------------------------------------
+
+struct ComputationGraphInstance::State {
+  ComputationGraph cg;
+  Allocator allocator;
+  OptimizerAttrs optimizer_attrs;
+  std::vector<GenericTensorAccessorW> value;
+  std::vector<std::optional<GenericTensorAccessorW>> grad, master, opt_v, opt_m;
+  std::optional<tensor_guid_t> logit;
+  std::vector<DynamicNodeInvocation> order;
+  char *arena = nullptr;
+  size_t arena_bytes = 0, cleared_bytes = 0;
+  bool masters_valid = false;
+  uint64_t iteration = 0;
+
+  State(ComputationGraph const &g, Allocator const &a, OptimizerAttrs const &o) : cg(g), allocator(a), optimizer_attrs(o) {}
+  State(State const &) = delete;
+  State &operator=(State const &) = delete;
+  ~State() {
+    if (arena != nullptr) allocator.deallocate(arena);
+  }
+};
+
+ComputationGraphInstance::ComputationGraphInstance(std::shared_ptr<State> s) : state(std::move(s)) {}
+std::vector<DynamicNodeInvocation> const &ComputationGraphInstance::get_execution_order() const { return state->order; }
+Allocator &ComputationGraphInstance::get_allocator() const { return state->allocator; }
+OptimizerAttrs const &ComputationGraphInstance::get_optimizer_attrs() const { return state->optimizer_attrs; }
+void ComputationGraphInstance::update_optimizer_attrs_for_next_iter() {
+  state->optimizer_attrs = get_optimizer_attrs_for_next_iter(state->optimizer_attrs);
+  state->iteration++;
+}
+std::optional<GenericTensorAccessorR> ComputationGraphInstance::get_loss_tensor_accessor() const {
+  if (!state->logit.has_value()) return std::nullopt;
+  return read_only_accessor_from_write_accessor(state->grad.at(state->logit->raw).value());
+}
+GenericTensorAccessorW ComputationGraphInstance::get_tensor_accessor(tensor_guid_t t) const {
+  return state->value.at(t.raw);
+}
+std::optional<GenericTensorAccessorW> ComputationGraphInstance::get_gradient_accessor(tensor_guid_t t) const {
+  return state->grad.at(t.raw);
+}
+std::optional<GenericTensorAccessorW> ComputationGraphInstance::get_master_weight_accessor(tensor_guid_t t) const {
+  return state->master.at(t.raw);
+}
+size_t ComputationGraphInstance::bytes_allocated() const { return state->arena_bytes; }
+
+void ComputationGraphInstance::sync_master_weights() const {
+  ffk_stream_t st = get_gpu_device_stream().require_gpu();
+  for (size_t t = 0; t < state->master.size(); t++) {
+    if (!state->master[t].has_value()) continue;
+    GenericTensorAccessorW const &w = state->value[t];
+    check_ffk(ffk_cast_forward(st, dt(w.shape.data_type), FFK_FLOAT, w.ptr, state->master[t]->ptr,
+                               get_num_elements(w.shape.dims)),
+              "sync_master_weights");
+  }
+  state->masters_valid = true;
+}
+
+void ComputationGraphInstance::clear_accumulated_gradients(device_stream_t const &stream) const {
+  if (state->cleared_bytes > 0) {
+    check_ffk(ffk_fill_zero(state->arena, state->cleared_bytes, stream.require_gpu()), "clear gradients");
+  }
+}
+
+// ---- planning -------------------------------------------------------------------
+
+namespace {
+
+// how each operator's backward treats the gradients it produces
+struct BackwardPlan {
+  bool has_backward = false;
+  bool accumulate = false;                 // one switch for all input gradients of the op
+  std::vector<bool> accumulate_input;      // Linear only: input, weight, bias
+  bool softmax_via_scratch = false;
+};
+
+struct Slot {
+  size_t offset = 0, bytes = 0;
+};
+
+struct Planner {
+  size_t total = 0;
+  Slot take(size_t bytes) {
+    Slot s{total, bytes};
+    total += align_up(bytes);
+    return s;
+  }
+};
+
+struct LayerPlan {
+  BackwardPlan bwd;
+  Slot saved;        // state kept from forward to backward (LayerNorm statistics, attention reserve)
+  size_t scratch_bytes = 0;  // backward scratch, shared between layers
+};
+
+bool is_op_layer(ComputationGraph::Layer const &l) {
+  return !std::holds_alternative<InputAttrs>(l.attrs.op_attrs) && !std::holds_alternative<WeightAttrs>(l.attrs.op_attrs);
+}
+
+ffk_mha_desc_t mha_desc(MultiHeadAttentionAttrs const &a, TensorShape const &q, TensorShape const &k, TensorShape const &v) {
+  ffk_mha_desc_t d{};
+  d.num_samples = dim_at_idx(q.dims, 0);
+  d.num_heads = a.num_heads;
+  d.q_size = dim_at_idx(q.dims, -1);
+  d.k_size = dim_at_idx(k.dims, -1);
+  d.v_size = dim_at_idx(v.dims, -1);
+  d.q_proj_size = a.kdim;
+  d.k_proj_size = a.kdim;
+  d.v_proj_size = a.vdim;
+  d.o_proj_size = a.embed_dim;
+  d.qo_seq_length = dim_at_idx(q.dims, 1);
+  d.kv_seq_length = dim_at_idx(k.dims, 1);
+  d.scale = a.scale;
+  d.causal = a.causal ? 1 : 0;
+  return d;
+}
+
+int activation_code(std::optional<Activation> const &a) { return a.has_value() ? static_cast<int>(*a) : FFK_ACT_NONE; }
+
+int aggr_code(std::optional<AggregateOp> const &a) {
+  if (!a.has_value()) return FFK_AGGR_NONE;
+  return *a == AggregateOp::SUM ? FFK_AGGR_SUM : FFK_AGGR_AVG;
+}
+
+}  // namespace
+
+ComputationGraphInstance create_computation_graph_instance(
+    ComputationGraph const &cg, OptimizerAttrs const &optimizer_attrs, std::optional<LossConfig> const &loss,
+    std::unordered_map<tensor_guid_t, GenericTensorAccessorW> const &input_tensors, Allocator &allocator,
+    ProfilingSettings const &, device_handle_t const &device_handle, device_id_t device_idx) {
+  if (device_idx.device_type != DeviceType::GPU || !device_handle.is_for_gpu() ||
+      allocator.get_allocation_device_type() != DeviceType::GPU) {
+    bad("NOT_IMPLEMENTED for the CPU device type in this library");
+  }
+  auto st = std::make_shared<ComputationGraphInstance::State>(cg, allocator, optimizer_attrs);
+  size_t const T = cg.tensors.size(), L = cg.layers.size();
+  auto shape_of = [&](tensor_guid_t t) -> TensorShape const & { return cg.tensors.at(t.raw).shape; };
+  auto numel = [&](tensor_guid_t t) { return get_num_elements(shape_of(t).dims); };
+
+  // -- which tensors carry a gradient, and who writes it
+  std::vector<bool> has_grad(T, false), is_weight(T, false);
+  for (size_t t = 0; t < T; t++) {
+    ComputationGraph::Layer const &src = cg.layers.at(cg.tensors[t].source.raw);
+    bool const input_without_grad = std::holds_alternative<InputAttrs>(src.attrs.op_attrs) && cg.tensors[t].create_grad == CreateGrad::NO;
+    has_grad[t] = is_float_type(cg.tensors[t].shape.data_type) && !input_without_grad;
+    is_weight[t] = std::holds_alternative<WeightAttrs>(src.attrs.op_attrs);
+  }
+  if (loss.has_value()) {
+    st->logit = loss->logit_tensor;
+    if (!has_grad.at(loss->logit_tensor.raw)) bad("the logit tensor carries no gradient");
+    if (shape_of(loss->logit_tensor).data_type != DataType::FLOAT) bad("the loss kernels take FLOAT logits (cast first)");
+  }
+  std::vector<int> writers(T, 0);
+  for (size_t l = 0; l < L; l++) {
+    ComputationGraph::Layer const &layer = cg.layers[l];
+    if (!is_op_layer(layer)) continue;
+    bool const self_attention = std::holds_alternative<MultiHeadAttentionAttrs>(layer.attrs.op_attrs) &&
+                                layer.inputs[0] == layer.inputs[1] && layer.inputs[0] == layer.inputs[2];
+    for (size_t i = 0; i < layer.inputs.size(); i++) {
+      if (self_attention && i > 0) break;  // key and value gradients are folded into the query's
+      if (has_grad[layer.inputs[i].raw]) writers[layer.inputs[i].raw]++;
+    }
+    for (tensor_guid_t w : layer.weights) writers[w.raw]++;
+  }
+  auto must_accumulate = [&](tensor_guid_t t) {
+    return writers[t.raw] > 1 || (st->logit.has_value() && *st->logit == t);
+  };
+
+  // -- per-layer backward mode, saved state and scratch
+  std::vector<LayerPlan> plan(L);
+  std::vector<bool> cleared(T, false);  // gradient must be zero before the backward pass
+  Planner saved_planner;
+  size_t scratch_bytes = 0, discard_bytes = 0;
+  for (size_t l = 0; l < L; l++) {
+    ComputationGraph::Layer const &layer = cg.layers[l];
+    if (!is_op_layer(layer)) continue;
+    LayerPlan &p = plan[l];
+    ComputationGraphOpAttrs const &oa = layer.attrs.op_attrs;
+    bool any_grad = false;
+    for (tensor_guid_t t : layer.inputs) any_grad = any_grad || has_grad[t.raw];
+    for (tensor_guid_t t : layer.weights) any_grad = any_grad || has_grad[t.raw];
+    p.bwd.has_backward = any_grad && has_grad[layer.outputs.at(0).raw];
+    bool acc = false;
+    for (tensor_guid_t t : layer.inputs) acc = acc || (has_grad[t.raw] && must_accumulate(t));
+    if (auto const *a = std::get_if<LinearAttrs>(&oa)) {
+      int64_t batch = numel(layer.inputs[0]) / dim_at_idx(shape_of(layer.inputs[0]).dims, -1);
+      p.scratch_bytes = ffk_linear_backward_workspace_bytes(dt(shape_of(layer.outputs[0]).data_type), activation_code(a->activation),
+                                                            a->use_bias, batch, a->out_channels);
+      // one flag per gradient: input, weight, bias (a weight shared between layers is added into)
+      p.bwd.accumulate_input = {acc};
+      for (tensor_guid_t w : layer.weights) p.bwd.accumulate_input.push_back(writers[w.raw] > 1);
+      acc = false;
+      if (p.bwd.accumulate_input[0]) cleared[layer.inputs[0].raw] = true;
+      for (size_t i = 0; i < layer.weights.size(); i++) {
+        if (p.bwd.accumulate_input[1 + i]) cleared[layer.weights[i].raw] = true;
+      }
+    } else if (std::get_if<LayerNormAttrs>(&oa)) {
+      int64_t N = layer.weights.empty() ? 0 : numel(layer.weights[0]);
+      auto const *a = std::get_if<LayerNormAttrs>(&oa);
+      if (N == 0) {
+        N = 1;
+        int nd = get_num_dims(shape_of(layer.inputs[0]).dims);
+        for (size_t i = 0; i < a->axes.size(); i++) N *= shape_of(layer.inputs[0]).dims.ff_ordered[nd - 1 - (int)i];
+      }
+      int64_t M = numel(layer.inputs[0]) / N;
+      for (tensor_guid_t w : layer.weights) {
+        if (writers[w.raw] > 1) bad("LayerNorm weights cannot be shared between layers (their gradients are overwritten)");
+      }
+      p.saved = saved_planner.take(align_up((size_t)M * 4) * 2);
+      p.scratch_bytes = ffk_layer_norm_backward_workspace_bytes(M, N);
+    } else if (auto const *a = std::get_if<MultiHeadAttentionAttrs>(&oa)) {
+      ffk_mha_desc_t d = mha_desc(*a, shape_of(layer.inputs[0]), shape_of(layer.inputs[1]), shape_of(layer.inputs[2]));
+      p.saved = saved_planner.take(ffk_mha_reserve_bytes(&d, dt(shape_of(layer.inputs[0]).data_type)));
+      // key == value but not the query: both gradients land in one tensor
+      if (layer.inputs[1] == layer.inputs[2] && layer.inputs[0] != layer.inputs[1]) acc = true;
+      if (layer.inputs[0] == layer.inputs[1] && layer.inputs[0] != layer.inputs[2]) acc = true;
+      if (layer.inputs[0] == layer.inputs[2] && layer.inputs[0] != layer.inputs[1]) acc = true;
+      cleared[layer.weights.at(0).raw] = true;  // the weight gradient is always added into
+    } else if (auto const *a = std::get_if<EmbeddingAttrs>(&oa)) {
+      p.scratch_bytes = ffk_embedding_backward_workspace_bytes(numel(layer.inputs[0]), a->num_entries);
+      cleared[layer.weights.at(0).raw] = true;
+    } else if (std::get_if<SoftmaxAttrs>(&oa)) {
+      // the kernel overwrites; with other producers it goes through scratch and is added
+      if (acc) {
+        p.bwd.softmax_via_scratch = true;
+        p.scratch_bytes = (size_t)get_size_in_bytes(shape_of(layer.inputs[0]));
+      }
+    } else if (std::get_if<CastAttrs>(&oa)) {
+      acc = true;  // cast_backward always adds
+    } else if (std::get_if<ElementBinaryAttrs>(&oa)) {
+      if (p.bwd.has_backward && numel(layer.inputs[0]) != numel(layer.inputs[1])) {
+        bad("element binary backward needs operands of equal size");
+      }
+      if (layer.inputs[0] == layer.inputs[1]) acc = true;
+    }
+    p.bwd.accumulate = acc;
+    if (acc) {
+      for (tensor_guid_t t : layer.inputs) {
+        if (has_grad[t.raw]) cleared[t.raw] = true;
+      }
+    }
+    scratch_bytes = std::max(scratch_bytes, p.scratch_bytes);
+    // an input without a gradient still needs somewhere for the kernel to write
+    if (p.bwd.has_backward && !std::holds_alternative<LinearAttrs>(oa) && !std::holds_alternative<EmbeddingAttrs>(oa)) {
+      for (tensor_guid_t t : layer.inputs) {
+        if (!has_grad[t.raw]) discard_bytes = std::max(discard_bytes, (size_t)get_size_in_bytes(shape_of(t)));
+      }
+    }
+  }
+  if (st->logit.has_value()) cleared[st->logit->raw] = false;  // written by the loss before any producer adds
+
+  // -- placement: cleared gradients first, then everything else
+  Planner arena;
+  std::vector<Slot> grad_slot(T), value_slot(T), master_slot(T), v_slot(T), m_slot(T);
+  for (size_t t = 0; t < T; t++) {
+    if (has_grad[t] && cleared[t]) grad_slot[t] = arena.take((size_t)get_size_in_bytes(cg.tensors[t].shape));
+  }
+  st->cleared_bytes = arena.total;
+  bool const adam = std::holds_alternative<AdamOptimizerAttrs>(optimizer_attrs);
+  bool const sgd_momentum = !adam && std::get<SGDOptimizerAttrs>(optimizer_attrs).momentum > 0.0;
+  for (size_t t = 0; t < T; t++) {
+    TensorShape const &s = cg.tensors[t].shape;
+    if (has_grad[t] && !cleared[t]) grad_slot[t] = arena.take((size_t)get_size_in_bytes(s));
+    if (input_tensors.count(tensor_guid_t{(int)t}) == 0) value_slot[t] = arena.take((size_t)get_size_in_bytes(s));
+    if (is_weight[t] && has_grad[t]) {
+      if (s.data_type != DataType::FLOAT && s.data_type != DataType::BF16) bad("weights must be FLOAT or BF16");
+      size_t f32 = (size_t)get_num_elements(s.dims) * 4;
+      if (s.data_type == DataType::BF16) master_slot[t] = arena.take(f32);
+      if (adam || sgd_momentum) v_slot[t] = arena.take(f32);
+      if (adam) m_slot[t] = arena.take(f32);
+    }
+  }
+  size_t const saved_base = arena.take(saved_planner.total).offset;
+  size_t const scratch_base = arena.take(scratch_bytes).offset;
+  size_t const discard_base = arena.take(discard_bytes).offset;
+  st->arena_bytes = arena.total;
+  st->arena = static_cast<char *>(allocator.allocate(std::max<size_t>(arena.total, 256)));
+  // optimizer moments start at zero; so do gradients nobody writes
+  check_ffk(ffk_fill_zero(st->arena, std::max<size_t>(arena.total, 256), nullptr), "create_computation_graph_instance");
+  check_ffk(ffk_stream_synchronize(nullptr), "create_computation_graph_instance");
+
+  char *const base = st->arena;
+  auto f32_accessor = [&](size_t t, Slot const &s) -> std::optional<GenericTensorAccessorW> {
+    if (s.bytes == 0) return std::nullopt;
+    return GenericTensorAccessorW{TensorShape{cg.tensors[t].shape.dims, DataType::FLOAT}, base + s.offset, DeviceType::GPU};
+  };
+  st->value.resize(T, GenericTensorAccessorW{TensorShape{TensorDims{{}}, DataType::FLOAT}, nullptr, DeviceType::GPU});
+  st->grad.resize(T);
+  st->master.resize(T);
+  st->opt_v.resize(T);
+  st->opt_m.resize(T);
+  for (size_t t = 0; t < T; t++) {
+    auto bound = input_tensors.find(tensor_guid_t{(int)t});
+    if (bound != input_tensors.end()) {
+      if (bound->second.shape != cg.tensors[t].shape) bad("a bound tensor has the wrong shape");
+      if (bound->second.device_type != DeviceType::GPU) bad("a bound tensor is not device-resident");
+      st->value[t] = bound->second;
+    } else {
+      st->value[t] = GenericTensorAccessorW{cg.tensors[t].shape, base + value_slot[t].offset, DeviceType::GPU};
+    }
+    if (has_grad[t]) st->grad[t] = GenericTensorAccessorW{cg.tensors[t].shape, base + grad_slot[t].offset, DeviceType::GPU};
+    st->master[t] = f32_accessor(t, master_slot[t]);
+    st->opt_v[t] = f32_accessor(t, v_slot[t]);
+    st->opt_m[t] = f32_accessor(t, m_slot[t]);
+  }
+  void *const scratch = base + scratch_base;
+  void *const discard = base + discard_base;
+  ComputationGraphInstance::State *const S = st.get();  // closures must not own the state they live in
+
+  auto val = [&](tensor_guid_t t) { return st->value[t.raw].ptr; };
+  auto grd = [&](tensor_guid_t t) -> void * { return has_grad[t.raw] ? st->grad[t.raw]->ptr : nullptr; };
+  auto grd_or_discard = [&](tensor_guid_t t) -> void * { return has_grad[t.raw] ? st->grad[t.raw]->ptr : discard; };
+
+  // -- FWD / BWD invocations
+  std::vector<DynamicNodeInvocation> fwd, bwd;
+  for (size_t l = 0; l < L; l++) {
+    ComputationGraph::Layer const &layer = cg.layers[l];
+    if (!is_op_layer(layer)) continue;
+    LayerPlan const &p = plan[l];
+    ComputationGraphOpAttrs const &oa = layer.attrs.op_attrs;
+    layer_guid_t const id{(int)l};
+    tensor_guid_t const out = layer.outputs.at(0);
+    void *const y = val(out);
+    void *const dy = grd(out);
+    size_t const ws_bytes = p.scratch_bytes;
+    std::function<void(device_stream_t const &)> f, b;
+
+    if (auto const *a = std::get_if<LinearAttrs>(&oa)) {
+      tensor_guid_t x = layer.inputs[0];
+      int const type = dt(shape_of(x).data_type), act = activation_code(a->activation);
+      int64_t const in_dim = dim_at_idx(shape_of(x).dims, -1), out_dim = a->out_channels, batch = numel(x) / in_dim;
+      void *xp = val(x), *w = val(layer.weights[0]), *bias = a->use_bias ? val(layer.weights[1]) : nullptr;
+      void *dx = grd(x), *dw = grd(layer.weights[0]), *dbias = a->use_bias ? grd(layer.weights[1]) : nullptr;
+      int const accumulate = (p.bwd.accumulate_input[0] ? FFK_ACC_INPUT : 0) | (p.bwd.accumulate_input[1] ? FFK_ACC_WEIGHT : 0) |
+                             (a->use_bias && p.bwd.accumulate_input[2] ? FFK_ACC_BIAS : 0);
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_linear_forward(s.require_gpu(), type, act, xp, y, w, bias, batch, in_dim, out_dim), "Linear forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_linear_backward(s.require_gpu(), type, act, 0, y, dy, xp, dx, w, dw, dbias, batch, in_dim, out_dim,
+                                      ws_bytes ? scratch : nullptr, ws_bytes, accumulate),
+                  "Linear backward");
+      };
+    } else if (auto const *a = std::get_if<LayerNormAttrs>(&oa)) {
+      tensor_guid_t x = layer.inputs[0];
+      int const type = dt(shape_of(x).data_type);
+      int64_t N = 1;
+      int nd = get_num_dims(shape_of(x).dims);
+      for (size_t i = 0; i < a->axes.size(); i++) N *= shape_of(x).dims.ff_ordered[nd - 1 - (int)i];
+      int64_t const M = numel(x) / N;
+      float *mean = reinterpret_cast<float *>(base + saved_base + p.saved.offset);
+      float *rstd = reinterpret_cast<float *>(base + saved_base + p.saved.offset + align_up((size_t)M * 4));
+      void *xp = val(x), *dx = grd_or_discard(x);
+      void *gamma = a->elementwise_affine ? val(layer.weights[0]) : nullptr;
+      void *beta = a->elementwise_affine ? val(layer.weights[1]) : nullptr;
+      void *dgamma = a->elementwise_affine ? grd(layer.weights[0]) : nullptr;
+      void *dbeta = a->elementwise_affine ? grd(layer.weights[1]) : nullptr;
+      float const eps = a->eps;
+      int const accumulate = p.bwd.accumulate ? 1 : 0;
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_layer_norm_forward(s.require_gpu(), type, xp, y, gamma, beta, mean, rstd, M, N, eps), "LayerNorm forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_layer_norm_backward(s.require_gpu(), type, dy, xp, mean, rstd, gamma, dx, dgamma, dbeta, M, N, scratch,
+                                          ws_bytes, accumulate),
+                  "LayerNorm backward");
+      };
+    } else if (auto const *a = std::get_if<MultiHeadAttentionAttrs>(&oa)) {
+      tensor_guid_t q = layer.inputs[0], k = layer.inputs[1], v = layer.inputs[2];
+      int const type = dt(shape_of(q).data_type);
+      ffk_mha_desc_t const d = mha_desc(*a, shape_of(q), shape_of(k), shape_of(v));
+      void *reserve = base + saved_base + p.saved.offset;
+      size_t const reserve_bytes = p.saved.bytes;
+      void *qp = val(q), *kp = val(k), *vp = val(v), *w = val(layer.weights[0]), *dw = grd(layer.weights[0]);
+      void *dq = grd_or_discard(q);
+      void *dk = k == q ? nullptr : grd_or_discard(k);
+      void *dv = v == q ? nullptr : grd_or_discard(v);
+      if ((dk == nullptr) != (dv == nullptr)) bad("attention: key and value must both alias the query, or neither");
+      int const accumulate = p.bwd.accumulate ? 1 : 0;
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_mha_forward(s.require_gpu(), type, &d, qp, kp, vp, w, y, reserve, reserve_bytes), "MultiHeadAttention forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_mha_backward(s.require_gpu(), type, &d, qp, dq, kp, dk, vp, dv, w, dw, dy, reserve, reserve_bytes, accumulate),
+                  "MultiHeadAttention backward");
+      };
+    } else if (auto const *a = std::get_if<DropoutAttrs>(&oa)) {
+      tensor_guid_t x = layer.inputs[0];
+      int const type = dt(shape_of(x).data_type);
+      int64_t const n = numel(x);
+      float const rate = a->rate;
+      uint64_t const seed = a->seed + (uint64_t)l;
+      void *xp = val(x), *dx = grd_or_discard(x);
+      int const accumulate = p.bwd.accumulate ? 1 : 0;
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_dropout_forward(s.require_gpu(), type, xp, y, n, rate, seed, S->iteration * (uint64_t)n), "Dropout forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_dropout_backward(s.require_gpu(), type, dy, dx, n, rate, seed, S->iteration * (uint64_t)n, accumulate),
+                  "Dropout backward");
+      };
+    } else if (auto const *a = std::get_if<ElementUnaryAttrs>(&oa)) {
+      tensor_guid_t x = layer.inputs[0];
+      int const type = dt(shape_of(x).data_type), op = static_cast<int>(a->op_type);
+      int64_t const n = numel(x);
+      float const scalar = a->scalar.value_or(0.0f);
+      void *xp = val(x), *dx = grd_or_discard(x);
+      int const accumulate = p.bwd.accumulate ? 1 : 0;
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_element_unary_forward(s.require_gpu(), type, op, scalar, xp, y, n), "ElementUnary forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_element_unary_backward(s.require_gpu(), type, op, scalar, y, dy, xp, dx, n, accumulate), "ElementUnary backward");
+      };
+    } else if (auto const *a = std::get_if<ElementBinaryAttrs>(&oa)) {
+      tensor_guid_t lhs = layer.inputs[0], rhs = layer.inputs[1];
+      int const type = dt(shape_of(out).data_type), op = static_cast<int>(a->type);
+      int64_t const n = numel(out), nl = numel(lhs), nr = numel(rhs);
+      void *lp = val(lhs), *rp = val(rhs), *dl = grd_or_discard(lhs), *dr = grd_or_discard(rhs);
+      int const accumulate = p.bwd.accumulate ? 1 : 0;
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_element_binary_forward(s.require_gpu(), type, op, lp, rp, y, n, nl, nr), "ElementBinary forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_element_binary_backward(s.require_gpu(), type, op, dy, lp, rp, dl, dr, n, accumulate), "ElementBinary backward");
+      };
+    } else if (auto const *a = std::get_if<SoftmaxAttrs>(&oa)) {
+      tensor_guid_t x = layer.inputs[0];
+      int const type = dt(shape_of(x).data_type);
+      int nd = get_num_dims(shape_of(x).dims), dim = a->dim < 0 ? nd + a->dim : a->dim;
+      int64_t outer = 1, inner = 1;
+      for (int i = 0; i < dim; i++) outer *= shape_of(x).dims.ff_ordered[i];
+      for (int i = dim + 1; i < nd; i++) inner *= shape_of(x).dims.ff_ordered[i];
+      int64_t const size = shape_of(x).dims.ff_ordered[dim], n = numel(x);
+      void *xp = val(x), *dx = grd_or_discard(x);
+      bool const via_scratch = p.bwd.softmax_via_scratch;
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_softmax_forward(s.require_gpu(), type, xp, y, outer, size, inner), "Softmax forward");
+      };
+      // the true gradient; the reference's backward is a copy (softmax_kernels.cu:68-78)
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_softmax_backward(s.require_gpu(), type, y, dy, via_scratch ? scratch : dx, outer, size, inner), "Softmax backward");
+        if (via_scratch) {
+          check_ffk(ffk_element_binary_forward(s.require_gpu(), type, FFK_OP_EW_ADD, dx, scratch, dx, n, n, n), "Softmax backward");
+        }
+      };
+    } else if (auto const *a = std::get_if<EmbeddingAttrs>(&oa)) {
+      tensor_guid_t x = layer.inputs[0];
+      int const itype = dt(shape_of(x).data_type), otype = dt(a->data_type), aggr = aggr_code(a->aggr);
+      int64_t const bag = a->aggr.has_value() ? dim_at_idx(shape_of(x).dims, -1) : 1;
+      int64_t const bags = numel(x) / bag, dim = a->out_channels, entries = a->num_entries;
+      void *xp = val(x), *w = val(layer.weights[0]);
+      float *dw = static_cast<float *>(grd(layer.weights[0]));
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_embedding_forward(s.require_gpu(), itype, FFK_FLOAT, otype, xp, y, w, aggr, bags, bag, dim, entries), "Embedding forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_embedding_backward(s.require_gpu(), itype, otype, xp, dy, dw, aggr, bags, bag, dim, entries, 0,
+                                         ws_bytes ? scratch : nullptr, ws_bytes),
+                  "Embedding backward");
+      };
+    } else if (std::get_if<CastAttrs>(&oa)) {
+      tensor_guid_t x = layer.inputs[0];
+      int const itype = dt(shape_of(x).data_type), otype = dt(shape_of(out).data_type);
+      int64_t const n = numel(x);
+      void *xp = val(x), *dx = grd(x);
+      f = [=](device_stream_t const &s) { check_ffk(ffk_cast_forward(s.require_gpu(), itype, otype, xp, y, n), "Cast forward"); };
+      b = [=](device_stream_t const &s) { check_ffk(ffk_cast_backward(s.require_gpu(), otype, itype, dy, dx, n), "Cast backward"); };
+    } else {
+      bad("operator has no task implementation");
+    }
+    fwd.push_back(DynamicNodeInvocation{DynamicTaskType::FWD, id, f});
+    if (p.bwd.has_backward) bwd.push_back(DynamicNodeInvocation{DynamicTaskType::BWD, id, b});
+  }
+
+  // -- LOSS (loss_functions.cc:24-150)
+  std::vector<DynamicNodeInvocation> order = fwd;
+  if (loss.has_value()) {
+    TensorShape const &ls = shape_of(loss->logit_tensor);
+    GenericTensorAccessorW const label = loss->label_tensor;
+    if (label.device_type != DeviceType::GPU) bad("the label tensor is not device-resident");
+    if (get_num_dims(ls.dims) < 2) bad("the logit tensor is [batch, classes]");
+    int const batch_size = (int)dim_at_idx(ls.dims, -2);
+    int const num_classes = (int)dim_at_idx(ls.dims, -1);
+    int64_t const volume = get_num_elements(ls.dims);
+    float *logit = static_cast<float *>(val(loss->logit_tensor));
+    float *dlogit = static_cast<float *>(grd(loss->logit_tensor));
+    LossFunction const kind = get_loss_function(loss->loss_attrs);
+    std::function<void(device_stream_t const &)> f;
+    if (kind == LossFunction::SPARSE_CATEGORICAL_CROSSENTROPY) {
+      if (label.shape.data_type != DataType::INT32) bad("sparse labels are INT32");
+      int k = 1;
+      if (std::get<SparseCategoricalCrossEntropyLossAttrs>(loss->loss_attrs).replace_labels) {
+        k = (int)(dim_at_idx(ls.dims, 0) / dim_at_idx(label.shape.dims, 0));
+      }
+      if ((int64_t)k * get_num_elements(label.shape.dims) != volume / num_classes) bad("label count does not match the logits");
+      int const samples = (int)(volume / num_classes);
+      float const scale = 1.0f / batch_size;
+      int const *lab = static_cast<int const *>(label.ptr);
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_sparse_categorical_crossentropy_loss_backward(s.require_gpu(), dlogit, logit, lab, volume, volume, samples,
+                                                                    num_classes, k, scale),
+                  "SparseCategoricalCrossEntropyLoss backward");
+      };
+    } else {
+      if (kind != LossFunction::IDENTITY && (label.shape.data_type != DataType::FLOAT || get_num_elements(label.shape.dims) != volume)) {
+        bad("the label tensor must match the FLOAT logits");
+      }
+      float const *lab = static_cast<float const *>(label.ptr);
+      if (kind == LossFunction::CATEGORICAL_CROSSENTROPY) {
+        float const scale = 1.0f / batch_size;
+        f = [=](device_stream_t const &s) {
+          check_ffk(ffk_categorical_crossentropy_loss_backward(s.require_gpu(), dlogit, logit, lab, volume, volume, scale),
+                    "CategoricalCrossEntropyLoss backward");
+        };
+      } else if (kind == LossFunction::MEAN_SQUARED_ERROR_AVG_REDUCE) {
+        float const scale = 2.0f / (float)volume;
+        f = [=](device_stream_t const &s) {
+          check_ffk(ffk_mean_squared_error_avg_loss_backward(s.require_gpu(), dlogit, logit, lab, volume, volume, scale),
+                    "MeanSquaredErrorAvgLoss backward");
+        };
+      } else if (kind == LossFunction::IDENTITY) {
+        float const scale = 1.0f / batch_size;
+        f = [=](device_stream_t const &s) {
+          check_ffk(ffk_identity_loss_backward(s.require_gpu(), dlogit, logit, volume, volume, scale), "IdentityLoss backward");
+        };
+      } else {
+        bad("unsupported loss function");  // the reference panics on MEAN_SQUARED_ERROR_SUM_REDUCE too
+      }
+    }
+    order.push_back(DynamicNodeInvocation{DynamicTaskType::LOSS, layer_guid_t{-1}, f});
+  }
+  for (auto it = bwd.rbegin(); it != bwd.rend(); ++it) order.push_back(*it);
+
+  // -- UPD, one per weight (optimizer.cc:10-108)
+  for (size_t t = 0; t < T; t++) {
+    if (!is_weight[t] || !has_grad[t]) continue;
+    TensorShape const &s = cg.tensors[t].shape;
+    int const grad_type = dt(s.data_type);
+    int64_t const n = get_num_elements(s.dims);
+    bool const lowp = s.data_type == DataType::BF16;
+    float *w32 = static_cast<float *>(lowp ? st->master[t]->ptr : st->value[t].ptr);
+    void *wlow = lowp ? st->value[t].ptr : nullptr;
+    void *g = st->grad[t]->ptr;
+    float *v = st->opt_v[t].has_value() ? static_cast<float *>(st->opt_v[t]->ptr) : nullptr;
+    float *m = st->opt_m[t].has_value() ? static_cast<float *>(st->opt_m[t]->ptr) : nullptr;
+    std::function<void(device_stream_t const &)> f = [=](device_stream_t const &stream) {
+      if (auto const *sgd = std::get_if<SGDOptimizerAttrs>(&S->optimizer_attrs)) {
+        check_ffk(ffk_sgd_update(stream.require_gpu(), grad_type, (float)sgd->lr, (float)sgd->momentum, sgd->nesterov,
+                                 (float)sgd->weight_decay, g, n, 1, w32, v, wlow),
+                  "SGD update");
+      } else {
+        AdamOptimizerAttrs const &adam_attrs = std::get<AdamOptimizerAttrs>(S->optimizer_attrs);
+        check_ffk(ffk_adam_update(stream.require_gpu(), grad_type, (float)adam_attrs.alpha_t, (float)adam_attrs.beta1,
+                                  (float)adam_attrs.beta2, (float)adam_attrs.weight_decay, (float)adam_attrs.epsilon, g, n, 1,
+                                  w32, v, m, wlow),
+                  "Adam update");
+      }
+    };
+    order.push_back(DynamicNodeInvocation{DynamicTaskType::UPD, cg.tensors[t].source, f});
+  }
+  st->order = order;
+  return ComputationGraphInstance{st};
+}
+
+// ---- execution ------------------------------------------------------------------
+
+static LayerTimings execute(ComputationGraphInstance const &instance, ProfilingSettings const &profiling,
+                            std::function<bool(DynamicTaskType)> const &selected) {
+  LayerTimings result;
+  bool cleared = false, masters = false;
+  for (DynamicNodeInvocation const &inv : instance.get_execution_order()) {
+    if (!selected(inv.task_type)) continue;
+    if (!cleared && (inv.task_type == DynamicTaskType::LOSS || inv.task_type == DynamicTaskType::BWD)) {
+      instance.clear_accumulated_gradients(get_gpu_device_stream());
+      cleared = true;
+    }
+    if (!masters && inv.task_type == DynamicTaskType::UPD) {
+      if (!instance.state->masters_valid) instance.sync_master_weights();
+      masters = true;
+    }
+    result[inv.layer_guid] = profiling_wrapper(inv.run, profiling, DeviceType::GPU);
+  }
+  return result;
+}
+
+LayerTimings perform_all_passes_for_computation_graph_instance(ComputationGraphInstance &instance,
+                                                               ProfilingSettings const &profiling, device_handle_t const &,
+                                                               device_id_t) {
+  LayerTimings r = execute(instance, profiling, [](DynamicTaskType) { return true; });
+  instance.update_optimizer_attrs_for_next_iter();
+  return r;
+}
+LayerTimings perform_forward_pass_for_computation_graph_instance(ComputationGraphInstance const &instance,
+                                                                 ProfilingSettings const &profiling, device_handle_t const &,
+                                                                 device_id_t) {
+  return execute(instance, profiling, [](DynamicTaskType t) { return t == DynamicTaskType::FWD; });
+}
+LayerTimings perform_backward_pass_for_computation_graph_instance(ComputationGraphInstance const &instance,
+                                                                  ProfilingSettings const &profiling, device_handle_t const &,
+                                                                  device_id_t) {
+  return execute(instance, profiling, [](DynamicTaskType t) { return t == DynamicTaskType::BWD; });
+}
+void perform_update_pass_for_computation_graph_instance(ComputationGraphInstance &instance, ProfilingSettings const &profiling,
+                                                        device_handle_t const &, device_id_t) {
+  execute(instance, profiling, [](DynamicTaskType t) { return t == DynamicTaskType::UPD; });
+  instance.update_optimizer_attrs_for_next_iter();
+}
+
+}  // namespace FlexFlow

@@ -3,6 +3,7 @@
 // the entry point, copy back, compare).  The CPU oracle is the checker.
 //   test_host --cpu   host-only checks (no device needed)
 //   test_host --gpu   every operator entry point on the device
+//   test_host --bench-step [steps]   times the step driver on the encoder layer
 #include "ffk_oracle.h"
 #include "kernels/allocation.h"
 #include "kernels/attention_kernels.h"
@@ -16,6 +17,9 @@
 #include "kernels/optimizer_kernels.h"
 #include "kernels/profiling.h"
 #include "kernels/softmax_kernels.h"
+#include "ffk.h"
+#include "local-execution/computation_graph_instance.h"
+#include "pcg/computation_graph_builder.h"
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -163,6 +167,58 @@ static void cpu_tests() {
                               DataType::FLOAT, DataType::FLOAT, DataType::FLOAT, 4, 2)
                .has_value());
     CHECK_THROWS(linear_forward_kernel(get_cpu_device_stream(), std::nullopt, attrs, x, y, w, std::nullopt));
+  });
+  run("ComputationGraphBuilder: shape inference, weight layers, errors", [] {
+    ComputationGraphBuilder cgb;
+    tensor_guid_t ids = cgb.create_input(shape({4, 16}, DataType::INT32), CreateGrad::NO);
+    tensor_guid_t emb = cgb.embedding(ids, 1000, 64, std::nullopt, DataType::BF16);
+    CHECK(cgb.get_shape(emb) == shape({4, 16, 64}, DataType::BF16));
+    CHECK(cgb.get_shape(cgb.get_weights_of(emb).at(0)) == shape({1000, 64}, DataType::FLOAT));
+    tensor_guid_t bag = cgb.embedding(ids, 1000, 64, AggregateOp::SUM);
+    CHECK(cgb.get_shape(bag) == shape({4, 64}, DataType::FLOAT));  // embedding.cc:31-36
+    tensor_guid_t att = cgb.multihead_attention(emb, emb, emb, 64, 1, 64, 64, 0.0f, false);
+    CHECK(cgb.get_shape(att) == shape({4, 16, 64}, DataType::BF16));
+    // q, k, v projections [64 x 64] and the output projection (attention.cc:165-185)
+    CHECK(get_num_elements(cgb.get_shape(cgb.get_weights_of(att).at(0)).dims) == 4 * 64 * 64);
+    tensor_guid_t ln = cgb.layer_norm(cgb.add(att, emb), {-1}, true, 1e-5f);
+    CHECK(cgb.get_weights_of(ln).size() == 2 && cgb.get_shape(cgb.get_weights_of(ln)[0]) == shape({64}, DataType::BF16));
+    tensor_guid_t fc = cgb.dense(ln, 96, Activation::RELU, true);
+    CHECK(cgb.get_shape(fc) == shape({4, 16, 96}, DataType::BF16));
+    CHECK(cgb.get_shape(cgb.get_weights_of(fc).at(0)) == shape({96, 64}, DataType::BF16));
+    CHECK(cgb.get_shape(cgb.get_weights_of(fc).at(1)) == shape({96}, DataType::BF16));
+    CHECK(cgb.get_shape(cgb.softmax(cgb.cast(fc, DataType::FLOAT))) == shape({4, 16, 96}, DataType::FLOAT));
+    CHECK(cgb.get_weights_of(cgb.dropout(fc, 0.1f)).empty());
+    // GELU after a dense layer is a layer of its own (Linear's backward has no GELU)
+    tensor_guid_t ge = cgb.dense(ln, 96, Activation::GELU, true);
+    CHECK(std::holds_alternative<ElementUnaryAttrs>(cgb.computation_graph.layers[cgb.computation_graph.tensors[ge.raw].source.raw].attrs.op_attrs));
+    CHECK_THROWS(cgb.add(fc, ln));                                   // 96 vs 64 wide: sizes do not divide
+    CHECK_THROWS(cgb.layer_norm(fc, {0}, true, 1e-5f));              // a leading axis
+    CHECK_THROWS(cgb.embedding(fc, 10, 4, std::nullopt));            // float indices
+    CHECK_THROWS(cgb.multihead_attention(fc, ln, ln, 64, 1, 64, 64, 0.0f, false, true));  // add_bias_kv
+    CHECK_THROWS(add_layer(cgb.computation_graph,
+                           LayerAttrs{LinearAttrs{8, false, DataType::BF16, std::nullopt, std::nullopt}, std::nullopt}, {ln},
+                           {cgb.get_weights_of(fc).at(0)}));         // a weight of the wrong shape
+    ComputationGraph const &cg = cgb.computation_graph;
+    CHECK(topological_ordering(cg).size() == cg.layers.size());
+    bool producers_first = true;
+    for (size_t l = 0; l < cg.layers.size(); l++) {
+      for (tensor_guid_t t : cg.layers[l].inputs) producers_first = producers_first && cg.tensors[t.raw].source.raw < (int)l;
+      for (tensor_guid_t t : cg.layers[l].weights) producers_first = producers_first && cg.tensors[t.raw].source.raw < (int)l;
+    }
+    CHECK(producers_first);
+  });
+
+  run("get_optimizer_attrs_for_next_iter (lib/pcg/src/pcg/optimizer_attrs.cc:6-26)", [] {
+    OptimizerAttrs sgd = SGDOptimizerAttrs{0.1, 0.9, true, 0.0};
+    CHECK(std::get<SGDOptimizerAttrs>(get_optimizer_attrs_for_next_iter(sgd)).lr == 0.1);
+    AdamOptimizerAttrs a{1e-3, 0.9, 0.999, 0.0, 1e-3, 1.0, 1.0, 1e-8};
+    for (int t = 1; t <= 3; t++) {
+      a = std::get<AdamOptimizerAttrs>(get_optimizer_attrs_for_next_iter(OptimizerAttrs{a}));
+      CHECK(std::fabs(a.beta_t - std::pow(0.9, t)) < 1e-12 && std::fabs(a.beta2_t - std::pow(0.999, t)) < 1e-12);
+      CHECK(std::fabs(a.alpha_t - 1e-3 * std::sqrt(1 - std::pow(0.999, t)) / (1 - std::pow(0.9, t))) < 1e-12);
+    }
+    CHECK(get_loss_function(LossAttrs{SparseCategoricalCrossEntropyLossAttrs{false}}) == LossFunction::SPARSE_CATEGORICAL_CROSSENTROPY);
+    CHECK(get_loss_function(LossAttrs{NonconfigurableLossAttrs{LossFunction::IDENTITY}}) == LossFunction::IDENTITY);
   });
 }
 
@@ -441,16 +497,284 @@ static void gpu_tests() {
     for (int64_t i = 0; i < n; i++) want[i] += x[i];
     CHECK(to_host(DX) == want);
   });
+  // lib/local-execution/test/src/local-execution/computation_graph_instance.cc:33-189
+  // (CUDA twin :192-355): the same graph, loss, optimizer and assertion, and the
+  // same five steps replayed with the CPU oracle.
+  run("LocalBackend e2e Training: 2-layer MLP, categorical CE, SGD with momentum, 5 steps", [&] {
+    int64_t batch = 10, data_dim = 16, hidden_dim = 32, output_dim = 1;
+    ComputationGraph cg = make_empty_computation_graph();
+    tensor_guid_t t_input = add_input_layer(cg, shape({batch, data_dim}, DataType::FLOAT)).outputs.at(0);
+    tensor_guid_t t_w1 = add_weight_layer(cg, shape({hidden_dim, data_dim}, DataType::FLOAT)).outputs.at(0);
+    tensor_guid_t t_w2 = add_weight_layer(cg, shape({output_dim, hidden_dim}, DataType::FLOAT)).outputs.at(0);
+    tensor_guid_t t_l1 = add_layer(cg, LayerAttrs{LinearAttrs{(int)hidden_dim, false, DataType::FLOAT, Activation::RELU, std::nullopt}, std::nullopt},
+                                   {t_input}, {t_w1}).outputs.at(0);
+    tensor_guid_t t_l2 = add_layer(cg, LayerAttrs{LinearAttrs{(int)output_dim, false, DataType::FLOAT, Activation::RELU, std::nullopt}, std::nullopt},
+                                   {t_l1}, {t_w2}).outputs.at(0);
+    auto x = random_vec(batch * data_dim, 30), w1 = random_vec(hidden_dim * data_dim, 31, -0.3f, 0.5f),
+         w2 = random_vec(output_dim * hidden_dim, 32, 0.0f, 0.5f);
+    std::vector<float> label(batch * output_dim, 0.0f);
+    auto LABEL = device_accessor(gpu, shape({batch, output_dim}, DataType::FLOAT), label);
+    OptimizerAttrs optimizer = SGDOptimizerAttrs{0.001, 0.9, false, 0.001};
+    device_id_t device_idx = make_device_id_t_from_idx(0, DeviceType::GPU);
+    ComputationGraphInstance instance = create_computation_graph_instance(
+        cg, optimizer, LossConfig{NonconfigurableLossAttrs{LossFunction::CATEGORICAL_CROSSENTROPY}, LABEL, t_l2}, {}, gpu,
+        ProfilingSettings{0, 0}, handle, device_idx);
+    Allocator cpu = create_local_cpu_memory_allocator();
+    auto put = [&](tensor_guid_t t, std::vector<float> const &v) {
+      GenericTensorAccessorW h = cpu.allocate_tensor(instance.get_tensor_accessor(t).shape);
+      memcpy(h.ptr, v.data(), v.size() * 4);
+      copy_accessor_data_to_l_from_r(instance.get_tensor_accessor(t), h);
+    };
+    put(t_input, x); put(t_w1, w1); put(t_w2, w2);
+
+    std::vector<float> v1(w1.size(), 0.0f), v2(w2.size(), 0.0f), h(batch * hidden_dim), y(batch), dlogit(batch),
+        dh(h.size()), dw1(w1.size()), dw2(w2.size()), first, last;
+    for (int step = 0; step < 5; step++) {
+      perform_all_passes_for_computation_graph_instance(instance, ProfilingSettings{0, 0}, handle, device_idx);
+      std::vector<float> got = to_host(GenericTensorAccessorW{instance.get_loss_tensor_accessor()->shape,
+                                                              const_cast<void *>(instance.get_loss_tensor_accessor()->ptr), DeviceType::GPU});
+      if (step == 0) first = got;
+      last = got;
+      orc_linear_forward(0, x.data(), h.data(), w1.data(), nullptr, batch, data_dim, hidden_dim);
+      orc_linear_forward(0, h.data(), y.data(), w2.data(), nullptr, batch, hidden_dim, output_dim);
+      orc_difference_loss_backward(dlogit.data(), y.data(), label.data(), batch, 1.0f / batch);
+      CHECK(close(got, dlogit, 1e-5));
+      orc_linear_backward(0, 0, y.data(), dlogit.data(), h.data(), dh.data(), w2.data(), dw2.data(), nullptr, batch, hidden_dim, output_dim);
+      orc_linear_backward(0, 0, h.data(), dh.data(), x.data(), nullptr, w1.data(), dw1.data(), nullptr, batch, data_dim, hidden_dim);
+      orc_sgd_update(0.001f, 0.9f, 0, 0.001f, dw1.data(), (int64_t)w1.size(), 1, w1.data(), v1.data());
+      orc_sgd_update(0.001f, 0.9f, 0, 0.001f, dw2.data(), (int64_t)w2.size(), 1, w2.data(), v2.data());
+    }
+    CHECK(contains_non_zero(first));
+    CHECK(close(to_host(instance.get_tensor_accessor(t_w1)), w1, 1e-5));
+    CHECK(close(to_host(instance.get_tensor_accessor(t_w2)), w2, 1e-5));
+    bool did_loss_decrease = true;  // every sample's logit gradient is <= its first-step value
+    for (size_t i = 0; i < first.size(); i++) did_loss_decrease = did_loss_decrease && last[i] <= first[i];
+    CHECK(did_loss_decrease);
+    // per-layer timings when profiling is on; FWD, LOSS, BWD, UPD all present in the order
+    auto timings = perform_forward_pass_for_computation_graph_instance(instance, ProfilingSettings{1, 2}, handle, device_idx);
+    CHECK(timings.size() == 2 && timings.begin()->second.has_value() && timings.begin()->second->value > 0.0f);
+    int n_fwd = 0, n_bwd = 0, n_upd = 0, n_loss = 0;
+    for (auto const &inv : instance.get_execution_order()) {
+      n_fwd += inv.task_type == DynamicTaskType::FWD;
+      n_bwd += inv.task_type == DynamicTaskType::BWD;
+      n_upd += inv.task_type == DynamicTaskType::UPD;
+      n_loss += inv.task_type == DynamicTaskType::LOSS;
+    }
+    CHECK(n_fwd == 2 && n_bwd == 2 && n_upd == 2 && n_loss == 1);
+    Allocator cpu_alloc = create_local_cpu_memory_allocator();
+    CHECK_THROWS(create_computation_graph_instance(cg, optimizer, std::nullopt, {}, cpu_alloc, ProfilingSettings{0, 0},
+                                                   device_handle_t::for_cpu(), make_device_id_t_from_idx(0, DeviceType::CPU)));
+  });
+
+  // The encoder layer of lib/models/src/models/transformer/transformer.cc:18-67 built through the
+  // builder (BF16), a cast and a mean-squared-error loss behind it, Adam.  One step of the
+  // instance must equal, bit for bit, the same operators called by hand with every gradient
+  // added into zeroed memory: that pins the order, the placement, which gradients are
+  // overwritten or cleared, the dropout streams and the mixed-precision update.
+  run("Transformer encoder layer from the builder: one Adam step equals the hand-sequenced operators", [&] {
+    int const B = 2, S = 24, E = 64, H = 4, FF = 256;  // head size FF / H = 64
+    float const rate = 0.1f, eps = 1e-5f;
+    ComputationGraphBuilder cgb;
+    tensor_guid_t input = cgb.create_input(shape({B, S, E}, DataType::BF16), CreateGrad::NO);
+    tensor_guid_t attn = cgb.multihead_attention(input, input, input, E, H, FF / H, FF / H, rate, false);
+    CHECK(are_tensor_guid_shapes_equivalent(cgb.computation_graph, input, attn));
+    tensor_guid_t res1 = cgb.add(attn, input);
+    tensor_guid_t norm1 = cgb.layer_norm(res1, {-1}, true, eps);
+    tensor_guid_t ff1 = cgb.dense(norm1, FF, Activation::RELU, true);
+    tensor_guid_t drop1 = cgb.dropout(ff1, rate);
+    tensor_guid_t ff2 = cgb.dense(drop1, E, std::nullopt, true);
+    tensor_guid_t drop2 = cgb.dropout(ff2, rate);
+    tensor_guid_t res2 = cgb.add(norm1, drop2);
+    tensor_guid_t norm2 = cgb.layer_norm(res2, {-1}, true, eps);
+    tensor_guid_t logits = cgb.cast(norm2, DataType::FLOAT);
+    ComputationGraph const &cg = cgb.computation_graph;
+    int64_t const n = (int64_t)B * S * E, nf = (int64_t)B * S * FF, M = B * S;
+
+    auto LABEL = device_accessor(gpu, shape({B, S, E}, DataType::FLOAT), random_vec(n, 40));
+    AdamOptimizerAttrs adam{1e-3, 0.9, 0.999, 1e-2, 1e-3, 0.9, 0.999, 1e-8};
+    device_id_t device_idx = make_device_id_t_from_idx(0, DeviceType::GPU);
+    ComputationGraphInstance inst = create_computation_graph_instance(
+        cg, OptimizerAttrs{adam}, LossConfig{NonconfigurableLossAttrs{LossFunction::MEAN_SQUARED_ERROR_AVG_REDUCE}, LABEL, logits},
+        {}, gpu, ProfilingSettings{0, 0}, handle, device_idx);
+
+    // fill the input and every weight; keep device copies for the hand-sequenced run
+    std::unordered_map<int, GenericTensorAccessorW> mine;  // tensor -> private copy
+    unsigned seed = 50;
+    auto init = [&](tensor_guid_t t, float lo, float hi) {
+      TensorShape ts = inst.get_tensor_accessor(t).shape;
+      GenericTensorAccessorW d = device_accessor(gpu, ts, random_vec((size_t)get_num_elements(ts.dims), seed++, lo, hi));
+      copy_accessor_data_to_l_from_r(inst.get_tensor_accessor(t), d);
+      mine[t.raw] = d;
+    };
+    init(input, -1.0f, 1.0f);
+    std::vector<tensor_guid_t> weights;
+    for (tensor_guid_t out : {attn, norm1, ff1, ff2, norm2}) {
+      for (tensor_guid_t w : cgb.get_weights_of(out)) {
+        weights.push_back(w);
+        bool gamma = (out == norm1 || out == norm2) && w == cgb.get_weights_of(out)[0];
+        init(w, gamma ? 0.5f : -0.2f, gamma ? 1.5f : 0.2f);
+      }
+    }
+    CHECK(weights.size() == 9);
+
+    perform_all_passes_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, device_idx);
+
+    // ---- by hand ----
+    ffk_stream_t st = stream.require_gpu();
+    auto buf = [&](std::vector<int64_t> dims, DataType t) {
+      GenericTensorAccessorW a = gpu.allocate_tensor(shape(dims, t));
+      fill_with_zeros(a);
+      return a;
+    };
+    auto W = [&](tensor_guid_t out, int i) { return mine.at(cgb.get_weights_of(out).at(i).raw); };
+    std::unordered_map<int, GenericTensorAccessorW> dW;
+    for (tensor_guid_t w : weights) dW[w.raw] = buf(mine.at(w.raw).shape.dims.ff_ordered, DataType::BF16);
+    auto G = [&](tensor_guid_t out, int i) { return dW.at(cgb.get_weights_of(out).at(i).raw); };
+    int const BT = FFK_BF16;
+    auto x = mine.at(input.raw);
+    auto a = buf({B, S, E}, DataType::BF16), r1 = buf({B, S, E}, DataType::BF16), n1 = buf({B, S, E}, DataType::BF16),
+         f1 = buf({B, S, FF}, DataType::BF16), d1 = buf({B, S, FF}, DataType::BF16), f2 = buf({B, S, E}, DataType::BF16),
+         d2 = buf({B, S, E}, DataType::BF16), r2 = buf({B, S, E}, DataType::BF16), n2 = buf({B, S, E}, DataType::BF16),
+         lf = buf({B, S, E}, DataType::FLOAT);
+    auto g_a = buf({B, S, E}, DataType::BF16), g_r1 = buf({B, S, E}, DataType::BF16), g_n1 = buf({B, S, E}, DataType::BF16),
+         g_f1 = buf({B, S, FF}, DataType::BF16), g_d1 = buf({B, S, FF}, DataType::BF16), g_f2 = buf({B, S, E}, DataType::BF16),
+         g_d2 = buf({B, S, E}, DataType::BF16), g_r2 = buf({B, S, E}, DataType::BF16), g_n2 = buf({B, S, E}, DataType::BF16),
+         g_lf = buf({B, S, E}, DataType::FLOAT), g_x = buf({B, S, E}, DataType::BF16);
+    ffk_mha_desc_t d{B, H, E, E, E, FF / H, FF / H, FF / H, E, S, S, 1.0f, 0};
+    size_t reserve_bytes = ffk_mha_reserve_bytes(&d, BT);
+    void *reserve = gpu.allocate(reserve_bytes);
+    size_t ws_bytes = std::max({ffk_linear_backward_workspace_bytes(BT, FFK_ACT_RELU, 1, M, FF),
+                                ffk_linear_backward_workspace_bytes(BT, FFK_ACT_NONE, 1, M, E),
+                                ffk_layer_norm_backward_workspace_bytes(M, E)});
+    void *ws = gpu.allocate(ws_bytes);
+    auto stats = buf({4, M}, DataType::FLOAT);
+    float *mean1 = stats.get_float_ptr(), *rstd1 = mean1 + M, *mean2 = mean1 + 2 * M, *rstd2 = mean1 + 3 * M;
+    auto layer_of = [&](tensor_guid_t t) { return (uint64_t)cg.tensors.at(t.raw).source.raw; };
+    auto ok = [&](int status) { check_ffk(status, "hand-sequenced step"); };
+    ok(ffk_mha_forward(st, BT, &d, x.ptr, x.ptr, x.ptr, W(attn, 0).ptr, a.ptr, reserve, reserve_bytes));
+    ok(ffk_element_binary_forward(st, BT, FFK_OP_EW_ADD, a.ptr, x.ptr, r1.ptr, n, n, n));
+    ok(ffk_layer_norm_forward(st, BT, r1.ptr, n1.ptr, W(norm1, 0).ptr, W(norm1, 1).ptr, mean1, rstd1, M, E, eps));
+    ok(ffk_linear_forward(st, BT, FFK_ACT_RELU, n1.ptr, f1.ptr, W(ff1, 0).ptr, W(ff1, 1).ptr, M, E, FF));
+    ok(ffk_dropout_forward(st, BT, f1.ptr, d1.ptr, nf, rate, layer_of(drop1), 0));
+    ok(ffk_linear_forward(st, BT, FFK_ACT_NONE, d1.ptr, f2.ptr, W(ff2, 0).ptr, W(ff2, 1).ptr, M, FF, E));
+    ok(ffk_dropout_forward(st, BT, f2.ptr, d2.ptr, n, rate, layer_of(drop2), 0));
+    ok(ffk_element_binary_forward(st, BT, FFK_OP_EW_ADD, n1.ptr, d2.ptr, r2.ptr, n, n, n));
+    ok(ffk_layer_norm_forward(st, BT, r2.ptr, n2.ptr, W(norm2, 0).ptr, W(norm2, 1).ptr, mean2, rstd2, M, E, eps));
+    ok(ffk_cast_forward(st, BT, FFK_FLOAT, n2.ptr, lf.ptr, n));
+    ok(ffk_mean_squared_error_avg_loss_backward(st, g_lf.get_float_ptr(), lf.get_float_ptr(), LABEL.get_float_ptr(), n, n, 2.0f / n));
+    ok(ffk_cast_backward(st, FFK_FLOAT, BT, g_lf.ptr, g_n2.ptr, n));
+    ok(ffk_layer_norm_backward(st, BT, g_n2.ptr, r2.ptr, mean2, rstd2, W(norm2, 0).ptr, g_r2.ptr, G(norm2, 0).ptr, G(norm2, 1).ptr, M, E, ws, ws_bytes, 1));
+    ok(ffk_element_binary_backward(st, BT, FFK_OP_EW_ADD, g_r2.ptr, n1.ptr, d2.ptr, g_n1.ptr, g_d2.ptr, n, 1));
+    ok(ffk_dropout_backward(st, BT, g_d2.ptr, g_f2.ptr, n, rate, layer_of(drop2), 0, 1));
+    ok(ffk_linear_backward(st, BT, FFK_ACT_NONE, 0, f2.ptr, g_f2.ptr, d1.ptr, g_d1.ptr, W(ff2, 0).ptr, G(ff2, 0).ptr, G(ff2, 1).ptr, M, FF, E, ws, ws_bytes, FFK_ACC_ALL));
+    ok(ffk_dropout_backward(st, BT, g_d1.ptr, g_f1.ptr, nf, rate, layer_of(drop1), 0, 1));
+    ok(ffk_linear_backward(st, BT, FFK_ACT_RELU, 0, f1.ptr, g_f1.ptr, n1.ptr, g_n1.ptr, W(ff1, 0).ptr, G(ff1, 0).ptr, G(ff1, 1).ptr, M, E, FF, ws, ws_bytes, FFK_ACC_ALL));
+    ok(ffk_layer_norm_backward(st, BT, g_n1.ptr, r1.ptr, mean1, rstd1, W(norm1, 0).ptr, g_r1.ptr, G(norm1, 0).ptr, G(norm1, 1).ptr, M, E, ws, ws_bytes, 1));
+    ok(ffk_element_binary_backward(st, BT, FFK_OP_EW_ADD, g_r1.ptr, a.ptr, x.ptr, g_a.ptr, g_x.ptr, n, 1));
+    ok(ffk_mha_backward(st, BT, &d, x.ptr, g_x.ptr, x.ptr, nullptr, x.ptr, nullptr, W(attn, 0).ptr, G(attn, 0).ptr, g_a.ptr, reserve, reserve_bytes, 1));
+    ok(ffk_stream_synchronize(st));
+
+    CHECK(contains_non_zero(to_host(n2)));
+    CHECK(to_host(inst.get_tensor_accessor(norm2)) == to_host(n2));
+    CHECK(to_host(inst.get_tensor_accessor(drop1)) == to_host(d1));
+    CHECK(to_host(*inst.get_gradient_accessor(norm1)) == to_host(g_n1));
+    CHECK(to_host(*inst.get_gradient_accessor(attn)) == to_host(g_a));
+    for (tensor_guid_t w : weights) {
+      CHECK(contains_non_zero(to_host(dW.at(w.raw))));
+      CHECK(to_host(*inst.get_gradient_accessor(w)) == to_host(dW.at(w.raw)));
+    }
+    // the update: fp32 master taken from the BF16 weights, Adam on it, BF16 copy rounded out
+    for (tensor_guid_t w : weights) {
+      int64_t nw = get_num_elements(mine.at(w.raw).shape.dims);
+      auto master = buf({nw}, DataType::FLOAT), v = buf({nw}, DataType::FLOAT), m = buf({nw}, DataType::FLOAT);
+      ok(ffk_cast_forward(st, BT, FFK_FLOAT, mine.at(w.raw).ptr, master.ptr, nw));
+      ok(ffk_adam_update(st, BT, (float)adam.alpha_t, (float)adam.beta1, (float)adam.beta2, (float)adam.weight_decay,
+                         (float)adam.epsilon, dW.at(w.raw).ptr, nw, 1, master.get_float_ptr(), v.get_float_ptr(),
+                         m.get_float_ptr(), mine.at(w.raw).ptr));
+      ok(ffk_stream_synchronize(st));
+      CHECK(to_host(inst.get_tensor_accessor(w)) == to_host(mine.at(w.raw)));
+      CHECK(to_host(*inst.get_master_weight_accessor(w)) == to_host(master));
+    }
+    // attrs advanced as lib/pcg/src/pcg/optimizer_attrs.cc:6-26 does
+    AdamOptimizerAttrs next = std::get<AdamOptimizerAttrs>(inst.get_optimizer_attrs());
+    CHECK(std::fabs(next.beta_t - 0.81) < 1e-12 && std::fabs(next.beta2_t - 0.999 * 0.999) < 1e-12);
+    CHECK(std::fabs(next.alpha_t - 1e-3 * std::sqrt(1 - 0.999 * 0.999) / (1 - 0.81)) < 1e-15);
+    // a second step draws different dropout masks (offset = iteration * elements)
+    perform_forward_pass_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, device_idx);
+    CHECK(!(to_host(inst.get_tensor_accessor(drop1)) == to_host(d1)));
+  });
+}
+
+// One training step of the BASELINE encoder layer (pre-LN, GELU, dropout 0.1,
+// batch 8 x 512 tokens, d_model 1024, 16 heads, FFN 4096, BF16) run through the
+// step driver, operator by operator, with SGD.
+static void bench_step(int steps) {
+  ManagedPerDeviceFFHandle managed = initialize_single_gpu_handle(1 << 20, true);
+  device_handle_t handle = device_handle_t_from_managed_ff_handle(managed);
+  Allocator gpu = create_local_cuda_memory_allocator();
+  int const B = 8, S = 512, E = 1024, H = 16, FF = 4096;
+  ComputationGraphBuilder cgb;
+  tensor_guid_t x = cgb.create_input(shape({B, S, E}, DataType::BF16), CreateGrad::YES);
+  tensor_guid_t n1 = cgb.layer_norm(x, {-1}, true, 1e-5f);
+  tensor_guid_t att = cgb.multihead_attention(n1, n1, n1, E, H, E / H, E / H, 0.0f, false, false, false, std::nullopt, 0.125f);
+  tensor_guid_t r1 = cgb.add(x, cgb.dropout(att, 0.1f));
+  tensor_guid_t n2 = cgb.layer_norm(r1, {-1}, true, 1e-5f);
+  tensor_guid_t f1 = cgb.dense(n2, FF, Activation::GELU, true);
+  tensor_guid_t f2 = cgb.dense(cgb.dropout(f1, 0.1f), E, std::nullopt, true);
+  tensor_guid_t out = cgb.add(r1, cgb.dropout(f2, 0.1f));
+  device_id_t dev = make_device_id_t_from_idx(0, DeviceType::GPU);
+  ComputationGraphInstance inst = create_computation_graph_instance(
+      cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{1e-3, 0.0, false, 0.0}}, std::nullopt, {}, gpu,
+      ProfilingSettings{0, 0}, handle, dev);
+  unsigned seed = 1;
+  for (size_t t = 0; t < cgb.computation_graph.tensors.size(); t++) {
+    auto const &src = cgb.computation_graph.layers[cgb.computation_graph.tensors[t].source.raw];
+    bool weight = std::holds_alternative<WeightAttrs>(src.attrs.op_attrs);
+    if (!weight && tensor_guid_t{(int)t} != x) continue;
+    GenericTensorAccessorW a = inst.get_tensor_accessor(tensor_guid_t{(int)t});
+    GenericTensorAccessorW d = device_accessor(gpu, a.shape, random_vec((size_t)get_num_elements(a.shape.dims), seed++, -0.05f, 0.05f));
+    copy_accessor_data_to_l_from_r(a, d);
+    gpu.deallocate_tensor(d);
+  }
+  GenericTensorAccessorW dout = *inst.get_gradient_accessor(out);
+  GenericTensorAccessorW g = device_accessor(gpu, dout.shape, random_vec((size_t)get_num_elements(dout.shape.dims), 99));
+  copy_accessor_data_to_l_from_r(dout, g);
+  device_stream_t stream = get_gpu_device_stream();
+  auto step = [&] { perform_all_passes_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, dev); };
+  for (int i = 0; i < 3; i++) step();
+  ffEvent_t t0, t1;
+  check_ffk(ffk_event_create(&t0), "event");
+  check_ffk(ffk_event_create(&t1), "event");
+  check_ffk(ffk_event_record(t0, stream.require_gpu()), "event");
+  for (int i = 0; i < steps; i++) step();
+  check_ffk(ffk_event_record(t1, stream.require_gpu()), "event");
+  check_ffk(ffk_event_synchronize(t1), "event");
+  float ms = 0;
+  check_ffk(ffk_event_elapsed_ms(t0, t1, &ms), "event");
+  int launches = 0;
+  for (auto const &inv : inst.get_execution_order()) launches += 1, (void)inv;
+  printf("step driver, encoder layer B8 S512 d1024 h16 ffn4096 bf16, FWD+BWD+SGD: %.3f ms/step over %d steps, "
+         "%d invocations, %.1f MiB placed, %.2f M tokens/s\n",
+         ms / steps, steps, launches, inst.bytes_allocated() / 1048576.0, B * S / (ms / steps) / 1e3);
 }
 
 int main(int argc, char **argv) {
   std::string mode = argc > 1 ? argv[1] : "--cpu";
+  if (mode == "--bench-step") {
+    try {
+      bench_step(argc > 2 ? atoi(argv[2]) : 20);
+    } catch (std::exception const &e) {
+      printf("bench-step failed: %s\n", e.what());
+      return 1;
+    }
+    return 0;
+  }
   if (mode == "--cpu") {
     cpu_tests();
   } else if (mode == "--gpu") {
     gpu_tests();
   } else {
-    printf("usage: test_host --cpu | --gpu\n");
+    printf("usage: test_host --cpu | --gpu | --bench-step [steps]\n");
     return 2;
   }
   printf("%d checks, %d failed\n", g_checks, g_failed);
