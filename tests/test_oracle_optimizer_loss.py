@@ -85,3 +85,56 @@ def test_loss_backward_closed_forms(oracle):
     np.testing.assert_allclose(oracle.difference_loss_backward(logit, lab, 0.25),
                                (logit.astype(np.float64) - lab) * 0.25, rtol=1e-6, atol=1e-7)
     assert np.array_equal(oracle.identity_loss_backward((5, 3), 0.125), np.full((5, 3), 0.125, np.float32))
+
+
+def test_adam_trajectory_matches_torch_optim_adam(oracle):
+    """With epsilon = 0 the reference's form (alpha_t = alpha sqrt(1 - b2^t) / (1 - b1^t) folded
+    into the step, lib/pcg/src/pcg/optimizer_attrs.cc:6-26) is algebraically torch.optim.Adam's
+    bias-corrected step, L2 weight decay included; five steps of both must agree."""
+    import torch
+    g = rng(5)
+    w0 = g.standard_normal(200).astype(np.float32)
+    grads = [g.standard_normal(200).astype(np.float32) for _ in range(5)]
+    alpha, b1, b2, wd = 1e-2, 0.9, 0.99, 0.03
+    p = torch.nn.Parameter(torch.tensor(w0, dtype=torch.float64))
+    opt = torch.optim.Adam([p], lr=alpha, betas=(b1, b2), eps=0.0, weight_decay=wd)
+    w = w0.copy()
+    m = np.zeros(200, np.float32)
+    v = np.zeros(200, np.float32)
+    beta1_t, beta2_t = 1.0, 1.0
+    for grad in grads:
+        # the attrs as they stand after get_optimizer_attrs_for_next_iter has run t times
+        beta1_t *= b1
+        beta2_t *= b2
+        alpha_t = alpha * np.sqrt(1 - beta2_t) / (1 - beta1_t)
+        w, m, v = oracle.adam_update(w, grad, m, v, alpha_t, b1, b2, wd, 0.0)
+        p.grad = torch.tensor(grad, dtype=torch.float64)
+        opt.step()
+    np.testing.assert_allclose(w, p.detach().numpy(), rtol=2e-5, atol=2e-6)
+
+
+def test_loss_backward_is_the_gradient_of_the_loss(oracle):
+    """Autograd of the loss each kernel differentiates: cross-entropy of softmax outputs with
+    respect to the pre-softmax scores (the kernels are handed the softmax output as `logit`),
+    and the mean squared error."""
+    import torch
+    g = rng(6)
+    B, C = 9, 11
+    z = torch.tensor(g.standard_normal((B, C)), dtype=torch.float64, requires_grad=True)
+    label = g.integers(0, C, size=B)
+    torch.nn.functional.cross_entropy(z, torch.tensor(label), reduction="mean").backward()
+    probs = torch.softmax(z.detach(), dim=1).numpy().astype(np.float32)
+    got = oracle.sparse_cce_loss_backward(probs, label, B, C, 1, 1.0 / B)
+    np.testing.assert_allclose(got, z.grad.numpy(), rtol=1e-5, atol=1e-7)
+    # dense labels: soft targets that sum to one
+    soft = g.random((B, C))
+    soft /= soft.sum(axis=1, keepdims=True)
+    z.grad = None
+    (-(torch.tensor(soft) * torch.log_softmax(z, dim=1)).sum(dim=1).mean()).backward()
+    got = oracle.difference_loss_backward(probs, soft.astype(np.float32), 1.0 / B)
+    np.testing.assert_allclose(got, z.grad.numpy(), rtol=1e-5, atol=1e-7)
+    x = torch.tensor(g.standard_normal((B, C)), dtype=torch.float64, requires_grad=True)
+    target = g.standard_normal((B, C))
+    torch.nn.functional.mse_loss(x, torch.tensor(target)).backward()
+    got = oracle.difference_loss_backward(x.detach().numpy().astype(np.float32), target.astype(np.float32), 2.0 / (B * C))
+    np.testing.assert_allclose(got, x.grad.numpy(), rtol=1e-5, atol=1e-7)
