@@ -127,6 +127,8 @@ SIGNATURES = {
     "ffk_identity_loss_backward": (c_int, [c_p, c_p, c_p, c_i64, c_i64, c_f]),
     "ffk_cast_forward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_i64]),
     "ffk_cast_backward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_i64]),
+    "ffk_concat_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_int, c_i64]),
+    "ffk_concat_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_int, c_i64, c_int]),
     "ffk_embedding_forward": (c_int, [c_p, c_int, c_int, c_int, c_p, c_p, c_p, c_int, c_i64,
                                       c_i64, c_i64, c_i64]),
     "ffk_embedding_backward_workspace_bytes": (c_sz, [c_i64, c_i64]),
@@ -553,3 +555,45 @@ def encoder_layer_backward(desc, weights, grads, x, dy, dx, workspace):
                                            ctypes.byref(weights), ctypes.byref(grads), ptr(x),
                                            ptr(dy), ptr(dx), ptr(workspace), workspace.numel()))
     return dx
+
+
+def _concat_args(tensors, axis):
+    import ctypes
+    shape0 = tuple(tensors[0].shape)
+    axis = axis if axis >= 0 else len(shape0) + axis
+    num_blocks = 1
+    for d in shape0[:axis]:
+        num_blocks *= d
+    blk = []
+    for t in tensors:
+        sh = tuple(t.shape)
+        if len(sh) != len(shape0) or sh[:axis] != shape0[:axis] or sh[axis + 1:] != shape0[axis + 1:]:
+            raise ValueError("concat: shapes differ outside the axis")
+        n = 1
+        for d in sh[axis:]:
+            n *= d
+        blk.append(n)
+    ptrs = (ctypes.c_void_p * len(tensors))(*[ptr(t) for t in tensors])
+    blks = (ctypes.c_int64 * len(tensors))(*blk)
+    return axis, num_blocks, ptrs, blks
+
+
+def concat_forward(inputs, axis, out=None):
+    """out = concatenation of `inputs` (contiguous tensors of one dtype) along `axis`."""
+    torch = _torch()
+    axis, num_blocks, ptrs, blks = _concat_args(inputs, axis)
+    if out is None:
+        shape = list(inputs[0].shape)
+        shape[axis] = sum(t.shape[axis] for t in inputs)
+        out = torch.empty(shape, dtype=inputs[0].dtype, device=inputs[0].device)
+    check(lib().ffk_concat_forward(current_stream(), dtype_of(out), ptr(out), ptrs, blks, len(inputs),
+                                   num_blocks))
+    return out
+
+
+def concat_backward(out_grad, input_grads, axis, accumulate=True):
+    """input_grads[i] (+)= the slice of out_grad that input i produced."""
+    axis, num_blocks, ptrs, blks = _concat_args(input_grads, axis)
+    check(lib().ffk_concat_backward(current_stream(), dtype_of(out_grad), ptr(out_grad), ptrs, blks,
+                                    len(input_grads), num_blocks, int(accumulate)))
+    return input_grads

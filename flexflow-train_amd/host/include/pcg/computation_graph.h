@@ -58,10 +58,11 @@ struct EmbeddingAttrs {
   DataType data_type;
 };
 struct CastAttrs { DataType dtype; };
+struct ConcatAttrs { int axis; };  // relative dim
 
 using ComputationGraphOpAttrs =
     std::variant<InputAttrs, WeightAttrs, LinearAttrs, LayerNormAttrs, MultiHeadAttentionAttrs, DropoutAttrs,
-                 ElementUnaryAttrs, ElementBinaryAttrs, SoftmaxAttrs, EmbeddingAttrs, CastAttrs>;
+                 ElementUnaryAttrs, ElementBinaryAttrs, SoftmaxAttrs, EmbeddingAttrs, CastAttrs, ConcatAttrs>;
 
 struct LayerAttrs {
   ComputationGraphOpAttrs op_attrs;

@@ -48,6 +48,8 @@ struct ComputationGraphBuilder {
   tensor_guid_t dense(tensor_guid_t const &input, int outDim, std::optional<Activation> activation = std::nullopt,
                       bool use_bias = true, std::optional<std::string> const &name = std::nullopt);
   tensor_guid_t cast(tensor_guid_t const &input, DataType dtype, std::optional<std::string> const &name = std::nullopt);
+  tensor_guid_t concat(std::vector<tensor_guid_t> const &tensors, int axis,
+                       std::optional<std::string> const &name = std::nullopt);
   tensor_guid_t softmax(tensor_guid_t const &input, std::optional<int> dim = std::nullopt,
                         std::optional<std::string> const &name = std::nullopt);
   // `scale` and `causal` extend the reference's signature (its kernel fixes 1.0 / false).

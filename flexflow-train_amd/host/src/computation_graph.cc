@@ -121,6 +121,23 @@ std::vector<TensorShape> get_output_shapes(ComputationGraphOpAttrs const &attrs,
     o.data_type = a->data_type;
     return {o};
   }
+  if (auto const *a = std::get_if<ConcatAttrs>(&attrs)) {
+    // concat.cc: equal shapes outside the axis, extents add along it
+    if (in.empty()) bad("concat expects at least one input");
+    int nd = get_num_dims(in[0].dims);
+    int axis = a->axis < 0 ? nd + a->axis : a->axis;
+    if (axis < 0 || axis >= nd) bad("concat axis out of range");
+    TensorShape o = in[0];
+    o.dims.ff_ordered[axis] = 0;
+    for (TensorShape const &s : in) {
+      if (s.data_type != in[0].data_type || get_num_dims(s.dims) != nd) bad("concat: inputs differ in data type or rank");
+      for (int i = 0; i < nd; i++) {
+        if (i != axis && s.dims.ff_ordered[i] != in[0].dims.ff_ordered[i]) bad("concat: shapes differ outside the axis");
+      }
+      o.dims.ff_ordered[axis] += s.dims.ff_ordered[axis];
+    }
+    return {o};
+  }
   if (auto const *a = std::get_if<CastAttrs>(&attrs)) {
     need(1);
     TensorShape o = in[0];
@@ -321,6 +338,10 @@ tensor_guid_t ComputationGraphBuilder::dense(tensor_guid_t const &input, int out
 tensor_guid_t ComputationGraphBuilder::cast(tensor_guid_t const &input, DataType dtype,
                                             std::optional<std::string> const &name) {
   return add_op(CastAttrs{dtype}, {input}, name);
+}
+tensor_guid_t ComputationGraphBuilder::concat(std::vector<tensor_guid_t> const &tensors, int axis,
+                                              std::optional<std::string> const &name) {
+  return add_op(ConcatAttrs{axis}, tensors, name);
 }
 tensor_guid_t ComputationGraphBuilder::softmax(tensor_guid_t const &input, std::optional<int> dim,
                                                std::optional<std::string> const &name) {

@@ -269,6 +269,15 @@ ComputationGraphInstance create_computation_graph_instance(
         p.bwd.softmax_via_scratch = true;
         p.scratch_bytes = (size_t)get_size_in_bytes(shape_of(layer.inputs[0]));
       }
+    } else if (std::get_if<ConcatAttrs>(&oa)) {
+      // one switch for all parts; the same tensor twice among the inputs is added into
+      for (size_t i = 0; i < layer.inputs.size(); i++) {
+        for (size_t j = i + 1; j < layer.inputs.size(); j++) acc = acc || layer.inputs[i] == layer.inputs[j];
+      }
+      if (p.bwd.has_backward && acc && shape_of(layer.outputs[0]).data_type != DataType::FLOAT &&
+          shape_of(layer.outputs[0]).data_type != DataType::BF16) {
+        bad("concat backward adds in FLOAT or BF16 only");
+      }
     } else if (std::get_if<CastAttrs>(&oa)) {
       acc = true;  // cast_backward always adds
     } else if (std::get_if<ElementBinaryAttrs>(&oa)) {
@@ -502,6 +511,27 @@ ComputationGraphInstance create_computation_graph_instance(
         check_ffk(ffk_embedding_backward(s.require_gpu(), itype, otype, xp, dy, dw, aggr, bags, bag, dim, entries, 0,
                                          ws_bytes ? scratch : nullptr, ws_bytes),
                   "Embedding backward");
+      };
+    } else if (auto const *a = std::get_if<ConcatAttrs>(&oa)) {
+      int const type = dt(shape_of(out).data_type);
+      int nd = get_num_dims(shape_of(out).dims), axis = a->axis < 0 ? nd + a->axis : a->axis;
+      int64_t blocks = 1;
+      for (int i = 0; i < axis; i++) blocks *= shape_of(out).dims.ff_ordered[i];
+      std::vector<void const *> in_ptrs;
+      std::vector<void *> grad_ptrs;
+      std::vector<int64_t> blks;
+      for (tensor_guid_t t : layer.inputs) {
+        in_ptrs.push_back(val(t));
+        grad_ptrs.push_back(grd_or_discard(t));
+        blks.push_back(numel(t) / blocks);
+      }
+      int const parts = (int)layer.inputs.size(), accumulate = p.bwd.accumulate ? 1 : 0;
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_concat_forward(s.require_gpu(), type, y, in_ptrs.data(), blks.data(), parts, blocks), "Concat forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_concat_backward(s.require_gpu(), type, dy, grad_ptrs.data(), blks.data(), parts, blocks, accumulate),
+                  "Concat backward");
       };
     } else if (std::get_if<CastAttrs>(&oa)) {
       tensor_guid_t x = layer.inputs[0];

@@ -7,6 +7,7 @@
 #include "kernels/element_kernels.h"
 #include "kernels/embedding_kernels.h"
 #include "kernels/cast_kernels.h"
+#include "kernels/concat_kernels.h"
 #include "kernels/loss_function_kernels.h"
 #include "kernels/optimizer_kernels.h"
 #include "kernels/layer_norm_kernels.h"
@@ -573,5 +574,65 @@ void backward_kernel(device_stream_t const &stream, GenericTensorAccessorR const
 }
 
 }  // namespace Kernels::Cast
+
+namespace Kernels::Concat {
+
+// [num_blocks, blk] view of a tensor cut at `axis` (concat_kernels.cu:22-31)
+static int64_t blk_size(TensorShape const &s, ff_dim_t axis) {
+  int64_t n = 1;
+  for (int i = axis.value; i < get_num_dims(s.dims); i++) n *= s.dims.ff_ordered[i];
+  return n;
+}
+static int64_t block_count(TensorShape const &s, ff_dim_t axis) {
+  int64_t n = 1;
+  for (int i = 0; i < axis.value; i++) n *= s.dims.ff_ordered[i];
+  return n;
+}
+
+template <typename A>
+static void check_parts(char const *who, TensorShape const &whole, std::vector<A> const &parts, ff_dim_t axis) {
+  if (axis.value < 0 || axis.value >= get_num_dims(whole.dims)) throw std::runtime_error(std::string(who) + ": axis out of range");
+  int64_t sum = 0;
+  for (A const &p : parts) {
+    if (p.shape.data_type != whole.data_type) throw std::runtime_error(std::string(who) + ": data types differ");
+    if (get_num_dims(p.shape.dims) != get_num_dims(whole.dims) || block_count(p.shape, axis) != block_count(whole, axis)) {
+      throw std::runtime_error(std::string(who) + ": shapes differ outside the axis");
+    }
+    sum += blk_size(p.shape, axis);
+  }
+  if (sum != blk_size(whole, axis)) throw std::runtime_error(std::string(who) + ": the parts do not fill the concatenated tensor");
+}
+
+void forward_kernel(device_stream_t const &stream, GenericTensorAccessorW const &output,
+                    std::vector<GenericTensorAccessorR> const &inputs, ff_dim_t axis) {
+  if (!stream.is_gpu()) no_cpu("Concat::forward_kernel");
+  check_parts("Concat::forward_kernel", output.shape, inputs, axis);
+  std::vector<void const *> ptrs;
+  std::vector<int64_t> blks;
+  for (GenericTensorAccessorR const &in : inputs) {
+    ptrs.push_back(in.ptr);
+    blks.push_back(blk_size(in.shape, axis));
+  }
+  check_ffk(ffk_concat_forward(stream.require_gpu(), dt(output.shape.data_type), output.ptr, ptrs.data(), blks.data(),
+                               (int)inputs.size(), block_count(output.shape, axis)),
+            "Concat::forward_kernel");
+}
+
+void backward_kernel(device_stream_t const &stream, GenericTensorAccessorR const &output_grad,
+                     std::vector<GenericTensorAccessorW> const &input_grads, ff_dim_t axis) {
+  if (!stream.is_gpu()) no_cpu("Concat::backward_kernel");
+  check_parts("Concat::backward_kernel", output_grad.shape, input_grads, axis);
+  std::vector<void *> ptrs;
+  std::vector<int64_t> blks;
+  for (GenericTensorAccessorW const &g : input_grads) {
+    ptrs.push_back(g.ptr);
+    blks.push_back(blk_size(g.shape, axis));
+  }
+  check_ffk(ffk_concat_backward(stream.require_gpu(), dt(output_grad.shape.data_type), output_grad.ptr, ptrs.data(),
+                                blks.data(), (int)input_grads.size(), block_count(output_grad.shape, axis), 1),
+            "Concat::backward_kernel");
+}
+
+}  // namespace Kernels::Concat
 
 }  // namespace FlexFlow

@@ -8,6 +8,7 @@
 #include "kernels/allocation.h"
 #include "kernels/attention_kernels.h"
 #include "kernels/cast_kernels.h"
+#include "kernels/concat_kernels.h"
 #include "kernels/dropout_kernels.h"
 #include "kernels/element_kernels.h"
 #include "kernels/embedding_kernels.h"
@@ -702,6 +703,144 @@ static void gpu_tests() {
     // a second step draws different dropout masks (offset = iteration * elements)
     perform_forward_pass_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, device_idx);
     CHECK(!(to_host(inst.get_tensor_accessor(drop1)) == to_host(d1)));
+  });
+  // lib/kernels/test/src/test_concat_kernel.cc:8-117: four inputs, axis 0 and axis 1
+  run("Concat forward/backward equal the oracle (the reference test's shapes)", [&] {
+    for (int axis = 0; axis < 2; axis++) {
+      int64_t rows = axis == 0 ? 2 : 4, cols = axis == 0 ? 4 : 2;
+      TensorShape in_shape = shape({rows, cols}, DataType::FLOAT);
+      TensorShape out_shape = axis == 0 ? shape({4 * rows, cols}, DataType::FLOAT) : shape({rows, 4 * cols}, DataType::FLOAT);
+      std::vector<std::vector<float>> host;
+      std::vector<GenericTensorAccessorR> ins;
+      std::vector<GenericTensorAccessorW> grads;
+      std::vector<float const *> hp;
+      for (int i = 0; i < 4; i++) {
+        host.push_back(random_vec(rows * cols, 60 + i));
+        ins.push_back(device_accessor(gpu, in_shape, host.back()));
+        grads.push_back(gpu.allocate_tensor(in_shape));
+        fill_with_zeros(grads.back());
+      }
+      for (auto const &h : host) hp.push_back(h.data());
+      int64_t blocks = axis == 0 ? 1 : rows, blk = axis == 0 ? rows * cols : cols;
+      std::vector<int64_t> blks(4, blk);
+      std::vector<float> want(4 * rows * cols);
+      orc_concat_forward(want.data(), hp.data(), blks.data(), 4, blocks);
+      auto OUT = gpu.allocate_tensor(out_shape);
+      Kernels::Concat::forward_kernel(stream, OUT, ins, ff_dim_t{axis});
+      CHECK(contains_non_zero(to_host(OUT)));
+      CHECK(to_host(OUT) == want);
+      Kernels::Concat::backward_kernel(stream, OUT, grads, ff_dim_t{axis});
+      for (int i = 0; i < 4; i++) CHECK(to_host(grads[i]) == host[i]);  // split of the concatenation, added to zero
+      CHECK_THROWS(Kernels::Concat::forward_kernel(stream, OUT, {ins[0], ins[1]}, ff_dim_t{axis}));
+    }
+  });
+
+  // The graph of lib/models/src/models/dlrm/dlrm.cc:76-172 at a small size: embedding bags
+  // (summed, BF16 out, cast to FLOAT), a bottom MLP on the dense features, the CAT
+  // interaction, a top MLP; mean-squared-error loss, SGD.  One step against the oracle.
+  run("DLRM-shaped graph (embedding bags, cast, concat, MLPs): one SGD step vs oracle", [&] {
+    int64_t const B = 24, bag = 3, V = 50, D = 16, dense_in = 13, top = 32;
+    int const tables = 3;
+    ComputationGraphBuilder cgb;
+    std::vector<tensor_guid_t> sparse, emb;
+    for (int i = 0; i < tables; i++) {
+      sparse.push_back(cgb.create_input(shape({B, bag}, DataType::INT64), CreateGrad::YES));
+    }
+    tensor_guid_t dense = cgb.create_input(shape({B, dense_in}, DataType::FLOAT), CreateGrad::YES);
+    tensor_guid_t bottom = cgb.dense(dense, (int)D, Activation::RELU, true);
+    for (int i = 0; i < tables; i++) {
+      emb.push_back(cgb.cast(cgb.embedding(sparse[i], (int)V, (int)D, AggregateOp::SUM, DataType::BF16), DataType::FLOAT));
+    }
+    std::vector<tensor_guid_t> cat_in = {bottom};
+    cat_in.insert(cat_in.end(), emb.begin(), emb.end());
+    tensor_guid_t interact = cgb.concat(cat_in, 1);
+    CHECK(cgb.get_shape(interact) == shape({B, D * (tables + 1)}, DataType::FLOAT));
+    tensor_guid_t hidden = cgb.dense(interact, (int)top, Activation::RELU, true);
+    tensor_guid_t out = cgb.dense(hidden, 1, Activation::RELU, true);
+
+    auto label = random_vec(B, 70, 0.0f, 1.0f);
+    auto LABEL = device_accessor(gpu, shape({B, 1}, DataType::FLOAT), label);
+    device_id_t dev = make_device_id_t_from_idx(0, DeviceType::GPU);
+    float const lr = 0.05f;
+    ComputationGraphInstance inst = create_computation_graph_instance(
+        cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{lr, 0.0, false, 0.0}},
+        LossConfig{NonconfigurableLossAttrs{LossFunction::MEAN_SQUARED_ERROR_AVG_REDUCE}, LABEL, out}, {}, gpu,
+        ProfilingSettings{0, 0}, handle, dev);
+
+    Allocator cpu = create_local_cpu_memory_allocator();
+    auto put = [&](tensor_guid_t t, std::vector<float> const &v) {
+      GenericTensorAccessorW d = device_accessor(gpu, inst.get_tensor_accessor(t).shape, v);
+      copy_accessor_data_to_l_from_r(inst.get_tensor_accessor(t), d);
+    };
+    std::vector<std::vector<int64_t>> idx(tables, std::vector<int64_t>(B * bag));
+    std::mt19937 gen(7);
+    for (int i = 0; i < tables; i++) {
+      for (auto &v : idx[i]) v = gen() % V;
+      GenericTensorAccessorW h = cpu.allocate_tensor(shape({B, bag}, DataType::INT64));
+      memcpy(h.ptr, idx[i].data(), idx[i].size() * 8);
+      copy_accessor_data_to_l_from_r(inst.get_tensor_accessor(sparse[i]), h);
+    }
+    auto x = random_vec(B * dense_in, 71);
+    put(dense, x);
+    auto wb = random_vec(D * dense_in, 72, -0.4f, 0.4f), bb = random_vec(D, 73, 0.0f, 0.2f);
+    auto wh = random_vec(top * D * (tables + 1), 74, -0.2f, 0.2f), bh = random_vec(top, 75, 0.0f, 0.2f);
+    auto wo = random_vec(top, 76, 0.0f, 0.3f), bo = random_vec(1, 77, 0.1f, 0.2f);
+    put(cgb.get_weights_of(bottom)[0], wb); put(cgb.get_weights_of(bottom)[1], bb);
+    put(cgb.get_weights_of(hidden)[0], wh); put(cgb.get_weights_of(hidden)[1], bh);
+    put(cgb.get_weights_of(out)[0], wo); put(cgb.get_weights_of(out)[1], bo);
+    std::vector<std::vector<float>> table(tables);
+    std::vector<tensor_guid_t> table_guid;
+    for (int i = 0; i < tables; i++) {
+      table[i] = random_vec(V * D, 80 + i, -0.5f, 0.5f);
+      table_guid.push_back(cgb.computation_graph.layers[cgb.computation_graph.tensors[emb[i].raw].source.raw].inputs[0]);
+      table_guid[i] = cgb.get_weights_of(table_guid[i])[0];
+      put(table_guid[i], table[i]);
+    }
+
+    perform_all_passes_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, dev);
+
+    // oracle
+    int64_t const W = D * (tables + 1);
+    std::vector<float> bot(B * D), cat(B * W), hid(B * top), y(B), dy(B), dhid(B * top), dcat(B * W), dbot(B * D), dx(B * dense_in);
+    std::vector<std::vector<float>> e(tables, std::vector<float>(B * D)), de(tables, std::vector<float>(B * D));
+    orc_linear_forward(0, x.data(), bot.data(), wb.data(), bb.data(), B, dense_in, D);
+    for (int i = 0; i < tables; i++) {
+      orc_embedding_forward(idx[i].data(), e[i].data(), table[i].data(), 0, B, bag, D, V);
+      orc_round_bf16_array(e[i].data(), e[i].size());
+    }
+    std::vector<float const *> parts = {bot.data()};
+    for (auto const &v : e) parts.push_back(v.data());
+    std::vector<int64_t> blks(tables + 1, D);
+    orc_concat_forward(cat.data(), parts.data(), blks.data(), tables + 1, B);
+    orc_linear_forward(0, cat.data(), hid.data(), wh.data(), bh.data(), B, W, top);
+    orc_linear_forward(0, hid.data(), y.data(), wo.data(), bo.data(), B, top, 1);
+    CHECK(close(to_host(inst.get_tensor_accessor(interact)), cat, 1e-5));
+    CHECK(close(to_host(inst.get_tensor_accessor(out)), y, 1e-5) && contains_non_zero(y));
+    orc_difference_loss_backward(dy.data(), y.data(), label.data(), B, 2.0f / B);
+    std::vector<float> dwo(wo.size()), dbo(1), dwh(wh.size()), dbh(top), dwb(wb.size()), dbb(D);
+    orc_linear_backward(0, 0, y.data(), dy.data(), hid.data(), dhid.data(), wo.data(), dwo.data(), dbo.data(), B, top, 1);
+    orc_linear_backward(0, 0, hid.data(), dhid.data(), cat.data(), dcat.data(), wh.data(), dwh.data(), dbh.data(), B, W, top);
+    std::vector<float *> dparts = {dbot.data()};
+    for (auto &v : de) dparts.push_back(v.data());
+    orc_concat_backward(dcat.data(), dparts.data(), blks.data(), tables + 1, B, 0);
+    orc_linear_backward(0, 0, bot.data(), dbot.data(), x.data(), dx.data(), wb.data(), dwb.data(), dbb.data(), B, dense_in, D);
+    CHECK(close(to_host(*inst.get_gradient_accessor(cgb.get_weights_of(hidden)[0])), dwh, 1e-5));
+    CHECK(close(to_host(*inst.get_gradient_accessor(cgb.get_weights_of(bottom)[0])), dwb, 1e-5));
+    CHECK(close(to_host(*inst.get_gradient_accessor(cgb.get_weights_of(bottom)[1])), dbb, 1e-5));
+    CHECK(close(to_host(*inst.get_gradient_accessor(dense)), dx, 1e-5));
+    for (int i = 0; i < tables; i++) {
+      // the cast's backward rounds the gradient to BF16 before the scatter-add, so an fp32
+      // last-bit difference upstream can move an addend by one BF16 step: BF16 tolerance
+      orc_round_bf16_array(de[i].data(), de[i].size());
+      std::vector<float> dtab(V * D, 0.0f);
+      orc_embedding_backward_f64(idx[i].data(), de[i].data(), dtab.data(), 0, B, bag, D, V);
+      CHECK(contains_non_zero(dtab));
+      CHECK(close(to_host(*inst.get_gradient_accessor(table_guid[i])), dtab, 2e-2));
+      for (size_t j = 0; j < dtab.size(); j++) table[i][j] -= lr * dtab[j];
+      CHECK(close(to_host(inst.get_tensor_accessor(table_guid[i])), table[i], 1e-4));
+    }
+    for (size_t j = 0; j < wh.size(); j++) wh[j] -= lr * dwh[j];
+    CHECK(close(to_host(inst.get_tensor_accessor(cgb.get_weights_of(hidden)[0])), wh, 1e-5));
   });
 }
 

@@ -497,6 +497,27 @@ int ffk_cast_backward(ffk_stream_t stream, int output_grad_dtype,
                       int input_grad_dtype, void const *output_grad,
                       void *input_grad, int64_t num_elements);
 
+/* ------------------------------------------------------------------------ */
+/* Concat -- Kernels::Concat::gpu_forward_kernel / gpu_backward_kernel
+ * (lib/kernels/include/kernels/concat_kernels.h:9-17; lib/kernels/src/cuda/
+ * ops/concat_kernels.cu:22-97).  With the concatenation axis at position a,
+ * num_blocks = product of the dims before a and input_blk_elems[i] = product
+ * of input i's dims from a on; the output row is the inputs' rows one after
+ * another.  All inputs move in one launch (any number of inputs, any data
+ * type; pointer arrays are host memory).
+ * backward: input_grads[i] (+)= the matching slice of output_grad; the
+ *   reference adds (add_with_stride) = accumulate 1 (float and bf16 only),
+ *   accumulate 0 overwrites (any data type).                                 */
+/* ------------------------------------------------------------------------ */
+int ffk_concat_forward(ffk_stream_t stream, int dtype, void *output,
+                       void const *const *inputs,
+                       int64_t const *input_blk_elems, int num_inputs,
+                       int64_t num_blocks);
+int ffk_concat_backward(ffk_stream_t stream, int dtype, void const *output_grad,
+                        void *const *input_grads,
+                        int64_t const *input_blk_elems, int num_inputs,
+                        int64_t num_blocks, int accumulate);
+
 #ifdef __cplusplus
 }
 #endif

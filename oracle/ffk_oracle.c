@@ -59,6 +59,13 @@
  *      no reference test (PARITY UNPINNED there); pinned by the closed forms
  *      (gradient of mean softmax-cross-entropy w.r.t. the softmax output path
  *      the reference uses: logit - onehot, times the scale).
+ *      Also pinned by a five-step trajectory against torch.optim.Adam with
+ *      epsilon = 0 (where the two forms coincide) and, for the losses, by
+ *      autograd of the loss each kernel differentiates.
+ *  orc_concat_*               src/cuda/ops/concat_kernels.cu:22-97 with
+ *      copy_with_stride / add_with_stride (src/cuda/cuda_helper.cu:160-173).
+ *      The reference's test only asserts non-zero output (PARITY UNPINNED
+ *      there); pinned by numpy.concatenate and by split-after-concat.
  *  orc_cast_*                 src/kernels/cast_kernels_cpu.cc:6-20
  *      the reference tests only compare its GPU and CPU kernels on random
  *      data; pinned by numpy astype on exactly representable values and on
@@ -1047,5 +1054,45 @@ void orc_difference_loss_backward(float *dlogit, float const *logit,
 void orc_identity_loss_backward(float *dloss, int64_t volume, float scale_factor) {
   for (int64_t i = 0; i < volume; i++) {
     dloss[i] = 1.0f * scale_factor;
+  }
+}
+
+/* ------------------------------------------------------------------ concat */
+void orc_concat_forward(float *out, float const *const *in, int64_t const *blk,
+                        int n, int64_t num_blocks) {
+  int64_t out_blk = 0;
+  for (int i = 0; i < n; i++) {
+    out_blk += blk[i];
+  }
+  int64_t offset = 0;
+  for (int i = 0; i < n; i++) {
+    /* copy_with_stride(output + offset, input, num_blocks, out_blk, blk[i]) */
+    for (int64_t b = 0; b < num_blocks; b++) {
+      for (int64_t j = 0; j < blk[i]; j++) {
+        out[b * out_blk + offset + j] = in[i][b * blk[i] + j];
+      }
+    }
+    offset += blk[i];
+  }
+}
+
+void orc_concat_backward(float const *dout, float *const *din,
+                         int64_t const *blk, int n, int64_t num_blocks,
+                         int accumulate) {
+  int64_t out_blk = 0;
+  for (int i = 0; i < n; i++) {
+    out_blk += blk[i];
+  }
+  int64_t offset = 0;
+  for (int i = 0; i < n; i++) {
+    /* add_with_stride(input_grad, output_grad + offset, ...) */
+    for (int64_t b = 0; b < num_blocks; b++) {
+      for (int64_t j = 0; j < blk[i]; j++) {
+        float g = dout[b * out_blk + offset + j];
+        float *d = &din[i][b * blk[i] + j];
+        *d = accumulate ? *d + g : g;
+      }
+    }
+    offset += blk[i];
   }
 }

@@ -153,6 +153,13 @@ void orc_difference_loss_backward(float *dlogit, float const *logit,
                                   float scale_factor);
 void orc_identity_loss_backward(float *dloss, int64_t volume, float scale_factor);
 
+/* ---- Concat: out [num_blocks, sum blk], in[i] [num_blocks, blk[i]] ---- */
+void orc_concat_forward(float *out, float const *const *in, int64_t const *blk,
+                        int n, int64_t num_blocks);
+void orc_concat_backward(float const *dout, float *const *din,
+                         int64_t const *blk, int n, int64_t num_blocks,
+                         int accumulate);
+
 #ifdef __cplusplus
 }
 #endif

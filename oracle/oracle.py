@@ -401,3 +401,36 @@ def cast(x, out_dtype):
     """static_cast element by element (cast_kernels_cpu.cc:6-11); numpy's astype
     is the same conversion for the type pairs used here."""
     return np.ascontiguousarray(x).astype(out_dtype)
+
+
+def _concat_blocks(shapes, axis):
+    axis = axis if axis >= 0 else len(shapes[0]) + axis
+    num_blocks = int(np.prod(shapes[0][:axis], dtype=np.int64))
+    blk = [int(np.prod(sh[axis:], dtype=np.int64)) for sh in shapes]
+    return axis, num_blocks, blk
+
+
+def concat_forward(inputs, axis):
+    """concat_kernels.cu:36-66: every input is copied into its column window of the
+    [num_blocks, sum blk] view of the output."""
+    ins = [_f32(a) for a in inputs]
+    axis, num_blocks, blk = _concat_blocks([a.shape for a in ins], axis)
+    shape = list(ins[0].shape)
+    shape[axis] = sum(a.shape[axis] for a in ins)
+    out = np.empty(shape, np.float32)
+    ptrs = (ctypes.c_void_p * len(ins))(*[a.ctypes.data for a in ins])
+    blks = (c_i64 * len(ins))(*blk)
+    lib().orc_concat_forward(_p(out), ptrs, blks, ctypes.c_int(len(ins)), c_i64(num_blocks))
+    return out
+
+
+def concat_backward(out_grad, input_grads, axis, accumulate=True):
+    """Returns the new input gradients (concat_kernels.cu:68-97 adds into them)."""
+    g = _f32(out_grad)
+    dins = [_f32(a).copy() for a in input_grads]
+    axis, num_blocks, blk = _concat_blocks([a.shape for a in dins], axis)
+    ptrs = (ctypes.c_void_p * len(dins))(*[a.ctypes.data for a in dins])
+    blks = (c_i64 * len(dins))(*blk)
+    lib().orc_concat_backward(_p(g), ptrs, blks, ctypes.c_int(len(dins)), c_i64(num_blocks),
+                              ctypes.c_int(1 if accumulate else 0))
+    return dins
