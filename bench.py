@@ -44,7 +44,8 @@ def make_device_state(ffk, torch, cfg):
     gen = torch.Generator(device="cuda").manual_seed(1)
     desc = ffk.EncoderLayerDesc(cfg["batch"], cfg["seq"], cfg["d_model"], cfg["heads"], cfg["d_ff"],
                                 cfg["p"], cfg["seed"], cfg["eps"], cfg["scale"], int(cfg["causal"]),
-                                int(cfg["pre_ln"]), ffk.ACT_GELU if cfg["gelu"] else ffk.ACT_RELU)
+                                int(cfg["pre_ln"]), ffk.ACT_GELU if cfg["gelu"] else ffk.ACT_RELU,
+                                1)  # every weight gradient is stored, not added: nothing to clear per step
     shapes = ffk.encoder_layer_param_shapes(desc)
     wt = {}
     for name, shape in shapes.items():
@@ -52,8 +53,7 @@ def make_device_state(ffk, torch, cfg):
         if name.endswith("gamma"):
             t = t + 1.0
         wt[name] = t.to(bt)
-    # all weight gradients live in one flat buffer (16-byte aligned slices) so a
-    # training step clears them with a single fill
+    # all weight gradients live in one flat buffer (16-byte aligned slices)
     sizes = {k: (v.numel() + 7) // 8 * 8 for k, v in wt.items()}
     flat = torch.zeros((sum(sizes.values()),), dtype=bt, device="cuda")
     gt, off = {}, 0
@@ -70,10 +70,7 @@ def make_device_state(ffk, torch, cfg):
 
 
 def step(ffk, st):
-    # one training step of the layer: fresh weight gradients, forward, backward
-    g = st["grad_flat"]
-    ffk.check(ffk.lib().ffk_fill_zero(g.data_ptr(), g.numel() * g.element_size(),
-                                      ffk.current_stream()))
+    # one training step of the layer: forward, backward (which stores fresh weight gradients)
     ffk.encoder_layer_forward(st["desc"], st["W"], st["x"], st["y"], st["ws"])
     ffk.encoder_layer_backward(st["desc"], st["W"], st["G"], st["x"], st["dy"], st["dx"], st["ws"])
 

@@ -67,6 +67,7 @@ class EncoderLayerDesc(ctypes.Structure):
         ("batch", c_i64), ("seq", c_i64), ("d_model", c_i64), ("heads", c_i64), ("d_ff", c_i64),
         ("dropout_rate", c_f), ("seed", c_u64), ("ln_eps", c_f), ("attn_scale", c_f),
         ("causal", c_int), ("pre_layer_norm", c_int), ("activation", c_int),
+        ("overwrite_weight_grads", c_int),
     ]
 
 

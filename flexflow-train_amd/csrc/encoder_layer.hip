@@ -194,6 +194,8 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   bool const gelu = d->activation == FFK_ACT_GELU;
   auto mean = [&](size_t o) { return reinterpret_cast<float *>(ws + o); };
   size_t const ln_ws_bytes = L.lin_ws - L.ln_ws, lin_ws_bytes = L.total - L.lin_ws;
+  int const wacc = d->overwrite_weight_grads ? 0 : (FFK_ACC_WEIGHT | FFK_ACC_BIAS);
+  int const mha_mode = d->overwrite_weight_grads ? FFK_MHA_OVERWRITE_WEIGHT_GRAD : 0;
 
   // ---- tail: y = x1 + f2_drop (pre-LN) or y = LN2(x1 + f2_drop) (post-LN)
   void const *g_sum = dy;  // gradient of (x1 + f2_drop)
@@ -205,7 +207,7 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   // ---- FFN backward
   FFK_TRY(ffk_dropout_backward(st, dtype, g_sum, ws + L.g_f2, T * E, p, d->seed + 2, 0, 0));
   FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_NONE, 0, ws + L.f2, ws + L.g_f2, ws + L.act1_drop,
-                              ws + L.g_act1_drop, w->w2, g->w2, g->b2, T, F, E, ws + L.lin_ws, lin_ws_bytes, FFK_ACC_WEIGHT | FFK_ACC_BIAS));
+                              ws + L.g_act1_drop, w->w2, g->w2, g->b2, T, F, E, ws + L.lin_ws, lin_ws_bytes, wacc));
   void const *ffn_in = d->pre_layer_norm ? ws + L.h2 : ws + L.x1;
   bool const fuse_gelu_bwd = gelu && layer_fusion_enabled() &&
                              dropout_fusable(dtype, ws + L.g_act1_drop, ws + L.f1, ws + L.g_f1, T * F, 0);
@@ -221,10 +223,10 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
                                          ws + L.g_f1, T * F, 0));
     }
     FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_NONE, 0, ws + L.f1, ws + L.g_f1, ffn_in, ws + L.g_h2,
-                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws, lin_ws_bytes, FFK_ACC_WEIGHT | FFK_ACC_BIAS));
+                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws, lin_ws_bytes, wacc));
   } else {
     FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_RELU, 0, ws + L.act1, ws + L.g_act1, ffn_in, ws + L.g_h2,
-                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws, lin_ws_bytes, FFK_ACC_WEIGHT | FFK_ACC_BIAS));
+                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws, lin_ws_bytes, wacc));
   }
   // ---- gradient reaching x1
   if (d->pre_layer_norm) {
@@ -251,7 +253,7 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
     FFK_TRY(ffk_dropout_backward(st, dtype, g_attn_res, ws + L.g_attn, T * E, p, d->seed + 0, 0, 0));
     FFK_TRY(ffk_mha_backward(st, dtype, &m, ws + L.h1, ws + L.g_h1, ws + L.h1, nullptr, ws + L.h1, nullptr,
                              w->attn_weight, g->attn_weight, ws + L.g_attn, ws + L.mha_reserve,
-                             L.ln_ws - L.mha_reserve, 0));
+                             L.ln_ws - L.mha_reserve, mha_mode));
     // dx = LN1_backward(g_h1) + g_x1
     int rc = FFK_ERR_UNSUPPORTED;
     if (layer_fusion_enabled()) {
@@ -270,7 +272,7 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
                                     ws + L.g_attn, g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
     g_attn_res = ws + L.g_attn;
     FFK_TRY(ffk_mha_backward(st, dtype, &m, x, dx, x, nullptr, x, nullptr, w->attn_weight, g->attn_weight,
-                             g_attn_res, ws + L.mha_reserve, L.ln_ws - L.mha_reserve, 0));
+                             g_attn_res, ws + L.mha_reserve, L.ln_ws - L.mha_reserve, mha_mode));
     FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, dx, g_attn_res, dx, T * E, T * E, T * E));
   }
   return FFK_OK;

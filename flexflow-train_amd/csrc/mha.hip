@@ -179,8 +179,8 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
   uint8_t *qkv = rs + L.off_qkv, *dqkv = rs + L.off_dqkv;
   uint8_t *ctx = rs + L.off_ctx, *dctx = rs + L.off_dctx;
   GemmEpilogue over, acc, in_ep;
-  acc.accumulate = true;
-  in_ep.accumulate = accumulate != 0;
+  acc.accumulate = (accumulate & FFK_MHA_OVERWRITE_WEIGHT_GRAD) == 0;
+  in_ep.accumulate = (accumulate & FFK_MHA_ACC_INPUT_GRADS) != 0;
 
   // d(context) = dOut . W_O ; dW_O += dOut^T . context
   rc = gemm_dispatch(st, dtype, false, false, L.TQ, HD, d->o_proj_size, output_grad,

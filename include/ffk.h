@@ -354,7 +354,10 @@ int ffk_attention_backward(ffk_stream_t stream, int dtype,
  *   key_grad/value_grad may be NULL when key/value alias query (their
  *   gradients are then folded into query_grad, as the reference's task impl
  *   expects, lib/task-spec/src/task-spec/ops/impl/attention.cc:129-133);
- *   weight_grad is accumulated into (CUDNN_WGRAD_MODE_ADD).                  */
+ *   weight_grad is accumulated into (CUDNN_WGRAD_MODE_ADD).  `accumulate` is
+ *   0 / 1 as just described, optionally or-ed with
+ *   FFK_MHA_OVERWRITE_WEIGHT_GRAD to store the weight gradient instead of
+ *   adding it (a caller that would otherwise clear it first).                */
 /* ------------------------------------------------------------------------ */
 typedef struct {
   int64_t num_samples, num_heads;
@@ -365,6 +368,7 @@ typedef struct {
   int causal;  /* reference: 0   */
 } ffk_mha_desc_t;
 
+enum { FFK_MHA_ACC_INPUT_GRADS = 1, FFK_MHA_OVERWRITE_WEIGHT_GRAD = 2 };
 size_t ffk_mha_weight_elements(ffk_mha_desc_t const *desc);
 size_t ffk_mha_reserve_bytes(ffk_mha_desc_t const *desc, int dtype);
 int ffk_mha_forward(ffk_stream_t stream, int dtype, ffk_mha_desc_t const *desc,
@@ -394,8 +398,9 @@ int ffk_mha_backward(ffk_stream_t stream, int dtype, ffk_mha_desc_t const *desc,
  *   ElementUnary op).  MHA: heads x (d_model/heads), no bias, `attn_scale`,
  *   `causal`.  Dropout op i uses seed + i.
  * Tensors: x, y, dy, dx [batch*seq, d_model]; weights as named.  Weight
- * gradients are accumulated into (zero them for a fresh step); dx is
- * overwritten.  The workspace keeps every saved activation between the two
+ * gradients are accumulated into (zero them for a fresh step) unless
+ * overwrite_weight_grads is set, in which case every one of them is stored
+ * and nothing needs clearing; dx is overwritten.  The workspace keeps every saved activation between the two
  * calls.                                                                     */
 /* ------------------------------------------------------------------------ */
 typedef struct {
@@ -407,6 +412,7 @@ typedef struct {
   int causal;
   int pre_layer_norm;
   int activation;
+  int overwrite_weight_grads; /* 0: add into the weight gradients (reference GPU semantics) */
 } ffk_encoder_layer_desc_t;
 
 typedef struct {

@@ -18,12 +18,14 @@ def say(*a):
     sys.stdout.flush()
 
 
-def run_device(ffk, cfg, params, x, dy):
+def run_device(ffk, cfg, params, x, dy, overwrite_weight_grads=False):
     desc = ffk.EncoderLayerDesc(cfg["batch"], cfg["seq"], cfg["d_model"], cfg["heads"], cfg["d_ff"],
                                 cfg["p"], cfg["seed"], cfg["eps"], cfg["scale"], int(cfg["causal"]),
-                                int(cfg["pre_ln"]), ffk.ACT_GELU if cfg["gelu"] else ffk.ACT_RELU)
+                                int(cfg["pre_ln"]), ffk.ACT_GELU if cfg["gelu"] else ffk.ACT_RELU,
+                                int(overwrite_weight_grads))
     wt = {k: to_dev(v, torch, BT) for k, v in params.items()}
-    gt = {k: torch.zeros_like(v) for k, v in wt.items()}
+    # storing mode must not care what the gradient tensors hold
+    gt = {k: (torch.full_like(v, 3.0) if overwrite_weight_grads else torch.zeros_like(v)) for k, v in wt.items()}
     xd, dyd = to_dev(x, torch, BT), to_dev(dy, torch, BT)
     y, dx = torch.empty_like(xd), torch.empty_like(xd)
     ws = ffk.encoder_layer_workspace(desc, ffk.BF16)
@@ -132,3 +134,22 @@ def test_split_k_weight_gradient_matches_unsplit(ffk, monkeypatch):
     wo_split = g_split["attn_weight"][3 * E * E:]
     assert np.abs(wo_plain).max() > 0
     assert_close(wo_split, wo_plain, 1e-2, "dW_O split-K vs unsplit")
+
+
+@pytest.mark.parametrize("pre_ln,gelu", [(True, True), (False, False)])
+def test_stored_weight_gradients_equal_added_into_zero(ffk, pre_ln, gelu):
+    """overwrite_weight_grads stores every weight gradient: the same bits as adding into
+    cleared tensors, whatever the tensors held before."""
+    cfg = dict(batch=2, seq=48, d_model=128, heads=2, d_ff=256, p=0.1, seed=99, eps=1e-5,
+               scale=1.0 / 8.0, causal=False, pre_ln=pre_ln, gelu=gelu)
+    say("stored weight gradients", cfg)
+    g = rng(23)
+    params = make_params(g, cfg, bf16_round)
+    x = bf16_round(g.standard_normal((cfg["batch"], cfg["seq"], cfg["d_model"])))
+    dy = bf16_round(g.standard_normal(x.shape))
+    y0, dx0, g0 = run_device(ffk, cfg, params, x, dy)
+    y1, dx1, g1 = run_device(ffk, cfg, params, x, dy, overwrite_weight_grads=True)
+    assert np.array_equal(y0, y1) and np.array_equal(dx0, dx1)
+    for k in g0:
+        assert np.any(g0[k] != 0), k
+        assert np.array_equal(g0[k], g1[k]), k
