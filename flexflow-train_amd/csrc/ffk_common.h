@@ -69,21 +69,18 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) {
   return __uint_as_float(bits16 << 16);
 }
-// Round-to-nearest-even fp32 -> bf16 (the single rounding point of every
-// bf16 kernel: inputs bf16 -> fp32 arithmetic -> one rounding at the store).
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) {
-    return (u >> 16) | 0x40u;  // quiet NaN
-  }
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
-}
 // Two fp32 -> packed bf16x2 in one instruction (v_cvt_pk_bf16_f32, RNE).
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   f32x2 v = {lo, hi};
   bf16x2 b = __builtin_convertvector(v, bf16x2);
   return __builtin_bit_cast(uint32_t, b);
+}
+// Round-to-nearest-even fp32 -> bf16 (the single rounding point of every
+// bf16 kernel: inputs bf16 -> fp32 arithmetic -> one rounding at the store).
+// The same hardware conversion as the packed stores, so a value rounded here
+// and a value rounded by a vector store have the same bits, NaNs included.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  return pack_bf16x2(f, 0.0f) & 0xffffu;
 }
 
 // ---- typed vector access: N elements of T <-> N floats --------------------
@@ -180,7 +177,8 @@ __device__ __forceinline__ void unpack_raw(u32x4 r, float (&v)[8], bf16 const *)
 // with the caller: returns erf(z) given e = exp(-z*z).
 __device__ __forceinline__ float erf_from_exp(float z, float e) {
   float const az = fabsf(z);
-  float const t = __frcp_rn(1.0f + 0.3275911f * az);
+  // v_rcp_f32 (1 ulp) instead of an IEEE division: the polynomial's own error is 1.5e-7
+  float const t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * az);
   float poly = 1.061405429f;
   poly = poly * t - 1.453152027f;
   poly = poly * t + 1.421413741f;
@@ -210,7 +208,7 @@ template <>
 __device__ __forceinline__ float storage_round<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ float storage_round<bf16>(float v) {
-  return bf16_bits_to_f32(f32_to_bf16_bits(v));
+  return __uint_as_float(pack_bf16x2(v, 0.0f) << 16);
 }
 
 // ---- wavefront reductions (64 lanes, DPP/shuffle based) -------------------
