@@ -107,7 +107,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
   using C = AttnCfg<D>;
   __shared__ __attribute__((aligned(16))) bf16 Ks[2][C::kBKV * C::kKStride];
   __shared__ __attribute__((aligned(16))) bf16 Vs[2][C::kBKV * C::kVStride];
-  int const t = threadIdx.x, lane = t & 63, wave = t >> 6, h32 = lane >> 5;
+  int const t = threadIdx.x, lane = t & 63, h32 = lane >> 5;
+  // the wave index as a scalar: tile-level decisions taken from it are branches, not lane masks
+  int const wave = __builtin_amdgcn_readfirstlane(t >> 6);
   // 1-D grid ordered so that, under a causal mask, the heaviest (latest) query
   // blocks of every (batch, head) are dispatched first and light ones fill the tail.
   int const nqb = (p.Sq + C::kBQ - 1) / C::kBQ;
@@ -190,23 +192,26 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
           s[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[j], 0, 0, 0);
         }
       }
-      // scale, mask, running max
+      // mask (only tiles that straddle the end of the keys or the causal diagonal), running
+      // max of the raw scores (the scale is positive, so it commutes with the max)
       bool const need_mask = (kv0 + C::kBKV > p.Skv) || (p.causal && kv0 + C::kBKV - 1 > q0 + wave * 32);
+      if (need_mask) {
+#pragma unroll
+        for (int j = 0; j < C::kBKV / 32; j++) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            int kv = kv0 + j * 32 + 8 * (r >> 2) + 4 * h32 + (r & 3);
+            if (kv >= p.Skv || (p.causal && kv > qrow)) s[j][r] = -INFINITY;
+          }
+        }
+      }
       float mx = -INFINITY;
 #pragma unroll
       for (int j = 0; j < C::kBKV / 32; j++) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          float v = s[j][r] * p.scale_log2;
-          if (need_mask) {
-            int kv = kv0 + j * 32 + 8 * (r >> 2) + 4 * h32 + (r & 3);
-            if (kv >= p.Skv || (p.causal && kv > qrow)) v = -INFINITY;
-          }
-          s[j][r] = v;
-          mx = fmaxf(mx, v);
-        }
+        for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[j][r]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
       float const m_new = fmaxf(m_run, mx);
       // m_new is finite: key 0 is visible to every query and tile 0 comes first.
       float const alpha = __builtin_amdgcn_exp2f(m_run - m_new);
@@ -217,7 +222,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
         float pv[16];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          float e = __builtin_amdgcn_exp2f(s[j][r] - m_new);
+          float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r], p.scale_log2, -m_new));
           pv[r] = e;
           sum += e;
         }
@@ -332,7 +337,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
   __shared__ __attribute__((aligned(16))) bf16 Qs[2][C::kTile * C::kStride];
   __shared__ __attribute__((aligned(16))) bf16 Gs[2][C::kTile * C::kStride];  // dO
   __shared__ __attribute__((aligned(16))) float Ls[2][C::kTile], Ds[2][C::kTile];
-  int const t = threadIdx.x, lane = t & 63, wave = t >> 6, h32 = lane >> 5;
+  int const t = threadIdx.x, lane = t & 63, h32 = lane >> 5;
+  // the wave index as a scalar: tile-level decisions taken from it are branches, not lane masks
+  int const wave = __builtin_amdgcn_readfirstlane(t >> 6);
   // key block 0 sees every query under a causal mask: heaviest first for all heads
   int const hb = blockIdx.x % (p.H * p.B);
   int const head = hb % p.H, b = hb / p.H;
@@ -401,7 +408,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
     }
     if (t < C::kTile) {
       Ls[R][t] = rl[R];
-      Ds[R][t] = rd[R];
+      Ds[R][t] = rd[R] * p.scale;  // delta * scale, so dS is one fma and one multiply per element
     }
   };
   using Set0 = std::integral_constant<int, 0>;
@@ -439,7 +446,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
         dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[kk], dp, 0, 0, 0);
       }
       float pv[16], dsv[16];
-      bool const edge = qt0 + C::kTile > p.Sq || kvrow >= p.Skv || (p.causal && kv0 + wave * 32 + 31 > qt0);
+      // wave-uniform: does any element of this wave's 32 x 32 block need masking?
+      bool const edge = qt0 + C::kTile > p.Sq || kv0 + wave * 32 + 32 > p.Skv || (p.causal && kv0 + wave * 32 + 31 > qt0);
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         // rows 8 g + 4 h + 0..3 of the tile: one 16-byte read each
@@ -448,14 +456,19 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
 #pragma unroll
         for (int e4 = 0; e4 < 4; e4++) {
           int const r = 4 * g + e4;
-          float e = __builtin_amdgcn_exp2f(s[r] * p.scale_log2 - lrow[e4]);
-          if (edge) {
-            int const qg = qt0 + 8 * g + 4 * h32 + e4;
-            bool const masked = qg >= p.Sq || kvrow >= p.Skv || (p.causal && kvrow > qg);
-            e = masked ? 0.0f : e;
-          }
+          float const e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], p.scale_log2, -lrow[e4]));
           pv[r] = e;
-          dsv[r] = e * (dp[r] - drow[e4]) * p.scale;
+          // dS = P (dP - delta) scale; Ds holds delta * scale
+          dsv[r] = e * __builtin_fmaf(dp[r], p.scale, -drow[e4]);
+        }
+      }
+      if (edge) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          int const qg = qt0 + 8 * (r >> 2) + 4 * h32 + (r & 3);
+          bool const masked = qg >= p.Sq || kvrow >= p.Skv || (p.causal && kvrow > qg);
+          pv[r] = masked ? 0.0f : pv[r];
+          dsv[r] = masked ? 0.0f : dsv[r];
         }
       }
       // dV += P^T dO ; dK += dS^T Q.  A = accumulator re-used (row = key),
@@ -504,7 +517,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
   using C = AttnBwdCfg<D>;
   __shared__ __attribute__((aligned(16))) bf16 Ks[2][C::kTile * C::kStride];
   __shared__ __attribute__((aligned(16))) bf16 Vs[2][C::kTile * C::kStride];
-  int const t = threadIdx.x, lane = t & 63, wave = t >> 6, h32 = lane >> 5;
+  int const t = threadIdx.x, lane = t & 63, h32 = lane >> 5;
+  // the wave index as a scalar: tile-level decisions taken from it are branches, not lane masks
+  int const wave = __builtin_amdgcn_readfirstlane(t >> 6);
   int const nqb = (p.Sq + C::kBlk - 1) / C::kBlk;
   int const hb = blockIdx.x % (p.H * p.B);
   int const qb = nqb - 1 - blockIdx.x / (p.H * p.B);
@@ -517,7 +532,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
   bf16 const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * D;
 
   bf16x8 qf[D / 16], gf[D / 16];
-  float lse2, delta;
+  float lse2, delta_s;  // delta_s = delta * scale
   {
     int const r = min(qrow, p.Sq - 1);
 #pragma unroll
@@ -526,7 +541,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
       gf[kk] = *reinterpret_cast<bf16x8 const *>(gp + (int64_t)r * p.o_ss + kk * 16 + h32 * 8);
     }
     lse2 = p.lse[((int64_t)b * p.H + head) * p.Sq + r] * kLog2e;
-    delta = p.delta[((int64_t)b * p.H + head) * p.Sq + r];
+    delta_s = p.delta[((int64_t)b * p.H + head) * p.Sq + r] * p.scale;
   }
   f32x16 dq[D / 32];
 #pragma unroll
@@ -595,13 +610,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
       bool const edge = kt0 + C::kTile > p.Skv || (p.causal && kt0 + C::kTile - 1 > q0 + wave * 32);
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        float e = __builtin_amdgcn_exp2f(s[r] * p.scale_log2 - lse2);
-        if (edge) {
+        float const e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], p.scale_log2, -lse2));
+        dsv[r] = e * __builtin_fmaf(dp[r], p.scale, -delta_s);
+      }
+      if (edge) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
           int const kv = kt0 + 8 * (r >> 2) + 4 * h32 + (r & 3);
           bool const masked = kv >= p.Skv || (p.causal && kv > qrow);
-          e = masked ? 0.0f : e;
+          dsv[r] = masked ? 0.0f : dsv[r];
         }
-        dsv[r] = e * (dp[r] - delta) * p.scale;
       }
       // dQ^T += K^T dS^T : A = K^T (rows d) via transposing loads, B = dS^T.
 #pragma unroll
