@@ -319,16 +319,18 @@ __device__ __forceinline__ void wait_vmcnt() {
 // orders these loads against its LDS reads itself, with wait_vmcnt and the
 // barrier.  Loads the compiler does know about stay correct: its vmcnt waits
 // count these extra, younger loads too, which only makes them stricter.
-__device__ __forceinline__ void lds_dma16(void const *g, void *lds_base) {
-  // wave-uniform by construction; readfirstlane moves it to a scalar register
-  unsigned const base = __builtin_amdgcn_readfirstlane(
-      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_base);
+__device__ __forceinline__ void lds_dma16(void const *g, unsigned lds_byte_addr) {
+  // lds_byte_addr is wave-uniform and held in a scalar register by the caller
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                :
-               : "s"(base), "v"(g)
+               : "s"(lds_byte_addr), "v"(g)
                : "memory");  // M0 is not in the clobber list (the compiler rejects
                              // reserved registers there); nothing else in these
                              // kernels uses M0 (no GDS, message or relative-move ops)
+}
+// The LDS byte address of a __shared__ object, as a scalar.
+__device__ __forceinline__ unsigned lds_address_of(void *p) {
+  return __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)p);
 }
 
 // PF = how many k-steps ahead of its use a fragment is read from LDS (PF + 1
@@ -409,18 +411,21 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   bf16 const *const panel_a = TA ? A + m0 : A + (int64_t)m0 * lda;
   bf16 const *const panel_b = TBL ? B + n0 : B + (int64_t)n0 * ldb;
 
+  // LDS destinations of the direct loads are scalar byte addresses: base + stage + chunk row
+  unsigned const smem_addr = lds_address_of(smem);
+  int const wave_s = __builtin_amdgcn_readfirstlane(wave);
   auto issue = [&](int kt, int stage) {
-    bf16 *sa = smem + stage * STAGE_ELEMS;
-    bf16 *sb = sa + A_ELEMS;
+    unsigned const sa = smem_addr + (unsigned)(stage * STAGE_ELEMS) * 2u;
+    unsigned const sb = sa + (unsigned)A_ELEMS * 2u;
     bf16 const *ga = panel_a + (TA ? (int64_t)(kt0 + kt) * BK * lda : (int64_t)(kt0 + kt) * BK);
     bf16 const *gb = panel_b + (TBL ? (int64_t)(kt0 + kt) * BK * ldb : (int64_t)(kt0 + kt) * BK);
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
-      lds_dma16(ga + i * step_a + voff_a, sa + (i * NW + wave) * 512);
+      lds_dma16(ga + i * step_a + voff_a, sa + (unsigned)(i * NW + wave_s) * 1024u);
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
-      lds_dma16(gb + i * step_b + voff_b, sb + (i * NW + wave) * 512);
+      lds_dma16(gb + i * step_b + voff_b, sb + (unsigned)(i * NW + wave_s) * 1024u);
     }
   };
 
