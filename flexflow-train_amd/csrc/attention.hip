@@ -494,21 +494,34 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
     if (it + 1 < ntiles) step(it + 1, Set1{});
   }
 
-  // dK / dV accumulators: row = key (32 per wave, 8*(r/4)+4*h+r%4), column = d.
-  bf16 *dkp = p.dk + (int64_t)b * p.k_bs + (int64_t)head * D;
-  bf16 *dvp = p.dv + (int64_t)b * p.v_bs + (int64_t)head * D;
+  // dK / dV accumulators: row = key (32 per wave, 8*(r/4)+4*h+r%4), column = d: a lane
+  // holds one column of 16 rows.  Each wave turns its 32 x D block around in LDS (the
+  // streamed tiles are done with) and writes whole 16-byte pieces of rows.
+  __syncthreads();
+  constexpr int kOutStride = D + 8;
+  bf16 *const stage = (wave < 2 ? &Qs[0][0] : &Gs[0][0]) + (wave & 1) * 32 * kOutStride;
+  static_assert(2 * 32 * kOutStride <= 2 * C::kTile * C::kStride, "staging fits the tile buffers");
+  auto write_out = [&](f32x16 const (&acc)[D / 32], bf16 *out, int64_t row_stride) {
 #pragma unroll
-  for (int i = 0; i < D / 32; i++) {
+    for (int i = 0; i < D / 32; i++) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      int const row = kv0 + wave * 32 + 8 * (r >> 2) + 4 * h32 + (r & 3);
-      int const d = i * 32 + (lane & 31);
-      if (row < p.Skv) {
-        VecIO<bf16>::store1(dkp + (int64_t)row * p.k_ss + d, dk[i][r]);
-        VecIO<bf16>::store1(dvp + (int64_t)row * p.v_ss + d, dv[i][r]);
+      for (int r = 0; r < 16; r++) {
+        int const row = 8 * (r >> 2) + 4 * h32 + (r & 3);
+        VecIO<bf16>::store1(stage + row * kOutStride + i * 32 + (lane & 31), acc[i][r]);
       }
     }
-  }
+    // LDS operations of one wave complete in order: the reads below see the writes above
+#pragma unroll
+    for (int k = 0; k < 32 * (D / 8) / 64; k++) {
+      int const c = lane + k * 64;
+      int const row = c / (D / 8), ch = c % (D / 8);
+      u32x4 const v = *reinterpret_cast<u32x4 const *>(stage + row * kOutStride + ch * 8);
+      int const grow = kv0 + wave * 32 + row;
+      if (grow < p.Skv) *reinterpret_cast<u32x4 *>(out + (int64_t)grow * row_stride + ch * 8) = v;
+    }
+  };
+  write_out(dk, p.dk + (int64_t)b * p.k_bs + (int64_t)head * D, p.k_ss);
+  write_out(dv, p.dv + (int64_t)b * p.v_bs + (int64_t)head * D, p.v_ss);
 }
 
 // (B) dQ: workgroup owns 128 query rows (32 per wave), streams key tiles.
