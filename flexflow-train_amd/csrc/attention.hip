@@ -391,8 +391,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
       rq[R][i] = *reinterpret_cast<u32x4 const *>(qp + (int64_t)gr * p.q_ss + ch * 8);
       rg[R][i] = *reinterpret_cast<u32x4 const *>(gp + (int64_t)gr * p.o_ss + ch * 8);
     }
-    if (t < C::kTile) {
-      int gr = min(qt0 + t, p.Sq - 1);
+    // every lane loads (lanes >= kTile a duplicate): a load under a branch would make the
+    // number of loads in flight path-dependent and force full waits on the older tile
+    {
+      int gr = min(qt0 + (t & (C::kTile - 1)), p.Sq - 1);
       rl[R] = lsep[gr] * kLog2e;
       rd[R] = delp[gr];
     }
@@ -420,14 +422,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
     gload(q_begin, Set0{});
     lstore(Set0{});
   }
-  if (ntiles > 1) gload(q_begin + C::kTile, Set1{});
+  // Tiles past the end are loaded too (their rows clamp to the last row, nothing is done with
+  // them): with the same loads in flight on every path, a step waits for exactly the tile it
+  // needs and leaves the younger prefetch in flight.
+  gload(q_begin + C::kTile, Set1{});
   __syncthreads();
   auto step = [&](int it, auto parity) {
     constexpr int cur = decltype(parity)::value;  // == it % 2
     int const qt0 = q_begin + it * C::kTile;
-    if (it + 2 < ntiles) gload(qt0 + 2 * C::kTile, parity);
+    gload(qt0 + 2 * C::kTile, parity);
     // A wave whose keys all lie after this query tile (causal) contributes 0.
-    bool const active = !p.causal || kv0 + wave * 32 <= qt0 + C::kTile - 1;
+    bool const active = it < ntiles && (!p.causal || kv0 + wave * 32 <= qt0 + C::kTile - 1);
     if (active) {
       bf16 const *qk = Qs[cur] + koff, *gk = Gs[cur] + koff;
       bf16 const *qtr = Qs[cur] + toff, *gtr = Gs[cur] + toff;
@@ -489,9 +494,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
     if (it + 1 < ntiles) lstore(std::integral_constant<int, cur ^ 1>{});
     __syncthreads();
   };
+  // always in pairs (an odd count runs one idle step): the loop body then issues the same
+  // loads whatever the tile count, which keeps the waits on them exact
   for (int it = 0; it < ntiles; it += 2) {
     step(it, Set0{});
-    if (it + 1 < ntiles) step(it + 1, Set1{});
+    step(it + 1, Set1{});
   }
 
   // dK / dV accumulators: row = key (32 per wave, 8*(r/4)+4*h+r%4), column = d: a lane
@@ -596,13 +603,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
   int const toff = lane_tr_off(C::kStride, lane);
   gload(0, Set0{});
   lstore(Set0{});
-  if (ntiles > 1) gload(C::kTile, Set1{});
+  gload(C::kTile, Set1{});  // unconditional, like every prefetch below (see the dK/dV kernel)
   __syncthreads();
   auto step = [&](int it, auto parity) {
     constexpr int cur = decltype(parity)::value;  // == it % 2
     int const kt0 = it * C::kTile;
-    if (it + 2 < ntiles) gload(kt0 + 2 * C::kTile, parity);
-    bool const active = !p.causal || kt0 <= q0 + wave * 32 + 31;
+    gload(kt0 + 2 * C::kTile, parity);
+    bool const active = it < ntiles && (!p.causal || kt0 <= q0 + wave * 32 + 31);
     if (active) {
       bf16 const *kk_ = Ks[cur] + koff, *vk_ = Vs[cur] + koff, *ktr = Ks[cur] + toff;
       // S^T = K Q^T, dP^T = V dO^T: rows = keys of the tile, column = query.
@@ -648,9 +655,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
     if (it + 1 < ntiles) lstore(std::integral_constant<int, cur ^ 1>{});
     __syncthreads();
   };
+  // always in pairs (an odd count runs one idle step): the loop body then issues the same
+  // loads whatever the tile count, which keeps the waits on them exact
   for (int it = 0; it < ntiles; it += 2) {
     step(it, Set0{});
-    if (it + 1 < ntiles) step(it + 1, Set1{});
+    step(it + 1, Set1{});
   }
 
   if (qrow < p.Sq) {
