@@ -11,6 +11,7 @@
 // Indices outside [0, num_entries) are skipped (the reference reads or writes
 // out of bounds for them).
 #include "ffk_common.h"
+#include <cstdlib>
 #include <cstring>
 #include <rocprim/device/device_radix_sort.hpp>
 
@@ -323,8 +324,9 @@ __global__ __launch_bounds__(kEmbBlockThreads) void embedding_bwd_sorted_block_k
     if (active) {
       float acc[CPL][4], cur[CPL][4], nxt[CPL][4];
       auto fetch = [&](int64_t p, float (&v)[CPL][4]) {
-        int64_t const l = (int64_t)vals[p];
-        GT const *row = dY + (l / bag) * dim;
+        // lookups are 32-bit positions: a 32-bit unsigned division, and none for bags of one
+        uint32_t const l = vals[p];
+        GT const *row = dY + (int64_t)(bag == 1 ? l : l / (uint32_t)bag) * dim;
 #pragma unroll
         for (int k = 0; k < CPL; k++) {
           int64_t const c = cbase + ((int64_t)k * LPR + wl) * 4;
