@@ -128,6 +128,12 @@ SIGNATURES = {
     "ffk_identity_loss_backward": (c_int, [c_p, c_p, c_p, c_i64, c_i64, c_f]),
     "ffk_cast_forward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_i64]),
     "ffk_cast_backward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_i64]),
+    "ffk_transpose_forward": (c_int, [c_p, c_int, c_p, c_p, c_int, c_p, c_p]),
+    "ffk_transpose_backward": (c_int, [c_p, c_int, c_p, c_p, c_int, c_p, c_p, c_int]),
+    "ffk_gather_forward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_i64, c_i64, c_i64, c_i64]),
+    "ffk_gather_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_i64, c_i64, c_i64]),
+    "ffk_split_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_int, c_i64]),
+    "ffk_split_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_int, c_i64, c_int]),
     "ffk_concat_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_int, c_i64]),
     "ffk_concat_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_int, c_i64, c_int]),
     "ffk_embedding_forward": (c_int, [c_p, c_int, c_int, c_int, c_p, c_p, c_p, c_int, c_i64,
@@ -598,3 +604,77 @@ def concat_backward(out_grad, input_grads, axis, accumulate=True):
     check(lib().ffk_concat_backward(current_stream(), dtype_of(out_grad), ptr(out_grad), ptrs, blks,
                                     len(input_grads), num_blocks, int(accumulate)))
     return input_grads
+
+
+def transpose_forward(x, perm, out=None):
+    """out = x.permute(perm), materialised (x contiguous)."""
+    import ctypes
+    torch = _torch()
+    dims = (ctypes.c_int64 * x.dim())(*x.shape)
+    pm = (ctypes.c_int * x.dim())(*perm)
+    if out is None:
+        out = torch.empty([x.shape[p] for p in perm], dtype=x.dtype, device=x.device)
+    check(lib().ffk_transpose_forward(current_stream(), dtype_of(x), ptr(x), ptr(out), x.dim(), dims, pm))
+    return out
+
+
+def transpose_backward(out_grad, in_grad, perm, accumulate=True):
+    """in_grad (+)= out_grad moved back through the inverse of `perm`; in_grad has the input's shape."""
+    import ctypes
+    dims = (ctypes.c_int64 * in_grad.dim())(*in_grad.shape)
+    pm = (ctypes.c_int * in_grad.dim())(*perm)
+    check(lib().ffk_transpose_backward(current_stream(), dtype_of(out_grad), ptr(out_grad), ptr(in_grad),
+                                       in_grad.dim(), dims, pm, int(accumulate)))
+    return in_grad
+
+
+def _gather_view(shape, out_shape, dim):
+    dim = dim if dim >= 0 else len(shape) + dim
+    outer = 1
+    for d in shape[:dim]:
+        outer *= d
+    stride = 1
+    for d in shape[dim + 1:]:
+        stride *= d
+    return outer, shape[dim], out_shape[dim], stride
+
+
+def gather_forward(x, index, dim, out=None):
+    """torch.gather(x, dim, index) for index of x's shape except along `dim`."""
+    torch = _torch()
+    outer, ind, outd, stride = _gather_view(tuple(x.shape), tuple(index.shape), dim)
+    if out is None:
+        out = torch.empty(index.shape, dtype=x.dtype, device=x.device)
+    check(lib().ffk_gather_forward(current_stream(), dtype_of(x), dtype_of(index), ptr(x), ptr(index), ptr(out),
+                                   outer, ind, outd, stride))
+    return out
+
+
+def gather_backward(out_grad, index, in_grad, dim):
+    """in_grad[.., index, ..] += out_grad (fp32, atomics)."""
+    outer, ind, outd, stride = _gather_view(tuple(in_grad.shape), tuple(index.shape), dim)
+    check(lib().ffk_gather_backward(current_stream(), dtype_of(index), ptr(out_grad), ptr(index), ptr(in_grad),
+                                    outer, ind, outd, stride))
+    return in_grad
+
+
+def split_forward(x, sizes, axis):
+    """The pieces of x along `axis` with extents `sizes`, as new contiguous tensors."""
+    torch = _torch()
+    axis = axis if axis >= 0 else x.dim() + axis
+    outs = []
+    for n in sizes:
+        shape = list(x.shape)
+        shape[axis] = n
+        outs.append(torch.empty(shape, dtype=x.dtype, device=x.device))
+    _, num_blocks, ptrs, blks = _concat_args(outs, axis)
+    check(lib().ffk_split_forward(current_stream(), dtype_of(x), ptrs, ptr(x), blks, len(outs), num_blocks))
+    return outs
+
+
+def split_backward(out_grads, in_grad, axis, accumulate=True):
+    """in_grad (+)= the output gradients side by side along `axis`."""
+    axis, num_blocks, ptrs, blks = _concat_args(out_grads, axis)
+    check(lib().ffk_split_backward(current_stream(), dtype_of(in_grad), ptr(in_grad), ptrs, blks,
+                                   len(out_grads), num_blocks, int(accumulate)))
+    return in_grad

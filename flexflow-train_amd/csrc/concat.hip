@@ -24,7 +24,8 @@ struct ConcatArgs {
   int64_t num_blocks;
 };
 
-enum ConcatMode { kGather = 0, kScatter = 1, kScatterAddF32 = 2, kScatterAddBf16 = 3 };
+// gather: concatenated row <- parts; scatter: parts <- concatenated row; "Add" adds to the destination
+enum ConcatMode { kGather = 0, kScatter = 1, kScatterAddF32 = 2, kScatterAddBf16 = 3, kGatherAddF32 = 4, kGatherAddBf16 = 5 };
 
 // U: the unit a lane moves (uint8/16/32/64 or 16 bytes)
 template <typename U, int MODE>
@@ -59,25 +60,29 @@ __global__ __launch_bounds__(kConcatThreads) void concat_kernel(char *cat, Conca
       *cp = *pp;
     } else if (MODE == kScatter) {
       *pp = *cp;
-    } else if (MODE == kScatterAddF32) {
-      // U is f32x4 or float
-      *pp = *pp + *cp;
     } else {
-      // U is u32x4 (8 bf16) or uint16_t (1 bf16): add in fp32, round once
-      if constexpr (sizeof(U) == 16) {
-        u32x4 const g = *reinterpret_cast<u32x4 const *>(cp);
-        u32x4 o = *reinterpret_cast<u32x4 *>(pp);
+      // adding: src -> dst depends on the direction
+      constexpr bool kToParts = MODE == kScatterAddF32 || MODE == kScatterAddBf16;
+      U *const dst = kToParts ? pp : cp;
+      U const *const src = kToParts ? cp : pp;
+      if constexpr (MODE == kScatterAddF32 || MODE == kGatherAddF32) {
+        // U is f32x4 or float
+        *dst = *dst + *src;
+      } else if constexpr (sizeof(U) == 16) {
+        // 8 bf16: add in fp32, round once
+        u32x4 const g = *reinterpret_cast<u32x4 const *>(src);
+        u32x4 o = *reinterpret_cast<u32x4 *>(dst);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           float const l = __uint_as_float(o[i] << 16) + __uint_as_float(g[i] << 16);
           float const h = __uint_as_float(o[i] & 0xffff0000u) + __uint_as_float(g[i] & 0xffff0000u);
           o[i] = pack_bf16x2(l, h);
         }
-        *reinterpret_cast<u32x4 *>(pp) = o;
+        *reinterpret_cast<u32x4 *>(dst) = o;
       } else {
-        uint16_t const g = *reinterpret_cast<uint16_t const *>(cp);
-        uint16_t const o = *reinterpret_cast<uint16_t *>(pp);
-        *reinterpret_cast<uint16_t *>(pp) = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(o) + bf16_bits_to_f32(g));
+        uint16_t const g = *reinterpret_cast<uint16_t const *>(src);
+        uint16_t const o = *reinterpret_cast<uint16_t *>(dst);
+        *reinterpret_cast<uint16_t *>(dst) = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(o) + bf16_bits_to_f32(g));
       }
     }
   }
@@ -109,14 +114,14 @@ static int elem_bytes(int dtype) {
   }
 }
 
-// mode: 0 forward, 1 backward overwriting, 2 backward accumulating
+// mode: 0 row <- parts, 1 parts <- row, 2 parts += row, 3 row += parts
 static int concat_any(char const *who, ffk_stream_t stream, int dtype, void *cat, void *const *parts,
                       int64_t const *part_blk_elems, int num_parts, int64_t num_blocks, int mode) {
   int const eb = elem_bytes(dtype);
   FFK_REQUIRE(eb != 0, "%s: data type %d not supported", who, dtype);
   FFK_REQUIRE(num_parts >= 1 && num_blocks >= 0, "%s: bad sizes", who);
   FFK_REQUIRE(parts != nullptr && part_blk_elems != nullptr, "%s: NULL argument", who);
-  FFK_REQUIRE(mode != 2 || dtype == FFK_FLOAT || dtype == FFK_BF16,
+  FFK_REQUIRE(mode < 2 || dtype == FFK_FLOAT || dtype == FFK_BF16,
               "%s: accumulating backward supports float and bf16 (got data type %d)", who, dtype);
   hipStream_t st = as_stream(stream);
   int64_t row_bytes = 0;
@@ -162,12 +167,18 @@ static int concat_any(char const *who, ffk_stream_t stream, int dtype, void *cat
         else if (eb == 2) e = concat_launch<uint16_t, kScatter>(st, base, a, off);
         else if (eb == 4) e = concat_launch<uint32_t, kScatter>(st, base, a, off);
         else e = concat_launch<uint64_t, kScatter>(st, base, a, off);
-      } else if (dtype == FFK_FLOAT) {
+      } else if (mode == 2 && dtype == FFK_FLOAT) {
         if (wide) e = concat_launch<f32x4, kScatterAddF32>(st, base, a, off);
         else e = concat_launch<float, kScatterAddF32>(st, base, a, off);
-      } else {
+      } else if (mode == 2) {
         if (wide) e = concat_launch<u32x4, kScatterAddBf16>(st, base, a, off);
         else e = concat_launch<uint16_t, kScatterAddBf16>(st, base, a, off);
+      } else if (dtype == FFK_FLOAT) {
+        if (wide) e = concat_launch<f32x4, kGatherAddF32>(st, base, a, off);
+        else e = concat_launch<float, kGatherAddF32>(st, base, a, off);
+      } else {
+        if (wide) e = concat_launch<u32x4, kGatherAddBf16>(st, base, a, off);
+        else e = concat_launch<uint16_t, kGatherAddBf16>(st, base, a, off);
       }
       FFK_HIP(e);
     }
@@ -191,4 +202,19 @@ extern "C" int ffk_concat_backward(ffk_stream_t stream, int dtype, void const *o
                                    int accumulate) {
   return concat_any("concat_backward", stream, dtype, const_cast<void *>(output_grad), input_grads, input_blk_elems,
                     num_inputs, num_blocks, accumulate ? 2 : 1);
+}
+
+// Split is Concat read the other way (reference: lib/kernels/src/cuda/ops/split_kernels.cu).
+extern "C" int ffk_split_forward(ffk_stream_t stream, int dtype, void *const *outputs, void const *input,
+                                 int64_t const *output_blk_elems, int num_outputs, int64_t num_blocks) {
+  return concat_any("split_forward", stream, dtype, const_cast<void *>(input), outputs, output_blk_elems, num_outputs,
+                    num_blocks, 1);
+}
+
+extern "C" int ffk_split_backward(ffk_stream_t stream, int dtype, void *input_grad, void const *const *output_grads,
+                                  int64_t const *output_blk_elems, int num_outputs, int64_t num_blocks,
+                                  int accumulate) {
+  return concat_any("split_backward", stream, dtype, input_grad,
+                    const_cast<void *const *>(reinterpret_cast<void const *const *>(output_grads)), output_blk_elems,
+                    num_outputs, num_blocks, accumulate ? 3 : 0);
 }

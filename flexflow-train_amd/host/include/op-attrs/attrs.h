@@ -7,10 +7,12 @@
 //   LinearAttrs       lib/op-attrs/include/op-attrs/ops/linear_attrs.dtg.toml:32-50
 //   ElementUnaryAttrs lib/op-attrs/include/op-attrs/ops/element_unary_attrs.dtg.toml
 //   DropoutAttrs      lib/op-attrs/include/op-attrs/ops/dropout_attrs.dtg.toml
+//   TransposeAttrs    lib/op-attrs/include/op-attrs/ops/transpose_attrs.dtg.toml
 #pragma once
 #include "op-attrs/datatype.h"
 #include <optional>
 #include <variant>
+#include <vector>
 
 namespace FlexFlow {
 
@@ -47,6 +49,11 @@ struct LinearAttrs {
 struct ElementUnaryAttrs {
   OperatorType op_type;
   std::optional<float> scalar;
+};
+
+// output dim i is input dim permutation[i] (FF order)
+struct TransposeAttrs {
+  std::vector<int> permutation;
 };
 
 struct DropoutAttrs {

@@ -59,10 +59,13 @@ struct EmbeddingAttrs {
 };
 struct CastAttrs { DataType dtype; };
 struct ConcatAttrs { int axis; };  // relative dim
+struct ReshapeAttrs { TensorDims shape; };
+struct GatherAttrs { int dim; };  // relative dim; inputs: values, index
 
 using ComputationGraphOpAttrs =
     std::variant<InputAttrs, WeightAttrs, LinearAttrs, LayerNormAttrs, MultiHeadAttentionAttrs, DropoutAttrs,
-                 ElementUnaryAttrs, ElementBinaryAttrs, SoftmaxAttrs, EmbeddingAttrs, CastAttrs, ConcatAttrs>;
+                 ElementUnaryAttrs, ElementBinaryAttrs, SoftmaxAttrs, EmbeddingAttrs, CastAttrs, ConcatAttrs, TransposeAttrs, ReshapeAttrs,
+                 GatherAttrs>;
 
 struct LayerAttrs {
   ComputationGraphOpAttrs op_attrs;

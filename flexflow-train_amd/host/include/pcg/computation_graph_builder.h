@@ -50,6 +50,12 @@ struct ComputationGraphBuilder {
   tensor_guid_t cast(tensor_guid_t const &input, DataType dtype, std::optional<std::string> const &name = std::nullopt);
   tensor_guid_t concat(std::vector<tensor_guid_t> const &tensors, int axis,
                        std::optional<std::string> const &name = std::nullopt);
+  tensor_guid_t transpose(tensor_guid_t const &input, std::vector<int> const &perm,
+                          std::optional<std::string> const &name = std::nullopt);
+  tensor_guid_t reshape(tensor_guid_t const &input, std::vector<int64_t> const &shape,
+                        std::optional<std::string> const &name = std::nullopt);
+  tensor_guid_t gather(tensor_guid_t const &input, tensor_guid_t const &index, int dim,
+                       std::optional<std::string> const &name = std::nullopt);
   tensor_guid_t softmax(tensor_guid_t const &input, std::optional<int> dim = std::nullopt,
                         std::optional<std::string> const &name = std::nullopt);
   // `scale` and `causal` extend the reference's signature (its kernel fixes 1.0 / false).

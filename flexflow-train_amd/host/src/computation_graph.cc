@@ -138,6 +138,37 @@ std::vector<TensorShape> get_output_shapes(ComputationGraphOpAttrs const &attrs,
     }
     return {o};
   }
+  if (auto const *a = std::get_if<TransposeAttrs>(&attrs)) {
+    need(1);
+    int nd = get_num_dims(in[0].dims);
+    if ((int)a->permutation.size() != nd) bad("transpose: permutation length differs from the rank");
+    std::vector<bool> seen(nd, false);
+    TensorShape o = in[0];
+    for (int i = 0; i < nd; i++) {
+      int p = a->permutation[i];
+      if (p < 0 || p >= nd || seen[p]) bad("transpose: not a permutation");
+      seen[p] = true;
+      o.dims.ff_ordered[i] = in[0].dims.ff_ordered[p];
+    }
+    return {o};
+  }
+  if (auto const *a = std::get_if<ReshapeAttrs>(&attrs)) {
+    need(1);
+    if (get_num_elements(a->shape) != get_num_elements(in[0].dims)) bad("reshape: element counts differ");
+    return {TensorShape{a->shape, in[0].data_type}};
+  }
+  if (auto const *a = std::get_if<GatherAttrs>(&attrs)) {
+    // gather.cc: the output takes the index's dims and the values' data type
+    need(2);
+    if (!is_integer(in[1].data_type)) bad("gather expects INT32 or INT64 indices");
+    int nd = get_num_dims(in[0].dims);
+    int d = a->dim < 0 ? nd + a->dim : a->dim;
+    if (d < 0 || d >= nd || get_num_dims(in[1].dims) != nd) bad("gather: dim or ranks out of range");
+    for (int i = 0; i < nd; i++) {
+      if (i != d && in[0].dims.ff_ordered[i] != in[1].dims.ff_ordered[i]) bad("gather: shapes differ outside the dim");
+    }
+    return {TensorShape{in[1].dims, in[0].data_type}};
+  }
   if (auto const *a = std::get_if<CastAttrs>(&attrs)) {
     need(1);
     TensorShape o = in[0];
@@ -342,6 +373,18 @@ tensor_guid_t ComputationGraphBuilder::cast(tensor_guid_t const &input, DataType
 tensor_guid_t ComputationGraphBuilder::concat(std::vector<tensor_guid_t> const &tensors, int axis,
                                               std::optional<std::string> const &name) {
   return add_op(ConcatAttrs{axis}, tensors, name);
+}
+tensor_guid_t ComputationGraphBuilder::transpose(tensor_guid_t const &input, std::vector<int> const &perm,
+                                                 std::optional<std::string> const &name) {
+  return add_op(TransposeAttrs{perm}, {input}, name);
+}
+tensor_guid_t ComputationGraphBuilder::reshape(tensor_guid_t const &input, std::vector<int64_t> const &shape,
+                                               std::optional<std::string> const &name) {
+  return add_op(ReshapeAttrs{TensorDims{shape}}, {input}, name);
+}
+tensor_guid_t ComputationGraphBuilder::gather(tensor_guid_t const &input, tensor_guid_t const &index, int dim,
+                                              std::optional<std::string> const &name) {
+  return add_op(GatherAttrs{dim}, {input, index}, name);
 }
 tensor_guid_t ComputationGraphBuilder::softmax(tensor_guid_t const &input, std::optional<int> dim,
                                                std::optional<std::string> const &name) {

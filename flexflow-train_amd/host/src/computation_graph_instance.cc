@@ -278,6 +278,17 @@ ComputationGraphInstance create_computation_graph_instance(
           shape_of(layer.outputs[0]).data_type != DataType::BF16) {
         bad("concat backward adds in FLOAT or BF16 only");
       }
+    } else if (std::get_if<GatherAttrs>(&oa)) {
+      // the scatter adds (atomics) into the values' gradient; the index carries none
+      if (has_grad[layer.inputs[0].raw]) {
+        if (shape_of(layer.inputs[0]).data_type != DataType::FLOAT) bad("gather backward adds FLOAT gradients");
+        cleared[layer.inputs[0].raw] = true;
+      }
+      acc = false;
+    } else if (std::get_if<TransposeAttrs>(&oa) || std::get_if<ReshapeAttrs>(&oa)) {
+      if (acc && shape_of(layer.outputs[0]).data_type != DataType::FLOAT && shape_of(layer.outputs[0]).data_type != DataType::BF16) {
+        bad("transpose / reshape backward adds in FLOAT or BF16 only");
+      }
     } else if (std::get_if<CastAttrs>(&oa)) {
       acc = true;  // cast_backward always adds
     } else if (std::get_if<ElementBinaryAttrs>(&oa)) {
@@ -532,6 +543,55 @@ ComputationGraphInstance create_computation_graph_instance(
       b = [=](device_stream_t const &s) {
         check_ffk(ffk_concat_backward(s.require_gpu(), type, dy, grad_ptrs.data(), blks.data(), parts, blocks, accumulate),
                   "Concat backward");
+      };
+    } else if (auto const *a = std::get_if<TransposeAttrs>(&oa)) {
+      tensor_guid_t x = layer.inputs[0];
+      int const type = dt(shape_of(x).data_type), nd = get_num_dims(shape_of(x).dims);
+      std::vector<int64_t> const dims = shape_of(x).dims.ff_ordered;
+      std::vector<int> const perm = a->permutation;
+      void *xp = val(x), *dx = grd_or_discard(x);
+      int const accumulate = p.bwd.accumulate ? 1 : 0;
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_transpose_forward(s.require_gpu(), type, xp, y, nd, dims.data(), perm.data()), "Transpose forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_transpose_backward(s.require_gpu(), type, dy, dx, nd, dims.data(), perm.data(), accumulate),
+                  "Transpose backward");
+      };
+    } else if (std::get_if<ReshapeAttrs>(&oa)) {
+      // the same elements in the same order: a flat copy forward, a flat copy or add backward
+      tensor_guid_t x = layer.inputs[0];
+      int const type = dt(shape_of(x).data_type);
+      int64_t const n = numel(x);
+      int64_t const flat = n;
+      int const one = 0;
+      void *xp = val(x), *dx = grd_or_discard(x);
+      int const accumulate = p.bwd.accumulate ? 1 : 0;
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_transpose_forward(s.require_gpu(), type, xp, y, 1, &flat, &one), "Reshape forward");
+      };
+      b = [=](device_stream_t const &s) {
+        check_ffk(ffk_transpose_backward(s.require_gpu(), type, dy, dx, 1, &flat, &one, accumulate), "Reshape backward");
+      };
+    } else if (auto const *a = std::get_if<GatherAttrs>(&oa)) {
+      tensor_guid_t x = layer.inputs[0], index = layer.inputs[1];
+      int const type = dt(shape_of(x).data_type), itype = dt(shape_of(index).data_type);
+      int nd = get_num_dims(shape_of(x).dims), d = a->dim < 0 ? nd + a->dim : a->dim;
+      int64_t outer = 1, stride = 1;
+      for (int i = 0; i < d; i++) outer *= shape_of(x).dims.ff_ordered[i];
+      for (int i = d + 1; i < nd; i++) stride *= shape_of(x).dims.ff_ordered[i];
+      int64_t const in_dim = shape_of(x).dims.ff_ordered[d], out_dim = shape_of(index).dims.ff_ordered[d];
+      void *xp = val(x), *ip = val(index);
+      float *dx = static_cast<float *>(grd(x));
+      f = [=](device_stream_t const &s) {
+        check_ffk(ffk_gather_forward(s.require_gpu(), type, itype, xp, ip, y, outer, in_dim, out_dim, stride), "Gather forward");
+      };
+      b = [=](device_stream_t const &s) {
+        if (dx != nullptr) {
+          check_ffk(ffk_gather_backward(s.require_gpu(), itype, static_cast<float const *>(dy), ip, dx, outer, in_dim,
+                                        out_dim, stride),
+                    "Gather backward");
+        }
       };
     } else if (std::get_if<CastAttrs>(&oa)) {
       tensor_guid_t x = layer.inputs[0];

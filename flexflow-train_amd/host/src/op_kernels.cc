@@ -10,6 +10,7 @@
 #include "kernels/concat_kernels.h"
 #include "kernels/loss_function_kernels.h"
 #include "kernels/optimizer_kernels.h"
+#include "kernels/shape_kernels.h"
 #include "kernels/layer_norm_kernels.h"
 #include "kernels/linear_kernels.h"
 #include "kernels/softmax_kernels.h"
@@ -634,5 +635,145 @@ void backward_kernel(device_stream_t const &stream, GenericTensorAccessorR const
 }
 
 }  // namespace Kernels::Concat
+
+namespace Kernels::Transpose {
+
+static void check_transpose(char const *who, TransposeAttrs const &attrs, TensorShape const &in, TensorShape const &out) {
+  int const nd = get_num_dims(in.dims);
+  if ((int)attrs.permutation.size() != nd || get_num_dims(out.dims) != nd || in.data_type != out.data_type) {
+    throw std::runtime_error(std::string(who) + ": permutation, input and output disagree");
+  }
+  for (int i = 0; i < nd; i++) {
+    int const p = attrs.permutation[i];
+    if (p < 0 || p >= nd || out.dims.ff_ordered[i] != in.dims.ff_ordered[p]) {
+      throw std::runtime_error(std::string(who) + ": output dims are not the permuted input dims");
+    }
+  }
+}
+
+void forward_kernel(device_stream_t const &stream, TransposeAttrs const &attrs, GenericTensorAccessorR const &input,
+                    GenericTensorAccessorW const &output) {
+  if (!stream.is_gpu()) no_cpu("Transpose::forward_kernel");
+  check_transpose("Transpose::forward_kernel", attrs, input.shape, output.shape);
+  check_ffk(ffk_transpose_forward(stream.require_gpu(), dt(input.shape.data_type), input.ptr, output.ptr,
+                                  get_num_dims(input.shape.dims), input.shape.dims.ff_ordered.data(),
+                                  attrs.permutation.data()),
+            "Transpose::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, TransposeAttrs const &attrs, GenericTensorAccessorR const &out_grad,
+                     GenericTensorAccessorW const &in_grad) {
+  if (!stream.is_gpu()) no_cpu("Transpose::backward_kernel");
+  check_transpose("Transpose::backward_kernel", attrs, in_grad.shape, out_grad.shape);
+  check_ffk(ffk_transpose_backward(stream.require_gpu(), dt(in_grad.shape.data_type), out_grad.ptr, in_grad.ptr,
+                                   get_num_dims(in_grad.shape.dims), in_grad.shape.dims.ff_ordered.data(),
+                                   attrs.permutation.data(), 1),
+            "Transpose::backward_kernel");
+}
+
+}  // namespace Kernels::Transpose
+
+namespace Kernels::Reshape {
+
+// reshape_kernels.cu: a copy forward, an add backward; the two shapes hold the same elements
+void forward_kernel(device_stream_t const &stream, GenericTensorAccessorR const &input,
+                    GenericTensorAccessorW const &output) {
+  if (!stream.is_gpu()) no_cpu("Reshape::forward_kernel");
+  if (get_num_elements(input.shape.dims) != get_num_elements(output.shape.dims) || input.shape.data_type != output.shape.data_type) {
+    throw std::runtime_error("Reshape::forward_kernel: shapes hold different element counts or data types");
+  }
+  check_ffk(ffk_cast_forward(stream.require_gpu(), dt(input.shape.data_type), dt(output.shape.data_type), input.ptr,
+                             output.ptr, get_num_elements(input.shape.dims)),
+            "Reshape::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, GenericTensorAccessorR const &output,
+                     GenericTensorAccessorW const &input) {
+  if (!stream.is_gpu()) no_cpu("Reshape::backward_kernel");
+  if (get_num_elements(input.shape.dims) != get_num_elements(output.shape.dims) || input.shape.data_type != output.shape.data_type) {
+    throw std::runtime_error("Reshape::backward_kernel: shapes hold different element counts or data types");
+  }
+  check_ffk(ffk_cast_backward(stream.require_gpu(), dt(output.shape.data_type), dt(input.shape.data_type), output.ptr,
+                              input.ptr, get_num_elements(input.shape.dims)),
+            "Reshape::backward_kernel");
+}
+
+}  // namespace Kernels::Reshape
+
+namespace Kernels::Split {
+
+void forward_kernel(device_stream_t const &stream, float **out_ptrs, float const *in_ptr, int const *out_blk_sizes,
+                    int in_blk_size, int num_blks, int numOutputs) {
+  if (!stream.is_gpu()) no_cpu("Split::forward_kernel");
+  std::vector<void *> ptrs(out_ptrs, out_ptrs + numOutputs);
+  std::vector<int64_t> blks(out_blk_sizes, out_blk_sizes + numOutputs);
+  int64_t sum = 0;
+  for (int64_t b : blks) sum += b;
+  if (sum != in_blk_size) throw std::runtime_error("Split::forward_kernel: the outputs do not add up to the input block");
+  check_ffk(ffk_split_forward(stream.require_gpu(), FFK_FLOAT, ptrs.data(), in_ptr, blks.data(), numOutputs, num_blks),
+            "Split::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, float *in_grad_ptr, float const **out_grad_ptr,
+                     int const *out_blk_sizes, int in_blk_size, int num_blks, int numOutputs) {
+  if (!stream.is_gpu()) no_cpu("Split::backward_kernel");
+  std::vector<void const *> ptrs(out_grad_ptr, out_grad_ptr + numOutputs);
+  std::vector<int64_t> blks(out_blk_sizes, out_blk_sizes + numOutputs);
+  int64_t sum = 0;
+  for (int64_t b : blks) sum += b;
+  if (sum != in_blk_size) throw std::runtime_error("Split::backward_kernel: the outputs do not add up to the input block");
+  check_ffk(ffk_split_backward(stream.require_gpu(), FFK_FLOAT, in_grad_ptr, ptrs.data(), blks.data(), numOutputs,
+                               num_blks, 1),
+            "Split::backward_kernel");
+}
+
+}  // namespace Kernels::Split
+
+namespace Kernels::Gather {
+
+std::optional<GatherPerDeviceState> init_kernel(DeviceType device_type, device_handle_t const &handle, ff_dim_t dim) {
+  if (device_type != DeviceType::GPU) return std::nullopt;
+  return GatherPerDeviceState{handle.require_for_gpu(), dim};
+}
+
+struct GatherView {
+  int64_t outer, in_dim, out_dim, stride;
+};
+static GatherView gather_view(char const *who, ff_dim_t dim, TensorShape const &in, TensorShape const &index) {
+  int const nd = get_num_dims(in.dims);
+  if (dim.value < 0 || dim.value >= nd || get_num_dims(index.dims) != nd) {
+    throw std::runtime_error(std::string(who) + ": dim or ranks out of range");
+  }
+  GatherView v{1, in.dims.ff_ordered[dim.value], index.dims.ff_ordered[dim.value], 1};
+  for (int i = 0; i < nd; i++) {
+    if (i != dim.value && in.dims.ff_ordered[i] != index.dims.ff_ordered[i]) {
+      throw std::runtime_error(std::string(who) + ": input and index differ outside the gathered dim");
+    }
+    if (i < dim.value) v.outer *= in.dims.ff_ordered[i];
+    if (i > dim.value) v.stride *= in.dims.ff_ordered[i];
+  }
+  return v;
+}
+
+void forward_kernel(device_stream_t const &stream, std::optional<GatherPerDeviceState> const &state,
+                    GenericTensorAccessorR const &input, GenericTensorAccessorR const &index,
+                    GenericTensorAccessorW const &output) {
+  if (!stream.is_gpu()) no_cpu("Gather::forward_kernel");
+  if (output.shape.dims != index.shape.dims || output.shape.data_type != input.shape.data_type) {
+    throw std::runtime_error("Gather::forward_kernel: the output takes the index's dims and the input's data type");
+  }
+  GatherView v = gather_view("Gather::forward_kernel", state.value().dim, input.shape, index.shape);
+  check_ffk(ffk_gather_forward(stream.require_gpu(), dt(input.shape.data_type), dt(index.shape.data_type), input.ptr,
+                               index.ptr, output.ptr, v.outer, v.in_dim, v.out_dim, v.stride),
+            "Gather::forward_kernel");
+}
+void backward_kernel(device_stream_t const &stream, std::optional<GatherPerDeviceState> const &state,
+                     GenericTensorAccessorR const &output_grad, GenericTensorAccessorR const &index,
+                     GenericTensorAccessorW const &input_grad) {
+  if (!stream.is_gpu()) no_cpu("Gather::backward_kernel");
+  GatherView v = gather_view("Gather::backward_kernel", state.value().dim, input_grad.shape, index.shape);
+  check_ffk(ffk_gather_backward(stream.require_gpu(), dt(index.shape.data_type), output_grad.get_float_ptr(), index.ptr,
+                                input_grad.get_float_ptr(), v.outer, v.in_dim, v.out_dim, v.stride),
+            "Gather::backward_kernel");
+}
+
+}  // namespace Kernels::Gather
 
 }  // namespace FlexFlow

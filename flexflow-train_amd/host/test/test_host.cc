@@ -17,6 +17,7 @@
 #include "kernels/loss_function_kernels.h"
 #include "kernels/optimizer_kernels.h"
 #include "kernels/profiling.h"
+#include "kernels/shape_kernels.h"
 #include "kernels/softmax_kernels.h"
 #include "ffk.h"
 #include "local-execution/computation_graph_instance.h"
@@ -841,6 +842,113 @@ static void gpu_tests() {
     }
     for (size_t j = 0; j < wh.size(); j++) wh[j] -= lr * dwh[j];
     CHECK(close(to_host(inst.get_tensor_accessor(cgb.get_weights_of(hidden)[0])), wh, 1e-5));
+  });
+  run("Transpose, Reshape, Split and Gather equal the oracle", [&] {
+    // transpose [4, 6, 10] -> perm (2, 0, 1), and its backward into a non-zero gradient
+    std::vector<int64_t> dims = {4, 6, 10};
+    TransposeAttrs tattrs{{2, 0, 1}};
+    int64_t const n = 4 * 6 * 10;
+    auto x = random_vec(n, 90), old = random_vec(n, 91), dout = random_vec(n, 92);
+    auto X = device_accessor(gpu, shape(dims, DataType::FLOAT), x);
+    auto Y = gpu.allocate_tensor(shape({10, 4, 6}, DataType::FLOAT));
+    Kernels::Transpose::forward_kernel(stream, tattrs, X, Y);
+    std::vector<float> want(n);
+    orc_transpose_nd(x.data(), want.data(), 3, dims.data(), tattrs.permutation.data(), 0);
+    CHECK(to_host(Y) == want);
+    auto DY = device_accessor(gpu, Y.shape, dout);
+    auto DX = device_accessor(gpu, X.shape, old);
+    Kernels::Transpose::backward_kernel(stream, tattrs, DY, DX);
+    std::vector<int64_t> odims = {10, 4, 6};
+    int inverse[3] = {1, 2, 0};
+    std::vector<float> wantb = old;
+    orc_transpose_nd(dout.data(), wantb.data(), 3, odims.data(), inverse, 1);
+    CHECK(to_host(DX) == wantb);
+    CHECK_THROWS(Kernels::Transpose::forward_kernel(stream, TransposeAttrs{{0, 1, 2}}, X, Y));  // dims do not match
+
+    // reshape: same elements
+    auto R = gpu.allocate_tensor(shape({24, 10}, DataType::FLOAT));
+    Kernels::Reshape::forward_kernel(stream, X, R);
+    CHECK(to_host(R) == x);
+    Kernels::Reshape::backward_kernel(stream, R, DX);
+    for (int64_t i = 0; i < n; i++) wantb[i] += x[i];
+    CHECK(to_host(DX) == wantb);
+
+    // split [6, 10] into column blocks 3 | 7, then back
+    auto IN = device_accessor(gpu, shape({6, 10}, DataType::FLOAT), random_vec(60, 93));
+    auto O1 = gpu.allocate_tensor(shape({6, 3}, DataType::FLOAT)), O2 = gpu.allocate_tensor(shape({6, 7}, DataType::FLOAT));
+    float *outs[2] = {O1.get_float_ptr(), O2.get_float_ptr()};
+    int blk[2] = {3, 7};
+    Kernels::Split::forward_kernel(stream, outs, IN.get_float_ptr(), blk, 10, 6, 2);
+    auto in_host = to_host(IN), o1 = to_host(O1), o2 = to_host(O2);
+    bool split_ok = true;
+    for (int r = 0; r < 6; r++) {
+      for (int c = 0; c < 10; c++) split_ok = split_ok && in_host[r * 10 + c] == (c < 3 ? o1[r * 3 + c] : o2[r * 7 + c - 3]);
+    }
+    CHECK(split_ok);
+    auto DIN = gpu.allocate_tensor(IN.shape);
+    fill_with_zeros(DIN);
+    float const *grads[2] = {O1.get_float_ptr(), O2.get_float_ptr()};
+    Kernels::Split::backward_kernel(stream, DIN.get_float_ptr(), grads, blk, 10, 6, 2);
+    CHECK(to_host(DIN) == in_host);
+
+    // gather along dim 1 of [4, 6, 10] with an int32 index [4, 3, 10]
+    std::vector<int64_t> idx(4 * 3 * 10);
+    std::mt19937 gen(3);
+    for (auto &v : idx) v = gen() % 6;
+    std::vector<int32_t> idx32(idx.begin(), idx.end());
+    Allocator cpu = create_local_cpu_memory_allocator();
+    GenericTensorAccessorW hidx = cpu.allocate_tensor(shape({4, 3, 10}, DataType::INT32));
+    memcpy(hidx.ptr, idx32.data(), idx32.size() * 4);
+    GenericTensorAccessorW I = copy_tensor_accessor_w(hidx, gpu);
+    auto gstate = Kernels::Gather::init_kernel(DeviceType::GPU, handle, ff_dim_t{1});
+    auto G = gpu.allocate_tensor(shape({4, 3, 10}, DataType::FLOAT));
+    Kernels::Gather::forward_kernel(stream, gstate, X, I, G);
+    std::vector<float> gwant(idx.size());
+    orc_gather_forward(x.data(), idx.data(), gwant.data(), 4, 6, 3, 10);
+    CHECK(to_host(G) == gwant && contains_non_zero(gwant));
+    auto gd = random_vec(idx.size(), 94);
+    auto GD = device_accessor(gpu, G.shape, gd);
+    auto DXg = device_accessor(gpu, X.shape, old);
+    Kernels::Gather::backward_kernel(stream, gstate, GD, I, DXg);
+    std::vector<float> gb = old;
+    orc_gather_backward(gd.data(), idx.data(), gb.data(), 4, 6, 3, 10);
+    CHECK(close(to_host(DXg), gb, 1e-5));
+  });
+
+  run("Step driver: transpose, reshape and gather layers carry values and gradients", [&] {
+    // y = gather(reshape(transpose(x, (1, 0, 2)), [6, 40]), index, dim 1); loss gradient = 1 / batch
+    ComputationGraphBuilder cgb;
+    tensor_guid_t x = cgb.create_input(shape({4, 6, 10}, DataType::FLOAT), CreateGrad::YES);
+    tensor_guid_t index = cgb.create_input(shape({6, 5}, DataType::INT64), CreateGrad::NO);
+    tensor_guid_t t = cgb.transpose(x, {1, 0, 2});
+    tensor_guid_t r = cgb.reshape(t, {6, 40});
+    tensor_guid_t y = cgb.gather(r, index, 1);
+    CHECK(cgb.get_shape(y) == shape({6, 5}, DataType::FLOAT));
+    device_id_t dev = make_device_id_t_from_idx(0, DeviceType::GPU);
+    auto LABEL = gpu.allocate_tensor(shape({6, 5}, DataType::FLOAT));
+    ComputationGraphInstance inst = create_computation_graph_instance(
+        cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{0.1, 0.0, false, 0.0}},
+        LossConfig{NonconfigurableLossAttrs{LossFunction::IDENTITY}, LABEL, y}, {}, gpu, ProfilingSettings{0, 0}, handle, dev);
+    auto xv = random_vec(240, 95);
+    copy_accessor_data_to_l_from_r(inst.get_tensor_accessor(x), device_accessor(gpu, shape({4, 6, 10}, DataType::FLOAT), xv));
+    std::vector<int64_t> idx(30);
+    std::mt19937 gen(5);
+    for (auto &v : idx) v = gen() % 40;
+    Allocator cpu = create_local_cpu_memory_allocator();
+    GenericTensorAccessorW hidx = cpu.allocate_tensor(shape({6, 5}, DataType::INT64));
+    memcpy(hidx.ptr, idx.data(), idx.size() * 8);
+    copy_accessor_data_to_l_from_r(inst.get_tensor_accessor(index), hidx);
+    perform_all_passes_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, dev);
+    // oracle: the same three steps, and the scatter / reshape / inverse transpose of a constant gradient
+    std::vector<int64_t> dims = {4, 6, 10}, tdims = {6, 4, 10};
+    int perm[3] = {1, 0, 2};
+    std::vector<float> tv(240), yv(30), dy(30, 1.0f / 6.0f), dr(240, 0.0f), dxw(240);
+    orc_transpose_nd(xv.data(), tv.data(), 3, dims.data(), perm, 0);
+    orc_gather_forward(tv.data(), idx.data(), yv.data(), 6, 40, 5, 1);
+    CHECK(to_host(inst.get_tensor_accessor(y)) == yv);
+    orc_gather_backward(dy.data(), idx.data(), dr.data(), 6, 40, 5, 1);
+    orc_transpose_nd(dr.data(), dxw.data(), 3, tdims.data(), perm, 0);  // (1, 0, 2) is its own inverse
+    CHECK(close(to_host(*inst.get_gradient_accessor(x)), dxw, 1e-6) && contains_non_zero(dxw));
   });
 }
 

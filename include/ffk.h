@@ -524,6 +524,56 @@ int ffk_concat_backward(ffk_stream_t stream, int dtype, void const *output_grad,
                         int64_t const *input_blk_elems, int num_inputs,
                         int64_t num_blocks, int accumulate);
 
+/* Split -- Kernels::Split::gpu_forward_kernel / gpu_backward_kernel
+ * (lib/kernels/include/kernels/split_kernels.h:9-25; lib/kernels/src/cuda/ops/
+ * split_kernels.cu): Concat read the other way.  outputs[i] takes its column
+ * window of every input row; backward: input_grad (+)= the output gradients
+ * side by side (the reference adds, add_with_stride = accumulate 1).         */
+int ffk_split_forward(ffk_stream_t stream, int dtype, void *const *outputs,
+                      void const *input, int64_t const *output_blk_elems,
+                      int num_outputs, int64_t num_blocks);
+int ffk_split_backward(ffk_stream_t stream, int dtype, void *input_grad,
+                       void const *const *output_grads,
+                       int64_t const *output_blk_elems, int num_outputs,
+                       int64_t num_blocks, int accumulate);
+
+/* ------------------------------------------------------------------------ */
+/* Transpose -- Kernels::Transpose::gpu_forward_kernel / gpu_backward_kernel
+ * (lib/kernels/include/kernels/transpose_kernels.h:11-19; lib/kernels/src/
+ * cuda/ops/transpose_kernels.cu:27-110).  Dims in FF order (dim 0 outermost);
+ * output dim i is input dim perm[i], up to 8 dims, any data type.
+ * backward: input_grad (+)= output_grad moved back through the inverse
+ *   permutation; accumulate 1 (the reference's intent, float and bf16) adds,
+ *   0 stores.  input_dims / perm describe the FORWARD transpose in both calls. */
+/* ------------------------------------------------------------------------ */
+int ffk_transpose_forward(ffk_stream_t stream, int dtype, void const *input,
+                          void *output, int num_dims, int64_t const *input_dims,
+                          int const *perm);
+int ffk_transpose_backward(ffk_stream_t stream, int dtype,
+                           void const *output_grad, void *input_grad,
+                           int num_dims, int64_t const *input_dims,
+                           int const *perm, int accumulate);
+
+/* ------------------------------------------------------------------------ */
+/* Gather -- Kernels::Gather::gpu_forward_kernel / gpu_backward_kernel
+ * (lib/kernels/include/kernels/gather_kernels.h:12-30; lib/kernels/src/cuda/
+ * ops/gather_kernels.cu:23-190).  Tensors viewed as [outer, dim_size, stride]
+ * around the gathered dim; index has the output's shape, int32 or int64:
+ *   output[o, j, s] = input[o, index[o, j, s], s]
+ * (an index outside [0, input_dim_size) yields 0 / is skipped).  Forward moves
+ * any data type; backward adds float gradients with hardware atomics, like the
+ * reference (input_grad is accumulated into).                                */
+/* ------------------------------------------------------------------------ */
+int ffk_gather_forward(ffk_stream_t stream, int dtype, int index_dtype,
+                       void const *input, void const *index, void *output,
+                       int64_t outer, int64_t input_dim_size,
+                       int64_t output_dim_size, int64_t stride);
+int ffk_gather_backward(ffk_stream_t stream, int index_dtype,
+                        float const *output_grad, void const *index,
+                        float *input_grad, int64_t outer,
+                        int64_t input_dim_size, int64_t output_dim_size,
+                        int64_t stride);
+
 #ifdef __cplusplus
 }
 #endif

@@ -66,6 +66,15 @@
  *      copy_with_stride / add_with_stride (src/cuda/cuda_helper.cu:160-173).
  *      The reference's test only asserts non-zero output (PARITY UNPINNED
  *      there); pinned by numpy.concatenate and by split-after-concat.
+ *  orc_transpose_nd           src/cuda/ops/transpose_kernels.cu:27-110 (the
+ *      intended `out = in` over the same stride walk; the reference's kernel
+ *      adds into uninitialised memory) and the CPU helper
+ *      tensor_accessor_transpose (src/kernels/tensor_accessor_unary_ops.cc),
+ *      whose known-answer test (test/src/kernels/tensor_accessor_unary_ops.cc)
+ *      is among the golden vectors.  Also pinned by numpy.transpose.
+ *  orc_gather_*               src/cuda/ops/gather_kernels.cu:23-82; the
+ *      reference has no value test (PARITY UNPINNED there); pinned by
+ *      numpy.take_along_axis and numpy.add.at.
  *  orc_cast_*                 src/kernels/cast_kernels_cpu.cc:6-20
  *      the reference tests only compare its GPU and CPU kernels on random
  *      data; pinned by numpy astype on exactly representable values and on
@@ -1094,5 +1103,63 @@ void orc_concat_backward(float const *dout, float *const *din,
       }
     }
     offset += blk[i];
+  }
+}
+
+/* --------------------------------------------------------------- transpose */
+void orc_transpose_nd(float const *in, float *out, int nd, int64_t const *in_dim,
+                      int const *perm, int accumulate) {
+  int64_t in_stride[8], out_dim[8], idx[8];
+  int64_t s = 1, total = 1;
+  for (int i = nd - 1; i >= 0; i--) {
+    in_stride[i] = s;
+    s *= in_dim[i];
+  }
+  for (int i = 0; i < nd; i++) {
+    out_dim[i] = in_dim[perm[i]];
+    total *= out_dim[i];
+    idx[i] = 0;
+  }
+  for (int64_t o = 0; o < total; o++) {
+    int64_t src = 0;
+    for (int i = 0; i < nd; i++) {
+      src += idx[i] * in_stride[perm[i]];
+    }
+    out[o] = accumulate ? out[o] + in[src] : in[src];
+    for (int i = nd - 1; i >= 0; i--) { /* next output coordinate, row-major */
+      if (++idx[i] < out_dim[i]) {
+        break;
+      }
+      idx[i] = 0;
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ gather */
+void orc_gather_forward(float const *in, int64_t const *index, float *out,
+                        int64_t outer, int64_t in_dim, int64_t out_dim,
+                        int64_t stride) {
+  int64_t total = outer * out_dim * stride;
+  for (int64_t o = 0; o < total; o++) {
+    int64_t outer_index = o / (stride * out_dim);
+    int64_t left_over = o % stride;
+    int64_t j = index[o];
+    out[o] = (j >= 0 && j < in_dim)
+                 ? in[outer_index * (stride * in_dim) + j * stride + left_over]
+                 : 0.0f;
+  }
+}
+
+void orc_gather_backward(float const *dout, int64_t const *index, float *din,
+                         int64_t outer, int64_t in_dim, int64_t out_dim,
+                         int64_t stride) {
+  int64_t total = outer * out_dim * stride;
+  for (int64_t o = 0; o < total; o++) {
+    int64_t outer_index = o / (stride * out_dim);
+    int64_t left_over = o % stride;
+    int64_t j = index[o];
+    if (j >= 0 && j < in_dim) {
+      din[outer_index * (stride * in_dim) + j * stride + left_over] += dout[o];
+    }
   }
 }

@@ -160,6 +160,17 @@ void orc_concat_backward(float const *dout, float *const *din,
                          int64_t const *blk, int n, int64_t num_blocks,
                          int accumulate);
 
+/* ---- Transpose: out dim i = in dim perm[i] (dims outermost first) ---- */
+void orc_transpose_nd(float const *in, float *out, int nd, int64_t const *in_dim,
+                      int const *perm, int accumulate);
+/* ---- Gather along the middle dim of [outer, dim, stride] ---- */
+void orc_gather_forward(float const *in, int64_t const *index, float *out,
+                        int64_t outer, int64_t in_dim, int64_t out_dim,
+                        int64_t stride);
+void orc_gather_backward(float const *dout, int64_t const *index, float *din,
+                         int64_t outer, int64_t in_dim, int64_t out_dim,
+                         int64_t stride);
+
 #ifdef __cplusplus
 }
 #endif

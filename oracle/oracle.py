@@ -434,3 +434,42 @@ def concat_backward(out_grad, input_grads, axis, accumulate=True):
     lib().orc_concat_backward(_p(g), ptrs, blks, ctypes.c_int(len(dins)), c_i64(num_blocks),
                               ctypes.c_int(1 if accumulate else 0))
     return dins
+
+
+def transpose_nd(x, perm, into=None):
+    """out = x permuted (output dim i = input dim perm[i]); with `into`, added to it."""
+    x = _f32(x)
+    nd = x.ndim
+    out = np.empty([x.shape[p] for p in perm], np.float32) if into is None else _f32(into).copy()
+    dims = (c_i64 * nd)(*x.shape)
+    pm = (ctypes.c_int * nd)(*perm)
+    lib().orc_transpose_nd(_p(x), _p(out), ctypes.c_int(nd), dims, pm, ctypes.c_int(0 if into is None else 1))
+    return out
+
+
+def _gather_view(shape, out_shape, dim):
+    dim = dim if dim >= 0 else len(shape) + dim
+    outer = int(np.prod(shape[:dim], dtype=np.int64))
+    stride = int(np.prod(shape[dim + 1:], dtype=np.int64))
+    return outer, int(shape[dim]), int(out_shape[dim]), stride
+
+
+def gather_forward(x, index, dim):
+    x = _f32(x)
+    idx = np.ascontiguousarray(index, dtype=np.int64)
+    outer, ind, outd, stride = _gather_view(x.shape, idx.shape, dim)
+    out = np.empty(idx.shape, np.float32)
+    lib().orc_gather_forward(_p(x), idx.ctypes.data_as(ctypes.c_void_p), _p(out), c_i64(outer), c_i64(ind),
+                             c_i64(outd), c_i64(stride))
+    return out
+
+
+def gather_backward(out_grad, index, in_grad, dim):
+    """Returns in_grad with the gradient scattered into it."""
+    g = _f32(out_grad)
+    idx = np.ascontiguousarray(index, dtype=np.int64)
+    din = _f32(in_grad).copy()
+    outer, ind, outd, stride = _gather_view(din.shape, idx.shape, dim)
+    lib().orc_gather_backward(_p(g), idx.ctypes.data_as(ctypes.c_void_p), _p(din), c_i64(outer), c_i64(ind),
+                              c_i64(outd), c_i64(stride))
+    return din

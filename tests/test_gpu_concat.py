@@ -71,3 +71,22 @@ def test_concat_on_unaligned_views(ffk, oracle):
     da.copy_(to_dev(a, torch))
     out = ffk.concat_forward([da, to_dev(b, torch)], 1)
     assert np.array_equal(to_np(out), np.concatenate([a, b], axis=1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_split_is_concat_read_the_other_way(ffk, oracle, dtype):
+    say("split", dtype)
+    g = rng(8)
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda a: a)
+    x = rnd(g.standard_normal((6, 29, 8)).astype(np.float32))
+    sizes = [5, 1, 16, 7]
+    outs = ffk.split_forward(to_dev(x, torch, dtype), sizes, 1)
+    for got, want in zip(outs, np.split(x, np.cumsum(sizes)[:-1], axis=1)):
+        assert np.array_equal(to_np(got), want)
+    douts = [rnd(g.standard_normal(o.shape).astype(np.float32)) for o in outs]
+    old = rnd(g.standard_normal(x.shape).astype(np.float32))
+    for accumulate in (True, False):
+        din = to_dev(old, torch, dtype)
+        ffk.split_backward([to_dev(d, torch, dtype) for d in douts], din, 1, accumulate=accumulate)
+        want = oracle.concat_forward(douts, 1) + (old if accumulate else 0.0)
+        assert np.array_equal(to_np(din), rnd(want.astype(np.float32)))

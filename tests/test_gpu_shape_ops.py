@@ -1,0 +1,88 @@
+"""Transpose and Gather through the C ABI against the oracle.  Transpose moves bits (and
+makes one fp32 add per element when accumulating): exact.  Gather forward is exact;
+its backward adds with atomics in an order that varies, so fp32 tolerance 1e-5."""
+import itertools
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from util import assert_close, bf16_round, rng, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+CASES = [
+    ((2, 3, 4, 5), None),            # every permutation
+    ((64, 96), [(1, 0)]),            # plain 2-D, whole tiles and a ragged one
+    ((70, 130), [(1, 0)]),
+    ((8, 512, 16, 64), [(0, 2, 1, 3), (0, 2, 3, 1), (3, 2, 1, 0)]),   # the head split of attention
+    ((3, 1, 40, 1, 24), [(2, 1, 0, 3, 4), (4, 3, 2, 1, 0)]),          # extents of one
+    ((5,), [(0,)]),
+]
+
+
+@pytest.mark.parametrize("shape,perms", CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_transpose_forward_backward(ffk, oracle, shape, perms, dtype):
+    g = rng(5)
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda a: a)
+    x = rnd(g.standard_normal(shape).astype(np.float32))
+    xd = to_dev(x, torch, dtype)
+    for perm in (perms or list(itertools.permutations(range(len(shape))))):
+        say("transpose", shape, perm, dtype)
+        out = ffk.transpose_forward(xd, perm)
+        want = oracle.transpose_nd(x, perm)
+        assert tuple(out.shape) == want.shape
+        assert np.array_equal(to_np(out), want), perm
+        # backward: the inverse permutation of the output gradient, added or stored
+        dout = rnd(g.standard_normal(want.shape).astype(np.float32))
+        old = rnd(g.standard_normal(shape).astype(np.float32))
+        inverse = np.argsort(perm)
+        for accumulate in (True, False):
+            din = to_dev(old, torch, dtype)
+            ffk.transpose_backward(to_dev(dout, torch, dtype), din, perm, accumulate=accumulate)
+            ref = np.transpose(dout, inverse) + (old if accumulate else 0.0)
+            assert np.array_equal(to_np(din), rnd(ref.astype(np.float32))), (perm, accumulate)
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64, torch.bool, torch.float16, torch.float64])
+def test_transpose_moves_any_data_type(ffk, dtype):
+    say("transpose", dtype)
+    x = (torch.arange(6 * 70 * 9, device="cuda").reshape(6, 70, 9) % (2 if dtype == torch.bool else 1000)).to(dtype)
+    for perm in ((2, 0, 1), (0, 2, 1), (1, 0, 2)):
+        assert torch.equal(ffk.transpose_forward(x, perm), x.permute(perm).contiguous())
+    with pytest.raises(ffk.FFKError, match="not a permutation"):
+        ffk.transpose_forward(x, (0, 0, 1))
+    if dtype not in (torch.float32, torch.bfloat16):
+        with pytest.raises(ffk.FFKError, match="adding supports"):
+            ffk.transpose_backward(x.permute(1, 0, 2).contiguous(), torch.zeros_like(x), (1, 0, 2), accumulate=True)
+
+
+@pytest.mark.parametrize("dim", [0, 1, 2])
+@pytest.mark.parametrize("itype", [torch.int32, torch.int64])
+def test_gather_forward_backward(ffk, oracle, dim, itype):
+    say("gather", dim, itype)
+    g = rng(6)
+    x = g.standard_normal((7, 33, 20)).astype(np.float32)
+    shape = list(x.shape)
+    shape[dim] = 11
+    idx = g.integers(0, x.shape[dim], size=shape)
+    idx.flat[::97] = -1                       # out-of-range entries read 0 and scatter nothing
+    out = ffk.gather_forward(to_dev(x, torch), to_dev(idx, torch, itype), dim)
+    assert np.array_equal(to_np(out), oracle.gather_forward(x, idx, dim))
+    dout = g.standard_normal(shape).astype(np.float32)
+    old = g.standard_normal(x.shape).astype(np.float32)
+    din = to_dev(old, torch)
+    ffk.gather_backward(to_dev(dout, torch), to_dev(idx, torch, itype), din, dim)
+    assert_close(to_np(din), oracle.gather_backward(dout, idx, old, dim), 1e-5, "gather backward")
+    # bf16 values move bit for bit
+    xb = bf16_round(x)
+    outb = ffk.gather_forward(to_dev(xb, torch, torch.bfloat16), to_dev(idx, torch, itype), dim)
+    assert np.array_equal(to_np(outb), oracle.gather_forward(xb, idx, dim))
