@@ -319,14 +319,32 @@ __device__ __forceinline__ void wait_vmcnt() {
 // orders these loads against its LDS reads itself, with wait_vmcnt and the
 // barrier.  Loads the compiler does know about stay correct: its vmcnt waits
 // count these extra, younger loads too, which only makes them stricter.
-__device__ __forceinline__ void lds_dma16(void const *g, unsigned lds_byte_addr) {
+// The load is the buffer form (a scalar resource descriptor for the operand
+// panel, a scalar byte offset for what is uniform, one 32-bit byte offset per
+// lane that never changes) rather than the flat-global form with a 64-bit
+// address per lane: no vector address arithmetic remains in the k-loop, and
+// the instruction issues through the vector-memory port alone.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void lds_dma16(i32x4 rsrc, unsigned lane_byte_off, unsigned uniform_byte_off,
+                                          unsigned lds_byte_addr) {
   // lds_byte_addr is wave-uniform and held in a scalar register by the caller
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
-               : "s"(lds_byte_addr), "v"(g)
+               : "s"(lds_byte_addr), "v"(lane_byte_off), "s"(rsrc), "s"(uniform_byte_off)
                : "memory");  // M0 is not in the clobber list (the compiler rejects
                              // reserved registers there); nothing else in these
                              // kernels uses M0 (no GDS, message or relative-move ops)
+}
+// Raw buffer descriptor over everything from `base` on: stride 0, no bound
+// (the callers' offsets are checked on the host), 32-bit data format.
+__device__ __forceinline__ i32x4 buffer_resource(void const *base) {
+  uint64_t const a = reinterpret_cast<uint64_t>(base);
+  i32x4 r;
+  r[0] = (int)__builtin_amdgcn_readfirstlane((unsigned)a);
+  r[1] = (int)(__builtin_amdgcn_readfirstlane((unsigned)(a >> 32)) & 0xffffu);
+  r[2] = -1;
+  r[3] = 0x00020000;
+  return r;
 }
 // The LDS byte address of a __shared__ object, as a scalar.
 __device__ __forceinline__ unsigned lds_address_of(void *p) {
@@ -358,7 +376,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   constexpr int RPW = 256 / (BK * 2);      // K-contiguous rows per 256-byte bank window
   constexpr int CS = WN + 8;               // row stride of a wave's staged output tile
   static_assert(A_ELEMS / 8 % NT == 0 && B_ELEMS / 8 % NT == 0, "tile/threads");
-  static_assert((STAGES - 1) * LPT <= 63, "vmcnt range");
+  static_assert(STAGES * LPT <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
 
@@ -388,22 +406,22 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
     if (!TA) {
       int row = c / CPRK, pc = c % CPRK;
       int lc = pc ^ ((row / RPW) & (CPRK - 1));
-      voff_a = (unsigned)(row * lda + lc * 8);
+      voff_a = (unsigned)(row * lda + lc * 8) * 2u;
     } else {
       constexpr int CPR = BM / 8;
       int krow = c / CPR, pc = c % CPR;
       int lc = ((((pc >> 2) ^ (krow & 3)) << 2) | (pc & 3));
-      voff_a = (unsigned)(krow * lda + lc * 8);
+      voff_a = (unsigned)(krow * lda + lc * 8) * 2u;
     }
     if (!TBL) {
       int row = c / CPRK, pc = c % CPRK;
       int lc = pc ^ ((row / RPW) & (CPRK - 1));
-      voff_b = (unsigned)(row * ldb + lc * 8);
+      voff_b = (unsigned)(row * ldb + lc * 8) * 2u;
     } else {
       constexpr int CPR = BN / 8;
       int krow = c / CPR, pc = c % CPR;
       int lc = ((((pc >> 2) ^ (krow & 3)) << 2) | (pc & 3));
-      voff_b = (unsigned)(krow * ldb + lc * 8);
+      voff_b = (unsigned)(krow * ldb + lc * 8) * 2u;
     }
   }
   int64_t const step_a = TA ? (int64_t)(NT * 8 / BM) * lda : (int64_t)ROWS_PER_LOAD_KC * lda;
@@ -414,19 +432,26 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // LDS destinations of the direct loads are scalar byte addresses: base + stage + chunk row
   unsigned const smem_addr = lds_address_of(smem);
   int const wave_s = __builtin_amdgcn_readfirstlane(wave);
-  auto issue = [&](int kt, int stage) {
+  // Loads [first, first + count) of a k-tile's LPT direct loads (A's, then B's).
+  // (first and count are constants once the caller's loops are unrolled)
+  auto issue_some = [&](int kt, int stage, int first, int count) __attribute__((always_inline)) {
     unsigned const sa = smem_addr + (unsigned)(stage * STAGE_ELEMS) * 2u;
     unsigned const sb = sa + (unsigned)A_ELEMS * 2u;
-    bf16 const *ga = panel_a + (TA ? (int64_t)(kt0 + kt) * BK * lda : (int64_t)(kt0 + kt) * BK);
-    bf16 const *gb = panel_b + (TBL ? (int64_t)(kt0 + kt) * BK * ldb : (int64_t)(kt0 + kt) * BK);
+    i32x4 const ra = buffer_resource(panel_a + (TA ? (int64_t)(kt0 + kt) * BK * lda : (int64_t)(kt0 + kt) * BK));
+    i32x4 const rb = buffer_resource(panel_b + (TBL ? (int64_t)(kt0 + kt) * BK * ldb : (int64_t)(kt0 + kt) * BK));
 #pragma unroll
-    for (int i = 0; i < A_LOADS; i++) {
-      lds_dma16(ga + i * step_a + voff_a, sa + (unsigned)(i * NW + wave_s) * 1024u);
+    for (int q = 0; q < LPT; q++) {
+      if (q < first || q >= first + count) continue;
+      if (q < A_LOADS) {
+        lds_dma16(ra, voff_a, (unsigned)(q * step_a) * 2u, sa + (unsigned)(q * NW + wave_s) * 1024u);
+      } else {
+        int const i = q - A_LOADS;
+        lds_dma16(rb, voff_b, (unsigned)(i * step_b) * 2u, sb + (unsigned)(i * NW + wave_s) * 1024u);
+      }
     }
-#pragma unroll
-    for (int i = 0; i < B_LOADS; i++) {
-      lds_dma16(gb + i * step_b + voff_b, sb + (unsigned)(i * NW + wave_s) * 1024u);
-    }
+  };
+  auto issue = [&](int kt, int stage) {
+    issue_some(kt, stage, 0, LPT);
   };
 
   // Fragment readers (see the layouts above).  Everything lane-dependent in
@@ -489,9 +514,22 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   constexpr int NB = PF + 1;  // fragment buffers
   static_assert(KS % NB == 0, "buffer index must not depend on the tile");
   static_assert(STAGES >= 2, "one stage in use, at least one in flight");
+  // With three or more stages a refill is not issued in one burst after the
+  // barrier that frees its stage, but in KS equal parts: part 0 after that
+  // barrier, part j in k-step j-1 of the following tile.  A burst of LPT loads
+  // from every wave at once overruns the memory pipeline's instruction queue;
+  // a wave that cannot issue its next load cannot issue its next MFMA either.
+  constexpr bool SPREAD = STAGES >= 3 && LPT % KS == 0;
+  constexpr int PART = SPREAD ? LPT / KS : LPT;
 #pragma unroll
   for (int s = 0; s < STAGES; s++) {
-    if (s < KT) issue(s, s);
+    if (s < KT) {
+      if (SPREAD && s == STAGES - 1) {
+        issue_some(s, s, 0, PART);  // tile 0's steps issue the rest
+      } else {
+        issue(s, s);
+      }
+    }
   }
   // Fragments are double-buffered in registers: while the MFMAs of one k-step
   // run, the LDS reads of the next step (of the next tile, at a tile's last
@@ -511,7 +549,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   };
   // Tile 0 must have landed (STAGES-1 younger tiles may still be in flight).
   if (STAGES - 1 < KT) {
-    wait_vmcnt<(STAGES - 1) * LPT>();
+    wait_vmcnt<(STAGES - 2) * LPT + PART>();
   } else {
     wait_vmcnt<0>();
   }
@@ -536,6 +574,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       __builtin_amdgcn_sched_barrier(0);
       acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0], af[cur][0], acc[0][0], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
+      if (SPREAD && kk + 1 < KS) {
+        // part kk+1 of the tile that goes into the stage freed one tile ago
+        if (STEADY || kt + STAGES - 1 < KT) {
+          issue_some(kt + STAGES - 1, (kt + STAGES - 1) % STAGES, (kk + 1) * PART, PART);
+        }
+      }
       if (kk + PF < KS) {
         read_frags(nxt, stage, kk + PF);
       } else if (STEADY || kt + 1 < KT) {
@@ -550,7 +594,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
             wait_vmcnt<0>();
           }
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-          if (STEADY || kt + STAGES < KT) issue(kt + STAGES, stage);
+          if (STEADY || kt + STAGES < KT) {
+            issue_some(kt + STAGES, stage, 0, PART);
+          }
         }
         read_frags(nxt, (kt + 1) % STAGES, kk + PF - KS);
       }
@@ -902,7 +948,9 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
   int const variant = gemm_variant_override();
   // the pipelined kernels fetch the bias in 8-byte pieces
   bool const aux_ok = reinterpret_cast<uintptr_t>(ep.bias) % 8 == 0;
-  if (c_vec && aux_ok && K % 64 == 0 && variant != 1) {
+  // the direct loads address an operand panel with 32-bit byte offsets
+  bool const panel_ok = 2 * 256 * std::max(lda, ldb) < (int64_t(1) << 31);
+  if (c_vec && aux_ok && panel_ok && K % 64 == 0 && variant != 1) {
     bool const fits256 = M % 256 == 0 && N % 256 == 0;
     bool const fits128 = M % 128 == 0 && N % 128 == 0;
     int64_t const t256 = fits256 ? (int64_t)(M / 256) * (N / 256) : 0;
@@ -911,8 +959,11 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
     // traffic per flop and fetch whole 128-byte lines; they win whenever they
     // still occupy most CUs.  Otherwise 128x128x64 tiles with 8 waves of 64x32
     // keep two waves per SIMD on every CU.
-    if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) {
+    if (variant == 2562 && fits256) {
       return launch_pipe<256, 256, 128, 64, 64, 2, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+    }
+    if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) {
+      return launch_pipe<256, 256, 128, 64, 32, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
     if ((variant == 0 && t128 >= kNumCU / 2) || (variant == 128 && fits128)) {
       return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
