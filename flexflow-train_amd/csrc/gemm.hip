@@ -625,38 +625,29 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // Each wave stages its own WM x WN tile and writes it out in 16-byte chunks.
   bf16 *cs = smem + wave * (WM * CS);
   constexpr int CCH = WM * WN / 8 / 64;  // 16-byte chunks per lane
-  // The lane's bias values depend on (j, g, lane / 32) only: fetch them once.
-  float bv[TN][4][4];
-#pragma unroll
-  for (int j = 0; j < TN; j++)
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      u32x2 raw = {0u, 0u};
-      if (bias != nullptr) {
-        raw = *reinterpret_cast<u32x2 const *>(bias + n0 + wn0 + j * 32 + 8 * g + 4 * (lane >> 5));
-      }
-      bv[j][g][0] = __uint_as_float(raw[0] << 16);
-      bv[j][g][1] = __uint_as_float(raw[0] & 0xffff0000u);
-      bv[j][g][2] = __uint_as_float(raw[1] << 16);
-      bv[j][g][3] = __uint_as_float(raw[1] & 0xffff0000u);
-    }
   // The activation is a compile-time functor here: a per-element switch inside
   // the unrolled loops made the epilogue several times longer than the GEMM's
   // own store traffic.
   auto finish = [&](auto actf) __attribute__((always_inline)) {
     bf16 *const dst = C;
     bool const add_old = accumulate != 0;
+    // The lane's bias values depend on (j, g, lane / 32) only: they are
+    // fetched once per (j, g) and used for the TM row blocks.
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-      int const m = i * 32 + (lane & 31);
+    for (int j = 0; j < TN; j++) {
 #pragma unroll
-      for (int j = 0; j < TN; j++) {
+      for (int g = 0; g < 4; g++) {
+        int const n = j * 32 + 8 * g + 4 * (lane >> 5);
+        u32x2 raw = {0u, 0u};
+        if (bias != nullptr) raw = *reinterpret_cast<u32x2 const *>(bias + n0 + wn0 + n);
+        float const bv[4] = {__uint_as_float(raw[0] << 16), __uint_as_float(raw[0] & 0xffff0000u),
+                             __uint_as_float(raw[1] << 16), __uint_as_float(raw[1] & 0xffff0000u)};
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-          int const n = j * 32 + 8 * g + 4 * (lane >> 5);
+        for (int i = 0; i < TM; i++) {
+          int const m = i * 32 + (lane & 31);
           float v[4];
 #pragma unroll
-          for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + bv[j][g][e];
+          for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + bv[e];
 #pragma unroll
           for (int e = 0; e < 4; e++) v[e] = actf(v[e]);
           if (add_old) {
