@@ -4,10 +4,14 @@
 // state and reserve space are opaque (lib/kernels/src/cuda/ops/
 // dropout_kernels.cu:24-95).  Here the keep mask is a pure function of
 // (seed, element index): Philox4x32-10, key = (seed lo, seed hi), counter =
-// (block lo, block hi, 0, 0) with block = (offset + i) / 4, and element
-// (offset + i) uses word (offset + i) % 4; it is kept iff
-// word >= ceil(rate * 2^32).  Nothing is stored between forward and backward:
-// backward regenerates the mask, so both directions move 2 tensors only.
+// (block lo, block hi, 0, 0) with block = (offset + i) / 8; element
+// e = offset + i uses 16 bits of the block's 128: half (e % 8) % 2 (0 = low)
+// of word (e % 8) / 2, and is kept iff half >= ceil(rate * 2^16).  Sixteen
+// bits per element keep the generator's integer multiplies (20 per block, all
+// quarter-rate) off the critical path: with a 32-bit word per element the
+// bf16 passes were bound by them, not by HBM.  Nothing is stored between
+// forward and backward: backward regenerates the mask, so both directions
+// move 2 tensors only.
 #include "ffk_common.h"
 #include "fused_ops.h"
 #include <math.h>
@@ -40,13 +44,23 @@ __device__ __forceinline__ void philox4x32_10(uint64_t block, PhiloxKey key,
 struct DropoutParams {
   PhiloxKey key;
   uint64_t offset;
-  uint32_t threshold;  // keep iff word >= threshold ...
-  int drop_all;        // ... unless rate rounds to 2^32 (everything dropped)
+  uint32_t threshold;  // keep iff the element's 16 bits >= threshold (0 .. 65536)
   float scale;         // 1 / (1 - rate)
 };
 
-__device__ __forceinline__ bool keep(uint32_t word, DropoutParams const &p) {
-  return !p.drop_all && word >= p.threshold;
+// h: position of the element in its block of 8
+__device__ __forceinline__ bool keep(uint32_t const (&w)[4], int h, DropoutParams const &p) {
+  uint32_t const word = w[h >> 1];
+  uint32_t const half = (h & 1) ? (word >> 16) : (word & 0xffffu);
+  return half >= p.threshold;
+}
+__device__ __forceinline__ bool keep_dynamic(uint32_t const (&w)[4], uint32_t h, DropoutParams const &p) {
+  uint32_t word = w[0];
+  if ((h >> 1) == 1) word = w[1];
+  if ((h >> 1) == 2) word = w[2];
+  if ((h >> 1) == 3) word = w[3];
+  uint32_t const half = (h & 1) ? (word >> 16) : (word & 0xffffu);
+  return half >= p.threshold;
 }
 
 constexpr int kDropThreads = 256;
@@ -61,7 +75,8 @@ constexpr int kDropThreads = 256;
 //                                             before the mask is applied)
 enum DropMode { kDropPlain = 0, kDropAddResidual = 1, kDropGeluGrad = 2, kDropAfterGelu = 3 };
 
-// offset % 4 == 0, 16-byte aligned pointers: each lane owns whole Philox blocks.
+// offset % 8 == 0, 16-byte aligned pointers: a lane's V elements (8 bf16 or 4
+// float) are a whole Philox block or an aligned half of one.
 template <typename T, bool ACC, int MODE>
 __global__ __launch_bounds__(kDropThreads) void dropout_vec_kernel(
     T const *__restrict__ X, T const *__restrict__ AUX, T *Y, int64_t n, DropoutParams p) {
@@ -81,18 +96,20 @@ __global__ __launch_bounds__(kDropThreads) void dropout_vec_kernel(
       VecIO<T>::load_stream(AUX + i * V, aux);
     }
     if (ACC) VecIO<T>::load(Y + i * V, y);
-    uint64_t const blk0 = (p.offset + (uint64_t)i * V) >> 2;
+    static_assert(V == 4 || V == 8, "a lane owns a block of 8 elements or half of one");
+    uint64_t const e0 = p.offset + (uint64_t)i * V;
+    uint32_t w[4];
+    philox4x32_10(e0 >> 3, p.key, w);
+    if (V == 4 && (e0 & 4)) {  // upper half of the block
+      w[0] = w[2];
+      w[1] = w[3];
+    }
 #pragma unroll
-    for (int b = 0; b < V / 4; b++) {
-      uint32_t w[4];
-      philox4x32_10(blk0 + b, p.key, w);
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        float v = keep(w[e], p) ? x[4 * b + e] * p.scale : 0.0f;
-        if (MODE == kDropAddResidual) v = storage_round<T>(v) + aux[4 * b + e];
-        if (MODE == kDropGeluGrad) v = storage_round<T>(v) * gelu_derivative(aux[4 * b + e]);
-        y[4 * b + e] = ACC ? y[4 * b + e] + v : v;
-      }
+    for (int e = 0; e < V; e++) {
+      float v = keep(w, e, p) ? x[e] * p.scale : 0.0f;
+      if (MODE == kDropAddResidual) v = storage_round<T>(v) + aux[e];
+      if (MODE == kDropGeluGrad) v = storage_round<T>(v) * gelu_derivative(aux[e]);
+      y[e] = ACC ? y[e] + v : v;
     }
     VecIO<T>::store(Y + i * V, y);
   }
@@ -106,12 +123,8 @@ __global__ __launch_bounds__(kDropThreads) void dropout_scalar_kernel(
   for (int64_t i = first + (int64_t)blockIdx.x * kDropThreads + threadIdx.x; i < n; i += stride) {
     uint64_t const e = p.offset + (uint64_t)i;
     uint32_t w[4];
-    philox4x32_10(e >> 2, p.key, w);
-    uint32_t word = w[0];
-    if ((e & 3) == 1) word = w[1];
-    if ((e & 3) == 2) word = w[2];
-    if ((e & 3) == 3) word = w[3];
-    float v = keep(word, p) ? VecIO<T>::load1(X + i) * p.scale : 0.0f;
+    philox4x32_10(e >> 3, p.key, w);
+    float v = keep_dynamic(w, (uint32_t)(e & 7), p) ? VecIO<T>::load1(X + i) * p.scale : 0.0f;
     if (ACC) v += VecIO<T>::load1(Y + i);
     VecIO<T>::store1(Y + i, v);
   }
@@ -123,21 +136,15 @@ __global__ __launch_bounds__(kDropThreads) void dropout_mask_kernel(
   for (int64_t i = (int64_t)blockIdx.x * kDropThreads + threadIdx.x; i < n; i += stride) {
     uint64_t const e = p.offset + (uint64_t)i;
     uint32_t w[4];
-    philox4x32_10(e >> 2, p.key, w);
-    uint32_t word = w[0];
-    if ((e & 3) == 1) word = w[1];
-    if ((e & 3) == 2) word = w[2];
-    if ((e & 3) == 3) word = w[3];
-    mask[i] = keep(word, p) ? 1 : 0;
+    philox4x32_10(e >> 3, p.key, w);
+    mask[i] = keep_dynamic(w, (uint32_t)(e & 7), p) ? 1 : 0;
   }
 }
 
 static int make_params(char const *who, float rate, uint64_t seed,
                        uint64_t offset, DropoutParams &p) {
   FFK_REQUIRE(rate >= 0.0f && rate <= 1.0f, "%s: rate %f outside [0, 1]", who, (double)rate);
-  double t = ceil((double)rate * 4294967296.0);
-  p.drop_all = t >= 4294967296.0;
-  p.threshold = p.drop_all ? 0xffffffffu : (uint32_t)t;
+  p.threshold = (uint32_t)ceil((double)rate * 65536.0);  // 65536 (rate above 1 - 2^-16): everything dropped
   p.key.k0 = (uint32_t)seed;
   p.key.k1 = (uint32_t)(seed >> 32);
   p.offset = offset;
@@ -159,7 +166,7 @@ static int dropout_run(hipStream_t st, void const *x, void *y, int64_t n,
   T const *X = static_cast<T const *>(x);
   T *Y = static_cast<T *>(y);
   int64_t done = 0;
-  if ((p.offset & 3) == 0 && aligned16(x) && aligned16(y) && n >= V) {
+  if ((p.offset & 7) == 0 && aligned16(x) && aligned16(y) && n >= V) {
     int64_t nvec = n / V;
     dropout_vec_kernel<T, ACC, kDropPlain><<<grid_for(nvec), kDropThreads, 0, st>>>(X, nullptr, Y, n, p);
     FFK_CHECK_LAUNCH();
@@ -189,7 +196,7 @@ bool dropout_fusable(int dtype, void const *x, void const *aux, void const *y,
                      int64_t n, uint64_t offset) {
   int64_t const V = dtype == FFK_BF16 ? 8 : 4;
   return (dtype == FFK_BF16 || dtype == FFK_FLOAT) && n > 0 && n % V == 0 &&
-         (offset & 3) == 0 && aligned16(x) && aligned16(aux) && aligned16(y);
+         (offset & 7) == 0 && aligned16(x) && aligned16(aux) && aligned16(y);
 }
 
 static int dropout_fused(char const *who, int mode, hipStream_t st, int dtype,

@@ -254,8 +254,9 @@ int ffk_softmax_backward(ffk_stream_t stream, int dtype, void const *output,
  * (dropout_kernels_gpu.h:18-26; lib/kernels/src/cuda/ops/dropout_kernels.cu:
  * 60-95, where the mask comes from cuDNN's opaque generator).  Here the mask
  * is a pure function of (seed, offset + element index): Philox4x32-10 with
- * key = (seed low 32, seed high 32), counter = ((offset+i)/4 low, high, 0, 0),
- * word (offset+i) % 4; element i is kept iff word >= ceil(rate * 2^32);
+ * key = (seed low 32, seed high 32), counter = (e/8 low, e/8 high, 0, 0) for
+ * e = offset + i; element e owns 16 of the block's 128 bits -- half (e%8)%2
+ * (0 = low) of word (e%8)/2 -- and is kept iff they are >= ceil(rate * 2^16);
  * kept elements are scaled by 1/(1-rate).  No mask is stored: backward
  * regenerates it.                                                            */
 /* ------------------------------------------------------------------------ */

@@ -625,34 +625,38 @@ void orc_philox4x32_10(uint32_t const ctr_in[4], uint32_t const key_in[2],
   out[0] = c[0]; out[1] = c[1]; out[2] = c[2]; out[3] = c[3];
 }
 
-static uint64_t dropout_threshold(float rate) {
-  double t = ceil((double)rate * 4294967296.0);
+static uint32_t dropout_threshold(float rate) {
+  double t = ceil((double)rate * 65536.0);
   if (t < 0) {
     t = 0;
   }
-  if (t > 4294967296.0) {
-    t = 4294967296.0;
+  if (t > 65536.0) {
+    t = 65536.0;
   }
-  return (uint64_t)t;
+  return (uint32_t)t;
 }
 
-/* element i (global index e = offset + i): counter (e/4 lo, e/4 hi, 0, 0),
- * key (seed lo, seed hi), word e % 4; kept iff word >= ceil(rate * 2^32). */
+/* element i (global index e = offset + i): counter (e/8 lo, e/8 hi, 0, 0),
+ * key (seed lo, seed hi); the element's 16 bits are half (e%8)%2 (0 = low) of
+ * word (e%8)/2; kept iff they are >= ceil(rate * 2^16). */
 void orc_dropout_mask(uint8_t *mask, int64_t n, float rate, uint64_t seed,
                       uint64_t offset) {
-  uint64_t thr = dropout_threshold(rate);
+  uint32_t thr = dropout_threshold(rate);
   uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
   uint64_t cached_block = ~(uint64_t)0;
   uint32_t w[4] = {0, 0, 0, 0};
   for (int64_t i = 0; i < n; i++) {
     uint64_t e = offset + (uint64_t)i;
-    uint64_t blk = e >> 2;
+    uint64_t blk = e >> 3;
     if (blk != cached_block) {
       uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), 0u, 0u};
       orc_philox4x32_10(ctr, key, w);
       cached_block = blk;
     }
-    mask[i] = ((uint64_t)w[e & 3] >= thr) ? 1 : 0;
+    uint32_t h = (uint32_t)(e & 7);
+    uint32_t word = w[h >> 1];
+    uint32_t half = (h & 1) ? (word >> 16) : (word & 0xffffu);
+    mask[i] = (half >= thr) ? 1 : 0;
   }
 }
 

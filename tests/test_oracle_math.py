@@ -179,11 +179,13 @@ def test_dropout_stream_properties(oracle):
     # pure function of (seed, offset + i): a shifted window equals a slice
     assert np.array_equal(oracle.dropout_mask(1000, rate, seed, offset=37), m[37:1037])
     assert not np.array_equal(oracle.dropout_mask(n, rate, seed + 1), m)
-    # element e uses word e % 4 of block e / 4 with threshold ceil(rate * 2^32)
-    thr = int(np.ceil(np.float32(rate).astype(np.float64) * 2 ** 32))
-    for e in (0, 1, 2, 3, 4, 9, 1022):
-        w = oracle.philox4x32_10([e // 4, 0, 0, 0], [seed & 0xffffffff, seed >> 32])
-        assert m[e] == (1 if int(w[e % 4]) >= thr else 0)
+    # element e uses 16 bits of block e / 8: half (e % 8) % 2 of word (e % 8) / 2, threshold ceil(rate * 2^16)
+    thr = int(np.ceil(np.float32(rate).astype(np.float64) * 2 ** 16))
+    for e in (0, 1, 2, 3, 4, 7, 8, 9, 1022, 1023):
+        w = oracle.philox4x32_10([e // 8, 0, 0, 0], [seed & 0xffffffff, seed >> 32])
+        word = int(w[(e % 8) // 2])
+        half = (word >> 16) if e % 2 else (word & 0xffff)
+        assert m[e] == (1 if half >= thr else 0)
     x = rng(7).standard_normal((n,)).astype(np.float32)
     y = oracle.dropout_forward(x, rate, seed)
     scale = np.float32(1.0) / (np.float32(1.0) - np.float32(rate))
