@@ -19,6 +19,11 @@
 //    BF16 values at the first update, or when sync_master_weights is called).
 //  * a dropout layer's mask differs per layer and per iteration: seed + layer
 //    index, offset = iteration * elements.
+//  * the weights the instance places itself are grouped by data type: value,
+//    gradient, master and moments of a group lie in parallel arrays, and the
+//    UPD invocation of the group's first weight updates all of them with one
+//    launch (the UPD invocations of the other members are empty).  A weight
+//    bound to caller memory is updated by its own launch.
 #pragma once
 #include "kernels/accessor.h"
 #include "kernels/allocation.h"

@@ -259,7 +259,8 @@ ComputationGraphInstance create_computation_graph_instance(
       if (layer.inputs[1] == layer.inputs[2] && layer.inputs[0] != layer.inputs[1]) acc = true;
       if (layer.inputs[0] == layer.inputs[1] && layer.inputs[0] != layer.inputs[2]) acc = true;
       if (layer.inputs[0] == layer.inputs[2] && layer.inputs[0] != layer.inputs[1]) acc = true;
-      cleared[layer.weights.at(0).raw] = true;  // the weight gradient is always added into
+      // a weight used by one layer has its gradient stored; a shared one is added into
+      if (writers[layer.weights.at(0).raw] > 1) cleared[layer.weights.at(0).raw] = true;
     } else if (auto const *a = std::get_if<EmbeddingAttrs>(&oa)) {
       p.scratch_bytes = ffk_embedding_backward_workspace_bytes(numel(layer.inputs[0]), a->num_entries);
       cleared[layer.weights.at(0).raw] = true;
@@ -313,21 +314,77 @@ ComputationGraphInstance create_computation_graph_instance(
   }
   if (st->logit.has_value()) cleared[st->logit->raw] = false;  // written by the loss before any producer adds
 
-  // -- placement: cleared gradients first, then everything else
+  // -- placement: cleared gradients first, then everything else.
+  // Trainable weights that the instance places itself are laid out in groups
+  // (same data type, gradient cleared or not): within a group the gradient, the
+  // value, the fp32 master and the optimizer moments of all members lie in
+  // parallel arrays at the same element offsets (members padded to 128
+  // elements), so that ONE update launch over the group's extent updates every
+  // member; the padding is updated too and never read.
   Planner arena;
   std::vector<Slot> grad_slot(T), value_slot(T), master_slot(T), v_slot(T), m_slot(T);
-  for (size_t t = 0; t < T; t++) {
-    if (has_grad[t] && cleared[t]) grad_slot[t] = arena.take((size_t)get_size_in_bytes(cg.tensors[t].shape));
-  }
-  st->cleared_bytes = arena.total;
   bool const adam = std::holds_alternative<AdamOptimizerAttrs>(optimizer_attrs);
   bool const sgd_momentum = !adam && std::get<SGDOptimizerAttrs>(optimizer_attrs).momentum > 0.0;
+  struct WeightGroup {
+    DataType type;
+    bool cleared;
+    std::vector<size_t> members;
+    std::vector<size_t> elem_offset;
+    size_t elems = 0;
+    Slot grad, value, master, v, m;
+  };
+  std::vector<WeightGroup> groups;
+  std::vector<int> group_of(T, -1);
   for (size_t t = 0; t < T; t++) {
+    if (!is_weight[t] || !has_grad[t]) continue;
+    TensorShape const &s = cg.tensors[t].shape;
+    if (s.data_type != DataType::FLOAT && s.data_type != DataType::BF16) bad("weights must be FLOAT or BF16");
+    if (input_tensors.count(tensor_guid_t{(int)t}) != 0) continue;  // lives in the caller's memory: updated on its own
+    size_t g = 0;
+    while (g < groups.size() && !(groups[g].type == s.data_type && groups[g].cleared == cleared[t])) g++;
+    if (g == groups.size()) groups.push_back(WeightGroup{s.data_type, cleared[t], {}, {}, 0, {}, {}, {}, {}, {}});
+    group_of[t] = (int)g;
+    groups[g].members.push_back(t);
+    groups[g].elem_offset.push_back(groups[g].elems);
+    groups[g].elems += ((size_t)get_num_elements(s.dims) + 127) & ~(size_t)127;
+  }
+  auto place_group_gradients = [&](bool cleared_ones) {
+    for (WeightGroup &g : groups) {
+      if (g.cleared != cleared_ones) continue;
+      size_t const es = (size_t)size_of_datatype(g.type);
+      g.grad = arena.take(g.elems * es);
+      for (size_t i = 0; i < g.members.size(); i++) {
+        size_t const t = g.members[i];
+        grad_slot[t] = Slot{g.grad.offset + g.elem_offset[i] * es, (size_t)get_size_in_bytes(cg.tensors[t].shape)};
+      }
+    }
+  };
+  place_group_gradients(true);
+  for (size_t t = 0; t < T; t++) {
+    if (has_grad[t] && cleared[t] && group_of[t] < 0) grad_slot[t] = arena.take((size_t)get_size_in_bytes(cg.tensors[t].shape));
+  }
+  st->cleared_bytes = arena.total;
+  place_group_gradients(false);
+  for (WeightGroup &g : groups) {
+    size_t const es = (size_t)size_of_datatype(g.type);
+    g.value = arena.take(g.elems * es);
+    if (g.type == DataType::BF16) g.master = arena.take(g.elems * 4);
+    if (adam || sgd_momentum) g.v = arena.take(g.elems * 4);
+    if (adam) g.m = arena.take(g.elems * 4);
+    for (size_t i = 0; i < g.members.size(); i++) {
+      size_t const t = g.members[i], n = (size_t)get_num_elements(cg.tensors[t].shape.dims), eo = g.elem_offset[i];
+      value_slot[t] = Slot{g.value.offset + eo * es, n * es};
+      if (g.master.bytes) master_slot[t] = Slot{g.master.offset + eo * 4, n * 4};
+      if (g.v.bytes) v_slot[t] = Slot{g.v.offset + eo * 4, n * 4};
+      if (g.m.bytes) m_slot[t] = Slot{g.m.offset + eo * 4, n * 4};
+    }
+  }
+  for (size_t t = 0; t < T; t++) {
+    if (group_of[t] >= 0) continue;
     TensorShape const &s = cg.tensors[t].shape;
     if (has_grad[t] && !cleared[t]) grad_slot[t] = arena.take((size_t)get_size_in_bytes(s));
     if (input_tensors.count(tensor_guid_t{(int)t}) == 0) value_slot[t] = arena.take((size_t)get_size_in_bytes(s));
     if (is_weight[t] && has_grad[t]) {
-      if (s.data_type != DataType::FLOAT && s.data_type != DataType::BF16) bad("weights must be FLOAT or BF16");
       size_t f32 = (size_t)get_num_elements(s.dims) * 4;
       if (s.data_type == DataType::BF16) master_slot[t] = arena.take(f32);
       if (adam || sgd_momentum) v_slot[t] = arena.take(f32);
@@ -440,7 +497,8 @@ ComputationGraphInstance create_computation_graph_instance(
       void *dk = k == q ? nullptr : grd_or_discard(k);
       void *dv = v == q ? nullptr : grd_or_discard(v);
       if ((dk == nullptr) != (dv == nullptr)) bad("attention: key and value must both alias the query, or neither");
-      int const accumulate = p.bwd.accumulate ? 1 : 0;
+      int const accumulate = (p.bwd.accumulate ? FFK_MHA_ACC_INPUT_GRADS : 0) |
+                             (writers[layer.weights[0].raw] > 1 ? 0 : FFK_MHA_OVERWRITE_WEIGHT_GRAD);
       f = [=](device_stream_t const &s) {
         check_ffk(ffk_mha_forward(s.require_gpu(), type, &d, qp, kp, vp, w, y, reserve, reserve_bytes), "MultiHeadAttention forward");
       };
@@ -666,19 +724,11 @@ ComputationGraphInstance create_computation_graph_instance(
   }
   for (auto it = bwd.rbegin(); it != bwd.rend(); ++it) order.push_back(*it);
 
-  // -- UPD, one per weight (optimizer.cc:10-108)
-  for (size_t t = 0; t < T; t++) {
-    if (!is_weight[t] || !has_grad[t]) continue;
-    TensorShape const &s = cg.tensors[t].shape;
-    int const grad_type = dt(s.data_type);
-    int64_t const n = get_num_elements(s.dims);
-    bool const lowp = s.data_type == DataType::BF16;
-    float *w32 = static_cast<float *>(lowp ? st->master[t]->ptr : st->value[t].ptr);
-    void *wlow = lowp ? st->value[t].ptr : nullptr;
-    void *g = st->grad[t]->ptr;
-    float *v = st->opt_v[t].has_value() ? static_cast<float *>(st->opt_v[t]->ptr) : nullptr;
-    float *m = st->opt_m[t].has_value() ? static_cast<float *>(st->opt_m[t]->ptr) : nullptr;
-    std::function<void(device_stream_t const &)> f = [=](device_stream_t const &stream) {
+  // -- UPD, one invocation per weight (optimizer.cc:10-108).  The first member of a
+  // weight group updates the whole group with one launch; the invocations of the
+  // other members are empty.
+  auto make_update = [S](int grad_type, void *g, int64_t n, float *w32, float *v, float *m, void *wlow) {
+    return [=](device_stream_t const &stream) {
       if (auto const *sgd = std::get_if<SGDOptimizerAttrs>(&S->optimizer_attrs)) {
         check_ffk(ffk_sgd_update(stream.require_gpu(), grad_type, (float)sgd->lr, (float)sgd->momentum, sgd->nesterov,
                                  (float)sgd->weight_decay, g, n, 1, w32, v, wlow),
@@ -691,6 +741,29 @@ ComputationGraphInstance create_computation_graph_instance(
                   "Adam update");
       }
     };
+  };
+  for (size_t t = 0; t < T; t++) {
+    if (!is_weight[t] || !has_grad[t]) continue;
+    std::function<void(device_stream_t const &)> f = [](device_stream_t const &) {};
+    if (group_of[t] >= 0) {
+      WeightGroup const &g = groups[(size_t)group_of[t]];
+      if (g.members.front() == t) {
+        bool const lowp = g.type == DataType::BF16;
+        f = make_update(dt(g.type), base + g.grad.offset, (int64_t)g.elems,
+                        reinterpret_cast<float *>(base + (lowp ? g.master.offset : g.value.offset)),
+                        g.v.bytes ? reinterpret_cast<float *>(base + g.v.offset) : nullptr,
+                        g.m.bytes ? reinterpret_cast<float *>(base + g.m.offset) : nullptr,
+                        lowp ? static_cast<void *>(base + g.value.offset) : nullptr);
+      }
+    } else {
+      TensorShape const &s = cg.tensors[t].shape;
+      bool const lowp = s.data_type == DataType::BF16;
+      f = make_update(dt(s.data_type), st->grad[t]->ptr, get_num_elements(s.dims),
+                      static_cast<float *>(lowp ? st->master[t]->ptr : st->value[t].ptr),
+                      st->opt_v[t].has_value() ? static_cast<float *>(st->opt_v[t]->ptr) : nullptr,
+                      st->opt_m[t].has_value() ? static_cast<float *>(st->opt_m[t]->ptr) : nullptr,
+                      lowp ? st->value[t].ptr : nullptr);
+    }
     order.push_back(DynamicNodeInvocation{DynamicTaskType::UPD, cg.tensors[t].source, f});
   }
   st->order = order;

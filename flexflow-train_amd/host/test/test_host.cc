@@ -697,6 +697,19 @@ static void gpu_tests() {
       CHECK(to_host(inst.get_tensor_accessor(w)) == to_host(mine.at(w.raw)));
       CHECK(to_host(*inst.get_master_weight_accessor(w)) == to_host(master));
     }
+    // all weights here are BF16 with stored gradients: one group, updated by one launch, so
+    // value, gradient and master of every member lie at the same element offset of their arrays
+    {
+      tensor_guid_t w0 = weights.front();
+      bool parallel = true;
+      for (tensor_guid_t w : weights) {
+        ptrdiff_t dv = (char *)inst.get_tensor_accessor(w).ptr - (char *)inst.get_tensor_accessor(w0).ptr;
+        ptrdiff_t dg = (char *)inst.get_gradient_accessor(w)->ptr - (char *)inst.get_gradient_accessor(w0)->ptr;
+        ptrdiff_t dm = (char *)inst.get_master_weight_accessor(w)->ptr - (char *)inst.get_master_weight_accessor(w0)->ptr;
+        parallel = parallel && dv == dg && dm == 2 * dv && dv % 256 == 0;
+      }
+      CHECK(parallel);
+    }
     // attrs advanced as lib/pcg/src/pcg/optimizer_attrs.cc:6-26 does
     AdamOptimizerAttrs next = std::get<AdamOptimizerAttrs>(inst.get_optimizer_attrs());
     CHECK(std::fabs(next.beta_t - 0.81) < 1e-12 && std::fabs(next.beta2_t - 0.999 * 0.999) < 1e-12);
