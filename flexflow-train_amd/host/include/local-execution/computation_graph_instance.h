@@ -19,6 +19,10 @@
 //    BF16 values at the first update, or when sync_master_weights is called).
 //  * a dropout layer's mask differs per layer and per iteration: seed + layer
 //    index, offset = iteration * elements.
+//  * the backward of an element-wise add copies nothing: an operand whose
+//    gradient has no other producer shares the output gradient's memory
+//    (get_gradient_accessor of both returns the same pointer), an operand that
+//    other operators also add into gets grad += dy.
 //  * the weights the instance places itself are grouped by data type: value,
 //    gradient, master and moments of a group lie in parallel arrays, and the
 //    UPD invocation of the group's first weight updates all of them with one

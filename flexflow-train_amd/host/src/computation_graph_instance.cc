@@ -116,6 +116,7 @@ struct BackwardPlan {
   bool accumulate = false;                 // one switch for all input gradients of the op
   std::vector<bool> accumulate_input;      // Linear only: input, weight, bias
   bool softmax_via_scratch = false;
+  bool add_by_alias = false;               // ElementBinary add: see alias_of below
 };
 
 struct Slot {
@@ -213,6 +214,12 @@ ComputationGraphInstance create_computation_graph_instance(
   // -- per-layer backward mode, saved state and scratch
   std::vector<LayerPlan> plan(L);
   std::vector<bool> cleared(T, false);  // gradient must be zero before the backward pass
+  // The backward of y = a + b hands dy to both operands.  An operand whose gradient has no
+  // other producer does not get a copy: its gradient IS y's gradient memory (complete by the
+  // time the add's backward runs, since every consumer of y ran before it, and not written
+  // afterwards).  alias_of[a] = y records that; an operand several producers add into gets
+  // grad += dy, an operand without a gradient nothing.
+  std::vector<int> alias_of(T, -1);
   Planner saved_planner;
   size_t scratch_bytes = 0, discard_bytes = 0;
   for (size_t l = 0; l < L; l++) {
@@ -292,11 +299,31 @@ ComputationGraphInstance create_computation_graph_instance(
       }
     } else if (std::get_if<CastAttrs>(&oa)) {
       acc = true;  // cast_backward always adds
-    } else if (std::get_if<ElementBinaryAttrs>(&oa)) {
+    } else if (auto const *a = std::get_if<ElementBinaryAttrs>(&oa)) {
       if (p.bwd.has_backward && numel(layer.inputs[0]) != numel(layer.inputs[1])) {
         bad("element binary backward needs operands of equal size");
       }
       if (layer.inputs[0] == layer.inputs[1]) acc = true;
+      tensor_guid_t const out = layer.outputs[0];
+      if (a->type == OperatorType::EW_ADD && p.bwd.has_backward && layer.inputs[0] != layer.inputs[1]) {
+        int aliased = 0;
+        bool all_handled = true;
+        for (tensor_guid_t t : layer.inputs) {
+          bool const same = shape_of(t) == shape_of(out);
+          if (!has_grad[t.raw]) continue;
+          if (same && !must_accumulate(t) && !is_weight[t.raw]) aliased++;
+          else if (!(same && must_accumulate(t))) all_handled = false;
+        }
+        if (all_handled && aliased > 0) {
+          p.bwd.add_by_alias = true;
+          acc = false;
+          for (tensor_guid_t t : layer.inputs) {
+            if (!has_grad[t.raw]) continue;
+            if (must_accumulate(t)) cleared[t.raw] = true;
+            else alias_of[t.raw] = out.raw;
+          }
+        }
+      }
     }
     p.bwd.accumulate = acc;
     if (acc) {
@@ -382,7 +409,7 @@ ComputationGraphInstance create_computation_graph_instance(
   for (size_t t = 0; t < T; t++) {
     if (group_of[t] >= 0) continue;
     TensorShape const &s = cg.tensors[t].shape;
-    if (has_grad[t] && !cleared[t]) grad_slot[t] = arena.take((size_t)get_size_in_bytes(s));
+    if (has_grad[t] && !cleared[t] && alias_of[t] < 0) grad_slot[t] = arena.take((size_t)get_size_in_bytes(s));
     if (input_tensors.count(tensor_guid_t{(int)t}) == 0) value_slot[t] = arena.take((size_t)get_size_in_bytes(s));
     if (is_weight[t] && has_grad[t]) {
       size_t f32 = (size_t)get_num_elements(s.dims) * 4;
@@ -390,6 +417,12 @@ ComputationGraphInstance create_computation_graph_instance(
       if (adam || sgd_momentum) v_slot[t] = arena.take(f32);
       if (adam) m_slot[t] = arena.take(f32);
     }
+  }
+  for (size_t t = 0; t < T; t++) {
+    if (alias_of[t] < 0) continue;
+    int root = alias_of[t];
+    while (alias_of[(size_t)root] >= 0) root = alias_of[(size_t)root];
+    grad_slot[t] = grad_slot[(size_t)root];
   }
   size_t const saved_base = arena.take(saved_planner.total).offset;
   size_t const scratch_base = arena.take(scratch_bytes).offset;
@@ -543,9 +576,22 @@ ComputationGraphInstance create_computation_graph_instance(
       f = [=](device_stream_t const &s) {
         check_ffk(ffk_element_binary_forward(s.require_gpu(), type, op, lp, rp, y, n, nl, nr), "ElementBinary forward");
       };
-      b = [=](device_stream_t const &s) {
-        check_ffk(ffk_element_binary_backward(s.require_gpu(), type, op, dy, lp, rp, dl, dr, n, accumulate), "ElementBinary backward");
-      };
+      if (p.bwd.add_by_alias) {
+        // operands whose gradient is dy's own memory need nothing; the others get grad += dy
+        void *add_l = has_grad[lhs.raw] && alias_of[lhs.raw] < 0 ? grd(lhs) : nullptr;
+        void *add_r = has_grad[rhs.raw] && alias_of[rhs.raw] < 0 ? grd(rhs) : nullptr;
+        b = [=](device_stream_t const &s) {
+          for (void *g : {add_l, add_r}) {
+            if (g != nullptr) {
+              check_ffk(ffk_element_binary_forward(s.require_gpu(), type, FFK_OP_EW_ADD, g, dy, g, n, n, n), "ElementBinary backward");
+            }
+          }
+        };
+      } else {
+        b = [=](device_stream_t const &s) {
+          check_ffk(ffk_element_binary_backward(s.require_gpu(), type, op, dy, lp, rp, dl, dr, n, accumulate), "ElementBinary backward");
+        };
+      }
     } else if (auto const *a = std::get_if<SoftmaxAttrs>(&oa)) {
       tensor_guid_t x = layer.inputs[0];
       int const type = dt(shape_of(x).data_type);

@@ -697,6 +697,11 @@ static void gpu_tests() {
       CHECK(to_host(inst.get_tensor_accessor(w)) == to_host(mine.at(w.raw)));
       CHECK(to_host(*inst.get_master_weight_accessor(w)) == to_host(master));
     }
+    // res1 = attn + input: attn's gradient has no other producer, so it is res1's gradient
+    // memory itself; res2 = norm1 + drop2: drop2's likewise, norm1's (also fed by ff1) is added into
+    CHECK(inst.get_gradient_accessor(attn)->ptr == inst.get_gradient_accessor(res1)->ptr);
+    CHECK(inst.get_gradient_accessor(drop2)->ptr == inst.get_gradient_accessor(res2)->ptr);
+    CHECK(inst.get_gradient_accessor(norm1)->ptr != inst.get_gradient_accessor(res2)->ptr);
     // all weights here are BF16 with stored gradients: one group, updated by one launch, so
     // value, gradient and master of every member lie at the same element offset of their arrays
     {
