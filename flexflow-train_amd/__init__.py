@@ -118,6 +118,9 @@ SIGNATURES = {
     "ffk_dropout_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
     "ffk_dropout_backward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64, c_int]),
     "ffk_dropout_mask": (c_int, [c_p, c_p, c_i64, c_f, c_u64, c_u64]),
+    "ffk_dropout_add_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
+    "ffk_gelu_dropout_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
+    "ffk_dropout_gelu_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
     "ffk_sgd_update": (c_int, [c_p, c_int, c_f, c_f, c_int, c_f, c_p, c_i64, c_int, c_p, c_p, c_p]),
     "ffk_adam_update": (c_int, [c_p, c_int, c_f, c_f, c_f, c_f, c_f, c_p, c_i64, c_int, c_p, c_p,
                                 c_p, c_p]),
@@ -352,6 +355,29 @@ def dropout_backward(dy, rate, seed, offset=0, dx=None, accumulate=False):
         dx = torch.empty_like(dy)
     check(lib().ffk_dropout_backward(current_stream(), dtype_of(dy), ptr(dy), ptr(dx),
                                      dy.numel(), rate, seed, offset, int(accumulate)))
+    return dx
+
+
+def dropout_add_forward(x, residual, rate, seed, offset=0):
+    """residual + dropout(x), one pass."""
+    out = _torch().empty_like(x)
+    check(lib().ffk_dropout_add_forward(current_stream(), dtype_of(x), ptr(x), ptr(residual), ptr(out), x.numel(),
+                                        rate, seed, offset))
+    return out
+
+
+def gelu_dropout_forward(x, rate, seed, offset=0):
+    """dropout(GELU(x)), one pass."""
+    out = _torch().empty_like(x)
+    check(lib().ffk_gelu_dropout_forward(current_stream(), dtype_of(x), ptr(x), ptr(out), x.numel(), rate, seed, offset))
+    return out
+
+
+def dropout_gelu_backward(dy, gelu_input, rate, seed, offset=0):
+    """dropout_backward(dy) * GELU'(gelu_input), one pass."""
+    dx = _torch().empty_like(dy)
+    check(lib().ffk_dropout_gelu_backward(current_stream(), dtype_of(dy), ptr(dy), ptr(gelu_input), ptr(dx),
+                                          dy.numel(), rate, seed, offset))
     return dx
 
 

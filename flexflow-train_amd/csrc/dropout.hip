@@ -275,6 +275,29 @@ extern "C" int ffk_dropout_backward(ffk_stream_t stream, int dtype,
   return fail(FFK_ERR_UNSUPPORTED, "dropout_backward: dtype %d not supported", dtype);
 }
 
+extern "C" int ffk_dropout_add_forward(ffk_stream_t stream, int dtype, void const *input,
+                                       void const *residual, void *output, int64_t num_elements,
+                                       float rate, uint64_t seed, uint64_t offset) {
+  FFK_REQUIRE(input && residual && output, "dropout_add_forward: NULL operand");
+  return ffk::dropout_add_residual(as_stream(stream), dtype, input, residual, output, num_elements, rate, seed, offset);
+}
+
+extern "C" int ffk_gelu_dropout_forward(ffk_stream_t stream, int dtype, void const *input,
+                                        void *output, int64_t num_elements, float rate,
+                                        uint64_t seed, uint64_t offset) {
+  FFK_REQUIRE(input && output, "gelu_dropout_forward: NULL operand");
+  return ffk::gelu_dropout_forward(as_stream(stream), dtype, input, output, num_elements, rate, seed, offset);
+}
+
+extern "C" int ffk_dropout_gelu_backward(ffk_stream_t stream, int dtype, void const *output_grad,
+                                         void const *gelu_input, void *input_grad,
+                                         int64_t num_elements, float rate, uint64_t seed,
+                                         uint64_t offset) {
+  FFK_REQUIRE(output_grad && gelu_input && input_grad, "dropout_gelu_backward: NULL operand");
+  return ffk::dropout_backward_gelu_backward(as_stream(stream), dtype, output_grad, gelu_input, input_grad,
+                                             num_elements, rate, seed, offset);
+}
+
 extern "C" int ffk_dropout_mask(ffk_stream_t stream, uint8_t *mask,
                                 int64_t num_elements, float rate, uint64_t seed,
                                 uint64_t offset) {

@@ -19,6 +19,12 @@
 //    BF16 values at the first update, or when sync_master_weights is called).
 //  * a dropout layer's mask differs per layer and per iteration: seed + layer
 //    index, offset = iteration * elements.
+//  * two neighbouring operators run as one kernel where the library has one
+//    that produces the same bits: GELU -> Dropout (forward and backward) and
+//    Dropout -> element-wise add (forward).  The tensor between them must have
+//    no other consumer; it is then never written (get_tensor_accessor on it
+//    returns memory nobody filled).  FFK_LAYER_UNFUSED=1 in the environment at
+//    creation keeps one kernel per operator.
 //  * the backward of an element-wise add copies nothing: an operand whose
 //    gradient has no other producer shares the output gradient's memory
 //    (get_gradient_accessor of both returns the same pointer), an operand that

@@ -11,6 +11,7 @@
 // pointers that makes one C-ABI call.
 #include "ffk.h"
 #include "local-execution/computation_graph_instance.h"
+#include <cstdlib>
 #include <cmath>
 #include <cstring>
 
@@ -341,6 +342,65 @@ ComputationGraphInstance create_computation_graph_instance(
   }
   if (st->logit.has_value()) cleared[st->logit->raw] = false;  // written by the loss before any producer adds
 
+  // -- neighbouring operators run as one kernel where the library has one that produces the
+  // same bits (FFK_LAYER_UNFUSED=1 switches this off).  The intermediate tensor of a fused pair
+  // has that pair's second operator as its only consumer and is never written.
+  //   GELU -> Dropout:            forward one kernel at the Dropout, backward one at the GELU
+  //   Dropout -> element-wise add: forward one kernel at the add (the backward of the add copies
+  //                                nothing, see alias_of, and the Dropout's is its own)
+  enum class Fused { NONE, GELU_DROPOUT_HEAD, GELU_DROPOUT_TAIL, DROPOUT_ADD_HEAD, DROPOUT_ADD_TAIL };
+  std::vector<Fused> fused(L, Fused::NONE);
+  std::vector<size_t> partner(L, 0);
+  {
+    char const *off = std::getenv("FFK_LAYER_UNFUSED");
+    bool const enabled = !(off != nullptr && off[0] == '1');
+    std::vector<int> uses(T, 0);
+    std::vector<size_t> consumer(T, 0);
+    for (size_t l = 0; l < L; l++) {
+      if (!is_op_layer(cg.layers[l])) continue;
+      for (tensor_guid_t t : cg.layers[l].inputs) uses[t.raw]++, consumer[t.raw] = l;
+    }
+    auto vectorizable = [&](tensor_guid_t t) {
+      DataType const d = shape_of(t).data_type;
+      return (d == DataType::FLOAT || d == DataType::BF16) && numel(t) % 8 == 0;
+    };
+    // what the instance places is 256-byte aligned; caller memory has to be looked at
+    auto aligned = [&](tensor_guid_t t) {
+      auto bound = input_tensors.find(t);
+      return bound == input_tensors.end() || reinterpret_cast<uintptr_t>(bound->second.ptr) % 16 == 0;
+    };
+    auto only_consumer = [&](tensor_guid_t t, size_t &c) {
+      if (uses[t.raw] != 1 || (st->logit.has_value() && *st->logit == t)) return false;
+      c = consumer[t.raw];
+      return fused[c] == Fused::NONE;
+    };
+    for (size_t l = 0; enabled && l < L; l++) {
+      ComputationGraph::Layer const &layer = cg.layers[l];
+      if (!is_op_layer(layer) || fused[l] != Fused::NONE) continue;
+      tensor_guid_t const out = layer.outputs.at(0);
+      size_t c = 0;
+      if (auto const *u = std::get_if<ElementUnaryAttrs>(&layer.attrs.op_attrs)) {
+        if (u->op_type != OperatorType::GELU || !vectorizable(out) || !only_consumer(out, c)) continue;
+        if (!std::holds_alternative<DropoutAttrs>(cg.layers[c].attrs.op_attrs)) continue;
+        bool const any_bwd = plan[l].bwd.has_backward || plan[c].bwd.has_backward;
+        bool const both_bwd = plan[l].bwd.has_backward && plan[c].bwd.has_backward && !plan[l].bwd.accumulate &&
+                              has_grad[layer.inputs[0].raw];
+        if (any_bwd && !both_bwd) continue;
+        if (!aligned(layer.inputs[0]) || !aligned(cg.layers[c].outputs.at(0))) continue;
+        fused[l] = Fused::GELU_DROPOUT_HEAD, fused[c] = Fused::GELU_DROPOUT_TAIL, partner[l] = c, partner[c] = l;
+      } else if (std::holds_alternative<DropoutAttrs>(layer.attrs.op_attrs)) {
+        if (!vectorizable(out) || !only_consumer(out, c)) continue;
+        auto const *b = std::get_if<ElementBinaryAttrs>(&cg.layers[c].attrs.op_attrs);
+        if (b == nullptr || b->type != OperatorType::EW_ADD) continue;
+        ComputationGraph::Layer const &add = cg.layers[c];
+        tensor_guid_t const other = add.inputs[0] == out ? add.inputs[1] : add.inputs[0];
+        if (other == out || !(shape_of(other) == shape_of(out))) continue;
+        if (!aligned(layer.inputs[0]) || !aligned(other) || !aligned(add.outputs.at(0))) continue;
+        fused[l] = Fused::DROPOUT_ADD_HEAD, fused[c] = Fused::DROPOUT_ADD_TAIL, partner[l] = c, partner[c] = l;
+      }
+    }
+  }
+
   // -- placement: cleared gradients first, then everything else.
   // Trainable weights that the instance places itself are laid out in groups
   // (same data type, gradient cleared or not): within a group the gradient, the
@@ -554,6 +614,17 @@ ComputationGraphInstance create_computation_graph_instance(
         check_ffk(ffk_dropout_backward(s.require_gpu(), type, dy, dx, n, rate, seed, S->iteration * (uint64_t)n, accumulate),
                   "Dropout backward");
       };
+      if (fused[l] == Fused::GELU_DROPOUT_TAIL) {
+        // y = dropout(GELU(u)) from the GELU's input; the backward of both runs at the GELU
+        void *u = val(cg.layers[partner[l]].inputs[0]);
+        f = [=](device_stream_t const &s) {
+          check_ffk(ffk_gelu_dropout_forward(s.require_gpu(), type, u, y, n, rate, seed, S->iteration * (uint64_t)n),
+                    "GELU + Dropout forward");
+        };
+        b = [](device_stream_t const &) {};
+      } else if (fused[l] == Fused::DROPOUT_ADD_HEAD) {
+        f = [](device_stream_t const &) {};  // the add computes residual + dropout(x)
+      }
     } else if (auto const *a = std::get_if<ElementUnaryAttrs>(&oa)) {
       tensor_guid_t x = layer.inputs[0];
       int const type = dt(shape_of(x).data_type), op = static_cast<int>(a->op_type);
@@ -567,6 +638,20 @@ ComputationGraphInstance create_computation_graph_instance(
       b = [=](device_stream_t const &s) {
         check_ffk(ffk_element_unary_backward(s.require_gpu(), type, op, scalar, y, dy, xp, dx, n, accumulate), "ElementUnary backward");
       };
+      if (fused[l] == Fused::GELU_DROPOUT_HEAD) {
+        size_t const d = partner[l];
+        DropoutAttrs const &da = std::get<DropoutAttrs>(cg.layers[d].attrs.op_attrs);
+        float const rate = da.rate;
+        uint64_t const seed = da.seed + (uint64_t)d;
+        void *d_out = grd(cg.layers[d].outputs.at(0));
+        f = [](device_stream_t const &) {};  // the Dropout computes dropout(GELU(x))
+        if (p.bwd.has_backward) {
+          b = [=](device_stream_t const &s) {
+            check_ffk(ffk_dropout_gelu_backward(s.require_gpu(), type, d_out, xp, dx, n, rate, seed, S->iteration * (uint64_t)n),
+                      "Dropout + GELU backward");
+          };
+        }
+      }
     } else if (auto const *a = std::get_if<ElementBinaryAttrs>(&oa)) {
       tensor_guid_t lhs = layer.inputs[0], rhs = layer.inputs[1];
       int const type = dt(shape_of(out).data_type), op = static_cast<int>(a->type);
@@ -576,6 +661,19 @@ ComputationGraphInstance create_computation_graph_instance(
       f = [=](device_stream_t const &s) {
         check_ffk(ffk_element_binary_forward(s.require_gpu(), type, op, lp, rp, y, n, nl, nr), "ElementBinary forward");
       };
+      if (fused[l] == Fused::DROPOUT_ADD_TAIL) {
+        size_t const d = partner[l];
+        ComputationGraph::Layer const &drop = cg.layers[d];
+        DropoutAttrs const &da = std::get<DropoutAttrs>(drop.attrs.op_attrs);
+        float const rate = da.rate;
+        uint64_t const seed = da.seed + (uint64_t)d;
+        void *dropped_in = val(drop.inputs[0]);
+        void *residual = lhs == drop.outputs.at(0) ? rp : lp;
+        f = [=](device_stream_t const &s) {
+          check_ffk(ffk_dropout_add_forward(s.require_gpu(), type, dropped_in, residual, y, n, rate, seed, S->iteration * (uint64_t)n),
+                    "Dropout + add forward");
+        };
+      }
       if (p.bwd.add_by_alias) {
         // operands whose gradient is dy's own memory need nothing; the others get grad += dy
         void *add_l = has_grad[lhs.raw] && alias_of[lhs.raw] < 0 ? grd(lhs) : nullptr;

@@ -968,6 +968,63 @@ static void gpu_tests() {
     orc_transpose_nd(dr.data(), dxw.data(), 3, tdims.data(), perm, 0);  // (1, 0, 2) is its own inverse
     CHECK(close(to_host(*inst.get_gradient_accessor(x)), dxw, 1e-6) && contains_non_zero(dxw));
   });
+  run("Step driver: fused operator pairs give the bits of one kernel per operator", [&] {
+    // x -> dense -> GELU -> dropout -> dense -> dropout -> (+ x) -> cast -> loss; two instances of the
+    // same graph, one created with FFK_LAYER_UNFUSED=1, stepped twice each (the second step uses
+    // the next dropout offsets)
+    int64_t const B = 16, E = 64, FF = 128;
+    auto build = [&](ComputationGraphBuilder &cgb, tensor_guid_t &x, tensor_guid_t &logits, std::vector<tensor_guid_t> &ws) {
+      x = cgb.create_input(shape({B, E}, DataType::BF16), CreateGrad::YES);
+      tensor_guid_t h = cgb.dense(x, (int)FF, Activation::GELU, true);
+      ws = {};  // collected below: every weight tensor of the graph
+      tensor_guid_t d1 = cgb.dropout(h, 0.25f);
+      tensor_guid_t f2 = cgb.dense(d1, (int)E, std::nullopt, true);
+      tensor_guid_t r = cgb.add(cgb.dropout(f2, 0.25f), x);
+      logits = cgb.cast(r, DataType::FLOAT);
+    };
+    device_id_t dev = make_device_id_t_from_idx(0, DeviceType::GPU);
+    auto LABEL = device_accessor(gpu, shape({B, E}, DataType::FLOAT), random_vec(B * E, 71));
+    std::vector<std::vector<float>> results[2];
+    auto ok = [](int rc) {
+      if (rc != FFK_OK) throw std::runtime_error(ffk_last_error());
+    };
+    for (int unfused = 0; unfused < 2; unfused++) {
+      ComputationGraphBuilder cgb;
+      tensor_guid_t x, logits;
+      std::vector<tensor_guid_t> ws;
+      build(cgb, x, logits, ws);
+      if (unfused) setenv("FFK_LAYER_UNFUSED", "1", 1);
+      ComputationGraphInstance inst = create_computation_graph_instance(
+          cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{0.05, 0.9, false, 0.0}},
+          LossConfig{NonconfigurableLossAttrs{LossFunction::MEAN_SQUARED_ERROR_AVG_REDUCE}, LABEL, logits}, {}, gpu,
+          ProfilingSettings{0, 0}, handle, dev);
+      if (unfused) unsetenv("FFK_LAYER_UNFUSED");
+      // the GELU of dense(.., GELU) is its own layer: find the weights by layer order (same in both graphs)
+      int seed = 80;
+      for (size_t t = 0; t < cgb.computation_graph.tensors.size(); t++) {
+        tensor_guid_t g{(int)t};
+        auto const &src = cgb.computation_graph.layers.at(cgb.computation_graph.tensors[t].source.raw);
+        bool const weight = std::holds_alternative<WeightAttrs>(src.attrs.op_attrs);
+        if (!weight && !(g == x)) continue;
+        if (weight) ws.push_back(g);
+        TensorShape s16 = cgb.computation_graph.tensors[t].shape;
+        auto host = random_vec(get_num_elements(s16.dims), seed++);
+        for (auto &v : host) v *= 0.3f;
+        auto f32 = device_accessor(gpu, TensorShape{s16.dims, DataType::FLOAT}, host);
+        ok(ffk_cast_forward(nullptr, FFK_FLOAT, FFK_BF16, f32.ptr, inst.get_tensor_accessor(g).ptr, get_num_elements(s16.dims)));
+      }
+      ok(ffk_stream_synchronize(nullptr));
+      for (int step = 0; step < 2; step++) perform_all_passes_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, dev);
+      results[unfused].push_back(to_host(inst.get_tensor_accessor(logits)));
+      results[unfused].push_back(to_host(*inst.get_gradient_accessor(x)));
+      for (tensor_guid_t w : ws) results[unfused].push_back(to_host(inst.get_tensor_accessor(w)));
+    }
+    CHECK(results[0].size() == results[1].size() && results[0].size() == 6);
+    for (size_t i = 0; i < results[0].size(); i++) {
+      CHECK(contains_non_zero(results[0][i]));
+      CHECK(results[0][i] == results[1][i]);
+    }
+  });
 }
 
 // One training step of the BASELINE encoder layer (pre-LN, GELU, dropout 0.1,

@@ -270,6 +270,32 @@ int ffk_dropout_backward(ffk_stream_t stream, int dtype,
 /* The keep mask itself (1 byte per element), for bit-exact checks. */
 int ffk_dropout_mask(ffk_stream_t stream, uint8_t *mask, int64_t num_elements,
                      float rate, uint64_t seed, uint64_t offset);
+/* Dropout fused with a neighbouring operator.  No counterpart in the
+ * reference, whose executor launches one kernel per operator
+ * (lib/local-execution/src/local-execution/computation_graph_instance.cc);
+ * for executors that find the pair in their graph (the step driver of this
+ * library's host mirror does).  Each entry produces exactly the bits of the
+ * two separate entries run one after the other (the intermediate is rounded
+ * to the storage type where the first operator would have stored it) without
+ * the intermediate's trip through memory.  FLOAT or BF16; pointers 16-byte
+ * aligned, num_elements a multiple of 8 (BF16) or 4 (FLOAT), offset a
+ * multiple of 8 -- anything else is FFK_ERR_INVALID_ARGUMENT and the caller
+ * runs the separate operators.
+ *   ffk_dropout_add_forward:  output = residual + dropout(input)
+ *   ffk_gelu_dropout_forward: output = dropout(GELU(input))
+ *   ffk_dropout_gelu_backward: input_grad = dropout_backward(output_grad)
+ *                                           * GELU'(gelu_input)             */
+int ffk_dropout_add_forward(ffk_stream_t stream, int dtype, void const *input,
+                            void const *residual, void *output,
+                            int64_t num_elements, float rate, uint64_t seed,
+                            uint64_t offset);
+int ffk_gelu_dropout_forward(ffk_stream_t stream, int dtype, void const *input,
+                             void *output, int64_t num_elements, float rate,
+                             uint64_t seed, uint64_t offset);
+int ffk_dropout_gelu_backward(ffk_stream_t stream, int dtype,
+                              void const *output_grad, void const *gelu_input,
+                              void *input_grad, int64_t num_elements,
+                              float rate, uint64_t seed, uint64_t offset);
 
 /* ------------------------------------------------------------------------ */
 /* Embedding -- Kernels::Embedding::gpu_forward_kernel / gpu_backward_kernel

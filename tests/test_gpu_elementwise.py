@@ -146,6 +146,32 @@ def test_dropout_forward_backward(ffk, oracle, dtype, n, offset):
     assert np.array_equal(to_np(dxa), wa)
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_dropout_fused_with_neighbour_equals_separate_operators(ffk, dtype):
+    """The three fused dropout entries against the separate entries run one after the other
+    (bit for bit), and their refusal of operands the vector kernels cannot take."""
+    say("dropout fused pairs", dtype)
+    n, rate, seed, offset = 4096 * 24, 0.1, 777, 16
+    tdt = torch.float32 if dtype == "fp32" else torch.bfloat16
+    g = rng(61)
+    x = to_dev(g.standard_normal((n,)).astype(np.float32), torch, tdt)
+    r = to_dev(g.standard_normal((n,)).astype(np.float32), torch, tdt)
+    dy = to_dev(g.standard_normal((n,)).astype(np.float32), torch, tdt)
+    gelu = ffk.OP["GELU"]
+    want = ffk.element_binary_forward(ffk.OP["EW_ADD"], ffk.dropout_forward(x, rate, seed, offset), r)
+    assert torch.equal(ffk.dropout_add_forward(x, r, rate, seed, offset), want)
+    want = ffk.dropout_forward(ffk.element_unary_forward(gelu, x), rate, seed, offset)
+    assert torch.equal(ffk.gelu_dropout_forward(x, rate, seed, offset), want)
+    act = ffk.element_unary_forward(gelu, x)
+    want = ffk.element_unary_backward(gelu, act, ffk.dropout_backward(dy, rate, seed, offset), x, torch.empty_like(x),
+                                      accumulate=0)
+    assert torch.equal(ffk.dropout_gelu_backward(dy, x, rate, seed, offset), want)
+    with pytest.raises(ffk.FFKError, match="fusable"):
+        ffk.gelu_dropout_forward(x[: n - 1], rate, seed, offset)
+    with pytest.raises(ffk.FFKError, match="fusable"):
+        ffk.dropout_add_forward(x, r, rate, seed, offset + 3)
+
+
 def test_dropout_full_size_statistics(ffk):
     """BASELINE config 3 size [16384, 4096] bf16, p = 0.1: keep rate within
     5 sigma, kept values scaled by 1/(1-p), backward mask == forward mask."""
