@@ -11,8 +11,9 @@
 // stepping.  Differences from the reference that a caller can see:
 //  * gradients are cleared by the instance: it knows, per gradient tensor,
 //    whether its only producer can overwrite it (then it is never cleared) or
-//    whether several producers add into it (then it sits in a region that one
-//    fill clears before the backward pass).  The reference leaves gradient
+//    whether several producers add into it; then the producer that runs first
+//    in the backward pass stores where it can, and otherwise the gradient sits
+//    in a region that one fill clears before the backward pass.  The reference leaves gradient
 //    memory as allocated and lets every GPU backward add into it.
 //  * weights of BF16 data type are trained with an fp32 master copy that the
 //    update kernel rounds into the BF16 tensor (the master is taken from the

@@ -212,6 +212,37 @@ ComputationGraphInstance create_computation_graph_instance(
     return writers[t.raw] > 1 || (st->logit.has_value() && *st->logit == t);
   };
 
+  // A gradient several operators add into needs no clearing if the one that runs first in the
+  // backward pass (the consumer with the highest layer index) stores instead of adding.  That is
+  // done where an operator has a switch for this gradient alone: operators with one
+  // differentiable input, Linear, and the add whose backward is a copy.
+  std::vector<int> first_writer(T, -1);
+  std::vector<bool> first_writer_stores(T, false);
+  for (size_t l = 0; l < L; l++) {
+    ComputationGraph::Layer const &layer = cg.layers[l];
+    if (!is_op_layer(layer) || !has_grad[layer.outputs.at(0).raw]) continue;
+    for (tensor_guid_t t : layer.inputs) {
+      if (has_grad[t.raw]) first_writer[t.raw] = (int)l;
+    }
+  }
+  for (size_t t = 0; t < T; t++) {
+    if (first_writer[t] < 0 || writers[t] < 2 || is_weight[t] || (st->logit.has_value() && st->logit->raw == (int)t)) continue;
+    ComputationGraph::Layer const &layer = cg.layers[(size_t)first_writer[t]];
+    ComputationGraphOpAttrs const &oa = layer.attrs.op_attrs;
+    int times = 0;
+    for (tensor_guid_t in : layer.inputs) times += in.raw == (int)t;
+    bool const one_input = std::holds_alternative<LayerNormAttrs>(oa) || std::holds_alternative<DropoutAttrs>(oa) ||
+                           std::holds_alternative<ElementUnaryAttrs>(oa) || std::holds_alternative<TransposeAttrs>(oa) ||
+                           std::holds_alternative<ReshapeAttrs>(oa);
+    bool const linear_input = std::holds_alternative<LinearAttrs>(oa);
+    auto const *bin = std::get_if<ElementBinaryAttrs>(&oa);
+    bool const add = bin != nullptr && bin->type == OperatorType::EW_ADD;  // confirmed below, where the add is planned
+    first_writer_stores[t] = times == 1 && (one_input || linear_input || add);
+  }
+  auto adds_here = [&](tensor_guid_t t, size_t l) {
+    return must_accumulate(t) && !(first_writer_stores[t.raw] && first_writer[t.raw] == (int)l);
+  };
+
   // -- per-layer backward mode, saved state and scratch
   std::vector<LayerPlan> plan(L);
   std::vector<bool> cleared(T, false);  // gradient must be zero before the backward pass
@@ -233,7 +264,7 @@ ComputationGraphInstance create_computation_graph_instance(
     for (tensor_guid_t t : layer.weights) any_grad = any_grad || has_grad[t.raw];
     p.bwd.has_backward = any_grad && has_grad[layer.outputs.at(0).raw];
     bool acc = false;
-    for (tensor_guid_t t : layer.inputs) acc = acc || (has_grad[t.raw] && must_accumulate(t));
+    for (tensor_guid_t t : layer.inputs) acc = acc || (has_grad[t.raw] && adds_here(t, l));
     if (auto const *a = std::get_if<LinearAttrs>(&oa)) {
       int64_t batch = numel(layer.inputs[0]) / dim_at_idx(shape_of(layer.inputs[0]).dims, -1);
       p.scratch_bytes = ffk_linear_backward_workspace_bytes(dt(shape_of(layer.outputs[0]).data_type), activation_code(a->activation),
@@ -307,23 +338,38 @@ ComputationGraphInstance create_computation_graph_instance(
       if (layer.inputs[0] == layer.inputs[1]) acc = true;
       tensor_guid_t const out = layer.outputs[0];
       if (a->type == OperatorType::EW_ADD && p.bwd.has_backward && layer.inputs[0] != layer.inputs[1]) {
-        int aliased = 0;
+        int cheaper = 0;  // operands that get no kernel (alias) or a copy that saves a clearing fill
         bool all_handled = true;
         for (tensor_guid_t t : layer.inputs) {
           bool const same = shape_of(t) == shape_of(out);
           if (!has_grad[t.raw]) continue;
-          if (same && !must_accumulate(t) && !is_weight[t.raw]) aliased++;
-          else if (!(same && must_accumulate(t))) all_handled = false;
+          if (same && !must_accumulate(t) && !is_weight[t.raw]) cheaper++;
+          else if (same && must_accumulate(t)) cheaper += !adds_here(t, l);
+          else all_handled = false;
         }
-        if (all_handled && aliased > 0) {
+        if (all_handled && cheaper > 0) {
           p.bwd.add_by_alias = true;
           acc = false;
           for (tensor_guid_t t : layer.inputs) {
             if (!has_grad[t.raw]) continue;
-            if (must_accumulate(t)) cleared[t.raw] = true;
-            else alias_of[t.raw] = out.raw;
+            if (!must_accumulate(t)) alias_of[t.raw] = out.raw;
+            else if (adds_here(t, l)) cleared[t.raw] = true;
           }
+        } else {
+          for (tensor_guid_t t : layer.inputs) {
+            if (first_writer[t.raw] == (int)l) first_writer_stores[t.raw] = false;  // the plain kernel adds
+          }
+          acc = false;
+          for (tensor_guid_t t : layer.inputs) acc = acc || (has_grad[t.raw] && adds_here(t, l));
+          if (layer.inputs[0] == layer.inputs[1]) acc = true;
         }
+      } else {
+        for (tensor_guid_t t : layer.inputs) {
+          if (first_writer[t.raw] == (int)l) first_writer_stores[t.raw] = false;  // not an add after all
+        }
+        acc = false;
+        for (tensor_guid_t t : layer.inputs) acc = acc || (has_grad[t.raw] && adds_here(t, l));
+        if (layer.inputs[0] == layer.inputs[1]) acc = true;
       }
     }
     p.bwd.accumulate = acc;
@@ -341,6 +387,9 @@ ComputationGraphInstance create_computation_graph_instance(
     }
   }
   if (st->logit.has_value()) cleared[st->logit->raw] = false;  // written by the loss before any producer adds
+  for (size_t t = 0; t < T; t++) {
+    if (first_writer_stores[t]) cleared[t] = false;  // its first producer stores
+  }
 
   // -- neighbouring operators run as one kernel where the library has one that produces the
   // same bits (FFK_LAYER_UNFUSED=1 switches this off).  The intermediate tensor of a fused pair
@@ -676,11 +725,17 @@ ComputationGraphInstance create_computation_graph_instance(
       }
       if (p.bwd.add_by_alias) {
         // operands whose gradient is dy's own memory need nothing; the others get grad += dy
+        // ... or, where this add is the first of them to run, grad = dy
         void *add_l = has_grad[lhs.raw] && alias_of[lhs.raw] < 0 ? grd(lhs) : nullptr;
         void *add_r = has_grad[rhs.raw] && alias_of[rhs.raw] < 0 ? grd(rhs) : nullptr;
+        bool const store_l = add_l != nullptr && !adds_here(lhs, l), store_r = add_r != nullptr && !adds_here(rhs, l);
         b = [=](device_stream_t const &s) {
-          for (void *g : {add_l, add_r}) {
-            if (g != nullptr) {
+          for (int side = 0; side < 2; side++) {
+            void *g = side == 0 ? add_l : add_r;
+            if (g == nullptr) continue;
+            if (side == 0 ? store_l : store_r) {
+              check_ffk(ffk_cast_forward(s.require_gpu(), type, type, dy, g, n), "ElementBinary backward");
+            } else {
               check_ffk(ffk_element_binary_forward(s.require_gpu(), type, FFK_OP_EW_ADD, g, dy, g, n, n, n), "ElementBinary backward");
             }
           }
