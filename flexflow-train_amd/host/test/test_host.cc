@@ -1046,7 +1046,7 @@ static void bench_step(int steps) {
   tensor_guid_t out = cgb.add(r1, cgb.dropout(f2, 0.1f));
   device_id_t dev = make_device_id_t_from_idx(0, DeviceType::GPU);
   ComputationGraphInstance inst = create_computation_graph_instance(
-      cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{1e-3, 0.0, false, 0.0}}, std::nullopt, {}, gpu,
+      cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{1e-5, 0.0, false, 0.0}}, std::nullopt, {}, gpu,
       ProfilingSettings{0, 0}, handle, dev);
   unsigned seed = 1;
   for (size_t t = 0; t < cgb.computation_graph.tensors.size(); t++) {
@@ -1059,7 +1059,9 @@ static void bench_step(int steps) {
     gpu.deallocate_tensor(d);
   }
   GenericTensorAccessorW dout = *inst.get_gradient_accessor(out);
-  GenericTensorAccessorW g = device_accessor(gpu, dout.shape, random_vec((size_t)get_num_elements(dout.shape.dims), 99));
+  // a small output gradient: with a gradient of order one per element and no loss to normalise
+  // it, a few SGD steps drive the weights to infinity
+  GenericTensorAccessorW g = device_accessor(gpu, dout.shape, random_vec((size_t)get_num_elements(dout.shape.dims), 99, -1e-3f, 1e-3f));
   copy_accessor_data_to_l_from_r(dout, g);
   device_stream_t stream = get_gpu_device_stream();
   auto step = [&] { perform_all_passes_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, dev); };
@@ -1073,6 +1075,15 @@ static void bench_step(int steps) {
   check_ffk(ffk_event_synchronize(t1), "event");
   float ms = 0;
   check_ffk(ffk_event_elapsed_ms(t0, t1, &ms), "event");
+  {
+    // the numbers are only meaningful on healthy data: a step that has diverged runs on NaNs,
+    // which toggle no bits and let the chip clock higher
+    std::vector<float> sample = to_host(inst.get_tensor_accessor(out));
+    size_t bad = 0;
+    double sum = 0;
+    for (float v : sample) bad += !std::isfinite(v), sum += std::isfinite(v) ? std::fabs(v) : 0.0;
+    printf("output after the run: %zu non-finite of %zu, mean |y| %.4f\n", bad, sample.size(), sum / (double)sample.size());
+  }
   int launches = 0;
   for (auto const &inv : inst.get_execution_order()) launches += 1, (void)inv;
   printf("step driver, encoder layer B8 S512 d1024 h16 ffn4096 bf16, FWD+BWD+SGD: %.3f ms/step over %d steps, "
