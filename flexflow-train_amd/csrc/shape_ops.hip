@@ -123,6 +123,77 @@ __global__ __launch_bounds__(kShapeThreads) void permute_tiles_kernel(E const *_
   }
 }
 
+// The same tiles moved in 16-byte pieces on both sides: a lane fetches V
+// consecutive a of one b, and later stores V consecutive b of one a, picking
+// them out of V rows of the staged tile.  Needs A, B, both strides and every
+// outer stride a multiple of V and 16-byte aligned tensors; one-element
+// transactions (128 bytes per wave for bf16) otherwise leave the bf16
+// transpose at under half of what the wide form moves.
+template <typename E, int MODE>
+__global__ __launch_bounds__(kShapeThreads) void permute_tiles_wide_kernel(E const *__restrict__ in, E *out, TileArgs t) {
+  constexpr int V = 16 / (int)sizeof(E);
+  // Row pitch of the staged tile.  4-byte elements: an odd pitch, so that the column reads of the
+  // second phase (pieces 4 rows apart, 4 output rows per wave) fall into distinct banks; the first
+  // phase then stores its piece as 4 words.  Other sizes: rows stay 16-byte aligned.
+  constexpr bool kOddPitch = sizeof(E) == 4;
+  constexpr int S = kOddPitch ? kTile + 1 : kTile + V;
+  constexpr int CPR = kTile / V;         // 16-byte pieces per tile row
+  constexpr int RPP = kShapeThreads / CPR;  // tile rows per pass
+  __shared__ __attribute__((aligned(16))) E tile[kTile * S];
+  int const piece = threadIdx.x % CPR, row = threadIdx.x / CPR;
+  int64_t const a0 = (int64_t)blockIdx.x * kTile, b0 = (int64_t)blockIdx.y * kTile;
+  for (int64_t o = blockIdx.z; o < t.outer_total; o += gridDim.z) {
+    int64_t rest = o, in_off = 0, out_off = 0;
+#pragma unroll 1
+    for (int i = t.n_outer - 1; i >= 0; i--) {
+      int64_t const r = rest / t.outer_dim[i];
+      int64_t const c = rest - r * t.outer_dim[i];
+      in_off += c * t.outer_in_stride[i];
+      out_off += c * t.outer_out_stride[i];
+      rest = r;
+    }
+#pragma unroll
+    for (int k = 0; k < kTile; k += RPP) {
+      int64_t const bb = b0 + row + k, aa = a0 + piece * V;
+      if (bb < t.B && aa < t.A) {  // A and B are multiples of V: a piece is inside or outside as a whole
+        u32x4 const q = *reinterpret_cast<u32x4 const *>(in + in_off + bb * t.in_stride_b + aa);
+        if constexpr (kOddPitch) {
+#pragma unroll
+          for (int e = 0; e < V; e++) tile[(row + k) * S + piece * V + e] = (E)q[e];
+        } else {
+          *reinterpret_cast<u32x4 *>(tile + (row + k) * S + piece * V) = q;
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kTile; k += RPP) {
+      int64_t const aa = a0 + row + k, bb = b0 + piece * V;
+      if (aa < t.A && bb < t.B) {
+        union {
+          u32x4 q;
+          E e[V];
+        } v;
+#pragma unroll
+        for (int e = 0; e < V; e++) v.e[e] = tile[(piece * V + e) * S + row + k];
+        E *dst = out + out_off + aa * t.out_stride_a + bb;
+        if constexpr (MODE != kStore) {
+          union {
+            u32x4 q;
+            E e[V];
+          } old;
+          old.q = *reinterpret_cast<u32x4 const *>(dst);
+#pragma unroll
+          for (int e = 0; e < V; e++) put<E, MODE>(&old.e[e], v.e[e]);
+          v.q = old.q;
+        }
+        *reinterpret_cast<u32x4 *>(dst) = v.q;
+      }
+    }
+    __syncthreads();
+  }
+}
+
 template <typename U, int MODE, typename E>
 __global__ __launch_bounds__(kShapeThreads) void flat_move_kernel(U const *__restrict__ in, U *out, int64_t units) {
   constexpr int EPU = sizeof(U) / sizeof(E);
@@ -244,8 +315,18 @@ static hipError_t permute_typed(hipStream_t st, void const *in, void *out, int n
   int64_t const gx = ceil_div(t.A, kTile), gy = ceil_div(t.B, kTile);
   if (gx > 0x7fffffff || gy > 65535) return hipErrorInvalidValue;
   int64_t gz = t.outer_total < 65535 ? t.outer_total : 65535;
-  permute_tiles_kernel<E, MODE><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), kShapeThreads, 0, st>>>(
-      static_cast<E const *>(in), static_cast<E *>(out), t);
+  bool wide_tiles = wide_ok && sizeof(E) >= 2 && t.A % VE == 0 && t.B % VE == 0 && t.in_stride_b % VE == 0 &&
+                    t.out_stride_a % VE == 0;
+  for (int i = 0; i < t.n_outer; i++) {
+    wide_tiles = wide_tiles && t.outer_in_stride[i] % VE == 0 && t.outer_out_stride[i] % VE == 0;
+  }
+  if (wide_tiles) {
+    permute_tiles_wide_kernel<E, MODE><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), kShapeThreads, 0, st>>>(
+        static_cast<E const *>(in), static_cast<E *>(out), t);
+  } else {
+    permute_tiles_kernel<E, MODE><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), kShapeThreads, 0, st>>>(
+        static_cast<E const *>(in), static_cast<E *>(out), t);
+  }
   return hipGetLastError();
 }
 

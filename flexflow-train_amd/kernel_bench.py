@@ -6,7 +6,7 @@ Groups: gemm (config 2 and config 5 projection GEMMs), bandwidth (config 3:
 LayerNorm, Softmax, ElementBinary, Dropout, plus GELU), embedding (config 4:
 token gather / scatter-add, DLRM bags), attention (config 5 and the config 2
 core), update (optimizer steps, Cast and loss backward over a parameter-sized
-buffer).  Every line gives the mean launch time over the timed iterations
+buffer), shape (Concat, Transpose, Gather).  Every line gives the mean launch time over the timed iterations
 (HIP events on torch's current stream, which is the stream the entry points are
 given) and the ALGORITHMIC bytes or flops of the op divided by that time,
 against 8 TB/s HBM or the 2.5 PFLOP/s dense bf16 MFMA peak.  Inputs are
@@ -197,8 +197,56 @@ def bench_update():
     report("sparse CCE loss backward [4096, 50257]", t, bytes_=8 * samples * classes)
 
 
+def bench_shape():
+    # the data-movement operators around the hot path: DLRM's interaction concat (27 parts of
+    # [16384, 128]) and a wide one, head split / merge transposes of configs 2 and 5, a 2-D
+    # transpose, a gather along the vocabulary (one logit per token)
+    parts = [torch.randn((16384, 128), device="cuda").to(BT) for _ in range(27)]
+    cat = torch.empty((16384, 27 * 128), device="cuda", dtype=BT)
+    grads = [torch.empty_like(p) for p in parts]
+    t = timeit(lambda: ffk.concat_forward(parts, 1, out=cat))
+    report("Concat 27 x [16384,128] bf16 fwd", t, bytes_=2 * cat.numel() * 2)
+    t = timeit(lambda: ffk.concat_backward(cat, grads, 1, accumulate=False))
+    report("Concat 27 x [16384,128] bf16 bwd (store)", t, bytes_=2 * cat.numel() * 2)
+    t = timeit(lambda: ffk.concat_backward(cat, grads, 1, accumulate=True))
+    report("Concat 27 x [16384,128] bf16 bwd (add)", t, bytes_=3 * cat.numel() * 2)
+    wide = [torch.randn((4096, 4096), device="cuda").to(BT) for _ in range(4)]
+    wcat = torch.empty((4096, 16384), device="cuda", dtype=BT)
+    t = timeit(lambda: ffk.concat_forward(wide, 1, out=wcat))
+    report("Concat 4 x [4096,4096] bf16 fwd", t, bytes_=2 * wcat.numel() * 2)
+    for (B, S, H, D) in [(8, 512, 16, 64), (4, 4096, 32, 128)]:
+        x = torch.randn((B, S, H, D), device="cuda").to(BT)
+        y = torch.empty((B, H, S, D), device="cuda", dtype=BT)
+        t = timeit(lambda: ffk.transpose_forward(x, (0, 2, 1, 3), out=y))
+        report("Transpose [%d,%d,%d,%d] -> (0,2,1,3) bf16" % (B, S, H, D), t, bytes_=2 * x.numel() * 2)
+    x = torch.randn((16384, 4096), device="cuda").to(BT)
+    y = torch.empty((4096, 16384), device="cuda", dtype=BT)
+    t = timeit(lambda: ffk.transpose_forward(x, (1, 0), out=y))
+    report("Transpose [16384,4096] -> (1,0) bf16", t, bytes_=2 * x.numel() * 2)
+    g = torch.zeros((16384, 4096), device="cuda", dtype=BT)
+    t = timeit(lambda: ffk.transpose_backward(y, g, (1, 0), accumulate=True))
+    report("Transpose backward (adds) [16384,4096] bf16", t, bytes_=3 * x.numel() * 2)
+    xf = torch.randn((16384, 4096), device="cuda")
+    yf = torch.empty((4096, 16384), device="cuda")
+    t = timeit(lambda: ffk.transpose_forward(xf, (1, 0), out=yf))
+    report("Transpose [16384,4096] -> (1,0) fp32", t, bytes_=2 * xf.numel() * 4)
+    logits = torch.randn((16384, 50257), device="cuda")
+    idx = torch.randint(0, 50257, (16384, 1), device="cuda", dtype=torch.int64)
+    out = torch.empty((16384, 1), device="cuda")
+    t = timeit(lambda: ffk.gather_forward(logits, idx, 1, out=out))
+    report("Gather 1 of 50257 per row, 16384 rows (fp32)", t, bytes_=16384 * (8 + 64 + 4))
+    idx2 = torch.randint(0, 4096, (16384, 1024), device="cuda", dtype=torch.int32)
+    src = torch.randn((16384, 4096), device="cuda")
+    out2 = torch.empty((16384, 1024), device="cuda")
+    t = timeit(lambda: ffk.gather_forward(src, idx2, 1, out=out2))
+    report("Gather [16384,4096] -> [16384,1024] along dim 1 (fp32)", t, bytes_=idx2.numel() * (4 + 4) + src.numel() * 4)
+    gin = torch.zeros_like(src)
+    t = timeit(lambda: ffk.gather_backward(out2, idx2, gin, 1))
+    report("Gather backward (atomics) [16384,1024] -> [16384,4096]", t, bytes_=idx2.numel() * (4 + 4 + 8))
+
+
 GROUPS = dict(gemm=bench_gemm, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention,
-              update=bench_update)
+              update=bench_update, shape=bench_shape)
 
 if __name__ == "__main__":
     ffk.lib()
