@@ -4,6 +4,7 @@
 // Host code only: every arithmetic step is one of the ffk_* kernels.
 #include "ffk_common.h"
 #include "fused_ops.h"
+#include "colreduce.h"
 #include <stdlib.h>
 
 namespace ffk {
@@ -14,7 +15,7 @@ struct LayerWs {
   size_t f1, act1, act1_drop, f2, f2_drop, pre2;
   // backward scratch
   size_t g_f2, g_act1_drop, g_act1, g_f1, g_h2, g_x1, g_attn, g_h1, g_tmp;
-  size_t mha_reserve, ln_ws, lin_ws;
+  size_t mha_reserve, ln_ws, ln_ws_b, lin_ws, lin_ws_b;  // two of each: their column sums are reduced together at the end
   size_t total;
 };
 
@@ -53,9 +54,11 @@ static LayerWs layout(ffk_encoder_layer_desc_t const *d, int dtype) {
   ffk_mha_desc_t m = mha_desc(d);
   L.mha_reserve = take(a256(ffk_mha_reserve_bytes(&m, dtype)));
   L.ln_ws = take(a256(ffk_layer_norm_backward_workspace_bytes((int64_t)T, d->d_model)));
+  L.ln_ws_b = take(a256(ffk_layer_norm_backward_workspace_bytes((int64_t)T, d->d_model)));
   size_t l1 = ffk_linear_backward_workspace_bytes(dtype, FFK_ACT_RELU, 1, (int64_t)T, d->d_ff);
   size_t l2 = ffk_linear_backward_workspace_bytes(dtype, FFK_ACT_NONE, 1, (int64_t)T, d->d_model);
   L.lin_ws = take(a256(l1 > l2 ? l1 : l2));
+  L.lin_ws_b = take(a256(l1 > l2 ? l1 : l2));
   L.total = off;
   return L;
 }
@@ -193,9 +196,19 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   float const p = d->dropout_rate;
   bool const gelu = d->activation == FFK_ACT_GELU;
   auto mean = [&](size_t o) { return reinterpret_cast<float *>(ws + o); };
-  size_t const ln_ws_bytes = L.lin_ws - L.ln_ws, lin_ws_bytes = L.total - L.lin_ws;
+  size_t const ln_ws_bytes = L.ln_ws_b - L.ln_ws, lin_ws_bytes = L.lin_ws_b - L.lin_ws;
   int const wacc = d->overwrite_weight_grads ? 0 : (FFK_ACC_WEIGHT | FFK_ACC_BIAS);
   int const mha_mode = d->overwrite_weight_grads ? FFK_MHA_OVERWRITE_WEIGHT_GRAD : 0;
+
+  // The four small column reductions of this pass (two bias gradients, two pairs of LayerNorm
+  // parameter gradients) are collected and run as one launch at the end: each is a few
+  // microseconds of launch latency for almost no work.  Their producers get scratch of their own.
+  ColreduceBatch reductions;
+  struct Collect {
+    ColreduceBatch *saved;
+    explicit Collect(ColreduceBatch *b) : saved(tl_colreduce_batch) { tl_colreduce_batch = b; }
+    ~Collect() { tl_colreduce_batch = saved; }
+  } collect(layer_fusion_enabled() ? &reductions : tl_colreduce_batch);
 
   // ---- tail: y = x1 + f2_drop (pre-LN) or y = LN2(x1 + f2_drop) (post-LN)
   void const *g_sum = dy;  // gradient of (x1 + f2_drop)
@@ -223,10 +236,10 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
                                          ws + L.g_f1, T * F, 0));
     }
     FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_NONE, 0, ws + L.f1, ws + L.g_f1, ffn_in, ws + L.g_h2,
-                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws, lin_ws_bytes, wacc));
+                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws_b, lin_ws_bytes, wacc));
   } else {
     FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_RELU, 0, ws + L.act1, ws + L.g_act1, ffn_in, ws + L.g_h2,
-                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws, lin_ws_bytes, wacc));
+                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws_b, lin_ws_bytes, wacc));
   }
   // ---- gradient reaching x1
   if (d->pre_layer_norm) {
@@ -259,21 +272,22 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
     if (layer_fusion_enabled()) {
       rc = layer_norm_backward_add_residual(as_stream(st), dtype, ws + L.g_h1, x, mean(L.mean1), mean(L.rstd1),
                                             w->ln1_gamma, g_attn_res, dx, g->ln1_gamma, g->ln1_beta, T, E,
-                                            ws + L.ln_ws, ln_ws_bytes);
+                                            ws + L.ln_ws_b, ln_ws_bytes);
       if (rc != FFK_OK && rc != FFK_ERR_UNSUPPORTED) return rc;
     }
     if (rc == FFK_ERR_UNSUPPORTED) {
       FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h1, x, mean(L.mean1), mean(L.rstd1), w->ln1_gamma, dx,
-                                      g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+                                      g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws_b, ln_ws_bytes, 0));
       FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, dx, g_attn_res, dx, T * E, T * E, T * E));
     }
   } else {
     FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_x1, ws + L.h1, mean(L.mean1), mean(L.rstd1), w->ln1_gamma,
-                                    ws + L.g_attn, g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+                                    ws + L.g_attn, g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws_b, ln_ws_bytes, 0));
     g_attn_res = ws + L.g_attn;
     FFK_TRY(ffk_mha_backward(st, dtype, &m, x, dx, x, nullptr, x, nullptr, w->attn_weight, g->attn_weight,
                              g_attn_res, ws + L.mha_reserve, L.ln_ws - L.mha_reserve, mha_mode));
     FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, dx, g_attn_res, dx, T * E, T * E, T * E));
   }
+  FFK_HIP(colreduce_flush(as_stream(st), reductions));
   return FFK_OK;
 }
