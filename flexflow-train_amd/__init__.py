@@ -118,6 +118,8 @@ SIGNATURES = {
     "ffk_dropout_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
     "ffk_dropout_backward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64, c_int]),
     "ffk_dropout_mask": (c_int, [c_p, c_p, c_i64, c_f, c_u64, c_u64]),
+    "ffk_column_reductions_begin": (c_int, []),
+    "ffk_column_reductions_end": (c_int, [c_p]),
     "ffk_dropout_add_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
     "ffk_gelu_dropout_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
     "ffk_dropout_gelu_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_f, c_u64, c_u64]),

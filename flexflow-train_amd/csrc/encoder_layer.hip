@@ -291,3 +291,23 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   FFK_HIP(colreduce_flush(as_stream(st), reductions));
   return FFK_OK;
 }
+
+// ---------------------------------------------------------------------------
+// The same collection for callers that sequence the operators themselves.
+// ---------------------------------------------------------------------------
+static thread_local ffk::ColreduceBatch tl_caller_batch;
+
+extern "C" int ffk_column_reductions_begin(void) {
+  tl_caller_batch.count = 0;
+  tl_caller_batch.dtype = -1;
+  ffk::tl_colreduce_batch = &tl_caller_batch;
+  return FFK_OK;
+}
+
+extern "C" int ffk_column_reductions_end(ffk_stream_t stream) {
+  if (ffk::tl_colreduce_batch != &tl_caller_batch) return FFK_OK;  // nothing was begun on this thread
+  ffk::tl_colreduce_batch = nullptr;
+  FFK_HIP(ffk::colreduce_flush(as_stream(stream), tl_caller_batch));
+  return FFK_OK;
+}
+

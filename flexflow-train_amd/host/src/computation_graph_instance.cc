@@ -136,7 +136,9 @@ struct Planner {
 struct LayerPlan {
   BackwardPlan bwd;
   Slot saved;        // state kept from forward to backward (LayerNorm statistics, attention reserve)
-  size_t scratch_bytes = 0;  // backward scratch, shared between layers
+  size_t scratch_bytes = 0;  // backward scratch, shared between layers ...
+  bool own_scratch = false;  // ... unless its partial sums must survive until the end of the pass
+  Slot scratch;
 };
 
 bool is_op_layer(ComputationGraph::Layer const &l) {
@@ -270,6 +272,7 @@ ComputationGraphInstance create_computation_graph_instance(
       p.scratch_bytes = ffk_linear_backward_workspace_bytes(dt(shape_of(layer.outputs[0]).data_type), activation_code(a->activation),
                                                             a->use_bias, batch, a->out_channels);
       // one flag per gradient: input, weight, bias (a weight shared between layers is added into)
+      p.own_scratch = a->use_bias;  // the bias gradient's last step is collected (ffk_column_reductions_begin)
       p.bwd.accumulate_input = {acc};
       for (tensor_guid_t w : layer.weights) p.bwd.accumulate_input.push_back(writers[w.raw] > 1);
       acc = false;
@@ -291,6 +294,7 @@ ComputationGraphInstance create_computation_graph_instance(
       }
       p.saved = saved_planner.take(align_up((size_t)M * 4) * 2);
       p.scratch_bytes = ffk_layer_norm_backward_workspace_bytes(M, N);
+      p.own_scratch = !layer.weights.empty();
     } else if (auto const *a = std::get_if<MultiHeadAttentionAttrs>(&oa)) {
       ffk_mha_desc_t d = mha_desc(*a, shape_of(layer.inputs[0]), shape_of(layer.inputs[1]), shape_of(layer.inputs[2]));
       p.saved = saved_planner.take(ffk_mha_reserve_bytes(&d, dt(shape_of(layer.inputs[0]).data_type)));
@@ -378,7 +382,7 @@ ComputationGraphInstance create_computation_graph_instance(
         if (has_grad[t.raw]) cleared[t.raw] = true;
       }
     }
-    scratch_bytes = std::max(scratch_bytes, p.scratch_bytes);
+    if (!p.own_scratch) scratch_bytes = std::max(scratch_bytes, p.scratch_bytes);
     // an input without a gradient still needs somewhere for the kernel to write
     if (p.bwd.has_backward && !std::holds_alternative<LinearAttrs>(oa) && !std::holds_alternative<EmbeddingAttrs>(oa)) {
       for (tensor_guid_t t : layer.inputs) {
@@ -535,6 +539,9 @@ ComputationGraphInstance create_computation_graph_instance(
   }
   size_t const saved_base = arena.take(saved_planner.total).offset;
   size_t const scratch_base = arena.take(scratch_bytes).offset;
+  for (size_t l = 0; l < L; l++) {
+    if (plan[l].own_scratch && plan[l].scratch_bytes > 0) plan[l].scratch = arena.take(plan[l].scratch_bytes);
+  }
   size_t const discard_base = arena.take(discard_bytes).offset;
   st->arena_bytes = arena.total;
   st->arena = static_cast<char *>(allocator.allocate(std::max<size_t>(arena.total, 256)));
@@ -566,7 +573,7 @@ ComputationGraphInstance create_computation_graph_instance(
     st->opt_v[t] = f32_accessor(t, v_slot[t]);
     st->opt_m[t] = f32_accessor(t, m_slot[t]);
   }
-  void *const scratch = base + scratch_base;
+  void *const shared_scratch = base + scratch_base;
   void *const discard = base + discard_base;
   ComputationGraphInstance::State *const S = st.get();  // closures must not own the state they live in
 
@@ -586,6 +593,7 @@ ComputationGraphInstance create_computation_graph_instance(
     void *const y = val(out);
     void *const dy = grd(out);
     size_t const ws_bytes = p.scratch_bytes;
+    void *const scratch = p.own_scratch ? static_cast<void *>(base + p.scratch.offset) : shared_scratch;
     std::function<void(device_stream_t const &)> f, b;
 
     if (auto const *a = std::get_if<LinearAttrs>(&oa)) {
@@ -974,18 +982,36 @@ ComputationGraphInstance create_computation_graph_instance(
 static LayerTimings execute(ComputationGraphInstance const &instance, ProfilingSettings const &profiling,
                             std::function<bool(DynamicTaskType)> const &selected) {
   LayerTimings result;
-  bool cleared = false, masters = false;
-  for (DynamicNodeInvocation const &inv : instance.get_execution_order()) {
-    if (!selected(inv.task_type)) continue;
-    if (!cleared && (inv.task_type == DynamicTaskType::LOSS || inv.task_type == DynamicTaskType::BWD)) {
-      instance.clear_accumulated_gradients(get_gpu_device_stream());
-      cleared = true;
+  bool cleared = false, masters = false, collecting = false;
+  // The last step of every bias and LayerNorm parameter gradient is collected over the backward
+  // pass and run as one launch behind it (not when invocations are repeated for timing).
+  bool const collect = profiling.warmup_iters == 0 && profiling.measure_iters == 0;
+  auto end_collection = [&] {
+    if (collecting) check_ffk(ffk_column_reductions_end(get_gpu_device_stream().require_gpu()), "column reductions");
+    collecting = false;
+  };
+  try {
+    for (DynamicNodeInvocation const &inv : instance.get_execution_order()) {
+      if (!selected(inv.task_type)) continue;
+      if (!cleared && (inv.task_type == DynamicTaskType::LOSS || inv.task_type == DynamicTaskType::BWD)) {
+        instance.clear_accumulated_gradients(get_gpu_device_stream());
+        cleared = true;
+      }
+      if (inv.task_type == DynamicTaskType::BWD && collect && !collecting) {
+        check_ffk(ffk_column_reductions_begin(), "column reductions");
+        collecting = true;
+      }
+      if (inv.task_type == DynamicTaskType::UPD) end_collection();
+      if (!masters && inv.task_type == DynamicTaskType::UPD) {
+        if (!instance.state->masters_valid) instance.sync_master_weights();
+        masters = true;
+      }
+      result[inv.layer_guid] = profiling_wrapper(inv.run, profiling, DeviceType::GPU);
     }
-    if (!masters && inv.task_type == DynamicTaskType::UPD) {
-      if (!instance.state->masters_valid) instance.sync_master_weights();
-      masters = true;
-    }
-    result[inv.layer_guid] = profiling_wrapper(inv.run, profiling, DeviceType::GPU);
+    end_collection();
+  } catch (...) {
+    if (collecting) ffk_column_reductions_end(get_gpu_device_stream().require_gpu());
+    throw;
   }
   return result;
 }

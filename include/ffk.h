@@ -464,6 +464,20 @@ int ffk_encoder_layer_backward(ffk_stream_t stream, int dtype,
                                void const *x, void const *dy, void *dx,
                                void *workspace, size_t workspace_bytes);
 
+/* Between _begin and _end, on the calling thread, the last step of every bias
+ * gradient (ffk_linear_backward) and LayerNorm parameter gradient
+ * (ffk_layer_norm_backward) -- a column sum over a few hundred partial rows,
+ * microseconds of launch latency for almost no work -- is not launched but
+ * collected (up to 8; further ones run at once); _end runs the collected ones
+ * as ONE launch on `stream`, which must be the stream the operators ran on.
+ * Until then their outputs are not written, and each collected call must have
+ * been given workspace of its own (the partial sums stay there).  No
+ * counterpart in the reference, which launches every kernel separately; for
+ * executors that run a whole backward pass (the step driver of the host
+ * mirror does this).  ffk_encoder_layer_backward does the same internally.   */
+int ffk_column_reductions_begin(void);
+int ffk_column_reductions_end(ffk_stream_t stream);
+
 /* ------------------------------------------------------------------------ */
 /* Optimizer updates -- sgd_update_task / adam_update_task
  * (lib/kernels/include/kernels/optimizer_kernels.h:11-36; CUDA bodies
