@@ -232,3 +232,41 @@ def test_linear_bf16_pipelined(ffk, oracle, act):
     dw_ref = oracle.gemm_f64(np.ascontiguousarray(gmat[:, orows]), x, trans_a=True)
     assert_close(to_np(dw)[orows], dw_ref, BF16_RTOL, "dw rows")
     assert_close(to_np(db), gmat.astype(np.float64).sum(0), BF16_RTOL, "db")
+
+
+def test_collected_column_reductions_equal_immediate_ones(ffk):
+    """Between ffk_column_reductions_begin and _end the bias gradients are not written; _end
+    writes all of them with one launch, and they equal the ones computed call by call."""
+    say("collected column reductions")
+    g = rng(77)
+    bt = torch.bfloat16
+    cases = []
+    for (batch, in_dim, out_dim) in [(512, 256, 384), (300, 128, 1000), (64, 64, 32)]:
+        x = to_dev(bf16_round(g.standard_normal((batch, in_dim)).astype(np.float32)), torch, bt)
+        w = to_dev(bf16_round(g.standard_normal((out_dim, in_dim)).astype(np.float32) * 0.1), torch, bt)
+        dy = to_dev(bf16_round(g.standard_normal((batch, out_dim)).astype(np.float32)), torch, bt)
+        cases.append((x, w, dy))
+    want = []
+    for x, w, dy in cases:
+        db = torch.zeros((w.shape[0],), dtype=bt, device="cuda")
+        ffk.linear_backward(dy, dy, x, w, db=db, accumulate=0)
+        want.append(db)
+    got = [torch.full((w.shape[0],), 7.0, dtype=bt, device="cuda") for _, w, _ in cases]
+    keep = []  # every collected call needs workspace of its own until _end
+    ffk.check(ffk.lib().ffk_column_reductions_begin())
+    try:
+        for (x, w, dy), db in zip(cases, got):
+            need = ffk.lib().ffk_linear_backward_workspace_bytes(ffk.BF16, ffk.ACT_NONE, 1, x.shape[0], w.shape[0])
+            ws = torch.empty((need,), dtype=torch.uint8, device="cuda")
+            keep.append(ws)
+            ffk.linear_backward(dy, dy, x, w, db=db, accumulate=0, workspace=ws)
+        torch.cuda.synchronize()
+        assert all(bool((db == 7.0).all()) for db in got)  # nothing written yet
+    finally:
+        ffk.check(ffk.lib().ffk_column_reductions_end(ffk.current_stream()))
+    torch.cuda.synchronize()
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    # _end without _begin is a no-op
+    ffk.check(ffk.lib().ffk_column_reductions_end(ffk.current_stream()))
+
