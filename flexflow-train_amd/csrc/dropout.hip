@@ -14,54 +14,10 @@
 // move 2 tensors only.
 #include "ffk_common.h"
 #include "fused_ops.h"
+#include "dropout_rng.h"
 #include <math.h>
 
 namespace ffk {
-
-struct PhiloxKey {
-  uint32_t k0, k1;
-};
-
-__device__ __forceinline__ void philox4x32_10(uint64_t block, PhiloxKey key,
-                                              uint32_t (&out)[4]) {
-  uint32_t c0 = (uint32_t)block, c1 = (uint32_t)(block >> 32), c2 = 0u, c3 = 0u;
-  uint32_t k0 = key.k0, k1 = key.k1;
-#pragma unroll
-  for (int r = 0; r < 10; r++) {
-    uint64_t p0 = (uint64_t)0xD2511F53u * c0;
-    uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
-    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
-    uint32_t n1 = (uint32_t)p1;
-    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
-    uint32_t n3 = (uint32_t)p0;
-    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
-    k0 += 0x9E3779B9u;
-    k1 += 0xBB67AE85u;
-  }
-  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
-}
-
-struct DropoutParams {
-  PhiloxKey key;
-  uint64_t offset;
-  uint32_t threshold;  // keep iff the element's 16 bits >= threshold (0 .. 65536)
-  float scale;         // 1 / (1 - rate)
-};
-
-// h: position of the element in its block of 8
-__device__ __forceinline__ bool keep(uint32_t const (&w)[4], int h, DropoutParams const &p) {
-  uint32_t const word = w[h >> 1];
-  uint32_t const half = (h & 1) ? (word >> 16) : (word & 0xffffu);
-  return half >= p.threshold;
-}
-__device__ __forceinline__ bool keep_dynamic(uint32_t const (&w)[4], uint32_t h, DropoutParams const &p) {
-  uint32_t word = w[0];
-  if ((h >> 1) == 1) word = w[1];
-  if ((h >> 1) == 2) word = w[2];
-  if ((h >> 1) == 3) word = w[3];
-  uint32_t const half = (h & 1) ? (word >> 16) : (word & 0xffffu);
-  return half >= p.threshold;
-}
 
 constexpr int kDropThreads = 256;
 
@@ -141,17 +97,6 @@ __global__ __launch_bounds__(kDropThreads) void dropout_mask_kernel(
   }
 }
 
-static int make_params(char const *who, float rate, uint64_t seed,
-                       uint64_t offset, DropoutParams &p) {
-  FFK_REQUIRE(rate >= 0.0f && rate <= 1.0f, "%s: rate %f outside [0, 1]", who, (double)rate);
-  p.threshold = (uint32_t)ceil((double)rate * 65536.0);  // 65536 (rate above 1 - 2^-16): everything dropped
-  p.key.k0 = (uint32_t)seed;
-  p.key.k1 = (uint32_t)(seed >> 32);
-  p.offset = offset;
-  p.scale = 1.0f / (1.0f - rate);
-  return FFK_OK;
-}
-
 // one pass over the tensor (a capped, looping grid measured slower)
 static int grid_for(int64_t items) {
   int64_t b = ceil_div(items > 0 ? items : 1, kDropThreads);
@@ -204,7 +149,7 @@ static int dropout_fused(char const *who, int mode, hipStream_t st, int dtype,
                          float rate, uint64_t seed, uint64_t offset) {
   FFK_REQUIRE(dropout_fusable(dtype, x, aux, y, n, offset), "%s: operands not fusable", who);
   DropoutParams p;
-  int rc = make_params(who, rate, seed, offset, p);
+  int rc = make_dropout_params(who, rate, seed, offset, p);
   if (rc != FFK_OK) return rc;
   if (dtype == FFK_FLOAT) {
     if (mode == kDropAfterGelu) return dropout_fused_typed<float, kDropAfterGelu>(st, x, aux, y, n, p);
@@ -243,7 +188,7 @@ extern "C" int ffk_dropout_forward(ffk_stream_t stream, int dtype,
                                    uint64_t seed, uint64_t offset) {
   FFK_REQUIRE(num_elements >= 0, "dropout_forward: negative size");
   DropoutParams p;
-  int rc = make_params("dropout_forward", rate, seed, offset, p);
+  int rc = make_dropout_params("dropout_forward", rate, seed, offset, p);
   if (rc != FFK_OK) return rc;
   if (num_elements == 0) return FFK_OK;
   FFK_REQUIRE(input && output, "dropout_forward: NULL tensor");
@@ -259,7 +204,7 @@ extern "C" int ffk_dropout_backward(ffk_stream_t stream, int dtype,
                                     int accumulate) {
   FFK_REQUIRE(num_elements >= 0, "dropout_backward: negative size");
   DropoutParams p;
-  int rc = make_params("dropout_backward", rate, seed, offset, p);
+  int rc = make_dropout_params("dropout_backward", rate, seed, offset, p);
   if (rc != FFK_OK) return rc;
   if (num_elements == 0) return FFK_OK;
   FFK_REQUIRE(output_grad && input_grad, "dropout_backward: NULL tensor");
@@ -303,7 +248,7 @@ extern "C" int ffk_dropout_mask(ffk_stream_t stream, uint8_t *mask,
                                 uint64_t offset) {
   FFK_REQUIRE(num_elements >= 0, "dropout_mask: negative size");
   DropoutParams p;
-  int rc = make_params("dropout_mask", rate, seed, offset, p);
+  int rc = make_dropout_params("dropout_mask", rate, seed, offset, p);
   if (rc != FFK_OK) return rc;
   if (num_elements == 0) return FFK_OK;
   FFK_REQUIRE(mask != nullptr, "dropout_mask: NULL mask");

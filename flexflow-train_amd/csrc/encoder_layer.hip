@@ -141,9 +141,17 @@ extern "C" int ffk_encoder_layer_forward(ffk_stream_t st, int dtype,
   void *ffn_in;
   if (d->pre_layer_norm) {
     // x1 = dropout(attn) + x (the reference's encoder applies no dropout here)
-    FFK_TRY(dropout_then_add(st, dtype, ws + L.attn_out, ws + L.attn_drop, x, ws + L.x1, T * E, p, d->seed + 0));
-    FFK_TRY(ffk_layer_norm_forward(st, dtype, ws + L.x1, ws + L.h2, w->ln2_gamma, w->ln2_beta,
-                                   mean(L.mean2), mean(L.rstd2), T, E, d->ln_eps));
+    int rc = FFK_ERR_UNSUPPORTED;
+    if (layer_fusion_enabled()) {
+      rc = dropout_add_layer_norm_forward(as_stream(st), dtype, ws + L.attn_out, x, ws + L.x1, ws + L.h2, w->ln2_gamma,
+                                          w->ln2_beta, mean(L.mean2), mean(L.rstd2), T, E, d->ln_eps, p, d->seed + 0, 0);
+      if (rc != FFK_OK && rc != FFK_ERR_UNSUPPORTED) return rc;
+    }
+    if (rc == FFK_ERR_UNSUPPORTED) {
+      FFK_TRY(dropout_then_add(st, dtype, ws + L.attn_out, ws + L.attn_drop, x, ws + L.x1, T * E, p, d->seed + 0));
+      FFK_TRY(ffk_layer_norm_forward(st, dtype, ws + L.x1, ws + L.h2, w->ln2_gamma, w->ln2_beta,
+                                     mean(L.mean2), mean(L.rstd2), T, E, d->ln_eps));
+    }
     ffn_in = ws + L.h2;
   } else {
     // h1 = attn + x ; x1 = LN1(h1)

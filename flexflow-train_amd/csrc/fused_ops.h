@@ -28,6 +28,14 @@ int dropout_backward_gelu_backward(hipStream_t st, int dtype, void const *dy,
 int gelu_dropout_forward(hipStream_t st, int dtype, void const *x, void *y,
                          int64_t n, float rate, uint64_t seed, uint64_t offset);
 
+// summed = residual + dropout(in); y = LayerNorm(summed), statistics kept as the separate
+// LayerNorm would.  Returns FFK_ERR_UNSUPPORTED (without setting an error
+// message) when the row length or the alignment has no vector kernel.
+int dropout_add_layer_norm_forward(hipStream_t st, int dtype, void const *in, void const *residual,
+                                   void *summed, void *y, void const *gamma, void const *beta,
+                                   float *mean, float *rstd, int64_t M, int64_t N, float eps,
+                                   float rate, uint64_t seed, uint64_t offset);
+
 // dx = residual + LayerNorm_backward(dy) (dgamma/dbeta as the separate op);
 // FFK_ERR_UNSUPPORTED when the row length has no vector kernel.
 int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,

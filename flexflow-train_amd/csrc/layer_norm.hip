@@ -14,14 +14,19 @@
 #include "rowwise.h"
 #include "colreduce.h"
 #include "fused_ops.h"
+#include "dropout_rng.h"
 
 namespace ffk {
 
-template <typename T, int EPT, int WPR>
+// PRE: the row normalised is residual + dropout(X), computed here, rounded to T where the two
+// separate operators would have stored it, and written to `summed` as well.
+template <typename T, int EPT, int WPR, bool PRE = false>
 __global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_kernel(
     T const *__restrict__ X, T *__restrict__ Y, T const *__restrict__ gamma,
     T const *__restrict__ beta, float *__restrict__ mean,
-    float *__restrict__ rstd, int64_t M, int N, float eps) {
+    float *__restrict__ rstd, int64_t M, int N, float eps,
+    T const *__restrict__ residual = nullptr, T *__restrict__ summed = nullptr,
+    DropoutParams drop = DropoutParams{}) {
   constexpr int V = VecIO<T>::kVec;
   constexpr int RPB = 4 / WPR;  // rows per workgroup
   constexpr int LANES = 64 * WPR;
@@ -40,6 +45,27 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_kernel(
     int v = lane + j * LANES;
     if (v < nvec) {
       VecIO<T>::load(xr + (int64_t)v * V, x[j]);
+      if constexpr (PRE) {
+        static_assert(V == 4 || V == 8, "a lane's vector is a Philox block or half of one");
+        if (row_ok) {
+          int64_t const at = row * (int64_t)N + (int64_t)v * V;
+          float r[V];
+          VecIO<T>::load(residual + at, r);
+          uint64_t const e0 = drop.offset + (uint64_t)at;
+          uint32_t w[4];
+          philox4x32_10(e0 >> 3, drop.key, w);
+          if (V == 4 && (e0 & 4)) {
+            w[0] = w[2];
+            w[1] = w[3];
+          }
+#pragma unroll
+          for (int e = 0; e < V; e++) {
+            float const d = keep(w, e, drop) ? x[j][e] * drop.scale : 0.0f;
+            x[j][e] = storage_round<T>(storage_round<T>(d) + r[e]);
+          }
+          VecIO<T>::store(summed + at, x[j]);
+        }
+      }
 #pragma unroll
       for (int e = 0; e < V; e++) s += x[j][e];
     } else {
@@ -432,6 +458,42 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
     }
   }
   return FFK_OK;
+}
+
+template <typename T>
+static int ln_forward_pre(hipStream_t st, void const *in, void const *residual, void *summed, void *y,
+                          void const *gamma, void const *beta, float *mean, float *rstd, int64_t M, int64_t N,
+                          float eps, DropoutParams const &drop) {
+  constexpr int V = VecIO<T>::kVec;
+  int ept = 0, wpr = 0;
+  bool vec = (N % 8 == 0) && (drop.offset & 7) == 0 && aligned16(in) && aligned16(residual) && aligned16(summed) &&
+             aligned16(y) && (gamma == nullptr || aligned16(gamma)) && (beta == nullptr || aligned16(beta)) &&
+             pick_row_config_small(N / V, ept, wpr);
+  if (!vec) return FFK_ERR_UNSUPPORTED;
+  int64_t blocks = ceil_div(M, 4 / wpr);
+#define CALL(E, W)                                                                                  \
+  layer_norm_fwd_kernel<T, E, W, true><<<(unsigned)blocks, kRowThreads, 0, st>>>(                  \
+      static_cast<T const *>(in), static_cast<T *>(y), static_cast<T const *>(gamma),             \
+      static_cast<T const *>(beta), mean, rstd, M, (int)N, eps, static_cast<T const *>(residual), \
+      static_cast<T *>(summed), drop)
+  FFK_ROW_DISPATCH_SMALL(ept, wpr, CALL);
+#undef CALL
+  FFK_CHECK_LAUNCH();
+  return FFK_OK;
+}
+
+int dropout_add_layer_norm_forward(hipStream_t st, int dtype, void const *in, void const *residual,
+                                   void *summed, void *y, void const *gamma, void const *beta,
+                                   float *mean, float *rstd, int64_t M, int64_t N, float eps,
+                                   float rate, uint64_t seed, uint64_t offset) {
+  FFK_REQUIRE(M > 0 && N > 0 && M < (1ll << 31) && N < (1ll << 31), "dropout_add_layer_norm: bad shape");
+  FFK_REQUIRE(in && residual && summed && y && mean && rstd, "dropout_add_layer_norm: NULL tensor");
+  DropoutParams drop;
+  int rc = make_dropout_params("dropout_add_layer_norm", rate, seed, offset, drop);
+  if (rc != FFK_OK) return rc;
+  if (dtype == FFK_FLOAT) return ln_forward_pre<float>(st, in, residual, summed, y, gamma, beta, mean, rstd, M, N, eps, drop);
+  if (dtype == FFK_BF16) return ln_forward_pre<bf16>(st, in, residual, summed, y, gamma, beta, mean, rstd, M, N, eps, drop);
+  return FFK_ERR_UNSUPPORTED;
 }
 
 int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
