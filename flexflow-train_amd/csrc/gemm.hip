@@ -946,13 +946,10 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
     bool const fits128 = M % 128 == 0 && N % 128 == 0;
     int64_t const t256 = fits256 ? (int64_t)(M / 256) * (N / 256) : 0;
     int64_t const t128 = fits128 ? (int64_t)(M / 128) * (N / 128) : 0;
-    // 256x256x64 tiles (8 waves of 128x64, two 64 KB stages) halve the L2->LDS
-    // traffic per flop and fetch whole 128-byte lines; they win whenever they
-    // still occupy most CUs.  Otherwise 128x128x64 tiles with 8 waves of 64x32
-    // keep two waves per SIMD on every CU.
-    if (variant == 2562 && fits256) {
-      return launch_pipe<256, 256, 128, 64, 64, 2, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
-    }
+    // 256x256 tiles (8 waves of 128x64, four 32-deep stages of 32 KB whose
+    // refills are spread over the k-steps) halve the L2->LDS traffic per flop;
+    // they win whenever they still occupy most CUs.  Otherwise 128x128x64 tiles
+    // with 8 waves of 64x32 keep two waves per SIMD on every CU.
     if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) {
       return launch_pipe<256, 256, 128, 64, 32, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
