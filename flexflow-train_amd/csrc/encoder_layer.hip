@@ -250,14 +250,19 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
                                 w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws_b, lin_ws_bytes, wacc));
   }
   // ---- gradient reaching x1
+  bool g_attn_ready = false;  // the attention branch's dropout backward already done
   if (d->pre_layer_norm) {
     // g_x1 = LN2_backward(g_h2) + dy
     int rc = FFK_ERR_UNSUPPORTED;
     if (layer_fusion_enabled()) {
+      // ... and g_attn = dropout_backward(g_x1) on the way, when the mask comes in whole blocks
+      bool const with_drop = T * E % 8 == 0 && E % 8 == 0;
       rc = layer_norm_backward_add_residual(as_stream(st), dtype, ws + L.g_h2, ws + L.x1, mean(L.mean2),
                                             mean(L.rstd2), w->ln2_gamma, dy, ws + L.g_x1, g->ln2_gamma,
-                                            g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes);
+                                            g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes,
+                                            with_drop ? ws + L.g_attn : nullptr, p, d->seed + 0, 0);
       if (rc != FFK_OK && rc != FFK_ERR_UNSUPPORTED) return rc;
+      g_attn_ready = rc == FFK_OK && with_drop;
     }
     if (rc == FFK_ERR_UNSUPPORTED) {
       FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h2, ws + L.x1, mean(L.mean2), mean(L.rstd2), w->ln2_gamma,
@@ -271,7 +276,7 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   void const *g_attn_res;  // gradient of (attn (+dropout) + x)
   if (d->pre_layer_norm) {
     g_attn_res = ws + L.g_x1;
-    FFK_TRY(ffk_dropout_backward(st, dtype, g_attn_res, ws + L.g_attn, T * E, p, d->seed + 0, 0, 0));
+    if (!g_attn_ready) FFK_TRY(ffk_dropout_backward(st, dtype, g_attn_res, ws + L.g_attn, T * E, p, d->seed + 0, 0, 0));
     FFK_TRY(ffk_mha_backward(st, dtype, &m, ws + L.h1, ws + L.g_h1, ws + L.h1, nullptr, ws + L.h1, nullptr,
                              w->attn_weight, g->attn_weight, ws + L.g_attn, ws + L.mha_reserve,
                              L.ln_ws - L.mha_reserve, mha_mode));

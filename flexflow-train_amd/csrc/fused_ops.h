@@ -44,6 +44,9 @@ int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
                                      void const *residual, void *dx,
                                      void *dgamma, void *dbeta, int64_t M,
                                      int64_t N, void *workspace,
-                                     size_t workspace_bytes);
+                                     size_t workspace_bytes,
+                                     // optional: dropped = dropout_backward(dx as stored)
+                                     void *dropped = nullptr, float rate = 0.0f,
+                                     uint64_t seed = 0, uint64_t offset = 0);
 
 }  // namespace ffk

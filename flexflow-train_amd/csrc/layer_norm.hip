@@ -151,12 +151,15 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_generic_kernel(
 
 // Backward, persistent over rows so that the dgamma/dbeta partial sums stay
 // in registers until the workgroup is done.
-template <typename T, int EPT, int WPR, bool ACC>
+// DROP: dropout_backward(dX as stored) is written to `dropped` as well (the gradient entering
+// a dropout whose output fed the residual sum that this LayerNorm normalised).
+template <typename T, int EPT, int WPR, bool ACC, bool DROP = false>
 __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
     T const *__restrict__ dY, T const *__restrict__ X,
     float const *__restrict__ mean, float const *__restrict__ rstd,
     T const *__restrict__ gamma, T *dX, float *__restrict__ partials,
-    int64_t M, int N, T const *res) {
+    int64_t M, int N, T const *res, T *__restrict__ dropped = nullptr,
+    DropoutParams drop = DropoutParams{}) {
   // ACC with res == nullptr: dX += gradient (one rounding).  ACC with res set:
   // dX = res + gradient rounded to the storage type, i.e. what a separate
   // element-wise add of res to the stored gradient would give.
@@ -260,6 +263,20 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
             o[e] = ACC ? o[e] + val : val;
           }
           VecIO<T>::store(dst, o);
+          if constexpr (DROP) {
+            static_assert(V == 4 || V == 8, "a lane's vector is a Philox block or half of one");
+            int64_t const at = row * (int64_t)N + (int64_t)v * V;
+            uint64_t const e0 = drop.offset + (uint64_t)at;
+            uint32_t w[4];
+            philox4x32_10(e0 >> 3, drop.key, w);
+            if (V == 4 && (e0 & 4)) {
+              w[0] = w[2];
+              w[1] = w[3];
+            }
+#pragma unroll
+            for (int e = 0; e < V; e++) o[e] = keep(w, e, drop) ? storage_round<T>(o[e]) * drop.scale : 0.0f;
+            VecIO<T>::store(dropped + at, o);
+          }
         }
       }
     }
@@ -401,10 +418,14 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
                        float const *mean, float const *rstd, void const *gamma,
                        void *dx, void *dgamma, void *dbeta, int64_t M, int64_t N,
                        void *workspace, size_t workspace_bytes, bool acc,
-                       void const *residual = nullptr) {
+                       void const *residual = nullptr, void *dropped = nullptr,
+                       DropoutParams const *drop = nullptr) {
   constexpr int V = VecIO<T>::kVec;
   T const *RES = static_cast<T const *>(residual);
   if (RES != nullptr) acc = true;
+  if (dropped != nullptr && (RES == nullptr || dx == nullptr || N % 8 != 0 || (drop->offset & 7) != 0 || !aligned16(dropped))) {
+    return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: the dropped copy needs the residual form and whole Philox blocks");
+  }
   T const *DY = static_cast<T const *>(dy);
   T const *X = static_cast<T const *>(x);
   T const *G = static_cast<T const *>(gamma);
@@ -427,7 +448,11 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
     float *partials = static_cast<float *>(workspace);
 #define CALL(E, W)                                                             \
   do {                                                                         \
-    if (acc)                                                                   \
+    if (dropped != nullptr)                                                    \
+      layer_norm_bwd_kernel<T, E, W, true, true><<<blocks, kRowThreads, 0, st>>>( \
+          DY, X, mean, rstd, G, DX, partials, M, (int)N, RES,                  \
+          static_cast<T *>(dropped), *drop);                                   \
+    else if (acc)                                                              \
       layer_norm_bwd_kernel<T, E, W, true><<<blocks, kRowThreads, 0, st>>>(    \
           DY, X, mean, rstd, G, DX, partials, M, (int)N, RES);                 \
     else                                                                       \
@@ -502,16 +527,22 @@ int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
                                      void const *residual, void *dx,
                                      void *dgamma, void *dbeta, int64_t M,
                                      int64_t N, void *workspace,
-                                     size_t workspace_bytes) {
+                                     size_t workspace_bytes, void *dropped,
+                                     float rate, uint64_t seed, uint64_t offset) {
   FFK_REQUIRE(M > 0 && N > 0 && M < (1ll << 31) && N < (1ll << 31),
               "layer_norm_backward: bad shape");
   FFK_REQUIRE(dy && x && mean && rstd && residual && dx, "layer_norm_backward: NULL tensor");
+  DropoutParams drop;
+  if (dropped != nullptr) {
+    int rc = make_dropout_params("layer_norm_backward", rate, seed, offset, drop);
+    if (rc != FFK_OK) return rc;
+  }
   if (dtype == FFK_FLOAT)
     return ln_backward<float>(st, dy, x, mean, rstd, gamma, dx, dgamma, dbeta, M, N,
-                              workspace, workspace_bytes, true, residual);
+                              workspace, workspace_bytes, true, residual, dropped, &drop);
   if (dtype == FFK_BF16)
     return ln_backward<bf16>(st, dy, x, mean, rstd, gamma, dx, dgamma, dbeta, M, N,
-                             workspace, workspace_bytes, true, residual);
+                             workspace, workspace_bytes, true, residual, dropped, &drop);
   return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: dtype %d not supported", dtype);
 }
 
