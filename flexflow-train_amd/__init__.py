@@ -123,6 +123,12 @@ SIGNATURES = {
     "ffk_dropout_add_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
     "ffk_gelu_dropout_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
     "ffk_dropout_gelu_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_f, c_u64, c_u64]),
+    "ffk_linear_gelu_dropout_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_i64, c_i64, c_i64, c_f,
+                                                c_u64, c_u64]),
+    "ffk_linear_dropout_add_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_i64, c_i64, c_i64, c_f,
+                                               c_u64, c_u64]),
+    "ffk_linear_backward_dropout_gelu": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_i64, c_i64,
+                                                 c_i64, c_p, c_sz, c_int, c_f, c_u64, c_u64]),
     "ffk_sgd_update": (c_int, [c_p, c_int, c_f, c_f, c_int, c_f, c_p, c_i64, c_int, c_p, c_p, c_p]),
     "ffk_adam_update": (c_int, [c_p, c_int, c_f, c_f, c_f, c_f, c_f, c_p, c_i64, c_int, c_p, c_p,
                                 c_p, c_p]),
@@ -246,6 +252,44 @@ def linear_backward(y, dy, x, w, dx=None, dw=None, db=None, activation=ACT_NONE,
                                     batch, in_dim, out_dim, ptr(workspace), ws_bytes,
                                     7 if accumulate is True else int(accumulate)))
     return dx, dw, db
+
+
+def linear_gelu_dropout_forward(x, w, b, rate, seed, offset=0):
+    """(y, dropped): y = x . w^T + b, dropped = dropout(GELU(y)), one GEMM launch.
+    Raises FFKError (FFK_ERR_UNSUPPORTED) for shapes without a fused kernel."""
+    torch = _torch()
+    batch, in_dim = x.shape
+    out_dim = w.shape[0]
+    y = torch.empty((batch, out_dim), dtype=x.dtype, device=x.device)
+    dropped = torch.empty_like(y)
+    check(lib().ffk_linear_gelu_dropout_forward(current_stream(), dtype_of(x), ptr(x), ptr(y), ptr(dropped),
+                                                ptr(w), ptr(b), batch, in_dim, out_dim, rate, seed, offset))
+    return y, dropped
+
+
+def linear_dropout_add_forward(x, residual, w, b, rate, seed, offset=0):
+    """residual + dropout(x . w^T + b), one GEMM launch."""
+    torch = _torch()
+    batch, in_dim = x.shape
+    out_dim = w.shape[0]
+    y = torch.empty((batch, out_dim), dtype=x.dtype, device=x.device)
+    check(lib().ffk_linear_dropout_add_forward(current_stream(), dtype_of(x), ptr(x), ptr(residual), ptr(y),
+                                               ptr(w), ptr(b), batch, in_dim, out_dim, rate, seed, offset))
+    return y
+
+
+def linear_backward_dropout_gelu(dy, x, gelu_input, w, rate, seed, offset=0, dw=None, db=None, accumulate=0):
+    """Linear backward whose input gradient is dropout_backward(dy . w) * GELU'(gelu_input)."""
+    torch = _torch()
+    batch, in_dim = x.shape
+    out_dim = w.shape[0]
+    dx = torch.empty_like(x)
+    need = lib().ffk_linear_backward_workspace_bytes(dtype_of(x), ACT_NONE, int(db is not None), batch, out_dim)
+    workspace = torch.empty((max(need, 1),), dtype=torch.uint8, device=x.device)
+    check(lib().ffk_linear_backward_dropout_gelu(current_stream(), dtype_of(x), ptr(dy), ptr(x), ptr(gelu_input),
+                                                 ptr(dx), ptr(w), ptr(dw), ptr(db), batch, in_dim, out_dim,
+                                                 ptr(workspace), need, int(accumulate), rate, seed, offset))
+    return dx
 
 
 def gemm(A, B, C, trans_a=False, trans_b=False, accumulate=False):

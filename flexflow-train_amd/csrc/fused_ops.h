@@ -28,6 +28,32 @@ int dropout_backward_gelu_backward(hipStream_t st, int dtype, void const *dy,
 int gelu_dropout_forward(hipStream_t st, int dtype, void const *x, void *y,
                          int64_t n, float rate, uint64_t seed, uint64_t offset);
 
+// output = input . weight^T + bias (stored: backward reads it);
+// dropped = dropout(GELU(output)), written by the GEMM while it stores its
+// tile.  FFK_ERR_UNSUPPORTED (no error message) when the shape does not run on
+// the pipelined bf16 GEMM tiles.
+int linear_gelu_dropout_forward(hipStream_t st, int dtype, void const *input, void *output,
+                                void *dropped, void const *weight, void const *bias, int64_t batch,
+                                int64_t in_dim, int64_t out_dim, float rate, uint64_t seed,
+                                uint64_t offset);
+
+// output = residual + dropout(input . weight^T + bias); Linear's own output
+// is not stored.  FFK_ERR_UNSUPPORTED as above.
+int linear_dropout_add_forward(hipStream_t st, int dtype, void const *input, void const *residual,
+                               void *output, void const *weight, void const *bias, int64_t batch,
+                               int64_t in_dim, int64_t out_dim, float rate, uint64_t seed,
+                               uint64_t offset);
+
+// Linear backward (no activation) whose input gradient is
+// dropout_backward(output_grad . weight) * GELU'(gelu_input): the gradient of
+// Linear's input never reaches memory on its own.  weight_grad / bias_grad as
+// ffk_linear_backward.  FFK_ERR_UNSUPPORTED as above, before any launch.
+int linear_backward_dropout_gelu(hipStream_t st, int dtype, void const *output_grad, void const *input,
+                                 void const *gelu_input, void *input_grad, void const *weight,
+                                 void *weight_grad, void *bias_grad, int64_t batch, int64_t in_dim,
+                                 int64_t out_dim, void *workspace, size_t workspace_bytes,
+                                 int accumulate, float rate, uint64_t seed, uint64_t offset);
+
 // summed = residual + dropout(in); y = LayerNorm(summed), statistics kept as the separate
 // LayerNorm would.  Returns FFK_ERR_UNSUPPORTED (without setting an error
 // message) when the row length or the alignment has no vector kernel.

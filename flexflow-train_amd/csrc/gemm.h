@@ -2,6 +2,7 @@
 // public ffk_gemm entry point.
 #pragma once
 #include "ffk_common.h"
+#include "dropout_rng.h"
 
 namespace ffk {
 
@@ -13,7 +14,28 @@ struct GemmEpilogue {
   // to occupy the chip); gemm_splitk_workspace_bytes() says how much helps.
   void *splitk_ws = nullptr;
   size_t splitk_ws_bytes = 0;
+  // Optional element-wise operators applied to the output tile while it is
+  // written (bf16 only, see gemm_tail_supported).  With a tail the GEMM gives
+  // the bits of the separate kernels run after it:
+  //   kTailGeluDropout     C = result (kept: backward reads the pre-activation),
+  //                        tail_out = dropout(GELU(C))
+  //   kTailDropoutGeluGrad C = dropout_backward(result) * GELU'(tail_in); the
+  //                        plain result is not stored
+  //   kTailDropoutAdd      C = tail_in + dropout(result); the plain result is
+  //                        not stored
+  // tail_in / tail_out are dense [M, N] tensors, the dropout stream is indexed
+  // by m * N + n from tail_dropout.offset.
+  enum Tail { kTailNone = 0, kTailGeluDropout = 1, kTailDropoutGeluGrad = 2, kTailDropoutAdd = 3 };
+  int tail = kTailNone;
+  void const *tail_in = nullptr;
+  void *tail_out = nullptr;
+  DropoutParams tail_dropout = {};
 };
+
+// Whether gemm_dispatch can run this GEMM with ep.tail (it fails otherwise).
+bool gemm_tail_supported(int dtype, bool trans_a, bool trans_b, int64_t M, int64_t N,
+                         int64_t K, void const *A, int64_t lda, void const *B, int64_t ldb,
+                         void const *C, int64_t ldc, GemmEpilogue const &ep);
 
 // C[M,N] (+)= op(A) . op(B), fp32 accumulation.
 //   trans_a == false: A is [M,K] row-major (lda = K); true: A is [K,M] (lda = M)

@@ -354,12 +354,20 @@ __device__ __forceinline__ unsigned lds_address_of(void *p) {
 // PF = how many k-steps ahead of its use a fragment is read from LDS (PF + 1
 // register buffers).  PF = 1 is what both tile configurations use; PF = 3 was
 // measured on the 128x128 tile (2 MFMAs per k-step per wave) and gained nothing.
-template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, bool TB>
+struct GemmTailArgs {
+  bf16 const *in;
+  bf16 *out;
+  DropoutParams dropout;
+};
+
+// TAIL (GemmEpilogue::Tail): element-wise operators applied to the 8-element
+// pieces of the output tile on their way from LDS to memory.
+template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, bool TB, int TAIL = 0>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
     bf16 const *__restrict__ bias, int act, int accumulate,
-    float *__restrict__ partial, int k_tiles_per_split) {
+    float *__restrict__ partial, int k_tiles_per_split, GemmTailArgs tail) {
   // partial != nullptr: split-K.  Workgroup (tile, split) reduces k-tiles
   // [split * k_tiles_per_split, +k_tiles_per_split) and stores its fp32
   // accumulators to partial[split][M][N]; a second kernel sums the splits and
@@ -669,7 +677,43 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       int c = lane + i * 64;
       int row = c / (WN / 8), ch = c % (WN / 8);
       u32x4 v = *reinterpret_cast<u32x4 const *>(cs + row * CS + ch * 8);
-      *reinterpret_cast<u32x4 *>(dst + (int64_t)(m0 + wm0 + row) * ldc + n0 + wn0 + ch * 8) = v;
+      int64_t const at = (int64_t)(m0 + wm0 + row) * ldc + n0 + wn0 + ch * 8;
+      if constexpr (TAIL == GemmEpilogue::kTailNone) {
+        *reinterpret_cast<u32x4 *>(dst + at) = v;
+      } else {
+        // ldc == N here: `at` is the element's index in the dense tensor, and
+        // the piece is one block of the dropout stream
+        uint32_t w[4];
+        philox4x32_10((tail.dropout.offset + (uint64_t)at) >> 3, tail.dropout.key, w);
+        u32x4 aux = {0u, 0u, 0u, 0u};
+        if constexpr (TAIL == GemmEpilogue::kTailGeluDropout) {
+          *reinterpret_cast<u32x4 *>(dst + at) = v;
+        } else {
+          aux = *reinterpret_cast<u32x4 const *>(tail.in + at);
+        }
+        u32x4 r;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          float x[2] = {__uint_as_float(v[q] << 16), __uint_as_float(v[q] & 0xffff0000u)};
+          float const a[2] = {__uint_as_float(aux[q] << 16), __uint_as_float(aux[q] & 0xffff0000u)};
+#pragma unroll
+          for (int h = 0; h < 2; h++) {
+            if constexpr (TAIL == GemmEpilogue::kTailGeluDropout) {
+              x[h] = storage_round<bf16>(gelu_forward(x[h]));
+            }
+            x[h] = keep(w, 2 * q + h, tail.dropout) ? x[h] * tail.dropout.scale : 0.0f;
+            if constexpr (TAIL == GemmEpilogue::kTailDropoutGeluGrad) {
+              x[h] = storage_round<bf16>(x[h]) * gelu_derivative(a[h]);
+            }
+            if constexpr (TAIL == GemmEpilogue::kTailDropoutAdd) {
+              x[h] = storage_round<bf16>(x[h]) + a[h];
+            }
+          }
+          r[q] = pack_bf16x2(x[0], x[1]);
+        }
+        bf16 *const to = TAIL == GemmEpilogue::kTailGeluDropout ? tail.out : dst;
+        *reinterpret_cast<u32x4 *>(to + at) = r;
+      }
     }
   };
   if (partial != nullptr) {
@@ -742,14 +786,16 @@ struct PipeCfg {
   static_assert(kLds <= 160 * 1024, "LDS budget");
 };
 
-template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, bool TB>
+template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, bool TB, int TAIL = 0>
 static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
                               bf16 *C, int M, int N, int K, int64_t lda,
                               int64_t ldb, int64_t ldc, GemmEpilogue const &ep,
                               int splits = 1) {
   using Cfg = PipeCfg<BM, BN, WM, WN, BK, STAGES>;
   constexpr int NT = Cfg::NW * 64;
-  auto kern = gemm_bf16_pipe_kernel<BM, BN, WM, WN, BK, STAGES, PF, TA, TB>;
+  auto kern = gemm_bf16_pipe_kernel<BM, BN, WM, WN, BK, STAGES, PF, TA, TB, TAIL>;
+  GemmTailArgs const tail = {static_cast<bf16 const *>(ep.tail_in), static_cast<bf16 *>(ep.tail_out),
+                             ep.tail_dropout};
   static bool configured = false;  // per template instance
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const *>(kern),
@@ -761,7 +807,7 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
   if (splits > 1) {
     float *partial = static_cast<float *>(ep.splitk_ws);
     kern<<<blocks * splits, NT, Cfg::kLds, st>>>(A, B, C, M, N, K, lda, ldb, ldc, nullptr,
-                                                FFK_ACT_NONE, 0, partial, K / BK / splits);
+                                                FFK_ACT_NONE, 0, partial, K / BK / splits, tail);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     int64_t const quads = (int64_t)M * N / 4;
@@ -772,7 +818,7 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
   }
   kern<<<blocks, NT, Cfg::kLds, st>>>(A, B, C, M, N, K, lda, ldb, ldc,
                                      static_cast<bf16 const *>(ep.bias), ep.activation,
-                                     ep.accumulate, nullptr, 0);
+                                     ep.accumulate, nullptr, 0, tail);
   return hipGetLastError();
 }
 
@@ -931,37 +977,81 @@ size_t gemm_splitk_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K) {
   return s > 1 ? (size_t)s * (size_t)(M * N) * sizeof(float) : 0;
 }
 
-template <bool TA, bool TB>
-static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
-                            bf16 *C, int M, int N, int K, int64_t lda,
-                            int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
+// Which pipelined tile a bf16 GEMM runs on: 256, 128, or 0 (none of the two:
+// split-K or the register-staged kernels).
+static int pipe_tile_for(bf16 const *C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                         GemmEpilogue const &ep, int variant) {
   bool const c_vec = (ldc % 8 == 0) && aligned16(C);
-  int const variant = gemm_variant_override();
   // the pipelined kernels fetch the bias in 8-byte pieces
   bool const aux_ok = reinterpret_cast<uintptr_t>(ep.bias) % 8 == 0;
   // the direct loads address an operand panel with 32-bit byte offsets
   bool const panel_ok = 2 * 256 * std::max(lda, ldb) < (int64_t(1) << 31);
-  if (c_vec && aux_ok && panel_ok && K % 64 == 0 && variant != 1) {
-    bool const fits256 = M % 256 == 0 && N % 256 == 0;
+  if (!(c_vec && aux_ok && panel_ok && K % 64 == 0 && variant != 1)) return 0;
+  bool const fits256 = M % 256 == 0 && N % 256 == 0;
+  bool const fits128 = M % 128 == 0 && N % 128 == 0;
+  int64_t const t256 = fits256 ? (int64_t)(M / 256) * (N / 256) : 0;
+  int64_t const t128 = fits128 ? (int64_t)(M / 128) * (N / 128) : 0;
+  // 256x256 tiles (8 waves of 128x64, four 32-deep stages of 32 KB whose
+  // refills are spread over the k-steps) halve the L2->LDS traffic per flop;
+  // they win whenever they still occupy most CUs.  Otherwise 128x128x64 tiles
+  // with 8 waves of 64x32 keep two waves per SIMD on every CU.
+  if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) return 256;
+  if ((variant == 0 && t128 >= kNumCU / 2) || (variant == 128 && fits128)) return 128;
+  return 0;
+}
+
+template <bool TA, bool TB>
+static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
+                            bf16 *C, int M, int N, int K, int64_t lda,
+                            int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
+  int const variant = gemm_variant_override();
+  int const pipe_tile = pipe_tile_for(C, M, N, K, lda, ldb, ldc, ep, variant);
+  {
     bool const fits128 = M % 128 == 0 && N % 128 == 0;
-    int64_t const t256 = fits256 ? (int64_t)(M / 256) * (N / 256) : 0;
-    int64_t const t128 = fits128 ? (int64_t)(M / 128) * (N / 128) : 0;
-    // 256x256 tiles (8 waves of 128x64, four 32-deep stages of 32 KB whose
-    // refills are spread over the k-steps) halve the L2->LDS traffic per flop;
-    // they win whenever they still occupy most CUs.  Otherwise 128x128x64 tiles
-    // with 8 waves of 64x32 keep two waves per SIMD on every CU.
-    if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) {
+    bool const use256 = pipe_tile == 256, use128 = pipe_tile == 128;
+    if (ep.tail != GemmEpilogue::kTailNone) {
+      // gemm_tail_supported() has been asked: one of the two tiles fits
+      if constexpr (!TA && TB) {
+        constexpr int kTail = GemmEpilogue::kTailGeluDropout;
+        if (ep.tail == kTail && use256) {
+          return launch_pipe<256, 256, 128, 64, 32, 4, 1, TA, TB, kTail>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+        }
+        if (ep.tail == kTail && use128) {
+          return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB, kTail>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+        }
+        constexpr int kAdd = GemmEpilogue::kTailDropoutAdd;
+        if (ep.tail == kAdd && use256) {
+          return launch_pipe<256, 256, 128, 64, 32, 4, 1, TA, TB, kAdd>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+        }
+        if (ep.tail == kAdd && use128) {
+          return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB, kAdd>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+        }
+      }
+      if constexpr (!TA && !TB) {
+        constexpr int kTail = GemmEpilogue::kTailDropoutGeluGrad;
+        if (ep.tail == kTail && use256) {
+          return launch_pipe<256, 256, 128, 64, 32, 4, 1, TA, TB, kTail>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+        }
+        if (ep.tail == kTail && use128) {
+          return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB, kTail>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+        }
+      }
+      return hipErrorInvalidValue;
+    }
+    if (use256) {
       return launch_pipe<256, 256, 128, 64, 32, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
-    if ((variant == 0 && t128 >= kNumCU / 2) || (variant == 128 && fits128)) {
+    if (use128) {
       return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
     // Few output tiles and a long reduction: split K so every CU has a tile.
-    int const splits = fits128 ? splitk_splits(M, N, K, ep.splitk_ws_bytes) : 1;
+    bool const pipe_ok = pipe_tile_for(C, M, N, K, lda, ldb, ldc, ep, 128) == 128;  // but for the tile count
+    int const splits = fits128 && pipe_ok ? splitk_splits(M, N, K, ep.splitk_ws_bytes) : 1;
     if (variant == 0 && splits > 1 && ep.splitk_ws != nullptr && aligned16(ep.splitk_ws)) {
       return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep, splits);
     }
   }
+  if (ep.tail != GemmEpilogue::kTailNone) return hipErrorInvalidValue;
   // Largest tile that still gives every CU a workgroup.
   int64_t const b128 = ceil_div(M, 128) * ceil_div(N, 128);
   if (b128 >= kNumCU) {
@@ -1094,6 +1184,27 @@ int colsum_dispatch(hipStream_t st, int dtype, void const *X, int64_t ldx,
   return fail(FFK_ERR_UNSUPPORTED, "colsum: dtype %d not supported", dtype);
 }
 
+bool gemm_tail_supported(int dtype, bool ta, bool tb, int64_t M, int64_t N, int64_t K,
+                         void const *A, int64_t lda, void const *B, int64_t ldb,
+                         void const *C, int64_t ldc, GemmEpilogue const &ep) {
+  if (dtype != FFK_BF16 || ta || ep.accumulate || ldc != N || M <= 0 || N <= 0 || K <= 0) return false;
+  if (M >= (1ll << 31) || N >= (1ll << 31) || K >= (1ll << 31)) return false;
+  if ((ep.tail_dropout.offset & 7) != 0) return false;
+  if (ep.tail == GemmEpilogue::kTailGeluDropout) {
+    if (!tb || ep.tail_out == nullptr || !aligned16(ep.tail_out)) return false;
+  } else if (ep.tail == GemmEpilogue::kTailDropoutGeluGrad) {
+    if (tb || ep.tail_in == nullptr || !aligned16(ep.tail_in)) return false;
+  } else if (ep.tail == GemmEpilogue::kTailDropoutAdd) {
+    if (!tb || ep.tail_in == nullptr || !aligned16(ep.tail_in)) return false;
+  } else {
+    return false;
+  }
+  bool const vec_ok = (K % 8 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && aligned16(A) && aligned16(B) &&
+                      (tb || N % 8 == 0);
+  return vec_ok && pipe_tile_for(static_cast<bf16 const *>(C), (int)M, (int)N, (int)K, lda, ldb, ldc, ep,
+                                 gemm_variant_override()) != 0;
+}
+
 int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
                   int64_t N, int64_t K, void const *A, int64_t lda,
                   void const *B, int64_t ldb, void *C, int64_t ldc,
@@ -1107,6 +1218,7 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
               "gemm: leading dimension smaller than the row length");
   hipError_t e;
   if (dtype == FFK_FLOAT) {
+    FFK_REQUIRE(ep.tail == GemmEpilogue::kTailNone, "gemm: fused tails exist for bf16 only");
     float const *a = static_cast<float const *>(A);
     float const *b = static_cast<float const *>(B);
     float *c = static_cast<float *>(C);
@@ -1123,6 +1235,9 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
 #undef FFK_LAUNCH_F32
     e = hipGetLastError();
   } else if (dtype == FFK_BF16) {
+    FFK_REQUIRE(ep.tail == GemmEpilogue::kTailNone ||
+                    gemm_tail_supported(dtype, ta, tb, M, N, K, A, lda, B, ldb, C, ldc, ep),
+                "gemm: this shape has no fused tail (ask gemm_tail_supported first)");
     bf16 const *a = static_cast<bf16 const *>(A);
     bf16 const *b = static_cast<bf16 const *>(B);
     bf16 *c = static_cast<bf16 *>(C);

@@ -93,12 +93,14 @@ extern "C" int ffk_linear_forward(ffk_stream_t stream, int dtype,
                        in_dim, input, in_dim, weight, in_dim, output, out_dim, ep);
 }
 
-extern "C" int ffk_linear_backward(
+// input_tail: operators the input gradient passes through while it is written
+// (GemmEpilogue's tail fields), or nullptr.
+static int linear_backward_impl(
     ffk_stream_t stream, int dtype, int activation, int relu_grad_mode,
     void const *output, void const *output_grad, void const *input,
     void *input_grad, void const *weight, void *weight_grad, void *bias_grad,
     int64_t batch, int64_t in_dim, int64_t out_dim, void *workspace,
-    size_t workspace_bytes, int accumulate) {
+    size_t workspace_bytes, int accumulate, GemmEpilogue const *input_tail) {
   FFK_REQUIRE(dtype == FFK_FLOAT || dtype == FFK_BF16,
               "linear_backward: dtype %d not supported", dtype);
   FFK_REQUIRE(activation >= FFK_ACT_NONE && activation <= FFK_ACT_TANH,
@@ -131,10 +133,16 @@ extern "C" int ffk_linear_backward(
   GemmEpilogue ep;
   int rc;
   if (input_grad != nullptr) {
-    ep.accumulate = (accumulate & FFK_ACC_INPUT) != 0;
+    GemmEpilogue dx = input_tail != nullptr ? *input_tail : ep;
+    dx.accumulate = (accumulate & FFK_ACC_INPUT) != 0;
     // input_grad[batch,in] = g[batch,out] . weight[out,in]
+    if (input_tail != nullptr &&
+        !gemm_tail_supported(dtype, false, false, batch, in_dim, out_dim, g, out_dim, weight, in_dim,
+                             input_grad, in_dim, dx)) {
+      return FFK_ERR_UNSUPPORTED;  // before anything is launched: the caller runs the separate operators
+    }
     rc = gemm_dispatch(st, dtype, false, false, batch, in_dim, out_dim, g, out_dim,
-                       weight, in_dim, input_grad, in_dim, ep);
+                       weight, in_dim, input_grad, in_dim, dx);
     if (rc != FFK_OK) return rc;
   }
   if (weight_grad != nullptr) {
@@ -150,4 +158,122 @@ extern "C" int ffk_linear_backward(
     if (rc != FFK_OK) return rc;
   }
   return FFK_OK;
+}
+
+extern "C" int ffk_linear_backward(
+    ffk_stream_t stream, int dtype, int activation, int relu_grad_mode,
+    void const *output, void const *output_grad, void const *input,
+    void *input_grad, void const *weight, void *weight_grad, void *bias_grad,
+    int64_t batch, int64_t in_dim, int64_t out_dim, void *workspace,
+    size_t workspace_bytes, int accumulate) {
+  return linear_backward_impl(stream, dtype, activation, relu_grad_mode, output, output_grad, input,
+                              input_grad, weight, weight_grad, bias_grad, batch, in_dim, out_dim,
+                              workspace, workspace_bytes, accumulate, nullptr);
+}
+
+namespace ffk {
+
+int linear_gelu_dropout_forward(hipStream_t st, int dtype, void const *input, void *output,
+                                void *dropped, void const *weight, void const *bias, int64_t batch,
+                                int64_t in_dim, int64_t out_dim, float rate, uint64_t seed,
+                                uint64_t offset) {
+  FFK_REQUIRE(input && output && dropped && weight, "linear_gelu_dropout_forward: NULL tensor");
+  FFK_REQUIRE(batch > 0 && in_dim > 0 && out_dim > 0, "linear_gelu_dropout_forward: non-positive dimension");
+  GemmEpilogue ep;
+  ep.bias = bias;
+  ep.tail = GemmEpilogue::kTailGeluDropout;
+  ep.tail_out = dropped;
+  int const prc = make_dropout_params("linear_gelu_dropout_forward", rate, seed, offset, ep.tail_dropout);
+  if (prc != FFK_OK) return prc;
+  if (!gemm_tail_supported(dtype, false, true, batch, out_dim, in_dim, input, in_dim, weight, in_dim,
+                           output, out_dim, ep)) {
+    return FFK_ERR_UNSUPPORTED;
+  }
+  return gemm_dispatch(st, dtype, false, true, batch, out_dim, in_dim, input, in_dim, weight, in_dim,
+                       output, out_dim, ep);
+}
+
+int linear_dropout_add_forward(hipStream_t st, int dtype, void const *input, void const *residual,
+                               void *output, void const *weight, void const *bias, int64_t batch,
+                               int64_t in_dim, int64_t out_dim, float rate, uint64_t seed,
+                               uint64_t offset) {
+  FFK_REQUIRE(input && residual && output && weight, "linear_dropout_add_forward: NULL tensor");
+  FFK_REQUIRE(batch > 0 && in_dim > 0 && out_dim > 0, "linear_dropout_add_forward: non-positive dimension");
+  GemmEpilogue ep;
+  ep.bias = bias;
+  ep.tail = GemmEpilogue::kTailDropoutAdd;
+  ep.tail_in = residual;
+  int const prc = make_dropout_params("linear_dropout_add_forward", rate, seed, offset, ep.tail_dropout);
+  if (prc != FFK_OK) return prc;
+  if (!gemm_tail_supported(dtype, false, true, batch, out_dim, in_dim, input, in_dim, weight, in_dim,
+                           output, out_dim, ep)) {
+    return FFK_ERR_UNSUPPORTED;
+  }
+  return gemm_dispatch(st, dtype, false, true, batch, out_dim, in_dim, input, in_dim, weight, in_dim,
+                       output, out_dim, ep);
+}
+
+int linear_backward_dropout_gelu(hipStream_t st, int dtype, void const *output_grad, void const *input,
+                                 void const *gelu_input, void *input_grad, void const *weight,
+                                 void *weight_grad, void *bias_grad, int64_t batch, int64_t in_dim,
+                                 int64_t out_dim, void *workspace, size_t workspace_bytes,
+                                 int accumulate, float rate, uint64_t seed, uint64_t offset) {
+  FFK_REQUIRE(output_grad && input && gelu_input && input_grad && weight,
+              "linear_backward_dropout_gelu: NULL tensor");
+  FFK_REQUIRE((accumulate & FFK_ACC_INPUT) == 0,
+              "linear_backward_dropout_gelu: the input gradient is stored, not added");
+  GemmEpilogue tail;
+  tail.tail = GemmEpilogue::kTailDropoutGeluGrad;
+  tail.tail_in = gelu_input;
+  int const prc = make_dropout_params("linear_backward_dropout_gelu", rate, seed, offset, tail.tail_dropout);
+  if (prc != FFK_OK) return prc;
+  return linear_backward_impl(st, dtype, FFK_ACT_NONE, 0, nullptr, output_grad, input, input_grad, weight,
+                              weight_grad, bias_grad, batch, in_dim, out_dim, workspace, workspace_bytes,
+                              accumulate, &tail);
+}
+
+}  // namespace ffk
+
+extern "C" int ffk_linear_gelu_dropout_forward(ffk_stream_t stream, int dtype, void const *input,
+                                               void *output, void *dropped, void const *weight,
+                                               void const *bias, int64_t batch, int64_t in_dim,
+                                               int64_t out_dim, float rate, uint64_t seed,
+                                               uint64_t offset) {
+  int const rc = ffk::linear_gelu_dropout_forward(as_stream(stream), dtype, input, output, dropped, weight,
+                                                  bias, batch, in_dim, out_dim, rate, seed, offset);
+  if (rc == FFK_ERR_UNSUPPORTED) {
+    return fail(FFK_ERR_UNSUPPORTED, "linear_gelu_dropout_forward: no fused kernel for this shape; "
+                                     "run Linear, GELU and Dropout one after the other");
+  }
+  return rc;
+}
+
+extern "C" int ffk_linear_dropout_add_forward(ffk_stream_t stream, int dtype, void const *input,
+                                              void const *residual, void *output, void const *weight,
+                                              void const *bias, int64_t batch, int64_t in_dim,
+                                              int64_t out_dim, float rate, uint64_t seed,
+                                              uint64_t offset) {
+  int const rc = ffk::linear_dropout_add_forward(as_stream(stream), dtype, input, residual, output, weight,
+                                                 bias, batch, in_dim, out_dim, rate, seed, offset);
+  if (rc == FFK_ERR_UNSUPPORTED) {
+    return fail(FFK_ERR_UNSUPPORTED, "linear_dropout_add_forward: no fused kernel for this shape; "
+                                     "run Linear, Dropout and the addition one after the other");
+  }
+  return rc;
+}
+
+extern "C" int ffk_linear_backward_dropout_gelu(
+    ffk_stream_t stream, int dtype, void const *output_grad, void const *input, void const *gelu_input,
+    void *input_grad, void const *weight, void *weight_grad, void *bias_grad, int64_t batch,
+    int64_t in_dim, int64_t out_dim, void *workspace, size_t workspace_bytes, int accumulate,
+    float rate, uint64_t seed, uint64_t offset) {
+  int const rc = ffk::linear_backward_dropout_gelu(as_stream(stream), dtype, output_grad, input, gelu_input,
+                                                   input_grad, weight, weight_grad, bias_grad, batch,
+                                                   in_dim, out_dim, workspace, workspace_bytes,
+                                                   accumulate, rate, seed, offset);
+  if (rc == FFK_ERR_UNSUPPORTED) {
+    return fail(FFK_ERR_UNSUPPORTED, "linear_backward_dropout_gelu: no fused kernel for this shape; "
+                                     "run Linear backward, Dropout backward and GELU backward one after the other");
+  }
+  return rc;
 }

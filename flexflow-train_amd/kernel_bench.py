@@ -75,6 +75,61 @@ def bench_gemm():
                flops=2.0 * M * N * K)
 
 
+def bench_fused_linear():
+    # Config 2's feed-forward block (4096 tokens, 1024 -> 4096 -> 1024): each Linear with the
+    # element-wise operators around it as separate launches and on the GEMM's tile store
+    T, E, F, rate, seed = 4096, 1024, 4096, 0.1, 2024
+    L = ffk.lib()
+    st = ffk.current_stream()
+    p = ffk.ptr
+    x = torch.randn((T, E), device="cuda").to(BT)
+    w1 = (torch.randn((F, E), device="cuda") * 0.03).to(BT)
+    b1 = torch.zeros((F,), device="cuda", dtype=BT)
+    w2 = (torch.randn((E, F), device="cuda") * 0.015).to(BT)
+    b2 = torch.zeros((E,), device="cuda", dtype=BT)
+    h, act = torch.empty((T, F), device="cuda", dtype=BT), torch.empty((T, F), device="cuda", dtype=BT)
+    y, out = torch.empty((T, E), device="cuda", dtype=BT), torch.empty((T, E), device="cuda", dtype=BT)
+    dy = torch.randn((T, E), device="cuda").to(BT)
+    dact, dh = torch.empty_like(act), torch.empty_like(h)
+    need = L.ffk_linear_backward_workspace_bytes(ffk.BF16, ffk.ACT_NONE, 0, T, E)
+    ws = torch.empty((max(need, 1),), dtype=torch.uint8, device="cuda")
+
+    def up_separate():
+        ffk.linear_forward(x, w1, b1, ffk.ACT_NONE, h)
+        ffk.check(L.ffk_gelu_dropout_forward(st, ffk.BF16, p(h), p(act), T * F, rate, seed, 0))
+
+    def up_tail():
+        ffk.check(L.ffk_linear_gelu_dropout_forward(st, ffk.BF16, p(x), p(h), p(act), p(w1), p(b1), T, E, F,
+                                                    rate, seed, 0))
+
+    def down_separate():
+        ffk.linear_forward(act, w2, b2, ffk.ACT_NONE, y)
+        ffk.check(L.ffk_dropout_add_forward(st, ffk.BF16, p(y), p(x), p(out), T * E, rate, seed, 0))
+
+    def down_tail():
+        ffk.check(L.ffk_linear_dropout_add_forward(st, ffk.BF16, p(act), p(x), p(out), p(w2), p(b2), T, F, E,
+                                                   rate, seed, 0))
+
+    def grad_separate():
+        ffk.check(L.ffk_linear_backward(st, ffk.BF16, ffk.ACT_NONE, 0, None, p(dy), p(act), p(dact), p(w2), None,
+                                        None, T, F, E, p(ws), need, 0))
+        ffk.check(L.ffk_dropout_gelu_backward(st, ffk.BF16, p(dact), p(h), p(dh), T * F, rate, seed, 0))
+
+    def grad_tail():
+        ffk.check(L.ffk_linear_backward_dropout_gelu(st, ffk.BF16, p(dy), p(act), p(h), p(dh), p(w2), None, None,
+                                                     T, F, E, p(ws), need, 0, rate, seed, 0))
+
+    flops = 2.0 * T * E * F
+    up_separate()  # h, act hold finite values for the backward timings
+    for name, fn in [("Linear 1024->4096, GELU+Dropout: 2 launches", up_separate),
+                     ("Linear 1024->4096, GELU+Dropout: on the tile store", up_tail),
+                     ("Linear 4096->1024, Dropout+add: 2 launches", down_separate),
+                     ("Linear 4096->1024, Dropout+add: on the tile store", down_tail),
+                     ("Linear 4096->1024 dX, Dropout/GELU bwd: 2 launches", grad_separate),
+                     ("Linear 4096->1024 dX, Dropout/GELU bwd: tile store", grad_tail)]:
+        report(name, timeit(fn), flops=flops)
+
+
 def bench_bandwidth():
     n = 16384 * 4096
     a = torch.randn(n, device="cuda").to(BT)
@@ -245,7 +300,7 @@ def bench_shape():
     report("Gather backward (atomics) [16384,1024] -> [16384,4096]", t, bytes_=idx2.numel() * (4 + 4 + 8))
 
 
-GROUPS = dict(gemm=bench_gemm, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention,
+GROUPS = dict(gemm=bench_gemm, fused_linear=bench_fused_linear, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention,
               update=bench_update, shape=bench_shape)
 
 if __name__ == "__main__":

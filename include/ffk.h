@@ -297,6 +297,49 @@ int ffk_dropout_gelu_backward(ffk_stream_t stream, int dtype,
                               void *input_grad, int64_t num_elements,
                               float rate, uint64_t seed, uint64_t offset);
 
+/* Linear with the GELU and the dropout that follow it, and the matching
+ * backward.  No counterpart in the reference (one kernel per operator, as
+ * above): the sequence is Linear forward (linear_kernels.cu:110-178) ->
+ * ElementUnary GELU -> Dropout, and on the way back Dropout backward -> GELU
+ * backward behind the input-gradient GEMM of the next Linear's backward
+ * (linear_kernels.cu:214-303).  The element-wise operators are applied to the
+ * GEMM's output tile while it is stored, so their intermediates never make a
+ * trip through memory; results are the bits of the separate entries run one
+ * after the other.  BF16 only, shapes that run on the pipelined GEMM tiles
+ * (batch and the GEMM's output width multiples of 128 with at least 128 tiles,
+ * reduction length a multiple of 64, 16-byte aligned tensors, offset a
+ * multiple of 8); anything else is FFK_ERR_UNSUPPORTED before any kernel is
+ * launched, and the caller runs the separate operators.
+ *   ffk_linear_gelu_dropout_forward:
+ *     output [batch, out_dim] = input . weight^T + bias   (kept for backward)
+ *     dropped [batch, out_dim] = dropout(GELU(output))
+ *   ffk_linear_dropout_add_forward:
+ *     output [batch, out_dim] = residual + dropout(input . weight^T + bias);
+ *     Linear's own output is not stored (no backward reads it)
+ *   ffk_linear_backward_dropout_gelu: Linear backward without activation
+ *     (arguments as ffk_linear_backward) of a Linear whose input [batch,
+ *     in_dim] was dropout(GELU(gelu_input)):
+ *     input_grad = dropout_backward(output_grad . weight) * GELU'(gelu_input);
+ *     FFK_ACC_INPUT is not allowed.                                          */
+int ffk_linear_gelu_dropout_forward(ffk_stream_t stream, int dtype,
+                                    void const *input, void *output,
+                                    void *dropped, void const *weight,
+                                    void const *bias, int64_t batch,
+                                    int64_t in_dim, int64_t out_dim, float rate,
+                                    uint64_t seed, uint64_t offset);
+int ffk_linear_dropout_add_forward(ffk_stream_t stream, int dtype,
+                                   void const *input, void const *residual,
+                                   void *output, void const *weight,
+                                   void const *bias, int64_t batch,
+                                   int64_t in_dim, int64_t out_dim, float rate,
+                                   uint64_t seed, uint64_t offset);
+int ffk_linear_backward_dropout_gelu(
+    ffk_stream_t stream, int dtype, void const *output_grad, void const *input,
+    void const *gelu_input, void *input_grad, void const *weight,
+    void *weight_grad, void *bias_grad, int64_t batch, int64_t in_dim,
+    int64_t out_dim, void *workspace, size_t workspace_bytes, int accumulate,
+    float rate, uint64_t seed, uint64_t offset);
+
 /* ------------------------------------------------------------------------ */
 /* Embedding -- Kernels::Embedding::gpu_forward_kernel / gpu_backward_kernel
  * (embedding_kernels_gpu.h:10-28; lib/kernels/src/cuda/embedding_kernels.cu:

@@ -270,3 +270,75 @@ def test_collected_column_reductions_equal_immediate_ones(ffk):
     # _end without _begin is a no-op
     ffk.check(ffk.lib().ffk_column_reductions_end(ffk.current_stream()))
 
+
+
+FUSED_TAIL_SHAPES = [  # (batch, in_dim, out_dim) of the forward Linear
+    (2048, 1024, 2048),  # 128x128 tiles, 256 of them (and 128 for the second Linear)
+    (1024, 192, 2048),   # 128x128 tiles, fewer k-tiles than pipeline stages
+    (3072, 256, 4096),   # 256x256 tiles in both directions
+    (4096, 4096, 1024),  # the second Linear on 256x256 tiles
+]
+
+
+@pytest.mark.parametrize("batch,in_dim,out_dim", FUSED_TAIL_SHAPES)
+def test_linear_with_gelu_and_dropout_on_the_tile_store_equals_separate_operators(ffk, batch, in_dim, out_dim):
+    """ffk_linear_gelu_dropout_forward and ffk_linear_backward_dropout_gelu give the bits of
+    Linear -> GELU -> Dropout and of Linear backward -> Dropout backward -> GELU backward."""
+    say("linear with GELU and dropout on the tile store %s" % ((batch, in_dim, out_dim),))
+    g = rng(batch + in_dim)
+    bt = torch.bfloat16
+    rate, seed, offset = 0.1, 987654321, 4096
+    x = to_dev(bf16_round(g.standard_normal((batch, in_dim)).astype(np.float32)), torch, bt)
+    w = to_dev(bf16_round(g.standard_normal((out_dim, in_dim)).astype(np.float32) / np.sqrt(in_dim)), torch, bt)
+    b = to_dev(bf16_round(g.standard_normal((out_dim,)).astype(np.float32)), torch, bt)
+    # forward
+    y_sep = torch.empty((batch, out_dim), dtype=bt, device="cuda")
+    ffk.linear_forward(x, w, b, ffk.ACT_NONE, y_sep)
+    act = ffk.element_unary_forward(ffk.OP["GELU"], y_sep)
+    dropped_sep = ffk.dropout_forward(act, rate, seed, offset)
+    y, dropped = ffk.linear_gelu_dropout_forward(x, w, b, rate, seed, offset)
+    assert torch.equal(y.view(torch.int16), y_sep.view(torch.int16))
+    assert torch.equal(dropped.view(torch.int16), dropped_sep.view(torch.int16))
+    assert 0.05 < float((dropped == 0).float().mean()) < 0.15
+    # the second Linear with its dropout and the residual addition: [batch, out_dim] -> [batch, in_dim]
+    w_down = to_dev(bf16_round(g.standard_normal((in_dim, out_dim)).astype(np.float32) * 0.05), torch, bt)
+    b_down = to_dev(bf16_round(g.standard_normal((in_dim,)).astype(np.float32)), torch, bt)
+    if batch * in_dim >= 128 * 128 * 128 and in_dim % 128 == 0:
+        y2 = torch.empty((batch, in_dim), dtype=bt, device="cuda")
+        ffk.linear_forward(dropped, w_down, b_down, ffk.ACT_NONE, y2)
+        want = ffk.dropout_add_forward(y2, x, rate, seed + 1, offset)
+        got = ffk.linear_dropout_add_forward(dropped, x, w_down, b_down, rate, seed + 1, offset)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # backward of the Linear that consumes `dropped`: [batch, out_dim] -> [batch, in_dim]
+    w2 = to_dev(bf16_round(g.standard_normal((in_dim, out_dim)).astype(np.float32) * 0.1), torch, bt)
+    dy2 = to_dev(bf16_round(g.standard_normal((batch, in_dim)).astype(np.float32)), torch, bt)
+    d_dropped = torch.empty_like(dropped)
+    dw_sep = torch.empty_like(w2)
+    db_sep = torch.empty((in_dim,), dtype=bt, device="cuda")
+    ffk.linear_backward(dy2, dy2, dropped, w2, dx=d_dropped, dw=dw_sep, db=db_sep, accumulate=0)
+    dx_sep = ffk.dropout_gelu_backward(d_dropped, y, rate, seed, offset)
+    dw = torch.empty_like(w2)
+    db = torch.empty_like(db_sep)
+    dx = ffk.linear_backward_dropout_gelu(dy2, dropped, y, w2, rate, seed, offset, dw=dw, db=db)
+    assert torch.equal(dx.view(torch.int16), dx_sep.view(torch.int16))
+    assert torch.equal(dw.view(torch.int16), dw_sep.view(torch.int16))
+    assert torch.equal(db.view(torch.int16), db_sep.view(torch.int16))
+
+
+def test_linear_with_fused_tail_refuses_shapes_without_a_kernel(ffk):
+    say("linear with fused tail: unsupported shapes")
+    bt = torch.bfloat16
+    x = torch.zeros((100, 64), dtype=bt, device="cuda")
+    w = torch.zeros((128, 64), dtype=bt, device="cuda")
+    b = torch.zeros((128,), dtype=bt, device="cuda")
+    with pytest.raises(ffk.FFKError, match="no fused kernel"):
+        ffk.linear_gelu_dropout_forward(x, w, b, 0.1, 1)
+    xf = torch.zeros((2048, 256), dtype=torch.float32, device="cuda")
+    wf = torch.zeros((2048, 256), dtype=torch.float32, device="cuda")
+    bf = torch.zeros((2048,), dtype=torch.float32, device="cuda")
+    with pytest.raises(ffk.FFKError, match="no fused kernel"):
+        ffk.linear_gelu_dropout_forward(xf, wf, bf, 0.1, 1)
+    with pytest.raises(ffk.FFKError, match="no fused kernel"):
+        ffk.linear_backward_dropout_gelu(x, torch.zeros((100, 128), dtype=bt, device="cuda"),
+                                         torch.zeros((100, 128), dtype=bt, device="cuda"),
+                                         torch.zeros((64, 128), dtype=bt, device="cuda"), 0.1, 1)
