@@ -404,6 +404,13 @@ ComputationGraphInstance create_computation_graph_instance(
   enum class Fused { NONE, GELU_DROPOUT_HEAD, GELU_DROPOUT_TAIL, DROPOUT_ADD_HEAD, DROPOUT_ADD_TAIL };
   std::vector<Fused> fused(L, Fused::NONE);
   std::vector<size_t> partner(L, 0);
+  // A Linear next to a fused pair takes the pair onto its GEMM's tile store (BF16 shapes the
+  // library has such a kernel for; for the others the Linear's invocation runs the two launches):
+  //   Linear -> (Dropout -> add):   linear_sum[linear] = the add, sum_linear[add] = the Linear;
+  //                                 the Linear's forward writes the add's output
+  //   (GELU -> Dropout) -> Linear:  linear_gelu[linear] = the GELU, gelu_linear[gelu] = the Linear;
+  //                                 the Linear's backward writes the gradient of the GELU's input
+  std::vector<int> linear_sum(L, -1), sum_linear(L, -1), linear_gelu(L, -1), gelu_linear(L, -1);
   {
     char const *off = std::getenv("FFK_LAYER_UNFUSED");
     bool const enabled = !(off != nullptr && off[0] == '1');
@@ -450,6 +457,35 @@ ComputationGraphInstance create_computation_graph_instance(
         if (other == out || !(shape_of(other) == shape_of(out))) continue;
         if (!aligned(layer.inputs[0]) || !aligned(other) || !aligned(add.outputs.at(0))) continue;
         fused[l] = Fused::DROPOUT_ADD_HEAD, fused[c] = Fused::DROPOUT_ADD_TAIL, partner[l] = c, partner[c] = l;
+      }
+    }
+    std::vector<int> producer(T, -1);  // the operator layer a tensor comes from (-1: an input or a weight)
+    for (size_t l = 0; l < L; l++) {
+      if (!is_op_layer(cg.layers[l])) continue;
+      for (tensor_guid_t t : cg.layers[l].outputs) producer[t.raw] = (int)l;
+    }
+    auto plain_bf16_linear = [&](int l) {
+      if (l < 0) return false;
+      auto const *a = std::get_if<LinearAttrs>(&cg.layers[l].attrs.op_attrs);
+      return a != nullptr && !a->activation.has_value() &&
+             shape_of(cg.layers[l].outputs.at(0)).data_type == DataType::BF16 && aligned(cg.layers[l].inputs[0]);
+    };
+    auto single_use = [&](tensor_guid_t t) { return uses[t.raw] == 1 && !(st->logit.has_value() && *st->logit == t); };
+    for (size_t l = 0; enabled && l < L; l++) {
+      if (fused[l] == Fused::DROPOUT_ADD_HEAD) {
+        ComputationGraph::Layer const &drop = cg.layers[l], &add = cg.layers[partner[l]];
+        int const lin = producer[drop.inputs[0].raw];
+        if (!plain_bf16_linear(lin) || !single_use(drop.inputs[0])) continue;
+        tensor_guid_t const other = add.inputs[0] == drop.outputs.at(0) ? add.inputs[1] : add.inputs[0];
+        if (producer[other.raw] >= lin) continue;  // the other operand must exist when the Linear runs
+        linear_sum[lin] = (int)partner[l], sum_linear[partner[l]] = lin;
+      } else if (fused[l] == Fused::GELU_DROPOUT_HEAD && plan[l].bwd.has_backward) {
+        tensor_guid_t const dropped = cg.layers[partner[l]].outputs.at(0);
+        if (!single_use(dropped)) continue;
+        int const lin = (int)consumer[dropped.raw];
+        if (!plain_bf16_linear(lin) || cg.layers[lin].inputs[0] != dropped) continue;
+        if (!plan[lin].bwd.has_backward || plan[lin].bwd.accumulate_input[0]) continue;
+        linear_gelu[lin] = (int)l, gelu_linear[l] = lin;
       }
     }
   }
@@ -612,6 +648,48 @@ ComputationGraphInstance create_computation_graph_instance(
                                       ws_bytes ? scratch : nullptr, ws_bytes, accumulate),
                   "Linear backward");
       };
+      if (linear_sum[l] >= 0) {
+        // residual + dropout(this Linear), written where the add's output lives
+        ComputationGraph::Layer const &add = cg.layers[linear_sum[l]];
+        size_t const d = partner[linear_sum[l]];
+        ComputationGraph::Layer const &drop = cg.layers[d];
+        DropoutAttrs const &da = std::get<DropoutAttrs>(drop.attrs.op_attrs);
+        float const rate = da.rate;
+        uint64_t const seed = da.seed + (uint64_t)d;
+        int64_t const n = numel(out);
+        void *residual = val(add.inputs[0] == drop.outputs.at(0) ? add.inputs[1] : add.inputs[0]);
+        void *sum = val(add.outputs.at(0));
+        f = [=](device_stream_t const &s) {
+          uint64_t const offset = S->iteration * (uint64_t)n;
+          int const rc = ffk_linear_dropout_add_forward(s.require_gpu(), type, xp, residual, sum, w, bias, batch, in_dim, out_dim,
+                                                        rate, seed, offset);
+          if (rc != FFK_ERR_UNSUPPORTED) return check_ffk(rc, "Linear + Dropout + add forward");
+          check_ffk(ffk_linear_forward(s.require_gpu(), type, act, xp, y, w, bias, batch, in_dim, out_dim), "Linear forward");
+          check_ffk(ffk_dropout_add_forward(s.require_gpu(), type, y, residual, sum, n, rate, seed, offset), "Dropout + add forward");
+        };
+      }
+      if (linear_gelu[l] >= 0) {
+        // the gradient of this Linear's input goes through the Dropout's and the GELU's backward on its way out
+        size_t const g = (size_t)linear_gelu[l], d = partner[g];
+        DropoutAttrs const &da = std::get<DropoutAttrs>(cg.layers[d].attrs.op_attrs);
+        float const rate = da.rate;
+        uint64_t const seed = da.seed + (uint64_t)d;
+        int64_t const n = numel(x);
+        void *gelu_in = val(cg.layers[g].inputs[0]), *gelu_in_grad = grd(cg.layers[g].inputs[0]);
+        int const acc_w = accumulate & ~FFK_ACC_INPUT;
+        b = [=](device_stream_t const &s) {
+          uint64_t const offset = S->iteration * (uint64_t)n;
+          int const rc = ffk_linear_backward_dropout_gelu(s.require_gpu(), type, dy, xp, gelu_in, gelu_in_grad, w, dw, dbias, batch,
+                                                          in_dim, out_dim, ws_bytes ? scratch : nullptr, ws_bytes, acc_w, rate, seed,
+                                                          offset);
+          if (rc != FFK_ERR_UNSUPPORTED) return check_ffk(rc, "Linear + Dropout + GELU backward");
+          check_ffk(ffk_linear_backward(s.require_gpu(), type, act, 0, y, dy, xp, dx, w, dw, dbias, batch, in_dim, out_dim,
+                                        ws_bytes ? scratch : nullptr, ws_bytes, accumulate),
+                    "Linear backward");
+          check_ffk(ffk_dropout_gelu_backward(s.require_gpu(), type, dx, gelu_in, gelu_in_grad, n, rate, seed, offset),
+                    "Dropout + GELU backward");
+        };
+      }
     } else if (auto const *a = std::get_if<LayerNormAttrs>(&oa)) {
       tensor_guid_t x = layer.inputs[0];
       int const type = dt(shape_of(x).data_type);
@@ -702,7 +780,9 @@ ComputationGraphInstance create_computation_graph_instance(
         uint64_t const seed = da.seed + (uint64_t)d;
         void *d_out = grd(cg.layers[d].outputs.at(0));
         f = [](device_stream_t const &) {};  // the Dropout computes dropout(GELU(x))
-        if (p.bwd.has_backward) {
+        if (gelu_linear[l] >= 0) {
+          b = [](device_stream_t const &) {};  // the Linear that reads the Dropout's output has written dx
+        } else if (p.bwd.has_backward) {
           b = [=](device_stream_t const &s) {
             check_ffk(ffk_dropout_gelu_backward(s.require_gpu(), type, d_out, xp, dx, n, rate, seed, S->iteration * (uint64_t)n),
                       "Dropout + GELU backward");
@@ -730,6 +810,7 @@ ComputationGraphInstance create_computation_graph_instance(
           check_ffk(ffk_dropout_add_forward(s.require_gpu(), type, dropped_in, residual, y, n, rate, seed, S->iteration * (uint64_t)n),
                     "Dropout + add forward");
         };
+        if (sum_linear[l] >= 0) f = [](device_stream_t const &) {};  // the Linear has written residual + dropout(Linear)
       }
       if (p.bwd.add_by_alias) {
         // operands whose gradient is dy's own memory need nothing; the others get grad += dy

@@ -972,7 +972,11 @@ static void gpu_tests() {
     // x -> dense -> GELU -> dropout -> dense -> dropout -> (+ x) -> cast -> loss; two instances of the
     // same graph, one created with FFK_LAYER_UNFUSED=1, stepped twice each (the second step uses
     // the next dropout offsets)
-    int64_t const B = 16, E = 64, FF = 128;
+    // ... at a size whose Linears run the two element-wise launches themselves, and at one where
+    // the library applies the pairs on the GEMMs' tile stores
+    for (int big = 0; big < 2; big++) {
+    int64_t const B = big ? 2048 : 16, E = big ? 1024 : 64, FF = big ? 2048 : 128;
+    float const init = big ? 0.05f : 0.3f;
     auto build = [&](ComputationGraphBuilder &cgb, tensor_guid_t &x, tensor_guid_t &logits, std::vector<tensor_guid_t> &ws) {
       x = cgb.create_input(shape({B, E}, DataType::BF16), CreateGrad::YES);
       tensor_guid_t h = cgb.dense(x, (int)FF, Activation::GELU, true);
@@ -1009,7 +1013,7 @@ static void gpu_tests() {
         if (weight) ws.push_back(g);
         TensorShape s16 = cgb.computation_graph.tensors[t].shape;
         auto host = random_vec(get_num_elements(s16.dims), seed++);
-        for (auto &v : host) v *= 0.3f;
+        for (auto &v : host) v *= init;
         auto f32 = device_accessor(gpu, TensorShape{s16.dims, DataType::FLOAT}, host);
         ok(ffk_cast_forward(nullptr, FFK_FLOAT, FFK_BF16, f32.ptr, inst.get_tensor_accessor(g).ptr, get_num_elements(s16.dims)));
       }
@@ -1023,6 +1027,7 @@ static void gpu_tests() {
     for (size_t i = 0; i < results[0].size(); i++) {
       CHECK(contains_non_zero(results[0][i]));
       CHECK(results[0][i] == results[1][i]);
+    }
     }
   });
 }
