@@ -24,8 +24,13 @@
 //    that produces the same bits: GELU -> Dropout (forward and backward) and
 //    Dropout -> element-wise add (forward).  The tensor between them must have
 //    no other consumer; it is then never written (get_tensor_accessor on it
-//    returns memory nobody filled).  FFK_LAYER_UNFUSED=1 in the environment at
-//    creation keeps one kernel per operator.
+//    returns memory nobody filled).  A BF16 Linear without activation whose
+//    output only feeds such a Dropout -> add pair writes the sum from its
+//    GEMM (its own output is never written); one whose input only comes from
+//    such a GELU -> Dropout pair writes the gradient of the GELU's input from
+//    its input-gradient GEMM (the gradient of its own input is never written).
+//    FFK_LAYER_UNFUSED=1 in the environment at creation keeps one kernel per
+//    operator.
 //  * the backward of an element-wise add copies nothing: an operand whose
 //    gradient has no other producer shares the output gradient's memory
 //    (get_gradient_accessor of both returns the same pointer), an operand that
