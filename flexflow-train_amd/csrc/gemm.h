@@ -54,6 +54,14 @@ size_t gemm_splitk_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K);
 // out[N] (+)= sum over the M rows of X[M,N] (ldx row stride); `partials` is
 // fp32 scratch of colsum_partials_elems(M, N) floats.
 int64_t colsum_partials_elems(int64_t M, int64_t N);
+// dx[M,N] = dropout_backward(dy) and colsum (+)= its column sums (the bias
+// gradient of the Linear whose output the dropout follows), one pass over dy.
+// The sums are taken over dx as stored, in the order colsum_dispatch uses, so
+// they are the bits of the two separate kernels.  FFK_ERR_UNSUPPORTED (nothing
+// launched, no message) when the shape has no vector kernel.
+int dropout_backward_colsum(hipStream_t stream, int dtype, void const *dy, void *dx, int64_t M,
+                            int64_t N, void *colsum, bool accumulate, float *partials,
+                            DropoutParams const &drop);
 int colsum_dispatch(hipStream_t stream, int dtype, void const *X, int64_t ldx,
                     int64_t M, int64_t N, void *out, bool accumulate,
                     float *partials);

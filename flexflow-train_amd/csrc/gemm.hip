@@ -1093,10 +1093,13 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(
 constexpr int kColsumRowsPerLane = 8;
 constexpr int kColsumRowsPerBlock = 4 * kColsumRowsPerLane;
 
-template <typename T>
+// DROP: X is the gradient of a dropout's output; what is summed is the
+// dropout's backward of it, rounded as stored, which is also written to G
+// (dense, ldx == N: a lane's V elements are a Philox block or half of one).
+template <typename T, bool DROP>
 __global__ __launch_bounds__(256) void colsum_partial_vec_kernel(
     T const *__restrict__ X, int64_t ldx, int M, int N, int rows_per_split,
-    float *__restrict__ partials) {
+    float *__restrict__ partials, T *__restrict__ G, DropoutParams drop) {
   constexpr int V = VecIO<T>::kVec;
   __shared__ float red[4][64][V + 1];
   int const cx = threadIdx.x & 63;
@@ -1118,6 +1121,18 @@ __global__ __launch_bounds__(256) void colsum_partial_vec_kernel(
 #pragma unroll
       for (int i = 0; i < kColsumRowsPerLane; i++) {
         if (m0 + i < r1) {
+          if constexpr (DROP) {
+            uint64_t const e0 = drop.offset + (uint64_t)(m0 + i) * (uint64_t)N + (uint64_t)n;
+            uint32_t w[4];
+            philox4x32_10(e0 >> 3, drop.key, w);
+            if (V == 4 && (e0 & 4)) {  // upper half of the block
+              w[0] = w[2];
+              w[1] = w[3];
+            }
+#pragma unroll
+            for (int e = 0; e < V; e++) v[i][e] = storage_round<T>(keep(w, e, drop) ? v[i][e] * drop.scale : 0.0f);
+            VecIO<T>::store(G + (int64_t)(m0 + i) * ldx + n, v[i]);
+          }
 #pragma unroll
           for (int e = 0; e < V; e++) s[e] += v[i][e];
         }
@@ -1145,19 +1160,37 @@ int64_t colsum_partials_elems(int64_t M, int64_t N) {
   return (int64_t)colsum_splits(M) * N;
 }
 
+// dropped != nullptr: the sums are taken over dropout_backward(X), which is
+// written to dropped; vector shapes only (FFK_ERR_UNSUPPORTED otherwise, before
+// any launch).
 template <typename T>
 static int colsum_typed(hipStream_t st, T const *X, int64_t ldx, int64_t M,
-                        int64_t N, T *out, bool accumulate, float *partials) {
+                        int64_t N, T *out, bool accumulate, float *partials,
+                        T *dropped = nullptr, DropoutParams const *drop = nullptr) {
   constexpr int V = VecIO<T>::kVec;
   int const splits = colsum_splits(M);
   int rows_per_split = (int)ceil_div(M, splits);
   bool const vec = (N % V == 0) && (ldx % V == 0) && aligned16(X);
+  if (dropped != nullptr) {
+    if (!vec || ldx != N || !aligned16(dropped) || (drop->offset & 7) != 0 || M >= (1ll << 31) || N >= (1ll << 31)) {
+      return FFK_ERR_UNSUPPORTED;
+    }
+    rows_per_split = (int)(ceil_div(rows_per_split, kColsumRowsPerBlock) * kColsumRowsPerBlock);
+    int const used = (int)ceil_div(M, rows_per_split);
+    dim3 grid((unsigned)ceil_div(N, 64 * V), (unsigned)used);
+    colsum_partial_vec_kernel<T, true><<<grid, 256, 0, st>>>(X, ldx, (int)M, (int)N, rows_per_split, partials,
+                                                            dropped, *drop);
+    FFK_CHECK_LAUNCH();
+    FFK_HIP(colreduce_launch<T>(st, partials, used, (int)N, (int)N, out, nullptr, accumulate));
+    return FFK_OK;
+  }
   if (vec) {
     // whole row blocks per split so that only the last split has a ragged end
     rows_per_split = (int)(ceil_div(rows_per_split, kColsumRowsPerBlock) * kColsumRowsPerBlock);
     int const used = (int)ceil_div(M, rows_per_split);
     dim3 grid((unsigned)ceil_div(N, 64 * V), (unsigned)used);
-    colsum_partial_vec_kernel<T><<<grid, 256, 0, st>>>(X, ldx, (int)M, (int)N, rows_per_split, partials);
+    colsum_partial_vec_kernel<T, false><<<grid, 256, 0, st>>>(X, ldx, (int)M, (int)N, rows_per_split, partials,
+                                                             nullptr, DropoutParams{});
     FFK_CHECK_LAUNCH();
     FFK_HIP(colreduce_launch<T>(st, partials, used, (int)N, (int)N, out, nullptr, accumulate));
     return FFK_OK;
@@ -1182,6 +1215,21 @@ int colsum_dispatch(hipStream_t st, int dtype, void const *X, int64_t ldx,
                               static_cast<bf16 *>(out), accumulate, partials);
   }
   return fail(FFK_ERR_UNSUPPORTED, "colsum: dtype %d not supported", dtype);
+}
+
+int dropout_backward_colsum(hipStream_t st, int dtype, void const *dy, void *dx, int64_t M, int64_t N,
+                            void *colsum, bool accumulate, float *partials, DropoutParams const &drop) {
+  FFK_REQUIRE(dy && dx && colsum && partials, "dropout_backward_colsum: NULL operand");
+  FFK_REQUIRE(M > 0 && N > 0, "dropout_backward_colsum: non-positive dimension");
+  if (dtype == FFK_FLOAT) {
+    return colsum_typed<float>(st, static_cast<float const *>(dy), N, M, N, static_cast<float *>(colsum),
+                               accumulate, partials, static_cast<float *>(dx), &drop);
+  }
+  if (dtype == FFK_BF16) {
+    return colsum_typed<bf16>(st, static_cast<bf16 const *>(dy), N, M, N, static_cast<bf16 *>(colsum),
+                              accumulate, partials, static_cast<bf16 *>(dx), &drop);
+  }
+  return FFK_ERR_UNSUPPORTED;
 }
 
 bool gemm_tail_supported(int dtype, bool ta, bool tb, int64_t M, int64_t N, int64_t K,
