@@ -47,6 +47,27 @@ int gemm_dispatch(hipStream_t stream, int dtype, bool trans_a, bool trans_b,
                   void const *B, int64_t ldb, void *C, int64_t ldc,
                   GemmEpilogue const &ep);
 
+// Two GEMMs of the same kind (same transposes, same reduction length K, no
+// bias or activation, same accumulate switch) in ONE launch: for two outputs
+// that each leave part of the chip idle (the two weight gradients of an
+// attention block).  Each problem's result is the bits of gemm_dispatch on it
+// alone with the 128x128 tile.  gemm_pair_supported says whether the pair
+// runs (BF16, outputs multiples of 128, K a multiple of 64, 16-byte aligned
+// operands); gemm_dispatch_pair fails otherwise.
+struct GemmProblem {
+  int64_t M, N;
+  void const *A;
+  int64_t lda;
+  void const *B;
+  int64_t ldb;
+  void *C;
+  int64_t ldc;
+};
+bool gemm_pair_supported(int dtype, bool trans_a, bool trans_b, int64_t K, GemmProblem const &p0,
+                         GemmProblem const &p1);
+int gemm_dispatch_pair(hipStream_t stream, int dtype, bool trans_a, bool trans_b, int64_t K,
+                       GemmProblem const &p0, GemmProblem const &p1, bool accumulate);
+
 // Scratch bytes with which a bf16 GEMM of this shape would split its reduction
 // (0: it would not).
 size_t gemm_splitk_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K);

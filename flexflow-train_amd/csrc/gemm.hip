@@ -360,14 +360,35 @@ struct GemmTailArgs {
   DropoutParams dropout;
 };
 
+// A second GEMM of the same kind and reduction length run by the same launch:
+// workgroups from first_tiles on compute it.
+struct GemmSecondProblem {
+  bf16 const *A, *B;
+  bf16 *C;
+  int M, N;
+  int64_t lda, ldb, ldc;
+  int first_tiles;  // number of tiles (= workgroups) of the first problem
+};
+
 // TAIL (GemmEpilogue::Tail): element-wise operators applied to the 8-element
 // pieces of the output tile on their way from LDS to memory.
-template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, bool TB, int TAIL = 0>
+// PAIR: the launch carries two problems (no bias, no split-K).
+template <int BM, int BN, int WM, int WN, int BK, int STAGES, int PF, bool TA, bool TB, int TAIL = 0,
+          bool PAIR = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_kernel(
     bf16 const *__restrict__ A, bf16 const *__restrict__ B, bf16 *C, int M,
     int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
     bf16 const *__restrict__ bias, int act, int accumulate,
-    float *__restrict__ partial, int k_tiles_per_split, GemmTailArgs tail) {
+    float *__restrict__ partial, int k_tiles_per_split, GemmTailArgs tail, GemmSecondProblem second) {
+  int bid = blockIdx.x;
+  if constexpr (PAIR) {
+    if (bid >= second.first_tiles) {  // uniform over the workgroup
+      bid -= second.first_tiles;
+      A = second.A, B = second.B, C = second.C;
+      M = second.M, N = second.N;
+      lda = second.lda, ldb = second.ldb, ldc = second.ldc;
+    }
+  }
   // partial != nullptr: split-K.  Workgroup (tile, split) reduces k-tiles
   // [split * k_tiles_per_split, +k_tiles_per_split) and stores its fp32
   // accumulators to partial[split][M][N]; a second kernel sums the splits and
@@ -393,8 +414,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   int const wn0 = (wave % (BN / WN)) * WN;
   int tm, tn;
   int const tiles = (M / BM) * (N / BN);
-  int const split = partial != nullptr ? blockIdx.x / tiles : 0;
-  tile_coords(partial != nullptr ? blockIdx.x % tiles : blockIdx.x, M / BM, N / BN, tm, tn);
+  int const split = partial != nullptr ? bid / tiles : 0;
+  tile_coords(partial != nullptr ? bid % tiles : bid, M / BM, N / BN, tm, tn);
   int const m0 = tm * BM, n0 = tn * BN;
   int const kt0 = split * k_tiles_per_split;  // first k-tile of this workgroup
 
@@ -807,7 +828,8 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
   if (splits > 1) {
     float *partial = static_cast<float *>(ep.splitk_ws);
     kern<<<blocks * splits, NT, Cfg::kLds, st>>>(A, B, C, M, N, K, lda, ldb, ldc, nullptr,
-                                                FFK_ACT_NONE, 0, partial, K / BK / splits, tail);
+                                                FFK_ACT_NONE, 0, partial, K / BK / splits, tail,
+                                                GemmSecondProblem{});
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     int64_t const quads = (int64_t)M * N / 4;
@@ -818,7 +840,30 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
   }
   kern<<<blocks, NT, Cfg::kLds, st>>>(A, B, C, M, N, K, lda, ldb, ldc,
                                      static_cast<bf16 const *>(ep.bias), ep.activation,
-                                     ep.accumulate, nullptr, 0, tail);
+                                     ep.accumulate, nullptr, 0, tail, GemmSecondProblem{});
+  return hipGetLastError();
+}
+
+// Two GEMMs of the same kind and reduction length on 128x128 tiles in one launch.
+template <bool TA, bool TB>
+static hipError_t launch_pipe_pair(hipStream_t st, GemmProblem const &p0, GemmProblem const &p1, int K,
+                                   bool accumulate) {
+  using Cfg = PipeCfg<128, 128, 64, 32, 64, 4>;
+  constexpr int NT = Cfg::NW * 64;
+  auto kern = gemm_bf16_pipe_kernel<128, 128, 64, 32, 64, 4, 1, TA, TB, 0, true>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg::kLds);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  int const t0 = (int)((p0.M / 128) * (p0.N / 128)), t1 = (int)((p1.M / 128) * (p1.N / 128));
+  GemmSecondProblem const second = {static_cast<bf16 const *>(p1.A), static_cast<bf16 const *>(p1.B),
+                                    static_cast<bf16 *>(p1.C), (int)p1.M, (int)p1.N, p1.lda, p1.ldb, p1.ldc, t0};
+  kern<<<t0 + t1, NT, Cfg::kLds, st>>>(static_cast<bf16 const *>(p0.A), static_cast<bf16 const *>(p0.B),
+                                       static_cast<bf16 *>(p0.C), (int)p0.M, (int)p0.N, K, p0.lda, p0.ldb, p0.ldc,
+                                       nullptr, FFK_ACT_NONE, accumulate ? 1 : 0, nullptr, 0, GemmTailArgs{}, second);
   return hipGetLastError();
 }
 
@@ -1230,6 +1275,37 @@ int dropout_backward_colsum(hipStream_t st, int dtype, void const *dy, void *dx,
                               accumulate, partials, static_cast<bf16 *>(dx), &drop);
   }
   return FFK_ERR_UNSUPPORTED;
+}
+
+static bool pair_member_ok(bool ta, bool tb, GemmProblem const &p, int64_t K) {
+  if (p.M <= 0 || p.N <= 0 || p.M % 128 != 0 || p.N % 128 != 0 || !p.A || !p.B || !p.C) return false;
+  if (p.M >= (1ll << 31) || p.N >= (1ll << 31)) return false;
+  if (p.lda < (ta ? p.M : K) || p.ldb < (tb ? K : p.N) || p.ldc < p.N) return false;
+  bool const vec_ok = (p.lda % 8 == 0) && (p.ldb % 8 == 0) && aligned16(p.A) && aligned16(p.B);
+  GemmEpilogue none;
+  return vec_ok && pipe_tile_for(static_cast<bf16 const *>(p.C), (int)p.M, (int)p.N, (int)K, p.lda, p.ldb, p.ldc, none,
+                                 128) == 128;
+}
+
+bool gemm_pair_supported(int dtype, bool ta, bool tb, int64_t K, GemmProblem const &p0, GemmProblem const &p1) {
+  if (dtype != FFK_BF16 || K <= 0 || K % 64 != 0 || K >= (1ll << 31) || gemm_variant_override() != 0) return false;
+  if (!pair_member_ok(ta, tb, p0, K) || !pair_member_ok(ta, tb, p1, K)) return false;
+  // worth it when neither problem fills the chip on its own and the two together come closer
+  int64_t const t0 = (p0.M / 128) * (p0.N / 128), t1 = (p1.M / 128) * (p1.N / 128);
+  return t0 < 2 * kNumCU && t1 < 2 * kNumCU && t0 + t1 >= kNumCU / 2;
+}
+
+int gemm_dispatch_pair(hipStream_t st, int dtype, bool ta, bool tb, int64_t K, GemmProblem const &p0,
+                       GemmProblem const &p1, bool accumulate) {
+  FFK_REQUIRE(gemm_pair_supported(dtype, ta, tb, K, p0, p1),
+              "gemm: these two problems do not run as one launch (ask gemm_pair_supported first)");
+  hipError_t e;
+  if (!ta && !tb) e = launch_pipe_pair<false, false>(st, p0, p1, (int)K, accumulate);
+  else if (!ta && tb) e = launch_pipe_pair<false, true>(st, p0, p1, (int)K, accumulate);
+  else if (ta && !tb) e = launch_pipe_pair<true, false>(st, p0, p1, (int)K, accumulate);
+  else e = launch_pipe_pair<true, true>(st, p0, p1, (int)K, accumulate);
+  FFK_HIP(e);
+  return FFK_OK;
 }
 
 bool gemm_tail_supported(int dtype, bool ta, bool tb, int64_t M, int64_t N, int64_t K,

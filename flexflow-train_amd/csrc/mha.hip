@@ -186,7 +186,17 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
   rc = gemm_dispatch(st, dtype, false, false, L.TQ, HD, d->o_proj_size, output_grad,
                      d->o_proj_size, w + L.wo * es, HD, dctx, HD, over);
   if (rc != FFK_OK) return rc;
-  if (dw != nullptr) {
+  // The two weight gradients of a self-attention block (output projection and
+  // folded Q/K/V projection) have the same reduction length and each leaves
+  // part of the chip idle: where the library can, they run as ONE launch after
+  // the core's backward.
+  bool const folded = fused && key_grad == nullptr && value_grad == nullptr;
+  GemmProblem const wo_grad = {d->o_proj_size, HD, output_grad, d->o_proj_size, ctx, HD,
+                               dw != nullptr ? dw + L.wo * es : nullptr, HD};
+  GemmProblem const wqkv_grad = {3 * HD, d->q_size, dqkv, 3 * HD, query, d->q_size,
+                                 dw != nullptr ? dw + L.wq * es : nullptr, d->q_size};
+  bool const paired = dw != nullptr && folded && gemm_pair_supported(dtype, true, false, L.TQ, wqkv_grad, wo_grad);
+  if (dw != nullptr && !paired) {
     // d(QKV projections) is not written before the core's backward: until
     // then it serves as split-K scratch for this small-output, long-K GEMM.
     GemmEpilogue acc_o = acc;
@@ -216,13 +226,15 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
                               reinterpret_cast<float *>(rs + L.off_delta), dqp, dkp, dvp);
   if (rc != FFK_OK) return rc;
 
-  bool const folded = fused && key_grad == nullptr && value_grad == nullptr;
   if (folded) {
     // dX (+)= dQKV[T,3HD] . [W_Q; W_K; W_V]  and  dW_QKV += dQKV^T . X
     if (query_grad != nullptr) {
       rc = gemm_dispatch(st, dtype, false, false, L.TQ, d->q_size, 3 * HD, dqkv, 3 * HD,
                          w + L.wq * es, d->q_size, query_grad, d->q_size, in_ep);
       if (rc != FFK_OK) return rc;
+    }
+    if (paired) {
+      return gemm_dispatch_pair(st, dtype, true, false, L.TQ, wqkv_grad, wo_grad, acc.accumulate);
     }
     if (dw != nullptr) {
       rc = gemm_dispatch(st, dtype, true, false, 3 * HD, d->q_size, L.TQ, dqkv, 3 * HD, query,

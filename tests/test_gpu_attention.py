@@ -155,6 +155,7 @@ MHA_CASES = [  # B, Sq, Skv, H, E(q), Ek, Ev, Dh, oProj, self-attention?
     (2, 33, 33, 2, 128, 128, 128, 64, 96, True),
     (1, 24, 40, 2, 64, 72, 80, 64, 64, False),
     (2, 64, 64, 2, 256, 256, 256, 128, 256, True),
+    (2, 64, 64, 12, 768, 768, 768, 64, 768, True),  # both weight gradients in one two-problem GEMM launch
 ]
 
 
