@@ -79,7 +79,7 @@ def step(ffk, st):
 # FETCH_SIZE` and `--pmc WRITE_SIZE` runs of `bench.py --roofline-only`, each
 # counter scaled by what it reads for the 256 MiB copy kernel that the same run
 # launches (profiles/ffn_up_gemm_hbm_traffic.md holds the runs and the factors).
-DOMINANT_KERNEL_TRAFFIC_BYTES = 84145447  # 48.2 MiB fetched + 32 MiB written; 48 MiB algorithmic
+DOMINANT_KERNEL_TRAFFIC_BYTES = 84137256  # 48.2 MiB fetched + 32 MiB written; 48 MiB algorithmic
 
 
 def time_dominant_kernel(ffk, torch, cfg, iters=50, calibration_copy=False):
@@ -119,7 +119,7 @@ def time_dominant_kernel(ffk, torch, cfg, iters=50, calibration_copy=False):
     return dict(bound="mfma", achieved=flops / sec / 1e12, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
                 frac=flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                 traffic=DOMINANT_KERNEL_TRAFFIC_BYTES,
-                kernel="gemm_bf16_pipe_kernel<256,256,128,64,32,4,1,false,true,0> "
+                kernel="gemm_bf16_pipe_kernel<256,256,128,64,32,4,1,false,true,0,false> "
                        "(FFN up-projection, M%d N%d K%d, bias)" % (T, F, E),
                 us_per_launch=sec * 1e6)
 
