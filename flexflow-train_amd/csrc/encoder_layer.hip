@@ -259,12 +259,23 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
     }
   }
   int g_f1_rc = FFK_ERR_UNSUPPORTED;
+  bool b1_done = false;  // the first Linear's bias gradient already computed
   if (gelu && layer_fusion_enabled()) {
     // the dropout's and GELU's backward ride on the tile store of the input-gradient GEMM
     // (52.7 us against 37.7 + 18.4 us: the separate kernel moves three tensors, this one adds one read)
-    g_f1_rc = linear_backward_dropout_gelu(as_stream(st), dtype, ws + L.g_f2, ws + L.act1_drop, ws + L.f1,
-                                           ws + L.g_f1, w->w2, g->w2, b2_grad, T, F, E, ws + L.lin_ws,
-                                           lin_ws_bytes, wacc, p, d->seed + 1, 0);
+    // ... and so do the column sums of what it stores, the first Linear's bias gradient
+    if (g->b1 != nullptr) {
+      g_f1_rc = linear_backward_dropout_gelu(as_stream(st), dtype, ws + L.g_f2, ws + L.act1_drop, ws + L.f1,
+                                             ws + L.g_f1, w->w2, g->w2, b2_grad, T, F, E, ws + L.lin_ws,
+                                             lin_ws_bytes, wacc, p, d->seed + 1, 0, g->b1,
+                                             reinterpret_cast<float *>(ws + L.lin_ws_b), (wacc & FFK_ACC_BIAS) != 0);
+      b1_done = g_f1_rc == FFK_OK;
+    }
+    if (g_f1_rc == FFK_ERR_UNSUPPORTED) {
+      g_f1_rc = linear_backward_dropout_gelu(as_stream(st), dtype, ws + L.g_f2, ws + L.act1_drop, ws + L.f1,
+                                             ws + L.g_f1, w->w2, g->w2, b2_grad, T, F, E, ws + L.lin_ws,
+                                             lin_ws_bytes, wacc, p, d->seed + 1, 0);
+    }
     if (g_f1_rc != FFK_OK && g_f1_rc != FFK_ERR_UNSUPPORTED) return g_f1_rc;
   }
   bool const g_f1_ready = g_f1_rc == FFK_OK;
@@ -289,7 +300,7 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
                                          ws + L.g_f1, T * F, 0));
     }
     FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_NONE, 0, ws + L.f1, ws + L.g_f1, ffn_in, ws + L.g_h2,
-                                w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws_b, lin_ws_bytes, wacc));
+                                w->w1, g->w1, b1_done ? nullptr : g->b1, T, E, F, ws + L.lin_ws_b, lin_ws_bytes, wacc));
   } else {
     FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_RELU, 0, ws + L.act1, ws + L.g_act1, ffn_in, ws + L.g_h2,
                                 w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws_b, lin_ws_bytes, wacc));

@@ -52,7 +52,14 @@ int linear_backward_dropout_gelu(hipStream_t st, int dtype, void const *output_g
                                  void const *gelu_input, void *input_grad, void const *weight,
                                  void *weight_grad, void *bias_grad, int64_t batch, int64_t in_dim,
                                  int64_t out_dim, void *workspace, size_t workspace_bytes,
-                                 int accumulate, float rate, uint64_t seed, uint64_t offset);
+                                 int accumulate, float rate, uint64_t seed, uint64_t offset,
+                                 // optional: input_grad_colsum [in_dim] (+)= column sums of input_grad as
+                                 // stored (the bias gradient of the Linear in front of the GELU), the bits
+                                 // of the separate column-sum kernel; colsum_partials: fp32 scratch of
+                                 // colsum_partials_elems(batch, in_dim) that nothing else uses until the
+                                 // sums are complete
+                                 void *input_grad_colsum = nullptr, float *colsum_partials = nullptr,
+                                 bool colsum_accumulate = false);
 
 // summed = residual + dropout(in); y = LayerNorm(summed), statistics kept as the separate
 // LayerNorm would.  Returns FFK_ERR_UNSUPPORTED (without setting an error

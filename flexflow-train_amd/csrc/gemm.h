@@ -30,7 +30,14 @@ struct GemmEpilogue {
   void const *tail_in = nullptr;
   void *tail_out = nullptr;
   DropoutParams tail_dropout = {};
+  // kTailDropoutGeluGrad, optional: the GEMM also leaves the partial column
+  // sums of what it stores (colsum_partials_elems(M, N) floats, the partials
+  // colsum_dispatch would compute from the stored tensor); colsum_finish adds
+  // them up into the column sums (+)= out.
+  float *tail_colsum_partials = nullptr;
 };
+int colsum_finish(hipStream_t stream, int dtype, float const *partials, int64_t M, int64_t N, void *out,
+                  bool accumulate);
 
 // Whether gemm_dispatch can run this GEMM with ep.tail (it fails otherwise).
 bool gemm_tail_supported(int dtype, bool trans_a, bool trans_b, int64_t M, int64_t N,

@@ -354,10 +354,17 @@ __device__ __forceinline__ unsigned lds_address_of(void *p) {
 // PF = how many k-steps ahead of its use a fragment is read from LDS (PF + 1
 // register buffers).  PF = 1 is what both tile configurations use; PF = 3 was
 // measured on the 128x128 tile (2 MFMAs per k-step per wave) and gained nothing.
+// Column sums add up blocks of 32 rows as four runs of 8 (colsum_partial_vec_kernel below).
+constexpr int kColsumRowsPerLane = 8;
+constexpr int kColsumRowsPerBlock = 4 * kColsumRowsPerLane;
+
 struct GemmTailArgs {
   bf16 const *in;
   bf16 *out;
   DropoutParams dropout;
+  // kTailDropoutGeluGrad only, optional: [M / 32][N] sums of 32-row blocks of
+  // what the tail stores, added up in colsum_partial_vec_kernel's order
+  float *colsum_partials;
 };
 
 // A second GEMM of the same kind and reduction length run by the same launch:
@@ -734,6 +741,34 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
         }
         bf16 *const to = TAIL == GemmEpilogue::kTailGeluDropout ? tail.out : dst;
         *reinterpret_cast<u32x4 *>(to + at) = r;
+        if constexpr (TAIL == GemmEpilogue::kTailDropoutGeluGrad) {
+          // kept for the column sums below (the lane's own piece: no other lane reads it before the barrier)
+          if (tail.colsum_partials != nullptr) *reinterpret_cast<u32x4 *>(cs + row * CS + ch * 8) = r;
+        }
+      }
+    }
+    if constexpr (TAIL == GemmEpilogue::kTailDropoutGeluGrad) {
+      if (tail.colsum_partials != nullptr) {  // uniform over the launch
+        __syncthreads();
+        // A lane owns a column of the wave's tile; per block of 32 rows: four
+        // runs of 8 rows summed in row order, then (0 + 1) + (2 + 3).
+        for (int col = lane; col < WN; col += 64) {
+#pragma unroll
+          for (int blk = 0; blk < WM / kColsumRowsPerBlock; blk++) {
+            float run[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              float acc_rows = 0.0f;
+#pragma unroll
+              for (int r = 0; r < kColsumRowsPerLane; r++) {
+                acc_rows += VecIO<bf16>::load1(cs + (blk * kColsumRowsPerBlock + q * kColsumRowsPerLane + r) * CS + col);
+              }
+              run[q] = acc_rows;
+            }
+            int64_t const part = (m0 + wm0) / kColsumRowsPerBlock + blk;
+            tail.colsum_partials[part * N + n0 + wn0 + col] = (run[0] + run[1]) + (run[2] + run[3]);
+          }
+        }
       }
     }
   };
@@ -816,7 +851,7 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
   constexpr int NT = Cfg::NW * 64;
   auto kern = gemm_bf16_pipe_kernel<BM, BN, WM, WN, BK, STAGES, PF, TA, TB, TAIL>;
   GemmTailArgs const tail = {static_cast<bf16 const *>(ep.tail_in), static_cast<bf16 *>(ep.tail_out),
-                             ep.tail_dropout};
+                             ep.tail_dropout, ep.tail_colsum_partials};
   static bool configured = false;  // per template instance
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const *>(kern),
@@ -1135,8 +1170,6 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(
 // Vectorised first pass: a thread reads 16 bytes (8 bf16 / 4 fp32 columns) of
 // kColsumRowsPerLane rows, all loads independent; 64 threads span the columns,
 // the 4 row lanes of the workgroup meet in LDS.
-constexpr int kColsumRowsPerLane = 8;
-constexpr int kColsumRowsPerBlock = 4 * kColsumRowsPerLane;
 
 // DROP: X is the gradient of a dropout's output; what is summed is the
 // dropout's backward of it, rounded as stored, which is also written to G
@@ -1199,6 +1232,21 @@ __global__ __launch_bounds__(256) void colsum_partial_vec_kernel(
 static int colsum_splits(int64_t M) {
   int64_t s = ceil_div(M, kColsumRowsPerBlock);
   return (int)(s < 1 ? 1 : (s > 256 ? 256 : s));
+}
+
+// Rows that one partial sum of the vector column-sum kernel covers.
+static int64_t colsum_rows_per_split(int64_t M) {
+  int64_t const rows = ceil_div(M, (int64_t)colsum_splits(M));
+  return ceil_div(rows, (int64_t)kColsumRowsPerBlock) * kColsumRowsPerBlock;
+}
+
+int colsum_finish(hipStream_t st, int dtype, float const *partials, int64_t M, int64_t N, void *out,
+                  bool accumulate) {
+  FFK_REQUIRE(dtype == FFK_BF16 && M % kColsumRowsPerBlock == 0 && colsum_rows_per_split(M) == kColsumRowsPerBlock,
+              "colsum_finish: partials of this shape do not come from a GEMM tail");
+  FFK_HIP(colreduce_launch<bf16>(st, partials, (int)(M / kColsumRowsPerBlock), (int)N, (int)N,
+                                 static_cast<bf16 *>(out), nullptr, accumulate));
+  return FFK_OK;
 }
 
 int64_t colsum_partials_elems(int64_t M, int64_t N) {
@@ -1318,6 +1366,7 @@ bool gemm_tail_supported(int dtype, bool ta, bool tb, int64_t M, int64_t N, int6
     if (!tb || ep.tail_out == nullptr || !aligned16(ep.tail_out)) return false;
   } else if (ep.tail == GemmEpilogue::kTailDropoutGeluGrad) {
     if (tb || ep.tail_in == nullptr || !aligned16(ep.tail_in)) return false;
+    if (ep.tail_colsum_partials != nullptr && colsum_rows_per_split(M) != kColsumRowsPerBlock) return false;
   } else if (ep.tail == GemmEpilogue::kTailDropoutAdd) {
     if (!tb || ep.tail_in == nullptr || !aligned16(ep.tail_in)) return false;
   } else {

@@ -217,19 +217,25 @@ int linear_backward_dropout_gelu(hipStream_t st, int dtype, void const *output_g
                                  void const *gelu_input, void *input_grad, void const *weight,
                                  void *weight_grad, void *bias_grad, int64_t batch, int64_t in_dim,
                                  int64_t out_dim, void *workspace, size_t workspace_bytes,
-                                 int accumulate, float rate, uint64_t seed, uint64_t offset) {
+                                 int accumulate, float rate, uint64_t seed, uint64_t offset,
+                                 void *input_grad_colsum, float *colsum_partials, bool colsum_accumulate) {
   FFK_REQUIRE(output_grad && input && gelu_input && input_grad && weight,
               "linear_backward_dropout_gelu: NULL tensor");
+  FFK_REQUIRE(input_grad_colsum == nullptr || colsum_partials != nullptr,
+              "linear_backward_dropout_gelu: column sums need scratch for their partial sums");
   FFK_REQUIRE((accumulate & FFK_ACC_INPUT) == 0,
               "linear_backward_dropout_gelu: the input gradient is stored, not added");
   GemmEpilogue tail;
   tail.tail = GemmEpilogue::kTailDropoutGeluGrad;
   tail.tail_in = gelu_input;
+  tail.tail_colsum_partials = input_grad_colsum != nullptr ? colsum_partials : nullptr;
   int const prc = make_dropout_params("linear_backward_dropout_gelu", rate, seed, offset, tail.tail_dropout);
   if (prc != FFK_OK) return prc;
-  return linear_backward_impl(st, dtype, FFK_ACT_NONE, 0, nullptr, output_grad, input, input_grad, weight,
-                              weight_grad, bias_grad, batch, in_dim, out_dim, workspace, workspace_bytes,
-                              accumulate, &tail);
+  int const rc = linear_backward_impl(st, dtype, FFK_ACT_NONE, 0, nullptr, output_grad, input, input_grad, weight,
+                                      weight_grad, bias_grad, batch, in_dim, out_dim, workspace, workspace_bytes,
+                                      accumulate, &tail);
+  if (rc != FFK_OK || input_grad_colsum == nullptr) return rc;
+  return colsum_finish(st, dtype, colsum_partials, batch, in_dim, input_grad_colsum, colsum_accumulate);
 }
 
 }  // namespace ffk
@@ -270,7 +276,7 @@ extern "C" int ffk_linear_backward_dropout_gelu(
   int const rc = ffk::linear_backward_dropout_gelu(as_stream(stream), dtype, output_grad, input, gelu_input,
                                                    input_grad, weight, weight_grad, bias_grad, batch,
                                                    in_dim, out_dim, workspace, workspace_bytes,
-                                                   accumulate, rate, seed, offset);
+                                                   accumulate, rate, seed, offset, nullptr, nullptr, false);
   if (rc == FFK_ERR_UNSUPPORTED) {
     return fail(FFK_ERR_UNSUPPORTED, "linear_backward_dropout_gelu: no fused kernel for this shape; "
                                      "run Linear backward, Dropout backward and GELU backward one after the other");
