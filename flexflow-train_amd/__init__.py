@@ -112,6 +112,8 @@ SIGNATURES = {
     "ffk_layer_norm_backward_workspace_bytes": (c_sz, [c_i64, c_i64]),
     "ffk_layer_norm_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
                                         c_i64, c_i64, c_p, c_sz, c_int]),
+    "ffk_layer_norm_backward_static": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
+                                               c_p, c_i64, c_i64, c_int]),
     "ffk_softmax_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_i64, c_i64]),
     "ffk_softmax_backward_copy": (c_int, [c_p, c_int, c_p, c_p, c_sz]),
     "ffk_softmax_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_i64, c_i64]),
@@ -356,6 +358,15 @@ def layer_norm_backward(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, accumulate=
                                         ptr(mean), ptr(rstd), ptr(gamma), ptr(dx), ptr(dgamma),
                                         ptr(dbeta), M, N, ptr(workspace), workspace.numel(),
                                         int(accumulate)))
+    return dx, dgamma, dbeta
+
+
+def layer_norm_backward_static(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, accumulate=False):
+    """ffk_layer_norm_backward without a workspace: the library's own per-device array."""
+    M, N = x.shape
+    check(lib().ffk_layer_norm_backward_static(current_stream(), dtype_of(x), ptr(dy), ptr(x),
+                                               ptr(mean), ptr(rstd), ptr(gamma), ptr(dx),
+                                               ptr(dgamma), ptr(dbeta), M, N, int(accumulate)))
     return dx, dgamma, dbeta
 
 

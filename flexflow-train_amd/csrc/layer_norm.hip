@@ -15,6 +15,7 @@
 #include "colreduce.h"
 #include "fused_ops.h"
 #include "dropout_rng.h"
+#include <mutex>
 
 namespace ffk {
 
@@ -419,7 +420,7 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
                        void *dx, void *dgamma, void *dbeta, int64_t M, int64_t N,
                        void *workspace, size_t workspace_bytes, bool acc,
                        void const *residual = nullptr, void *dropped = nullptr,
-                       DropoutParams const *drop = nullptr) {
+                       DropoutParams const *drop = nullptr, bool fit_blocks_to_workspace = false) {
   constexpr int V = VecIO<T>::kVec;
   T const *RES = static_cast<T const *>(residual);
   if (RES != nullptr) acc = true;
@@ -438,9 +439,15 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
     return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: residual form needs the vector kernel");
   }
   if (vec) {
-    int const blocks = ln_bwd_blocks(M, wpr);
-    size_t need = (size_t)blocks * 2 * (size_t)N * sizeof(float);
-    if (workspace == nullptr || workspace_bytes < need) {
+    int blocks = ln_bwd_blocks(M, wpr);
+    size_t const per_block = 2 * (size_t)N * sizeof(float);
+    if (fit_blocks_to_workspace && workspace_bytes / per_block < (size_t)blocks) {
+      // fewer, longer-running workgroups: dX is unchanged, the parameter
+      // gradients are summed over fewer partial rows
+      blocks = (int)(workspace_bytes / per_block);
+    }
+    size_t need = (size_t)blocks * per_block;
+    if (workspace == nullptr || blocks < 1 || workspace_bytes < need) {
       return fail(FFK_ERR_WORKSPACE,
                   "layer_norm_backward: workspace of %zu bytes needed, %zu given",
                   need, workspace_bytes);
@@ -593,4 +600,70 @@ extern "C" int ffk_layer_norm_backward(
                              input_grad, gamma_grad, beta_grad, M, N, workspace,
                              workspace_bytes, acc);
   return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: dtype %d not supported", dtype);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------
+// The per-workgroup partial sums of the parameter gradients, which
+// ffk_layer_norm_backward takes from its caller's workspace, live in this
+// array instead.  Every device the library runs on holds its own copy at its
+// own address until the process ends; host code only ever uses the address
+// that hipGetSymbolAddress returned for the device that was current.
+constexpr size_t kStaticScratchBytes = FFK_LAYER_NORM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float *g_scratch_ptr[kMaxDevices];  // per device, filled on that device's first call
+
+int static_scratch_for_current_device(float **out) {
+  int dev = -1;
+  FFK_HIP(hipGetDevice(&dev));
+  FFK_REQUIRE(dev >= 0 && dev < kMaxDevices, "layer_norm_backward_static: device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    float *p = nullptr;
+    FFK_HIP(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+    FFK_REQUIRE(p != nullptr, "layer_norm_backward_static: no device address for the scratch array");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return FFK_OK;
+}
+}  // namespace
+
+extern "C" int ffk_layer_norm_backward_static(
+    ffk_stream_t stream, int dtype, void const *output_grad, void const *input,
+    float const *mean, float const *rstd, void const *gamma, void *input_grad,
+    void *gamma_grad, void *beta_grad, int64_t M, int64_t N,
+    int accumulate_input_grad) {
+  FFK_REQUIRE(M >= 0 && N > 0 && N < (1ll << 31), "layer_norm_backward_static: bad shape");
+  if (M == 0) return FFK_OK;
+  FFK_REQUIRE(M < (1ll << 31), "layer_norm_backward_static: too many rows");
+  FFK_REQUIRE(output_grad && input && mean && rstd, "layer_norm_backward_static: NULL tensor");
+  FFK_REQUIRE(dtype == FFK_FLOAT || dtype == FFK_BF16, "layer_norm_backward_static: dtype %d not supported", dtype);
+  if (N > FFK_LAYER_NORM_STATIC_MAX_N) {
+    return fail(FFK_ERR_WORKSPACE,
+                "layer_norm_backward_static: rows of %lld elements exceed the limit of %d "
+                "(the scratch array is %zu bytes per device); use ffk_layer_norm_backward with a workspace",
+                (long long)N, FFK_LAYER_NORM_STATIC_MAX_N, kStaticScratchBytes);
+  }
+  float *ptr = nullptr;
+  int rc = static_scratch_for_current_device(&ptr);
+  if (rc != FFK_OK) return rc;
+  // The array is shared by every call on this device, so its column reduction
+  // runs here and now: a collected one would read the partial sums after a
+  // later call has overwritten them.
+  ColreduceBatch *const collecting = tl_colreduce_batch;
+  tl_colreduce_batch = nullptr;
+  bool const acc = accumulate_input_grad != 0;
+  if (dtype == FFK_FLOAT) {
+    rc = ln_backward<float>(as_stream(stream), output_grad, input, mean, rstd, gamma, input_grad, gamma_grad,
+                            beta_grad, M, N, ptr, kStaticScratchBytes, acc, nullptr, nullptr, nullptr, true);
+  } else {
+    rc = ln_backward<bf16>(as_stream(stream), output_grad, input, mean, rstd, gamma, input_grad, gamma_grad,
+                           beta_grad, M, N, ptr, kStaticScratchBytes, acc, nullptr, nullptr, nullptr, true);
+  }
+  tl_colreduce_batch = collecting;
+  return rc;
 }

@@ -229,6 +229,31 @@ int ffk_layer_norm_backward(ffk_stream_t stream, int dtype,
                             int64_t N, void *workspace, size_t workspace_bytes,
                             int accumulate_input_grad);
 
+/* ffk_layer_norm_backward for callers that cannot allocate device memory or
+ * bring a workspace: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference
+ * (whose LayerNorm state allocates its buffers at init,
+ * layer_norm_kernels.cu:292-325).  Same arguments and results as
+ * ffk_layer_norm_backward without the workspace pair: the partial column sums
+ * live in an array of FFK_LAYER_NORM_STATIC_SCRATCH_BYTES that every device
+ * the library runs on holds until the process ends.  The call allocates and
+ * frees nothing.  Rows longer than FFK_LAYER_NORM_STATIC_MAX_N elements are
+ * refused with FFK_ERR_WORKSPACE.  When the array holds fewer partial rows
+ * than ffk_layer_norm_backward would use (N above 2048), fewer workgroups
+ * walk the rows: input_grad has the same bits, gamma_grad / beta_grad are the
+ * same sums taken in a different order.  All calls on one device share the
+ * array: calls that overlap on one device (two streams, two threads) race;
+ * calls on one stream do not.  Inside ffk_column_reductions_begin/_end its
+ * column reduction is launched at once, not collected.                       */
+#define FFK_LAYER_NORM_STATIC_SCRATCH_BYTES (8u << 20)
+#define FFK_LAYER_NORM_STATIC_MAX_N 16384
+int ffk_layer_norm_backward_static(ffk_stream_t stream, int dtype,
+                                   void const *output_grad, void const *input,
+                                   float const *mean, float const *rstd,
+                                   void const *gamma, void *input_grad,
+                                   void *gamma_grad, void *beta_grad, int64_t M,
+                                   int64_t N, int accumulate_input_grad);
+
 /* ------------------------------------------------------------------------ */
 /* Softmax -- Kernels::Softmax::gpu_forward_kernel / gpu_backward_kernel
  * (softmax_kernels_gpu.h:18-26; lib/kernels/src/cuda/ops/softmax_kernels.cu:
