@@ -677,11 +677,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
   }
 }
 
+// the fp32 core (attention_f32.hip)
+int attention_f32_forward(hipStream_t st, ffk_attention_desc_t const *d, void const *q, void const *k,
+                          void const *v, void *o, float *lse);
+int attention_f32_backward(hipStream_t st, ffk_attention_desc_t const *d, void const *q, void const *k,
+                           void const *v, void const *o, void const *d_o, float const *lse, float *delta,
+                           void *dq, void *dk, void *dv);
+
 static int check_desc(char const *who, int dtype, ffk_attention_desc_t const *d) {
   FFK_REQUIRE(d != nullptr, "%s: NULL descriptor", who);
-  FFK_REQUIRE(dtype == FFK_BF16, "%s: dtype %d not supported (bf16 only)", who, dtype);
+  FFK_REQUIRE(dtype == FFK_BF16, "%s: dtype %d not supported (FLOAT or BF16)", who, dtype);
   FFK_REQUIRE(d->head_dim == 64 || d->head_dim == 128,
-              "%s: head_dim %lld not supported (64 or 128)", who, (long long)d->head_dim);
+              "%s: bf16 head_dim %lld not supported (64 or 128)", who, (long long)d->head_dim);
   FFK_REQUIRE(d->batch > 0 && d->heads > 0 && d->seq_q > 0 && d->seq_kv > 0, "%s: bad shape", who);
   FFK_REQUIRE(d->batch * d->heads * ((d->seq_q > d->seq_kv ? d->seq_q : d->seq_kv) / 128 + 1) < (1ll << 31),
               "%s: too many workgroups", who);
@@ -704,11 +711,13 @@ extern "C" int ffk_attention_forward(ffk_stream_t stream, int dtype,
                                      ffk_attention_desc_t const *d,
                                      void const *q, void const *k,
                                      void const *v, void *o, float *lse) {
-  int rc = check_desc("attention_forward", dtype, d);
-  if (rc != FFK_OK) return rc;
+  FFK_REQUIRE(d != nullptr, "attention_forward: NULL descriptor");
   FFK_REQUIRE(q && k && v && o, "attention_forward: NULL tensor");
   FFK_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o),
               "attention_forward: tensors must be 16-byte aligned");
+  if (dtype == FFK_FLOAT) return attention_f32_forward(as_stream(stream), d, q, k, v, o, lse);
+  int rc = check_desc("attention_forward", dtype, d);
+  if (rc != FFK_OK) return rc;
   AttnParams p;
   p.q = static_cast<bf16 const *>(q);
   p.k = static_cast<bf16 const *>(k);
@@ -739,13 +748,17 @@ extern "C" int ffk_attention_backward(ffk_stream_t stream, int dtype,
                                       void const *d_o, float const *lse,
                                       float *delta, void *dq, void *dk,
                                       void *dv) {
-  int rc = check_desc("attention_backward", dtype, d);
-  if (rc != FFK_OK) return rc;
+  FFK_REQUIRE(d != nullptr, "attention_backward: NULL descriptor");
   FFK_REQUIRE(q && k && v && o && d_o && lse && delta && dq && dk && dv,
               "attention_backward: NULL tensor");
   FFK_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) && aligned16(d_o) &&
                   aligned16(dq) && aligned16(dk) && aligned16(dv),
               "attention_backward: tensors must be 16-byte aligned");
+  if (dtype == FFK_FLOAT) {
+    return attention_f32_backward(as_stream(stream), d, q, k, v, o, d_o, lse, delta, dq, dk, dv);
+  }
+  int rc = check_desc("attention_backward", dtype, d);
+  if (rc != FFK_OK) return rc;
   AttnBwdParams p;
   p.q = static_cast<bf16 const *>(q);
   p.k = static_cast<bf16 const *>(k);

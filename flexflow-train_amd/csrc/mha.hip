@@ -8,7 +8,8 @@
 // W_O = [oProj, heads*vProj], all row-major.  When query, key and value are
 // the same tensor the three input projections run as one GEMM against the
 // contiguous [3*heads*proj, size] block and the core reads the fused buffer
-// through strides.
+// through strides.  FLOAT (the reference's data type) and BF16; the core is
+// attention_f32.hip / attention.hip.
 //
 // Reserve space layout (bytes, each region 256-byte aligned):
 //   QKV projections | context | lse | delta | d(context) | d(QKV projections)
@@ -50,21 +51,35 @@ static MhaLayout make_layout(ffk_mha_desc_t const *d, size_t es) {
 
 static int check_mha(char const *who, int dtype, ffk_mha_desc_t const *d) {
   FFK_REQUIRE(d != nullptr, "%s: NULL descriptor", who);
-  FFK_REQUIRE(dtype == FFK_BF16, "%s: dtype %d not supported (bf16 only)", who, dtype);
+  FFK_REQUIRE(dtype == FFK_BF16 || dtype == FFK_FLOAT, "%s: dtype %d not supported (FLOAT or BF16)", who, dtype);
   FFK_REQUIRE(d->num_samples > 0 && d->num_heads > 0 && d->q_size > 0 && d->k_size > 0 &&
                   d->v_size > 0 && d->o_proj_size > 0 && d->qo_seq_length > 0 && d->kv_seq_length > 0,
               "%s: non-positive size", who);
   FFK_REQUIRE(d->q_proj_size == d->k_proj_size, "%s: qProjSize must equal kProjSize", who);
   FFK_REQUIRE(d->v_proj_size == d->q_proj_size,
               "%s: vProjSize != qProjSize is not supported by the fused core", who);
-  FFK_REQUIRE(d->q_proj_size == 64 || d->q_proj_size == 128,
-              "%s: projection size %lld not supported (64 or 128)", who, (long long)d->q_proj_size);
+  if (dtype == FFK_BF16) {
+    FFK_REQUIRE(d->q_proj_size == 64 || d->q_proj_size == 128,
+                "%s: bf16 projection size %lld not supported (64 or 128)", who, (long long)d->q_proj_size);
+  } else {
+    FFK_REQUIRE(d->q_proj_size <= 128 && d->q_proj_size % 4 == 0,
+                "%s: fp32 projection size %lld not supported (a multiple of 4 up to 128)", who,
+                (long long)d->q_proj_size);
+  }
   return FFK_OK;
 }
 
-static bool is_fused(ffk_mha_desc_t const *d, void const *q, void const *k, void const *v) {
-  return q == k && k == v && d->q_size == d->k_size && d->k_size == d->v_size &&
-         d->qo_seq_length == d->kv_seq_length;
+// The reserve layout depends on the descriptor alone, so a backward call finds
+// what the forward call wrote whatever the caller's pointers are: with equal
+// input widths and sequence lengths the three projections are the column
+// blocks of ONE [tokens, 3*heads*proj] buffer (the core reads them through
+// strides), otherwise three dense tensors one after the other.
+static bool is_interleaved(ffk_mha_desc_t const *d) {
+  return d->q_size == d->k_size && d->k_size == d->v_size && d->qo_seq_length == d->kv_seq_length;
+}
+// Self-attention on one tensor: the three input projections are one GEMM.
+static bool is_aliased(ffk_mha_desc_t const *d, void const *q, void const *k, void const *v) {
+  return q == k && k == v && is_interleaved(d);
 }
 
 static ffk_attention_desc_t core_desc(ffk_mha_desc_t const *d, bool fused) {
@@ -119,11 +134,11 @@ extern "C" int ffk_mha_forward(ffk_stream_t stream, int dtype,
   uint8_t *rs = static_cast<uint8_t *>(reserve);
   uint8_t const *w = static_cast<uint8_t const *>(weight);
   int64_t const H = d->num_heads, D = d->q_proj_size, HD = H * D;
-  bool const fused = is_fused(d, query, key, value);
+  bool const fused = is_interleaved(d);
   uint8_t *qkv = rs + L.off_qkv;
   GemmEpilogue ep;
   void const *qp, *kp, *vp;
-  if (fused) {
+  if (is_aliased(d, query, key, value)) {
     // [T, 3HD] = X . [W_Q; W_K; W_V]^T
     rc = gemm_dispatch(st, dtype, false, true, L.TQ, 3 * HD, d->q_size, query, d->q_size,
                        w + L.wq * es, d->q_size, qkv, 3 * HD, ep);
@@ -132,15 +147,16 @@ extern "C" int ffk_mha_forward(ffk_stream_t stream, int dtype,
     kp = qkv + HD * es;
     vp = qkv + 2 * HD * es;
   } else {
-    uint8_t *Q = qkv, *K = qkv + L.nQ * es, *V = K + L.nK * es;
+    uint8_t *Q = qkv, *K = fused ? qkv + HD * es : qkv + L.nQ * es, *V = fused ? qkv + 2 * HD * es : K + L.nK * es;
+    int64_t const ld = fused ? 3 * HD : HD;
     rc = gemm_dispatch(st, dtype, false, true, L.TQ, HD, d->q_size, query, d->q_size,
-                       w + L.wq * es, d->q_size, Q, HD, ep);
+                       w + L.wq * es, d->q_size, Q, ld, ep);
     if (rc != FFK_OK) return rc;
     rc = gemm_dispatch(st, dtype, false, true, L.TK, HD, d->k_size, key, d->k_size,
-                       w + L.wk * es, d->k_size, K, HD, ep);
+                       w + L.wk * es, d->k_size, K, ld, ep);
     if (rc != FFK_OK) return rc;
     rc = gemm_dispatch(st, dtype, false, true, L.TK, HD, d->v_size, value, d->v_size,
-                       w + L.wv * es, d->v_size, V, HD, ep);
+                       w + L.wv * es, d->v_size, V, ld, ep);
     if (rc != FFK_OK) return rc;
     qp = Q; kp = K; vp = V;
   }
@@ -175,7 +191,13 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
   uint8_t const *w = static_cast<uint8_t const *>(weight);
   uint8_t *dw = static_cast<uint8_t *>(weight_grad);
   int64_t const H = d->num_heads, D = d->q_proj_size, HD = H * D;
-  bool const fused = is_fused(d, query, key, value);
+  bool const fused = is_interleaved(d);
+  bool const aliased = is_aliased(d, query, key, value);
+  // one tensor, three roles: its gradient is the sum of the three, which needs
+  // either all three outputs or query_grad alone
+  FFK_REQUIRE(!aliased || (key_grad == nullptr) == (value_grad == nullptr),
+              "mha_backward: query, key and value are one tensor: pass both key_grad and value_grad, or "
+              "neither (their gradients are then added into query_grad)");
   uint8_t *qkv = rs + L.off_qkv, *dqkv = rs + L.off_dqkv;
   uint8_t *ctx = rs + L.off_ctx, *dctx = rs + L.off_dctx;
   GemmEpilogue over, acc, in_ep;
@@ -190,7 +212,7 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
   // folded Q/K/V projection) have the same reduction length and each leaves
   // part of the chip idle: where the library can, they run as ONE launch after
   // the core's backward.
-  bool const folded = fused && key_grad == nullptr && value_grad == nullptr;
+  bool const folded = aliased && key_grad == nullptr && value_grad == nullptr;
   GemmProblem const wo_grad = {d->o_proj_size, HD, output_grad, d->o_proj_size, ctx, HD,
                                dw != nullptr ? dw + L.wo * es : nullptr, HD};
   GemmProblem const wqkv_grad = {3 * HD, d->q_size, dqkv, 3 * HD, query, d->q_size,

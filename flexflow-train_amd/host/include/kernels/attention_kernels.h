@@ -1,9 +1,12 @@
 // MultiHeadAttention entry points (reference:
 // lib/kernels/include/kernels/attention_kernels.h:12-51; state
 // mha_per_device_state.dtg.toml).  The float* signatures are the reference's
-// (fp32 tensors); the fused core is bf16, so those overloads raise, and the
-// accessor overloads below carry the dtype.  scale / causal are state fields
-// with the reference's values (1.0, false) as defaults.
+// (fp32 tensors, a state from the reference's init_kernel); the accessor
+// overloads carry the dtype (FLOAT or BF16).  scale / causal are state fields
+// with the reference's values (1.0, false) as defaults.  Like cuDNN's calls,
+// backward stores the input gradients and adds into the weight gradient.
+// Limits: qProjSize == kProjSize == vProjSize; FLOAT: a multiple of 4 up to
+// 128; BF16: 64 or 128.
 #pragma once
 #include "kernels/accessor.h"
 #include "kernels/allocation.h"

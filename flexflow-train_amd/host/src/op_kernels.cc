@@ -148,7 +148,8 @@ static void run_forward(device_stream_t const &stream, MHAPerDeviceState const &
 void forward_kernel(device_stream_t const &stream, std::optional<MHAPerDeviceState> const &state,
                     float const *q, float const *k, float const *v, float const *w, float *out) {
   if (!stream.is_gpu()) no_cpu("MultiHeadAttention::forward_kernel");
-  run_forward(stream, state.value(), q, k, v, w, out);  // fp32 state: the C ABI reports "bf16 only"
+  if (state.value().data_type != DataType::FLOAT) throw std::runtime_error("MultiHeadAttention: float pointers with a state that is not FLOAT");
+  run_forward(stream, state.value(), q, k, v, w, out);
 }
 
 void forward_kernel(device_stream_t const &stream, std::optional<MHAPerDeviceState> const &state,
@@ -164,9 +165,10 @@ static void run_backward(device_stream_t const &stream, MHAPerDeviceState const 
                          void const *k, void *dk, void const *v, void *dv, void const *w, void *dw,
                          void const *dout) {
   ffk_mha_desc_t d = make_desc(s);
-  // input gradients accumulate like every reference GPU backward (callers zero them first)
+  // cudnnMultiHeadAttnBackwardData stores the input gradients, BackwardWeights runs in
+  // CUDNN_WGRAD_MODE_ADD (src/cuda/ops/attention_kernels.cu:261-303): the same here
   check_ffk(ffk_mha_backward(stream.require_gpu(), dt(s.data_type), &d, q, dq, k, dk, v, dv, w, dw, dout,
-                             s.reserveSpace, s.reserveSpaceSize, 1),
+                             s.reserveSpace, s.reserveSpaceSize, 0),
             "MultiHeadAttention::backward_kernel");
 }
 
@@ -174,6 +176,7 @@ void backward_kernel(device_stream_t const &stream, std::optional<MHAPerDeviceSt
                      float const *q, float *dq, float const *k, float *dk, float const *v, float *dv,
                      float const *w, float *dw, float const *dout) {
   if (!stream.is_gpu()) no_cpu("MultiHeadAttention::backward_kernel");
+  if (state.value().data_type != DataType::FLOAT) throw std::runtime_error("MultiHeadAttention: float pointers with a state that is not FLOAT");
   run_backward(stream, state.value(), q, dq, k, dk, v, dv, w, dw, dout);
 }
 

@@ -402,7 +402,7 @@ static void gpu_tests() {
     CHECK(close(to_host(DW), dw, 1e-5));
   });
 
-  run("MultiHeadAttention (bf16 accessors) vs oracle; fp32 pointers are refused", [&] {
+  run("MultiHeadAttention (bf16 accessors) vs oracle", [&] {
     int B = 2, H = 4, E = 64, D = 64, S = 20;  // the reference test's sizes, [batch, seq, size]
     auto q = random_vec(B * S * E, 17), dout = random_vec(B * S * E, 18);
     size_t nw = (size_t)H * D * 3 * E + (size_t)E * H * D;
@@ -427,9 +427,47 @@ static void gpu_tests() {
     Kernels::MultiHeadAttention::backward_kernel(stream, state, Q, DQ, Q, std::nullopt, Q, std::nullopt, W, DW, DO);
     CHECK(close(to_host(DQ), dq, 2e-2) && close(to_host(DW), dw, 2e-2));
     Kernels::MultiHeadAttention::cleanup_kernel(DeviceType::GPU, gpu, state);
-    auto fstate = Kernels::MultiHeadAttention::init_kernel(DeviceType::GPU, handle, gpu, B, H, E, E, E, D, D, D, E, S, S, false);
-    CHECK_THROWS(Kernels::MultiHeadAttention::forward_kernel(stream, fstate, (float const *)Q.ptr, (float const *)Q.ptr,
+    // float pointers belong to a FLOAT state
+    CHECK_THROWS(Kernels::MultiHeadAttention::forward_kernel(stream, state, (float const *)Q.ptr, (float const *)Q.ptr,
                                                              (float const *)Q.ptr, (float const *)W.ptr, (float *)O.ptr));
+  });
+  run("MultiHeadAttention, the reference's float signature (fp32, scale 1, q = k = v, NULL dk/dv) vs oracle", [&] {
+    // the sizes of lib/kernels/test/src/test_attention_kernel.cc, [batch, seq, size]
+    int B = 2, H = 4, E = 64, D = 64, S = 20;
+    auto q = random_vec(B * S * E, 27, -0.5f, 0.5f), dout = random_vec(B * S * E, 28);
+    size_t nw = (size_t)H * D * 3 * E + (size_t)E * H * D;
+    auto w = random_vec(nw, 29, -0.2f, 0.2f);
+    orc_mha_desc_t od{B, H, E, E, E, D, D, D, E, S, S, 1.0f, 0};
+    std::vector<float> out(B * S * E), dq(q.size()), dk(q.size()), dv(q.size()), dw(nw, 0.0f);
+    orc_mha_forward(&od, q.data(), q.data(), q.data(), w.data(), out.data(), 0);
+    orc_mha_backward(&od, q.data(), q.data(), q.data(), w.data(), dout.data(), dq.data(), dk.data(), dv.data(), dw.data(), 0);
+    for (size_t i = 0; i < dq.size(); i++) dq[i] += dk[i] + dv[i];
+    auto state = Kernels::MultiHeadAttention::init_kernel(DeviceType::GPU, handle, gpu, B, H, E, E, E, D, D, D, E, S, S, false);
+    CHECK(state->weightSize == nw * 4);
+    auto Q = device_accessor(gpu, shape({B, S, E}, DataType::FLOAT), q);
+    auto W = device_accessor(gpu, shape({(int64_t)nw}, DataType::FLOAT), w);
+    auto DO = device_accessor(gpu, Q.shape, dout);
+    auto O = gpu.allocate_tensor(Q.shape), DW = gpu.allocate_tensor(W.shape);
+    // the input gradient is stored, not added to: start it from values that would show
+    auto DQ = device_accessor(gpu, Q.shape, random_vec(q.size(), 30, 5.0f, 6.0f));
+    fill_with_zeros(DW);
+    Kernels::MultiHeadAttention::forward_kernel(stream, state, Q.get_float_ptr(), Q.get_float_ptr(), Q.get_float_ptr(),
+                                                W.get_float_ptr(), O.get_float_ptr());
+    CHECK(contains_non_zero(to_host(O)));
+    CHECK(close(to_host(O), out, 1e-5));
+    Kernels::MultiHeadAttention::backward_kernel(stream, state, Q.get_float_ptr(), DQ.get_float_ptr(), Q.get_float_ptr(),
+                                                 nullptr, Q.get_float_ptr(), nullptr, W.get_float_ptr(), DW.get_float_ptr(),
+                                                 DO.get_float_ptr());
+    CHECK(close(to_host(DQ), dq, 1e-5));
+    CHECK(close(to_host(DW), dw, 1e-5));
+    // the weight gradient is added to (CUDNN_WGRAD_MODE_ADD): a second call doubles it
+    Kernels::MultiHeadAttention::backward_kernel(stream, state, Q.get_float_ptr(), DQ.get_float_ptr(), Q.get_float_ptr(),
+                                                 nullptr, Q.get_float_ptr(), nullptr, W.get_float_ptr(), DW.get_float_ptr(),
+                                                 DO.get_float_ptr());
+    for (auto &x : dw) x *= 2.0f;
+    CHECK(close(to_host(DQ), dq, 1e-5));
+    CHECK(close(to_host(DW), dw, 1e-5));
+    Kernels::MultiHeadAttention::cleanup_kernel(DeviceType::GPU, gpu, state);
   });
   run("sgd_update_task / adam_update_task equal the oracle bit for bit", [&] {
     int64_t n = 10007;

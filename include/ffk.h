@@ -402,13 +402,16 @@ int ffk_embedding_backward(ffk_stream_t stream, int index_dtype,
 /* Fused (flash-style) scaled-dot-product attention core: the QK^T / softmax /
  * PV contraction that cudnnMultiHeadAttnForward/BackwardData perform inside
  * lib/kernels/src/cuda/ops/attention_kernels.cu:224,261, without the S x S
- * score matrix ever reaching HBM.  dtype FFK_BF16.
+ * score matrix ever reaching HBM.  dtype FFK_BF16 (head_dim 64 or 128, strides
+ * multiples of 8) or FFK_FLOAT (the reference's data type; head_dim any
+ * multiple of 4 up to 128, strides multiples of 4).
  *   q,k,v,o: element (b, s, h, d) at  b*batch_stride + s*seq_stride +
  *   h*head_dim + d  (strides in elements), so the same kernel reads the
  *   [batch, seq, heads*head_dim] projections and a fused QKV buffer.
  *   lse [batch, heads, seq_q] fp32: log-sum-exp of the scaled scores, written
  *   by forward and read by backward.  scale multiplies QK^T (the reference
- *   uses 1.0, attention_kernels.cu:76); causal != 0 masks k > q.
+ *   uses 1.0, attention_kernels.cu:76); causal != 0 masks key index > query
+ *   index (aligned top-left when seq_q != seq_kv).
  * backward needs delta [batch, heads, seq_q] fp32 scratch (written inside).  */
 /* ------------------------------------------------------------------------ */
 typedef struct {
@@ -436,6 +439,8 @@ int ffk_attention_backward(ffk_stream_t stream, int dtype,
  * lib/kernels/src/cuda/ops/attention_kernels.cu:215-303).
  *   query [B,Sq,qSize], key [B,Skv,kSize], value [B,Skv,vSize],
  *   output [B,Sq,oProjSize].  No bias, no dropout (attention_kernels.cu:73-92).
+ *   dtype FFK_FLOAT (the reference's) or FFK_BF16.  q/k/v_proj_size must be
+ *   equal: FLOAT any multiple of 4 up to 128, BF16 64 or 128.
  *   weight blob (defined by this library; the reference never indexes it):
  *     [ W_Q | W_K | W_V | W_O ], W_Q = [heads*qProj, qSize] row-major with
  *     head-major rows (likewise W_K [heads*kProj, kSize], W_V [heads*vProj,
@@ -444,11 +449,15 @@ int ffk_attention_backward(ffk_stream_t stream, int dtype,
  *     attention.cc:165-185).
  *   The reserve space (ffk_mha_reserve_bytes) holds the projected Q,K,V, the
  *   pre-projection context and the log-sum-exp between forward and backward
- *   plus backward scratch, like MHAPerDeviceState.reserveSpace.
- * backward: query_grad/key_grad/value_grad are overwritten unless accumulate;
+ *   plus backward scratch, like MHAPerDeviceState.reserveSpace.  Its layout
+ *   follows from the descriptor alone, so backward needs the descriptor forward
+ *   had and nothing else.
+ * backward: query_grad/key_grad/value_grad are overwritten unless accumulate
+ *   (cudnnMultiHeadAttnBackwardData stores them);
  *   key_grad/value_grad may be NULL when key/value alias query (their
  *   gradients are then folded into query_grad, as the reference's task impl
- *   expects, lib/task-spec/src/task-spec/ops/impl/attention.cc:129-133);
+ *   expects, lib/task-spec/src/task-spec/ops/impl/attention.cc:129-133) --
+ *   both or neither: one of them NULL alone is FFK_ERR_INVALID;
  *   weight_grad is accumulated into (CUDNN_WGRAD_MODE_ADD).  `accumulate` is
  *   0 / 1 as just described, optionally or-ed with
  *   FFK_MHA_OVERWRITE_WEIGHT_GRAD to store the weight gradient instead of

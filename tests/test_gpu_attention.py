@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from util import BF16_RTOL, assert_close, bf16_round, rng, to_dev, to_np
+from util import BF16_RTOL, FP32_RTOL, assert_close, bf16_round, rng, to_dev, to_np
 
 pytestmark = pytest.mark.gpu
 BT = torch.bfloat16
@@ -25,9 +25,8 @@ SHAPES = [  # B, H, Sq, Skv, D
 @pytest.mark.parametrize("shape", SHAPES)
 @pytest.mark.parametrize("causal", [False, True])
 def test_attention_core(ffk, oracle, shape, causal):
+    # causal with Sq != Skv: key j is visible to query i iff j <= i (the mask is aligned top-left)
     B, H, Sq, Skv, D = shape
-    if causal and Sq != Skv:
-        pytest.skip("causal is defined for self-attention (Sq == Skv) here")
     say("attention core", shape, "causal", causal)
     g = rng(Sq * 7 + D + int(causal))
     q = bf16_round(g.standard_normal((B, Sq, H, D)))
@@ -45,6 +44,34 @@ def test_attention_core(ffk, oracle, shape, causal):
     assert_close(to_np(dq), dq_ref, BF16_RTOL, "dQ")
     assert_close(to_np(dk), dk_ref, BF16_RTOL, "dK")
     assert_close(to_np(dv), dv_ref, BF16_RTOL, "dV")
+
+
+F32_SHAPES = [  # B, H, Sq, Skv, D
+    (1, 1, 8, 8, 64), (2, 3, 11, 11, 32), (1, 2, 100, 100, 128), (2, 2, 129, 129, 64), (1, 2, 40, 40, 4),
+    (1, 4, 256, 256, 128), (1, 2, 300, 300, 48), (1, 1, 64, 200, 64), (2, 1, 160, 96, 100), (1, 3, 70, 33, 20),
+]
+
+
+@pytest.mark.parametrize("shape", F32_SHAPES)
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_core_fp32(ffk, oracle, shape, causal):
+    """The fp32 core behind the reference's float MultiHeadAttention signature."""
+    B, H, Sq, Skv, D = shape
+    say("attention core fp32", shape, "causal", causal)
+    g = rng(Sq * 5 + D + int(causal))
+    q, k, v, do = (g.standard_normal(s).astype(np.float32)
+                   for s in ((B, Sq, H, D), (B, Skv, H, D), (B, Skv, H, D), (B, Sq, H, D)))
+    scale = 1.0 / np.sqrt(D)
+    o_ref, lse_ref = oracle.attention_forward(q, k, v, scale, causal, bf16_mode=False)
+    qd, kd, vd, dod = (to_dev(a, torch) for a in (q, k, v, do))
+    o, lse = ffk.attention_forward(qd, kd, vd, scale, causal)
+    assert_close(to_np(o), o_ref, FP32_RTOL, "O")
+    assert_close(to_np(lse), lse_ref, FP32_RTOL, "lse")
+    dq_ref, dk_ref, dv_ref = oracle.attention_backward(q, k, v, do, scale, causal)
+    dq, dk, dv = ffk.attention_backward(qd, kd, vd, o, dod, lse, scale, causal)
+    assert_close(to_np(dq), dq_ref, FP32_RTOL, "dQ")
+    assert_close(to_np(dk), dk_ref, FP32_RTOL, "dK")
+    assert_close(to_np(dv), dv_ref, FP32_RTOL, "dV")
 
 
 def test_attention_reference_scale_one(ffk, oracle):
@@ -100,9 +127,14 @@ def test_attention_errors(ffk):
     q = torch.zeros((1, 8, 1, 32), dtype=BT, device="cuda")
     with pytest.raises(ffk.FFKError, match="head_dim"):
         ffk.attention_forward(q, q, q, 1.0, False)
-    q32 = torch.zeros((1, 8, 1, 64), dtype=torch.float32, device="cuda")
-    with pytest.raises(ffk.FFKError, match="dtype"):
+    q32 = torch.zeros((1, 8, 1, 132), dtype=torch.float32, device="cuda")
+    with pytest.raises(ffk.FFKError, match="head_dim"):
         ffk.attention_forward(q32, q32, q32, 1.0, False)
+    q16 = torch.zeros((1, 8, 1, 64), dtype=torch.float16, device="cuda")
+    desc = ffk.attention_desc_bshd(q16, q16, 1.0, False)
+    rc = ffk.lib().ffk_attention_forward(0, ffk.HALF, desc, q16.data_ptr(), q16.data_ptr(), q16.data_ptr(),
+                                         q16.data_ptr(), None)
+    assert rc == 1 and b"dtype" in ffk.lib().ffk_last_error()
 
 
 def test_attention_config5_causal_prefix(ffk, oracle):
@@ -156,16 +188,20 @@ MHA_CASES = [  # B, Sq, Skv, H, E(q), Ek, Ev, Dh, oProj, self-attention?
     (1, 24, 40, 2, 64, 72, 80, 64, 64, False),
     (2, 64, 64, 2, 256, 256, 256, 128, 256, True),
     (2, 64, 64, 12, 768, 768, 768, 64, 768, True),  # both weight gradients in one two-problem GEMM launch
+    (2, 24, 24, 2, 64, 64, 64, 64, 64, False),      # three tensors of one shape: one interleaved projection buffer
+]
+MHA_CASES_FP32 = MHA_CASES[:4] + [
+    (2, 20, 20, 4, 64, 64, 64, 16, 64, True),   # head sizes the bf16 core does not take
+    (1, 24, 40, 2, 64, 72, 80, 40, 56, False),
+    (2, 24, 24, 2, 64, 64, 64, 32, 64, False),
 ]
 
 
-@pytest.mark.parametrize("case", MHA_CASES)
-@pytest.mark.parametrize("causal", [False, True])
-def test_mha(ffk, oracle, case, causal):
+def _mha_case(ffk, oracle, case, causal, fp32):
     B, Sq, Skv, H, E, Ek, Ev, Dh, oP, self_attn = case
-    if causal and Sq != Skv:
-        pytest.skip("causal needs Sq == Skv")
-    say("mha", case, "causal", causal)
+    say("mha", "fp32" if fp32 else "bf16", case, "causal", causal)
+    BT, BF16_RTOL, dtype = (torch.float32, FP32_RTOL, ffk.FLOAT) if fp32 else (torch.bfloat16, 2e-2, ffk.BF16)
+    bf16_round = (lambda a: np.asarray(a, dtype=np.float32)) if fp32 else globals()["bf16_round"]
     g = rng(Sq + E + int(causal))
     scale = 1.0 / np.sqrt(Dh)
     query = bf16_round(g.standard_normal((B, Sq, E)))
@@ -177,24 +213,24 @@ def test_mha(ffk, oracle, case, causal):
     assert nw == H * Dh * (E + Ek + Ev) + oP * H * Dh
     w = bf16_round(g.standard_normal((nw,)) * (2.0 / np.sqrt(E)))
     dout = bf16_round(g.standard_normal((B, Sq, oP)))
-    out_ref = oracle.mha_forward(odesc, query, key, value, w, bf16_mode=True)
-    dq_ref, dk_ref, dv_ref, dw_ref = oracle.mha_backward(odesc, query, key, value, w, dout, bf16_mode=True)
+    out_ref = oracle.mha_forward(odesc, query, key, value, w, bf16_mode=not fp32)
+    dq_ref, dk_ref, dv_ref, dw_ref = oracle.mha_backward(odesc, query, key, value, w, dout, bf16_mode=not fp32)
 
     qd = to_dev(query, torch, BT)
     kd = qd if self_attn else to_dev(key, torch, BT)
     vd = qd if self_attn else to_dev(value, torch, BT)
     wd, doutd = to_dev(w, torch, BT), to_dev(dout, torch, BT)
-    reserve = ffk.mha_reserve(desc, ffk.BF16)
+    reserve = ffk.mha_reserve(desc, dtype)
     out = ffk.mha_forward(desc, qd, kd, vd, wd, reserve)
     assert_close(to_np(out), out_ref, BF16_RTOL, "out")
     dw = torch.zeros_like(wd)
-    dq = torch.zeros_like(qd)
+    dq = torch.full_like(qd, 3.0)  # input gradients are stored, not added to
     if self_attn:
         # key/value alias query: their gradients fold into query_grad
         ffk.mha_backward(desc, qd, dq, kd, None, vd, None, wd, dw, doutd, reserve)
         assert_close(to_np(dq), dq_ref + dk_ref + dv_ref, BF16_RTOL, "dquery (folded)")
     else:
-        dk, dv = torch.zeros_like(kd), torch.zeros_like(vd)
+        dk, dv = torch.full_like(kd, 3.0), torch.full_like(vd, 3.0)
         ffk.mha_backward(desc, qd, dq, kd, dk, vd, dv, wd, dw, doutd, reserve)
         assert_close(to_np(dq), dq_ref, BF16_RTOL, "dquery")
         assert_close(to_np(dk), dk_ref, BF16_RTOL, "dkey")
@@ -207,6 +243,40 @@ def test_mha(ffk, oracle, case, causal):
     else:
         ffk.mha_backward(desc, qd, dq2, kd, torch.zeros_like(kd), vd, torch.zeros_like(vd), wd, dw, doutd, reserve)
     assert_close(to_np(dw), 2 * dw_ref, BF16_RTOL * 1.5, "dweight accumulated")
+
+
+@pytest.mark.parametrize("case", MHA_CASES)
+@pytest.mark.parametrize("causal", [False, True])
+def test_mha(ffk, oracle, case, causal):
+    _mha_case(ffk, oracle, case, causal, fp32=False)
+
+
+@pytest.mark.parametrize("case", MHA_CASES_FP32)
+@pytest.mark.parametrize("causal", [False, True])
+def test_mha_fp32(ffk, oracle, case, causal):
+    """FLOAT is the data type of the reference's own entry points (attention_kernels.h:12-51)."""
+    _mha_case(ffk, oracle, case, causal, fp32=True)
+
+
+def test_mha_accumulate_input_grads(ffk, oracle):
+    say("mha input gradients added on request")
+    B, S, H, E, Dh = 1, 16, 2, 64, 64
+    g = rng(9)
+    x = g.standard_normal((B, S, E)).astype(np.float32)
+    odesc = oracle.mha_desc(B, H, E, E, E, Dh, Dh, Dh, E, S, S, 0.125, False)
+    desc = ffk.mha_desc(B, H, E, E, E, Dh, Dh, Dh, E, S, S, 0.125, False)
+    w = (g.standard_normal((ffk.lib().ffk_mha_weight_elements(desc),)) * 0.2).astype(np.float32)
+    dout = g.standard_normal((B, S, E)).astype(np.float32)
+    dq_ref, dk_ref, dv_ref, _ = oracle.mha_backward(odesc, x, x, x, w, dout)
+    xd, wd, dd = to_dev(x, torch), to_dev(w, torch), to_dev(dout, torch)
+    reserve = ffk.mha_reserve(desc, ffk.FLOAT)
+    ffk.mha_forward(desc, xd, xd, xd, wd, reserve)
+    dq = torch.full_like(xd, 2.0)
+    ffk.mha_backward(desc, xd, dq, xd, None, xd, None, wd, torch.zeros_like(wd), dd, reserve, accumulate=True)
+    assert_close(to_np(dq), 2.0 + dq_ref + dk_ref + dv_ref, FP32_RTOL, "dquery added")
+    # one tensor in three roles: key_grad without value_grad has no meaning
+    with pytest.raises(ffk.FFKError, match="one tensor"):
+        ffk.mha_backward(desc, xd, dq, xd, torch.zeros_like(xd), xd, None, wd, torch.zeros_like(wd), dd, reserve)
 
 
 def test_mha_separate_grads_when_aliased(ffk, oracle):
@@ -240,3 +310,7 @@ def test_mha_errors(ffk):
     bad = ffk.mha_desc(1, 2, 64, 64, 64, 48, 48, 48, 64, 8, 8)
     with pytest.raises(ffk.FFKError, match="projection size"):
         ffk.mha_forward(bad, x, x, x, w, ffk.mha_reserve(desc, ffk.BF16))
+    bad = ffk.mha_desc(1, 2, 64, 64, 64, 256, 256, 256, 64, 8, 8)
+    x32, w32 = x.float(), torch.zeros((ffk.lib().ffk_mha_weight_elements(bad),), dtype=torch.float32, device="cuda")
+    with pytest.raises(ffk.FFKError, match="projection size"):
+        ffk.mha_forward(bad, x32, x32, x32, w32, ffk.mha_reserve(bad, ffk.FLOAT))
