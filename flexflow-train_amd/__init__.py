@@ -95,6 +95,8 @@ SIGNATURES = {
     "ffk_event_record": (c_int, [c_p, c_p]),
     "ffk_event_synchronize": (c_int, [c_p]),
     "ffk_event_elapsed_ms": (c_int, [c_p, c_p, ctypes.POINTER(c_f)]),
+    "ffk_set_option": (c_int, [c_int, c_int]),
+    "ffk_get_option": (c_int, [c_int, ctypes.POINTER(c_int)]),
     "ffk_linear_forward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_p, c_i64, c_i64, c_i64]),
     "ffk_linear_backward_workspace_bytes": (c_sz, [c_int, c_int, c_int, c_i64, c_i64]),
     "ffk_linear_backward": (c_int, [c_p, c_int, c_int, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
@@ -192,6 +194,14 @@ def lib():
             fn.argtypes = args
         _lib = handle
     return _lib
+
+
+OPTION_GEMM_VARIANT, OPTION_LAYER_UNFUSED = 0, 1
+
+
+def set_option(which, value):
+    """Process-wide tuning / test switch (see ffk_set_option in ffk.h)."""
+    check(lib().ffk_set_option(which, int(value)))
 
 
 def check(rc):

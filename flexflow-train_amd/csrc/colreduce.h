@@ -78,24 +78,6 @@ __global__ __launch_bounds__(1024) void colreduce_batch_kernel(ColreduceBatch b)
   colreduce_block<T>(b.job[k], (int)blockIdx.x - b.first_block[k], red);
 }
 
-template <typename T>
-inline hipError_t colreduce_launch(hipStream_t st, float const *partials,
-                                   int nparts, int ncols, int split, T *out0,
-                                   T *out1, bool accumulate) {
-  ColreduceJob const job{partials, nparts, ncols, split, out0, out1, accumulate ? 1 : 0};
-  ColreduceBatch *b = tl_colreduce_batch;
-  int const dtype = sizeof(T) == 4 ? FFK_FLOAT : FFK_BF16;
-  if (b != nullptr && b->count < kMaxColreduceJobs && (b->count == 0 || b->dtype == dtype)) {
-    b->first_block[b->count] = b->count == 0 ? 0 : b->first_block[b->count - 1] + (int)ceil_div(b->job[b->count - 1].ncols, 32);
-    b->job[b->count] = job;
-    b->dtype = dtype;
-    b->count++;
-    return hipSuccess;
-  }
-  colreduce_kernel<T><<<(unsigned)ceil_div(ncols, 32), 1024, 0, st>>>(job);
-  return hipGetLastError();
-}
-
 // Runs what was collected (nothing to do for an empty batch) and empties it.
 inline hipError_t colreduce_flush(hipStream_t st, ColreduceBatch &b) {
   if (b.count == 0) return hipSuccess;
@@ -107,6 +89,39 @@ inline hipError_t colreduce_flush(hipStream_t st, ColreduceBatch &b) {
     colreduce_batch_kernel<bf16><<<(unsigned)blocks, 1024, 0, st>>>(b);
   }
   b.count = 0;
+  return hipGetLastError();
+}
+
+template <typename T>
+inline hipError_t colreduce_launch(hipStream_t st, float const *partials,
+                                   int nparts, int ncols, int split, T *out0,
+                                   T *out1, bool accumulate) {
+  ColreduceJob const job{partials, nparts, ncols, split, out0, out1, accumulate ? 1 : 0};
+  ColreduceBatch *b = tl_colreduce_batch;
+  int const dtype = sizeof(T) == 4 ? FFK_FLOAT : FFK_BF16;
+  if (b != nullptr) {
+    // The collected jobs run as one launch, in no order: a job that writes where a collected
+    // one writes (a bias shared by two Linear layers) would race with it.  Run what is
+    // collected first; this job then follows it on the stream.
+    for (int k = 0; k < b->count; k++) {
+      ColreduceJob const &c = b->job[k];
+      bool const clash = (out0 != nullptr && (c.out0 == out0 || c.out1 == out0)) ||
+                         (out1 != nullptr && (c.out0 == out1 || c.out1 == out1));
+      if (clash) {
+        hipError_t e = colreduce_flush(st, *b);
+        if (e != hipSuccess) return e;
+        break;
+      }
+    }
+  }
+  if (b != nullptr && b->count < kMaxColreduceJobs && (b->count == 0 || b->dtype == dtype)) {
+    b->first_block[b->count] = b->count == 0 ? 0 : b->first_block[b->count - 1] + (int)ceil_div(b->job[b->count - 1].ncols, 32);
+    b->job[b->count] = job;
+    b->dtype = dtype;
+    b->count++;
+    return hipSuccess;
+  }
+  colreduce_kernel<T><<<(unsigned)ceil_div(ncols, 32), 1024, 0, st>>>(job);
   return hipGetLastError();
 }
 

@@ -75,13 +75,10 @@ static int check_layer(char const *who, int dtype, ffk_encoder_layer_desc_t cons
   return FFK_OK;
 }
 
-// FFK_LAYER_UNFUSED=1 runs every op of the layer as its own kernel (the plain
-// operator sequence); the default fuses neighbours where the result is
-// bit-identical.  For tests that compare the two.
-static bool layer_fusion_enabled() {
-  char const *e = getenv("FFK_LAYER_UNFUSED");  // read per call: tests toggle it
-  return !(e != nullptr && atoi(e) != 0);
-}
+// FFK_OPTION_LAYER_UNFUSED != 0 runs every op of the layer as its own kernel
+// (the plain operator sequence); the default fuses neighbours where the result
+// is bit-identical.  For tests that compare the two.
+static bool layer_fusion_enabled() { return option(FFK_OPTION_LAYER_UNFUSED) == 0; }
 
 // out = residual + dropout(in): one fused pass when possible, else dropout
 // into `scratch` followed by the element-wise add.
@@ -221,6 +218,8 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   size_t const ln_ws_bytes = L.ln_ws_b - L.ln_ws, lin_ws_bytes = L.lin_ws_b - L.lin_ws;
   int const wacc = d->overwrite_weight_grads ? 0 : (FFK_ACC_WEIGHT | FFK_ACC_BIAS);
   int const mha_mode = d->overwrite_weight_grads ? FFK_MHA_OVERWRITE_WEIGHT_GRAD : 0;
+  bool const ln_acc = !d->overwrite_weight_grads;  // LayerNorm gamma / beta gradients follow the same switch
+  int const ln_mode = ln_acc ? FFK_LN_ACC_PARAMS : 0;
 
   // The four small column reductions of this pass (two bias gradients, two pairs of LayerNorm
   // parameter gradients) are collected and run as one launch at the end: each is a few
@@ -236,7 +235,7 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   void const *g_sum = dy;  // gradient of (x1 + f2_drop)
   if (!d->pre_layer_norm) {
     FFK_TRY(ffk_layer_norm_backward(st, dtype, dy, ws + L.pre2, mean(L.mean2), mean(L.rstd2), w->ln2_gamma,
-                                    ws + L.g_tmp, g->ln2_gamma, g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+                                    ws + L.g_tmp, g->ln2_gamma, g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes, ln_mode));
     g_sum = ws + L.g_tmp;
   }
   // ---- FFN backward
@@ -316,13 +315,13 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
       rc = layer_norm_backward_add_residual(as_stream(st), dtype, ws + L.g_h2, ws + L.x1, mean(L.mean2),
                                             mean(L.rstd2), w->ln2_gamma, dy, ws + L.g_x1, g->ln2_gamma,
                                             g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes,
-                                            with_drop ? ws + L.g_attn : nullptr, p, d->seed + 0, 0);
+                                            with_drop ? ws + L.g_attn : nullptr, p, d->seed + 0, 0, ln_acc);
       if (rc != FFK_OK && rc != FFK_ERR_UNSUPPORTED) return rc;
       g_attn_ready = rc == FFK_OK && with_drop;
     }
     if (rc == FFK_ERR_UNSUPPORTED) {
       FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h2, ws + L.x1, mean(L.mean2), mean(L.rstd2), w->ln2_gamma,
-                                      ws + L.g_x1, g->ln2_gamma, g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes, 0));
+                                      ws + L.g_x1, g->ln2_gamma, g->ln2_beta, T, E, ws + L.ln_ws, ln_ws_bytes, ln_mode));
       FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, ws + L.g_x1, dy, ws + L.g_x1, T * E, T * E, T * E));
     }
   } else {
@@ -341,17 +340,17 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
     if (layer_fusion_enabled()) {
       rc = layer_norm_backward_add_residual(as_stream(st), dtype, ws + L.g_h1, x, mean(L.mean1), mean(L.rstd1),
                                             w->ln1_gamma, g_attn_res, dx, g->ln1_gamma, g->ln1_beta, T, E,
-                                            ws + L.ln_ws_b, ln_ws_bytes);
+                                            ws + L.ln_ws_b, ln_ws_bytes, nullptr, 0.0f, 0, 0, ln_acc);
       if (rc != FFK_OK && rc != FFK_ERR_UNSUPPORTED) return rc;
     }
     if (rc == FFK_ERR_UNSUPPORTED) {
       FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_h1, x, mean(L.mean1), mean(L.rstd1), w->ln1_gamma, dx,
-                                      g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws_b, ln_ws_bytes, 0));
+                                      g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws_b, ln_ws_bytes, ln_mode));
       FFK_TRY(ffk_element_binary_forward(st, dtype, FFK_OP_EW_ADD, dx, g_attn_res, dx, T * E, T * E, T * E));
     }
   } else {
     FFK_TRY(ffk_layer_norm_backward(st, dtype, ws + L.g_x1, ws + L.h1, mean(L.mean1), mean(L.rstd1), w->ln1_gamma,
-                                    ws + L.g_attn, g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws_b, ln_ws_bytes, 0));
+                                    ws + L.g_attn, g->ln1_gamma, g->ln1_beta, T, E, ws + L.ln_ws_b, ln_ws_bytes, ln_mode));
     g_attn_res = ws + L.g_attn;
     FFK_TRY(ffk_mha_backward(st, dtype, &m, x, dx, x, nullptr, x, nullptr, w->attn_weight, g->attn_weight,
                              g_attn_res, ws + L.mha_reserve, L.ln_ws - L.mha_reserve, mha_mode));

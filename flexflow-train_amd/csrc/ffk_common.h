@@ -14,6 +14,8 @@ namespace ffk {
 // thread and read back through ffk_last_error().
 void set_error(char const *fmt, ...);
 int fail(int code, char const *fmt, ...);
+// current value of a process-wide switch (FFK_OPTION_*, see ffk_set_option)
+int option(int which);
 
 #define FFK_HIP(expr)                                                          \
   do {                                                                         \

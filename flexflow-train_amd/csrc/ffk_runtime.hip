@@ -5,7 +5,9 @@
 // lib/kernels/src/kernels/accessor.cc:45-74,
 // lib/kernels/include/kernels/profiling.h:78-106).
 #include "ffk_common.h"
+#include <atomic>
 #include <stdarg.h>
+#include <stdlib.h>
 #include <string.h>
 
 namespace ffk {
@@ -26,6 +28,19 @@ int fail(int code, char const *fmt, ...) {
   va_end(ap);
   return code;
 }
+
+// Process-wide switches (ffk_set_option).  Each starts from its environment
+// variable, read once when the library is loaded; the dispatch paths read an
+// atomic int, never the environment.
+static int env_int(char const *name) {
+  char const *e = getenv(name);
+  return e != nullptr ? atoi(e) : 0;
+}
+static std::atomic<int> g_option[FFK_OPTION_COUNT] = {
+    {env_int("FFK_GEMM_VARIANT")},
+    {env_int("FFK_LAYER_UNFUSED")},
+};
+int option(int which) { return g_option[which].load(std::memory_order_relaxed); }
 
 // Zero fill as a kernel (not hipMemsetAsync) so that callers may capture the
 // call into a HIP graph.
@@ -49,6 +64,18 @@ using namespace ffk;
 extern "C" {
 
 char const *ffk_last_error(void) { return g_err; }
+
+int ffk_set_option(int which, int value) {
+  FFK_REQUIRE(which >= 0 && which < FFK_OPTION_COUNT, "ffk_set_option: no option %d", which);
+  g_option[which].store(value, std::memory_order_relaxed);
+  return FFK_OK;
+}
+
+int ffk_get_option(int which, int *value) {
+  FFK_REQUIRE(which >= 0 && which < FFK_OPTION_COUNT && value != nullptr, "ffk_get_option: no option %d", which);
+  *value = option(which);
+  return FFK_OK;
+}
 
 int ffk_device_count(int *count) {
   FFK_REQUIRE(count != nullptr, "ffk_device_count: count is NULL");

@@ -80,6 +80,8 @@ int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
                                      size_t workspace_bytes,
                                      // optional: dropped = dropout_backward(dx as stored)
                                      void *dropped = nullptr, float rate = 0.0f,
-                                     uint64_t seed = 0, uint64_t offset = 0);
+                                     uint64_t seed = 0, uint64_t offset = 0,
+                                     // dgamma / dbeta are added to instead of stored
+                                     bool acc_params = false);
 
 }  // namespace ffk

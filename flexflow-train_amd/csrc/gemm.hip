@@ -1030,12 +1030,9 @@ static hipError_t launch_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
   return hipGetLastError();
 }
 
-// FFK_GEMM_VARIANT=128|256|1 forces a tile configuration (1 = the register-
-// staged kernel); unset or 0 = the heuristic.  For tuning runs only.
-static int gemm_variant_override() {
-  char const *e = getenv("FFK_GEMM_VARIANT");  // read per call: tests toggle it
-  return e ? atoi(e) : 0;
-}
+// FFK_OPTION_GEMM_VARIANT = 128|256|1 forces a tile configuration (1 = the
+// register-staged kernel); 0 = the heuristic.  For tuning runs and tests.
+static int gemm_variant_override() { return option(FFK_OPTION_GEMM_VARIANT); }
 
 // Number of K splits for an M x N output of 128x128 tiles: enough to give
 // every CU a workgroup, each split at least 8 k-tiles of 64 long, and no more

@@ -363,7 +363,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void layer_norm_bwd_generic_param_kernel(
     T const *__restrict__ dY, T const *__restrict__ X,
     float const *__restrict__ mean, float const *__restrict__ rstd, T *dgamma,
-    T *dbeta, int64_t M, int N) {
+    T *dbeta, int64_t M, int N, int acc) {
   int const j = blockIdx.x * 256 + threadIdx.x;
   if (j >= N) return;
   float sg = 0.0f, sb = 0.0f;
@@ -373,8 +373,8 @@ __global__ __launch_bounds__(256) void layer_norm_bwd_generic_param_kernel(
     sg += d * xh;
     sb += d;
   }
-  if (dgamma != nullptr) VecIO<T>::store1(dgamma + j, sg);
-  if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, sb);
+  if (dgamma != nullptr) VecIO<T>::store1(dgamma + j, acc ? sg + VecIO<T>::load1(dgamma + j) : sg);
+  if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, acc ? sb + VecIO<T>::load1(dbeta + j) : sb);
 }
 
 constexpr int kLnBwdMaxBlocks = 2 * kNumCU;
@@ -420,7 +420,8 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
                        void *dx, void *dgamma, void *dbeta, int64_t M, int64_t N,
                        void *workspace, size_t workspace_bytes, bool acc,
                        void const *residual = nullptr, void *dropped = nullptr,
-                       DropoutParams const *drop = nullptr, bool fit_blocks_to_workspace = false) {
+                       DropoutParams const *drop = nullptr, bool fit_blocks_to_workspace = false,
+                       bool acc_params = false) {
   constexpr int V = VecIO<T>::kVec;
   T const *RES = static_cast<T const *>(residual);
   if (RES != nullptr) acc = true;
@@ -473,7 +474,7 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
     if (dgamma != nullptr || dbeta != nullptr) {
       // partials are [blocks][2][N]: gamma sums in columns [0, N), beta after
       FFK_HIP(colreduce_launch<T>(st, partials, blocks, (int)(2 * N), (int)N,
-                                  static_cast<T *>(dgamma), static_cast<T *>(dbeta), false));
+                                  static_cast<T *>(dgamma), static_cast<T *>(dbeta), acc_params));
       FFK_CHECK_LAUNCH();
     }
   } else {
@@ -486,7 +487,7 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
       layer_norm_bwd_generic_param_kernel<T>
           <<<(unsigned)ceil_div(N, 256), 256, 0, st>>>(
               DY, X, mean, rstd, static_cast<T *>(dgamma),
-              static_cast<T *>(dbeta), M, (int)N);
+              static_cast<T *>(dbeta), M, (int)N, acc_params ? 1 : 0);
       FFK_CHECK_LAUNCH();
     }
   }
@@ -536,7 +537,7 @@ int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
                                      void *dgamma, void *dbeta, int64_t M,
                                      int64_t N, void *workspace,
                                      size_t workspace_bytes, void *dropped,
-                                     float rate, uint64_t seed, uint64_t offset) {
+                                     float rate, uint64_t seed, uint64_t offset, bool acc_params) {
   FFK_REQUIRE(M > 0 && N > 0 && M < (1ll << 31) && N < (1ll << 31),
               "layer_norm_backward: bad shape");
   FFK_REQUIRE(dy && x && mean && rstd && residual && dx, "layer_norm_backward: NULL tensor");
@@ -548,10 +549,10 @@ int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
   if (dtype == FFK_FLOAT && dropped != nullptr) return FFK_ERR_UNSUPPORTED;  // the dropped copy is bf16 only
   if (dtype == FFK_FLOAT)
     return ln_backward<float>(st, dy, x, mean, rstd, gamma, dx, dgamma, dbeta, M, N,
-                              workspace, workspace_bytes, true, residual);
+                              workspace, workspace_bytes, true, residual, nullptr, nullptr, false, acc_params);
   if (dtype == FFK_BF16)
     return ln_backward<bf16>(st, dy, x, mean, rstd, gamma, dx, dgamma, dbeta, M, N,
-                             workspace, workspace_bytes, true, residual, dropped, &drop);
+                             workspace, workspace_bytes, true, residual, dropped, &drop, false, acc_params);
   return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: dtype %d not supported", dtype);
 }
 
@@ -590,15 +591,16 @@ extern "C" int ffk_layer_norm_backward(
   if (M == 0) return FFK_OK;
   FFK_REQUIRE(M < (1ll << 31), "layer_norm_backward: too many rows");
   FFK_REQUIRE(output_grad && input && mean && rstd, "layer_norm_backward: NULL tensor");
-  bool acc = accumulate_input_grad != 0;
+  bool const acc = (accumulate_input_grad & FFK_LN_ACC_INPUT) != 0;
+  bool const acc_params = (accumulate_input_grad & FFK_LN_ACC_PARAMS) != 0;
   if (dtype == FFK_FLOAT)
     return ln_backward<float>(as_stream(stream), output_grad, input, mean, rstd, gamma,
                               input_grad, gamma_grad, beta_grad, M, N, workspace,
-                              workspace_bytes, acc);
+                              workspace_bytes, acc, nullptr, nullptr, nullptr, false, acc_params);
   if (dtype == FFK_BF16)
     return ln_backward<bf16>(as_stream(stream), output_grad, input, mean, rstd, gamma,
                              input_grad, gamma_grad, beta_grad, M, N, workspace,
-                             workspace_bytes, acc);
+                             workspace_bytes, acc, nullptr, nullptr, nullptr, false, acc_params);
   return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: dtype %d not supported", dtype);
 }
 
@@ -656,13 +658,14 @@ extern "C" int ffk_layer_norm_backward_static(
   // later call has overwritten them.
   ColreduceBatch *const collecting = tl_colreduce_batch;
   tl_colreduce_batch = nullptr;
-  bool const acc = accumulate_input_grad != 0;
+  bool const acc = (accumulate_input_grad & FFK_LN_ACC_INPUT) != 0;
+  bool const acc_params = (accumulate_input_grad & FFK_LN_ACC_PARAMS) != 0;
   if (dtype == FFK_FLOAT) {
     rc = ln_backward<float>(as_stream(stream), output_grad, input, mean, rstd, gamma, input_grad, gamma_grad,
-                            beta_grad, M, N, ptr, kStaticScratchBytes, acc, nullptr, nullptr, nullptr, true);
+                            beta_grad, M, N, ptr, kStaticScratchBytes, acc, nullptr, nullptr, nullptr, true, acc_params);
   } else {
     rc = ln_backward<bf16>(as_stream(stream), output_grad, input, mean, rstd, gamma, input_grad, gamma_grad,
-                           beta_grad, M, N, ptr, kStaticScratchBytes, acc, nullptr, nullptr, nullptr, true);
+                           beta_grad, M, N, ptr, kStaticScratchBytes, acc, nullptr, nullptr, nullptr, true, acc_params);
   }
   tl_colreduce_batch = collecting;
   return rc;

@@ -396,7 +396,7 @@ ComputationGraphInstance create_computation_graph_instance(
   }
 
   // -- neighbouring operators run as one kernel where the library has one that produces the
-  // same bits (FFK_LAYER_UNFUSED=1 switches this off).  The intermediate tensor of a fused pair
+  // same bits (ffk_set_option(FFK_OPTION_LAYER_UNFUSED, 1) switches this off).  The intermediate tensor of a fused pair
   // has that pair's second operator as its only consumer and is never written.
   //   GELU -> Dropout:            forward one kernel at the Dropout, backward one at the GELU
   //   Dropout -> element-wise add: forward one kernel at the add (the backward of the add copies
@@ -412,8 +412,9 @@ ComputationGraphInstance create_computation_graph_instance(
   //                                 the Linear's backward writes the gradient of the GELU's input
   std::vector<int> linear_sum(L, -1), sum_linear(L, -1), linear_gelu(L, -1), gelu_linear(L, -1);
   {
-    char const *off = std::getenv("FFK_LAYER_UNFUSED");
-    bool const enabled = !(off != nullptr && off[0] == '1');
+    int unfused = 0;
+    check_ffk(ffk_get_option(FFK_OPTION_LAYER_UNFUSED, &unfused), "ffk_get_option");
+    bool const enabled = unfused == 0;
     std::vector<int> uses(T, 0);
     std::vector<size_t> consumer(T, 0);
     for (size_t l = 0; l < L; l++) {
@@ -847,13 +848,32 @@ ComputationGraphInstance create_computation_graph_instance(
       f = [=](device_stream_t const &s) {
         check_ffk(ffk_softmax_forward(s.require_gpu(), type, xp, y, outer, size, inner), "Softmax forward");
       };
-      // the true gradient; the reference's backward is a copy (softmax_kernels.cu:68-78)
-      b = [=](device_stream_t const &s) {
-        check_ffk(ffk_softmax_backward(s.require_gpu(), type, y, dy, via_scratch ? scratch : dx, outer, size, inner), "Softmax backward");
-        if (via_scratch) {
-          check_ffk(ffk_element_binary_forward(s.require_gpu(), type, FFK_OP_EW_ADD, dx, scratch, dx, n, n, n), "Softmax backward");
-        }
-      };
+      // The cross-entropy loss kernels write (p - label) * scale into the gradient of the
+      // probabilities they are given (loss_function_kernels.cu:21-57): for a softmax output
+      // that is already the gradient of the softmax INPUT, which is why the reference's
+      // Softmax backward is a copy (softmax_kernels.cu:68-78).  Such a softmax passes the
+      // gradient through; every other softmax gets the true gradient.
+      bool feeds_cross_entropy = false;
+      if (loss.has_value() && loss->logit_tensor == layer.outputs[0]) {
+        LossFunction const kind = get_loss_function(loss->loss_attrs);
+        feeds_cross_entropy = kind == LossFunction::SPARSE_CATEGORICAL_CROSSENTROPY || kind == LossFunction::CATEGORICAL_CROSSENTROPY;
+      }
+      if (feeds_cross_entropy) {
+        b = [=](device_stream_t const &s) {
+          if (via_scratch) {
+            check_ffk(ffk_element_binary_forward(s.require_gpu(), type, FFK_OP_EW_ADD, dx, dy, dx, n, n, n), "Softmax backward");
+          } else {
+            check_ffk(ffk_softmax_backward_copy(s.require_gpu(), type, dy, dx, (size_t)n), "Softmax backward");
+          }
+        };
+      } else {
+        b = [=](device_stream_t const &s) {
+          check_ffk(ffk_softmax_backward(s.require_gpu(), type, y, dy, via_scratch ? scratch : dx, outer, size, inner), "Softmax backward");
+          if (via_scratch) {
+            check_ffk(ffk_element_binary_forward(s.require_gpu(), type, FFK_OP_EW_ADD, dx, scratch, dx, n, n, n), "Softmax backward");
+          }
+        };
+      }
     } else if (auto const *a = std::get_if<EmbeddingAttrs>(&oa)) {
       tensor_guid_t x = layer.inputs[0];
       int const itype = dt(shape_of(x).data_type), otype = dt(a->data_type), aggr = aggr_code(a->aggr);

@@ -54,12 +54,16 @@ static int g_failed = 0, g_checks = 0;
 static void run(char const *name, std::function<void()> const &f) {
   printf("TEST_CASE %s\n", name);
   fflush(stdout);
+  int const failed_before = g_failed;
   try {
     f();
   } catch (std::exception const &e) {
     g_failed++;
     printf("  exception: %s\n", e.what());
   }
+  // one line per case, so a harness can report every case on its own
+  printf("CASE_RESULT %s\n", g_failed == failed_before ? "ok" : "FAILED");
+  fflush(stdout);
 }
 
 static TensorShape shape(std::vector<int64_t> dims, DataType dtype) { return TensorShape{TensorDims{dims}, dtype}; }
@@ -606,6 +610,109 @@ static void gpu_tests() {
                                                    device_handle_t::for_cpu(), make_device_id_t_from_idx(0, DeviceType::CPU)));
   });
 
+  // The reference transformer ends in dense -> softmax with a sparse categorical cross-entropy
+  // on the softmax output (lib/models/src/models/transformer/transformer.cc:160-170).  The loss
+  // kernel writes (p - onehot) / batch into the gradient of p, which is the cross-entropy's
+  // gradient at the softmax INPUT: the softmax in front of the loss must pass it through.
+  run("Step driver: Dense -> Softmax -> sparse categorical CE; the Dense output's gradient is (p - y) / batch", [&] {
+    int64_t batch = 12, in_dim = 24, classes = 10;
+    ComputationGraphBuilder b;
+    tensor_guid_t x = b.create_input(shape({batch, in_dim}, DataType::FLOAT), CreateGrad::NO);
+    tensor_guid_t z = b.dense(x, (int)classes, std::nullopt, true);
+    tensor_guid_t prob = b.softmax(z);
+    auto xs = random_vec(batch * in_dim, 40), w = random_vec(classes * in_dim, 41, -0.5f, 0.5f), bias = random_vec(classes, 42);
+    std::vector<int> sparse(batch);
+    for (int64_t i = 0; i < batch; i++) sparse[i] = (int)((i * 7 + 3) % classes);
+    Allocator cpu = create_local_cpu_memory_allocator();
+    GenericTensorAccessorW hl = cpu.allocate_tensor(shape({batch}, DataType::INT32));
+    memcpy(hl.ptr, sparse.data(), sparse.size() * 4);
+    GenericTensorAccessorW LABEL = copy_tensor_accessor_w(hl, gpu);
+    OptimizerAttrs optimizer = SGDOptimizerAttrs{0.1, 0.0, false, 0.0};
+    device_id_t device_idx = make_device_id_t_from_idx(0, DeviceType::GPU);
+    ComputationGraphInstance instance = create_computation_graph_instance(
+        b.computation_graph, optimizer, LossConfig{SparseCategoricalCrossEntropyLossAttrs{false}, LABEL, prob}, {}, gpu,
+        ProfilingSettings{0, 0}, handle, device_idx);
+    auto put = [&](tensor_guid_t t, std::vector<float> const &v) {
+      GenericTensorAccessorW h = cpu.allocate_tensor(instance.get_tensor_accessor(t).shape);
+      memcpy(h.ptr, v.data(), v.size() * 4);
+      copy_accessor_data_to_l_from_r(instance.get_tensor_accessor(t), h);
+    };
+    std::vector<tensor_guid_t> weights = b.get_weights_of(z);
+    put(x, xs); put(weights.at(0), w); put(weights.at(1), bias);
+    perform_all_passes_for_computation_graph_instance(instance, ProfilingSettings{0, 0}, handle, device_idx);
+    std::vector<float> zs(batch * classes), p(zs.size()), dz(zs.size()), dw(w.size()), db(bias.size());
+    orc_linear_forward(-1, xs.data(), zs.data(), w.data(), bias.data(), batch, in_dim, classes);
+    orc_softmax_forward(zs.data(), p.data(), batch, classes, 1);
+    orc_sparse_cce_loss_backward(dz.data(), p.data(), sparse.data(), batch * classes, batch, classes, 1, 1.0f / batch);
+    CHECK(close(to_host(instance.get_tensor_accessor(prob)), p, 1e-5));
+    CHECK(close(to_host(*instance.get_gradient_accessor(z)), dz, 1e-5));
+    // every row of (p - onehot) sums to zero: a softmax gradient taken on top of it would not leave it so
+    orc_linear_backward(-1, 0, zs.data(), dz.data(), xs.data(), nullptr, w.data(), dw.data(), db.data(), batch, in_dim, classes);
+    std::vector<float> w1 = w, b1 = bias;
+    orc_sgd_update(0.1f, 0.0f, 0, 0.0f, dw.data(), (int64_t)w.size(), 1, w1.data(), nullptr);
+    orc_sgd_update(0.1f, 0.0f, 0, 0.0f, db.data(), (int64_t)bias.size(), 1, b1.data(), nullptr);
+    CHECK(close(to_host(instance.get_tensor_accessor(weights.at(0))), w1, 1e-5));
+    CHECK(close(to_host(instance.get_tensor_accessor(weights.at(1))), b1, 1e-5));
+    // an interior softmax (mean-squared error behind it) keeps the true gradient
+    ComputationGraphBuilder b2;
+    tensor_guid_t x2 = b2.create_input(shape({batch, classes}, DataType::FLOAT), CreateGrad::YES);
+    tensor_guid_t p2 = b2.softmax(x2);
+    auto target = random_vec(batch * classes, 43, 0.0f, 1.0f);
+    auto TARGET = device_accessor(gpu, shape({batch, classes}, DataType::FLOAT), target);
+    ComputationGraphInstance inst2 = create_computation_graph_instance(
+        b2.computation_graph, optimizer, LossConfig{NonconfigurableLossAttrs{LossFunction::MEAN_SQUARED_ERROR_AVG_REDUCE}, TARGET, p2},
+        {}, gpu, ProfilingSettings{0, 0}, handle, device_idx);
+    GenericTensorAccessorW hx = cpu.allocate_tensor(inst2.get_tensor_accessor(x2).shape);
+    memcpy(hx.ptr, zs.data(), zs.size() * 4);
+    copy_accessor_data_to_l_from_r(inst2.get_tensor_accessor(x2), hx);
+    perform_all_passes_for_computation_graph_instance(inst2, ProfilingSettings{0, 0}, handle, device_idx);
+    std::vector<float> dp = to_host(*inst2.get_gradient_accessor(p2)), dx_want(zs.size());
+    orc_softmax_backward(p.data(), dp.data(), dx_want.data(), batch, classes, 1);
+    CHECK(close(to_host(*inst2.get_gradient_accessor(x2)), dx_want, 1e-5));
+  });
+
+  // Two Linear layers that share one bias tensor: both bias gradients are column reductions
+  // whose last step the backward pass collects into one launch; they write the same tensor.
+  run("Step driver: a bias shared by two Linear layers receives both gradients", [&] {
+    int64_t batch = 64, dim = 96;
+    ComputationGraph cg = make_empty_computation_graph();
+    tensor_guid_t x = add_input_layer(cg, shape({batch, dim}, DataType::FLOAT)).outputs.at(0);
+    tensor_guid_t w1 = add_weight_layer(cg, shape({dim, dim}, DataType::FLOAT)).outputs.at(0);
+    tensor_guid_t w2 = add_weight_layer(cg, shape({dim, dim}, DataType::FLOAT)).outputs.at(0);
+    tensor_guid_t bias = add_weight_layer(cg, shape({dim}, DataType::FLOAT)).outputs.at(0);
+    LayerAttrs lin{LinearAttrs{(int)dim, true, DataType::FLOAT, std::nullopt, std::nullopt}, std::nullopt};
+    tensor_guid_t h = add_layer(cg, lin, {x}, {w1, bias}).outputs.at(0);
+    tensor_guid_t y = add_layer(cg, lin, {h}, {w2, bias}).outputs.at(0);
+    auto xs = random_vec(batch * dim, 50), a1 = random_vec(dim * dim, 51, -0.2f, 0.2f), a2 = random_vec(dim * dim, 52, -0.2f, 0.2f),
+         bs = random_vec(dim, 53), target = random_vec(batch * dim, 54);
+    auto TARGET = device_accessor(gpu, shape({batch, dim}, DataType::FLOAT), target);
+    device_id_t device_idx = make_device_id_t_from_idx(0, DeviceType::GPU);
+    ComputationGraphInstance instance = create_computation_graph_instance(
+        cg, OptimizerAttrs{SGDOptimizerAttrs{0.0, 0.0, false, 0.0}},
+        LossConfig{NonconfigurableLossAttrs{LossFunction::MEAN_SQUARED_ERROR_AVG_REDUCE}, TARGET, y}, {}, gpu,
+        ProfilingSettings{0, 0}, handle, device_idx);
+    Allocator cpu = create_local_cpu_memory_allocator();
+    auto put = [&](tensor_guid_t t, std::vector<float> const &v) {
+      GenericTensorAccessorW hh = cpu.allocate_tensor(instance.get_tensor_accessor(t).shape);
+      memcpy(hh.ptr, v.data(), v.size() * 4);
+      copy_accessor_data_to_l_from_r(instance.get_tensor_accessor(t), hh);
+    };
+    put(x, xs); put(w1, a1); put(w2, a2); put(bias, bs);
+    std::vector<float> hs(batch * dim), ys(batch * dim), dy(batch * dim), dh(batch * dim), dw(dim * dim), db2(dim), db1(dim);
+    orc_linear_forward(-1, xs.data(), hs.data(), a1.data(), bs.data(), batch, dim, dim);
+    orc_linear_forward(-1, hs.data(), ys.data(), a2.data(), bs.data(), batch, dim, dim);
+    for (int step = 0; step < 2; step++) {  // the second step sees what the first left in the gradient
+      perform_all_passes_for_computation_graph_instance(instance, ProfilingSettings{0, 0}, handle, device_idx);
+      dy = to_host(*instance.get_gradient_accessor(y));
+      orc_linear_backward(-1, 0, ys.data(), dy.data(), hs.data(), dh.data(), a2.data(), dw.data(), db2.data(), batch, dim, dim);
+      orc_linear_backward(-1, 0, hs.data(), dh.data(), xs.data(), nullptr, a1.data(), dw.data(), db1.data(), batch, dim, dim);
+      std::vector<float> want(dim);
+      for (int64_t j = 0; j < dim; j++) want[j] = db1[j] + db2[j];
+      CHECK(contains_non_zero(db1) && contains_non_zero(db2));
+      CHECK(close(to_host(*instance.get_gradient_accessor(bias)), want, 1e-5));
+    }
+  });
+
   // The encoder layer of lib/models/src/models/transformer/transformer.cc:18-67 built through the
   // builder (BF16), a cast and a mean-squared-error loss behind it, Adam.  One step of the
   // instance must equal, bit for bit, the same operators called by hand with every gradient
@@ -1008,7 +1115,7 @@ static void gpu_tests() {
   });
   run("Step driver: fused operator pairs give the bits of one kernel per operator", [&] {
     // x -> dense -> GELU -> dropout -> dense -> dropout -> (+ x) -> cast -> loss; two instances of the
-    // same graph, one created with FFK_LAYER_UNFUSED=1, stepped twice each (the second step uses
+    // same graph, one created with FFK_OPTION_LAYER_UNFUSED set, stepped twice each (the second step uses
     // the next dropout offsets)
     // ... at a size whose Linears run the two element-wise launches themselves, and at one where
     // the library applies the pairs on the GEMMs' tile stores
@@ -1035,12 +1142,12 @@ static void gpu_tests() {
       tensor_guid_t x, logits;
       std::vector<tensor_guid_t> ws;
       build(cgb, x, logits, ws);
-      if (unfused) setenv("FFK_LAYER_UNFUSED", "1", 1);
+      if (unfused) ffk_set_option(FFK_OPTION_LAYER_UNFUSED, 1);
       ComputationGraphInstance inst = create_computation_graph_instance(
           cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{0.05, 0.9, false, 0.0}},
           LossConfig{NonconfigurableLossAttrs{LossFunction::MEAN_SQUARED_ERROR_AVG_REDUCE}, LABEL, logits}, {}, gpu,
           ProfilingSettings{0, 0}, handle, dev);
-      if (unfused) unsetenv("FFK_LAYER_UNFUSED");
+      if (unfused) ffk_set_option(FFK_OPTION_LAYER_UNFUSED, 0);
       // the GELU of dense(.., GELU) is its own layer: find the weights by layer order (same in both graphs)
       int seed = 80;
       for (size_t t = 0; t < cgb.computation_graph.tensors.size(); t++) {

@@ -121,6 +121,18 @@ int ffk_event_record(ffk_event_t ev, ffk_stream_t stream);
 int ffk_event_synchronize(ffk_event_t ev);
 int ffk_event_elapsed_ms(ffk_event_t start, ffk_event_t stop, float *ms);
 
+/* Process-wide switches for tuning runs and tests; no counterpart in the
+ * reference.  Each starts from the environment variable of the same name,
+ * read once when the library is loaded.
+ *   FFK_OPTION_GEMM_VARIANT (FFK_GEMM_VARIANT): 0 = the dispatch heuristic;
+ *     128 / 256 force that pipelined bf16 tile, 1 the register-staged kernel.
+ *   FFK_OPTION_LAYER_UNFUSED (FFK_LAYER_UNFUSED): != 0 makes the encoder-layer
+ *     entry points (and a step-driver instance created while it is set) run
+ *     one kernel per operator.                                               */
+enum { FFK_OPTION_GEMM_VARIANT = 0, FFK_OPTION_LAYER_UNFUSED = 1, FFK_OPTION_COUNT = 2 };
+int ffk_set_option(int which, int value);
+int ffk_get_option(int which, int *value);
+
 /* ------------------------------------------------------------------------ */
 /* Linear -- replaces Kernels::Linear::gpu_forward_kernel / gpu_backward_kernel
  * (lib/kernels/include/kernels/linear_kernels_gpu.h:22-43; CUDA body
@@ -214,12 +226,15 @@ int ffk_element_binary_backward(ffk_stream_t stream, int dtype, int op_type,
  * formula of LayerNormBackwardCUDAKenrel (layer_norm_kernels.cu:163-181)
  * which the reference defines but never launches.
  * workspace: ffk_layer_norm_backward_workspace_bytes(M, N) bytes (partial
- * column sums for dgamma/dbeta); dgamma/dbeta are always overwritten.        */
+ * column sums for dgamma/dbeta).  accumulate_input_grad is a bit mask:
+ * FFK_LN_ACC_INPUT adds into input_grad, FFK_LN_ACC_PARAMS adds into
+ * gamma_grad / beta_grad (0: both are stored).                               */
 /* ------------------------------------------------------------------------ */
 int ffk_layer_norm_forward(ffk_stream_t stream, int dtype, void const *input,
                            void *output, void const *gamma, void const *beta,
                            float *mean, float *rstd, int64_t M, int64_t N,
                            float eps);
+enum { FFK_LN_ACC_INPUT = 1, FFK_LN_ACC_PARAMS = 2 };
 size_t ffk_layer_norm_backward_workspace_bytes(int64_t M, int64_t N);
 int ffk_layer_norm_backward(ffk_stream_t stream, int dtype,
                             void const *output_grad, void const *input,

@@ -86,12 +86,12 @@ def test_encoder_layer_config2_shape_runs_and_is_deterministic(ffk):
 
 @pytest.mark.parametrize("shape", ["small", "config2"])
 @pytest.mark.parametrize("pre_ln,gelu", [(True, True), (False, True), (False, False)])
-def test_fused_layer_equals_operator_sequence(ffk, shape, pre_ln, gelu, monkeypatch):
+def test_fused_layer_equals_operator_sequence(ffk, shape, pre_ln, gelu):
     """The layer entry points fuse neighbouring ops (GELU into the GEMM
     epilogue, dropout into the residual add, dropout backward into GELU
-    backward, the residual add into LayerNorm backward).  With
-    FFK_LAYER_UNFUSED=1 the same entry points run one kernel per operator;
-    both must give the same bits."""
+    backward, the residual add into LayerNorm backward).  With the option
+    FFK_OPTION_LAYER_UNFUSED set the same entry points run one kernel per
+    operator; both must give the same bits."""
     if shape == "small":
         cfg = dict(batch=2, seq=64, d_model=128, heads=2, d_ff=256)
     else:
@@ -102,9 +102,11 @@ def test_fused_layer_equals_operator_sequence(ffk, shape, pre_ln, gelu, monkeypa
     params = make_params(g, cfg, bf16_round)
     x = bf16_round(g.standard_normal((cfg["batch"], cfg["seq"], cfg["d_model"])))
     dy = bf16_round(g.standard_normal(x.shape))
-    monkeypatch.setenv("FFK_LAYER_UNFUSED", "1")
-    y_u, dx_u, g_u = run_device(ffk, cfg, params, x, dy)
-    monkeypatch.setenv("FFK_LAYER_UNFUSED", "0")
+    ffk.set_option(ffk.OPTION_LAYER_UNFUSED, 1)
+    try:
+        y_u, dx_u, g_u = run_device(ffk, cfg, params, x, dy)
+    finally:
+        ffk.set_option(ffk.OPTION_LAYER_UNFUSED, 0)
     y_f, dx_f, g_f = run_device(ffk, cfg, params, x, dy)
     assert np.array_equal(y_u, y_f)
     assert np.array_equal(dx_u, dx_f)
@@ -112,10 +114,10 @@ def test_fused_layer_equals_operator_sequence(ffk, shape, pre_ln, gelu, monkeypa
         assert np.array_equal(g_u[k], g_f[k]), k
 
 
-def test_split_k_weight_gradient_matches_unsplit(ffk, monkeypatch):
+def test_split_k_weight_gradient_matches_unsplit(ffk):
     """At config 2 the attention output projection's weight gradient
     ([1024 x 1024] output, reduction over 4096 tokens) runs as a split-K GEMM
-    with fp32 partial sums.  FFK_GEMM_VARIANT=128 forces the same tile
+    with fp32 partial sums.  FFK_OPTION_GEMM_VARIANT = 128 forces the same tile
     configuration without the split; the two differ only in fp32 summation
     order, so the bf16 results agree to a rounding step."""
     cfg = dict(batch=8, seq=512, d_model=1024, heads=16, d_ff=4096, p=0.1, seed=3, eps=1e-5,
@@ -125,9 +127,11 @@ def test_split_k_weight_gradient_matches_unsplit(ffk, monkeypatch):
     params = make_params(g, cfg, bf16_round)
     x = bf16_round(g.standard_normal((8, 512, 1024)))
     dy = bf16_round(g.standard_normal(x.shape))
-    monkeypatch.setenv("FFK_GEMM_VARIANT", "128")
-    _, _, g_plain = run_device(ffk, cfg, params, x, dy)
-    monkeypatch.delenv("FFK_GEMM_VARIANT")
+    ffk.set_option(ffk.OPTION_GEMM_VARIANT, 128)
+    try:
+        _, _, g_plain = run_device(ffk, cfg, params, x, dy)
+    finally:
+        ffk.set_option(ffk.OPTION_GEMM_VARIANT, 0)
     _, _, g_split = run_device(ffk, cfg, params, x, dy)
     E = 1024
     wo_plain = g_plain["attn_weight"][3 * E * E:]
@@ -153,3 +157,43 @@ def test_stored_weight_gradients_equal_added_into_zero(ffk, pre_ln, gelu):
     for k in g0:
         assert np.any(g0[k] != 0), k
         assert np.array_equal(g0[k], g1[k]), k
+
+
+@pytest.mark.parametrize("pre_ln,gelu", [(True, True), (False, False)])
+@pytest.mark.parametrize("fused", [True, False])
+def test_weight_gradients_add_up_over_two_backward_calls(ffk, pre_ln, gelu, fused):
+    """Without overwrite_weight_grads every weight gradient is added into (micro-batch
+    accumulation): two backward calls leave twice one call's gradient in every tensor,
+    the LayerNorm parameters included."""
+    cfg = dict(batch=2, seq=48, d_model=128, heads=2, d_ff=256, p=0.1, seed=5, eps=1e-5,
+               scale=1.0 / 8.0, causal=False, pre_ln=pre_ln, gelu=gelu)
+    say("weight gradients over two calls", cfg, "fused", fused)
+    g = rng(29)
+    params = make_params(g, cfg, bf16_round)
+    x = bf16_round(g.standard_normal((cfg["batch"], cfg["seq"], cfg["d_model"])))
+    dy = bf16_round(g.standard_normal(x.shape))
+    desc = ffk.EncoderLayerDesc(cfg["batch"], cfg["seq"], cfg["d_model"], cfg["heads"], cfg["d_ff"],
+                                cfg["p"], cfg["seed"], cfg["eps"], cfg["scale"], 0, int(pre_ln),
+                                ffk.ACT_GELU if gelu else ffk.ACT_RELU, 0)
+    wt = {k: to_dev(v, torch, torch.float32).to(BT) for k, v in params.items()}
+    xd, dyd = to_dev(x, torch, BT), to_dev(dy, torch, BT)
+    y, dx = torch.empty_like(xd), torch.empty_like(xd)
+    ws = ffk.encoder_layer_workspace(desc, ffk.BF16)
+    W = ffk.encoder_layer_params(wt)
+    ffk.set_option(ffk.OPTION_LAYER_UNFUSED, 0 if fused else 1)
+    try:
+        ffk.encoder_layer_forward(desc, W, xd, y, ws)
+        once = {k: torch.zeros_like(v) for k, v in wt.items()}
+        ffk.encoder_layer_backward(desc, W, ffk.encoder_layer_params(once), xd, dyd, dx, ws)
+        twice = {k: torch.zeros_like(v) for k, v in wt.items()}
+        G2 = ffk.encoder_layer_params(twice)
+        ffk.encoder_layer_backward(desc, W, G2, xd, dyd, dx, ws)
+        ffk.encoder_layer_backward(desc, W, G2, xd, dyd, dx, ws)
+    finally:
+        ffk.set_option(ffk.OPTION_LAYER_UNFUSED, 0)
+    torch.cuda.synchronize()
+    for k in once:
+        a, b = to_np(once[k]), to_np(twice[k])
+        assert np.any(a != 0), k
+        # g + g is exact in bf16 up to the rounding of the second addition's operand
+        assert_close(b, 2 * a, 1e-2, "twice " + k)
