@@ -245,6 +245,36 @@ def test_attention_against_torch_sdpa(oracle, causal):
         assert np.array_equal(o2[:, :6], o[:, :6])
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_bf16_mode_against_torch_with_rounded_probabilities(oracle, causal):
+    """bf16_mode is the mode every bf16 device test compares with: the unnormalised
+    probabilities exp(s - max) are rounded to bf16 before the PV product, the row sum is taken
+    over the unrounded ones, and the output is rounded to bf16.  The same composition, step by
+    step, in torch fp64."""
+    g = rng(19)
+    B, Sq, Skv, H, D = 2, 9, 13, 2, 8
+    def bf(a):
+        return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).to(torch.float32).numpy()
+    q, k, v = (bf(g.standard_normal(s)) for s in ((B, Sq, H, D), (B, Skv, H, D), (B, Skv, H, D)))
+    scale = 0.4
+    o, lse = oracle.attention_forward(q, k, v, scale, causal, bf16_mode=True)
+    qt, kt, vt = (t64(a).transpose(1, 2) for a in (q, k, v))
+    s = torch.einsum("bhqd,bhkd->bhqk", qt, kt) * scale
+    if causal:  # key j visible to query i iff j <= i
+        s = s.masked_fill(torch.triu(torch.ones(Sq, Skv, dtype=torch.bool), 1), float("-inf"))
+    p = torch.exp(s - s.max(dim=-1, keepdim=True).values)
+    p_rounded = p.to(torch.float32).to(torch.bfloat16).to(torch.float64)
+    want = torch.einsum("bhqk,bhkd->bhqd", p_rounded, vt) / p.sum(dim=-1, keepdim=True)
+    want = want.to(torch.float32).to(torch.bfloat16).to(torch.float32).transpose(1, 2).numpy()
+    # the same bits, except where an fp64 value sits within an fp32 rounding of a bf16 tie
+    diff = np.abs(o - want)
+    assert (diff > 0).mean() < 0.01 and diff.max() <= np.abs(want).max() * 2.0 ** -7
+    assert np.allclose(lse, torch.logsumexp(s, -1).numpy(), atol=1e-5)
+    # and it is not the unrounded mode
+    o32, _ = oracle.attention_forward(q, k, v, scale, causal, bf16_mode=False)
+    assert not np.array_equal(o, o32)
+
+
 def test_mha_against_torch_composition(oracle):
     g = rng(10)
     B, Sq, Skv, H, E, Dh = 2, 6, 7, 3, 10, 4
