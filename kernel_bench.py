@@ -1,6 +1,6 @@
 """Per-kernel measurements at the shapes of the baseline configurations.
 
-    python flexflow-train_amd/kernel_bench.py [group ...]
+    python kernel_bench.py [group ...]
 
 Groups: gemm (config 2 and config 5 projection GEMMs), bandwidth (config 3:
 LayerNorm, Softmax, ElementBinary, Dropout, plus GELU), embedding (config 4:
@@ -21,7 +21,8 @@ import numpy as np
 import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-_spec = importlib.util.spec_from_file_location("flexflow_train_amd", os.path.join(HERE, "__init__.py"))
+_spec = importlib.util.spec_from_file_location("flexflow_train_amd",
+                                               os.path.join(HERE, "flexflow-train_amd", "__init__.py"))
 ffk = importlib.util.module_from_spec(_spec)
 sys.modules["flexflow_train_amd"] = ffk
 _spec.loader.exec_module(ffk)
