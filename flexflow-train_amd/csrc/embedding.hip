@@ -11,9 +11,9 @@
 // Indices outside [0, num_entries) are skipped (the reference reads or writes
 // out of bounds for them).
 #include "ffk_common.h"
+#include "radix_sort.h"
 #include <cstdlib>
 #include <cstring>
-#include <rocprim/device/device_radix_sort.hpp>
 
 namespace ffk {
 
@@ -143,24 +143,12 @@ __global__ __launch_bounds__(kEmbThreads) void embedding_bwd_atomic_kernel(
 // Sorted scatter-add.  The atomic kernel above is bound by the rate at which
 // the memory side retires fp32 atomics (about 0.7 TB/s of payload measured on
 // MI355X, far below HBM).  With scratch from the caller the lookups are sorted
-// by row id first (stable radix sort of (id, lookup) pairs); equal ids then
+// by row id first (the stable radix sort of radix_sort.h); equal ids then
 // form runs, a walker sums the gradient rows of a run in registers and adds the
 // sum to the weight-gradient row with ordinary loads and stores, because a run
 // that lies inside one walker's chunk is touched by nobody else.  Only runs
 // that cross a chunk border (at most two per walker) go through atomics.
 constexpr int kEmbChunk = 16;  // sorted positions per walker
-
-template <typename IT>
-__global__ __launch_bounds__(256) void embedding_sort_keys_kernel(
-    IT const *__restrict__ idx, uint32_t *keys, uint32_t *vals, int64_t n,
-    int64_t num_entries) {
-  int64_t const i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  int64_t const r = (int64_t)idx[i];
-  // invalid ids get the key num_entries: they sort behind every valid row
-  keys[i] = (uint64_t)r < (uint64_t)num_entries ? (uint32_t)r : (uint32_t)num_entries;
-  vals[i] = (uint32_t)i;
-}
 
 template <typename GT>
 __device__ __forceinline__ void load_grad4(GT const *p, float (&v)[4]);
@@ -423,9 +411,10 @@ __global__ __launch_bounds__(kEmbBlockThreads) void embedding_bwd_sorted_block_k
   }
 }
 
-// Scratch layout: keys in | keys out | lookups in | lookups out | sort scratch
+// Scratch layout: keys A | keys B | lookups A | lookups B | digit table of the sort
 struct EmbSortLayout {
-  size_t keys_in, keys_out, vals_in, vals_out, temp, temp_bytes, total;
+  size_t keys_a, keys_b, vals_a, vals_b, table, total;
+  RadixSortPlan plan;
 };
 
 static unsigned key_bits(int64_t num_entries) {
@@ -436,19 +425,14 @@ static unsigned key_bits(int64_t num_entries) {
 
 static bool emb_sort_layout(int64_t n, int64_t num_entries, EmbSortLayout &L) {
   if (n <= 0 || n >= (1ll << 31) || num_entries >= 0xffffffffll) return false;
-  size_t temp = 0;
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, (uint32_t *)nullptr, (uint32_t *)nullptr,
-                                           (uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n, 0u,
-                                           key_bits(num_entries), (hipStream_t)0);
-  if (e != hipSuccess) return false;
+  L.plan = radix_sort_plan(n, key_bits(num_entries));
   size_t const arr = ((size_t)n * 4 + 255) & ~(size_t)255;
-  L.keys_in = 0;
-  L.keys_out = arr;
-  L.vals_in = 2 * arr;
-  L.vals_out = 3 * arr;
-  L.temp = 4 * arr;
-  L.temp_bytes = temp;
-  L.total = 4 * arr + ((temp + 255) & ~(size_t)255);
+  L.keys_a = 0;
+  L.keys_b = arr;
+  L.vals_a = 2 * arr;
+  L.vals_b = 3 * arr;
+  L.table = 4 * arr;
+  L.total = 4 * arr + ((L.plan.table_bytes + 255) & ~(size_t)255);
   return true;
 }
 
@@ -492,16 +476,11 @@ static int emb_backward(hipStream_t st, void const *indices, void const *dy,
                       emb_sort_layout(lookups, num_entries, L) && L.total <= workspace_bytes;
   if (sorted) {
     uint8_t *ws = static_cast<uint8_t *>(workspace);
-    uint32_t *keys_in = reinterpret_cast<uint32_t *>(ws + L.keys_in);
-    uint32_t *keys_out = reinterpret_cast<uint32_t *>(ws + L.keys_out);
-    uint32_t *vals_in = reinterpret_cast<uint32_t *>(ws + L.vals_in);
-    uint32_t *vals_out = reinterpret_cast<uint32_t *>(ws + L.vals_out);
-    embedding_sort_keys_kernel<IT><<<(unsigned)ceil_div(lookups, 256), 256, 0, st>>>(
-        static_cast<IT const *>(indices), keys_in, vals_in, lookups, num_entries);
-    FFK_CHECK_LAUNCH();
-    size_t temp = L.temp_bytes;
-    FFK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp, keys_in, keys_out, vals_in, vals_out,
-                                      (size_t)lookups, 0u, key_bits(num_entries), st));
+    uint32_t *keys_out = nullptr, *vals_out = nullptr;
+    FFK_HIP(radix_sort_lookups<IT>(st, static_cast<IT const *>(indices), lookups, num_entries, L.plan,
+                                   reinterpret_cast<uint32_t *>(ws + L.keys_a), reinterpret_cast<uint32_t *>(ws + L.keys_b),
+                                   reinterpret_cast<uint32_t *>(ws + L.vals_a), reinterpret_cast<uint32_t *>(ws + L.vals_b),
+                                   reinterpret_cast<uint32_t *>(ws + L.table), &keys_out, &vals_out));
     GT const *G = static_cast<GT const *>(dy);
     int64_t const walkers = ceil_div(lookups, kEmbChunk);
 #define FFK_EMB_SORTED(LPR_, CPL_)                                             \

@@ -167,7 +167,10 @@ def test_embedding_config4_dlrm_table(ffk, oracle):
                      ("atomic", dict(workspace=False))):
         dw = torch.zeros((V, D), device="cuda")
         ffk.embedding_backward(idd, dy, dw, aggr=0, **kw)
-        assert_close(to_np(dw[tidx]), want_rows, FP32_RTOL, "dW touched rows " + mode)
+        # the hottest row receives about 50 000 gradient rows; with atomics they are added one
+        # by one in fp32 in arrival order, whose rounding error grows with the run length
+        # (the sorted paths add partial sums of 16), so that path gets 1e-4
+        assert_close(to_np(dw[tidx]), want_rows, 1e-4 if mode == "atomic" else FP32_RTOL, "dW touched rows " + mode)
         assert float(dw.double().sum()) == pytest.approx(float(dy.double().sum()) * bag, rel=1e-6)
         assert int((dw != 0).any(dim=1).sum()) <= touched.size
 
