@@ -21,7 +21,7 @@ namespace ffk {
 
 // PRE: the row normalised is residual + dropout(X), computed here, rounded to T where the two
 // separate operators would have stored it, and written to `summed` as well.
-template <typename T, int EPT, int WPR, bool PRE = false>
+template <typename T, int EPT, int WPR, bool PRE = false, bool STREAM = false>
 __global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_kernel(
     T const *__restrict__ X, T *__restrict__ Y, T const *__restrict__ gamma,
     T const *__restrict__ beta, float *__restrict__ mean,
@@ -45,7 +45,11 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_kernel(
   for (int j = 0; j < EPT; j++) {
     int v = lane + j * LANES;
     if (v < nvec) {
-      VecIO<T>::load(xr + (int64_t)v * V, x[j]);
+      if (STREAM) {
+        VecIO<T>::load_stream(xr + (int64_t)v * V, x[j]);
+      } else {
+        VecIO<T>::load(xr + (int64_t)v * V, x[j]);
+      }
       if constexpr (PRE) {
         static_assert(V == 4 || V == 8, "a lane's vector is a Philox block or half of one");
         if (row_ok) {
@@ -114,7 +118,11 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_kernel(
         float bv = beta != nullptr ? b[e] : 0.0f;
         y[e] = xh * gv + bv;
       }
-      VecIO<T>::store(yr + (int64_t)v * V, y);
+      if (STREAM) {
+        VecIO<T>::store_stream(yr + (int64_t)v * V, y);
+      } else {
+        VecIO<T>::store(yr + (int64_t)v * V, y);
+      }
     }
   }
 }
@@ -160,7 +168,8 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
     float const *__restrict__ mean, float const *__restrict__ rstd,
     T const *__restrict__ gamma, T *dX, float *__restrict__ partials,
     int64_t M, int N, T const *res, T *__restrict__ dropped = nullptr,
-    DropoutParams drop = DropoutParams{}) {
+    DropoutParams drop = DropoutParams{}, bool stream_out = false) {
+  // stream_out: dX is too large to be found in cache by its reader; store it past the caches.
   // ACC with res == nullptr: dX += gradient (one rounding).  ACC with res set:
   // dX = res + gradient rounded to the storage type, i.e. what a separate
   // element-wise add of res to the stored gradient would give.
@@ -263,7 +272,11 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
             if (ACC && res != nullptr) val = storage_round<T>(val);
             o[e] = ACC ? o[e] + val : val;
           }
-          VecIO<T>::store(dst, o);
+          if (stream_out) {
+            VecIO<T>::store_stream(dst, o);
+          } else {
+            VecIO<T>::store(dst, o);
+          }
           if constexpr (DROP) {
             static_assert(V == 4 || V == 8, "a lane's vector is a Philox block or half of one");
             int64_t const at = row * (int64_t)N + (int64_t)v * V;
@@ -401,9 +414,16 @@ static int ln_forward(hipStream_t st, void const *x, void *y, void const *gamma,
              pick_row_config_small(N / V, ept, wpr);
   if (vec) {
     int64_t blocks = ceil_div(M, 4 / wpr);
+    bool const stream = stream_past_caches(M * N, sizeof(T));
 #define CALL(E, W)                                                             \
-  layer_norm_fwd_kernel<T, E, W><<<(unsigned)blocks, kRowThreads, 0, st>>>(    \
-      X, Y, G, Bt, mean, rstd, M, (int)N, eps)
+  do {                                                                         \
+    if (stream)                                                                \
+      layer_norm_fwd_kernel<T, E, W, false, true><<<(unsigned)blocks, kRowThreads, 0, st>>>( \
+          X, Y, G, Bt, mean, rstd, M, (int)N, eps);                            \
+    else                                                                       \
+      layer_norm_fwd_kernel<T, E, W><<<(unsigned)blocks, kRowThreads, 0, st>>>( \
+          X, Y, G, Bt, mean, rstd, M, (int)N, eps);                            \
+  } while (0)
     FFK_ROW_DISPATCH_SMALL(ept, wpr, CALL);
 #undef CALL
   } else {
@@ -454,19 +474,20 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
                   need, workspace_bytes);
     }
     float *partials = static_cast<float *>(workspace);
+    bool const stream = stream_past_caches(M * N, sizeof(T));
 #define CALL(E, W)                                                             \
   do {                                                                         \
     if (dropped != nullptr) {                                                  \
       if constexpr (sizeof(T) == 2)                                            \
         layer_norm_bwd_kernel<T, E, W, true, true><<<blocks, kRowThreads, 0, st>>>( \
             DY, X, mean, rstd, G, DX, partials, M, (int)N, RES,                \
-            static_cast<T *>(dropped), *drop);                                 \
+            static_cast<T *>(dropped), *drop, stream);                         \
     } else if (acc)                                                            \
       layer_norm_bwd_kernel<T, E, W, true><<<blocks, kRowThreads, 0, st>>>(    \
-          DY, X, mean, rstd, G, DX, partials, M, (int)N, RES);                 \
+          DY, X, mean, rstd, G, DX, partials, M, (int)N, RES, nullptr, DropoutParams{}, stream); \
     else                                                                       \
       layer_norm_bwd_kernel<T, E, W, false><<<blocks, kRowThreads, 0, st>>>(   \
-          DY, X, mean, rstd, G, DX, partials, M, (int)N, nullptr);             \
+          DY, X, mean, rstd, G, DX, partials, M, (int)N, nullptr, nullptr, DropoutParams{}, stream); \
   } while (0)
     FFK_ROW_DISPATCH_SMALL(ept, wpr, CALL);
 #undef CALL

@@ -11,7 +11,7 @@
 
 namespace ffk {
 
-template <typename T, int EPT, int WPR>
+template <typename T, int EPT, int WPR, bool STREAM>
 __global__ __launch_bounds__(kRowThreads) void softmax_fwd_kernel(
     T const *__restrict__ X, T *__restrict__ Y, int64_t rows, int N) {
   constexpr int V = VecIO<T>::kVec;
@@ -30,7 +30,11 @@ __global__ __launch_bounds__(kRowThreads) void softmax_fwd_kernel(
   for (int j = 0; j < EPT; j++) {
     int v = lane + j * LANES;
     if (v < nvec) {
-      VecIO<T>::load(xr + (int64_t)v * V, x[j]);
+      if (STREAM) {
+        VecIO<T>::load_stream(xr + (int64_t)v * V, x[j]);
+      } else {
+        VecIO<T>::load(xr + (int64_t)v * V, x[j]);
+      }
 #pragma unroll
       for (int e = 0; e < V; e++) mx = fmaxf(mx, x[j][e]);
     } else {
@@ -60,12 +64,16 @@ __global__ __launch_bounds__(kRowThreads) void softmax_fwd_kernel(
       float y[V];
 #pragma unroll
       for (int e = 0; e < V; e++) y[e] = x[j][e] * inv;
-      VecIO<T>::store(yr + (int64_t)v * V, y);
+      if (STREAM) {
+        VecIO<T>::store_stream(yr + (int64_t)v * V, y);
+      } else {
+        VecIO<T>::store(yr + (int64_t)v * V, y);
+      }
     }
   }
 }
 
-template <typename T, int EPT, int WPR>
+template <typename T, int EPT, int WPR, bool STREAM>
 __global__ __launch_bounds__(kRowThreads) void softmax_bwd_kernel(
     T const *__restrict__ Y, T const *__restrict__ dY, T *__restrict__ dX,
     int64_t rows, int N) {
@@ -101,7 +109,11 @@ __global__ __launch_bounds__(kRowThreads) void softmax_bwd_kernel(
       float o[V];
 #pragma unroll
       for (int e = 0; e < V; e++) o[e] = y[j][e] * (dy[j][e] - dot);
-      VecIO<T>::store(dX + row * (int64_t)N + (int64_t)v * V, o);
+      if (STREAM) {
+        VecIO<T>::store_stream(dX + row * (int64_t)N + (int64_t)v * V, o);
+      } else {
+        VecIO<T>::store(dX + row * (int64_t)N + (int64_t)v * V, o);
+      }
     }
   }
 }
@@ -195,8 +207,14 @@ static int softmax_fwd(hipStream_t st, void const *x, void *y, int64_t outer,
     int ept = 0, wpr = 0;
     if (dim % V == 0 && aligned16(x) && aligned16(y) && pick_row_config(dim / V, ept, wpr)) {
       int64_t blocks = ceil_div(outer, 4 / wpr);
+      bool const stream = stream_past_caches(outer * dim, sizeof(T));
 #define CALL(E, W)                                                             \
-  softmax_fwd_kernel<T, E, W><<<(unsigned)blocks, kRowThreads, 0, st>>>(X, Y, outer, (int)dim)
+  do {                                                                         \
+    if (stream)                                                                \
+      softmax_fwd_kernel<T, E, W, true><<<(unsigned)blocks, kRowThreads, 0, st>>>(X, Y, outer, (int)dim); \
+    else                                                                       \
+      softmax_fwd_kernel<T, E, W, false><<<(unsigned)blocks, kRowThreads, 0, st>>>(X, Y, outer, (int)dim); \
+  } while (0)
       FFK_ROW_DISPATCH(ept, wpr, CALL);
 #undef CALL
     } else {
@@ -222,8 +240,14 @@ static int softmax_bwd(hipStream_t st, void const *y, void const *dy, void *dx,
     if (dim % V == 0 && aligned16(y) && aligned16(dy) && aligned16(dx) &&
         pick_row_config(dim / V, ept, wpr)) {
       int64_t blocks = ceil_div(outer, 4 / wpr);
+      bool const stream = stream_past_caches(outer * dim, sizeof(T));
 #define CALL(E, W)                                                             \
-  softmax_bwd_kernel<T, E, W><<<(unsigned)blocks, kRowThreads, 0, st>>>(Y, DY, DX, outer, (int)dim)
+  do {                                                                         \
+    if (stream)                                                                \
+      softmax_bwd_kernel<T, E, W, true><<<(unsigned)blocks, kRowThreads, 0, st>>>(Y, DY, DX, outer, (int)dim); \
+    else                                                                       \
+      softmax_bwd_kernel<T, E, W, false><<<(unsigned)blocks, kRowThreads, 0, st>>>(Y, DY, DX, outer, (int)dim); \
+  } while (0)
       FFK_ROW_DISPATCH(ept, wpr, CALL);
 #undef CALL
     } else {
