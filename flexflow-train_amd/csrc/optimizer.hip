@@ -15,33 +15,43 @@
 namespace ffk {
 
 constexpr int kOptThreads = 256;
+constexpr int kOptUnroll = 2;  // Adam: vectors per thread
 
-template <typename GT>
-__device__ __forceinline__ void load_grad_sum(GT const *g, int64_t i, int64_t n,
-                                              int replicas, float (&v)[4]);
+// 16-byte accesses; STREAM: past the caches (parameter sets larger than the last-level cache
+// are touched once per step and never found there again)
+template <bool STREAM, typename VT>
+__device__ __forceinline__ VT opt_load(VT const *p) {
+  if constexpr (STREAM) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+template <bool STREAM, typename VT>
+__device__ __forceinline__ void opt_store(VT *p, VT v) {
+  if constexpr (STREAM) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
 
-template <>
-__device__ __forceinline__ void load_grad_sum<float>(float const *g, int64_t i, int64_t n,
-                                                     int replicas, float (&v)[4]) {
-  f32x4 r = *reinterpret_cast<f32x4 const *>(g + i);
+template <bool STREAM>
+__device__ __forceinline__ void load_grad_sum(float const *g, int64_t i, int64_t n,
+                                              int replicas, float (&v)[4]) {
+  f32x4 r = opt_load<STREAM>(reinterpret_cast<f32x4 const *>(g + i));
   v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
   for (int k = 1; k < replicas; k++) {
-    f32x4 x = *reinterpret_cast<f32x4 const *>(g + (int64_t)k * n + i);
+    f32x4 x = opt_load<STREAM>(reinterpret_cast<f32x4 const *>(g + (int64_t)k * n + i));
 #pragma unroll
     for (int e = 0; e < 4; e++) v[e] = __fadd_rn(v[e], x[e]);
   }
 }
 
-template <>
-__device__ __forceinline__ void load_grad_sum<bf16>(bf16 const *g, int64_t i, int64_t n,
-                                                    int replicas, float (&v)[4]) {
-  u32x2 r = *reinterpret_cast<u32x2 const *>(g + i);
+template <bool STREAM>
+__device__ __forceinline__ void load_grad_sum(bf16 const *g, int64_t i, int64_t n,
+                                              int replicas, float (&v)[4]) {
+  u32x2 r = opt_load<STREAM>(reinterpret_cast<u32x2 const *>(g + i));
   v[0] = __uint_as_float(r[0] << 16);
   v[1] = __uint_as_float(r[0] & 0xffff0000u);
   v[2] = __uint_as_float(r[1] << 16);
   v[3] = __uint_as_float(r[1] & 0xffff0000u);
   for (int k = 1; k < replicas; k++) {
-    u32x2 x = *reinterpret_cast<u32x2 const *>(g + (int64_t)k * n + i);
+    u32x2 x = opt_load<STREAM>(reinterpret_cast<u32x2 const *>(g + (int64_t)k * n + i));
     v[0] = __fadd_rn(v[0], __uint_as_float(x[0] << 16));
     v[1] = __fadd_rn(v[1], __uint_as_float(x[0] & 0xffff0000u));
     v[2] = __fadd_rn(v[2], __uint_as_float(x[1] << 16));
@@ -73,7 +83,7 @@ __device__ __forceinline__ float sgd_step(float g, float &w, float *v, SgdParams
   return w;
 }
 
-template <typename GT>
+template <typename GT, bool STREAM>
 __global__ __launch_bounds__(kOptThreads) void sgd_update_kernel(
     GT const *__restrict__ grad, float *W, float *V, bf16 *W_lowp, int64_t n,
     int replicas, SgdParams p) {
@@ -81,18 +91,18 @@ __global__ __launch_bounds__(kOptThreads) void sgd_update_kernel(
   int64_t const i = q * 4;
   if (i + 4 <= n) {
     float g[4];
-    load_grad_sum<GT>(grad, i, n, replicas, g);
-    f32x4 w = *reinterpret_cast<f32x4 const *>(W + i);
+    load_grad_sum<STREAM>(grad, i, n, replicas, g);
+    f32x4 w = opt_load<STREAM>(reinterpret_cast<f32x4 const *>(W + i));
     f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (p.momentum > 0.0f) v = *reinterpret_cast<f32x4 const *>(V + i);
+    if (p.momentum > 0.0f) v = opt_load<STREAM>(reinterpret_cast<f32x4 const *>(V + i));
     float wv[4] = {w[0], w[1], w[2], w[3]}, vv[4] = {v[0], v[1], v[2], v[3]};
 #pragma unroll
     for (int e = 0; e < 4; e++) sgd_step(g[e], wv[e], &vv[e], p);
-    *reinterpret_cast<f32x4 *>(W + i) = f32x4{wv[0], wv[1], wv[2], wv[3]};
-    if (p.momentum > 0.0f) *reinterpret_cast<f32x4 *>(V + i) = f32x4{vv[0], vv[1], vv[2], vv[3]};
+    opt_store<STREAM>(reinterpret_cast<f32x4 *>(W + i), f32x4{wv[0], wv[1], wv[2], wv[3]});
+    if (p.momentum > 0.0f) opt_store<STREAM>(reinterpret_cast<f32x4 *>(V + i), f32x4{vv[0], vv[1], vv[2], vv[3]});
     if (W_lowp != nullptr) {
       u32x2 lo = {pack_bf16x2(wv[0], wv[1]), pack_bf16x2(wv[2], wv[3])};
-      *reinterpret_cast<u32x2 *>(W_lowp + i) = lo;
+      opt_store<STREAM>(reinterpret_cast<u32x2 *>(W_lowp + i), lo);
     }
   } else {
     for (int64_t j = i; j < n; j++) {
@@ -127,38 +137,52 @@ __device__ __forceinline__ void adam_step(float g, float &w, float &m, float &v,
   w = w - q;
 }
 
-template <typename GT>
+template <typename GT, bool STREAM>
 __global__ __launch_bounds__(kOptThreads) void adam_update_kernel(
     GT const *__restrict__ grad, float *W, float *M, float *V, bf16 *W_lowp,
     int64_t n, int replicas, AdamParams p) {
-  int64_t const q = (int64_t)blockIdx.x * kOptThreads + threadIdx.x;
-  int64_t const i = q * 4;
-  if (i + 4 <= n) {
-    float g[4];
-    load_grad_sum<GT>(grad, i, n, replicas, g);
-    f32x4 w = *reinterpret_cast<f32x4 const *>(W + i);
-    f32x4 m = *reinterpret_cast<f32x4 const *>(M + i);
-    f32x4 v = *reinterpret_cast<f32x4 const *>(V + i);
-    float wv[4] = {w[0], w[1], w[2], w[3]}, mv[4] = {m[0], m[1], m[2], m[3]},
-          vv[4] = {v[0], v[1], v[2], v[3]};
+  // kOptUnroll vectors of 4 parameters per thread, a workgroup's vectors interleaved: all loads
+  // of a thread are issued before the first arithmetic, which keeps more bytes in flight
+  int64_t const first = ((int64_t)blockIdx.x * kOptThreads * kOptUnroll + threadIdx.x) * 4;
+  if (first + (int64_t)(kOptUnroll - 1) * kOptThreads * 4 + 4 <= n) {
+    float g[kOptUnroll][4];
+    f32x4 w[kOptUnroll], m[kOptUnroll], v[kOptUnroll];
 #pragma unroll
-    for (int e = 0; e < 4; e++) adam_step(g[e], wv[e], mv[e], vv[e], p);
-    *reinterpret_cast<f32x4 *>(W + i) = f32x4{wv[0], wv[1], wv[2], wv[3]};
-    *reinterpret_cast<f32x4 *>(M + i) = f32x4{mv[0], mv[1], mv[2], mv[3]};
-    *reinterpret_cast<f32x4 *>(V + i) = f32x4{vv[0], vv[1], vv[2], vv[3]};
-    if (W_lowp != nullptr) {
-      u32x2 lo = {pack_bf16x2(wv[0], wv[1]), pack_bf16x2(wv[2], wv[3])};
-      *reinterpret_cast<u32x2 *>(W_lowp + i) = lo;
+    for (int u = 0; u < kOptUnroll; u++) {
+      int64_t const i = first + (int64_t)u * kOptThreads * 4;
+      load_grad_sum<STREAM>(grad, i, n, replicas, g[u]);
+      w[u] = opt_load<STREAM>(reinterpret_cast<f32x4 const *>(W + i));
+      m[u] = opt_load<STREAM>(reinterpret_cast<f32x4 const *>(M + i));
+      v[u] = opt_load<STREAM>(reinterpret_cast<f32x4 const *>(V + i));
+    }
+#pragma unroll
+    for (int u = 0; u < kOptUnroll; u++) {
+      int64_t const i = first + (int64_t)u * kOptThreads * 4;
+      float wv[4] = {w[u][0], w[u][1], w[u][2], w[u][3]}, mv[4] = {m[u][0], m[u][1], m[u][2], m[u][3]},
+            vv[4] = {v[u][0], v[u][1], v[u][2], v[u][3]};
+#pragma unroll
+      for (int e = 0; e < 4; e++) adam_step(g[u][e], wv[e], mv[e], vv[e], p);
+      opt_store<STREAM>(reinterpret_cast<f32x4 *>(W + i), f32x4{wv[0], wv[1], wv[2], wv[3]});
+      opt_store<STREAM>(reinterpret_cast<f32x4 *>(M + i), f32x4{mv[0], mv[1], mv[2], mv[3]});
+      opt_store<STREAM>(reinterpret_cast<f32x4 *>(V + i), f32x4{vv[0], vv[1], vv[2], vv[3]});
+      if (W_lowp != nullptr) {
+        u32x2 lo = {pack_bf16x2(wv[0], wv[1]), pack_bf16x2(wv[2], wv[3])};
+        opt_store<STREAM>(reinterpret_cast<u32x2 *>(W_lowp + i), lo);
+      }
     }
   } else {
-    for (int64_t j = i; j < n; j++) {
-      float g = load_grad_sum1<GT>(grad, j, n, replicas);
-      float w = W[j], m = M[j], v = V[j];
-      adam_step(g, w, m, v, p);
-      W[j] = w;
-      M[j] = m;
-      V[j] = v;
-      if (W_lowp != nullptr) VecIO<bf16>::store1(W_lowp + j, w);
+    // the last workgroup: element by element
+    for (int u = 0; u < kOptUnroll; u++) {
+      int64_t const i = first + (int64_t)u * kOptThreads * 4;
+      for (int64_t j = i; j < min(i + 4, n); j++) {
+        float g = load_grad_sum1<GT>(grad, j, n, replicas);
+        float w = W[j], m = M[j], v = V[j];
+        adam_step(g, w, m, v, p);
+        W[j] = w;
+        M[j] = m;
+        V[j] = v;
+        if (W_lowp != nullptr) VecIO<bf16>::store1(W_lowp + j, w);
+      }
     }
   }
 }
@@ -196,15 +220,18 @@ extern "C" int ffk_sgd_update(ffk_stream_t stream, int grad_dtype, float lr,
   SgdParams p{lr, weight_decay, momentum, nesterov != 0};
   unsigned const blocks = (unsigned)ceil_div(ceil_div(num_elements, 4), kOptThreads);
   hipStream_t st = as_stream(stream);
+  // weights, velocity and gradient together: what one step walks through
+  bool const past_caches = stream_past_caches(num_elements, 12);
+#define FFK_SGD(GT_, S_)                                                       \
+  sgd_update_kernel<GT_, S_><<<blocks, kOptThreads, 0, st>>>(                  \
+      static_cast<GT_ const *>(weight_grad), weight, sgd_v, static_cast<bf16 *>(weight_lowp), \
+      num_elements, num_replicas, p)
   if (grad_dtype == FFK_FLOAT) {
-    sgd_update_kernel<float><<<blocks, kOptThreads, 0, st>>>(
-        static_cast<float const *>(weight_grad), weight, sgd_v, static_cast<bf16 *>(weight_lowp),
-        num_elements, num_replicas, p);
+    if (past_caches) FFK_SGD(float, true); else FFK_SGD(float, false);
   } else {
-    sgd_update_kernel<bf16><<<blocks, kOptThreads, 0, st>>>(
-        static_cast<bf16 const *>(weight_grad), weight, sgd_v, static_cast<bf16 *>(weight_lowp),
-        num_elements, num_replicas, p);
+    if (past_caches) FFK_SGD(bf16, true); else FFK_SGD(bf16, false);
   }
+#undef FFK_SGD
   FFK_CHECK_LAUNCH();
   return FFK_OK;
 }
@@ -221,17 +248,19 @@ extern "C" int ffk_adam_update(ffk_stream_t stream, int grad_dtype, float alpha_
   FFK_REQUIRE(adam_v && adam_m && aligned16(adam_v) && aligned16(adam_m),
               "adam_update: adam_v / adam_m must be given and 16-byte aligned");
   AdamParams p{alpha_t, beta1, beta2, weight_decay, epsilon};
-  unsigned const blocks = (unsigned)ceil_div(ceil_div(num_elements, 4), kOptThreads);
+  unsigned const blocks = (unsigned)ceil_div(ceil_div(num_elements, 4), kOptThreads * kOptUnroll);
   hipStream_t st = as_stream(stream);
+  bool const past_caches = stream_past_caches(num_elements, 16);
+#define FFK_ADAM(GT_, S_)                                                      \
+  adam_update_kernel<GT_, S_><<<blocks, kOptThreads, 0, st>>>(                 \
+      static_cast<GT_ const *>(weight_grad), weight, adam_m, adam_v, static_cast<bf16 *>(weight_lowp), \
+      num_elements, num_replicas, p)
   if (grad_dtype == FFK_FLOAT) {
-    adam_update_kernel<float><<<blocks, kOptThreads, 0, st>>>(
-        static_cast<float const *>(weight_grad), weight, adam_m, adam_v,
-        static_cast<bf16 *>(weight_lowp), num_elements, num_replicas, p);
+    if (past_caches) FFK_ADAM(float, true); else FFK_ADAM(float, false);
   } else {
-    adam_update_kernel<bf16><<<blocks, kOptThreads, 0, st>>>(
-        static_cast<bf16 const *>(weight_grad), weight, adam_m, adam_v,
-        static_cast<bf16 *>(weight_lowp), num_elements, num_replicas, p);
+    if (past_caches) FFK_ADAM(bf16, true); else FFK_ADAM(bf16, false);
   }
+#undef FFK_ADAM
   FFK_CHECK_LAUNCH();
   return FFK_OK;
 }

@@ -11,14 +11,6 @@ namespace ffk {
 
 constexpr int kRowThreads = 256;
 
-// A tensor this large does not stay in the 256 MB last-level cache between the kernel that
-// writes it and the one that reads it next: its accesses then bypass the caches (non-temporal
-// loads and stores), which measured 6-8% more bandwidth on 1 GB softmax tensors.  Smaller
-// tensors keep ordinary accesses so the next kernel finds them in cache.
-static inline bool stream_past_caches(int64_t elems, size_t elem_size) {
-  return (size_t)elems * elem_size > ((size_t)128 << 20);
-}
-
 template <int WPR>
 struct RowReducer {
   // smem: 2 phases x 4 waves x 2 values
