@@ -284,8 +284,27 @@ __global__ __launch_bounds__(kEmbBlockThreads) void embedding_bwd_sorted_block_k
   int64_t const block1 = min(block0 + (int64_t)WPB * kEmbChunk, n);
   int64_t const p0 = block0 + (int64_t)w * kEmbChunk;
   int64_t const p1 = min(p0 + (int64_t)kEmbChunk, n);
-  bool const active = p0 < n;
-  bool const head_shared = active && p0 > 0 && keys[p0 - 1] == keys[p0];
+  // The walker's 16 (row id, lookup) pairs are fetched once, one pair per lane, and handed round
+  // with lane shuffles.  What the walk would otherwise wait for at every position -- the
+  // gradient row of the lookup and, where a run ends, the weight-gradient row it is added to --
+  // is then asked for two positions ahead.  (Walkers of cold rows, where every position ends a
+  // run, set the pace of their workgroup: each of their positions used to cost two dependent
+  // memory round trips.)
+  int const cnt = (int)max((int64_t)0, min((int64_t)kEmbChunk, n - p0));  // positions that exist
+  bool const active = cnt > 0;
+  static_assert(LPR >= kEmbChunk, "one pair per lane");
+  uint32_t my_key = invalid_key, my_val = 0;
+  if (wl < cnt) {
+    my_key = keys[p0 + wl];
+    my_val = vals[p0 + wl];
+  }
+  int const wbase = ((threadIdx.x & 63) / LPR) * LPR;  // the walker's first lane in its wave
+  uint32_t const key_before = active && p0 > 0 ? keys[p0 - 1] : invalid_key;
+  uint32_t const key_after = active && p1 < n ? keys[p1] : invalid_key;
+  // every lane of the wave takes part in a shuffle, whatever its walker has to do
+  auto key_at = [&](int j) { return (uint32_t)__shfl((int)my_key, wbase + (j < kEmbChunk ? j : kEmbChunk - 1), 64); };
+  auto lookup_at = [&](int j) { return (uint32_t)__shfl((int)my_val, wbase + (j < kEmbChunk ? j : kEmbChunk - 1), 64); };
+  bool const head_shared = active && p0 > 0 && key_before == key_at(0);
   auto add_row = [&](uint32_t id, int64_t cbase, float const (&acc)[CPL][4], bool atomic) {
 #pragma unroll
     for (int k = 0; k < CPL; k++) {
@@ -309,17 +328,21 @@ __global__ __launch_bounds__(kEmbBlockThreads) void embedding_bwd_sorted_block_k
       part_valid[2 * w] = 0;
       part_valid[2 * w + 1] = 0;
     }
-    if (active) {
-      float acc[CPL][4], cur[CPL][4], nxt[CPL][4];
-      auto fetch = [&](int64_t p, float (&v)[CPL][4]) {
-        // lookups are 32-bit positions: a 32-bit unsigned division, and none for bags of one
-        uint32_t const l = vals[p];
+    {
+      float acc[CPL][4], rows[2][CPL][4];
+      f32x4 old[2][CPL];
+      // position j's gradient row, and the weight-gradient row of its id if a run of this
+      // walker alone ends there (nobody else touches that row during the kernel)
+      auto prefetch = [&](int j, uint32_t id, uint32_t next_id, uint32_t l, float (&v)[CPL][4], f32x4 (&o)[CPL]) {
+        if (j >= cnt) return;
         GT const *row = dY + (int64_t)(bag == 1 ? l : l / (uint32_t)bag) * dim;
+        bool const ends = j + 1 >= cnt || next_id != id;
 #pragma unroll
         for (int k = 0; k < CPL; k++) {
           int64_t const c = cbase + ((int64_t)k * LPR + wl) * 4;
           if (c < dim) {
             load_grad4<GT>(row + c, v[k]);
+            if (ends && id != invalid_key) o[k] = *reinterpret_cast<f32x4 const *>(dW + (int64_t)id * dim + c);
           } else {
             v[k][0] = v[k][1] = v[k][2] = v[k][3] = 0.0f;
           }
@@ -330,48 +353,70 @@ __global__ __launch_bounds__(kEmbBlockThreads) void embedding_bwd_sorted_block_k
 #pragma unroll
         for (int e = 0; e < 4; e++) acc[k][e] = 0.0f;
       bool shared_run = head_shared;
-      fetch(p0, cur);
-      for (int64_t p = p0; p < p1; p++) {
-        bool const more = p + 1 < p1;
-        if (more) fetch(p + 1, nxt);
-        uint32_t const id = keys[p];
-#pragma unroll
-        for (int k = 0; k < CPL; k++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) acc[k][e] += cur[k][e];
-        if (!more || keys[p + 1] != id) {
-          bool const tail_shared = !more && p + 1 < n && keys[p + 1] == id;
-          if (id != invalid_key) {
-            if (shared_run || tail_shared) {
-              // slot 2w: run shared with the previous walker (or both sides);
-              // slot 2w+1: run shared with the next walker only
-              int const slot = shared_run ? 2 * w : 2 * w + 1;
-#pragma unroll
-              for (int k = 0; k < CPL; k++) {
-                f32x4 v = {acc[k][0], acc[k][1], acc[k][2], acc[k][3]};
-                *reinterpret_cast<f32x4 *>(emb_part + slot * PW + (k * LPR + wl) * 4) = v;
-              }
-              if (wl == 0) {
-                part_id[slot] = id;
-                // 1: a border partial; 2 / 4: its run also extends before /
-                // beyond the workgroup's positions
-                part_valid[slot] = 1 | ((shared_run && p0 == block0) ? 2 : 0) |
-                                   ((tail_shared && p1 == block1) ? 4 : 0);
-              }
-            } else {
-              add_row(id, cbase, acc, false);
-            }
-          }
-          shared_run = false;
+      // the ids around position j: id_j, id_{j+1}, id_{j+2}, id_{j+3} slide along with j
+      uint32_t id0 = key_at(0), id1 = key_at(1), id2 = key_at(2), l0 = lookup_at(0), l1 = lookup_at(1);
+      prefetch(0, id0, id1, l0, rows[0], old[0]);
+      prefetch(1, id1, id2, l1, rows[1], old[1]);
+      auto step = [&](int j, float (&v)[CPL][4], f32x4 (&o)[CPL]) {
+        // shuffles first, by every lane
+        uint32_t const id3 = key_at(j + 3);
+        uint32_t const l2 = lookup_at(j + 2);
+        if (j < cnt) {
+          uint32_t const id = id0;
 #pragma unroll
           for (int k = 0; k < CPL; k++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) acc[k][e] = 0.0f;
+            for (int e = 0; e < 4; e++) acc[k][e] += v[k][e];
+          bool const more = j + 1 < cnt;
+          uint32_t const next_id = j + 1 < kEmbChunk ? id1 : key_after;
+          if (!more || next_id != id) {
+            bool const tail_shared = !more && p1 < n && key_after == id;
+            if (id != invalid_key) {
+              if (shared_run || tail_shared) {
+                // slot 2w: run shared with the previous walker (or both sides);
+                // slot 2w+1: run shared with the next walker only
+                int const slot = shared_run ? 2 * w : 2 * w + 1;
+#pragma unroll
+                for (int k = 0; k < CPL; k++) {
+                  f32x4 pv = {acc[k][0], acc[k][1], acc[k][2], acc[k][3]};
+                  *reinterpret_cast<f32x4 *>(emb_part + slot * PW + (k * LPR + wl) * 4) = pv;
+                }
+                if (wl == 0) {
+                  part_id[slot] = id;
+                  // 1: a border partial; 2 / 4: its run also extends before /
+                  // beyond the workgroup's positions
+                  part_valid[slot] = 1 | ((shared_run && p0 == block0) ? 2 : 0) |
+                                     ((tail_shared && p1 == block1) ? 4 : 0);
+                }
+              } else {
+#pragma unroll
+                for (int k = 0; k < CPL; k++) {
+                  int64_t const c = cbase + ((int64_t)k * LPR + wl) * 4;
+                  if (c < dim) {
+                    f32x4 upd = {o[k][0] + acc[k][0] * scale, o[k][1] + acc[k][1] * scale,
+                                 o[k][2] + acc[k][2] * scale, o[k][3] + acc[k][3] * scale};
+                    *reinterpret_cast<f32x4 *>(dW + (int64_t)id * dim + c) = upd;
+                  }
+                }
+              }
+            }
+            shared_run = false;
+#pragma unroll
+            for (int k = 0; k < CPL; k++)
+#pragma unroll
+              for (int e = 0; e < 4; e++) acc[k][e] = 0.0f;
+          }
         }
-#pragma unroll
-        for (int k = 0; k < CPL; k++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) cur[k][e] = nxt[k][e];
+        // this slot is free now: position j + 2 goes into it
+        prefetch(j + 2, id2, j + 3 < kEmbChunk ? id3 : key_after, l2, v, o);
+        id0 = id1;
+        id1 = id2;
+        id2 = id3;
+      };
+#pragma unroll 1
+      for (int j = 0; j < kEmbChunk; j += 2) {
+        step(j, rows[0], old[0]);
+        step(j + 1, rows[1], old[1]);
       }
     }
     __syncthreads();
