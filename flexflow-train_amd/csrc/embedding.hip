@@ -33,11 +33,34 @@ __device__ __forceinline__ void store_out<float, 8>(float *p, float const (&v)[8
 }
 template <>
 __device__ __forceinline__ void store_out<bf16, 4>(bf16 *p, float const (&v)[4]) {
-  *reinterpret_cast<u32x2 *>(p) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+  __builtin_nontemporal_store(u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])}, reinterpret_cast<u32x2 *>(p));
 }
 template <>
 __device__ __forceinline__ void store_out<bf16, 8>(bf16 *p, float const (&v)[8]) {
-  VecIO<bf16>::store(p, v);
+  VecIO<bf16>::store_stream(p, v);
+}
+
+// V elements of a table row as floats: 16-byte loads
+template <typename WT, int V>
+__device__ __forceinline__ void load_row(WT const *p, float (&v)[V]) {
+  if constexpr (sizeof(WT) == 4 && V == 8) {
+    float a[4], b[4];
+    VecIO<float>::load(p, a);
+    VecIO<float>::load(p + 4, b);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      v[e] = a[e];
+      v[4 + e] = b[e];
+    }
+  } else {
+    static_assert(V == VecIO<WT>::kVec, "one 16-byte load");
+    VecIO<WT>::load(p, v);
+  }
+}
+// elements per thread: what makes the store 16 bytes (8 for a bf16 output), at least one 16-byte load
+template <typename WT, typename OT>
+constexpr int emb_vec() {
+  return sizeof(OT) == 2 ? 8 : VecIO<WT>::kVec;
 }
 
 // One thread per (bag, 16-byte vector of the row).
@@ -46,7 +69,7 @@ __global__ __launch_bounds__(kEmbThreads) void embedding_fwd_vec_kernel(
     IT const *__restrict__ idx, OT *__restrict__ out, WT const *__restrict__ W,
     int64_t num_bags, int bag, int nvec, int64_t dim, int64_t num_entries,
     float scale) {
-  constexpr int V = VecIO<WT>::kVec;
+  constexpr int V = emb_vec<WT, OT>();
   int64_t const total = num_bags * nvec;
   int64_t const stride = (int64_t)gridDim.x * kEmbThreads;
   for (int64_t i = (int64_t)blockIdx.x * kEmbThreads + threadIdx.x; i < total; i += stride) {
@@ -65,7 +88,7 @@ __global__ __launch_bounds__(kEmbThreads) void embedding_fwd_vec_kernel(
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         bool ok = (uint64_t)r[u] < (uint64_t)num_entries;
-        VecIO<WT>::load(W + (ok ? r[u] : 0) * dim + (int64_t)v * V, w[u]);
+        load_row<WT, V>(W + (ok ? r[u] : 0) * dim + (int64_t)v * V, w[u]);
         if (!ok) {
 #pragma unroll
           for (int e = 0; e < V; e++) w[u][e] = 0.0f;
@@ -80,7 +103,7 @@ __global__ __launch_bounds__(kEmbThreads) void embedding_fwd_vec_kernel(
       int64_t r = (int64_t)ib[j];
       if ((uint64_t)r < (uint64_t)num_entries) {
         float w[V];
-        VecIO<WT>::load(W + r * dim + (int64_t)v * V, w);
+        load_row<WT, V>(W + r * dim + (int64_t)v * V, w);
 #pragma unroll
         for (int e = 0; e < V; e++) acc[e] = acc[e] + w[e];
       }
@@ -483,7 +506,7 @@ static bool emb_sort_layout(int64_t n, int64_t num_entries, EmbSortLayout &L) {
 
 static int emb_grid(int64_t threads_needed) {
   int64_t b = ceil_div(threads_needed > 0 ? threads_needed : 1, kEmbThreads);
-  int64_t const cap = (int64_t)kNumCU * 32;
+  int64_t const cap = (int64_t)kNumCU * 256;
   return (int)(b < cap ? b : cap);
 }
 
@@ -491,7 +514,7 @@ template <typename IT, typename WT, typename OT>
 static int emb_forward(hipStream_t st, void const *indices, void *output,
                        void const *weight, int64_t num_bags, int64_t bag,
                        int64_t dim, int64_t num_entries, float scale) {
-  constexpr int V = VecIO<WT>::kVec;
+  constexpr int V = emb_vec<WT, OT>();
   IT const *I = static_cast<IT const *>(indices);
   WT const *W = static_cast<WT const *>(weight);
   OT *O = static_cast<OT *>(output);
