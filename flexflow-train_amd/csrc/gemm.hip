@@ -557,11 +557,15 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // a wave that cannot issue its next load cannot issue its next MFMA either.
   constexpr bool SPREAD = STAGES >= 3 && LPT % KS == 0;
   constexpr int PART = SPREAD ? LPT / KS : LPT;
+  // One wave per SIMD and two stages: a refill goes out in two halves, the first behind the
+  // barrier that frees its stage, the second in the first k-step of the following tile.
+  constexpr bool WIDE2 = WM == 128 && WN == 128 && STAGES == 2;
+  constexpr int PRO_PART = WIDE2 ? LPT / 2 : PART;  // of the last tile the prologue starts
 #pragma unroll
   for (int s = 0; s < STAGES; s++) {
     if (s < KT) {
-      if (SPREAD && s == STAGES - 1) {
-        issue_some(s, s, 0, PART);  // tile 0's steps issue the rest
+      if ((SPREAD || WIDE2) && s == STAGES - 1) {
+        issue_some(s, s, 0, PRO_PART);  // tile 0's steps issue the rest
       } else {
         issue(s, s);
       }
@@ -585,7 +589,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   };
   // Tile 0 must have landed (STAGES-1 younger tiles may still be in flight).
   if (STAGES - 1 < KT) {
-    wait_vmcnt<(STAGES - 2) * LPT + PART>();
+    wait_vmcnt<(STAGES - 2) * LPT + PRO_PART>();
   } else {
     wait_vmcnt<0>();
   }
@@ -600,6 +604,65 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   auto tile_step = [&](int kt, auto steady_tag) {
     constexpr bool STEADY = decltype(steady_tag)::value;
     int const stage = kt % STAGES;
+    if constexpr (WIDE2) {
+      // One wave per SIMD: nothing but this wave's own instruction order hides a latency, so
+      // the order is written out.  A k-step is 16 MFMAs.  Behind each of them sits one of the 8
+      // fragment reads of the next step or one of up to 8 direct loads, alternating, fenced so
+      // that the compiler keeps them there.  The refill of a stage goes out in two halves: the
+      // first behind the barrier that frees the stage (last step of its tile), the second in
+      // step 0 of the following tile; the steps in between carry fragment reads only.
+      static_assert(PF == 1 && TM == 4 && TN == 4 && LPT == 16 && KS >= 2, "written for this shape");
+#pragma unroll
+      for (int kk = 0; kk < KS; kk++) {
+        int const cur = kk % NB, nxt = (kk + PF) % NB;
+        bool const within = kk + PF < KS;            // the next step lies in this tile
+        bool const reads = within || STEADY || kt + 1 < KT;
+        int const rstage = within ? stage : (kt + 1) % STAGES;
+        int const rkk = within ? kk + PF : kk + PF - KS;
+        bf16 const *ra = smem + rstage * STAGE_ELEMS;
+        bf16 const *rb = ra + A_ELEMS;
+        bool const loads = kk == 0 ? (STEADY || kt + 1 < KT) : !within ? (STEADY || kt + 2 < KT) : false;
+        int const ltile = kk == 0 ? kt + 1 : kt + 2;
+        int const lstage = kk == 0 ? (kt + 1) % STAGES : stage;
+        int const lfirst = kk == 0 ? LPT / 2 : 0;
+        // slot p follows MFMA p.  Even slots: a fragment read, in the order in which the next
+        // step's MFMAs (row block by row block) first use the fragments: A0, B0..B3, A1, A2, A3.
+        // Odd slots: a direct load.
+        auto aux = [&](int p) __attribute__((always_inline)) {
+          int const r = p / 2;
+          if (p % 2 == 1) {
+            if (loads) issue_some(ltile, lstage, lfirst + r, 1);
+          } else if (reads) {
+            if (r == 0 || r > TN) {
+              int const i = r == 0 ? 0 : r - TN;
+              af[nxt][i] = TA ? frag_tr(ra, BM, tr_tab_a, wm0 + i * 32, rkk) : frag_kc(ra, wm0 + i * 32, rkk);
+            } else {
+              int const j = r - 1;
+              bfr[nxt][j] = TBL ? frag_tr(rb, BN, tr_tab_b, wn0 + j * 32, rkk) : frag_kc(rb, wn0 + j * 32, rkk);
+            }
+          }
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0], af[cur][0], acc[0][0], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (!within && reads) {
+          // the next tile must have landed (nothing younger is in flight with two stages) and
+          // every wave must be done reading this one
+          wait_vmcnt<0>();
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        }
+#pragma unroll
+        for (int m = 1; m < TM * TN; m++) {
+          aux(m - 1);
+          __builtin_amdgcn_sched_barrier(0);
+          acc[m / TN][m % TN] =
+              __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][m % TN], af[cur][m / TN], acc[m / TN][m % TN], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        aux(TM * TN - 1);
+      }
+      return;
+    }
 #pragma unroll
     for (int kk = 0; kk < KS; kk++) {
       int const cur = kk % NB;
@@ -667,8 +730,16 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   auto finish = [&](auto actf) __attribute__((always_inline)) {
     bf16 *const dst = C;
     bool const add_old = accumulate != 0;
+    // A wave stages and writes out its own tile, so only its own LDS accesses have to be ordered,
+    // and those complete in program order: no barrier.  With one wave per SIMD (128x128 wave tiles)
+    // the tile goes out in two halves of 64 rows, so that the stores of the first half are under
+    // way while the second is converted.
+    constexpr int HALVES = (WM == 128 && WN == 128) ? 2 : 1;
+    constexpr int TMH = TM / HALVES;
+#pragma unroll
+    for (int half = 0; half < HALVES; half++) {
     // The lane's bias values depend on (j, g, lane / 32) only: they are
-    // fetched once per (j, g) and used for the TM row blocks.
+    // fetched once per (j, g) and used for the row blocks.
 #pragma unroll
     for (int j = 0; j < TN; j++) {
 #pragma unroll
@@ -679,7 +750,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
         float const bv[4] = {__uint_as_float(raw[0] << 16), __uint_as_float(raw[0] & 0xffff0000u),
                              __uint_as_float(raw[1] << 16), __uint_as_float(raw[1] & 0xffff0000u)};
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
+        for (int i = half * TMH; i < (half + 1) * TMH; i++) {
           int const m = i * 32 + (lane & 31);
           float v[4];
 #pragma unroll
@@ -699,9 +770,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
         }
       }
     }
-    __syncthreads();
 #pragma unroll
-    for (int i = 0; i < CCH; i++) {
+    for (int i = half * (CCH / HALVES); i < (half + 1) * (CCH / HALVES); i++) {
       int c = lane + i * 64;
       int row = c / (WN / 8), ch = c % (WN / 8);
       u32x4 v = *reinterpret_cast<u32x4 const *>(cs + row * CS + ch * 8);
@@ -747,6 +817,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
         }
       }
     }
+    }  // half
     if constexpr (TAIL == GemmEpilogue::kTailDropoutGeluGrad) {
       if (tail.colsum_partials != nullptr) {  // uniform over the launch
         __syncthreads();
@@ -772,6 +843,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       }
     }
   };
+  // One wave per SIMD with a 128x128 wave tile keeps 256 accumulator registers: only the plain
+  // epilogue (bias, no activation, no split-K) is compiled for it, so that nothing outside the
+  // loop competes for registers.
+  constexpr bool WIDE = WM == 128 && WN == 128;
+  if constexpr (WIDE) {
+    finish([](float v) { return v; });
+    return;
+  }
   if (partial != nullptr) {
     // raw accumulators, 16 bytes (4 consecutive columns) per store
     float *dst = partial + (int64_t)split * M * N;
@@ -1072,7 +1151,7 @@ static int pipe_tile_for(bf16 const *C, int M, int N, int K, int64_t lda, int64_
   // refills are spread over the k-steps) halve the L2->LDS traffic per flop;
   // they win whenever they still occupy most CUs.  Otherwise 128x128x64 tiles
   // with 8 waves of 64x32 keep two waves per SIMD on every CU.
-  if ((variant == 0 && t256 >= kNumCU * 3 / 4) || (variant == 256 && fits256)) return 256;
+  if ((variant == 0 && t256 >= kNumCU * 3 / 4) || ((variant == 256 || variant == 264) && fits256)) return 256;
   if ((variant == 0 && t128 >= kNumCU / 2) || (variant == 128 && fits128)) return 128;
   return 0;
 }
@@ -1114,6 +1193,12 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
         }
       }
       return hipErrorInvalidValue;
+    }
+    // Long reductions without an activation: one wave per SIMD on 128x128 wave tiles, two
+    // 64-deep stages, every instruction of the loop placed by hand.  (Up to about 1024 of K the
+    // eight-wave kernel's shorter prologue and epilogue weigh more than the faster loop.)
+    if (use256 && ep.activation == FFK_ACT_NONE && (variant == 264 || (variant == 0 && K >= 2048))) {
+      return launch_pipe<256, 256, 128, 128, 64, 2, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
     if (use256) {
       return launch_pipe<256, 256, 128, 64, 32, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);

@@ -207,6 +207,46 @@ def test_gemm_bf16_pipelined_tiles(ffk, oracle, trans_a, trans_b, mnk):
     assert_close(to_np(Cd)[rows], oracle.gemm_f64(A_rows, B, trans_a, trans_b) + C0[rows], 2.0 ** -7, "C acc")
 
 
+# Reductions from 2048 on take 256x256 tiles with one wave per SIMD (128x128 wave tiles, two 64-deep
+# stages); the option forces that kernel onto short reductions too: one, two and three k-tiles
+# exercise its prologue and drain, 33 an odd count in the steady loop.
+WIDE_SHAPES = [(2048, 2048, 64), (2048, 2048, 128), (2048, 2048, 192), (4096, 3072, 2112)]
+
+
+@pytest.mark.parametrize("trans_a,trans_b", [(False, True), (False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("mnk", WIDE_SHAPES)
+def test_gemm_bf16_one_wave_per_simd(ffk, oracle, trans_a, trans_b, mnk):
+    M, N, K = mnk
+    say("gemm bf16 one wave per SIMD", mnk, "ta", trans_a, "tb", trans_b)
+    g = rng(5 * M + 3 * N + K)
+    A = bf16_round(g.standard_normal((K, M) if trans_a else (M, K)))
+    B = bf16_round(g.standard_normal((N, K) if trans_b else (K, N)))
+    C0 = bf16_round(g.standard_normal((M, N)))
+    Ad, Bd = to_dev(A, torch, torch.bfloat16), to_dev(B, torch, torch.bfloat16)
+    out = {}
+    try:
+        for variant in (264, 256):
+            ffk.set_option(ffk.OPTION_GEMM_VARIANT, variant)
+            C = torch.full((M, N), 3.0, dtype=torch.bfloat16, device="cuda")
+            ffk.gemm(Ad, Bd, C, trans_a, trans_b)
+            Cacc = to_dev(C0, torch, torch.bfloat16)
+            ffk.gemm(Ad, Bd, Cacc, trans_a, trans_b, accumulate=True)
+            out[variant] = (C, Cacc)
+    finally:
+        ffk.set_option(ffk.OPTION_GEMM_VARIANT, 0)
+    Cn = to_np(out[264][0])
+    rows = np.sort(g.choice(M, 24, replace=False))
+    cols = np.sort(g.choice(N, 24, replace=False))
+    A_rows = np.ascontiguousarray(A[:, rows] if trans_a else A[rows])
+    B_cols = np.ascontiguousarray(B[cols] if trans_b else B[:, cols])
+    assert_close(Cn[rows], oracle.gemm_f64(A_rows, B, trans_a, trans_b), 2.0 ** -8, "C rows")
+    assert_close(Cn[:, cols], oracle.gemm_f64(A, B_cols, trans_a, trans_b), 2.0 ** -8, "C cols")
+    # both kernels add the k-steps up in the same order: every element agrees to the bit
+    assert torch.equal(out[264][0], out[256][0])
+    assert torch.equal(out[264][1], out[256][1])
+    assert_close(to_np(out[264][1])[rows], oracle.gemm_f64(A_rows, B, trans_a, trans_b) + C0[rows], 2.0 ** -7, "C acc")
+
+
 @pytest.mark.parametrize("act", [-1, 0])
 def test_linear_bf16_pipelined(ffk, oracle, act):
     """Linear at a size whose three products all take the pipelined kernels
