@@ -196,7 +196,7 @@ def lib():
     return _lib
 
 
-OPTION_GEMM_VARIANT, OPTION_LAYER_UNFUSED = 0, 1
+OPTION_GEMM_VARIANT, OPTION_LAYER_UNFUSED, OPTION_ATTENTION_VARIANT = 0, 1, 2
 
 
 def set_option(which, value):

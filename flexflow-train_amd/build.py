@@ -40,6 +40,7 @@ HIP_FLAGS = [
 # compiler's default contracts a * b + c into one fused operation.
 EXTRA_FLAGS = {
     "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "attention_fwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-fno-honor-nans"],
     "optimizer.hip": ["-ffp-contract=off"],
     "loss.hip": ["-ffp-contract=off"],
 }

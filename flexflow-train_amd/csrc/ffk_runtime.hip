@@ -39,6 +39,7 @@ static int env_int(char const *name) {
 static std::atomic<int> g_option[FFK_OPTION_COUNT] = {
     {env_int("FFK_GEMM_VARIANT")},
     {env_int("FFK_LAYER_UNFUSED")},
+    {env_int("FFK_ATTENTION_VARIANT")},
 };
 int option(int which) { return g_option[which].load(std::memory_order_relaxed); }
 

@@ -12,6 +12,7 @@
 //
 // These replace the cublasGemmEx calls of the reference
 // (lib/kernels/src/cuda/ops/linear_kernels.cu:143,163,249,298,321).
+#include "lds_dma.h"
 #include "gemm.h"
 #include "colreduce.h"
 #include <stdlib.h>
@@ -305,52 +306,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
 //    written to HBM as full 16-byte chunks with bias/activation/accumulate
 //    applied on the way.
 // ---------------------------------------------------------------------------
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-// One direct global->LDS load: lane l's 16 bytes at `g` land at LDS address
-// lds_base + 16 l (M0 carries the wave-uniform base).  Issued as inline
-// assembly on purpose: the compiler then does not know that LDS is being
-// written asynchronously, and therefore does not put a full `vmcnt(0)` wait in
-// front of later LDS reads it cannot prove disjoint (it did so in front of
-// every transposing read, which serialised load and compute).  The kernel
-// orders these loads against its LDS reads itself, with wait_vmcnt and the
-// barrier.  Loads the compiler does know about stay correct: its vmcnt waits
-// count these extra, younger loads too, which only makes them stricter.
-// The load is the buffer form (a scalar resource descriptor for the operand
-// panel, a scalar byte offset for what is uniform, one 32-bit byte offset per
-// lane that never changes) rather than the flat-global form with a 64-bit
-// address per lane: no vector address arithmetic remains in the k-loop, and
-// the instruction issues through the vector-memory port alone.
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void lds_dma16(i32x4 rsrc, unsigned lane_byte_off, unsigned uniform_byte_off,
-                                          unsigned lds_byte_addr) {
-  // lds_byte_addr is wave-uniform and held in a scalar register by the caller
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_byte_addr), "v"(lane_byte_off), "s"(rsrc), "s"(uniform_byte_off)
-               : "memory");  // M0 is not in the clobber list (the compiler rejects
-                             // reserved registers there); nothing else in these
-                             // kernels uses M0 (no GDS, message or relative-move ops)
-}
-// Raw buffer descriptor over everything from `base` on: stride 0, no bound
-// (the callers' offsets are checked on the host), 32-bit data format.
-__device__ __forceinline__ i32x4 buffer_resource(void const *base) {
-  uint64_t const a = reinterpret_cast<uint64_t>(base);
-  i32x4 r;
-  r[0] = (int)__builtin_amdgcn_readfirstlane((unsigned)a);
-  r[1] = (int)(__builtin_amdgcn_readfirstlane((unsigned)(a >> 32)) & 0xffffu);
-  r[2] = -1;
-  r[3] = 0x00020000;
-  return r;
-}
-// The LDS byte address of a __shared__ object, as a scalar.
-__device__ __forceinline__ unsigned lds_address_of(void *p) {
-  return __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)p);
-}
-
 // PF = how many k-steps ahead of its use a fragment is read from LDS (PF + 1
 // register buffers).  PF = 1 is what both tile configurations use; PF = 3 was
 // measured on the 128x128 tile (2 MFMAs per k-step per wave) and gained nothing.

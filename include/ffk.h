@@ -128,8 +128,16 @@ int ffk_event_elapsed_ms(ffk_event_t start, ffk_event_t stop, float *ms);
  *     128 / 256 force that pipelined bf16 tile, 1 the register-staged kernel.
  *   FFK_OPTION_LAYER_UNFUSED (FFK_LAYER_UNFUSED): != 0 makes the encoder-layer
  *     entry points (and a step-driver instance created while it is set) run
- *     one kernel per operator.                                               */
-enum { FFK_OPTION_GEMM_VARIANT = 0, FFK_OPTION_LAYER_UNFUSED = 1, FFK_OPTION_COUNT = 2 };
+ *     one kernel per operator.
+ *   FFK_OPTION_ATTENTION_VARIANT (FFK_ATTENTION_VARIANT): 0 = the default bf16
+ *     attention kernels; 1 = the forward kernel with 32 query rows per
+ *     wavefront (two workgroups per CU) that the default one replaced.       */
+enum {
+  FFK_OPTION_GEMM_VARIANT = 0,
+  FFK_OPTION_LAYER_UNFUSED = 1,
+  FFK_OPTION_ATTENTION_VARIANT = 2,
+  FFK_OPTION_COUNT = 3
+};
 int ffk_set_option(int which, int value);
 int ffk_get_option(int which, int *value);
 

@@ -46,6 +46,53 @@ def test_attention_core(ffk, oracle, shape, causal):
     assert_close(to_np(dv), dv_ref, BF16_RTOL, "dV")
 
 
+# Forward kernel: 256 query rows per workgroup, 64 per wavefront in two halves, 64 keys per tile.
+# Shapes around those sizes (blocks that end inside a half, a last key tile of 1 and of 63, more
+# keys than queries and the reverse), under both masks.
+FWD_SHAPES = [(1, 2, 600, 600, 128), (1, 1, 257, 705, 64), (1, 1, 513, 513, 128), (2, 1, 33, 449, 128), (1, 2, 320, 65, 64)]
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("shape", FWD_SHAPES)
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_forward_kernels(ffk, oracle, shape, causal, variant):
+    """Both forward kernels (option 1 selects the one with 32 query rows per wavefront)."""
+    B, H, Sq, Skv, D = shape
+    say("attention forward", shape, "causal", causal, "variant", variant)
+    g = rng(Sq * 3 + Skv + D + int(causal))
+    q = bf16_round(g.standard_normal((B, Sq, H, D)))
+    k = bf16_round(g.standard_normal((B, Skv, H, D)))
+    v = bf16_round(g.standard_normal((B, Skv, H, D)))
+    scale = 1.0 / np.sqrt(D)
+    o_ref, lse_ref = oracle.attention_forward(q, k, v, scale, causal, bf16_mode=True)
+    ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, variant)
+    try:
+        o, lse = ffk.attention_forward(*(to_dev(a, torch, BT) for a in (q, k, v)), scale, causal)
+    finally:
+        ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, 0)
+    assert_close(to_np(o), o_ref, BF16_RTOL, "O")
+    assert_close(to_np(lse), lse_ref, 1e-3, "lse")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_forward_growing_scores(ffk, oracle, causal):
+    """Keys grow along the sequence, so every tile raises the row maxima: by less than the
+    kernel's threshold for moving its reference point in the first half of the sequence
+    (probabilities above 1 are then summed), by more in the second."""
+    B, H, S, D = 1, 2, 1024, 128
+    say("attention growing scores, causal", causal)
+    g = rng(77 + int(causal))
+    q = bf16_round(np.abs(g.standard_normal((B, S, H, D))) * 0.5)
+    ramp = np.where(np.arange(S) < S // 2, 1.0 + np.arange(S) / S, 1.5 + 12.0 * (np.arange(S) - S // 2) / S)
+    k = bf16_round(np.abs(g.standard_normal((B, S, H, D))) * ramp[None, :, None, None] * 0.25)
+    v = bf16_round(g.standard_normal((B, S, H, D)))
+    scale = 1.0 / np.sqrt(D)
+    o_ref, lse_ref = oracle.attention_forward(q, k, v, scale, causal, bf16_mode=True)
+    o, lse = ffk.attention_forward(*(to_dev(a, torch, BT) for a in (q, k, v)), scale, causal)
+    assert_close(to_np(o), o_ref, BF16_RTOL, "O")
+    assert_close(to_np(lse), lse_ref, 1e-3, "lse")
+
+
 F32_SHAPES = [  # B, H, Sq, Skv, D
     (1, 1, 8, 8, 64), (2, 3, 11, 11, 32), (1, 2, 100, 100, 128), (2, 2, 129, 129, 64), (1, 2, 40, 40, 4),
     (1, 4, 256, 256, 128), (1, 2, 300, 300, 48), (1, 1, 64, 200, 64), (2, 1, 160, 96, 100), (1, 3, 70, 33, 20),
