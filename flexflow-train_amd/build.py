@@ -41,6 +41,7 @@ HIP_FLAGS = [
 EXTRA_FLAGS = {
     "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "attention_fwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-fno-honor-nans"],
+    "attention_bwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "optimizer.hip": ["-ffp-contract=off"],
     "loss.hip": ["-ffp-contract=off"],
 }

@@ -219,16 +219,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 // --------------------------------------------------------------------------
 // backward
 // --------------------------------------------------------------------------
-struct AttnBwdParams {
-  bf16 const *q, *k, *v, *o, *d_o;
-  float const *lse;
-  float *delta;
-  bf16 *dq, *dk, *dv;
-  int B, H, Sq, Skv;
-  int64_t q_bs, q_ss, k_bs, k_ss, v_bs, v_ss, o_bs, o_ss;
-  float scale, scale_log2;
-  int causal;
-};
 
 // delta[b,h,q] = sum_d O * dO.  D/8 lanes share a row (16 bytes each), so a
 // wave covers 64 / (D/8) rows and every access is a whole 128/256-byte row.
@@ -620,6 +610,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
 // 64 query rows per wavefront (attention_fwd.hip)
 hipError_t attention_bf16_forward_wide(hipStream_t st, AttnParams const &p, int head_dim);
 
+// dK/dV with direct loads, two workgroups per CU (attention_bwd.hip)
+hipError_t attention_bf16_dkdv(hipStream_t st, AttnBwdParams const &p, int head_dim);
+bool attention_bf16_bwd_direct_ok(AttnBwdParams const &p);
+
 // the fp32 core (attention_f32.hip)
 int attention_f32_forward(hipStream_t st, ffk_attention_desc_t const *d, void const *q, void const *k,
                           void const *v, void *o, float *lse);
@@ -727,18 +721,27 @@ extern "C" int ffk_attention_backward(ffk_stream_t stream, int dtype,
   p.causal = d->causal;
   hipStream_t st = as_stream(stream);
   int64_t rows = (int64_t)p.B * p.H * p.Sq;
+  bool const direct = option(FFK_OPTION_ATTENTION_VARIANT) != 1 && attention_bf16_bwd_direct_ok(p);
   dim3 gkv((unsigned)(ceil_div(p.Skv, 128) * p.H * p.B));
   dim3 gq((unsigned)(ceil_div(p.Sq, 128) * p.H * p.B));
   if (d->head_dim == 64) {
     attn_delta_kernel<64><<<(unsigned)ceil_div(rows, 4 * 8), 256, 0, st>>>(p);
     FFK_CHECK_LAUNCH();
-    attn_bwd_dkdv_kernel<64><<<gkv, 256, 0, st>>>(p);
+    if (direct) {
+      FFK_HIP(attention_bf16_dkdv(st, p, 64));
+    } else {
+      attn_bwd_dkdv_kernel<64><<<gkv, 256, 0, st>>>(p);
+    }
     FFK_CHECK_LAUNCH();
     attn_bwd_dq_kernel<64><<<gq, 256, 0, st>>>(p);
   } else {
     attn_delta_kernel<128><<<(unsigned)ceil_div(rows, 4 * 4), 256, 0, st>>>(p);
     FFK_CHECK_LAUNCH();
-    attn_bwd_dkdv_kernel<128><<<gkv, 256, 0, st>>>(p);
+    if (direct) {
+      FFK_HIP(attention_bf16_dkdv(st, p, 128));
+    } else {
+      attn_bwd_dkdv_kernel<128><<<gkv, 256, 0, st>>>(p);
+    }
     FFK_CHECK_LAUNCH();
     attn_bwd_dq_kernel<128><<<gq, 256, 0, st>>>(p);
   }

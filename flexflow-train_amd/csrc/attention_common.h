@@ -1,7 +1,8 @@
-// Pieces shared by the bf16 attention kernels: the parameter block of the
-// forward kernels and the LDS fragment readers for the 32x32x16 bf16 MFMA.
+// Pieces shared by the bf16 attention kernels: the parameter blocks of the
+// forward and backward kernels and the LDS fragment readers for the 32x32x16 bf16 MFMA.
 #pragma once
 #include "ffk_common.h"
+#include <type_traits>
 
 namespace ffk {
 
@@ -17,6 +18,17 @@ struct AttnParams {
   int B, H, Sq, Skv;
   int64_t q_bs, q_ss, k_bs, k_ss, v_bs, v_ss, o_bs, o_ss;
   float scale_log2;  // scale * log2(e)
+  int causal;
+};
+
+struct AttnBwdParams {
+  bf16 const *q, *k, *v, *o, *d_o;
+  float const *lse;
+  float *delta;
+  bf16 *dq, *dk, *dv;
+  int B, H, Sq, Skv;
+  int64_t q_bs, q_ss, k_bs, k_ss, v_bs, v_ss, o_bs, o_ss;
+  float scale, scale_log2;
   int causal;
 };
 
@@ -64,5 +76,19 @@ __device__ __forceinline__ bf16x8 frag_tr_acc(bf16 const *tile_plus_lane, int st
   u.h2[1] = hi;
   return u.v;
 }
+
+// Compile-time loop: f(std::integral_constant<int, I>) for I = 0 .. N-1.
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+// Ties a value to this point of the program: the arithmetic that produces it cannot be moved
+// behind it by the optimizer (which otherwise gathers a unit of vector work placed between two
+// MFMAs at the place where its result is first needed).
+__device__ __forceinline__ void pin_here(float &x) { asm volatile("" : "+v"(x)); }
 
 }  // namespace ffk

@@ -110,15 +110,6 @@ struct SoftmaxHalf {
   }
 };
 
-// Compile-time loop: f(std::integral_constant<int, I>) for I = 0 .. N-1.
-template <int I, int N, typename F>
-__device__ __forceinline__ void static_for(F &&f) {
-  if constexpr (I < N) {
-    f(std::integral_constant<int, I>{});
-    static_for<I + 1, N>(f);
-  }
-}
-
 template <int D>
 __global__ __launch_bounds__(256) void attn_fwd_wide_kernel(AttnParams p) {
   using C = AttnFwdCfg<D>;

@@ -36,6 +36,14 @@ __device__ __forceinline__ void lds_dma16(i32x4 rsrc, unsigned lane_byte_off, un
                              // reserved registers there); nothing else in these
                              // kernels uses M0 (no GDS, message or relative-move ops)
 }
+// The same for 4 bytes per lane: lane l's dword lands at lds_base + 4 l.
+__device__ __forceinline__ void lds_dma4(i32x4 rsrc, unsigned lane_byte_off, unsigned uniform_byte_off,
+                                         unsigned lds_byte_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :
+               : "s"(lds_byte_addr), "v"(lane_byte_off), "s"(rsrc), "s"(uniform_byte_off)
+               : "memory");
+}
 // Raw buffer descriptor over num_bytes bytes from `base` on (by default no bound: stride 0,
 // the offsets are then checked on the host), 32-bit data format.
 __device__ __forceinline__ i32x4 buffer_resource(void const *base, unsigned num_bytes = 0xffffffffu) {

@@ -131,7 +131,8 @@ int ffk_event_elapsed_ms(ffk_event_t start, ffk_event_t stop, float *ms);
  *     one kernel per operator.
  *   FFK_OPTION_ATTENTION_VARIANT (FFK_ATTENTION_VARIANT): 0 = the default bf16
  *     attention kernels; 1 = the forward kernel with 32 query rows per
- *     wavefront (two workgroups per CU) that the default one replaced.       */
+ *     wavefront (two workgroups per CU) and the dK/dV kernel with 32-row
+ *     query tiles that the default ones replaced.                            */
 enum {
   FFK_OPTION_GEMM_VARIANT = 0,
   FFK_OPTION_LAYER_UNFUSED = 1,
