@@ -125,7 +125,8 @@ int ffk_event_elapsed_ms(ffk_event_t start, ffk_event_t stop, float *ms);
  * reference.  Each starts from the environment variable of the same name,
  * read once when the library is loaded.
  *   FFK_OPTION_GEMM_VARIANT (FFK_GEMM_VARIANT): 0 = the dispatch heuristic;
- *     128 / 256 force that pipelined bf16 tile, 1 the register-staged kernel.
+ *     128 / 256 force that pipelined bf16 tile (eight waves), 264 the 256 tile
+ *     with one wave per SIMD, 1 the register-staged kernel.
  *   FFK_OPTION_LAYER_UNFUSED (FFK_LAYER_UNFUSED): != 0 makes the encoder-layer
  *     entry points (and a step-driver instance created while it is set) run
  *     one kernel per operator.
