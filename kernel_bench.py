@@ -74,6 +74,14 @@ def bench_gemm():
         t = timeit(lambda: ffk.gemm(A, B, C, bool(ta), bool(tb)))
         report("gemm bf16 M%d N%d K%d %s%s" % (M, N, K, "T" if ta else "N", "T" if tb else "N"), t,
                flops=2.0 * M * N * K)
+        if K >= 2048 and M % 256 == 0 and N % 256 == 0 and (M // 256) * (N // 256) >= 192:
+            # the eight-wave 256x256 kernel that the one-wave-per-SIMD kernel replaced at these sizes
+            ffk.set_option(ffk.OPTION_GEMM_VARIANT, 256)
+            try:
+                t = timeit(lambda: ffk.gemm(A, B, C, bool(ta), bool(tb)))
+            finally:
+                ffk.set_option(ffk.OPTION_GEMM_VARIANT, 0)
+            report("  previous kernel (8 waves, 4 x 32-deep stages)", t, flops=2.0 * M * N * K)
 
 
 def bench_fused_linear():
@@ -218,6 +226,15 @@ def bench_attention():
         report("attention fwd B%d H%d S%d D%d causal=%d" % (B, H, S, D, causal), t, flops=f)
         t = timeit(lambda: ffk.attention_backward(q, k, v, o, do, lse, scale, causal), iters=10)
         report("attention bwd B%d H%d S%d D%d causal=%d" % (B, H, S, D, causal), t, flops=2.5 * f)
+        # the kernels these replaced: 32 query rows per wavefront forward, 32-row tiles in dK/dV
+        ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, 1)
+        try:
+            t = timeit(lambda: ffk.attention_forward(q, k, v, scale, causal), iters=10)
+            report("  previous forward kernel", t, flops=f)
+            t = timeit(lambda: ffk.attention_backward(q, k, v, o, do, lse, scale, causal), iters=10)
+            report("  previous dK/dV kernel in the backward", t, flops=2.5 * f)
+        finally:
+            ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, 0)
 
 
 def bench_update():
