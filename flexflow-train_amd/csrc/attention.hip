@@ -668,7 +668,14 @@ extern "C" int ffk_attention_forward(ffk_stream_t stream, int dtype,
   p.o_bs = d->o_batch_stride; p.o_ss = d->o_seq_stride;
   p.scale_log2 = d->scale * kLog2e;
   p.causal = d->causal;
-  if (option(FFK_OPTION_ATTENTION_VARIANT) != 1) {
+  // 64 query rows per wavefront (256 per workgroup, one workgroup per CU) pay from about a
+  // thousand keys on and when the problem still gives every CU a workgroup; below that the
+  // kernel with 32 rows per wavefront and two workgroups per CU is ahead (config 2's 512 keys:
+  // 18.5 against 19.4 us).
+  int const variant = option(FFK_OPTION_ATTENTION_VARIANT);
+  bool const wide = variant == 2 || (variant == 0 && p.Skv >= 1024 &&
+                                     ceil_div(p.Sq, 256) * (int64_t)p.H * p.B >= kNumCU);
+  if (wide) {
     FFK_HIP(attention_bf16_forward_wide(as_stream(stream), p, (int)d->head_dim));
     return FFK_OK;
   }

@@ -131,9 +131,11 @@ int ffk_event_elapsed_ms(ffk_event_t start, ffk_event_t stop, float *ms);
  *     entry points (and a step-driver instance created while it is set) run
  *     one kernel per operator.
  *   FFK_OPTION_ATTENTION_VARIANT (FFK_ATTENTION_VARIANT): 0 = the default bf16
- *     attention kernels; 1 = the forward kernel with 32 query rows per
- *     wavefront (two workgroups per CU) and the dK/dV kernel with 32-row
- *     query tiles that the default ones replaced.                            */
+ *     attention kernels (forward: 64 query rows per wavefront from 1024 keys
+ *     on, 32 below; dK/dV: 64-row query tiles as two pipelined halves);
+ *     1 = the forward kernel with 32 query rows per wavefront and the dK/dV
+ *     kernel with 32-row query tiles at every size; 2 = the forward kernel
+ *     with 64 query rows per wavefront at every size.                        */
 enum {
   FFK_OPTION_GEMM_VARIANT = 0,
   FFK_OPTION_LAYER_UNFUSED = 1,

@@ -52,11 +52,12 @@ def test_attention_core(ffk, oracle, shape, causal):
 FWD_SHAPES = [(1, 2, 600, 600, 128), (1, 1, 257, 705, 64), (1, 1, 513, 513, 128), (2, 1, 33, 449, 128), (1, 2, 320, 65, 64)]
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [2, 1])
 @pytest.mark.parametrize("shape", FWD_SHAPES)
 @pytest.mark.parametrize("causal", [False, True])
 def test_attention_forward_kernels(ffk, oracle, shape, causal, variant):
-    """Both forward kernels (option 1 selects the one with 32 query rows per wavefront)."""
+    """Both forward kernels at every shape (option 2: 64 query rows per wavefront, option 1: 32;
+    the default picks by size)."""
     B, H, Sq, Skv, D = shape
     say("attention forward", shape, "causal", causal, "variant", variant)
     g = rng(Sq * 3 + Skv + D + int(causal))
@@ -118,7 +119,11 @@ def test_attention_forward_growing_scores(ffk, oracle, causal):
     v = bf16_round(g.standard_normal((B, S, H, D)))
     scale = 1.0 / np.sqrt(D)
     o_ref, lse_ref = oracle.attention_forward(q, k, v, scale, causal, bf16_mode=True)
-    o, lse = ffk.attention_forward(*(to_dev(a, torch, BT) for a in (q, k, v)), scale, causal)
+    ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, 2)  # the kernel with the lazily moved reference point
+    try:
+        o, lse = ffk.attention_forward(*(to_dev(a, torch, BT) for a in (q, k, v)), scale, causal)
+    finally:
+        ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, 0)
     assert_close(to_np(o), o_ref, BF16_RTOL, "O")
     assert_close(to_np(lse), lse_ref, 1e-3, "lse")
 
