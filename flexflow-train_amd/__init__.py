@@ -109,6 +109,8 @@ SIGNATURES = {
                                            c_i64]),
     "ffk_element_binary_backward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_p, c_p, c_i64,
                                             c_int]),
+    "ffk_element_binary_backward_broadcast": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_p, c_p, c_i64,
+                                                      c_i64, c_i64, c_int]),
     "ffk_layer_norm_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_i64, c_i64,
                                        c_f]),
     "ffk_layer_norm_backward_workspace_bytes": (c_sz, [c_i64, c_i64]),
@@ -340,6 +342,14 @@ def element_binary_backward(op, g, l, r, dl, dr, accumulate=False):
     check(lib().ffk_element_binary_backward(current_stream(), dtype_of(g), op, ptr(g), ptr(l),
                                             ptr(r), ptr(dl), ptr(dr), g.numel(),
                                             int(accumulate)))
+    return dl, dr
+
+
+def element_binary_backward_broadcast(op, g, l, r, dl, dr, accumulate=False):
+    """Backward with operands that were broadcast over the leading dims; dl / dr may be None."""
+    check(lib().ffk_element_binary_backward_broadcast(
+        current_stream(), dtype_of(g), op, ptr(g), ptr(l), ptr(r), ptr(dl) if dl is not None else None,
+        ptr(dr) if dr is not None else None, g.numel(), l.numel(), r.numel(), int(accumulate)))
     return dl, dr
 
 

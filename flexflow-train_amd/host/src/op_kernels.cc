@@ -403,10 +403,19 @@ void backward_kernel(device_stream_t const &stream, std::optional<ElementBinaryP
                      float const *dout, float const *lhs, float const *rhs, float *dl, float *dr,
                      OperatorType op_type, bool bl, bool br, device_handle_t const &) {
   if (!stream.is_gpu()) no_cpu("ElementBinary::backward_kernel");
-  if (bl || br) throw std::runtime_error("ElementBinary::backward_kernel: broadcast gradients are not supported "
-                                         "(shape inference rejects broadcasting, op-attrs/ops/element_binary.cc:5-21)");
+  ElementBinaryPerDeviceState const &s = state.value();
+  if (bl || br || dl == nullptr || dr == nullptr) {
+    // the reference's broadcast_inputLHS / broadcast_inputRHS branches (a reduction of the output
+    // gradient, element_binary_kernels.cu:268-396) and its NULL-gradient checks
+    check_ffk(ffk_element_binary_backward_broadcast(stream.require_gpu(), FFK_FLOAT, static_cast<int>(op_type), dout,
+                                                    lhs, rhs, dl, dr, get_num_elements(s.output_shape.dims),
+                                                    get_num_elements(s.lhs_shape.dims),
+                                                    get_num_elements(s.rhs_shape.dims), 1),
+              "ElementBinary::backward_kernel");
+    return;
+  }
   check_ffk(ffk_element_binary_backward(stream.require_gpu(), FFK_FLOAT, static_cast<int>(op_type), dout, lhs, rhs,
-                                        dl, dr, get_num_elements(state.value().output_shape.dims), 1),
+                                        dl, dr, get_num_elements(s.output_shape.dims), 1),
             "ElementBinary::backward_kernel");
 }
 void forward_kernel(device_stream_t const &stream, std::optional<ElementBinaryPerDeviceState> const &state,

@@ -382,6 +382,44 @@ static void gpu_tests() {
     }
   });
 
+  run("ElementBinary with a broadcast operand: its gradient is the reduction the reference asks cuDNN for", [&] {
+    // element_binary_kernels.cu:268-396 (broadcast_inputRHS): add reduces dy, mul reduces dy * lhs
+    int64_t rows = 50, cols = 100;
+    size_t n = rows * cols;
+    auto x = random_vec(n, 31, -2, 2), b = random_vec(cols, 32, 0.5f, 2.0f), dy = random_vec(n, 33);
+    TensorShape s = shape({rows, cols}, DataType::FLOAT), sb = shape({cols}, DataType::FLOAT);
+    auto X = device_accessor(gpu, s, x), B = device_accessor(gpu, sb, b), DY = device_accessor(gpu, s, dy);
+    auto Y = gpu.allocate_tensor(s), DX = gpu.allocate_tensor(s), DB = gpu.allocate_tensor(sb);
+    for (OperatorType op : {OperatorType::EW_ADD, OperatorType::EW_MUL}) {
+      bool const mul = op == OperatorType::EW_MUL;
+      auto bstate = Kernels::ElementBinary::init_kernel(DeviceType::GPU, handle, op, false, true, s, sb, s);
+      std::vector<float> o(n), dl(n), dr(cols);
+      for (int64_t j = 0; j < cols; j++) {
+        double acc = 0.0;
+        for (int64_t i = 0; i < rows; i++) {
+          size_t k = i * cols + j;
+          o[k] = mul ? x[k] * b[j] : x[k] + b[j];
+          dl[k] = mul ? dy[k] * b[j] : dy[k];
+          acc += mul ? (double)dy[k] * x[k] : (double)dy[k];
+        }
+        dr[j] = (float)acc;
+      }
+      Kernels::ElementBinary::forward_kernel(stream, bstate, X.get_float_ptr(), B.get_float_ptr(), Y.get_float_ptr(),
+                                             op, false, handle);
+      CHECK(close(to_host(Y), o, 1e-6));
+      fill_with_zeros(DX); fill_with_zeros(DB);
+      Kernels::ElementBinary::backward_kernel(stream, bstate, DY.get_float_ptr(), X.get_float_ptr(), B.get_float_ptr(),
+                                              DX.get_float_ptr(), DB.get_float_ptr(), op, false, true, handle);
+      CHECK(close(to_host(DX), dl, 1e-6));
+      CHECK(close(to_host(DB), dr, 1e-5));
+      // a second call adds (the reference's beta = 1)
+      Kernels::ElementBinary::backward_kernel(stream, bstate, DY.get_float_ptr(), X.get_float_ptr(), B.get_float_ptr(),
+                                              nullptr, DB.get_float_ptr(), op, false, true, handle);
+      for (auto &v : dr) v *= 2.0f;
+      CHECK(close(to_host(DB), dr, 1e-5));
+    }
+  });
+
   run("Embedding gather (exact) and scatter-add vs oracle", [&] {
     int64_t V = 97, D = 32, B = 40, bag = 4;
     auto w = random_vec(V * D, 15), dy = random_vec(B * D, 16);

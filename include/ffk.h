@@ -228,6 +228,19 @@ int ffk_element_binary_backward(ffk_stream_t stream, int dtype, int op_type,
                                 void const *out_grad, void const *lhs,
                                 void const *rhs, void *lhs_grad, void *rhs_grad,
                                 int64_t out_elems, int accumulate);
+/* The backward when an operand was broadcast (the reference's broadcast_inputLHS /
+ * broadcast_inputRHS branches, element_binary_kernels.cu:268-396: EW_ADD, EW_SUB,
+ * EW_MUL; other ops answer FFK_ERR_UNSUPPORTED).  An operand with out_elems
+ * elements gets its element-wise gradient; one with fewer gets the sum over the
+ * output elements it was broadcast to (index i % operand_elems), added up in a
+ * fixed order in fp32.  lhs_grad / rhs_grad may be NULL (that gradient is not
+ * computed, as in the reference); accumulate != 0 adds into them (the reference's
+ * beta = 1), 0 stores.  EW_MUL reads the other operand of each gradient.      */
+int ffk_element_binary_backward_broadcast(ffk_stream_t stream, int dtype, int op_type,
+                                          void const *out_grad, void const *lhs,
+                                          void const *rhs, void *lhs_grad, void *rhs_grad,
+                                          int64_t out_elems, int64_t lhs_elems,
+                                          int64_t rhs_elems, int accumulate);
 
 /* ------------------------------------------------------------------------ */
 /* LayerNorm -- Kernels::LayerNorm::gpu_forward_kernel / gpu_backward_kernel

@@ -199,6 +199,36 @@ def element_binary_backward(op, g, l, r, dl_init=None, dr_init=None, accumulate=
     return dl, dr
 
 
+def element_binary_backward_broadcast(op, g, l, r, dl_init=None, dr_init=None, accumulate=0):
+    """Gradients when an operand was broadcast over the leading dims (operand index = output index
+    modulo the operand's size): what lib/kernels/src/cuda/ops/element_binary_kernels.cu:268-396 asks
+    cuDNN for -- add / sub: reduce dy (sub negates the rhs); mul: reduce dy * other operand -- each
+    added into (accumulate) or stored to the operand's gradient.  Sums in float64, rounded once."""
+    g, l, r = _f32(g), _f32(l), _f32(r)
+    n = g.size
+    OP_EW_ADD, OP_EW_MUL, OP_EW_SUB = 28, 29, 35  # OperatorType ordinals (op-attrs/operator_type.dtg.toml order)
+
+    def spread(a):
+        return np.resize(a.reshape(-1), n).astype(np.float64)  # a[i % a.size]
+
+    gl = g.reshape(-1).astype(np.float64)
+    if op == OP_EW_ADD:
+        tl, tr = gl, gl
+    elif op == OP_EW_SUB:
+        tl, tr = gl, -gl
+    elif op == OP_EW_MUL:
+        tl, tr = gl * spread(r), gl * spread(l)
+    else:
+        raise ValueError("no broadcast gradient for binary op %d" % op)
+    out = []
+    for term, operand, init in ((tl, l, dl_init), (tr, r, dr_init)):
+        red = term.reshape(-1, operand.size).sum(axis=0)
+        if accumulate and init is not None:
+            red = red + _f32(init).reshape(-1).astype(np.float64)
+        out.append(red.astype(np.float32).reshape(operand.shape))
+    return out[0], out[1]
+
+
 def layer_norm_forward(x, gamma, beta, eps):
     x = _f32(x)
     M, N = x.shape

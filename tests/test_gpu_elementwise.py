@@ -109,6 +109,52 @@ def test_binary_broadcast_rhs(ffk, oracle, dtype):
                                    out=torch.empty((65, 48), dtype=tdt, device="cuda"))
 
 
+@pytest.mark.parametrize("name", ["EW_ADD", "EW_SUB", "EW_MUL"])
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("shapes", [((65, 48), (65, 48), (48,)), ((300, 7, 130), (130,), (300, 7, 130)),
+                                    ((1000, 70), (70,), (70,)), ((5, 3, 64), (3, 64), (64,))])
+def test_binary_broadcast_gradients(ffk, oracle, name, dtype, shapes):
+    """The reference's broadcast_inputLHS / broadcast_inputRHS branches: a smaller operand's
+    gradient is the sum over the output elements it was broadcast to."""
+    out_shape, ls, rs = shapes
+    say("binary broadcast gradients", name, dtype, shapes)
+    op = ffk.OP[name]
+    g = rng(47)
+    l = g.uniform(0.5, 2, ls).astype(np.float32)
+    r = g.uniform(0.5, 2, rs).astype(np.float32)
+    dy = g.standard_normal(out_shape).astype(np.float32)
+    i1 = g.standard_normal(ls).astype(np.float32)
+    i2 = g.standard_normal(rs).astype(np.float32)
+    tdt, rtol = (torch.float32, FP32_RTOL) if dtype == "fp32" else (torch.bfloat16, BF16_RTOL)
+    if dtype == "bf16":
+        l, r, dy, i1, i2 = (bf16_round(a) for a in (l, r, dy, i1, i2))
+    ld, rd, dyd = (to_dev(a, torch, tdt) for a in (l, r, dy))
+    for acc in (0, 1):
+        dl, dr = to_dev(i1, torch, tdt), to_dev(i2, torch, tdt)
+        ffk.element_binary_backward_broadcast(op, dyd, ld, rd, dl, dr, accumulate=bool(acc))
+        wl, wr = oracle.element_binary_backward_broadcast(op, dy, l, r, i1, i2, accumulate=acc)
+        assert_close(to_np(dl), wl, rtol, "dl acc=%d" % acc)
+        assert_close(to_np(dr), wr, rtol, "dr acc=%d" % acc)
+    # one gradient only, as the reference allows
+    dr = to_dev(i2, torch, tdt)
+    ffk.element_binary_backward_broadcast(op, dyd, ld, rd, None, dr, accumulate=False)
+    assert_close(to_np(dr), oracle.element_binary_backward_broadcast(op, dy, l, r)[1], rtol, "dr alone")
+    # twice the same call: the same bits (fixed summation order)
+    dr2 = to_dev(i2, torch, tdt)
+    ffk.element_binary_backward_broadcast(op, dyd, ld, rd, None, dr2, accumulate=False)
+    assert torch.equal(dr, dr2)
+
+
+def test_binary_broadcast_gradients_refusals(ffk):
+    x = torch.ones((8, 4), device="cuda")
+    b = torch.ones((4,), device="cuda")
+    with pytest.raises(ffk.FFKError, match="no broadcast gradient"):
+        ffk.element_binary_backward_broadcast(ffk.OP["EW_MAX"], x, x, b, torch.empty_like(x), torch.empty_like(b))
+    with pytest.raises(ffk.FFKError, match="broadcast"):
+        ffk.element_binary_backward_broadcast(ffk.OP["EW_ADD"], x, x, torch.ones((3,), device="cuda"),
+                                              torch.empty_like(x), torch.empty((3,), device="cuda"))
+
+
 @pytest.mark.parametrize("n,offset", [(1, 0), (4099, 0), (65536 + 3, 8), (5000, 3), (70001, 1 << 33)])
 @pytest.mark.parametrize("rate", [0.1, 0.5, 0.0, 1.0])
 def test_dropout_mask_bit_exact(ffk, oracle, n, offset, rate):

@@ -100,6 +100,30 @@ def test_gelu_reference_grad_is_the_literal_formula(oracle):
     assert not np.allclose(got, true, atol=1e-3)  # the two formulas do differ
 
 
+@pytest.mark.parametrize("name", ["EW_ADD", "EW_SUB", "EW_MUL"])
+@pytest.mark.parametrize("shapes", [((6, 5, 8), (8,), (6, 5, 8)), ((7, 12), (7, 12), (12,)), ((4, 3, 10), (3, 10), (10,))])
+def test_element_binary_broadcast_gradients_against_autograd(oracle, name, shapes):
+    """A trailing-dims operand is what torch broadcasts too: its gradient is autograd's reduction."""
+    out_shape, ls, rs = shapes
+    g = np.random.default_rng(5)
+    l64, r64 = g.standard_normal(ls), g.standard_normal(rs)
+    dy = g.standard_normal(out_shape).astype(np.float32)
+    fn = dict(EW_ADD=torch.add, EW_SUB=torch.sub, EW_MUL=torch.mul)[name]
+    lt = torch.tensor(l64.astype(np.float32), dtype=torch.float64, requires_grad=True)
+    rt = torch.tensor(r64.astype(np.float32), dtype=torch.float64, requires_grad=True)
+    fn(lt.expand(out_shape), rt.expand(out_shape)).backward(torch.tensor(dy, dtype=torch.float64))
+    dl, dr = oracle.element_binary_backward_broadcast(OP[name], dy, l64.astype(np.float32), r64.astype(np.float32))
+    assert dl.shape == ls and dr.shape == rs
+    assert np.allclose(dl, lt.grad.numpy(), rtol=1e-6, atol=1e-6)
+    assert np.allclose(dr, rt.grad.numpy(), rtol=1e-6, atol=1e-6)
+    # accumulate adds to what was there
+    i1, i2 = g.standard_normal(ls).astype(np.float32), g.standard_normal(rs).astype(np.float32)
+    dl2, dr2 = oracle.element_binary_backward_broadcast(OP[name], dy, l64.astype(np.float32), r64.astype(np.float32),
+                                                        i1, i2, accumulate=1)
+    assert np.allclose(dl2, lt.grad.numpy() + i1, rtol=1e-6, atol=1e-6)
+    assert np.allclose(dr2, rt.grad.numpy() + i2, rtol=1e-6, atol=1e-6)
+
+
 @pytest.mark.parametrize("name", ["EW_ADD", "EW_SUB", "EW_MUL", "EW_DIV", "EW_MAX", "EW_MIN"])
 def test_binary_against_autograd(oracle, name):
     g = rng(4)
