@@ -16,7 +16,8 @@
 //                accumulates dK, dV in registers;
 //            (B) one workgroup = 128 query rows, loops over key tiles and
 //                accumulates dQ in registers.
-//            Both recompute P from the saved log-sum-exp.
+//            Both recompute P from the saved log-sum-exp.  (B) runs first: it also computes
+//            delta = rowsum(O * dO) for its rows and leaves it in memory for (A).
 //
 // MFMA 32x32x16 bf16 register layouts used throughout (l = lane):
 //   A operand: row l%32, k = 8*(l/32) .. +7      B operand: column l%32, same k
@@ -219,37 +220,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 // --------------------------------------------------------------------------
 // backward
 // --------------------------------------------------------------------------
-
-// delta[b,h,q] = sum_d O * dO.  D/8 lanes share a row (16 bytes each), so a
-// wave covers 64 / (D/8) rows and every access is a whole 128/256-byte row.
-template <int D>
-__global__ __launch_bounds__(256) void attn_delta_kernel(AttnBwdParams p) {
-  constexpr int LPR = D / 8;        // lanes per row
-  constexpr int RPW = 64 / LPR;     // rows per wave
-  int const lane = threadIdx.x & 63;
-  int64_t const row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / LPR;
-  int64_t const total = (int64_t)p.B * p.H * p.Sq;
-  float s = 0.0f;
-  if (row < total) {
-    // rows are numbered (b, q, h) so that neighbouring rows are neighbours in memory
-    int const head = (int)(row % p.H);
-    int const q = (int)((row / p.H) % p.Sq);
-    int const b = (int)(row / ((int64_t)p.Sq * p.H));
-    int64_t const off = (int64_t)b * p.o_bs + (int64_t)q * p.o_ss + (int64_t)head * D + (lane % LPR) * 8;
-    float o[8], g[8];
-    VecIO<bf16>::load(p.o + off, o);
-    VecIO<bf16>::load(p.d_o + off, g);
-#pragma unroll
-    for (int e = 0; e < 8; e++) s += o[e] * g[e];
-#pragma unroll
-    for (int m = 1; m < LPR; m <<= 1) s += __shfl_xor(s, m, 64);
-    if (lane % LPR == 0) p.delta[((int64_t)b * p.H + head) * p.Sq + q] = s;
-  } else {
-    // keep the shuffles convergent for the tail wave
-#pragma unroll
-    for (int m = 1; m < LPR; m <<= 1) s += __shfl_xor(s, m, 64);
-  }
-}
 
 template <int D>
 struct AttnBwdCfg {
@@ -491,7 +461,21 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
       gf[kk] = *reinterpret_cast<bf16x8 const *>(gp + (int64_t)r * p.o_ss + kk * 16 + h32 * 8);
     }
     lse2 = p.lse[((int64_t)b * p.H + head) * p.Sq + r] * kLog2e;
-    delta_s = p.delta[((int64_t)b * p.H + head) * p.Sq + r] * p.scale;
+    // delta = sum_d O * dO of this lane's row: the lane holds half of the row's d (8 of every 16),
+    // its partner l ^ 32 the other half.  The kernel that owns a query row is the one place that
+    // has the row's dO in registers anyway; it leaves delta in memory for the dK/dV kernel, which
+    // runs after it.
+    bf16 const *op = p.o + (int64_t)b * p.o_bs + (int64_t)head * D;
+    float part = 0.0f;
+#pragma unroll
+    for (int kk = 0; kk < D / 16; kk++) {
+      bf16x8 const of = *reinterpret_cast<bf16x8 const *>(op + (int64_t)r * p.o_ss + kk * 16 + h32 * 8);
+#pragma unroll
+      for (int e = 0; e < 8; e++) part += (float)of[e] * (float)gf[kk][e];
+    }
+    float const delta = part + __shfl_xor(part, 32, 64);
+    if (h32 == 0 && qrow < p.Sq) p.delta[((int64_t)b * p.H + head) * p.Sq + qrow] = delta;
+    delta_s = delta * p.scale;
   }
   f32x16 dq[D / 32];
 #pragma unroll
@@ -727,30 +711,26 @@ extern "C" int ffk_attention_backward(ffk_stream_t stream, int dtype,
   p.scale_log2 = d->scale * kLog2e;
   p.causal = d->causal;
   hipStream_t st = as_stream(stream);
-  int64_t rows = (int64_t)p.B * p.H * p.Sq;
   bool const direct = option(FFK_OPTION_ATTENTION_VARIANT) != 1 && attention_bf16_bwd_direct_ok(p);
   dim3 gkv((unsigned)(ceil_div(p.Skv, 128) * p.H * p.B));
   dim3 gq((unsigned)(ceil_div(p.Sq, 128) * p.H * p.B));
+  // dQ first: it computes delta for its rows and leaves it in `delta` for the dK/dV kernel
   if (d->head_dim == 64) {
-    attn_delta_kernel<64><<<(unsigned)ceil_div(rows, 4 * 8), 256, 0, st>>>(p);
+    attn_bwd_dq_kernel<64><<<gq, 256, 0, st>>>(p);
     FFK_CHECK_LAUNCH();
     if (direct) {
       FFK_HIP(attention_bf16_dkdv(st, p, 64));
     } else {
       attn_bwd_dkdv_kernel<64><<<gkv, 256, 0, st>>>(p);
     }
-    FFK_CHECK_LAUNCH();
-    attn_bwd_dq_kernel<64><<<gq, 256, 0, st>>>(p);
   } else {
-    attn_delta_kernel<128><<<(unsigned)ceil_div(rows, 4 * 4), 256, 0, st>>>(p);
+    attn_bwd_dq_kernel<128><<<gq, 256, 0, st>>>(p);
     FFK_CHECK_LAUNCH();
     if (direct) {
       FFK_HIP(attention_bf16_dkdv(st, p, 128));
     } else {
       attn_bwd_dkdv_kernel<128><<<gkv, 256, 0, st>>>(p);
     }
-    FFK_CHECK_LAUNCH();
-    attn_bwd_dq_kernel<128><<<gq, 256, 0, st>>>(p);
   }
   FFK_CHECK_LAUNCH();
   return FFK_OK;
