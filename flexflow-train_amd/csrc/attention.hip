@@ -657,8 +657,10 @@ extern "C" int ffk_attention_forward(ffk_stream_t stream, int dtype,
   // kernel with 32 rows per wavefront and two workgroups per CU is ahead (config 2's 512 keys:
   // 18.5 against 19.4 us).
   int const variant = option(FFK_OPTION_ATTENTION_VARIANT);
-  bool const wide = variant == 2 || (variant == 0 && p.Skv >= 1024 &&
-                                     ceil_div(p.Sq, 256) * (int64_t)p.H * p.B >= kNumCU);
+  // (its direct loads address a 64-row tile with 32-bit byte offsets per lane)
+  bool const wide_ok = p.k_ss < (int64_t(1) << 24) && p.v_ss < (int64_t(1) << 24);
+  bool const wide = wide_ok && (variant == 2 || (variant == 0 && p.Skv >= 1024 &&
+                                                 ceil_div(p.Sq, 256) * (int64_t)p.H * p.B >= kNumCU));
   if (wide) {
     FFK_HIP(attention_bf16_forward_wide(as_stream(stream), p, (int)d->head_dim));
     return FFK_OK;
