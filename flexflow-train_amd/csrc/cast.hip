@@ -5,6 +5,7 @@
 // Any pair of {bool, int32, int64, half, float, double, bf16}; conversions follow
 // C++ static_cast except float -> bf16/half, which round to nearest even.
 #include "ffk_common.h"
+#include <type_traits>
 
 namespace ffk {
 
@@ -78,23 +79,84 @@ constexpr int cast_pack_width() {
   return (sizeof(IDT) > 4 || sizeof(ODT) > 4) ? 4 : 8;
 }
 
-template <typename IDT, typename ODT, bool BACKWARD>
+// A pack moved in its widest aligned units (16, 8 or 4 bytes); STREAM: past the caches, for
+// tensors that neither fit them nor are read again soon.
+template <typename P>
+struct PackUnit {
+  using type = std::conditional_t<sizeof(P) >= 16, u32x4, std::conditional_t<sizeof(P) == 8, uint64_t, uint32_t>>;
+  static_assert(sizeof(P) % sizeof(type) == 0 && alignof(P) >= (sizeof(P) >= 16 ? 16 : sizeof(P)), "pack layout");
+};
+template <bool STREAM, typename P>
+__device__ __forceinline__ P load_pack(P const *p) {
+  using U = typename PackUnit<P>::type;
+  union {
+    P pack;
+    U u[sizeof(P) / sizeof(U)];
+  } x;
+#pragma unroll
+  for (unsigned i = 0; i < sizeof(P) / sizeof(U); i++) {
+    U const *src = reinterpret_cast<U const *>(p) + i;
+    x.u[i] = STREAM ? __builtin_nontemporal_load(src) : *src;
+  }
+  return x.pack;
+}
+template <bool STREAM, typename P>
+__device__ __forceinline__ void store_pack(P *p, P const &v) {
+  using U = typename PackUnit<P>::type;
+  union {
+    P pack;
+    U u[sizeof(P) / sizeof(U)];
+  } x;
+  x.pack = v;
+#pragma unroll
+  for (unsigned i = 0; i < sizeof(P) / sizeof(U); i++) {
+    U *dst = reinterpret_cast<U *>(p) + i;
+    if (STREAM) {
+      __builtin_nontemporal_store(x.u[i], dst);
+    } else {
+      *dst = x.u[i];
+    }
+  }
+}
+
+// Two packs per thread and iteration: all loads of both are issued before the first conversion.
+template <typename IDT, typename ODT, bool BACKWARD, bool STREAM>
 __global__ __launch_bounds__(kCastThreads) void cast_vec_kernel(IDT const *__restrict__ in, ODT *out, int64_t n) {
   constexpr int V = cast_pack_width<IDT, ODT>();
+  using PI = CastPack<IDT, V>;
+  using PO = CastPack<ODT, V>;
   int64_t const packs = n / V;
   int64_t const stride = (int64_t)gridDim.x * kCastThreads;
   int64_t const tid = (int64_t)blockIdx.x * kCastThreads + threadIdx.x;
-  for (int64_t p = tid; p < packs; p += stride) {
-    CastPack<IDT, V> const a = reinterpret_cast<CastPack<IDT, V> const *>(in)[p];
-    CastPack<ODT, V> o;
-    if (BACKWARD) o = reinterpret_cast<CastPack<ODT, V> const *>(out)[p];
+  PI const *pin = reinterpret_cast<PI const *>(in);
+  PO *pout = reinterpret_cast<PO *>(out);
+  auto convert_pack = [](PI const &a, PO &o) {
 #pragma unroll
     for (int e = 0; e < V; e++) {
       ODT c = convert<ODT, IDT>(a.v[e]);
       if (BACKWARD) c = add_in_type<ODT>(c, o.v[e]);
       o.v[e] = c;
     }
-    reinterpret_cast<CastPack<ODT, V> *>(out)[p] = o;
+  };
+  int64_t p = tid;
+  for (; p + stride < packs; p += 2 * stride) {
+    PI const a0 = load_pack<STREAM>(pin + p), a1 = load_pack<STREAM>(pin + p + stride);
+    PO o0, o1;
+    if (BACKWARD) {
+      o0 = load_pack<STREAM>(pout + p);
+      o1 = load_pack<STREAM>(pout + p + stride);
+    }
+    convert_pack(a0, o0);
+    convert_pack(a1, o1);
+    store_pack<STREAM>(pout + p, o0);
+    store_pack<STREAM>(pout + p + stride, o1);
+  }
+  if (p < packs) {
+    PI const a = load_pack<STREAM>(pin + p);
+    PO o;
+    if (BACKWARD) o = load_pack<STREAM>(pout + p);
+    convert_pack(a, o);
+    store_pack<STREAM>(pout + p, o);
   }
   int64_t const j = packs * V + tid;
   if (j < n) {
@@ -115,8 +177,15 @@ static hipError_t cast_launch(hipStream_t st, void const *in, void *out, int64_t
   IDT const *ip = static_cast<IDT const *>(in);
   ODT *op = static_cast<ODT *>(out);
   if (vec) {
-    if (backward) cast_vec_kernel<IDT, ODT, true><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
-    else cast_vec_kernel<IDT, ODT, false><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
+    // input and output together beyond half the last-level cache: move them past the caches
+    bool const stream = (double)n * (sizeof(IDT) + sizeof(ODT)) > 128.0 * 1024 * 1024;
+    if (backward) {
+      if (stream) cast_vec_kernel<IDT, ODT, true, true><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
+      else cast_vec_kernel<IDT, ODT, true, false><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
+    } else {
+      if (stream) cast_vec_kernel<IDT, ODT, false, true><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
+      else cast_vec_kernel<IDT, ODT, false, false><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
+    }
   } else {
     if (backward) cast_kernel<IDT, ODT, true><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
     else cast_kernel<IDT, ODT, false><<<blocks, kCastThreads, 0, st>>>(ip, op, n);
