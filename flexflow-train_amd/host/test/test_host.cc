@@ -3,7 +3,6 @@
 // the entry point, copy back, compare).  The CPU oracle is the checker.
 //   test_host --cpu   host-only checks (no device needed)
 //   test_host --gpu   every operator entry point on the device
-//   test_host --bench-step [steps]   times the step driver on the encoder layer
 #include "ffk_oracle.h"
 #include "kernels/allocation.h"
 #include "kernels/attention_kernels.h"
@@ -1215,87 +1214,14 @@ static void gpu_tests() {
   });
 }
 
-// One training step of the BASELINE encoder layer (pre-LN, GELU, dropout 0.1,
-// batch 8 x 512 tokens, d_model 1024, 16 heads, FFN 4096, BF16) run through the
-// step driver, operator by operator, with SGD.
-static void bench_step(int steps) {
-  ManagedPerDeviceFFHandle managed = initialize_single_gpu_handle(1 << 20, true);
-  device_handle_t handle = device_handle_t_from_managed_ff_handle(managed);
-  Allocator gpu = create_local_cuda_memory_allocator();
-  int const B = 8, S = 512, E = 1024, H = 16, FF = 4096;
-  ComputationGraphBuilder cgb;
-  tensor_guid_t x = cgb.create_input(shape({B, S, E}, DataType::BF16), CreateGrad::YES);
-  tensor_guid_t n1 = cgb.layer_norm(x, {-1}, true, 1e-5f);
-  tensor_guid_t att = cgb.multihead_attention(n1, n1, n1, E, H, E / H, E / H, 0.0f, false, false, false, std::nullopt, 0.125f);
-  tensor_guid_t r1 = cgb.add(x, cgb.dropout(att, 0.1f));
-  tensor_guid_t n2 = cgb.layer_norm(r1, {-1}, true, 1e-5f);
-  tensor_guid_t f1 = cgb.dense(n2, FF, Activation::GELU, true);
-  tensor_guid_t f2 = cgb.dense(cgb.dropout(f1, 0.1f), E, std::nullopt, true);
-  tensor_guid_t out = cgb.add(r1, cgb.dropout(f2, 0.1f));
-  device_id_t dev = make_device_id_t_from_idx(0, DeviceType::GPU);
-  ComputationGraphInstance inst = create_computation_graph_instance(
-      cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{1e-5, 0.0, false, 0.0}}, std::nullopt, {}, gpu,
-      ProfilingSettings{0, 0}, handle, dev);
-  unsigned seed = 1;
-  for (size_t t = 0; t < cgb.computation_graph.tensors.size(); t++) {
-    auto const &src = cgb.computation_graph.layers[cgb.computation_graph.tensors[t].source.raw];
-    bool weight = std::holds_alternative<WeightAttrs>(src.attrs.op_attrs);
-    if (!weight && tensor_guid_t{(int)t} != x) continue;
-    GenericTensorAccessorW a = inst.get_tensor_accessor(tensor_guid_t{(int)t});
-    GenericTensorAccessorW d = device_accessor(gpu, a.shape, random_vec((size_t)get_num_elements(a.shape.dims), seed++, -0.05f, 0.05f));
-    copy_accessor_data_to_l_from_r(a, d);
-    gpu.deallocate_tensor(d);
-  }
-  GenericTensorAccessorW dout = *inst.get_gradient_accessor(out);
-  // a small output gradient: with a gradient of order one per element and no loss to normalise
-  // it, a few SGD steps drive the weights to infinity
-  GenericTensorAccessorW g = device_accessor(gpu, dout.shape, random_vec((size_t)get_num_elements(dout.shape.dims), 99, -1e-3f, 1e-3f));
-  copy_accessor_data_to_l_from_r(dout, g);
-  device_stream_t stream = get_gpu_device_stream();
-  auto step = [&] { perform_all_passes_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, dev); };
-  for (int i = 0; i < 3; i++) step();
-  ffEvent_t t0, t1;
-  check_ffk(ffk_event_create(&t0), "event");
-  check_ffk(ffk_event_create(&t1), "event");
-  check_ffk(ffk_event_record(t0, stream.require_gpu()), "event");
-  for (int i = 0; i < steps; i++) step();
-  check_ffk(ffk_event_record(t1, stream.require_gpu()), "event");
-  check_ffk(ffk_event_synchronize(t1), "event");
-  float ms = 0;
-  check_ffk(ffk_event_elapsed_ms(t0, t1, &ms), "event");
-  {
-    // the numbers are only meaningful on healthy data: a step that has diverged runs on NaNs,
-    // which toggle no bits and let the chip clock higher
-    std::vector<float> sample = to_host(inst.get_tensor_accessor(out));
-    size_t bad = 0;
-    double sum = 0;
-    for (float v : sample) bad += !std::isfinite(v), sum += std::isfinite(v) ? std::fabs(v) : 0.0;
-    printf("output after the run: %zu non-finite of %zu, mean |y| %.4f\n", bad, sample.size(), sum / (double)sample.size());
-  }
-  int launches = 0;
-  for (auto const &inv : inst.get_execution_order()) launches += 1, (void)inv;
-  printf("step driver, encoder layer B8 S512 d1024 h16 ffn4096 bf16, FWD+BWD+SGD: %.3f ms/step over %d steps, "
-         "%d invocations, %.1f MiB placed, %.2f M tokens/s\n",
-         ms / steps, steps, launches, inst.bytes_allocated() / 1048576.0, B * S / (ms / steps) / 1e3);
-}
-
 int main(int argc, char **argv) {
   std::string mode = argc > 1 ? argv[1] : "--cpu";
-  if (mode == "--bench-step") {
-    try {
-      bench_step(argc > 2 ? atoi(argv[2]) : 20);
-    } catch (std::exception const &e) {
-      printf("bench-step failed: %s\n", e.what());
-      return 1;
-    }
-    return 0;
-  }
   if (mode == "--cpu") {
     cpu_tests();
   } else if (mode == "--gpu") {
     gpu_tests();
   } else {
-    printf("usage: test_host --cpu | --gpu | --bench-step [steps]\n");
+    printf("usage: test_host --cpu | --gpu\n");
     return 2;
   }
   printf("%d checks, %d failed\n", g_checks, g_failed);
