@@ -213,20 +213,39 @@ __device__ __forceinline__ float storage_round<bf16>(float v) {
   return __uint_as_float(pack_bf16x2(v, 0.0f) << 16);
 }
 
-// ---- wavefront reductions (64 lanes, DPP/shuffle based) -------------------
+// ---- wavefront reductions (64 lanes) ---------------------------------------
+// Every lane ends with the result over all 64.  The first four steps read the partner lane
+// through the vector ALU's own lane-select (DPP) and the last two through the 16- and 32-lane
+// swaps: eight vector instructions and no trip through the LDS crossbar, which a shuffle-based
+// butterfly (ds_bpermute) pays six times in a row, each with an LDS round trip of latency.
+//   quad_perm [1,0,3,2], quad_perm [2,3,0,1]: partners 1 and 2 lanes away (all 4 of a quad equal);
+//   row_half_mirror: lane i of 8 reads lane 7 - i, which lies in the other quad;
+//   row_mirror: lane i of 16 reads lane 15 - i, which lies in the other group of 8.
+// Partners always apply the commutative operation to the same two values, so the lanes agree
+// bit for bit.
+template <int CTRL>
+__device__ __forceinline__ float dpp_read(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <typename F>
+__device__ __forceinline__ float wave_reduce(float v, F f) {
+  v = f(v, dpp_read<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = f(v, dpp_read<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = f(v, dpp_read<0x141>(v));  // row_half_mirror
+  v = f(v, dpp_read<0x140>(v));  // row_mirror
+  // swaps the odd 16-lane rows of the first operand with the even rows of the second: with the
+  // same value in both, the results hold rows {0,0,2,2} and {1,1,3,3}
+  auto const a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = f(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  // the same for the two 32-lane halves
+  auto const b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return f(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    v += __shfl_xor(v, off, 64);
-  }
-  return v;
+  return wave_reduce(v, [](float a, float b) { return a + b; });
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    v = fmaxf(v, __shfl_xor(v, off, 64));
-  }
-  return v;
+  return wave_reduce(v, [](float a, float b) { return fmaxf(a, b); });
 }
 
 // A tensor this large does not stay in the 256 MB last-level cache between the kernel that

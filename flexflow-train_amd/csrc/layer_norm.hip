@@ -199,25 +199,41 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
   }
 
   int64_t const row_step = (int64_t)gridDim.x * RPB;
-  // The loads of the next row are issued before the current row is reduced, so
-  // two rows of dY and X are in flight per wave.
-  u32x4 rx[EPT], rdy[EPT];
-  auto issue_row = [&](int64_t base) {
-    int64_t const r = min(base + sub, M - 1);
+  // Two row buffers used in turn: the loads of the next row are issued into the other buffer
+  // as soon as this row is unpacked, so they are in flight while this row is reduced.  (A
+  // third buffer, two rows ahead, measured 2% slower: the kernel is short of neither requests
+  // nor latency cover.)
+  // Lanes past the row's end never load: their registers keep these zeros, which add nothing
+  // to any sum, so the arithmetic below needs no bounds checks.
+  u32x4 rxa[EPT], rdya[EPT], rxb[EPT], rdyb[EPT];
 #pragma unroll
-    for (int j = 0; j < EPT; j++) {
-      int v = lane + j * LANES;
-      if (v < nvec) {
-        rx[j] = load_raw_stream(X + r * (int64_t)N + (int64_t)v * V);
-        rdy[j] = load_raw_stream(dY + r * (int64_t)N + (int64_t)v * V);
+  for (int j = 0; j < EPT; j++) {
+    rxa[j] = rdya[j] = rxb[j] = rdyb[j] = u32x4{0, 0, 0, 0};
+  }
+  // A wave whose row lies past the end (the last workgroup's spare waves) gets zeros, which
+  // leave dgamma / dbeta as they are.
+  auto issue_row = [&](u32x4 (&rx)[EPT], u32x4 (&rdy)[EPT], int64_t base) {
+    int64_t const r = base + sub;
+    if (r < M) {
+#pragma unroll
+      for (int j = 0; j < EPT; j++) {
+        int v = lane + j * LANES;
+        if (v < nvec) {
+          rx[j] = load_raw_stream(X + r * (int64_t)N + (int64_t)v * V);
+          rdy[j] = load_raw_stream(dY + r * (int64_t)N + (int64_t)v * V);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPT; j++) {
+        rx[j] = u32x4{0, 0, 0, 0};
+        rdy[j] = u32x4{0, 0, 0, 0};
       }
     }
   };
-  int64_t base = (int64_t)blockIdx.x * RPB;
-  if (base < M) issue_row(base);
-  // Every wave of a workgroup runs the same number of iterations so the
-  // barriers inside the reducer stay aligned.
-  for (; base < M; base += row_step) {
+  // One row from the buffers (rx, rdy); the next row goes into (ox, ody).  Every wave of a workgroup runs the same number of rows so the barriers
+  // inside the reducer stay aligned.
+  auto do_row = [&](u32x4 (&rx)[EPT], u32x4 (&rdy)[EPT], u32x4 (&ox)[EPT], u32x4 (&ody)[EPT], int64_t base) {
     int64_t const row = base + sub;
     bool const row_ok = row < M;
     int64_t const r = row_ok ? row : M - 1;
@@ -226,36 +242,28 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
     float s1 = 0.0f, s2 = 0.0f;  // sum dy*g, sum dy*g*xhat
 #pragma unroll
     for (int j = 0; j < EPT; j++) {
-      int v = lane + j * LANES;
-      if (v < nvec) {
-        unpack_raw(rx[j], x[j], (T const *)nullptr);
-        unpack_raw(rdy[j], dy[j], (T const *)nullptr);
-      } else {
-#pragma unroll
-        for (int e = 0; e < V; e++) {
-          x[j][e] = 0.0f;
-          dy[j][e] = 0.0f;
-        }
-      }
+      unpack_raw(rx[j], x[j], (T const *)nullptr);
+      unpack_raw(rdy[j], dy[j], (T const *)nullptr);
     }
-    if (base + row_step < M) issue_row(base + row_step);
+    if (base + row_step < M) issue_row(ox, ody, base + row_step);
 #pragma unroll
     for (int j = 0; j < EPT; j++) {
 #pragma unroll
       for (int e = 0; e < V; e++) {
         float xh = (x[j][e] - mu) * rs;
-        float dyg = dy[j][e] * g[j][e];
+        float const dyv = dy[j][e];
+        float dyg = dyv * g[j][e];
         s1 += dyg;
         s2 += dyg * xh;
         x[j][e] = xh;
-        if (row_ok) {
-          dg[j][e] += dy[j][e] * xh;
-          db[j][e] += dy[j][e];
-        }
+        dg[j][e] += dyv * xh;
+        db[j][e] += dyv;
+        dy[j][e] = dyg;
       }
     }
     red.sum2(s1, s2);
-    float const m1 = s1 * inv_n, m2 = s2 * inv_n;
+    // rs * (dy g - m1 - xhat m2) as two fused operations per element
+    float const c0 = -(s1 * inv_n) * rs, c1 = -(s2 * inv_n) * rs;
     if (row_ok && dX != nullptr) {
 #pragma unroll
       for (int j = 0; j < EPT; j++) {
@@ -268,7 +276,7 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
           }
 #pragma unroll
           for (int e = 0; e < V; e++) {
-            float val = rs * (dy[j][e] * g[j][e] - m1 - x[j][e] * m2);
+            float val = fmaf(dy[j][e], rs, fmaf(x[j][e], c1, c0));
             if (ACC && res != nullptr) val = storage_round<T>(val);
             o[e] = ACC ? o[e] + val : val;
           }
@@ -293,6 +301,17 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
           }
         }
       }
+    }
+  };
+  {
+    int64_t base = (int64_t)blockIdx.x * RPB;
+    if (base < M) issue_row(rxa, rdya, base);
+    while (base < M) {
+      do_row(rxa, rdya, rxb, rdyb, base);
+      base += row_step;
+      if (base >= M) break;
+      do_row(rxb, rdyb, rxa, rdya, base);
+      base += row_step;
     }
   }
 
@@ -390,6 +409,9 @@ __global__ __launch_bounds__(256) void layer_norm_bwd_generic_param_kernel(
   if (dbeta != nullptr) VecIO<T>::store1(dbeta + j, acc ? sb + VecIO<T>::load1(dbeta + j) : sb);
 }
 
+// Two workgroups per CU: with one the memory pipe runs short of requests (102 against 76 us on
+// [16384, 4096] bf16), with three or four every workgroup's partial sums (2 N floats) and the
+// kernel that adds them up cost more than the extra requests in flight gain (80 and 92 us).
 constexpr int kLnBwdMaxBlocks = 2 * kNumCU;
 
 static int ln_bwd_blocks(int64_t M, int wpr) {
