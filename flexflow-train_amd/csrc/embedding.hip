@@ -13,6 +13,7 @@
 #include "ffk_common.h"
 #include "radix_sort.h"
 #include <cstdlib>
+#include <type_traits>
 #include <cstring>
 
 namespace ffk {
@@ -63,23 +64,65 @@ constexpr int emb_vec() {
   return sizeof(OT) == 2 ? 8 : VecIO<WT>::kVec;
 }
 
-// One thread per (bag, 16-byte vector of the row).
-template <typename IT, typename WT, typename OT>
+// One thread per (bag, 16-byte vector of the row).  BIG: 2^31 and more threads' worth of
+// work, 64-bit index arithmetic; otherwise 32-bit with the division by nvec as a multiplication
+// (the 64-bit division alone was 130 of the 250 instructions a thread of the plain gather ran,
+// and made that kernel bound by the vector ALU).
+// CHUNKED: the kernel for bags of eight entries and more (its row buffers cost the plain
+// gather half its waves per CU, so single lookups run the instantiation without them).
+template <typename IT, typename WT, typename OT, bool BIG, bool CHUNKED>
 __global__ __launch_bounds__(kEmbThreads) void embedding_fwd_vec_kernel(
     IT const *__restrict__ idx, OT *__restrict__ out, WT const *__restrict__ W,
     int64_t num_bags, int bag, int nvec, int64_t dim, int64_t num_entries,
-    float scale) {
+    float scale, FastDiv by_nvec) {
   constexpr int V = emb_vec<WT, OT>();
-  int64_t const total = num_bags * nvec;
-  int64_t const stride = (int64_t)gridDim.x * kEmbThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kEmbThreads + threadIdx.x; i < total; i += stride) {
-    int64_t const b = i / nvec;
-    int const v = (int)(i % nvec);
+  using index_t = std::conditional_t<BIG, int64_t, uint32_t>;
+  index_t const total = (index_t)(num_bags * nvec);
+  index_t const stride = (index_t)gridDim.x * kEmbThreads;
+  for (index_t i = (index_t)blockIdx.x * kEmbThreads + threadIdx.x; i < total; i += stride) {
+    int64_t b;
+    int v;
+    if constexpr (BIG) {
+      b = i / nvec;
+      v = (int)(i % nvec);
+    } else {
+      uint32_t q, r;
+      by_nvec.divmod(i, q, r);
+      b = q;
+      v = (int)r;
+    }
     float acc[V];
 #pragma unroll
     for (int e = 0; e < V; e++) acc[e] = 0.0f;
     IT const *ib = idx + b * bag;
     int j = 0;
+    // Bags of eight entries and more: eight row reads in flight, and the indices of the next
+    // eight are asked for before this group's rows are waited for, so a bag of 32 costs one
+    // index round trip and four row round trips instead of eight of each.  The sum keeps the
+    // order of the entries.
+    if constexpr (CHUNKED) {
+      constexpr int CH = 8;
+      int64_t rn[CH];
+#pragma unroll
+      for (int u = 0; u < CH; u++) rn[u] = (int64_t)ib[u];
+      for (; j + CH <= bag; j += CH) {
+        float w[CH][V];
+        bool ok[CH];
+#pragma unroll
+        for (int u = 0; u < CH; u++) {
+          ok[u] = (uint64_t)rn[u] < (uint64_t)num_entries;
+          load_row<WT, V>(W + (ok[u] ? rn[u] : 0) * dim + (int64_t)v * V, w[u]);
+        }
+        if (j + 2 * CH <= bag) {
+#pragma unroll
+          for (int u = 0; u < CH; u++) rn[u] = (int64_t)ib[j + CH + u];
+        }
+#pragma unroll
+        for (int u = 0; u < CH; u++)
+#pragma unroll
+          for (int e = 0; e < V; e++) acc[e] = acc[e] + (ok[u] ? w[u][e] : 0.0f);
+      }
+    }
     for (; j + 4 <= bag; j += 4) {  // four row reads in flight
       int64_t r[4];
       float w[4][V];
@@ -520,8 +563,20 @@ static int emb_forward(hipStream_t st, void const *indices, void *output,
   OT *O = static_cast<OT *>(output);
   if (dim % V == 0 && aligned16(weight) && aligned16(output)) {
     int nvec = (int)(dim / V);
-    embedding_fwd_vec_kernel<IT, WT, OT><<<emb_grid(num_bags * nvec), kEmbThreads, 0, st>>>(
-        I, O, W, num_bags, (int)bag, nvec, dim, num_entries, scale);
+    // 32-bit thread indices while index + one grid stride cannot wrap
+    bool const fast = num_bags * nvec < ((int64_t)1 << 31) - (int64_t)kNumCU * 256 * kEmbThreads;
+    FastDiv const by_nvec = fast ? make_fast_div((uint32_t)nvec) : FastDiv{};
+#define FFK_EMB_FWD(BIG_, CHUNKED_)                                                                   \
+  embedding_fwd_vec_kernel<IT, WT, OT, BIG_, CHUNKED_><<<emb_grid(num_bags * nvec), kEmbThreads, 0, st>>>( \
+      I, O, W, num_bags, (int)bag, nvec, dim, num_entries, scale, by_nvec)
+    if (bag >= 8) {
+      if (fast) FFK_EMB_FWD(false, true);
+      else FFK_EMB_FWD(true, true);
+    } else {
+      if (fast) FFK_EMB_FWD(false, false);
+      else FFK_EMB_FWD(true, false);
+    }
+#undef FFK_EMB_FWD
   } else {
     embedding_fwd_scalar_kernel<IT, WT, OT><<<emb_grid(num_bags * dim), kEmbThreads, 0, st>>>(
         I, O, W, num_bags, (int)bag, dim, num_entries, scale);

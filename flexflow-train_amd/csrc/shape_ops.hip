@@ -22,6 +22,7 @@
 // [outer, dim_size, stride], output[o, j, s] = input[o, index[o, j, s], s].
 // Backward scatters with hardware fp32 atomics like the reference.
 #include "ffk_common.h"
+#include <type_traits>
 
 namespace ffk {
 
@@ -50,21 +51,49 @@ __device__ __forceinline__ void put(U *dst, U v) {
   }
 }
 
+// Divisions by the row length and by the outer output extents as multiplications (a 64-bit
+// division by a kernel argument is some 130 instructions, and a unit needs one per outer dim).
+struct PermuteDivs {
+  FastDiv by_units;
+  FastDiv by_dim[kMaxDims];
+};
+
+// 32-bit indices while index + one grid stride cannot wrap
+static inline bool fits_fast_index(int64_t total, int64_t threads_per_block) {
+  return total < ((int64_t)1 << 31) - (int64_t)kNumCU * 64 * threads_per_block;
+}
+
 // The last dim stays last: one unit (an element, or a 16-byte piece of a row)
-// per lane; its row is decomposed over the outer output dims.
-template <typename U, int MODE, int EPU /* elements per unit, for the typed add */, typename E>
+// per lane; its row is decomposed over the outer output dims.  BIG: 64-bit unit indices.
+template <typename U, int MODE, int EPU /* elements per unit, for the typed add */, typename E, bool BIG>
 __global__ __launch_bounds__(kShapeThreads) void permute_rows_kernel(U const *__restrict__ in, U *out, PermuteArgs a,
-                                                                      int64_t units_per_row, int64_t total_units) {
-  int64_t const stride = (int64_t)gridDim.x * kShapeThreads;
-  for (int64_t q = (int64_t)blockIdx.x * kShapeThreads + threadIdx.x; q < total_units; q += stride) {
-    int64_t row = q / units_per_row;
-    int64_t const cu = q - row * units_per_row;
+                                                                      int64_t units_per_row, int64_t total_units,
+                                                                      PermuteDivs dv) {
+  using index_t = std::conditional_t<BIG, int64_t, uint32_t>;
+  index_t const stride = (index_t)gridDim.x * kShapeThreads;
+  for (index_t q = (index_t)blockIdx.x * kShapeThreads + threadIdx.x; q < (index_t)total_units; q += stride) {
     int64_t in_row = 0;  // in units of elements
+    int64_t cu;
+    if constexpr (BIG) {
+      int64_t row = q / units_per_row;
+      cu = q - row * units_per_row;
 #pragma unroll 1
-    for (int i = a.nd - 2; i >= 0; i--) {
-      int64_t const r = row / a.out_dim[i];
-      in_row += (row - r * a.out_dim[i]) * a.in_stride[i];
-      row = r;
+      for (int i = a.nd - 2; i >= 0; i--) {
+        int64_t const r = row / a.out_dim[i];
+        in_row += (row - r * a.out_dim[i]) * a.in_stride[i];
+        row = r;
+      }
+    } else {
+      uint32_t row, c;
+      dv.by_units.divmod(q, row, c);
+      cu = c;
+#pragma unroll 1
+      for (int i = a.nd - 2; i >= 0; i--) {
+        uint32_t r, rem;
+        dv.by_dim[i].divmod(row, r, rem);
+        in_row += (int64_t)rem * a.in_stride[i];
+        row = r;
+      }
     }
     U const v = in[in_row / EPU + cu];
     if constexpr (MODE == kStore) {
@@ -274,13 +303,24 @@ static hipError_t permute_typed(hipStream_t st, void const *in, void *out, int n
     int64_t const L = od[n - 1];
     bool wide = wide_ok && L % VE == 0;
     for (int i = 0; i < n - 1; i++) wide = wide && is[i] % VE == 0;
-    if (wide) {
-      permute_rows_kernel<u32x4, MODE, VE, E><<<blocks_for(total / VE), kShapeThreads, 0, st>>>(
-          static_cast<u32x4 const *>(in), static_cast<u32x4 *>(out), a, L / VE, total / VE);
-    } else {
-      permute_rows_kernel<E, MODE, 1, E><<<blocks_for(total), kShapeThreads, 0, st>>>(
-          static_cast<E const *>(in), static_cast<E *>(out), a, L, total);
+    int64_t const units_per_row = wide ? L / VE : L, units = wide ? total / VE : total;
+    bool const fast = fits_fast_index(units, kShapeThreads);
+    PermuteDivs dv{};
+    if (fast) {
+      dv.by_units = make_fast_div((uint32_t)units_per_row);
+      for (int i = 0; i < n - 1; i++) dv.by_dim[i] = make_fast_div((uint32_t)od[i]);
     }
+#define FFK_PERMUTE_ROWS(U_, EPU_, BIG_)                                                                   \
+  permute_rows_kernel<U_, MODE, EPU_, E, BIG_><<<blocks_for(units), kShapeThreads, 0, st>>>(               \
+      static_cast<U_ const *>(in), static_cast<U_ *>(out), a, units_per_row, units, dv)
+    if (wide) {
+      if (fast) FFK_PERMUTE_ROWS(u32x4, VE, false);
+      else FFK_PERMUTE_ROWS(u32x4, VE, true);
+    } else {
+      if (fast) FFK_PERMUTE_ROWS(E, 1, false);
+      else FFK_PERMUTE_ROWS(E, 1, true);
+    }
+#undef FFK_PERMUTE_ROWS
     return hipGetLastError();
   }
   // tiles: a = the output position whose input stride is 1, b = the last output position
@@ -366,34 +406,65 @@ static int permute_any(char const *who, ffk_stream_t stream, int dtype, void con
 
 // ---- gather -------------------------------------------------------------------
 
-template <typename E, typename IT>
+// One output element per lane.  BIG: 64-bit element indices; otherwise 32-bit with the two
+// divisions as multiplications.
+struct GatherDivs {
+  FastDiv by_out_plane, by_stride;
+};
+
+template <bool BIG, typename index_t>
+__device__ __forceinline__ void gather_split(index_t o, int64_t out_plane, int64_t stride, GatherDivs const &dv,
+                                             int64_t &outer, int64_t &left) {
+  if constexpr (BIG) {
+    outer = o / out_plane;
+    left = o % stride;
+  } else {
+    uint32_t q, r;
+    dv.by_stride.divmod(o, q, r);
+    left = r;
+    outer = dv.by_out_plane.div(o);
+  }
+}
+
+template <typename E, typename IT, bool BIG>
 __global__ __launch_bounds__(kShapeThreads) void gather_fwd_kernel(E const *__restrict__ in, IT const *__restrict__ index,
                                                                     E *__restrict__ out, int64_t total, int64_t stride,
-                                                                    int64_t in_dim, int64_t out_dim) {
-  int64_t const step = (int64_t)gridDim.x * kShapeThreads;
+                                                                    int64_t in_dim, int64_t out_dim, GatherDivs dv) {
+  using index_t = std::conditional_t<BIG, int64_t, uint32_t>;
+  index_t const step = (index_t)gridDim.x * kShapeThreads;
   int64_t const out_plane = stride * out_dim, in_plane = stride * in_dim;
-  for (int64_t o = (int64_t)blockIdx.x * kShapeThreads + threadIdx.x; o < total; o += step) {
-    int64_t const outer = o / out_plane;
-    int64_t const left = o % stride;
+  for (index_t o = (index_t)blockIdx.x * kShapeThreads + threadIdx.x; o < (index_t)total; o += step) {
+    int64_t outer, left;
+    gather_split<BIG>(o, out_plane, stride, dv, outer, left);
     int64_t const j = (int64_t)index[o];
     // an index outside the dim reads nothing (the reference would read out of bounds)
     out[o] = (j >= 0 && j < in_dim) ? in[outer * in_plane + j * stride + left] : E(0);
   }
 }
 
-template <typename IT>
+template <typename IT, bool BIG>
 __global__ __launch_bounds__(kShapeThreads) void gather_bwd_kernel(float const *__restrict__ dout,
                                                                     IT const *__restrict__ index, float *din,
                                                                     int64_t total, int64_t stride, int64_t in_dim,
-                                                                    int64_t out_dim) {
-  int64_t const step = (int64_t)gridDim.x * kShapeThreads;
+                                                                    int64_t out_dim, GatherDivs dv) {
+  using index_t = std::conditional_t<BIG, int64_t, uint32_t>;
+  index_t const step = (index_t)gridDim.x * kShapeThreads;
   int64_t const out_plane = stride * out_dim, in_plane = stride * in_dim;
-  for (int64_t o = (int64_t)blockIdx.x * kShapeThreads + threadIdx.x; o < total; o += step) {
-    int64_t const outer = o / out_plane;
-    int64_t const left = o % stride;
+  for (index_t o = (index_t)blockIdx.x * kShapeThreads + threadIdx.x; o < (index_t)total; o += step) {
+    int64_t outer, left;
+    gather_split<BIG>(o, out_plane, stride, dv, outer, left);
     int64_t const j = (int64_t)index[o];
     if (j >= 0 && j < in_dim) atomicAdd(din + outer * in_plane + j * stride + left, dout[o]);
   }
+}
+
+// the divisors of a gather over `total` output elements, or false when 32-bit indices do not fit
+static bool gather_divs(int64_t total, int64_t stride, int64_t out_dim, GatherDivs &dv) {
+  if (!fits_fast_index(total, kShapeThreads) || total == 0) return false;
+  // total = outer * out_plane < 2^31, so both divisors are below 2^31
+  dv.by_out_plane = make_fast_div((uint32_t)(stride * out_dim));
+  dv.by_stride = make_fast_div((uint32_t)stride);
+  return true;
 }
 
 }  // namespace ffk
@@ -430,16 +501,21 @@ extern "C" int ffk_gather_forward(ffk_stream_t stream, int dtype, int index_dtyp
   FFK_REQUIRE(input && index && output, "gather_forward: NULL tensor");
   hipStream_t st = as_stream(stream);
   unsigned const blocks = blocks_for(total);
+  GatherDivs dv{};
+  bool const fast = gather_divs(total, stride, output_dim_size, dv);
+#define FFK_GATHER_ONE(E, IT, BIG)                                                                           \
+  gather_fwd_kernel<E, IT, BIG><<<blocks, kShapeThreads, 0, st>>>(                                           \
+      static_cast<E const *>(input), static_cast<IT const *>(index), static_cast<E *>(output), total, stride, \
+      input_dim_size, output_dim_size, dv)
 #define FFK_GATHER(E)                                                                                        \
   do {                                                                                                       \
-    if (index_dtype == FFK_INT32)                                                                            \
-      gather_fwd_kernel<E, int32_t><<<blocks, kShapeThreads, 0, st>>>(                                      \
-          static_cast<E const *>(input), static_cast<int32_t const *>(index), static_cast<E *>(output), total, \
-          stride, input_dim_size, output_dim_size);                                                          \
-    else                                                                                                     \
-      gather_fwd_kernel<E, int64_t><<<blocks, kShapeThreads, 0, st>>>(                                      \
-          static_cast<E const *>(input), static_cast<int64_t const *>(index), static_cast<E *>(output), total, \
-          stride, input_dim_size, output_dim_size);                                                          \
+    if (index_dtype == FFK_INT32) {                                                                          \
+      if (fast) FFK_GATHER_ONE(E, int32_t, false);                                                           \
+      else FFK_GATHER_ONE(E, int32_t, true);                                                                 \
+    } else {                                                                                                 \
+      if (fast) FFK_GATHER_ONE(E, int64_t, false);                                                           \
+      else FFK_GATHER_ONE(E, int64_t, true);                                                                 \
+    }                                                                                                        \
   } while (0)
   switch (dtype) {
     case FFK_BOOL: FFK_GATHER(uint8_t); break;
@@ -449,6 +525,7 @@ extern "C" int ffk_gather_forward(ffk_stream_t stream, int dtype, int index_dtyp
     default: return fail(FFK_ERR_UNSUPPORTED, "gather_forward: data type %d not supported", dtype);
   }
 #undef FFK_GATHER
+#undef FFK_GATHER_ONE
   FFK_CHECK_LAUNCH();
   return FFK_OK;
 }
@@ -463,15 +540,20 @@ extern "C" int ffk_gather_backward(ffk_stream_t stream, int index_dtype, float c
   FFK_REQUIRE(output_grad && index && input_grad, "gather_backward: NULL tensor");
   hipStream_t st = as_stream(stream);
   unsigned const blocks = blocks_for(total);
+  GatherDivs dv{};
+  bool const fast = gather_divs(total, stride, output_dim_size, dv);
+#define FFK_GATHER_BWD(IT, BIG)                                                                              \
+  gather_bwd_kernel<IT, BIG><<<blocks, kShapeThreads, 0, st>>>(output_grad, static_cast<IT const *>(index), \
+                                                               input_grad, total, stride, input_dim_size,   \
+                                                               output_dim_size, dv)
   if (index_dtype == FFK_INT32) {
-    gather_bwd_kernel<int32_t><<<blocks, kShapeThreads, 0, st>>>(output_grad, static_cast<int32_t const *>(index),
-                                                                 input_grad, total, stride, input_dim_size,
-                                                                 output_dim_size);
+    if (fast) FFK_GATHER_BWD(int32_t, false);
+    else FFK_GATHER_BWD(int32_t, true);
   } else {
-    gather_bwd_kernel<int64_t><<<blocks, kShapeThreads, 0, st>>>(output_grad, static_cast<int64_t const *>(index),
-                                                                 input_grad, total, stride, input_dim_size,
-                                                                 output_dim_size);
+    if (fast) FFK_GATHER_BWD(int64_t, false);
+    else FFK_GATHER_BWD(int64_t, true);
   }
+#undef FFK_GATHER_BWD
   FFK_CHECK_LAUNCH();
   return FFK_OK;
 }
