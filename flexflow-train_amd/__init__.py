@@ -25,6 +25,7 @@ c_sz = ctypes.c_size_t
 
 # DataType ordinals of include/ffk.h
 BOOL, INT32, INT64, HALF, FLOAT, DOUBLE, BF16 = range(7)
+ERR_INVALID, ERR_HIP, ERR_UNSUPPORTED, ERR_WORKSPACE = 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH, ACT_GELU = -1, 0, 1, 2, 3
 AGGR_NONE, AGGR_SUM, AGGR_AVG = -1, 0, 1
 OP = dict(
@@ -118,6 +119,16 @@ SIGNATURES = {
                                         c_i64, c_i64, c_p, c_sz, c_int]),
     "ffk_layer_norm_backward_static": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
                                                c_p, c_i64, c_i64, c_int]),
+    "ffk_dropout_backward_bias_grad_workspace_bytes": (c_sz, [c_i64, c_i64]),
+    "ffk_dropout_backward_bias_grad": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_i64, c_p, c_int, c_p, c_sz, c_f, c_u64,
+                                               c_u64]),
+    "ffk_linear_backward_dropout_gelu_bias_grad": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_i64, c_i64,
+                                                           c_i64, c_p, c_sz, c_int, c_f, c_u64, c_u64, c_p, c_int, c_p,
+                                                           c_sz]),
+    "ffk_layer_norm_backward_residual": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
+                                                 c_i64, c_i64, c_p, c_sz, c_int, c_p, c_f, c_u64, c_u64]),
+    "ffk_dropout_add_layer_norm_forward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
+                                                   c_i64, c_i64, c_f, c_f, c_u64, c_u64]),
     "ffk_softmax_forward": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_i64, c_i64]),
     "ffk_softmax_backward_copy": (c_int, [c_p, c_int, c_p, c_p, c_sz]),
     "ffk_softmax_backward": (c_int, [c_p, c_int, c_p, c_p, c_p, c_i64, c_i64, c_i64]),
@@ -306,6 +317,37 @@ def linear_backward_dropout_gelu(dy, x, gelu_input, w, rate, seed, offset=0, dw=
     return dx
 
 
+def linear_backward_dropout_gelu_bias_grad(dy, x, gelu_input, w, rate, seed, gelu_bias_grad, offset=0, dw=None, db=None,
+                                           accumulate=0, accumulate_gelu_bias=False):
+    """linear_backward_dropout_gelu that also adds up the columns of the input gradient it writes."""
+    torch = _torch()
+    batch, in_dim = x.shape
+    out_dim = w.shape[0]
+    dx = torch.empty_like(x)
+    need = lib().ffk_linear_backward_workspace_bytes(dtype_of(x), ACT_NONE, int(db is not None), batch, out_dim)
+    workspace = torch.empty((max(need, 1),), dtype=torch.uint8, device=x.device)
+    need2 = lib().ffk_dropout_backward_bias_grad_workspace_bytes(batch, in_dim)
+    workspace2 = torch.empty((need2,), dtype=torch.uint8, device=x.device)
+    check(lib().ffk_linear_backward_dropout_gelu_bias_grad(
+        current_stream(), dtype_of(x), ptr(dy), ptr(x), ptr(gelu_input), ptr(dx), ptr(w), ptr(dw), ptr(db), batch,
+        in_dim, out_dim, ptr(workspace), need, int(accumulate), rate, seed, offset, ptr(gelu_bias_grad),
+        int(accumulate_gelu_bias), ptr(workspace2), need2))
+    return dx
+
+
+def dropout_backward_bias_grad(dy, rate, seed, bias_grad, offset=0, accumulate_bias=False):
+    """dx = dropout_backward(dy) and bias_grad (+)= the column sums of dx, one pass."""
+    torch = _torch()
+    batch, out_dim = dy.shape
+    dx = torch.empty_like(dy)
+    need = lib().ffk_dropout_backward_bias_grad_workspace_bytes(batch, out_dim)
+    workspace = torch.empty((need,), dtype=torch.uint8, device=dy.device)
+    check(lib().ffk_dropout_backward_bias_grad(current_stream(), dtype_of(dy), ptr(dy), ptr(dx), batch, out_dim,
+                                               ptr(bias_grad), int(accumulate_bias), ptr(workspace), need, rate, seed,
+                                               offset))
+    return dx
+
+
 def gemm(A, B, C, trans_a=False, trans_b=False, accumulate=False):
     M, N = C.shape
     K = A.shape[0] if trans_a else A.shape[1]
@@ -388,6 +430,34 @@ def layer_norm_backward_static(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, accu
                                                ptr(mean), ptr(rstd), ptr(gamma), ptr(dx),
                                                ptr(dgamma), ptr(dbeta), M, N, int(accumulate)))
     return dx, dgamma, dbeta
+
+
+def layer_norm_backward_residual(dy, x, mean, rstd, gamma, residual, dx, dgamma, dbeta, accumulate_params=False,
+                                 dropped=None, rate=0.0, seed=0, offset=0, workspace=None):
+    """dx = residual + LayerNorm gradient (one rounding); dropped (optional) = dropout_backward(dx)."""
+    torch = _torch()
+    M, N = x.shape
+    if workspace is None:
+        workspace = torch.empty((lib().ffk_layer_norm_backward_workspace_bytes(M, N),), dtype=torch.uint8,
+                                device=x.device)
+    check(lib().ffk_layer_norm_backward_residual(current_stream(), dtype_of(x), ptr(dy), ptr(x), ptr(mean), ptr(rstd),
+                                                 ptr(gamma), ptr(residual), ptr(dx), ptr(dgamma), ptr(dbeta), M, N,
+                                                 ptr(workspace), workspace.numel(), int(accumulate_params),
+                                                 ptr(dropped), rate, seed, offset))
+    return dx, dgamma, dbeta
+
+
+def dropout_add_layer_norm_forward(x, residual, gamma, beta, eps, rate, seed, offset=0):
+    """sum = residual + dropout(x); y = LayerNorm(sum).  Returns (sum, y, mean, rstd)."""
+    torch = _torch()
+    M, N = x.shape
+    total, y = torch.empty_like(x), torch.empty_like(x)
+    mean = torch.empty((M,), dtype=torch.float32, device=x.device)
+    rstd = torch.empty((M,), dtype=torch.float32, device=x.device)
+    check(lib().ffk_dropout_add_layer_norm_forward(current_stream(), dtype_of(x), ptr(x), ptr(residual), ptr(total),
+                                                   ptr(y), ptr(gamma), ptr(beta), ptr(mean), ptr(rstd), M, N, eps,
+                                                   rate, seed, offset))
+    return total, y, mean, rstd
 
 
 def softmax_forward(x, outer, dim, inner, out=None):

@@ -82,6 +82,11 @@ int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
                                      void *dropped = nullptr, float rate = 0.0f,
                                      uint64_t seed = 0, uint64_t offset = 0,
                                      // dgamma / dbeta are added to instead of stored
-                                     bool acc_params = false);
+                                     bool acc_params = false,
+                                     // the gradient is rounded to the storage type before residual
+                                     // is added (what a separate add of the stored gradient gives);
+                                     // false: the sum is rounded once (what adding the gradient
+                                     // into a copy of residual gives)
+                                     bool round_first = true);
 
 }  // namespace ffk

@@ -168,11 +168,12 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
     float const *__restrict__ mean, float const *__restrict__ rstd,
     T const *__restrict__ gamma, T *dX, float *__restrict__ partials,
     int64_t M, int N, T const *res, T *__restrict__ dropped = nullptr,
-    DropoutParams drop = DropoutParams{}, bool stream_out = false) {
+    DropoutParams drop = DropoutParams{}, bool stream_out = false, bool round_first = true) {
   // stream_out: dX is too large to be found in cache by its reader; store it past the caches.
-  // ACC with res == nullptr: dX += gradient (one rounding).  ACC with res set:
-  // dX = res + gradient rounded to the storage type, i.e. what a separate
-  // element-wise add of res to the stored gradient would give.
+  // ACC with res == nullptr: dX += gradient (one rounding).  ACC with res set and round_first:
+  // dX = res + gradient rounded to the storage type, i.e. what a separate element-wise add of
+  // res to the stored gradient would give; without round_first the sum is rounded once, i.e.
+  // what dX += gradient gives when dX holds a copy of res.
   constexpr int V = VecIO<T>::kVec;
   constexpr int RPB = 4 / WPR;
   constexpr int LANES = 64 * WPR;
@@ -277,7 +278,7 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_bwd_kernel(
 #pragma unroll
           for (int e = 0; e < V; e++) {
             float val = fmaf(dy[j][e], rs, fmaf(x[j][e], c1, c0));
-            if (ACC && res != nullptr) val = storage_round<T>(val);
+            if (ACC && res != nullptr && round_first) val = storage_round<T>(val);
             o[e] = ACC ? o[e] + val : val;
           }
           if (stream_out) {
@@ -463,7 +464,7 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
                        void *workspace, size_t workspace_bytes, bool acc,
                        void const *residual = nullptr, void *dropped = nullptr,
                        DropoutParams const *drop = nullptr, bool fit_blocks_to_workspace = false,
-                       bool acc_params = false) {
+                       bool acc_params = false, bool round_first = true) {
   constexpr int V = VecIO<T>::kVec;
   T const *RES = static_cast<T const *>(residual);
   if (RES != nullptr) acc = true;
@@ -503,10 +504,10 @@ static int ln_backward(hipStream_t st, void const *dy, void const *x,
       if constexpr (sizeof(T) == 2)                                            \
         layer_norm_bwd_kernel<T, E, W, true, true><<<blocks, kRowThreads, 0, st>>>( \
             DY, X, mean, rstd, G, DX, partials, M, (int)N, RES,                \
-            static_cast<T *>(dropped), *drop, stream);                         \
+            static_cast<T *>(dropped), *drop, stream, round_first);            \
     } else if (acc)                                                            \
       layer_norm_bwd_kernel<T, E, W, true><<<blocks, kRowThreads, 0, st>>>(    \
-          DY, X, mean, rstd, G, DX, partials, M, (int)N, RES, nullptr, DropoutParams{}, stream); \
+          DY, X, mean, rstd, G, DX, partials, M, (int)N, RES, nullptr, DropoutParams{}, stream, round_first); \
     else                                                                       \
       layer_norm_bwd_kernel<T, E, W, false><<<blocks, kRowThreads, 0, st>>>(   \
           DY, X, mean, rstd, G, DX, partials, M, (int)N, nullptr, nullptr, DropoutParams{}, stream); \
@@ -580,7 +581,8 @@ int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
                                      void *dgamma, void *dbeta, int64_t M,
                                      int64_t N, void *workspace,
                                      size_t workspace_bytes, void *dropped,
-                                     float rate, uint64_t seed, uint64_t offset, bool acc_params) {
+                                     float rate, uint64_t seed, uint64_t offset, bool acc_params,
+                                     bool round_first) {
   FFK_REQUIRE(M > 0 && N > 0 && M < (1ll << 31) && N < (1ll << 31),
               "layer_norm_backward: bad shape");
   FFK_REQUIRE(dy && x && mean && rstd && residual && dx, "layer_norm_backward: NULL tensor");
@@ -592,10 +594,10 @@ int layer_norm_backward_add_residual(hipStream_t st, int dtype, void const *dy,
   if (dtype == FFK_FLOAT && dropped != nullptr) return FFK_ERR_UNSUPPORTED;  // the dropped copy is bf16 only
   if (dtype == FFK_FLOAT)
     return ln_backward<float>(st, dy, x, mean, rstd, gamma, dx, dgamma, dbeta, M, N,
-                              workspace, workspace_bytes, true, residual, nullptr, nullptr, false, acc_params);
+                              workspace, workspace_bytes, true, residual, nullptr, nullptr, false, acc_params, round_first);
   if (dtype == FFK_BF16)
     return ln_backward<bf16>(st, dy, x, mean, rstd, gamma, dx, dgamma, dbeta, M, N,
-                             workspace, workspace_bytes, true, residual, dropped, &drop, false, acc_params);
+                             workspace, workspace_bytes, true, residual, dropped, &drop, false, acc_params, round_first);
   return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: dtype %d not supported", dtype);
 }
 
@@ -645,6 +647,33 @@ extern "C" int ffk_layer_norm_backward(
                              input_grad, gamma_grad, beta_grad, M, N, workspace,
                              workspace_bytes, acc, nullptr, nullptr, nullptr, false, acc_params);
   return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward: dtype %d not supported", dtype);
+}
+
+extern "C" int ffk_layer_norm_backward_residual(
+    ffk_stream_t stream, int dtype, void const *output_grad, void const *input, float const *mean,
+    float const *rstd, void const *gamma, void const *residual, void *input_grad, void *gamma_grad,
+    void *beta_grad, int64_t M, int64_t N, void *workspace, size_t workspace_bytes, int accumulate_params,
+    void *dropped_grad, float rate, uint64_t seed, uint64_t offset) {
+  FFK_REQUIRE(M >= 0 && N > 0 && N < (1ll << 31), "layer_norm_backward_residual: bad shape");
+  if (M == 0) return FFK_OK;
+  FFK_REQUIRE(M < (1ll << 31), "layer_norm_backward_residual: too many rows");
+  FFK_REQUIRE(output_grad && input && mean && rstd && residual && input_grad,
+              "layer_norm_backward_residual: NULL tensor");
+  if (dtype != FFK_FLOAT && dtype != FFK_BF16)
+    return fail(FFK_ERR_UNSUPPORTED, "layer_norm_backward_residual: dtype %d not supported", dtype);
+  return layer_norm_backward_add_residual(as_stream(stream), dtype, output_grad, input, mean, rstd, gamma, residual,
+                                          input_grad, gamma_grad, beta_grad, M, N, workspace, workspace_bytes,
+                                          dropped_grad, rate, seed, offset, accumulate_params != 0, false);
+}
+
+extern "C" int ffk_dropout_add_layer_norm_forward(ffk_stream_t stream, int dtype, void const *input,
+                                                  void const *residual, void *sum, void *output, void const *gamma,
+                                                  void const *beta, float *mean, float *rstd, int64_t M, int64_t N,
+                                                  float eps, float rate, uint64_t seed, uint64_t offset) {
+  FFK_REQUIRE(M >= 0 && N > 0, "dropout_add_layer_norm_forward: bad shape");
+  if (M == 0) return FFK_OK;
+  return dropout_add_layer_norm_forward(as_stream(stream), dtype, input, residual, sum, output, gamma, beta, mean,
+                                        rstd, M, N, eps, rate, seed, offset);
 }
 
 // ---- the entry point that allocates nothing ---------------------------------

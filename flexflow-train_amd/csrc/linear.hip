@@ -283,3 +283,54 @@ extern "C" int ffk_linear_backward_dropout_gelu(
   }
   return rc;
 }
+
+extern "C" size_t ffk_dropout_backward_bias_grad_workspace_bytes(int64_t batch, int64_t out_dim) {
+  return align256((size_t)colsum_partials_elems(batch, out_dim) * sizeof(float));
+}
+
+extern "C" int ffk_dropout_backward_bias_grad(ffk_stream_t stream, int dtype, void const *output_grad,
+                                              void *input_grad, int64_t batch, int64_t out_dim, void *bias_grad,
+                                              int accumulate_bias, void *workspace, size_t workspace_bytes,
+                                              float rate, uint64_t seed, uint64_t offset) {
+  FFK_REQUIRE(output_grad && input_grad && bias_grad, "dropout_backward_bias_grad: NULL tensor");
+  FFK_REQUIRE(batch > 0 && out_dim > 0, "dropout_backward_bias_grad: non-positive dimension");
+  size_t const need = ffk_dropout_backward_bias_grad_workspace_bytes(batch, out_dim);
+  if (workspace == nullptr || workspace_bytes < need) {
+    return fail(FFK_ERR_WORKSPACE, "dropout_backward_bias_grad: workspace of %zu bytes needed, %zu given", need,
+                workspace_bytes);
+  }
+  DropoutParams dp;
+  int const prc = make_dropout_params("dropout_backward_bias_grad", rate, seed, offset, dp);
+  if (prc != FFK_OK) return prc;
+  int const rc = dropout_backward_colsum(as_stream(stream), dtype, output_grad, input_grad, batch, out_dim, bias_grad,
+                                         accumulate_bias != 0, static_cast<float *>(workspace), dp);
+  if (rc == FFK_ERR_UNSUPPORTED) {
+    return fail(FFK_ERR_UNSUPPORTED, "dropout_backward_bias_grad: no fused kernel for this shape; run Dropout "
+                                     "backward and let the Linear's backward sum its bias gradient");
+  }
+  return rc;
+}
+
+extern "C" int ffk_linear_backward_dropout_gelu_bias_grad(
+    ffk_stream_t stream, int dtype, void const *output_grad, void const *input, void const *gelu_input,
+    void *input_grad, void const *weight, void *weight_grad, void *bias_grad, int64_t batch, int64_t in_dim,
+    int64_t out_dim, void *workspace, size_t workspace_bytes, int accumulate, float rate, uint64_t seed,
+    uint64_t offset, void *gelu_bias_grad, int accumulate_gelu_bias, void *gelu_bias_workspace,
+    size_t gelu_bias_workspace_bytes) {
+  FFK_REQUIRE(gelu_bias_grad != nullptr, "linear_backward_dropout_gelu_bias_grad: NULL bias gradient");
+  size_t const need = ffk_dropout_backward_bias_grad_workspace_bytes(batch, in_dim);
+  if (gelu_bias_workspace == nullptr || gelu_bias_workspace_bytes < need) {
+    return fail(FFK_ERR_WORKSPACE, "linear_backward_dropout_gelu_bias_grad: workspace of %zu bytes needed for the "
+                                   "column sums, %zu given", need, gelu_bias_workspace_bytes);
+  }
+  int const rc = ffk::linear_backward_dropout_gelu(as_stream(stream), dtype, output_grad, input, gelu_input, input_grad,
+                                                   weight, weight_grad, bias_grad, batch, in_dim, out_dim, workspace,
+                                                   workspace_bytes, accumulate, rate, seed, offset, gelu_bias_grad,
+                                                   static_cast<float *>(gelu_bias_workspace), accumulate_gelu_bias != 0);
+  if (rc == FFK_ERR_UNSUPPORTED) {
+    return fail(FFK_ERR_UNSUPPORTED, "linear_backward_dropout_gelu_bias_grad: no fused kernel for this shape; "
+                                     "use ffk_linear_backward_dropout_gelu and let the first Linear's backward sum "
+                                     "its bias gradient");
+  }
+  return rc;
+}

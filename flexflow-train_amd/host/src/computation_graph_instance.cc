@@ -11,6 +11,7 @@
 // pointers that makes one C-ABI call.
 #include "ffk.h"
 #include "local-execution/computation_graph_instance.h"
+#include <memory>
 #include <cstdlib>
 #include <cmath>
 #include <cstring>
@@ -411,6 +412,26 @@ ComputationGraphInstance create_computation_graph_instance(
   //   (GELU -> Dropout) -> Linear:  linear_gelu[linear] = the GELU, gelu_linear[gelu] = the Linear;
   //                                 the Linear's backward writes the gradient of the GELU's input
   std::vector<int> linear_sum(L, -1), sum_linear(L, -1), linear_gelu(L, -1), gelu_linear(L, -1);
+  // A LayerNorm next to the residual add of its block:
+  //   ln_residual[ln] = the add (a LATER layer) that reads the LayerNorm's input t as an operand.  Going back, that
+  //     add runs first and would copy its output gradient into t's; instead the LayerNorm's backward reads that
+  //     output gradient as a residual and writes t's gradient whole (deferred_to_ln[t] = ln: the add skips t).
+  //   ln_drop[ln] = the Dropout whose output was the other operand of the add that PRODUCED t: t's gradient is
+  //     complete once the LayerNorm (its last producer) has run, and the same kernel writes the gradient of
+  //     the Dropout's input (drop_bwd_by_ln[dropout]: its own backward does nothing).
+  //   ln_pre[ln] = that producing add, when it and its Dropout are a fused pair no Linear has taken: the
+  //     LayerNorm's forward computes the sum as well (add_fwd_by_ln[add]: its own forward does nothing).
+  std::vector<int> ln_residual(L, -1), ln_drop(L, -1), ln_pre(L, -1), deferred_to_ln(T, -1);
+  std::vector<bool> drop_bwd_by_ln(L, false), add_fwd_by_ln(L, false);
+  // The bias gradient of a Linear (the column sums of its output's gradient) taken by the kernel that
+  // produces that gradient:
+  //   drop_bias[dropout] = the Linear whose output the Dropout reads: the Dropout's backward sums as it writes;
+  //   gelu_bias[linear]  = the Linear whose output the GELU of a (GELU -> Dropout) -> Linear chain reads: the
+  //                        second Linear's input-gradient GEMM sums on its tile store.
+  // Whether the library had such a kernel for the shape is only known when the call returns, so the producer
+  // leaves word for the Linear (bias_done[linear], written and read once per step, in that order).
+  std::vector<int> drop_bias(L, -1), gelu_bias(L, -1);
+  std::vector<std::shared_ptr<bool>> bias_done(L);
   {
     int unfused = 0;
     check_ffk(ffk_get_option(FFK_OPTION_LAYER_UNFUSED, &unfused), "ffk_get_option");
@@ -487,6 +508,69 @@ ComputationGraphInstance create_computation_graph_instance(
         if (!plain_bf16_linear(lin) || cg.layers[lin].inputs[0] != dropped) continue;
         if (!plan[lin].bwd.has_backward || plan[lin].bwd.accumulate_input[0]) continue;
         linear_gelu[lin] = (int)l, gelu_linear[l] = lin;
+      }
+    }
+    std::vector<int> first_consumer(T, -1);
+    for (size_t l = L; l-- > 0;) {
+      if (!is_op_layer(cg.layers[l])) continue;
+      for (tensor_guid_t t : cg.layers[l].inputs) first_consumer[t.raw] = (int)l;
+    }
+    for (size_t n = 0; enabled && n < L; n++) {
+      ComputationGraph::Layer const &ln = cg.layers[n];
+      if (!is_op_layer(ln) || !std::holds_alternative<LayerNormAttrs>(ln.attrs.op_attrs)) continue;
+      tensor_guid_t const t = ln.inputs[0];
+      DataType const type = shape_of(t).data_type;
+      if ((type != DataType::FLOAT && type != DataType::BF16) || !aligned(t) || !aligned(ln.outputs.at(0))) continue;
+      int const made_by = producer[t.raw];
+      bool const made_by_pair = made_by >= 0 && fused[made_by] == Fused::DROPOUT_ADD_TAIL;
+      // forward: Dropout -> add -> this LayerNorm, the LayerNorm being the sum's first reader
+      if (made_by_pair && sum_linear[made_by] < 0 && type == DataType::BF16 && first_consumer[t.raw] == (int)n) {
+        ln_pre[n] = made_by;
+        add_fwd_by_ln[made_by] = true;
+      }
+      // backward: the later add's copy into t's gradient becomes this LayerNorm's residual
+      if (!plan[n].bwd.has_backward || !has_grad[t.raw] || writers[t.raw] != 2 || is_weight[t.raw]) continue;
+      if (st->logit.has_value() && *st->logit == t) continue;
+      int const l = first_writer[t.raw];
+      if (l <= (int)n || !first_writer_stores[t.raw] || alias_of[t.raw] >= 0) continue;
+      auto const *b = std::get_if<ElementBinaryAttrs>(&cg.layers[l].attrs.op_attrs);
+      if (b == nullptr || b->type != OperatorType::EW_ADD || !plan[l].bwd.add_by_alias) continue;
+      if (!(shape_of(cg.layers[l].outputs.at(0)) == shape_of(t))) continue;
+      ln_residual[n] = l;
+      deferred_to_ln[t.raw] = (int)n;
+      // ... and with t's gradient complete here, the backward of the Dropout that fed the producing add
+      if (!made_by_pair || type != DataType::BF16) continue;
+      size_t const d = partner[made_by];
+      tensor_guid_t const dropped = cg.layers[d].outputs.at(0), drop_in = cg.layers[d].inputs[0];
+      if (alias_of[dropped.raw] != t.raw || !plan[d].bwd.has_backward || plan[d].bwd.accumulate) continue;
+      if (!has_grad[drop_in.raw] || writers[drop_in.raw] != 1 || !aligned(drop_in)) continue;
+      ln_drop[n] = (int)d;
+      drop_bwd_by_ln[d] = true;
+    }
+    auto biased_plain_linear = [&](int lin, tensor_guid_t out) {
+      if (lin < 0) return false;
+      auto const *a = std::get_if<LinearAttrs>(&cg.layers[lin].attrs.op_attrs);
+      if (a == nullptr || !a->use_bias || a->activation.has_value() || !single_use(out)) return false;
+      DataType const type = shape_of(out).data_type;
+      return (type == DataType::FLOAT || type == DataType::BF16) && plan[lin].bwd.has_backward &&
+             has_grad[cg.layers[lin].weights.at(1).raw] && has_grad[out.raw];
+    };
+    for (size_t l = 0; enabled && l < L; l++) {
+      ComputationGraph::Layer const &layer = cg.layers[l];
+      if (!is_op_layer(layer)) continue;
+      if (std::holds_alternative<DropoutAttrs>(layer.attrs.op_attrs)) {
+        if (drop_bwd_by_ln[l] || fused[l] == Fused::GELU_DROPOUT_TAIL) continue;  // its backward runs elsewhere
+        if (!plan[l].bwd.has_backward || plan[l].bwd.accumulate) continue;
+        int const lin = producer[layer.inputs[0].raw];
+        if (!biased_plain_linear(lin, layer.inputs[0])) continue;
+        drop_bias[l] = lin;
+        bias_done[lin] = std::make_shared<bool>(false);
+      } else if (linear_gelu[l] >= 0) {
+        tensor_guid_t const u = cg.layers[(size_t)linear_gelu[l]].inputs[0];
+        int const lin = producer[u.raw];
+        if (!biased_plain_linear(lin, u) || shape_of(u).data_type != DataType::BF16) continue;
+        gelu_bias[l] = lin;
+        bias_done[lin] = std::make_shared<bool>(false);
       }
     }
   }
@@ -644,8 +728,11 @@ ComputationGraphInstance create_computation_graph_instance(
       f = [=](device_stream_t const &s) {
         check_ffk(ffk_linear_forward(s.require_gpu(), type, act, xp, y, w, bias, batch, in_dim, out_dim), "Linear forward");
       };
+      // the bias gradient, unless the kernel that wrote dy has summed it already this step
+      std::shared_ptr<bool> const bias_elsewhere = bias_done[l];
+      auto bias_grad_now = [dbias, bias_elsewhere]() -> void * { return bias_elsewhere && *bias_elsewhere ? nullptr : dbias; };
       b = [=](device_stream_t const &s) {
-        check_ffk(ffk_linear_backward(s.require_gpu(), type, act, 0, y, dy, xp, dx, w, dw, dbias, batch, in_dim, out_dim,
+        check_ffk(ffk_linear_backward(s.require_gpu(), type, act, 0, y, dy, xp, dx, w, dw, bias_grad_now(), batch, in_dim, out_dim,
                                       ws_bytes ? scratch : nullptr, ws_bytes, accumulate),
                   "Linear backward");
       };
@@ -678,13 +765,29 @@ ComputationGraphInstance create_computation_graph_instance(
         int64_t const n = numel(x);
         void *gelu_in = val(cg.layers[g].inputs[0]), *gelu_in_grad = grd(cg.layers[g].inputs[0]);
         int const acc_w = accumulate & ~FFK_ACC_INPUT;
+        // the bias gradient of the Linear in front of the GELU, summed where this GEMM stores
+        int const first = gelu_bias[l];
+        std::shared_ptr<bool> const first_done = first >= 0 ? bias_done[(size_t)first] : nullptr;
+        void *first_dbias = first >= 0 ? grd(cg.layers[(size_t)first].weights.at(1)) : nullptr;
+        int const first_acc = first >= 0 && plan[(size_t)first].bwd.accumulate_input.at(2) ? 1 : 0;
+        void *first_scratch = first >= 0 ? static_cast<void *>(base + plan[(size_t)first].scratch.offset) : nullptr;
+        size_t const first_scratch_bytes = first >= 0 ? plan[(size_t)first].scratch_bytes : 0;
         b = [=](device_stream_t const &s) {
           uint64_t const offset = S->iteration * (uint64_t)n;
-          int const rc = ffk_linear_backward_dropout_gelu(s.require_gpu(), type, dy, xp, gelu_in, gelu_in_grad, w, dw, dbias, batch,
+          void *const bias_grad = bias_grad_now();
+          if (first_done) {
+            int const rc = ffk_linear_backward_dropout_gelu_bias_grad(
+                s.require_gpu(), type, dy, xp, gelu_in, gelu_in_grad, w, dw, bias_grad, batch, in_dim, out_dim,
+                ws_bytes ? scratch : nullptr, ws_bytes, acc_w, rate, seed, offset, first_dbias, first_acc, first_scratch,
+                first_scratch_bytes);
+            *first_done = rc == FFK_OK;
+            if (rc != FFK_ERR_UNSUPPORTED) return check_ffk(rc, "Linear + Dropout + GELU backward with bias gradient");
+          }
+          int const rc = ffk_linear_backward_dropout_gelu(s.require_gpu(), type, dy, xp, gelu_in, gelu_in_grad, w, dw, bias_grad, batch,
                                                           in_dim, out_dim, ws_bytes ? scratch : nullptr, ws_bytes, acc_w, rate, seed,
                                                           offset);
           if (rc != FFK_ERR_UNSUPPORTED) return check_ffk(rc, "Linear + Dropout + GELU backward");
-          check_ffk(ffk_linear_backward(s.require_gpu(), type, act, 0, y, dy, xp, dx, w, dw, dbias, batch, in_dim, out_dim,
+          check_ffk(ffk_linear_backward(s.require_gpu(), type, act, 0, y, dy, xp, dx, w, dw, bias_grad, batch, in_dim, out_dim,
                                         ws_bytes ? scratch : nullptr, ws_bytes, accumulate),
                     "Linear backward");
           check_ffk(ffk_dropout_gelu_backward(s.require_gpu(), type, dx, gelu_in, gelu_in_grad, n, rate, seed, offset),
@@ -715,6 +818,55 @@ ComputationGraphInstance create_computation_graph_instance(
                                           ws_bytes, accumulate),
                   "LayerNorm backward");
       };
+      if (ln_pre[l] >= 0) {
+        // x = residual + dropout(u) is computed here, where the add's output lives
+        ComputationGraph::Layer const &add = cg.layers[(size_t)ln_pre[l]];
+        size_t const d = partner[(size_t)ln_pre[l]];
+        ComputationGraph::Layer const &drop = cg.layers[d];
+        DropoutAttrs const &da = std::get<DropoutAttrs>(drop.attrs.op_attrs);
+        float const rate = da.rate;
+        uint64_t const seed = da.seed + (uint64_t)d;
+        int64_t const n = numel(x);
+        void *u = val(drop.inputs[0]);
+        void *residual = val(add.inputs[0] == drop.outputs.at(0) ? add.inputs[1] : add.inputs[0]);
+        f = [=](device_stream_t const &s) {
+          uint64_t const offset = S->iteration * (uint64_t)n;
+          int const rc = ffk_dropout_add_layer_norm_forward(s.require_gpu(), type, u, residual, xp, y, gamma, beta, mean, rstd, M,
+                                                            N, eps, rate, seed, offset);
+          if (rc != FFK_ERR_UNSUPPORTED) return check_ffk(rc, "Dropout + add + LayerNorm forward");
+          check_ffk(ffk_dropout_add_forward(s.require_gpu(), type, u, residual, xp, n, rate, seed, offset), "Dropout + add forward");
+          check_ffk(ffk_layer_norm_forward(s.require_gpu(), type, xp, y, gamma, beta, mean, rstd, M, N, eps), "LayerNorm forward");
+        };
+      }
+      if (ln_residual[l] >= 0) {
+        void *residual = grd(cg.layers[(size_t)ln_residual[l]].outputs.at(0));
+        int64_t const n = numel(x);
+        int const acc_params = 0;
+        void *dropped_grad = nullptr;
+        float rate = 0.0f;
+        uint64_t seed = 0;
+        if (ln_drop[l] >= 0) {
+          size_t const d = (size_t)ln_drop[l];
+          DropoutAttrs const &da = std::get<DropoutAttrs>(cg.layers[d].attrs.op_attrs);
+          dropped_grad = grd(cg.layers[d].inputs[0]);
+          rate = da.rate;
+          seed = da.seed + (uint64_t)d;
+        }
+        b = [=](device_stream_t const &s) {
+          uint64_t const offset = S->iteration * (uint64_t)n;
+          int const rc = ffk_layer_norm_backward_residual(s.require_gpu(), type, dy, xp, mean, rstd, gamma, residual, dx, dgamma,
+                                                          dbeta, M, N, scratch, ws_bytes, acc_params, dropped_grad, rate, seed,
+                                                          offset);
+          if (rc != FFK_ERR_UNSUPPORTED) return check_ffk(rc, "LayerNorm backward with residual");
+          check_ffk(ffk_cast_forward(s.require_gpu(), type, type, residual, dx, n), "ElementBinary backward");
+          check_ffk(ffk_layer_norm_backward(s.require_gpu(), type, dy, xp, mean, rstd, gamma, dx, dgamma, dbeta, M, N, scratch,
+                                            ws_bytes, FFK_LN_ACC_INPUT),
+                    "LayerNorm backward");
+          if (dropped_grad != nullptr) {
+            check_ffk(ffk_dropout_backward(s.require_gpu(), type, dx, dropped_grad, n, rate, seed, offset, 0), "Dropout backward");
+          }
+        };
+      }
     } else if (auto const *a = std::get_if<MultiHeadAttentionAttrs>(&oa)) {
       tensor_guid_t q = layer.inputs[0], k = layer.inputs[1], v = layer.inputs[2];
       int const type = dt(shape_of(q).data_type);
@@ -760,6 +912,25 @@ ComputationGraphInstance create_computation_graph_instance(
         b = [](device_stream_t const &) {};
       } else if (fused[l] == Fused::DROPOUT_ADD_HEAD) {
         f = [](device_stream_t const &) {};  // the add computes residual + dropout(x)
+      }
+      if (drop_bwd_by_ln[l]) b = [](device_stream_t const &) {};  // the LayerNorm behind the add has written dx
+      if (drop_bias[l] >= 0) {
+        size_t const lin = (size_t)drop_bias[l];
+        LinearAttrs const &la = std::get<LinearAttrs>(cg.layers[lin].attrs.op_attrs);
+        int64_t const out_dim = la.out_channels, batch = n / out_dim;
+        std::shared_ptr<bool> const done = bias_done[lin];
+        void *dbias = grd(cg.layers[lin].weights.at(1));
+        int const acc_bias = plan[lin].bwd.accumulate_input.at(2) ? 1 : 0;
+        void *lin_scratch = base + plan[lin].scratch.offset;
+        size_t const lin_scratch_bytes = plan[lin].scratch_bytes;
+        b = [=](device_stream_t const &s) {
+          uint64_t const offset = S->iteration * (uint64_t)n;
+          int const rc = ffk_dropout_backward_bias_grad(s.require_gpu(), type, dy, dx, batch, out_dim, dbias, acc_bias, lin_scratch,
+                                                        lin_scratch_bytes, rate, seed, offset);
+          *done = rc == FFK_OK;
+          if (rc != FFK_ERR_UNSUPPORTED) return check_ffk(rc, "Dropout backward with bias gradient");
+          check_ffk(ffk_dropout_backward(s.require_gpu(), type, dy, dx, n, rate, seed, offset, accumulate), "Dropout backward");
+        };
       }
     } else if (auto const *a = std::get_if<ElementUnaryAttrs>(&oa)) {
       tensor_guid_t x = layer.inputs[0];
@@ -812,12 +983,14 @@ ComputationGraphInstance create_computation_graph_instance(
                     "Dropout + add forward");
         };
         if (sum_linear[l] >= 0) f = [](device_stream_t const &) {};  // the Linear has written residual + dropout(Linear)
+        if (add_fwd_by_ln[l]) f = [](device_stream_t const &) {};    // the LayerNorm that reads the sum computes it
       }
       if (p.bwd.add_by_alias) {
         // operands whose gradient is dy's own memory need nothing; the others get grad += dy
         // ... or, where this add is the first of them to run, grad = dy
-        void *add_l = has_grad[lhs.raw] && alias_of[lhs.raw] < 0 ? grd(lhs) : nullptr;
-        void *add_r = has_grad[rhs.raw] && alias_of[rhs.raw] < 0 ? grd(rhs) : nullptr;
+        // ... and nothing where a LayerNorm that reads the operand takes dy as its residual
+        void *add_l = has_grad[lhs.raw] && alias_of[lhs.raw] < 0 && deferred_to_ln[lhs.raw] < 0 ? grd(lhs) : nullptr;
+        void *add_r = has_grad[rhs.raw] && alias_of[rhs.raw] < 0 && deferred_to_ln[rhs.raw] < 0 ? grd(rhs) : nullptr;
         bool const store_l = add_l != nullptr && !adds_here(lhs, l), store_r = add_r != nullptr && !adds_here(rhs, l);
         b = [=](device_stream_t const &s) {
           for (int side = 0; side < 2; side++) {

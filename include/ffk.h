@@ -405,6 +405,82 @@ int ffk_linear_backward_dropout_gelu(
     int64_t out_dim, void *workspace, size_t workspace_bytes, int accumulate,
     float rate, uint64_t seed, uint64_t offset);
 
+/* The bias gradient of a Linear taken where the gradient of its output is
+ * produced, instead of by a pass of its own over that gradient.  No
+ * counterpart in the reference, whose Linear backward sums the bias gradient
+ * with a GEMV against a vector of ones (linear_kernels.cu:286-300).  Results
+ * are the bits of the separate entries (the sums are taken over the gradient
+ * as stored, in the order ffk_linear_backward takes them).
+ *   ffk_dropout_backward_bias_grad: the Dropout that follows a Linear:
+ *     input_grad [batch, out_dim] = dropout_backward(output_grad);
+ *     bias_grad [out_dim] (+)= its column sums; the Linear's backward is then
+ *     called with bias_grad NULL.  FLOAT or BF16.  workspace:
+ *     ffk_dropout_backward_bias_grad_workspace_bytes(batch, out_dim).
+ *   ffk_linear_backward_dropout_gelu_bias_grad: ffk_linear_backward_dropout_
+ *     gelu that also gives the bias gradient of the Linear whose output was
+ *     gelu_input: gelu_bias_grad [in_dim] (+)= column sums of input_grad,
+ *     taken on the GEMM's tile store.  gelu_bias_workspace:
+ *     ffk_dropout_backward_bias_grad_workspace_bytes(batch, in_dim) bytes
+ *     that nothing else uses until the call returns (inside
+ *     ffk_column_reductions_begin/_end: until _end).
+ * FFK_ERR_UNSUPPORTED before any kernel is launched when the shape has no
+ * such kernel; the caller then runs the plain entries.                      */
+size_t ffk_dropout_backward_bias_grad_workspace_bytes(int64_t batch,
+                                                      int64_t out_dim);
+int ffk_dropout_backward_bias_grad(ffk_stream_t stream, int dtype,
+                                   void const *output_grad, void *input_grad,
+                                   int64_t batch, int64_t out_dim,
+                                   void *bias_grad, int accumulate_bias,
+                                   void *workspace, size_t workspace_bytes,
+                                   float rate, uint64_t seed, uint64_t offset);
+int ffk_linear_backward_dropout_gelu_bias_grad(
+    ffk_stream_t stream, int dtype, void const *output_grad, void const *input,
+    void const *gelu_input, void *input_grad, void const *weight,
+    void *weight_grad, void *bias_grad, int64_t batch, int64_t in_dim,
+    int64_t out_dim, void *workspace, size_t workspace_bytes, int accumulate,
+    float rate, uint64_t seed, uint64_t offset, void *gelu_bias_grad,
+    int accumulate_gelu_bias, void *gelu_bias_workspace,
+    size_t gelu_bias_workspace_bytes);
+
+/* LayerNorm next to the residual add and the dropout of a transformer block.
+ * No counterpart in the reference (one kernel per operator, as above): the
+ * sequences are Dropout -> ElementBinary add -> LayerNorm going forward
+ * (dropout_kernels.cu:60-79, element_binary_kernels.cu:104-170,
+ * layer_norm_kernels.cu:69-112) and, going back, the add's backward handing
+ * its output gradient to the residual branch, LayerNorm backward adding into
+ * it, and the Dropout's backward reading the sum.  Results are the bits of
+ * the separate entries run one after the other.  FLOAT or BF16 (the dropout
+ * forms BF16 only), rows of a multiple of 8 elements that fit the one-pass
+ * kernel, 16-byte aligned tensors, offset a multiple of 8; anything else is
+ * FFK_ERR_UNSUPPORTED before any kernel is launched and the caller runs the
+ * separate operators.
+ *   ffk_dropout_add_layer_norm_forward:
+ *     sum [M,N] = residual + dropout(input); output = LayerNorm(sum);
+ *     mean / rstd as ffk_layer_norm_forward writes them
+ *   ffk_layer_norm_backward_residual: ffk_layer_norm_backward whose input
+ *     gradient starts from another tensor:
+ *     input_grad = residual + (gradient of the LayerNorm's input), rounded
+ *     once -- what FFK_LN_ACC_INPUT gives when input_grad holds a copy of
+ *     residual (the gradient of the add's output); gamma_grad / beta_grad as
+ *     ffk_layer_norm_backward (accumulate_params != 0 adds into them);
+ *     dropped_grad (optional, BF16) = dropout_backward(input_grad as stored),
+ *     the gradient of the input of the Dropout whose output was the other
+ *     operand of the add that produced the LayerNorm's input.               */
+int ffk_dropout_add_layer_norm_forward(ffk_stream_t stream, int dtype,
+                                       void const *input, void const *residual,
+                                       void *sum, void *output,
+                                       void const *gamma, void const *beta,
+                                       float *mean, float *rstd, int64_t M,
+                                       int64_t N, float eps, float rate,
+                                       uint64_t seed, uint64_t offset);
+int ffk_layer_norm_backward_residual(
+    ffk_stream_t stream, int dtype, void const *output_grad, void const *input,
+    float const *mean, float const *rstd, void const *gamma,
+    void const *residual, void *input_grad, void *gamma_grad, void *beta_grad,
+    int64_t M, int64_t N, void *workspace, size_t workspace_bytes,
+    int accumulate_params, void *dropped_grad, float rate, uint64_t seed,
+    uint64_t offset);
+
 /* ------------------------------------------------------------------------ */
 /* Embedding -- Kernels::Embedding::gpu_forward_kernel / gpu_backward_kernel
  * (embedding_kernels_gpu.h:10-28; lib/kernels/src/cuda/embedding_kernels.cu:

@@ -363,6 +363,50 @@ def test_linear_with_gelu_and_dropout_on_the_tile_store_equals_separate_operator
     assert torch.equal(dx.view(torch.int16), dx_sep.view(torch.int16))
     assert torch.equal(dw.view(torch.int16), dw_sep.view(torch.int16))
     assert torch.equal(db.view(torch.int16), db_sep.view(torch.int16))
+    # ... and with the first Linear's bias gradient summed on the same tile store
+    db1_sep = torch.empty((out_dim,), dtype=bt, device="cuda")
+    ffk.linear_backward(None, dx_sep, x, w, dx=None, dw=None, db=db1_sep, accumulate=0)
+    db1 = torch.full_like(db1_sep, 5.0)
+    try:
+        dx = ffk.linear_backward_dropout_gelu_bias_grad(dy2, dropped, y, w2, rate, seed, db1, offset, dw=dw, db=db)
+    except ffk.FFKError as e:
+        assert "no fused kernel" in str(e) and (batch, in_dim, out_dim) != (4096, 1024, 4096)
+        return
+    assert torch.equal(dx.view(torch.int16), dx_sep.view(torch.int16))
+    assert torch.equal(dw.view(torch.int16), dw_sep.view(torch.int16))
+    assert torch.equal(db.view(torch.int16), db_sep.view(torch.int16))
+    assert torch.equal(db1.view(torch.int16), db1_sep.view(torch.int16))
+    ffk.linear_backward_dropout_gelu_bias_grad(dy2, dropped, y, w2, rate, seed, db1, offset, dw=dw, db=db,
+                                               accumulate_gelu_bias=True)
+    ffk.linear_backward(None, dx_sep, x, w, dx=None, dw=None, db=db1_sep, accumulate=4)  # FFK_ACC_BIAS
+    assert torch.equal(db1.view(torch.int16), db1_sep.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("batch,out_dim", [(4096, 1024), (512, 4096), (100, 64), (33, 8), (7, 5)])
+def test_dropout_backward_with_the_bias_gradient_equals_separate_operators(ffk, dtype, batch, out_dim):
+    """ffk_dropout_backward_bias_grad: the bits of ffk_dropout_backward followed by the column sums
+    ffk_linear_backward takes for the bias gradient; shapes without such a kernel are refused."""
+    say("dropout backward with bias gradient", dtype, (batch, out_dim))
+    g = rng(batch + out_dim)
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda a: a)
+    dy = to_dev(rnd(g.standard_normal((batch, out_dim)).astype(np.float32)), torch, dtype)
+    rate, seed, offset = 0.1, 4242, 64
+    dx_sep = ffk.dropout_backward(dy, rate, seed, offset)
+    x = torch.zeros((batch, 8), dtype=dtype, device="cuda")
+    w = torch.zeros((out_dim, 8), dtype=dtype, device="cuda")
+    db_sep = torch.empty((out_dim,), dtype=dtype, device="cuda")
+    ffk.linear_backward(None, dx_sep, x, w, dx=None, dw=None, db=db_sep, accumulate=0)
+    db = torch.full_like(db_sep, 3.0)
+    try:
+        dx = ffk.dropout_backward_bias_grad(dy, rate, seed, db, offset)
+    except ffk.FFKError as e:
+        assert "no fused kernel" in str(e) and (batch, out_dim) not in ((4096, 1024), (512, 4096))
+        return
+    assert torch.equal(dx, dx_sep) and torch.equal(db, db_sep)
+    ffk.dropout_backward_bias_grad(dy, rate, seed, db, offset, accumulate_bias=True)
+    ffk.linear_backward(None, dx_sep, x, w, dx=None, dw=None, db=db_sep, accumulate=4)  # FFK_ACC_BIAS
+    assert torch.equal(db, db_sep)
 
 
 def test_linear_with_fused_tail_refuses_shapes_without_a_kernel(ffk):

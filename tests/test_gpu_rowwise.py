@@ -81,6 +81,80 @@ def test_layer_norm_many_rows_bf16(ffk, oracle):
     assert_close(to_np(db), db_ref, BF16_RTOL, "dbeta")
 
 
+@pytest.mark.parametrize("shape", [(33, 1024), (64, 4096), (130, 768), (7, 64), (9, 8192), (4096, 1024)])
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_layer_norm_backward_residual_is_copy_then_accumulate(ffk, shape, dtype):
+    """input_grad = residual + gradient in one kernel has the bits of copying residual into
+    input_grad and letting the plain backward add into it (whose values the oracle checks
+    above); with a dropout the third output has the bits of ffk_dropout_backward on the sum."""
+    M, N = shape
+    say("layer_norm backward residual", shape, dtype)
+    g = rng(M + N)
+    td = torch.float32 if dtype == "fp32" else torch.bfloat16
+    rnd = (lambda a: a.astype(np.float32)) if dtype == "fp32" else bf16_round
+    x, dy, res = (rnd(g.standard_normal((M, N))) for _ in range(3))
+    gamma = rnd(1 + 0.02 * g.standard_normal((N,)))
+    beta = rnd(0.02 * g.standard_normal((N,)))
+    xd, dyd, rd, gd, bd = (to_dev(a, torch, td) for a in (x, dy, res, gamma, beta))
+    _, mean, rstd = ffk.layer_norm_forward(xd, gd, bd, 1e-5)
+    dx0, dg0, db0 = rd.clone(), torch.zeros_like(gd), torch.zeros_like(bd)
+    ffk.layer_norm_backward(dyd, xd, mean, rstd, gd, dx0, dg0, db0, accumulate=True)
+    dx1, dg1, db1 = torch.full_like(xd, 7.0), torch.zeros_like(gd), torch.zeros_like(bd)
+    ffk.layer_norm_backward_residual(dyd, xd, mean, rstd, gd, rd, dx1, dg1, db1)
+    assert torch.equal(dx0, dx1) and torch.equal(dg0, dg1) and torch.equal(db0, db1)
+    if dtype == "bf16":
+        rate, seed, offset = 0.1, 1234, 8 * 5
+        dx2, dropped = torch.empty_like(xd), torch.empty_like(xd)
+        ffk.layer_norm_backward_residual(dyd, xd, mean, rstd, gd, rd, dx2, dg1, db1, dropped=dropped, rate=rate,
+                                         seed=seed, offset=offset)
+        assert torch.equal(dx0, dx2)
+        assert torch.equal(dropped, ffk.dropout_backward(dx0, rate, seed, offset))
+        # parameter gradients added into what is there
+        dg3, db3 = dg0.clone(), db0.clone()
+        ffk.layer_norm_backward_residual(dyd, xd, mean, rstd, gd, rd, dx2, dg3, db3, accumulate_params=True)
+        dg4, db4 = dg0.clone(), db0.clone()
+        ffk.layer_norm_backward(dyd, xd, mean, rstd, gd, dx0.clone(), dg4, db4, accumulate=3)
+        assert torch.equal(dg3, dg4) and torch.equal(db3, db4)
+
+
+@pytest.mark.parametrize("shape", [(33, 1024), (64, 4096), (130, 768), (7, 64), (4096, 1024)])
+def test_dropout_add_layer_norm_forward_is_the_three_operators(ffk, shape):
+    M, N = shape
+    say("dropout + add + layer_norm forward", shape)
+    g = rng(M * 3 + N)
+    bt = torch.bfloat16
+    x, res = (to_dev(bf16_round(g.standard_normal((M, N))), torch, bt) for _ in range(2))
+    gamma = to_dev(bf16_round(1 + 0.02 * g.standard_normal((N,))), torch, bt)
+    beta = to_dev(bf16_round(0.02 * g.standard_normal((N,))), torch, bt)
+    rate, seed, offset = 0.1, 99, 16
+    total, y, mean, rstd = ffk.dropout_add_layer_norm_forward(x, res, gamma, beta, 1e-5, rate, seed, offset)
+    want_total = ffk.dropout_add_forward(x, res, rate, seed, offset)
+    want_y, want_mean, want_rstd = ffk.layer_norm_forward(want_total, gamma, beta, 1e-5)
+    assert torch.equal(total, want_total) and torch.equal(y, want_y)
+    assert torch.equal(mean, want_mean) and torch.equal(rstd, want_rstd)
+
+
+def test_layer_norm_fused_forms_refuse_what_they_cannot_run(ffk):
+    """Rows that are no multiple of 8 elements have no one-pass kernel: FFK_ERR_UNSUPPORTED, nothing written."""
+    bt = torch.bfloat16
+    x = torch.zeros((4, 100), device="cuda", dtype=bt)
+    gamma = torch.ones((100,), device="cuda", dtype=bt)
+    m = torch.zeros((4,), device="cuda")
+    dx = torch.full_like(x, 3.0)
+    ws = torch.empty((ffk.lib().ffk_layer_norm_backward_workspace_bytes(4, 100),), dtype=torch.uint8, device="cuda")
+    rc = ffk.lib().ffk_layer_norm_backward_residual(0, ffk.BF16, x.data_ptr(), x.data_ptr(), m.data_ptr(), m.data_ptr(),
+                                                    gamma.data_ptr(), x.data_ptr(), dx.data_ptr(), None, None, 4, 100,
+                                                    ws.data_ptr(), ws.numel(), 0, None, 0.0, 0, 0)
+    assert rc == ffk.ERR_UNSUPPORTED
+    y = torch.full_like(x, 3.0)
+    rc = ffk.lib().ffk_dropout_add_layer_norm_forward(0, ffk.BF16, x.data_ptr(), x.data_ptr(), dx.data_ptr(), y.data_ptr(),
+                                                      gamma.data_ptr(), gamma.data_ptr(), m.data_ptr(), m.data_ptr(), 4, 100,
+                                                      1e-5, 0.1, 1, 0)
+    assert rc == ffk.ERR_UNSUPPORTED
+    torch.cuda.synchronize()
+    assert bool((dx == 3.0).all()) and bool((y == 3.0).all())
+
+
 def test_layer_norm_workspace_error(ffk):
     x = torch.zeros((8, 64), device="cuda")
     m = torch.zeros((8,), device="cuda")
