@@ -408,7 +408,7 @@ int ffk_linear_backward_dropout_gelu(
 /* The bias gradient of a Linear taken where the gradient of its output is
  * produced, instead of by a pass of its own over that gradient.  No
  * counterpart in the reference, whose Linear backward sums the bias gradient
- * with a GEMV against a vector of ones (linear_kernels.cu:286-300).  Results
+ * with a GEMM against a vector of ones (linear_kernels.cu:294-317).  Results
  * are the bits of the separate entries (the sums are taken over the gradient
  * as stored, in the order ffk_linear_backward takes them).
  *   ffk_dropout_backward_bias_grad: the Dropout that follows a Linear:
@@ -445,8 +445,8 @@ int ffk_linear_backward_dropout_gelu_bias_grad(
 /* LayerNorm next to the residual add and the dropout of a transformer block.
  * No counterpart in the reference (one kernel per operator, as above): the
  * sequences are Dropout -> ElementBinary add -> LayerNorm going forward
- * (dropout_kernels.cu:60-79, element_binary_kernels.cu:104-170,
- * layer_norm_kernels.cu:69-112) and, going back, the add's backward handing
+ * (dropout_kernels.cu:67-97, element_binary_kernels.cu:146-248,
+ * layer_norm_kernels.cu:412-439) and, going back, the add's backward handing
  * its output gradient to the residual branch, LayerNorm backward adding into
  * it, and the Dropout's backward reading the sum.  Results are the bits of
  * the separate entries run one after the other.  FLOAT or BF16 (the dropout
