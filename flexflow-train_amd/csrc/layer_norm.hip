@@ -41,6 +41,28 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_kernel(
 
   float x[EPT][V];
   float s = 0.0f;
+  // Short rows (up to two vectors per lane): gamma and beta are asked for before the row's two
+  // reductions, not after them: such a kernel is one chain of memory round trips, and this one
+  // then runs under the others.  Longer rows load them where they are used; their registers
+  // are better spent on resident waves.
+  constexpr bool kEarly = EPT <= 2;
+  float g[EPT][V], b[EPT][V];
+  auto load_params = [&](int j) __attribute__((always_inline)) {
+    int v = lane + j * LANES;
+#pragma unroll
+    for (int e = 0; e < V; e++) {
+      g[j][e] = 1.0f;
+      b[j][e] = 0.0f;
+    }
+    if (v < nvec) {
+      if (gamma != nullptr) VecIO<T>::load(gamma + (int64_t)v * V, g[j]);
+      if (beta != nullptr) VecIO<T>::load(beta + (int64_t)v * V, b[j]);
+    }
+  };
+  if constexpr (kEarly) {
+#pragma unroll
+    for (int j = 0; j < EPT; j++) load_params(j);
+  }
 #pragma unroll
   for (int j = 0; j < EPT; j++) {
     int v = lane + j * LANES;
@@ -104,19 +126,12 @@ __global__ __launch_bounds__(kRowThreads) void layer_norm_fwd_kernel(
   for (int j = 0; j < EPT; j++) {
     int v = lane + j * LANES;
     if (v < nvec) {
-      float g[V], b[V], y[V];
-      if (gamma != nullptr) {
-        VecIO<T>::load(gamma + (int64_t)v * V, g);
-      }
-      if (beta != nullptr) {
-        VecIO<T>::load(beta + (int64_t)v * V, b);
-      }
+      float y[V];
+      if constexpr (!kEarly) load_params(j);
 #pragma unroll
       for (int e = 0; e < V; e++) {
         float xh = (x[j][e] - mu) * rs;
-        float gv = gamma != nullptr ? g[e] : 1.0f;
-        float bv = beta != nullptr ? b[e] : 0.0f;
-        y[e] = xh * gv + bv;
+        y[e] = xh * g[j][e] + b[j][e];
       }
       if (STREAM) {
         VecIO<T>::store_stream(yr + (int64_t)v * V, y);
