@@ -363,6 +363,9 @@ __global__ __launch_bounds__(kEmbBlockThreads) void embedding_bwd_sorted_block_k
   if (wl < cnt) {
     my_key = keys[p0 + wl];
     my_val = vals[p0 + wl];
+    // what the walk needs of a lookup is the gradient row it reads: its bag.  Divided once here,
+    // by the lane that holds the pair, not at every position by every lane of the walker.
+    if (bag != 1) my_val /= (uint32_t)bag;
   }
   int const wbase = ((threadIdx.x & 63) / LPR) * LPR;  // the walker's first lane in its wave
   uint32_t const key_before = active && p0 > 0 ? keys[p0 - 1] : invalid_key;
@@ -401,7 +404,7 @@ __global__ __launch_bounds__(kEmbBlockThreads) void embedding_bwd_sorted_block_k
       // walker alone ends there (nobody else touches that row during the kernel)
       auto prefetch = [&](int j, uint32_t id, uint32_t next_id, uint32_t l, float (&v)[CPL][4], f32x4 (&o)[CPL]) {
         if (j >= cnt) return;
-        GT const *row = dY + (int64_t)(bag == 1 ? l : l / (uint32_t)bag) * dim;
+        GT const *row = dY + (int64_t)l * dim;  // l: the lookup's bag (see my_val)
         bool const ends = j + 1 >= cnt || next_id != id;
 #pragma unroll
         for (int k = 0; k < CPL; k++) {
