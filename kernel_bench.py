@@ -82,6 +82,10 @@ def bench_gemm():
             finally:
                 ffk.set_option(ffk.OPTION_GEMM_VARIANT, 0)
             report("  previous kernel (8 waves, 4 x 32-deep stages)", t, flops=2.0 * M * N * K)
+        # the vendor library on the same operands (hipBLASLt, reached through torch.matmul), for scale
+        At, Bt = (A.t() if ta else A), (B.t() if tb else B)
+        t = timeit(lambda: torch.matmul(At, Bt, out=C))
+        report("  vendor library (torch.matmul)", t, flops=2.0 * M * N * K)
 
 
 def bench_fused_linear():
