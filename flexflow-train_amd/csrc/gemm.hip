@@ -674,10 +674,60 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   for (; kt < KT; kt++) {
     tile_step(kt, std::false_type{});
   }
-  __syncthreads();  // all stages are free now: reuse them for the output tile
-
   // acc[i][j][r]: output row m = wm0 + 32 i + lane % 32,
   //               column n = wn0 + 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4.
+  // The plain store (no tail, nothing to add to): straight from the registers.  A lane holds
+  // columns 8 g + 4 h .. + 3 of every group g of 8 (h = its lane half); one swap of the lane
+  // halves per pair of groups gives the lower half the 8 columns of group g and the upper half
+  // those of group g + 1, so that every lane stores 16 bytes and the two halves together 32
+  // contiguous bytes of a row.  No LDS, so no barrier either: a wave writes its tile as soon as
+  // its own loop is done.  Used by the one-wave-per-SIMD kernel, where it is 4-6% of a launch at
+  // reductions up to 2048 (FFN-up shape 37.6 -> 36.0 us); with two waves per SIMD the staged
+  // epilogue below, whose stores are whole 128-byte lines, is 2-5% ahead.
+  if constexpr (TAIL == GemmEpilogue::kTailNone && WM == 128 && WN == 128) {
+    if (partial == nullptr && accumulate == 0) {  // uniform over the launch
+      auto direct = [&](auto actf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          float bv[4][4];
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            u32x2 raw = {0u, 0u};
+            if (bias != nullptr) raw = *reinterpret_cast<u32x2 const *>(bias + n0 + wn0 + j * 32 + 8 * g + 4 * (lane >> 5));
+            bv[g][0] = __uint_as_float(raw[0] << 16);
+            bv[g][1] = __uint_as_float(raw[0] & 0xffff0000u);
+            bv[g][2] = __uint_as_float(raw[1] << 16);
+            bv[g][3] = __uint_as_float(raw[1] & 0xffff0000u);
+          }
+#pragma unroll
+          for (int i = 0; i < TM; i++) {
+            bf16 *const row = C + (int64_t)(m0 + wm0 + i * 32 + (lane & 31)) * ldc + n0 + wn0 + j * 32 + 8 * (lane >> 5);
+#pragma unroll
+            for (int g = 0; g < 4; g += 2) {
+              uint32_t w[2][2];
+#pragma unroll
+              for (int gg = 0; gg < 2; gg++) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = actf(acc[i][j][4 * (g + gg) + e] + bv[g + gg][e]);
+                w[gg][0] = pack_bf16x2(v[0], v[1]);
+                w[gg][1] = pack_bf16x2(v[2], v[3]);
+              }
+              // swaps the upper lane half of the first operand with the lower half of the second
+              auto const lo = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
+              auto const hi = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
+              u32x4 const out = {lo[0], hi[0], lo[1], hi[1]};
+              *reinterpret_cast<u32x4 *>(row + 8 * g) = out;
+            }
+          }
+        }
+      };
+      direct([](float v) { return v; });  // (this kernel is only launched without an activation)
+      return;
+    }
+  }
+  __syncthreads();  // all stages are free now: reuse them for the output tile
+
   // Each wave stages its own WM x WN tile and writes it out in 16-byte chunks.
   bf16 *cs = smem + wave * (WM * CS);
   constexpr int CCH = WM * WN / 8 / 64;  // 16-byte chunks per lane
@@ -1151,10 +1201,10 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
       }
       return hipErrorInvalidValue;
     }
-    // Long reductions without an activation: one wave per SIMD on 128x128 wave tiles, two
-    // 64-deep stages, every instruction of the loop placed by hand.  (Up to about 1024 of K the
-    // eight-wave kernel's shorter prologue and epilogue weigh more than the faster loop.)
-    if (use256 && ep.activation == FFK_ACT_NONE && (variant == 264 || (variant == 0 && K >= 2048))) {
+    // Reductions from 1024 on without an activation: one wave per SIMD on 128x128 wave tiles, two
+    // 64-deep stages, every instruction of the loop placed by hand.  (Below that the eight-wave
+    // kernel's shorter prologue weighs more than the faster loop.)
+    if (use256 && ep.activation == FFK_ACT_NONE && (variant == 264 || (variant == 0 && K >= 1024))) {
       return launch_pipe<256, 256, 128, 128, 64, 2, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
     }
     if (use256) {
