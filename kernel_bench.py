@@ -74,7 +74,7 @@ def bench_gemm():
         t = timeit(lambda: ffk.gemm(A, B, C, bool(ta), bool(tb)))
         report("gemm bf16 M%d N%d K%d %s%s" % (M, N, K, "T" if ta else "N", "T" if tb else "N"), t,
                flops=2.0 * M * N * K)
-        if K >= 2048 and M % 256 == 0 and N % 256 == 0 and (M // 256) * (N // 256) >= 192:
+        if K >= 1024 and M % 256 == 0 and N % 256 == 0 and (M // 256) * (N // 256) >= 192:
             # the eight-wave 256x256 kernel that the one-wave-per-SIMD kernel replaced at these sizes
             ffk.set_option(ffk.OPTION_GEMM_VARIANT, 256)
             try:
