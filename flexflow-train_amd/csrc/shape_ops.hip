@@ -458,6 +458,34 @@ __global__ __launch_bounds__(kShapeThreads) void gather_bwd_kernel(float const *
   }
 }
 
+// Gather along the last dim when most of a row is picked: a workgroup stages its row in LDS with
+// 16-byte loads and picks from there.  Picking from memory fetches a 128-byte line per lane for
+// one element, and a row's lines again for every pick that lands in them.
+constexpr int kGatherRowBytes = 64 * 1024;  // staged row, at most (two workgroups per CU)
+
+template <typename E, typename IT>
+__global__ __launch_bounds__(kShapeThreads) void gather_rows_lds_kernel(E const *__restrict__ in, IT const *__restrict__ index,
+                                                                         E *__restrict__ out, int64_t in_dim, int64_t out_dim) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char gather_row[];
+  E *const row = reinterpret_cast<E *>(gather_row);
+  int64_t const r = blockIdx.x;
+  E const *const src = in + r * in_dim;
+  constexpr int V = 16 / (int)sizeof(E);
+  if (in_dim % V == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0) {
+    for (int64_t c = threadIdx.x; c < in_dim / V; c += kShapeThreads) {
+      reinterpret_cast<u32x4 *>(row)[c] = reinterpret_cast<u32x4 const *>(src)[c];
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < in_dim; c += kShapeThreads) row[c] = src[c];
+  }
+  __syncthreads();
+  for (int64_t o = threadIdx.x; o < out_dim; o += kShapeThreads) {
+    int64_t const j = (int64_t)index[r * out_dim + o];
+    // an index outside the dim reads nothing (the reference would read out of bounds)
+    out[r * out_dim + o] = (j >= 0 && j < in_dim) ? row[j] : E(0);
+  }
+}
+
 // the divisors of a gather over `total` output elements, or false when 32-bit indices do not fit
 static bool gather_divs(int64_t total, int64_t stride, int64_t out_dim, GatherDivs &dv) {
   if (!fits_fast_index(total, kShapeThreads) || total == 0) return false;
@@ -501,6 +529,13 @@ extern "C" int ffk_gather_forward(ffk_stream_t stream, int dtype, int index_dtyp
   FFK_REQUIRE(input && index && output, "gather_forward: NULL tensor");
   hipStream_t st = as_stream(stream);
   unsigned const blocks = blocks_for(total);
+  // last-dim gather that picks at least an eighth of a row that fits LDS: stage the row
+  bool const staged = stride == 1 && output_dim_size * 8 >= input_dim_size && outer < (int64_t(1) << 31) &&
+                      input_dim_size * (int64_t)dtype_size(dtype) <= kGatherRowBytes;
+#define FFK_GATHER_STAGED(E, IT)                                                                             \
+  gather_rows_lds_kernel<E, IT><<<(unsigned)outer, kShapeThreads, (size_t)(input_dim_size * sizeof(E) + 15) / 16 * 16, st>>>( \
+      static_cast<E const *>(input), static_cast<IT const *>(index), static_cast<E *>(output), input_dim_size, \
+      output_dim_size)
   GatherDivs dv{};
   bool const fast = gather_divs(total, stride, output_dim_size, dv);
 #define FFK_GATHER_ONE(E, IT, BIG)                                                                           \
@@ -509,7 +544,10 @@ extern "C" int ffk_gather_forward(ffk_stream_t stream, int dtype, int index_dtyp
       input_dim_size, output_dim_size, dv)
 #define FFK_GATHER(E)                                                                                        \
   do {                                                                                                       \
-    if (index_dtype == FFK_INT32) {                                                                          \
+    if (staged) {                                                                                            \
+      if (index_dtype == FFK_INT32) FFK_GATHER_STAGED(E, int32_t);                                           \
+      else FFK_GATHER_STAGED(E, int64_t);                                                                    \
+    } else if (index_dtype == FFK_INT32) {                                                                   \
       if (fast) FFK_GATHER_ONE(E, int32_t, false);                                                           \
       else FFK_GATHER_ONE(E, int32_t, true);                                                                 \
     } else {                                                                                                 \
@@ -526,6 +564,7 @@ extern "C" int ffk_gather_forward(ffk_stream_t stream, int dtype, int index_dtyp
   }
 #undef FFK_GATHER
 #undef FFK_GATHER_ONE
+#undef FFK_GATHER_STAGED
   FFK_CHECK_LAUNCH();
   return FFK_OK;
 }

@@ -65,6 +65,24 @@ def test_transpose_moves_any_data_type(ffk, dtype):
             ffk.transpose_backward(x.permute(1, 0, 2).contiguous(), torch.zeros_like(x), (1, 0, 2), accumulate=True)
 
 
+@pytest.mark.parametrize("rows,in_dim,picks", [(5, 33, 17), (64, 4096, 1024), (9, 4100, 4100), (3, 20000, 5000), (7, 16384, 2048),
+                                               (4, 1000, 100)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int64])
+def test_gather_along_the_last_dim(ffk, oracle, rows, in_dim, picks, dtype):
+    """Rows picked from densely go through LDS (whole-row staging, vector or element loads), long
+    or sparsely picked rows straight from memory: both move values bit for bit."""
+    say("gather along the last dim", (rows, in_dim, picks), dtype)
+    g = rng(rows + in_dim)
+    x = g.integers(-1000, 1000, size=(rows, in_dim)).astype(np.float32)
+    idx = g.integers(0, in_dim, size=(rows, picks))
+    idx.flat[::53] = in_dim                   # out-of-range entries read 0
+    idx.flat[::59] = -3
+    xd = to_dev(x, torch).to(dtype)
+    out = ffk.gather_forward(xd, to_dev(idx, torch, torch.int64), 1)
+    want = oracle.gather_forward(xd.to(torch.float32).cpu().numpy(), idx, 1)   # values as the type holds them
+    assert np.array_equal(out.to(torch.float32).cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("dim", [0, 1, 2])
 @pytest.mark.parametrize("itype", [torch.int32, torch.int64])
 def test_gather_forward_backward(ffk, oracle, dim, itype):
