@@ -486,6 +486,47 @@ __global__ __launch_bounds__(kShapeThreads) void gather_rows_lds_kernel(E const 
   }
 }
 
+// The backward of such a Gather: the workgroup sums its row's gradient in LDS (LDS float adds: no
+// trip to memory per element, no contention between rows) and adds the touched elements to the
+// input gradient once, 16 bytes per lane where the row allows.  Adds through memory atomics run at
+// a few per cent of the memory rate.
+template <typename IT>
+__global__ __launch_bounds__(kShapeThreads) void gather_rows_lds_bwd_kernel(float const *__restrict__ dout,
+                                                                             IT const *__restrict__ index, float *din,
+                                                                             int64_t in_dim, int64_t out_dim) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char gather_row[];
+  float *const row = reinterpret_cast<float *>(gather_row);
+  int64_t const r = blockIdx.x;
+  float *const dst = din + r * in_dim;
+  bool const wide = in_dim % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+  // whole 16-byte groups are cleared (the LDS size is rounded up to them)
+  for (int64_t c = threadIdx.x; c < (in_dim + 3) / 4; c += kShapeThreads) {
+    reinterpret_cast<f32x4 *>(row)[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  __syncthreads();
+  for (int64_t o = threadIdx.x; o < out_dim; o += kShapeThreads) {
+    int64_t const j = (int64_t)index[r * out_dim + o];
+    if (j >= 0 && j < in_dim) atomicAdd(row + j, dout[r * out_dim + o]);
+  }
+  __syncthreads();
+  // an element nobody picked keeps its bits (the reference's atomics never touch it)
+  if (wide) {
+    for (int64_t c = threadIdx.x; c < in_dim / 4; c += kShapeThreads) {
+      f32x4 const v = reinterpret_cast<f32x4 const *>(row)[c];
+      if (v[0] != 0.f || v[1] != 0.f || v[2] != 0.f || v[3] != 0.f) {
+        f32x4 d = reinterpret_cast<f32x4 const *>(dst)[c];
+        for (int e = 0; e < 4; ++e) d[e] = v[e] != 0.f ? d[e] + v[e] : d[e];
+        reinterpret_cast<f32x4 *>(dst)[c] = d;
+      }
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < in_dim; c += kShapeThreads) {
+      float const v = row[c];
+      if (v != 0.f) dst[c] += v;
+    }
+  }
+}
+
 // the divisors of a gather over `total` output elements, or false when 32-bit indices do not fit
 static bool gather_divs(int64_t total, int64_t stride, int64_t out_dim, GatherDivs &dv) {
   if (!fits_fast_index(total, kShapeThreads) || total == 0) return false;
@@ -579,6 +620,20 @@ extern "C" int ffk_gather_backward(ffk_stream_t stream, int index_dtype, float c
   FFK_REQUIRE(output_grad && index && input_grad, "gather_backward: NULL tensor");
   hipStream_t st = as_stream(stream);
   unsigned const blocks = blocks_for(total);
+  // along the last dim, rows that fit LDS and are picked from at least once per 16 elements
+  if (stride == 1 && output_dim_size * 16 >= input_dim_size && outer < (int64_t(1) << 31) &&
+      input_dim_size * (int64_t)sizeof(float) <= kGatherRowBytes) {
+    size_t const lds = (size_t)(input_dim_size + 3) / 4 * 16;
+    if (index_dtype == FFK_INT32) {
+      gather_rows_lds_bwd_kernel<int32_t><<<(unsigned)outer, kShapeThreads, lds, st>>>(
+          output_grad, static_cast<int32_t const *>(index), input_grad, input_dim_size, output_dim_size);
+    } else {
+      gather_rows_lds_bwd_kernel<int64_t><<<(unsigned)outer, kShapeThreads, lds, st>>>(
+          output_grad, static_cast<int64_t const *>(index), input_grad, input_dim_size, output_dim_size);
+    }
+    FFK_CHECK_LAUNCH();
+    return FFK_OK;
+  }
   GatherDivs dv{};
   bool const fast = gather_divs(total, stride, output_dim_size, dv);
 #define FFK_GATHER_BWD(IT, BIG)                                                                              \

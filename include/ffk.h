@@ -795,8 +795,10 @@ int ffk_transpose_backward(ffk_stream_t stream, int dtype,
  * around the gathered dim; index has the output's shape, int32 or int64:
  *   output[o, j, s] = input[o, index[o, j, s], s]
  * (an index outside [0, input_dim_size) yields 0 / is skipped).  Forward moves
- * any data type; backward adds float gradients with hardware atomics, like the
- * reference (input_grad is accumulated into).                                */
+ * any data type; backward adds float gradients into input_grad: with hardware
+ * atomics like the reference, or, along the innermost dim (stride 1) into rows
+ * of at most 64 KB, summed per row in LDS first.  The order of the adds is
+ * not fixed in either form.                                                  */
 /* ------------------------------------------------------------------------ */
 int ffk_gather_forward(ffk_stream_t stream, int dtype, int index_dtype,
                        void const *input, void const *index, void *output,

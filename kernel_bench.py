@@ -323,7 +323,7 @@ def bench_shape():
     report("Gather [16384,4096] -> [16384,1024] along dim 1 (fp32)", t, bytes_=idx2.numel() * (4 + 4) + src.numel() * 4)
     gin = torch.zeros_like(src)
     t = timeit(lambda: ffk.gather_backward(out2, idx2, gin, 1))
-    report("Gather backward (atomics) [16384,1024] -> [16384,4096]", t, bytes_=idx2.numel() * (4 + 4 + 8))
+    report("Gather backward (row sums in LDS) [16384,1024] -> [16384,4096]", t, bytes_=idx2.numel() * (4 + 4 + 8))
 
 
 GROUPS = dict(gemm=bench_gemm, fused_linear=bench_fused_linear, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention,

@@ -83,6 +83,32 @@ def test_gather_along_the_last_dim(ffk, oracle, rows, in_dim, picks, dtype):
     assert np.array_equal(out.to(torch.float32).cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("rows,in_dim,picks", [(5, 33, 17), (64, 4096, 1024), (9, 4100, 300), (3, 20000, 5000), (7, 16384, 2048),
+                                               (4, 1000, 10)])
+@pytest.mark.parametrize("itype", [torch.int32, torch.int64])
+def test_gather_backward_along_the_last_dim(ffk, oracle, rows, in_dim, picks, itype):
+    """Rows summed in LDS and rows added to with memory atomics give the reference's sums; integer-valued
+    gradients make them exact whatever the order of the adds, and unpicked elements keep their bits."""
+    say("gather backward along the last dim", (rows, in_dim, picks), itype)
+    g = rng(rows + in_dim + 1)
+    idx = g.integers(0, in_dim, size=(rows, picks))
+    idx[:, : picks // 2] = idx[:, picks // 2: picks // 2 * 2] // 7   # repeated targets
+    idx.flat[::53] = in_dim
+    idx.flat[::59] = -3
+    dout = g.integers(-64, 64, size=(rows, picks)).astype(np.float32)
+    old = g.integers(-64, 64, size=(rows, in_dim)).astype(np.float32)
+    old.flat[::5] = -0.0
+    din = to_dev(old, torch)
+    ffk.gather_backward(to_dev(dout, torch), to_dev(idx, torch, itype), din, 1)
+    want = oracle.gather_backward(dout, idx, old, 1)
+    got = to_np(din)
+    assert np.array_equal(got, want)
+    untouched = np.ones_like(old, dtype=bool)
+    ok = (idx >= 0) & (idx < in_dim)
+    untouched[np.nonzero(ok)[0], idx[ok]] = False
+    assert np.array_equal(got.view(np.uint32)[untouched], old.view(np.uint32)[untouched])
+
+
 @pytest.mark.parametrize("dim", [0, 1, 2])
 @pytest.mark.parametrize("itype", [torch.int32, torch.int64])
 def test_gather_forward_backward(ffk, oracle, dim, itype):
