@@ -58,6 +58,26 @@ HBM_PEAK_GBPS = 8000.0
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "ffn_up_gemm_hbm_traffic.md")
 
 
+SETTLE_SECONDS = 0.2
+
+
+def settle_clocks(fn, least=0, seconds=SETTLE_SECONDS):
+    """Runs fn untimed, at least `least` times and for at least `seconds`: the card's shader clock
+    needs some tens of milliseconds of sustained load to reach the state it then holds (launches
+    in the first 50 ms after an idle spell measure 10-20% slow, 40 consecutive launches of one
+    kernel show the time falling launch by launch), and a timed region that starts inside that
+    ramp measures the ramp.  Returns the number of calls made."""
+    import torch
+    n = 0
+    t0 = time.perf_counter()
+    while n < least or time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        n += 20
+        torch.cuda.synchronize()
+    return n
+
+
 def event_timer(ffk):
     """us per call of fn, HIP events on the stream the entry points are launched on."""
     lib = ffk.lib()
@@ -67,8 +87,7 @@ def event_timer(ffk):
         e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
         ffk.check(lib.ffk_event_create(ctypes.byref(e0)))
         ffk.check(lib.ffk_event_create(ctypes.byref(e1)))
-        for _ in range(warm):
-            fn()
+        settle_clocks(fn, warm)
         ffk.check(lib.ffk_event_record(e0, stream))
         for _ in range(iters):
             fn()
@@ -493,6 +512,8 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
                     help="BASELINE configuration to measure (2 = the headline transformer layer)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle-seconds", type=float, default=SETTLE_SECONDS,
+                    help="untimed steps run for this long before the warm-up steps (0: none)")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant kernel's timing loop and a 256 MiB calibration "
                          "copy (for rocprofv3 counter runs)")
@@ -519,6 +540,7 @@ def main():
         return
     st = make_device_state(ffk, torch, CFG)
     check = check_before_timing(ffk, torch, st)
+    settled = settle_clocks(lambda: step(ffk, st), seconds=args.settle_seconds) if args.settle_seconds > 0 else 0
     for _ in range(args.warmup):
         step(ffk, st)
     torch.cuda.synchronize()
@@ -542,6 +564,8 @@ def main():
                                "dropout 0.1 (BASELINE config 2)",
                    "tokens_per_step": tokens, "algorithmic_gflop_per_step": 335.0},
         "step_tflops": 335.0e9 / (dt / args.steps) / 1e12,
+        "clock_settle": {"untimed_steps_before_warmup": settled, "seconds": args.settle_seconds,
+                         "why": "the shader clock ramps for tens of ms after idle; value is the steady state"},
         "check": check,
         "roofline": roof,
         "device_copy": measure_device_copy(ffk, torch),

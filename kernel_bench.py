@@ -14,6 +14,7 @@ synthetic (seeded normal / Zipf) and already resident in HBM.
 """
 import importlib.util
 import math
+import time
 import os
 import sys
 
@@ -31,9 +32,16 @@ HBM_PEAK = 8e12
 MFMA_PEAK = 2.5e15
 
 
-def timeit(fn, iters=20, warm=5):
-    for _ in range(warm):
+def timeit(fn, iters=20, warm=5, settle=0.1):
+    # at least `warm` calls and `settle` seconds of untimed load first: the shader clock takes tens
+    # of milliseconds of sustained work to reach the state it then holds, and the first launches
+    # after an idle spell (building the next case's tensors is one) run 10-20% slow
+    n, t0 = 0, time.perf_counter()
+    while n < warm or time.perf_counter() - t0 < settle:
         fn()
+        n += 1
+        if n % 10 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     s = torch.cuda.Event(enable_timing=True)
     e = torch.cuda.Event(enable_timing=True)
