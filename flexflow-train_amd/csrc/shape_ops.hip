@@ -158,7 +158,10 @@ __global__ __launch_bounds__(kShapeThreads) void permute_tiles_kernel(E const *_
 // outer stride a multiple of V and 16-byte aligned tensors; one-element
 // transactions (128 bytes per wave for bf16) otherwise leave the bf16
 // transpose at under half of what the wide form moves.
-template <typename E, int MODE>
+// STREAM: a tensor too large to stay in the last-level cache is read past the caches (its stores stay
+// ordinary: the strided 256-byte row pieces of a tile want the L2's write combining; streaming them too
+// cost 10%).
+template <typename E, int MODE, bool STREAM>
 __global__ __launch_bounds__(kShapeThreads) void permute_tiles_wide_kernel(E const *__restrict__ in, E *out, TileArgs t) {
   constexpr int V = 16 / (int)sizeof(E);
   // Row pitch of the staged tile.  4-byte elements: an odd pitch, so that the column reads of the
@@ -185,7 +188,8 @@ __global__ __launch_bounds__(kShapeThreads) void permute_tiles_wide_kernel(E con
     for (int k = 0; k < kTile; k += RPP) {
       int64_t const bb = b0 + row + k, aa = a0 + piece * V;
       if (bb < t.B && aa < t.A) {  // A and B are multiples of V: a piece is inside or outside as a whole
-        u32x4 const q = *reinterpret_cast<u32x4 const *>(in + in_off + bb * t.in_stride_b + aa);
+        u32x4 const *const src = reinterpret_cast<u32x4 const *>(in + in_off + bb * t.in_stride_b + aa);
+        u32x4 const q = STREAM ? __builtin_nontemporal_load(src) : *src;
         if constexpr (kOddPitch) {
 #pragma unroll
           for (int e = 0; e < V; e++) tile[(row + k) * S + piece * V + e] = (E)q[e];
@@ -360,8 +364,11 @@ static hipError_t permute_typed(hipStream_t st, void const *in, void *out, int n
   for (int i = 0; i < t.n_outer; i++) {
     wide_tiles = wide_tiles && t.outer_in_stride[i] % VE == 0 && t.outer_out_stride[i] % VE == 0;
   }
-  if (wide_tiles) {
-    permute_tiles_wide_kernel<E, MODE><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), kShapeThreads, 0, st>>>(
+  if (wide_tiles && MODE == kStore && stream_past_caches(total, sizeof(E))) {
+    permute_tiles_wide_kernel<E, MODE, true><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), kShapeThreads, 0, st>>>(
+        static_cast<E const *>(in), static_cast<E *>(out), t);
+  } else if (wide_tiles) {
+    permute_tiles_wide_kernel<E, MODE, false><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), kShapeThreads, 0, st>>>(
         static_cast<E const *>(in), static_cast<E *>(out), t);
   } else {
     permute_tiles_kernel<E, MODE><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), kShapeThreads, 0, st>>>(
