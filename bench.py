@@ -15,6 +15,12 @@ Prints one JSON line.  Besides the whole-step throughput it reports
                  bf16 MFMA peak;
   device_copy  : a plain device copy's GB/s, measured in the same run, beside
                  the 8 TB/s vendor figure;
+  mfma_loop    : the matrix rate every SIMD sustains issuing bf16 MFMAs back
+                 to back from registers, measured in the same run, beside the
+                 2.5 PFLOP/s vendor figure (roofline.frac_of_measured_mfma_loop
+                 restates the dominant kernel's fraction against it);
+  clock_settle : the untimed steps run before the warm-up steps, until the
+                 shader clock has reached the state it then holds;
   cpu_baseline : the CPU oracle's restatement of the same layer, timed on the
                  host cores on a bounded sample (one sequence of 128 tokens of
                  the same layer), scaled to tokens/s.
@@ -230,6 +236,16 @@ def time_dominant_kernel(ffk, torch, cfg, iters=50, calibration_copy=False):
                 kernel="gemm_bf16_pipe_kernel<256,256,128,128,64,2,1,false,true,0,false> "
                        "(FFN up-projection, M%d N%d K%d, bias)" % (T, F, E),
                 us_per_launch=us)
+
+
+def measure_mfma_loop(ffk, torch):
+    """The library's probe: every SIMD issues bf16 32x32x16 matrix instructions back to back from
+    registers.  What it reaches is the ceiling for a GEMM on this card at the clock it sustains."""
+    out = torch.empty((256 * 256,), device="cuda")
+    flops = ffk.probe_mfma_bf16(2000, out)
+    us = event_timer(ffk)(lambda: ffk.probe_mfma_bf16(2000, out), 20)
+    return {"TFLOP/s": flops / us / 1e6, "vendor_peak_TFLOP/s": MFMA_BF16_PEAK_TFLOPS,
+            "what": "256 CUs x 4 waves, 32000 back-to-back 32x32x16 bf16 MFMAs each on random operands in registers"}
 
 
 def measure_device_copy(ffk, torch):
@@ -507,8 +523,8 @@ def config5(ffk, torch, with_cpu):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
                     help="BASELINE configuration to measure (2 = the headline transformer layer)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -569,7 +585,9 @@ def main():
         "check": check,
         "roofline": roof,
         "device_copy": measure_device_copy(ffk, torch),
+        "mfma_loop": measure_mfma_loop(ffk, torch),
     }
+    out["roofline"]["frac_of_measured_mfma_loop"] = roof["achieved"] / out["mfma_loop"]["TFLOP/s"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(CFG)
     print(json.dumps(out))

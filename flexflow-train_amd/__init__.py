@@ -96,6 +96,7 @@ SIGNATURES = {
     "ffk_event_record": (c_int, [c_p, c_p]),
     "ffk_event_synchronize": (c_int, [c_p]),
     "ffk_event_elapsed_ms": (c_int, [c_p, c_p, ctypes.POINTER(c_f)]),
+    "ffk_probe_mfma_bf16": (c_int, [c_p, c_int, ctypes.c_uint32, c_p, c_sz, ctypes.POINTER(ctypes.c_double)]),
     "ffk_set_option": (c_int, [c_int, c_int]),
     "ffk_get_option": (c_int, [c_int, ctypes.POINTER(c_int)]),
     "ffk_linear_forward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_p, c_i64, c_i64, c_i64]),
@@ -248,6 +249,14 @@ def ptr(t):
 
 def current_stream():
     return _torch().cuda.current_stream().cuda_stream
+
+
+def probe_mfma_bf16(iterations, out, seed=1):
+    """Launches the matrix-rate probe on the current stream; returns the flops of the launch."""
+    flops = ctypes.c_double()
+    check(lib().ffk_probe_mfma_bf16(current_stream(), iterations, seed, ptr(out), out.numel() * out.element_size(),
+                                    ctypes.byref(flops)))
+    return flops.value
 
 
 def linear_forward(x, w, b=None, activation=ACT_NONE, out=None):

@@ -121,6 +121,16 @@ int ffk_event_record(ffk_event_t ev, ffk_stream_t stream);
 int ffk_event_synchronize(ffk_event_t ev);
 int ffk_event_elapsed_ms(ffk_event_t start, ffk_event_t stop, float *ms);
 
+/* Measurement aid; no counterpart in the reference.  One launch in which
+ * every SIMD of the chip issues `iterations` x 16 bf16 32x32x16 matrix
+ * instructions back to back from registers (no memory traffic): timed by the
+ * caller, *flops / time is the matrix rate this card sustains, the ceiling a
+ * GEMM kernel here can approach (the vendor's 2.5 PFLOP/s assumes a clock the
+ * chip does not hold under that load).  out: scratch of at least 256 KiB
+ * (one float per lane, so the work cannot be dropped).                      */
+int ffk_probe_mfma_bf16(ffk_stream_t stream, int iterations, uint32_t seed,
+                        float *out, size_t out_bytes, double *flops);
+
 /* Process-wide switches for tuning runs and tests; no counterpart in the
  * reference.  Each starts from the environment variable of the same name,
  * read once when the library is loaded.

@@ -426,3 +426,18 @@ def test_linear_with_fused_tail_refuses_shapes_without_a_kernel(ffk):
         ffk.linear_backward_dropout_gelu(x, torch.zeros((100, 128), dtype=bt, device="cuda"),
                                          torch.zeros((100, 128), dtype=bt, device="cuda"),
                                          torch.zeros((64, 128), dtype=bt, device="cuda"), 0.1, 1)
+
+
+@pytest.mark.gpu
+def test_matrix_rate_probe_runs_and_counts_its_flops(ffk):
+    """The measurement aid: finite sums out, the flops of the launch as documented, bad arguments refused."""
+    say("probe_mfma_bf16")
+    out = torch.empty((256 * 256,), device="cuda")
+    flops = ffk.probe_mfma_bf16(10, out)
+    torch.cuda.synchronize()
+    assert flops == 256 * 4 * 10 * 16 * 2.0 * 32 * 32 * 16
+    assert bool(torch.isfinite(out).all()) and float(out.abs().max()) > 0
+    rc = ffk.lib().ffk_probe_mfma_bf16(ffk.current_stream(), 10, 1, ffk.ptr(out), 1024, None)
+    assert rc == ffk.ERR_INVALID
+    rc = ffk.lib().ffk_probe_mfma_bf16(ffk.current_stream(), 0, 1, ffk.ptr(out), out.numel() * 4, None)
+    assert rc == ffk.ERR_INVALID
