@@ -174,7 +174,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv2_kernel(AttnBwdParams p) {
     issue_tile(q_begin, 0);
     issue_tile(min(q_begin + C::kTile, last_tile), 1);
   }
-  wait_vmcnt<kLoadsPerTile>();  // tile 0 has landed
+  // Tiles 0 and 1 have landed, and so have the K and V fragments: told to the compiler, which
+  // otherwise waits for those fragments at their uses in every step, where the counter holds the
+  // two tiles in flight.
+  wait_all_vmem_known_to_compiler();
   __syncthreads();
   int cur = 0;
   for (int it = 0; it < ntiles; it++) {

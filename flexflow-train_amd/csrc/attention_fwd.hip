@@ -162,26 +162,35 @@ __global__ __launch_bounds__(256) void attn_fwd_wide_kernel(AttnParams p) {
     k_voff[i] = (unsigned)((slot_row + i * C::kRowsPerLoad) * p.k_ss + k_lc * 8) * 2u;
     v_voff[i] = (unsigned)((slot_row + i * C::kRowsPerLoad) * p.v_ss + v_lc * 8) * 2u;
   }
-  // Load number n of the 2 * kLoads of the tile at kv0 (K's, then V's) into buffer buf.
+  // The 2 * kLoads loads of the tile at kv0 (K's, then V's) into buffer buf.  One wavefront per
+  // SIMD issues one instruction every four cycles whatever its kind, so what surrounds the loads
+  // counts: a tile wholly below Skv (all but the last) takes two descriptors and, per load, the
+  // LDS address, M0 and the load; the row clamp of the last tile sits behind one branch per tile.
   // (Placing the loads one by one between the MFMAs of phases 1 and 2 instead of issuing them
-  // together at the top of the tile was measured 10% slower: the descriptors and the branches
-  // they bring into those phases cost more than the burst.)
-  auto issue_one = [&](int kv0, int buf, int n) __attribute__((always_inline)) {
-    bool const is_k = n < C::kLoads;
-    int const i = is_k ? n : n - C::kLoads;
-    i32x4 const rsrc = is_k ? buffer_resource(kp + (int64_t)kv0 * p.k_ss) : buffer_resource(vp + (int64_t)kv0 * p.v_ss);
-    unsigned const dst = (is_k ? ks_addr : vs_addr) + (unsigned)(buf * C::kTileElems * 2 + (i * 4 + wave) * 1024);
-    unsigned off = is_k ? k_voff[i] : v_voff[i];
+  // together at the top of the tile was measured 10% slower.)
+  auto issue_tile = [&](int kv0, int buf) {
+    i32x4 const k_rsrc = buffer_resource(kp + (int64_t)kv0 * p.k_ss);
+    i32x4 const v_rsrc = buffer_resource(vp + (int64_t)kv0 * p.v_ss);
+    unsigned const k_dst = ks_addr + (unsigned)(buf * C::kTileElems * 2 + wave * 1024);
+    unsigned const v_dst = vs_addr + (unsigned)(buf * C::kTileElems * 2 + wave * 1024);
     if (kv0 + C::kBKV > p.Skv) {  // uniform
       // rows past the last key repeat it (their scores are masked, their probabilities 0)
-      int const r = min(slot_row + i * C::kRowsPerLoad, p.Skv - 1 - kv0);
-      off = is_k ? (unsigned)(r * p.k_ss + k_lc * 8) * 2u : (unsigned)(r * p.v_ss + v_lc * 8) * 2u;
-    }
-    lds_dma16(rsrc, off, 0u, dst);
-  };
-  auto issue_tile = [&](int kv0, int buf) {
 #pragma unroll
-    for (int n = 0; n < 2 * C::kLoads; n++) issue_one(kv0, buf, n);
+      for (int i = 0; i < C::kLoads; i++) {
+        int const r = min(slot_row + i * C::kRowsPerLoad, p.Skv - 1 - kv0);
+        lds_dma16(k_rsrc, (unsigned)(r * p.k_ss + k_lc * 8) * 2u, 0u, k_dst + (unsigned)(i * 4096));
+      }
+#pragma unroll
+      for (int i = 0; i < C::kLoads; i++) {
+        int const r = min(slot_row + i * C::kRowsPerLoad, p.Skv - 1 - kv0);
+        lds_dma16(v_rsrc, (unsigned)(r * p.v_ss + v_lc * 8) * 2u, 0u, v_dst + (unsigned)(i * 4096));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < C::kLoads; i++) lds_dma16(k_rsrc, k_voff[i], 0u, k_dst + (unsigned)(i * 4096));
+#pragma unroll
+      for (int i = 0; i < C::kLoads; i++) lds_dma16(v_rsrc, v_voff[i], 0u, v_dst + (unsigned)(i * 4096));
+    }
   };
 
   f32x16 oacc[2][D / 32];
@@ -228,7 +237,7 @@ __global__ __launch_bounds__(256) void attn_fwd_wide_kernel(AttnParams p) {
     return u.v;
   };
   issue_tile(0, 0);
-  wait_vmcnt<0>();
+  wait_all_vmem_known_to_compiler();  // the Q fragments too: no wait for them inside the loop
   __syncthreads();
   int cur = 0;
   for (int it = 0; it < ntiles; it++) {

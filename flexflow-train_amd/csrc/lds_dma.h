@@ -11,6 +11,14 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// Waits for every vector-memory load of the wave, as an instruction the compiler sees.  The
+// compiler counts only the loads it issued itself; after loads that it issued before a loop
+// (operand fragments fetched once) it repeats its waits for them at their uses in every
+// iteration, where the counter meanwhile holds the loop's direct loads: the wave then waits for
+// the tile it has just asked for.  This wait, placed before the loop, tells it that nothing of
+// its own is pending any more.  (simm16: vmcnt 0, expcnt 7, lgkmcnt 15.)
+__device__ __forceinline__ void wait_all_vmem_known_to_compiler() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 // One direct global->LDS load: lane l's 16 bytes at `g` land at LDS address
 // lds_base + 16 l (M0 carries the wave-uniform base).  Issued as inline
 // assembly on purpose: the compiler then does not know that LDS is being
