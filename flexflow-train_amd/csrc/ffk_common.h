@@ -285,6 +285,25 @@ static inline bool stream_past_caches(int64_t elems, size_t elem_size) {
   return (size_t)elems * elem_size > ((size_t)128 << 20);
 }
 
+// A kernel that uses more than 64 KB of dynamic LDS has to be given leave, once on every device
+// it is launched on (the attribute belongs to the device's copy of the code).  One object per
+// kernel instantiation; ensure() costs a hipGetDevice per launch after the first.  Concurrent
+// first calls may both set the attribute, which is harmless.
+struct LdsOptIn {
+  static constexpr int kMaxDevices = 64;
+  bool done[kMaxDevices] = {};
+  hipError_t ensure(void const *kernel, int bytes) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    bool const tracked = dev >= 0 && dev < kMaxDevices;
+    if (tracked && done[dev]) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && tracked) done[dev] = true;
+    return e;
+  }
+};
+
 static inline bool aligned16(void const *p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }

@@ -940,13 +940,8 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
   auto kern = gemm_bf16_pipe_kernel<BM, BN, WM, WN, BK, STAGES, PF, TA, TB, TAIL>;
   GemmTailArgs const tail = {static_cast<bf16 const *>(ep.tail_in), static_cast<bf16 *>(ep.tail_out),
                              ep.tail_dropout, ep.tail_colsum_partials};
-  static bool configured = false;  // per template instance
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg::kLds);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static LdsOptIn lds;  // per template instance
+  if (hipError_t e = lds.ensure(reinterpret_cast<void const *>(kern), (int)Cfg::kLds); e != hipSuccess) return e;
   int const blocks = (M / BM) * (N / BN);
   if (splits > 1) {
     float *partial = static_cast<float *>(ep.splitk_ws);
@@ -974,13 +969,8 @@ static hipError_t launch_pipe_pair(hipStream_t st, GemmProblem const &p0, GemmPr
   using Cfg = PipeCfg<128, 128, 64, 32, 64, 4>;
   constexpr int NT = Cfg::NW * 64;
   auto kern = gemm_bf16_pipe_kernel<128, 128, 64, 32, 64, 4, 1, TA, TB, 0, true>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg::kLds);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static LdsOptIn lds;
+  if (hipError_t e = lds.ensure(reinterpret_cast<void const *>(kern), (int)Cfg::kLds); e != hipSuccess) return e;
   int const t0 = (int)((p0.M / 128) * (p0.N / 128)), t1 = (int)((p1.M / 128) * (p1.N / 128));
   GemmSecondProblem const second = {static_cast<bf16 const *>(p1.A), static_cast<bf16 const *>(p1.B),
                                     static_cast<bf16 *>(p1.C), (int)p1.M, (int)p1.N, p1.lda, p1.ldb, p1.ldc, t0};
