@@ -32,7 +32,11 @@ HBM_PEAK = 8e12
 MFMA_PEAK = 2.5e15
 
 
-def timeit(fn, iters=20, warm=5, settle=0.1):
+SETTLE_SECONDS = 0.1   # --settle=S on the command line; 0 for counter runs, whose clock does not matter
+
+
+def timeit(fn, iters=20, warm=5, settle=None):
+    settle = SETTLE_SECONDS if settle is None else settle
     # at least `warm` calls and `settle` seconds of untimed load first: the shader clock takes tens
     # of milliseconds of sustained work to reach the state it then holds, and the first launches
     # after an idle spell (building the next case's tensors is one) run 10-20% slow
@@ -340,5 +344,11 @@ GROUPS = dict(gemm=bench_gemm, fused_linear=bench_fused_linear, bandwidth=bench_
 if __name__ == "__main__":
     ffk.lib()
     assert torch.cuda.is_available(), "kernel_bench.py needs a GPU"
-    for name in sys.argv[1:] or list(GROUPS):
+    names = []
+    for a in sys.argv[1:]:
+        if a.startswith("--settle="):
+            SETTLE_SECONDS = float(a.split("=", 1)[1])
+        else:
+            names.append(a)
+    for name in names or list(GROUPS):
         GROUPS[name]()
