@@ -109,6 +109,22 @@ def test_gather_backward_along_the_last_dim(ffk, oracle, rows, in_dim, picks, it
     assert np.array_equal(got.view(np.uint32)[untouched], old.view(np.uint32)[untouched])
 
 
+def test_gather_along_the_last_dim_at_the_benchmarked_size(ffk):
+    """[16384,4096] -> [16384,1024] as kernel_bench.py times it: the forward moves the values torch.gather
+    moves, the backward gives the sums of torch's scatter_add_ (integer-valued gradients: exact in any order)."""
+    say("gather [16384,4096] -> [16384,1024]")
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    src = torch.randn((16384, 4096), device="cuda", generator=gen)
+    idx = torch.randint(0, 4096, (16384, 1024), device="cuda", generator=gen)
+    out = ffk.gather_forward(src, idx.to(torch.int32), 1)
+    assert torch.equal(out, torch.gather(src, 1, idx))
+    dout = torch.randint(-8, 8, (16384, 1024), device="cuda", generator=gen).to(torch.float32)
+    old = torch.randint(-8, 8, (16384, 4096), device="cuda", generator=gen).to(torch.float32)
+    din = old.clone()
+    ffk.gather_backward(dout, idx.to(torch.int32), din, 1)
+    assert torch.equal(din, old.scatter_add(1, idx, dout))
+
+
 @pytest.mark.parametrize("dim", [0, 1, 2])
 @pytest.mark.parametrize("itype", [torch.int32, torch.int64])
 def test_gather_forward_backward(ffk, oracle, dim, itype):
