@@ -1212,6 +1212,86 @@ static void gpu_tests() {
     }
     }
   });
+
+  // Token embedding -> encoder layer -> vocabulary projection -> softmax -> sparse cross entropy:
+  // the shape of the reference's BERT builder (lib/models/src/models/bert/bert.cc) at toy size.
+  // Two instances, one created with one kernel per operator: the planner's fusions must not change
+  // a bit over three steps, and three more steps on the same batch must bring the loss down.
+  run("BERT-shaped graph (embedding, attention, FFN, vocabulary softmax, sparse CE): fused = unfused, loss falls", [&] {
+    int64_t const B = 2, S = 24, E = 64, FF = 256, V = 96, T = B * S;
+    int const H = 2, HD = 64;
+    float const rate = 0.1f, eps = 1e-5f;
+    tensor_guid_t ids, prob;
+    auto build = [&](ComputationGraphBuilder &cgb) {
+      ids = cgb.create_input(shape({B, S}, DataType::INT32), CreateGrad::NO);
+      tensor_guid_t tok = cgb.embedding(ids, (int)V, (int)E, std::nullopt, DataType::BF16);
+      tensor_guid_t attn = cgb.multihead_attention(tok, tok, tok, (int)E, H, HD, HD, rate, false);
+      tensor_guid_t n1 = cgb.layer_norm(cgb.add(attn, tok), {-1}, true, eps);
+      tensor_guid_t ff1 = cgb.dropout(cgb.dense(n1, (int)FF, Activation::GELU, true), rate);
+      tensor_guid_t ff2 = cgb.dropout(cgb.dense(ff1, (int)E, std::nullopt, true), rate);
+      tensor_guid_t n2 = cgb.layer_norm(cgb.add(n1, ff2), {-1}, true, eps);
+      tensor_guid_t logits = cgb.dense(cgb.reshape(n2, {T, E}), (int)V, std::nullopt, true);
+      prob = cgb.softmax(cgb.cast(logits, DataType::FLOAT));
+    };
+    std::vector<int> id_host(T), label_host(T);
+    for (int64_t i = 0; i < T; i++) {
+      id_host[i] = (int)((i * 37 + 11) % V);
+      label_host[i] = (int)((i * 53 + 7) % V);
+    }
+    Allocator cpu = create_local_cpu_memory_allocator();
+    GenericTensorAccessorW hl = cpu.allocate_tensor(shape({T}, DataType::INT32));
+    memcpy(hl.ptr, label_host.data(), label_host.size() * 4);
+    GenericTensorAccessorW LABEL = copy_tensor_accessor_w(hl, gpu);
+    device_id_t dev = make_device_id_t_from_idx(0, DeviceType::GPU);
+    auto loss_of = [&](std::vector<float> const &p) {
+      double l = 0;
+      for (int64_t i = 0; i < T; i++) l -= std::log((double)p[i * V + label_host[i]] + 1e-30);
+      return l / T;
+    };
+    std::vector<std::vector<float>> results[2];
+    std::vector<double> losses;
+    for (int unfused = 0; unfused < 2; unfused++) {
+      ComputationGraphBuilder cgb;
+      build(cgb);
+      if (unfused) ffk_set_option(FFK_OPTION_LAYER_UNFUSED, 1);
+      ComputationGraphInstance inst = create_computation_graph_instance(
+          cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{0.1, 0.9, false, 0.0}},
+          LossConfig{SparseCategoricalCrossEntropyLossAttrs{false}, LABEL, prob}, {}, gpu, ProfilingSettings{0, 0}, handle, dev);
+      if (unfused) ffk_set_option(FFK_OPTION_LAYER_UNFUSED, 0);
+      GenericTensorAccessorW hi = cpu.allocate_tensor(shape({B, S}, DataType::INT32));
+      memcpy(hi.ptr, id_host.data(), id_host.size() * 4);
+      copy_accessor_data_to_l_from_r(inst.get_tensor_accessor(ids), hi);
+      std::vector<tensor_guid_t> ws;
+      unsigned seed = 300;
+      for (size_t t = 0; t < cgb.computation_graph.tensors.size(); t++) {
+        tensor_guid_t g{(int)t};
+        auto const &src = cgb.computation_graph.layers.at(cgb.computation_graph.tensors[t].source.raw);
+        if (!std::holds_alternative<WeightAttrs>(src.attrs.op_attrs)) continue;
+        ws.push_back(g);
+        TensorShape ts = cgb.computation_graph.tensors[t].shape;
+        // one-dimensional weights are biases and LayerNorm parameters: around 1 keeps the scales alive
+        bool const vec = ts.dims.ff_ordered.size() == 1;
+        auto host = random_vec((size_t)get_num_elements(ts.dims), seed++, vec ? 0.5f : -0.2f, vec ? 1.5f : 0.2f);
+        copy_accessor_data_to_l_from_r(inst.get_tensor_accessor(g), device_accessor(gpu, ts, host));
+      }
+      for (int step = 0; step < (unfused ? 3 : 6); step++) {
+        perform_all_passes_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, dev);
+        if (step == 2) {
+          results[unfused].push_back(to_host(inst.get_tensor_accessor(prob)));
+          for (tensor_guid_t w : ws) results[unfused].push_back(to_host(inst.get_tensor_accessor(w)));
+        }
+        if (!unfused) losses.push_back(loss_of(to_host(inst.get_tensor_accessor(prob))));
+      }
+    }
+    CHECK(results[0].size() == results[1].size() && results[0].size() > 10);
+    for (size_t i = 0; i < results[0].size(); i++) {
+      CHECK(contains_non_zero(results[0][i]));
+      CHECK(results[0][i] == results[1][i]);
+    }
+    CHECK(losses.size() == 6 && std::isfinite(losses[5]));
+    CHECK(losses[5] < losses[0]);
+    printf("    loss per step: %.4f %.4f %.4f %.4f %.4f %.4f\n", losses[0], losses[1], losses[2], losses[3], losses[4], losses[5]);
+  });
 }
 
 int main(int argc, char **argv) {
