@@ -239,8 +239,12 @@ __global__ __launch_bounds__(256) void attn_fwd_wide_kernel(AttnParams p) {
   issue_tile(0, 0);
   wait_all_vmem_known_to_compiler();  // the Q fragments too: no wait for them inside the loop
   __syncthreads();
-  int cur = 0;
-  for (int it = 0; it < ntiles; it++) {
+  // One tile.  The buffer index is a compile-time constant (the loop below takes tiles in
+  // pairs), so that it reaches the LDS reads as an immediate offset and not through vector
+  // address arithmetic per fragment: a wave alone on its SIMD pays four cycles for every
+  // instruction it issues.
+  auto tile_step = [&](int it, auto buffer_tag) __attribute__((always_inline)) {
+    constexpr int cur = decltype(buffer_tag)::value;
     int const kv0 = it * C::kBKV;
     bool const more = it + 1 < ntiles;
     // the buffer that tile it-1 was read from is free since the barrier that ended that tile
@@ -355,7 +359,10 @@ __global__ __launch_bounds__(256) void attn_fwd_wide_kernel(AttnParams p) {
     }
     wait_vmcnt<0>();  // this wave's part of the next tile has landed
     __syncthreads();
-    cur ^= 1;
+  };
+  for (int it = 0; it < ntiles; it += 2) {
+    tile_step(it, std::integral_constant<int, 0>{});
+    if (it + 1 < ntiles) tile_step(it + 1, std::integral_constant<int, 1>{});
   }
 
 #pragma unroll
