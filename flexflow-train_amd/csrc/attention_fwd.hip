@@ -68,8 +68,8 @@ struct SoftmaxHalf {
     if constexpr (UNIT < 4) {
 #pragma unroll
       for (int r = 4 * UNIT; r < 4 * UNIT + 4; r++) {
-        float const pair = fmaxf(s[0][r], s[1][r]);
-        mx = (r == 0) ? pair : fmaxf(mx, pair);
+        // the running maximum and both blocks' scores in one three-operand maximum
+        mx = (r == 0) ? fmaxf(s[0][r], s[1][r]) : fmaxf(fmaxf(mx, s[0][r]), s[1][r]);
       }
       here(mx);
     } else if constexpr (UNIT == 4) {
