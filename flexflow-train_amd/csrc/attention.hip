@@ -152,7 +152,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[j][r]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
+      mx = max_across_halves(mx) * p.scale_log2;  // a lane swap, no trip through LDS
       float const m_new = fmaxf(m_run, mx);
       // m_new is finite: key 0 is visible to every query and tile 0 comes first.
       float const alpha = __builtin_amdgcn_exp2f(m_run - m_new);
@@ -170,8 +170,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
         pf[2 * j] = pack8(pv);
         pf[2 * j + 1] = pack8(pv + 8);
       }
-      sum += __shfl_xor(sum, 32, 64);
-      l_run = l_run * alpha + sum;
+      l_run = l_run * alpha + sum;  // this lane's 16 of every 32 keys; the two lane halves meet at the end
       m_run = m_new;
       // Rescale the running output only when some row's maximum moved.
       if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
@@ -198,6 +197,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
     cur ^= 1;
   }
 
+  l_run += __shfl_xor(l_run, 32, 64);
   if (qrow < p.Sq) {
     float const inv = 1.0f / l_run;
     bf16 *op = p.o + (int64_t)b * p.o_bs + (int64_t)qrow * p.o_ss + (int64_t)head * D;

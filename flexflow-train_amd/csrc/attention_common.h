@@ -91,4 +91,13 @@ __device__ __forceinline__ void static_for(F &&f) {
 // MFMAs at the place where its result is first needed).
 __device__ __forceinline__ void pin_here(float &x) { asm volatile("" : "+v"(x)); }
 
+// Maximum of a value over the two lanes l and l ^ 32 (they hold the same query's column).
+__device__ __forceinline__ float max_across_halves(float x) {
+  // swaps the upper 32 lanes of the first operand with the lower 32 of the second: with the same
+  // value in both, one result holds the lower half twice and the other the upper half twice
+  auto const r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+
 }  // namespace ffk

@@ -42,14 +42,6 @@ struct AttnFwdCfg {
   static_assert(D == 64 || D == 128, "swizzles are written for these two");
 };
 
-// Maximum of a value over the two lanes l and l ^ 32 (they hold the same query's column).
-__device__ __forceinline__ float max_across_halves(float x) {
-  // swaps the upper 32 lanes of the first operand with the lower 32 of the second: with the same
-  // value in both, one result holds the lower half twice and the other the upper half twice
-  auto const r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-
 // Online softmax of one half (32 queries x 64 keys: two score blocks, this lane's query column),
 // cut into 16 units of a few vector instructions so that the caller can put one behind each MFMA
 // of the product that runs next to it:
