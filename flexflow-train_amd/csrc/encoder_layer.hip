@@ -259,23 +259,35 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
   }
   int g_f1_rc = FFK_ERR_UNSUPPORTED;
   bool b1_done = false;  // the first Linear's bias gradient already computed
+  // The two FFN weight gradients, [E,F] and [F,E] over the same T rows, are off the path of the
+  // input gradients and each is one 128x128 tile per CU at this layer's sizes: both go out as one
+  // launch behind the first Linear's input gradient (the same kernel and tile each would run on
+  // alone, so the same bits; one launch and one tail fewer).
+  void const *ffn_in = d->pre_layer_norm ? ws + L.h2 : ws + L.x1;
+  GemmProblem const dw2_problem = {E, F, ws + L.g_f2, E, ws + L.act1_drop, F, g->w2, F};
+  GemmProblem const dw1_problem = {F, E, ws + L.g_f1, F, ffn_in, E, g->w1, E};
+  bool const pair_dw = gelu && layer_fusion_enabled() && g->w1 != nullptr && g->w2 != nullptr &&
+                       (E / 128) * (F / 128) >= kNumCU / 2 &&
+                       gemm_pair_supported(dtype, true, false, T, dw2_problem, dw1_problem);
+  bool dw_pending = false;  // both weight gradients still to be computed, as a pair
   if (gelu && layer_fusion_enabled()) {
     // the dropout's and GELU's backward ride on the tile store of the input-gradient GEMM
     // (52.7 us against 37.7 + 18.4 us: the separate kernel moves three tensors, this one adds one read)
     // ... and so do the column sums of what it stores, the first Linear's bias gradient
     if (g->b1 != nullptr) {
       g_f1_rc = linear_backward_dropout_gelu(as_stream(st), dtype, ws + L.g_f2, ws + L.act1_drop, ws + L.f1,
-                                             ws + L.g_f1, w->w2, g->w2, b2_grad, T, F, E, ws + L.lin_ws,
+                                             ws + L.g_f1, w->w2, pair_dw ? nullptr : g->w2, b2_grad, T, F, E, ws + L.lin_ws,
                                              lin_ws_bytes, wacc, p, d->seed + 1, 0, g->b1,
                                              reinterpret_cast<float *>(ws + L.lin_ws_b), (wacc & FFK_ACC_BIAS) != 0);
       b1_done = g_f1_rc == FFK_OK;
     }
     if (g_f1_rc == FFK_ERR_UNSUPPORTED) {
       g_f1_rc = linear_backward_dropout_gelu(as_stream(st), dtype, ws + L.g_f2, ws + L.act1_drop, ws + L.f1,
-                                             ws + L.g_f1, w->w2, g->w2, b2_grad, T, F, E, ws + L.lin_ws,
+                                             ws + L.g_f1, w->w2, pair_dw ? nullptr : g->w2, b2_grad, T, F, E, ws + L.lin_ws,
                                              lin_ws_bytes, wacc, p, d->seed + 1, 0);
     }
     if (g_f1_rc != FFK_OK && g_f1_rc != FFK_ERR_UNSUPPORTED) return g_f1_rc;
+    dw_pending = pair_dw && g_f1_rc == FFK_OK;  // refused: nothing was launched, the separate operators follow
   }
   bool const g_f1_ready = g_f1_rc == FFK_OK;
   if (!g_f1_ready) {
@@ -283,7 +295,6 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
                                 ws + L.g_act1_drop, w->w2, g->w2, b2_grad, T, F, E, ws + L.lin_ws, lin_ws_bytes,
                                 wacc));
   }
-  void const *ffn_in = d->pre_layer_norm ? ws + L.h2 : ws + L.x1;
   bool const fuse_gelu_bwd = g_f1_ready || (gelu && layer_fusion_enabled() &&
                              dropout_fusable(dtype, ws + L.g_act1_drop, ws + L.f1, ws + L.g_f1, T * F, 0));
   if (g_f1_ready) {
@@ -299,7 +310,12 @@ extern "C" int ffk_encoder_layer_backward(ffk_stream_t st, int dtype,
                                          ws + L.g_f1, T * F, 0));
     }
     FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_NONE, 0, ws + L.f1, ws + L.g_f1, ffn_in, ws + L.g_h2,
-                                w->w1, g->w1, b1_done ? nullptr : g->b1, T, E, F, ws + L.lin_ws_b, lin_ws_bytes, wacc));
+                                w->w1, dw_pending ? nullptr : g->w1, b1_done ? nullptr : g->b1, T, E, F,
+                                ws + L.lin_ws_b, lin_ws_bytes, wacc));
+    if (dw_pending) {
+      FFK_TRY(gemm_dispatch_pair(as_stream(st), dtype, true, false, T, dw2_problem, dw1_problem,
+                                 (wacc & FFK_ACC_WEIGHT) != 0));
+    }
   } else {
     FFK_TRY(ffk_linear_backward(st, dtype, FFK_ACT_RELU, 0, ws + L.act1, ws + L.g_act1, ffn_in, ws + L.g_h2,
                                 w->w1, g->w1, g->b1, T, E, F, ws + L.lin_ws_b, lin_ws_bytes, wacc));
