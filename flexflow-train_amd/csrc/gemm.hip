@@ -1211,6 +1211,12 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
     if (variant == 0 && splits > 1 && ep.splitk_ws != nullptr && aligned16(ep.splitk_ws)) {
       return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep, splits);
     }
+    // No scratch to split the reduction with: from 32 tiles and a reduction of 2048 on, the
+    // pipelined tile on the CUs it reaches is still ahead of the register-staged 64x64 kernel on
+    // four times as many ([1024,1024] over 4096 rows, 64 tiles: 30.5 against 34.5 us).
+    if (variant == 0 && pipe_ok && fits128 && (int64_t)(M / 128) * (N / 128) >= kNumCU / 8 && K >= 2048) {
+      return launch_pipe<128, 128, 64, 32, 64, 4, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+    }
   }
   if (ep.tail != GemmEpilogue::kTailNone) return hipErrorInvalidValue;
   // Largest tile that still gives every CU a workgroup.
