@@ -67,7 +67,7 @@ def test_transpose_moves_any_data_type(ffk, dtype):
 
 @pytest.mark.parametrize("rows,in_dim,picks", [(5, 33, 17), (64, 4096, 1024), (9, 4100, 4100), (3, 20000, 5000), (7, 16384, 2048),
                                                (4, 1000, 100)])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int64])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int64, torch.bool])
 def test_gather_along_the_last_dim(ffk, oracle, rows, in_dim, picks, dtype):
     """Rows picked from densely go through LDS (whole-row staging, vector or element loads), long
     or sparsely picked rows straight from memory: both move values bit for bit."""
@@ -77,7 +77,7 @@ def test_gather_along_the_last_dim(ffk, oracle, rows, in_dim, picks, dtype):
     idx = g.integers(0, in_dim, size=(rows, picks))
     idx.flat[::53] = in_dim                   # out-of-range entries read 0
     idx.flat[::59] = -3
-    xd = to_dev(x, torch).to(dtype)
+    xd = to_dev(x, torch).to(dtype) if dtype != torch.bool else to_dev(x, torch) > 0
     out = ffk.gather_forward(xd, to_dev(idx, torch, torch.int64), 1)
     want = oracle.gather_forward(xd.to(torch.float32).cpu().numpy(), idx, 1)   # values as the type holds them
     assert np.array_equal(out.to(torch.float32).cpu().numpy(), want)
