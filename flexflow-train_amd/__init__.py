@@ -103,6 +103,7 @@ SIGNATURES = {
     "ffk_linear_backward_workspace_bytes": (c_sz, [c_int, c_int, c_int, c_i64, c_i64]),
     "ffk_linear_backward": (c_int, [c_p, c_int, c_int, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
                                     c_i64, c_i64, c_i64, c_p, c_sz, c_int]),
+    "ffk_linear_l2_regularizer_grad": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f]),
     "ffk_gemm": (c_int, [c_p, c_int, c_int, c_int, c_i64, c_i64, c_i64, c_p, c_p, c_p, c_int]),
     "ffk_element_unary_forward": (c_int, [c_p, c_int, c_int, c_f, c_p, c_p, c_i64]),
     "ffk_element_unary_backward": (c_int, [c_p, c_int, c_int, c_f, c_p, c_p, c_p, c_p, c_i64,
@@ -286,6 +287,12 @@ def linear_backward(y, dy, x, w, dx=None, dw=None, db=None, activation=ACT_NONE,
                                     batch, in_dim, out_dim, ptr(workspace), ws_bytes,
                                     7 if accumulate is True else int(accumulate)))
     return dx, dw, db
+
+
+def linear_l2_regularizer_grad(w, dw, lam):
+    """dw = dw + lam * w in place (the L2 regulariser's term of Linear's weight gradient)."""
+    check(lib().ffk_linear_l2_regularizer_grad(current_stream(), dtype_of(w), ptr(w), ptr(dw), w.numel(), lam))
+    return dw
 
 
 def linear_gelu_dropout_forward(x, w, b, rate, seed, offset=0):
@@ -681,6 +688,10 @@ def mha_desc(num_samples, num_heads, q_size, k_size, v_size, q_proj, k_proj, v_p
              sq, skv, scale=1.0, causal=False):
     return MHADesc(num_samples, num_heads, q_size, k_size, v_size, q_proj, k_proj, v_proj, o_proj,
                    sq, skv, scale, int(causal))
+
+
+# bits of ffk_mha_backward's `accumulate`
+MHA_ACC_INPUT_GRADS, MHA_OVERWRITE_WEIGHT_GRAD = 1, 2
 
 
 def mha_reserve(desc, dtype, device="cuda"):

@@ -55,6 +55,26 @@ static hipError_t act_grad(hipStream_t st, int act, int mode, void const *y,
 
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// in = (weight, weight_grad); out = weight_grad + lambda * weight
+struct L2RegGrad {
+  float lambda;
+  __device__ __forceinline__ void operator()(float const (&in)[2], float (&out)[1]) const {
+    out[0] = in[1] + lambda * in[0];
+  }
+};
+
+template <typename T>
+static hipError_t l2_reg_grad(hipStream_t st, void const *w, void *dw, int64_t n, float lambda) {
+  EwArgs<T, 2, 1> a;
+  a.in[0] = static_cast<T const *>(w);
+  a.in[1] = static_cast<T const *>(dw);
+  a.in_elems[0] = n;
+  a.in_elems[1] = n;
+  a.out[0] = static_cast<T *>(dw);
+  a.n = n;
+  return ew_launch<T, 2, 1>(st, a, L2RegGrad{lambda});
+}
+
 }  // namespace ffk
 
 using namespace ffk;
@@ -169,6 +189,17 @@ extern "C" int ffk_linear_backward(
   return linear_backward_impl(stream, dtype, activation, relu_grad_mode, output, output_grad, input,
                               input_grad, weight, weight_grad, bias_grad, batch, in_dim, out_dim,
                               workspace, workspace_bytes, accumulate, nullptr);
+}
+
+extern "C" int ffk_linear_l2_regularizer_grad(ffk_stream_t stream, int dtype, void const *weight,
+                                              void *weight_grad, int64_t elems, float lambda) {
+  FFK_REQUIRE(dtype == FFK_FLOAT || dtype == FFK_BF16, "linear_l2_regularizer_grad: dtype %d not supported", dtype);
+  FFK_REQUIRE(weight && weight_grad, "linear_l2_regularizer_grad: NULL tensor");
+  FFK_REQUIRE(elems > 0, "linear_l2_regularizer_grad: non-positive element count");
+  hipStream_t st = as_stream(stream);
+  FFK_HIP(dtype == FFK_FLOAT ? l2_reg_grad<float>(st, weight, weight_grad, elems, lambda)
+                             : l2_reg_grad<bf16>(st, weight, weight_grad, elems, lambda));
+  return FFK_OK;
 }
 
 namespace ffk {

@@ -38,6 +38,20 @@ inline int64_t get_num_elements(TensorDims const &d) {
   for (int64_t v : d.ff_ordered) n *= v;
   return n;
 }
+// True when `operand` lines up with the trailing dims of `out` once its leading
+// 1s are dropped: the only broadcast the element-wise kernels implement (the
+// smaller operand repeats every get_num_elements(operand) elements).  A size-1
+// dim in the middle or at the end of the operand is a different pattern.
+inline bool broadcasts_over_leading_dims(TensorDims const &operand, TensorDims const &out) {
+  size_t first = 0;
+  while (first < operand.ff_ordered.size() && operand.ff_ordered[first] == 1) first++;
+  size_t const n = operand.ff_ordered.size() - first, m = out.ff_ordered.size();
+  if (n > m) return false;
+  for (size_t i = 0; i < n; i++) {
+    if (operand.ff_ordered[first + i] != out.ff_ordered[m - n + i]) return false;
+  }
+  return true;
+}
 inline int64_t get_size_in_bytes(TensorShape const &s) {
   return get_num_elements(s.dims) * (int64_t)size_of_datatype(s.data_type);
 }

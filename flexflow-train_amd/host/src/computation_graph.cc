@@ -98,6 +98,10 @@ std::vector<TensorShape> get_output_shapes(ComputationGraphOpAttrs const &attrs,
     TensorShape const &big = nl >= nr ? in[0] : in[1];
     int64_t small = nl >= nr ? nr : nl;
     if (get_num_elements(big.dims) % small != 0) bad("element binary: operand does not broadcast over trailing dims");
+    TensorShape const &little = nl >= nr ? in[1] : in[0];
+    if (!broadcasts_over_leading_dims(little.dims, big.dims)) {
+      bad("element binary: broadcast pattern not supported (the smaller operand must equal the output's trailing dims)");
+    }
     return {big};
   }
   if (auto const *a = std::get_if<SoftmaxAttrs>(&attrs)) {

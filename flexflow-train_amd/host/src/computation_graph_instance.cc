@@ -794,6 +794,20 @@ ComputationGraphInstance create_computation_graph_instance(
                     "Dropout + GELU backward");
         };
       }
+      if (a->regularizer.has_value()) {
+        // the regulariser's term behind the weight-gradient product of every backward call
+        // (lib/kernels/src/cuda/ops/linear_kernels.cu:269-290)
+        auto const *l2 = std::get_if<L2RegularizerAttrs>(&*a->regularizer);
+        if (l2 == nullptr) throw std::runtime_error("Linear: Only L2 regularization is supported");
+        float const lambda = l2->lambda;
+        int64_t const w_elems = numel(layer.weights[0]);
+        int const w_type = dt(shape_of(layer.weights[0]).data_type);
+        auto const inner = b;
+        b = [=](device_stream_t const &s) {
+          inner(s);
+          check_ffk(ffk_linear_l2_regularizer_grad(s.require_gpu(), w_type, w, dw, w_elems, lambda), "Linear L2 regularizer");
+        };
+      }
     } else if (auto const *a = std::get_if<LayerNormAttrs>(&oa)) {
       tensor_guid_t x = layer.inputs[0];
       int const type = dt(shape_of(x).data_type);

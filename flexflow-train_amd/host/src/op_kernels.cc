@@ -35,6 +35,11 @@ std::optional<LinearPerDeviceState> linear_init_kernel(
     std::optional<RegularizerAttrs> regularizer, bool use_bias, DataType input_type,
     DataType weight_type, DataType output_type, int batch_size, int output_num_channels) {
   if (device_type != DeviceType::GPU) return std::nullopt;
+  // the reference asserts "Only L2 regularization is supported" in its backward
+  // (src/cuda/ops/linear_kernels.cu:286-288); here the state is refused up front
+  if (regularizer.has_value() && !std::holds_alternative<L2RegularizerAttrs>(*regularizer)) {
+    throw std::runtime_error("linear_init_kernel: Only L2 regularization is supported");
+  }
   LinearPerDeviceState s;
   s.handle = handle.require_for_gpu();
   // ReLU sizes the scratch for any activation (same bytes for all of them)
@@ -85,6 +90,15 @@ void linear_backward_kernel(device_stream_t const &stream, std::optional<LinearP
                                 projection_grad.ptr, bias_grad ? bias_grad->ptr : nullptr, batch, in_dim, out_dim,
                                 state->workspace, state->workspace_bytes, FFK_ACC_ALL),
             "linear_backward_kernel");
+  // the regulariser's term, once per call behind the weight-gradient product
+  // (src/cuda/ops/linear_kernels.cu:269-290)
+  if (state->regularizer.has_value()) {
+    auto const *l2 = std::get_if<L2RegularizerAttrs>(&*state->regularizer);
+    if (l2 == nullptr) throw std::runtime_error("linear_backward_kernel: Only L2 regularization is supported");
+    check_ffk(ffk_linear_l2_regularizer_grad(stream.require_gpu(), dt(projection.shape.data_type), projection.ptr,
+                                             projection_grad.ptr, get_num_elements(projection.shape.dims), l2->lambda),
+              "linear_backward_kernel (L2 regularizer)");
+  }
 }
 
 void linear_cleanup_kernel(DeviceType device_type, std::optional<LinearPerDeviceState> &state) {
@@ -387,6 +401,13 @@ std::optional<ElementBinaryPerDeviceState> init_kernel(DeviceType device_type, d
                                                        TensorShape const &lhs, TensorShape const &rhs,
                                                        TensorShape const &out) {
   if (device_type != DeviceType::GPU) return std::nullopt;
+  // The reference reduces through tensor descriptors built from the shapes, so any
+  // size-1 dim of an operand is summed over (src/cuda/ops/element_binary_kernels.cu:85-130,
+  // 268-396); the kernels here repeat the smaller operand over the leading dims only.
+  if (!broadcasts_over_leading_dims(lhs.dims, out.dims) || !broadcasts_over_leading_dims(rhs.dims, out.dims)) {
+    throw std::runtime_error("ElementBinary::init_kernel: broadcast pattern not supported (an operand must equal "
+                             "the output's trailing dims after its leading 1s are dropped)");
+  }
   return ElementBinaryPerDeviceState{handle.require_for_gpu(), op_type, bl, br, lhs, rhs, out};
 }
 void forward_kernel(device_stream_t const &stream, std::optional<ElementBinaryPerDeviceState> const &state,
@@ -422,6 +443,10 @@ void forward_kernel(device_stream_t const &stream, std::optional<ElementBinaryPe
                     GenericTensorAccessorR const &lhs, GenericTensorAccessorR const &rhs,
                     GenericTensorAccessorW const &out) {
   if (!stream.is_gpu()) no_cpu("ElementBinary::forward_kernel");
+  if (!broadcasts_over_leading_dims(lhs.shape.dims, out.shape.dims) ||
+      !broadcasts_over_leading_dims(rhs.shape.dims, out.shape.dims)) {
+    throw std::runtime_error("ElementBinary::forward_kernel: broadcast pattern not supported");
+  }
   check_ffk(ffk_element_binary_forward(stream.require_gpu(), dt(out.shape.data_type),
                                        static_cast<int>(state.value().op_type), lhs.ptr, rhs.ptr, out.ptr,
                                        get_num_elements(out.shape.dims), get_num_elements(lhs.shape.dims),

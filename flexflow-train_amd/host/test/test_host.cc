@@ -294,6 +294,35 @@ static void gpu_tests() {
     linear_cleanup_kernel(DeviceType::GPU, state);
   });
 
+  run("linear backward with an L2 regularizer (reference KAT + lambda W), L1 refused", [&] {
+    std::vector<float> x = {3, 3, 6, 2, 1, 5, 1, 2, -2, 8, 0.5, -3}, w = {1, 2, 1.5, 0.5, 4, -1};
+    std::vector<float> dy = {1, -0.5, 2, -2, 1, 9, -3.5, 1};
+    float const lambda = 0.5f;
+    std::optional<RegularizerAttrs> reg = RegularizerAttrs{L2RegularizerAttrs{lambda}};
+    LinearAttrs attrs{2, false, DataType::FLOAT, std::nullopt, reg};
+    auto state = linear_init_kernel(DeviceType::GPU, handle, std::nullopt, reg, false, DataType::FLOAT, DataType::FLOAT,
+                                    DataType::FLOAT, 4, 2);
+    auto X = device_accessor(gpu, shape({4, 3}, DataType::FLOAT), x);
+    auto W = device_accessor(gpu, shape({2, 3}, DataType::FLOAT), w);
+    auto DY = device_accessor(gpu, shape({4, 2}, DataType::FLOAT), dy);
+    auto Y = gpu.allocate_tensor(shape({4, 2}, DataType::FLOAT));
+    auto DX = gpu.allocate_tensor(X.shape), DW = gpu.allocate_tensor(W.shape);
+    fill_with_zeros(DX); fill_with_zeros(DW);
+    linear_forward_kernel(stream, state, attrs, X, Y, W, std::nullopt);
+    linear_backward_kernel(stream, state, attrs, Y, DY, X, DX, W, DW, std::nullopt);
+    // the known-answer weight gradient {-20, 5.25, 24.5, 11.5, 15, -34} plus 0.5 W
+    CHECK(to_host(DW) == (std::vector<float>{-19.5, 6.25, 25.25, 11.75, 17, -34.5}));
+    std::vector<float> want = {-20, 5.25, 24.5, 11.5, 15, -34};
+    orc_linear_l2_regularizer_grad(w.data(), want.data(), 6, lambda);
+    CHECK(to_host(DW) == want);
+    // second call: (dW + g^T x) + lambda W again
+    linear_backward_kernel(stream, state, attrs, Y, DY, X, DX, W, DW, std::nullopt);
+    CHECK(to_host(DW) == (std::vector<float>{-39, 12.5, 50.5, 23.5, 34, -69}));
+    linear_cleanup_kernel(DeviceType::GPU, state);
+    CHECK_THROWS(linear_init_kernel(DeviceType::GPU, handle, std::nullopt, RegularizerAttrs{L1RegularizerAttrs{0.1f}}, false,
+                                    DataType::FLOAT, DataType::FLOAT, DataType::FLOAT, 4, 2));
+  });
+
   run("LayerNorm forward/backward vs oracle", [&] {
     int64_t M = 37, N = 96;
     auto x = random_vec(M * N, 5, -2, 2), g = random_vec(N, 6, 0.5f, 1.5f), b = random_vec(N, 7), dy = random_vec(M * N, 8);
@@ -416,6 +445,22 @@ static void gpu_tests() {
                                               nullptr, DB.get_float_ptr(), op, false, true, handle);
       for (auto &v : dr) v *= 2.0f;
       CHECK(close(to_host(DB), dr, 1e-5));
+    }
+    // leading 1s are the same pattern; a size-1 dim in the middle or at the end is another one
+    // (the kernels would repeat the operand over the wrong elements) and is refused
+    TensorShape out3 = shape({4, 5, 6}, DataType::FLOAT);
+    CHECK(Kernels::ElementBinary::init_kernel(DeviceType::GPU, handle, OperatorType::EW_ADD, false, true, out3,
+                                              shape({1, 1, 6}, DataType::FLOAT), out3).has_value());
+    CHECK(Kernels::ElementBinary::init_kernel(DeviceType::GPU, handle, OperatorType::EW_ADD, false, true, out3,
+                                              shape({5, 6}, DataType::FLOAT), out3).has_value());
+    CHECK_THROWS(Kernels::ElementBinary::init_kernel(DeviceType::GPU, handle, OperatorType::EW_ADD, true, false,
+                                                     shape({4, 1, 6}, DataType::FLOAT), out3, out3));
+    CHECK_THROWS(Kernels::ElementBinary::init_kernel(DeviceType::GPU, handle, OperatorType::EW_MUL, false, true, out3,
+                                                     shape({4, 5, 1}, DataType::FLOAT), out3));
+    {
+      ComputationGraphBuilder bld;
+      tensor_guid_t a = bld.create_input(out3, CreateGrad::YES), c = bld.create_input(shape({4, 1, 6}, DataType::FLOAT), CreateGrad::YES);
+      CHECK_THROWS(bld.add(a, c));
     }
   });
 

@@ -195,6 +195,17 @@ int ffk_linear_backward(ffk_stream_t stream, int dtype, int activation,
                         int64_t out_dim, void *workspace,
                         size_t workspace_bytes, int accumulate);
 
+/* The L2 regulariser's term of Linear's weight gradient: weight_grad = 1 *
+ * weight_grad + lambda * weight over `elems` elements, what the reference does
+ * with one cublasSgeam behind the weight-gradient GEMM of every backward call
+ * (lib/kernels/src/cuda/ops/linear_kernels.cu:269-290).  FLOAT or BF16 (fp32
+ * arithmetic, one rounding at the store).  The reference asserts on any other
+ * regulariser (L1); callers do the same.                                      */
+int ffk_linear_l2_regularizer_grad(ffk_stream_t stream, int dtype,
+                                   void const *weight, void *weight_grad,
+                                   int64_t elems, float lambda);
+
+
 /* General GEMM behind Linear and the attention projections:
  *   C[M,N] (+)= op(A) . op(B)   with fp32 accumulation.
  *   trans_a == 0: A is [M,K] row-major; 1: A is [K,M] row-major.

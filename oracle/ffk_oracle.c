@@ -19,6 +19,11 @@
  *      (source text only -- no reference test runs an activation through the
  *      kernel: PARITY UNPINNED by the reference's tests); mode 0 =
  *      cuda_helper.cu:60-64, pinned by finite differences.
+ *  orc_linear_l2_regularizer_grad   src/cuda/ops/linear_kernels.cu:269-290
+ *      (dW = 1 dW + lambda W once per backward call); no reference test runs a
+ *      regulariser (PARITY UNPINNED there); pinned by the closed form: it is
+ *      the gradient of lambda/2 |W|^2, checked by finite differences, and
+ *      with a zero output gradient a Linear backward leaves exactly lambda W.
  *  orc_element_unary_*        src/cuda/ops/element_unary_kernels.cu:104-250
  *      the reference has no test for this op (PARITY UNPINNED there); pinned
  *      here by closed forms / libm and finite differences.
@@ -84,6 +89,9 @@
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 
 /* OperatorType ordinals (lib/op-attrs/include/op-attrs/operator_type.dtg.toml:12-94) */
 enum {
@@ -96,6 +104,24 @@ enum {
 };
 
 /* ------------------------------------------------------------------ helpers */
+
+/* Threads for the loops marked parallel (matrix products by row, attention by
+ * (batch, head)); 1 = the reference's single-threaded CPU evaluation.  Results
+ * are the same bits for any count. */
+void orc_set_num_threads(int n) {
+#ifdef _OPENMP
+  omp_set_num_threads(n > 0 ? n : 1);
+#else
+  (void)n;
+#endif
+}
+int orc_get_max_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
 
 float orc_round_bf16(float x) {
   uint32_t u;
@@ -135,6 +161,8 @@ int64_t orc_offset(int64_t const *dims, int rank, int64_t const *coord) {
 /* tensor_accessor_binary_ops.cc:126-138 */
 void orc_matmul(float const *lhs, float const *rhs, float *out, int64_t M,
                 int64_t K, int64_t N) {
+  /* rows are independent: threads change who computes an element, not how */
+#pragma omp parallel for schedule(static) if (M * N * K > 1000000)
   for (int64_t i = 0; i < M; i++) {
     for (int64_t j = 0; j < N; j++) {
       float accum = 0.0f;
@@ -323,8 +351,17 @@ int orc_linear_backward(int activation, int relu_grad_mode,
   return 0;
 }
 
+/* linear_kernels.cu:269-290: cublasSgeam(alpha = 1, dW, beta = lambda, W) -> dW */
+void orc_linear_l2_regularizer_grad(float const *weight, float *weight_grad,
+                                    int64_t n, float lambda) {
+  for (int64_t i = 0; i < n; i++) {
+    weight_grad[i] = 1.0f * weight_grad[i] + lambda * weight[i];
+  }
+}
+
 void orc_gemm_f64(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K,
                   float const *A, float const *B, float *C) {
+#pragma omp parallel for schedule(static) if (M * N * K > 1000000)
   for (int64_t i = 0; i < M; i++) {
     for (int64_t j = 0; j < N; j++) {
       double acc = 0.0;
@@ -760,119 +797,131 @@ int orc_embedding_backward_f64(int64_t const *idx, float const *g, float *dw,
 
 #define QI(b, s, h, d, S, H, D) ((((b) * (S) + (s)) * (H) + (h)) * (D) + (d))
 
+/* q, k: [B, S, H, D]; v, o: [B, S, H, Dv] (the value head size may differ from
+ * the query/key head size: vProjSize vs qProjSize in attention_kernels.cu:78-80).
+ * Every (batch, head) pair is independent and is computed by one thread in a
+ * fixed order, so the result does not depend on the thread count. */
 void orc_attention_forward(float const *q, float const *k, float const *v,
                            float *o, float *lse, int64_t B, int64_t H,
-                           int64_t Sq, int64_t Skv, int64_t D, float scale,
-                           int causal, int bf16_mode) {
-  double *p = (double *)malloc(sizeof(double) * (size_t)(Skv + 1));
-  for (int64_t b = 0; b < B; b++) {
-    for (int64_t h = 0; h < H; h++) {
-      for (int64_t i = 0; i < Sq; i++) {
-        int64_t lim = causal ? (i + 1 < Skv ? i + 1 : Skv) : Skv;
-        double mx = -INFINITY;
-        for (int64_t j = 0; j < lim; j++) {
-          double s = 0.0;
-          for (int64_t d = 0; d < D; d++) {
-            s += (double)q[QI(b, i, h, d, Sq, H, D)] *
-                 (double)k[QI(b, j, h, d, Skv, H, D)];
-          }
-          s *= (double)scale;
-          p[j] = s;
-          if (s > mx) {
-            mx = s;
-          }
-        }
-        double sum = 0.0;
-        for (int64_t j = 0; j < lim; j++) {
-          p[j] = exp(p[j] - mx);
-          sum += p[j];
-        }
-        if (lse) {
-          lse[(b * H + h) * Sq + i] = (float)(mx + log(sum));
-        }
+                           int64_t Sq, int64_t Skv, int64_t D, int64_t Dv,
+                           float scale, int causal, int bf16_mode) {
+#pragma omp parallel for schedule(dynamic) if (B * H * Sq * Skv > 100000)
+  for (int64_t bh = 0; bh < B * H; bh++) {
+    int64_t const b = bh / H, h = bh % H;
+    double *p = (double *)malloc(sizeof(double) * (size_t)(Skv + 1));
+    for (int64_t i = 0; i < Sq; i++) {
+      int64_t lim = causal ? (i + 1 < Skv ? i + 1 : Skv) : Skv;
+      double mx = -INFINITY;
+      for (int64_t j = 0; j < lim; j++) {
+        double s = 0.0;
         for (int64_t d = 0; d < D; d++) {
-          double acc = 0.0;
-          for (int64_t j = 0; j < lim; j++) {
-            double pj = p[j];
-            if (bf16_mode) {
-              /* the device rounds the unnormalised probabilities to bf16
-               * before the PV product and divides by the fp32 row sum after */
-              pj = (double)orc_round_bf16((float)pj);
-            }
-            acc += pj * (double)v[QI(b, j, h, d, Skv, H, D)];
-          }
-          float r = (float)(acc / sum);
-          o[QI(b, i, h, d, Sq, H, D)] = bf16_mode ? orc_round_bf16(r) : r;
+          s += (double)q[QI(b, i, h, d, Sq, H, D)] *
+               (double)k[QI(b, j, h, d, Skv, H, D)];
+        }
+        s *= (double)scale;
+        p[j] = s;
+        if (s > mx) {
+          mx = s;
         }
       }
+      double sum = 0.0;
+      for (int64_t j = 0; j < lim; j++) {
+        p[j] = exp(p[j] - mx);
+        sum += p[j];
+      }
+      if (lse) {
+        lse[(b * H + h) * Sq + i] = (float)(mx + log(sum));
+      }
+      if (bf16_mode) {
+        /* the device rounds the unnormalised probabilities to bf16 before
+         * the PV product and divides by the fp32 row sum after */
+        for (int64_t j = 0; j < lim; j++) {
+          p[j] = (double)orc_round_bf16((float)p[j]);
+        }
+      }
+      for (int64_t d = 0; d < Dv; d++) {
+        double acc = 0.0;
+        for (int64_t j = 0; j < lim; j++) {
+          acc += p[j] * (double)v[QI(b, j, h, d, Skv, H, Dv)];
+        }
+        float r = (float)(acc / sum);
+        o[QI(b, i, h, d, Sq, H, Dv)] = bf16_mode ? orc_round_bf16(r) : r;
+      }
     }
+    free(p);
   }
-  free(p);
 }
 
 void orc_attention_backward(float const *q, float const *k, float const *v,
                             float const *d_o, float *dq, float *dk, float *dv,
                             int64_t B, int64_t H, int64_t Sq, int64_t Skv,
-                            int64_t D, float scale, int causal) {
-  double *p = (double *)malloc(sizeof(double) * (size_t)(Skv + 1));
-  double *dp = (double *)malloc(sizeof(double) * (size_t)(Skv + 1));
+                            int64_t D, int64_t Dv, float scale, int causal) {
   double *dqa = (double *)calloc((size_t)(B * Sq * H * D) + 1, sizeof(double));
   double *dka = (double *)calloc((size_t)(B * Skv * H * D) + 1, sizeof(double));
-  double *dva = (double *)calloc((size_t)(B * Skv * H * D) + 1, sizeof(double));
-  for (int64_t b = 0; b < B; b++) {
-    for (int64_t h = 0; h < H; h++) {
-      for (int64_t i = 0; i < Sq; i++) {
-        int64_t lim = causal ? (i + 1 < Skv ? i + 1 : Skv) : Skv;
-        double mx = -INFINITY;
-        for (int64_t j = 0; j < lim; j++) {
-          double s = 0.0;
-          for (int64_t d = 0; d < D; d++) {
-            s += (double)q[QI(b, i, h, d, Sq, H, D)] *
-                 (double)k[QI(b, j, h, d, Skv, H, D)];
-          }
-          p[j] = s * (double)scale;
-          if (p[j] > mx) {
-            mx = p[j];
-          }
+  double *dva = (double *)calloc((size_t)(B * Skv * H * Dv) + 1, sizeof(double));
+  /* a (batch, head) pair touches only its own slices of the accumulators */
+#pragma omp parallel for schedule(dynamic) if (B * H * Sq * Skv > 100000)
+  for (int64_t bh = 0; bh < B * H; bh++) {
+    int64_t const b = bh / H, h = bh % H;
+    double *p = (double *)malloc(sizeof(double) * (size_t)(Skv + 1));
+    double *dp = (double *)malloc(sizeof(double) * (size_t)(Skv + 1));
+    for (int64_t i = 0; i < Sq; i++) {
+      int64_t lim = causal ? (i + 1 < Skv ? i + 1 : Skv) : Skv;
+      double mx = -INFINITY;
+      for (int64_t j = 0; j < lim; j++) {
+        double s = 0.0;
+        for (int64_t d = 0; d < D; d++) {
+          s += (double)q[QI(b, i, h, d, Sq, H, D)] *
+               (double)k[QI(b, j, h, d, Skv, H, D)];
         }
-        double sum = 0.0;
-        for (int64_t j = 0; j < lim; j++) {
-          p[j] = exp(p[j] - mx);
-          sum += p[j];
+        p[j] = s * (double)scale;
+        if (p[j] > mx) {
+          mx = p[j];
         }
-        double dot = 0.0; /* sum_j P_ij dP_ij */
-        for (int64_t j = 0; j < lim; j++) {
-          p[j] /= sum;
-          double t = 0.0;
-          for (int64_t d = 0; d < D; d++) {
-            t += (double)d_o[QI(b, i, h, d, Sq, H, D)] *
-                 (double)v[QI(b, j, h, d, Skv, H, D)];
-          }
-          dp[j] = t;
-          dot += p[j] * t;
+      }
+      double sum = 0.0;
+      for (int64_t j = 0; j < lim; j++) {
+        p[j] = exp(p[j] - mx);
+        sum += p[j];
+      }
+      double dot = 0.0; /* sum_j P_ij dP_ij */
+      for (int64_t j = 0; j < lim; j++) {
+        p[j] /= sum;
+        double t = 0.0;
+        for (int64_t d = 0; d < Dv; d++) {
+          t += (double)d_o[QI(b, i, h, d, Sq, H, Dv)] *
+               (double)v[QI(b, j, h, d, Skv, H, Dv)];
         }
-        for (int64_t j = 0; j < lim; j++) {
-          double ds = p[j] * (dp[j] - dot) * (double)scale;
-          for (int64_t d = 0; d < D; d++) {
-            dqa[QI(b, i, h, d, Sq, H, D)] +=
-                ds * (double)k[QI(b, j, h, d, Skv, H, D)];
-            dka[QI(b, j, h, d, Skv, H, D)] +=
-                ds * (double)q[QI(b, i, h, d, Sq, H, D)];
-            dva[QI(b, j, h, d, Skv, H, D)] +=
-                p[j] * (double)d_o[QI(b, i, h, d, Sq, H, D)];
-          }
+        dp[j] = t;
+        dot += p[j] * t;
+      }
+      for (int64_t j = 0; j < lim; j++) {
+        double ds = p[j] * (dp[j] - dot) * (double)scale;
+        for (int64_t d = 0; d < D; d++) {
+          dqa[QI(b, i, h, d, Sq, H, D)] +=
+              ds * (double)k[QI(b, j, h, d, Skv, H, D)];
+          dka[QI(b, j, h, d, Skv, H, D)] +=
+              ds * (double)q[QI(b, i, h, d, Sq, H, D)];
+        }
+        for (int64_t d = 0; d < Dv; d++) {
+          dva[QI(b, j, h, d, Skv, H, Dv)] +=
+              p[j] * (double)d_o[QI(b, i, h, d, Sq, H, Dv)];
         }
       }
     }
+    free(p);
+    free(dp);
   }
   for (int64_t i = 0; i < B * Sq * H * D; i++) {
     dq[i] = (float)dqa[i];
   }
   for (int64_t i = 0; i < B * Skv * H * D; i++) {
     dk[i] = (float)dka[i];
+  }
+  for (int64_t i = 0; i < B * Skv * H * Dv; i++) {
     dv[i] = (float)dva[i];
   }
-  free(p); free(dp); free(dqa); free(dka); free(dva);
+  free(dqa); free(dka); free(dva);
 }
 
 /* ------------------------------------------------------- MultiHeadAttention */
@@ -906,8 +955,9 @@ void orc_mha_forward(orc_mha_desc_t const *d, float const *query,
   maybe_round(Q, B * Sq * H * Dq, bf16_mode);
   maybe_round(K, B * Skv * H * Dk, bf16_mode);
   maybe_round(V, B * Skv * H * Dv, bf16_mode);
-  /* the core assumes one head_dim; the reference asserts kProj == qProj */
-  orc_attention_forward(Q, K, V, C, NULL, B, H, Sq, Skv, Dq, d->scale,
+  /* the reference asserts kProjSize == qProjSize (attention_kernels.cu:61);
+   * the value head size is its own */
+  orc_attention_forward(Q, K, V, C, NULL, B, H, Sq, Skv, Dq, Dv, d->scale,
                         d->causal, bf16_mode);
   orc_gemm_f64(0, 1, B * Sq, d->o_proj_size, H * Dv, C, wo, output);
   maybe_round(output, B * Sq * d->o_proj_size, bf16_mode);
@@ -943,7 +993,7 @@ void orc_mha_backward(orc_mha_desc_t const *d, float const *query,
   maybe_round(Q, TQ * H * Dq, bf16_mode);
   maybe_round(K, TK * H * Dk, bf16_mode);
   maybe_round(V, TK * H * Dv, bf16_mode);
-  orc_attention_forward(Q, K, V, C, NULL, B, H, Sq, Skv, Dq, d->scale,
+  orc_attention_forward(Q, K, V, C, NULL, B, H, Sq, Skv, Dq, Dv, d->scale,
                         d->causal, bf16_mode);
   /* dC = dOut . W_O ; dW_O += dOut^T . C */
   orc_gemm_f64(0, 0, TQ, H * Dv, d->o_proj_size, output_grad, wo, dC);
@@ -954,8 +1004,8 @@ void orc_mha_backward(orc_mha_desc_t const *d, float const *query,
   for (int64_t i = 0; i < no; i++) {
     dweight[nq + nk + nv + i] += tmp[i];
   }
-  orc_attention_backward(Q, K, V, dC, dQ, dK, dV, B, H, Sq, Skv, Dq, d->scale,
-                         d->causal);
+  orc_attention_backward(Q, K, V, dC, dQ, dK, dV, B, H, Sq, Skv, Dq, Dv,
+                         d->scale, d->causal);
   maybe_round(dQ, TQ * H * Dq, bf16_mode);
   maybe_round(dK, TK * H * Dk, bf16_mode);
   maybe_round(dV, TK * H * Dv, bf16_mode);

@@ -21,6 +21,8 @@ extern "C" {
 #endif
 
 /* ---- helpers ---- */
+void orc_set_num_threads(int n);
+int orc_get_max_threads(void);
 float orc_round_bf16(float x);
 void orc_round_bf16_array(float *x, int64_t n);
 int64_t orc_offset(int64_t const *dims, int rank, int64_t const *coord);
@@ -49,6 +51,8 @@ int orc_linear_backward(int activation, int relu_grad_mode,
                         float const *weight, float *weight_grad,
                         float *bias_grad, int64_t batch, int64_t in_dim,
                         int64_t out_dim);
+void orc_linear_l2_regularizer_grad(float const *weight, float *weight_grad,
+                                    int64_t n, float lambda);
 /* C[M,N] = op(A).op(B) accumulated in double, for GEMM checks at any size. */
 void orc_gemm_f64(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K,
                   float const *A, float const *B, float *C);
@@ -107,16 +111,17 @@ int orc_embedding_backward_f64(int64_t const *indices, float const *out_grad,
                                int64_t bag, int64_t dim, int64_t num_entries);
 
 /* ---- attention core and MultiHeadAttention ---- */
-/* q [B,Sq,H,D], k,v [B,Skv,H,D] (dense), o [B,Sq,H,D], lse [B,H,Sq].
- * bf16_mode: round P to bf16 before the PV product and O at the store. */
+/* q [B,Sq,H,D], k [B,Skv,H,D], v [B,Skv,H,Dv] (dense), o [B,Sq,H,Dv],
+ * lse [B,H,Sq].  bf16_mode: round P to bf16 before the PV product and O at the
+ * store. */
 void orc_attention_forward(float const *q, float const *k, float const *v,
                            float *o, float *lse, int64_t B, int64_t H,
-                           int64_t Sq, int64_t Skv, int64_t D, float scale,
-                           int causal, int bf16_mode);
+                           int64_t Sq, int64_t Skv, int64_t D, int64_t Dv,
+                           float scale, int causal, int bf16_mode);
 void orc_attention_backward(float const *q, float const *k, float const *v,
                             float const *d_o, float *dq, float *dk, float *dv,
                             int64_t B, int64_t H, int64_t Sq, int64_t Skv,
-                            int64_t D, float scale, int causal);
+                            int64_t D, int64_t Dv, float scale, int causal);
 
 typedef struct {
   int64_t num_samples, num_heads;

@@ -49,6 +49,15 @@ def lib():
     return _lib
 
 
+def set_num_threads(n):
+    """Threads for the oracle's row- and head-parallel loops (same bits for any count)."""
+    lib().orc_set_num_threads(c_int(int(n)))
+
+
+def max_threads():
+    return int(lib().orc_get_max_threads())
+
+
 def _f32(a):
     a = np.ascontiguousarray(a, dtype=np.float32)
     return a
@@ -145,6 +154,14 @@ def linear_backward(y, dy, x, w, activation=-1, relu_grad_mode=0, use_bias=True)
     if rc:
         raise ValueError("Unhandled activation function")
     return dx, dw, db
+
+
+def linear_l2_regularizer_grad(w, dw, lam):
+    """Returns dw + lam * w (the reference adds the term once per backward call)."""
+    w = _f32(w)
+    out = np.array(_f32(dw), copy=True)
+    lib().orc_linear_l2_regularizer_grad(_p(w), _p(out), c_i64(w.size), c_f(lam))
+    return out
 
 
 def gemm_f64(A, B, trans_a=False, trans_b=False):
@@ -333,27 +350,27 @@ def embedding_backward(indices, out_grad, num_entries, aggr=-1, f64=False, dw_in
 
 
 def attention_forward(q, k, v, scale, causal, bf16_mode=False):
-    """q [B,Sq,H,D], k/v [B,Skv,H,D] -> o [B,Sq,H,D], lse [B,H,Sq]."""
+    """q [B,Sq,H,D], k [B,Skv,H,D], v [B,Skv,H,Dv] -> o [B,Sq,H,Dv], lse [B,H,Sq]."""
     q, k, v = _f32(q), _f32(k), _f32(v)
     B, Sq, H, D = q.shape
-    Skv = k.shape[1]
-    o = np.empty_like(q)
+    Skv, Dv = k.shape[1], v.shape[3]
+    o = np.empty((B, Sq, H, Dv), np.float32)
     lse = np.empty((B, H, Sq), np.float32)
     lib().orc_attention_forward(_p(q), _p(k), _p(v), _p(o), _p(lse), c_i64(B), c_i64(H),
-                                c_i64(Sq), c_i64(Skv), c_i64(D), c_f(scale), c_int(int(causal)),
-                                c_int(int(bf16_mode)))
+                                c_i64(Sq), c_i64(Skv), c_i64(D), c_i64(Dv), c_f(scale),
+                                c_int(int(causal)), c_int(int(bf16_mode)))
     return o, lse
 
 
 def attention_backward(q, k, v, d_o, scale, causal):
     q, k, v, d_o = _f32(q), _f32(k), _f32(v), _f32(d_o)
     B, Sq, H, D = q.shape
-    Skv = k.shape[1]
+    Skv, Dv = k.shape[1], v.shape[3]
     dq = np.empty_like(q)
     dk = np.empty_like(k)
     dv = np.empty_like(v)
     lib().orc_attention_backward(_p(q), _p(k), _p(v), _p(d_o), _p(dq), _p(dk), _p(dv), c_i64(B),
-                                 c_i64(H), c_i64(Sq), c_i64(Skv), c_i64(D), c_f(scale),
+                                 c_i64(H), c_i64(Sq), c_i64(Skv), c_i64(D), c_i64(Dv), c_f(scale),
                                  c_int(int(causal)))
     return dq, dk, dv
 

@@ -51,15 +51,12 @@ def test_encoder_layer_small(ffk, oracle, pre_ln, gelu, p):
     dy = bf16_round(g.standard_normal(x.shape))
     y_ref, dx_ref, g_ref = layer_forward_backward(oracle, cfg, params, x, dy)
     y, dx, grads = run_device(ffk, cfg, params, x, dy)
-    # bf16 tolerance with headroom for a dozen chained bf16 roundings.  ReLU's
-    # gradient is discontinuous: a pre-activation that rounds to +-tiny on one
-    # side and to the other sign on the other flips one mask bit and moves a
-    # handful of gradient elements, so the ReLU variant tolerates 1% outliers.
-    frac = 0.0 if gelu else 1e-2
+    # every tensor within the bf16 tolerance of 2e-2 (measured: at most 0.17 of that bound,
+    # through a dozen chained bf16 roundings, both variants)
     assert_close(y, y_ref, 2e-2, "y")
-    assert_close(dx, dx_ref, 3e-2, "dx", frac)
+    assert_close(dx, dx_ref, 2e-2, "dx")
     for k in g_ref:
-        assert_close(grads[k].reshape(g_ref[k].shape), g_ref[k], 3e-2, "grad " + k, frac)
+        assert_close(grads[k].reshape(g_ref[k].shape), g_ref[k], 2e-2, "grad " + k)
 
 
 def test_encoder_layer_config2_shape_runs_and_is_deterministic(ffk):
@@ -82,6 +79,31 @@ def test_encoder_layer_config2_shape_runs_and_is_deterministic(ffk):
     cfg0 = dict(cfg, p=0.0)
     y0, _, _ = run_device(ffk, cfg0, params, x, dy)
     assert not np.array_equal(y0, y1)
+
+
+def test_encoder_layer_config2_full_size_against_the_oracle_on_one_sequence(ffk, oracle):
+    """BASELINE config 2 at full size against the oracle.  The layer mixes tokens only inside a
+    sequence, and the dropout streams are indexed by flat element position, so sequence 0 of the
+    batch of 8 (the first 512 x 1024 elements of every activation) is what the oracle computes for
+    a batch of that one sequence with the same weights, seeds and upstream gradient: y[0] and dx[0]
+    are compared with it.  This runs the kernels the full size dispatches to (the pipelined GEMMs
+    with the element-wise tails, the paired weight-gradient launches, split-K), which the small
+    layer tests do not reach.  The weight gradients sum over all 8 sequences; they are covered at
+    this size by the bit-equality with the one-kernel-per-operator sequence below."""
+    cfg = dict(batch=8, seq=512, d_model=1024, heads=16, d_ff=4096, p=0.1, seed=7, eps=1e-5,
+               scale=0.125, causal=False, pre_ln=True, gelu=True)
+    say("encoder layer cfg2 full size vs oracle on sequence 0")
+    g = rng(2)
+    params = make_params(g, cfg, bf16_round)
+    x = bf16_round(g.standard_normal((8, 512, 1024)))
+    dy = bf16_round(g.standard_normal(x.shape))
+    y, dx, _ = run_device(ffk, cfg, params, x, dy)
+    cfg1 = dict(cfg, batch=1)
+    y_ref, dx_ref, _ = layer_forward_backward(oracle, cfg1, params, x[:1], dy[:1])
+    assert_close(y[:1], y_ref, 2e-2, "y[0]")
+    assert_close(dx[:1], dx_ref, 2e-2, "dx[0]")
+    # and the other sequences are not copies of sequence 0
+    assert not np.array_equal(y[1], y[0])
 
 
 @pytest.mark.parametrize("shape", ["small", "config2"])

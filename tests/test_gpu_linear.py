@@ -87,6 +87,40 @@ def test_linear_fp32_ragged(ffk, oracle, shape, act):
     assert_close(to_np(db), db_ref, FP32_RTOL, "db")
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("shape", [(32, 64, 128), (7, 5, 3), (128, 1024, 512)])
+def test_linear_backward_with_l2_regularizer(ffk, oracle, dtype, shape):
+    """Linear backward followed by the regulariser's term (linear_kernels.cu:269-290):
+    dW = (dW + g^T x) + lambda W, twice in a row as the reference's accumulating path runs it."""
+    batch, in_dim, out_dim = shape
+    lam = 0.25
+    say("linear backward + L2 regulariser", dtype, shape)
+    x, w, b, dy = _cfg1_inputs(seed=3, batch=batch, in_dim=in_dim, out_dim=out_dim)
+    w = w * 20
+    bf = dtype == "bf16"
+    if bf:
+        x, w, dy = bf16_round(x), bf16_round(w), bf16_round(dy)
+    rnd = bf16_round if bf else (lambda a: a)
+    _, dw1, _ = oracle.linear_backward(None, dy, x, w)
+    want1 = rnd(oracle.linear_l2_regularizer_grad(w, rnd(dw1), lam))
+    want2 = rnd(oracle.linear_l2_regularizer_grad(w, rnd(want1 + dw1), lam))
+    tt = torch.bfloat16 if bf else torch.float32
+    xd, wd, dyd = (to_dev(a, torch, tt) for a in (x, w, dy))
+    dw = torch.zeros_like(wd)
+    ffk.linear_backward(None, dyd, xd, wd, None, dw, None, accumulate=True)
+    ffk.linear_l2_regularizer_grad(wd, dw, lam)
+    tol = BF16_RTOL if bf else FP32_RTOL
+    assert_close(to_np(dw), want1, tol, "dw + lambda w")
+    ffk.linear_backward(None, dyd, xd, wd, None, dw, None, accumulate=True)
+    ffk.linear_l2_regularizer_grad(wd, dw, lam)
+    assert_close(to_np(dw), want2, tol, "second call")
+    # the term alone, on a gradient of zeros, is lambda W to the last bit in fp32
+    z = torch.zeros_like(wd)
+    ffk.linear_l2_regularizer_grad(wd, z, lam)
+    if not bf:
+        assert np.array_equal(to_np(z), oracle.linear_l2_regularizer_grad(w, np.zeros_like(w), lam))
+
+
 def test_linear_no_bias_and_skipped_grads(ffk, oracle):
     x, w, b, dy = _cfg1_inputs(seed=5, batch=16, in_dim=24, out_dim=40)
     say("linear fp32 no bias / NULL grads")

@@ -58,6 +58,25 @@ def test_linear_relu_modes(oracle):
         oracle.linear_forward(x, w, b, activation=3)  # the reference PANICs on GELU
 
 
+def test_linear_l2_regularizer_grad_is_the_gradient_of_the_penalty(oracle):
+    """dW' = dW + lambda W: lambda W is the gradient of lambda/2 |W|^2 (autograd), it is added
+    to what the tensor holds (not stored over it, not scaled into it), and it uses W, not dW."""
+    g = rng(12)
+    w = g.standard_normal((4, 5)).astype(np.float32)
+    dw = g.standard_normal((4, 5)).astype(np.float32)
+    lam = 0.37
+    wt = t64(w).requires_grad_()
+    (0.5 * lam * (wt * wt).sum()).backward()
+    got = oracle.linear_l2_regularizer_grad(w, dw, lam)
+    assert np.allclose(got, dw + wt.grad.numpy(), atol=1e-6)
+    assert np.allclose(oracle.linear_l2_regularizer_grad(w, np.zeros_like(w), lam), lam * w, atol=1e-7)
+    assert np.array_equal(oracle.linear_l2_regularizer_grad(w, dw, 0.0), dw)
+    # a full backward with a zero output gradient leaves exactly lambda W behind the GEMM
+    x = g.standard_normal((6, 5)).astype(np.float32)
+    _, dw0, _ = oracle.linear_backward(None, np.zeros((6, 4), np.float32), x, w)
+    assert np.allclose(oracle.linear_l2_regularizer_grad(w, dw0, lam), lam * w, atol=1e-7)
+
+
 @pytest.mark.parametrize("name,fn,scalar", [
     ("EXP", torch.exp, 0.0), ("IDENTITY", lambda v: v * 1.0, 0.0),
     ("GELU", lambda v: F.gelu(v), 0.0), ("RSQRT", torch.rsqrt, 0.0),
@@ -242,11 +261,14 @@ def test_embedding_against_torch(oracle):
         oracle.embedding_forward(np.array([V]), w)
 
 
+@pytest.mark.parametrize("Dv", [8, 5, 12])
 @pytest.mark.parametrize("causal", [False, True])
-def test_attention_against_torch_sdpa(oracle, causal):
+def test_attention_against_torch_sdpa(oracle, causal, Dv):
+    """Dv != D: the value head size (vProjSize) is independent of the query/key one."""
     g = rng(9)
     B, S, H, D = 2, 11, 3, 8
-    q, k, v, do = (g.standard_normal((B, S, H, D)).astype(np.float32) for _ in range(4))
+    q, k = (g.standard_normal((B, S, H, D)).astype(np.float32) for _ in range(2))
+    v, do = (g.standard_normal((B, S, H, Dv)).astype(np.float32) for _ in range(2))
     scale = 0.31
     o, lse = oracle.attention_forward(q, k, v, scale, causal)
     qt, kt, vt = (t64(a).transpose(1, 2).requires_grad_() for a in (q, k, v))
@@ -299,26 +321,27 @@ def test_attention_bf16_mode_against_torch_with_rounded_probabilities(oracle, ca
     assert not np.array_equal(o, o32)
 
 
-def test_mha_against_torch_composition(oracle):
+@pytest.mark.parametrize("Dv", [4, 6])
+def test_mha_against_torch_composition(oracle, Dv):
     g = rng(10)
     B, Sq, Skv, H, E, Dh = 2, 6, 7, 3, 10, 4
-    desc = oracle.mha_desc(B, H, E, E + 1, E + 2, Dh, Dh, Dh, E, Sq, Skv, scale=0.5, causal=False)
+    desc = oracle.mha_desc(B, H, E, E + 1, E + 2, Dh, Dh, Dv, E, Sq, Skv, scale=0.5, causal=False)
     q = g.standard_normal((B, Sq, E)).astype(np.float32)
     k = g.standard_normal((B, Skv, E + 1)).astype(np.float32)
     v = g.standard_normal((B, Skv, E + 2)).astype(np.float32)
-    nq, nk, nv, no = H * Dh * E, H * Dh * (E + 1), H * Dh * (E + 2), E * H * Dh
+    nq, nk, nv, no = H * Dh * E, H * Dh * (E + 1), H * Dv * (E + 2), E * H * Dv
     w = (g.standard_normal((nq + nk + nv + no,)) * 0.3).astype(np.float32)
     dout = g.standard_normal((B, Sq, E)).astype(np.float32)
     out = oracle.mha_forward(desc, q, k, v, w)
     qt, kt, vt, wt = (t64(a).requires_grad_() for a in (q, k, v, w))
     wq = wt[:nq].view(H * Dh, E)
     wk = wt[nq:nq + nk].view(H * Dh, E + 1)
-    wv = wt[nq + nk:nq + nk + nv].view(H * Dh, E + 2)
-    wo = wt[nq + nk + nv:].view(E, H * Dh)
+    wv = wt[nq + nk:nq + nk + nv].view(H * Dv, E + 2)
+    wo = wt[nq + nk + nv:].view(E, H * Dv)
     Q = (qt @ wq.T).view(B, Sq, H, Dh).transpose(1, 2)
     K = (kt @ wk.T).view(B, Skv, H, Dh).transpose(1, 2)
-    Vv = (vt @ wv.T).view(B, Skv, H, Dh).transpose(1, 2)
-    ctx = F.scaled_dot_product_attention(Q, K, Vv, scale=0.5).transpose(1, 2).reshape(B, Sq, H * Dh)
+    Vv = (vt @ wv.T).view(B, Skv, H, Dv).transpose(1, 2)
+    ctx = F.scaled_dot_product_attention(Q, K, Vv, scale=0.5).transpose(1, 2).reshape(B, Sq, H * Dv)
     ot = ctx @ wo.T
     ot.backward(t64(dout))
     assert np.allclose(out, ot.detach().numpy(), atol=1e-5)
@@ -327,6 +350,28 @@ def test_mha_against_torch_composition(oracle):
     assert np.allclose(dk, kt.grad.numpy(), atol=2e-5)
     assert np.allclose(dv, vt.grad.numpy(), atol=2e-5)
     assert np.allclose(dw, wt.grad.numpy(), atol=5e-5)
+
+
+def test_thread_count_does_not_change_a_bit(oracle):
+    """The oracle's parallel loops (matrix products by row, attention by (batch, head)) give
+    every output element to one thread in the serial order."""
+    g = rng(33)
+    A = g.standard_normal((130, 90)).astype(np.float32)
+    Bm = g.standard_normal((90, 110)).astype(np.float32)
+    B, S, H, D = 2, 70, 4, 8
+    q, k, v, do = (g.standard_normal((B, S, H, D)).astype(np.float32) for _ in range(4))
+    before = oracle.max_threads()
+    try:
+        oracle.set_num_threads(1)
+        one = [oracle.matmul(A, Bm), oracle.gemm_f64(A, Bm), *oracle.attention_forward(q, k, v, 0.3, True),
+               *oracle.attention_backward(q, k, v, do, 0.3, True)]
+        oracle.set_num_threads(4)
+        four = [oracle.matmul(A, Bm), oracle.gemm_f64(A, Bm), *oracle.attention_forward(q, k, v, 0.3, True),
+                *oracle.attention_backward(q, k, v, do, 0.3, True)]
+    finally:
+        oracle.set_num_threads(before)
+    for a, b in zip(one, four):
+        assert np.array_equal(a, b)
 
 
 def test_round_bf16_matches_torch(oracle):
