@@ -49,6 +49,7 @@ class AttentionDesc(ctypes.Structure):
         ("v_batch_stride", c_i64), ("v_seq_stride", c_i64),
         ("o_batch_stride", c_i64), ("o_seq_stride", c_i64),
         ("scale", c_f), ("causal", c_int),
+        ("v_head_dim", c_i64),  # 0 = head_dim
     ]
 
 
@@ -653,18 +654,19 @@ def embedding_backward(indices, out_grad, weight_grad, aggr=AGGR_NONE, determini
     return weight_grad
 
 
-def attention_desc_bshd(q, k, scale, causal):
-    """Descriptor for dense [B, S, H, D] tensors."""
+def attention_desc_bshd(q, k, scale, causal, v=None):
+    """Descriptor for dense q [B, Sq, H, D], k [B, Skv, H, D], v [B, Skv, H, Dv] tensors."""
     B, Sq, H, D = q.shape
     Skv = k.shape[1]
+    Dv = D if v is None else v.shape[3]
     return AttentionDesc(B, H, Sq, Skv, D, Sq * H * D, H * D, Skv * H * D, H * D,
-                         Skv * H * D, H * D, Sq * H * D, H * D, scale, int(causal))
+                         Skv * H * Dv, H * Dv, Sq * H * Dv, H * Dv, scale, int(causal), Dv)
 
 
 def attention_forward(q, k, v, scale, causal, desc=None):
     torch = _torch()
-    desc = desc or attention_desc_bshd(q, k, scale, causal)
-    o = torch.empty_like(q)
+    desc = desc or attention_desc_bshd(q, k, scale, causal, v)
+    o = torch.empty(tuple(q.shape[:3]) + (v.shape[3],), dtype=q.dtype, device=q.device)
     lse = torch.empty((desc.batch, desc.heads, desc.seq_q), dtype=torch.float32, device=q.device)
     check(lib().ffk_attention_forward(current_stream(), dtype_of(q), ctypes.byref(desc), ptr(q),
                                       ptr(k), ptr(v), ptr(o), ptr(lse)))
@@ -673,7 +675,7 @@ def attention_forward(q, k, v, scale, causal, desc=None):
 
 def attention_backward(q, k, v, o, d_o, lse, scale, causal, desc=None):
     torch = _torch()
-    desc = desc or attention_desc_bshd(q, k, scale, causal)
+    desc = desc or attention_desc_bshd(q, k, scale, causal, v)
     dq = torch.empty_like(q)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)

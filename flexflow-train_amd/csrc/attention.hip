@@ -605,11 +605,23 @@ int attention_f32_backward(hipStream_t st, ffk_attention_desc_t const *d, void c
                            void const *v, void const *o, void const *d_o, float const *lse, float *delta,
                            void *dq, void *dk, void *dv);
 
+// any multiple of 8 up to 256 for either head size (attention_gen.hip)
+int attention_bf16_general_forward(hipStream_t st, ffk_attention_desc_t const *d, void const *q, void const *k,
+                                   void const *v, void *o, float *lse);
+int attention_bf16_general_backward(hipStream_t st, ffk_attention_desc_t const *d, void const *q, void const *k,
+                                    void const *v, void const *o, void const *d_o, float const *lse,
+                                    float *delta, void *dq, void *dk, void *dv);
+
+// the kernels of this file and of attention_fwd.hip / attention_bwd.hip: one head size, 64 or 128
+static bool tuned_head_size(ffk_attention_desc_t const *d) {
+  return (d->head_dim == 64 || d->head_dim == 128) && (d->v_head_dim == 0 || d->v_head_dim == d->head_dim);
+}
+
 static int check_desc(char const *who, int dtype, ffk_attention_desc_t const *d) {
   FFK_REQUIRE(d != nullptr, "%s: NULL descriptor", who);
-  FFK_REQUIRE(dtype == FFK_BF16, "%s: dtype %d not supported (FLOAT or BF16)", who, dtype);
-  FFK_REQUIRE(d->head_dim == 64 || d->head_dim == 128,
-              "%s: bf16 head_dim %lld not supported (64 or 128)", who, (long long)d->head_dim);
+  // FLOAT was dispatched to the fp32 core before this check: what is left must be BF16
+  FFK_REQUIRE(dtype == FFK_BF16, "%s: dtype %d not supported (the entry point takes FLOAT or BF16)", who, dtype);
+  FFK_REQUIRE(d->head_dim > 0 && d->v_head_dim >= 0, "%s: bad head size", who);
   FFK_REQUIRE(d->batch > 0 && d->heads > 0 && d->seq_q > 0 && d->seq_kv > 0, "%s: bad shape", who);
   FFK_REQUIRE(d->batch * d->heads * ((d->seq_q > d->seq_kv ? d->seq_q : d->seq_kv) / 128 + 1) < (1ll << 31),
               "%s: too many workgroups", who);
@@ -618,9 +630,11 @@ static int check_desc(char const *who, int dtype, ffk_attention_desc_t const *d)
                   d->o_seq_stride % 8 == 0 && d->q_batch_stride % 8 == 0 && d->k_batch_stride % 8 == 0 &&
                   d->v_batch_stride % 8 == 0 && d->o_batch_stride % 8 == 0,
               "%s: strides must be multiples of 8 elements", who);
-  FFK_REQUIRE(d->q_seq_stride >= d->heads * d->head_dim && d->k_seq_stride >= d->heads * d->head_dim &&
-                  d->v_seq_stride >= d->heads * d->head_dim && d->o_seq_stride >= d->heads * d->head_dim,
-              "%s: sequence stride smaller than heads * head_dim", who);
+  if (tuned_head_size(d)) {
+    FFK_REQUIRE(d->q_seq_stride >= d->heads * d->head_dim && d->k_seq_stride >= d->heads * d->head_dim &&
+                    d->v_seq_stride >= d->heads * d->head_dim && d->o_seq_stride >= d->heads * d->head_dim,
+                "%s: sequence stride smaller than heads * head_dim", who);
+  }
   return FFK_OK;
 }
 
@@ -639,6 +653,7 @@ extern "C" int ffk_attention_forward(ffk_stream_t stream, int dtype,
   if (dtype == FFK_FLOAT) return attention_f32_forward(as_stream(stream), d, q, k, v, o, lse);
   int rc = check_desc("attention_forward", dtype, d);
   if (rc != FFK_OK) return rc;
+  if (!tuned_head_size(d)) return attention_bf16_general_forward(as_stream(stream), d, q, k, v, o, lse);
   AttnParams p;
   p.q = static_cast<bf16 const *>(q);
   p.k = static_cast<bf16 const *>(k);
@@ -693,6 +708,9 @@ extern "C" int ffk_attention_backward(ffk_stream_t stream, int dtype,
   }
   int rc = check_desc("attention_backward", dtype, d);
   if (rc != FFK_OK) return rc;
+  if (!tuned_head_size(d)) {
+    return attention_bf16_general_backward(as_stream(stream), d, q, k, v, o, d_o, lse, delta, dq, dk, dv);
+  }
   AttnBwdParams p;
   p.q = static_cast<bf16 const *>(q);
   p.k = static_cast<bf16 const *>(k);

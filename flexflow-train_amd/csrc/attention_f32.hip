@@ -14,8 +14,16 @@
 // accumulator tile as an operand: step r takes element r of every lane, whose
 // reduction index is 8*(r/4) + 4*h + r%4, and the other operand is read from
 // the LDS tile row of that index.
-// head_dim: any multiple of 4 up to 128; DP is head_dim rounded up to 32, 64
-// or 128 and the missing columns are read as zeros.
+// head sizes: any multiple of 4 up to 256, and the value head size (V, O, dO,
+// dV) may differ from the query/key one (Q, K, dQ, dK): the reference's model
+// builders ask for kdim = vdim = 256 (lib/models/src/models/transformer/
+// transformer.cc:37-38, bert/bert.cc:64-65) and the projection sizes are free
+// (lib/op-attrs/src/op-attrs/ops/attention.cc:23-37).  DP is the larger of
+// the two rounded up to 32, 64, 128 or 256; the missing columns of either
+// kind are read as zeros.  At DP = 256 a wave's operands and accumulators no
+// longer fit its 512 registers in one pass: tiles are then loaded without a
+// register prefetch and dK and dV are produced by two launches of the dK/dV
+// kernel (WHAT = 1: dV only, needs K; WHAT = 2: dK only, needs K and V).
 #include "ffk_common.h"
 
 namespace ffk {
@@ -29,7 +37,7 @@ struct AttnF32Params {
   float *lse;  // forward: written; backward: read
   float *delta;
   float *dq, *dk, *dv;
-  int B, H, Sq, Skv, D;
+  int B, H, Sq, Skv, Dq, Dv;  // Dq: head size of Q, K, dQ, dK; Dv: of V, O, dO, dV
   int64_t q_bs, q_ss, k_bs, k_ss, v_bs, v_ss, o_bs, o_ss;
   float scale, scale_log2;
   int causal;
@@ -43,6 +51,8 @@ struct AttnF32Cfg {
   static constexpr int kStrideB = DP + 8; // tile also read one row per half-wave: 4 rows apart = 32 banks apart
   static constexpr int kChunks = kTile * DP / 4 / 256;  // 16-byte chunks per thread
   static_assert(kTile * DP / 4 % 256 == 0, "tile chunks");
+  // next tile fetched into registers while this one is computed on (not at DP = 256: no room)
+  static constexpr bool kPrefetch = DP <= 128;
 };
 
 __device__ __forceinline__ f32x4 load4_or_zero(float const *row, int d0, int D) {
@@ -115,12 +125,12 @@ __global__ __launch_bounds__(256) void attn_f32_fwd_kernel(AttnF32Params p) {
   int const head = hb % p.H, b = hb / p.H;
   int const q0 = qb * C::kBlk;
   int const qrow = q0 + wave * 32 + l32;
-  float const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * p.D;
-  float const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * p.D;
-  float const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * p.D;
+  float const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * p.Dq;
+  float const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * p.Dq;
+  float const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * p.Dv;
 
   float qf[DP / 2];
-  load_owned_row<DP>(qp + (int64_t)min(qrow, p.Sq - 1) * p.q_ss, p.D, h32, qf);
+  load_owned_row<DP>(qp + (int64_t)min(qrow, p.Sq - 1) * p.q_ss, p.Dq, h32, qf);
 
   int kv_end = p.Skv;
   if (p.causal) kv_end = min(p.Skv, q0 + C::kBlk);
@@ -134,19 +144,22 @@ __global__ __launch_bounds__(256) void attn_f32_fwd_kernel(AttnF32Params p) {
   float m_run = -INFINITY, l_run = 0.0f;
 
   f32x4 rk[C::kChunks], rv[C::kChunks];
-  tile_gload<DP>(kp, p.k_ss, 0, p.Skv - 1, p.D, t, rk);
-  tile_gload<DP>(vp, p.v_ss, 0, p.Skv - 1, p.D, t, rv);
-  tile_lstore<DP, C::kStrideA>(Ks[0], t, rk);
-  tile_lstore<DP, C::kStrideB>(Vs[0], t, rv);
+  auto fetch = [&](int kv0) {
+    tile_gload<DP>(kp, p.k_ss, kv0, p.Skv - 1, p.Dq, t, rk);
+    tile_gload<DP>(vp, p.v_ss, kv0, p.Skv - 1, p.Dv, t, rv);
+  };
+  auto stash = [&](int buf) {
+    tile_lstore<DP, C::kStrideA>(Ks[buf], t, rk);
+    tile_lstore<DP, C::kStrideB>(Vs[buf], t, rv);
+  };
+  fetch(0);
+  stash(0);
   __syncthreads();
   int cur = 0;
   for (int it = 0; it < ntiles; it++) {
     int const kv0 = it * C::kTile;
     bool const more = it + 1 < ntiles;
-    if (more) {
-      tile_gload<DP>(kp, p.k_ss, kv0 + C::kTile, p.Skv - 1, p.D, t, rk);
-      tile_gload<DP>(vp, p.v_ss, kv0 + C::kTile, p.Skv - 1, p.D, t, rv);
-    }
+    if (C::kPrefetch && more) fetch(kv0 + C::kTile);
     // a wave whose rows all lie before this tile (causal) has nothing to add
     bool const active = !p.causal || kv0 <= q0 + wave * 32 + 31;
     if (active) {
@@ -198,8 +211,8 @@ __global__ __launch_bounds__(256) void attn_f32_fwd_kernel(AttnF32Params p) {
       }
     }
     if (more) {
-      tile_lstore<DP, C::kStrideA>(Ks[cur ^ 1], t, rk);
-      tile_lstore<DP, C::kStrideB>(Vs[cur ^ 1], t, rv);
+      if (!C::kPrefetch) fetch(kv0 + C::kTile);
+      stash(cur ^ 1);
     }
     __syncthreads();
     cur ^= 1;
@@ -207,13 +220,13 @@ __global__ __launch_bounds__(256) void attn_f32_fwd_kernel(AttnF32Params p) {
 
   if (qrow < p.Sq) {
     float const inv = 1.0f / l_run;
-    float *op = p.out + (int64_t)b * p.o_bs + (int64_t)qrow * p.o_ss + (int64_t)head * p.D;
+    float *op = p.out + (int64_t)b * p.o_bs + (int64_t)qrow * p.o_ss + (int64_t)head * p.Dv;
 #pragma unroll
     for (int i = 0; i < DP / 32; i++) {
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         int const d = i * 32 + 8 * g + 4 * h32;
-        if (d < p.D) {
+        if (d < p.Dv) {
           f32x4 w = {oacc[i][4 * g] * inv, oacc[i][4 * g + 1] * inv, oacc[i][4 * g + 2] * inv,
                      oacc[i][4 * g + 3] * inv};
           *reinterpret_cast<f32x4 *>(op + d) = w;
@@ -241,10 +254,10 @@ __global__ __launch_bounds__(256) void attn_f32_delta_kernel(AttnF32Params p) {
     head = (int)(row % p.H);
     q = (int)((row / p.H) % p.Sq);
     b = (int)(row / ((int64_t)p.Sq * p.H));
-    int64_t const off = (int64_t)b * p.o_bs + (int64_t)q * p.o_ss + (int64_t)head * p.D;
+    int64_t const off = (int64_t)b * p.o_bs + (int64_t)q * p.o_ss + (int64_t)head * p.Dv;
     int const d0 = (lane % LPR) * 4;
-    f32x4 const o = load4_or_zero(p.o + off, d0, p.D);
-    f32x4 const g = load4_or_zero(p.d_o + off, d0, p.D);
+    f32x4 const o = load4_or_zero(p.o + off, d0, p.Dv);
+    f32x4 const g = load4_or_zero(p.d_o + off, d0, p.Dv);
     s = o[0] * g[0] + o[1] * g[1] + o[2] * g[2] + o[3] * g[3];
   }
 #pragma unroll
@@ -254,10 +267,13 @@ __global__ __launch_bounds__(256) void attn_f32_delta_kernel(AttnF32Params p) {
 
 // --------------------------------------------------------------------------
 // backward (A): dK, dV.  Workgroup owns 128 key rows, streams query tiles.
+// WHAT: bit 0 = produce dV, bit 1 = produce dK.
 // --------------------------------------------------------------------------
-template <int DP>
+template <int DP, int WHAT>
 __global__ __launch_bounds__(256) void attn_f32_bwd_dkdv_kernel(AttnF32Params p) {
   using C = AttnF32Cfg<DP>;
+  constexpr bool kDV = (WHAT & 1) != 0, kDK = (WHAT & 2) != 0;
+  // dV needs the dO tile as an operand, dK needs it for dP: both
   __shared__ __attribute__((aligned(16))) float Qs[2][C::kTile * C::kStrideB];
   __shared__ __attribute__((aligned(16))) float Gs[2][C::kTile * C::kStrideB];  // dO
   __shared__ __attribute__((aligned(16))) float Ls[2][C::kTile], Ds[2][C::kTile];
@@ -267,24 +283,26 @@ __global__ __launch_bounds__(256) void attn_f32_bwd_dkdv_kernel(AttnF32Params p)
   int const head = hb % p.H, b = hb / p.H;
   int const kv0 = (blockIdx.x / (p.H * p.B)) * C::kBlk;
   int const kvrow = kv0 + wave * 32 + l32;
-  float const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * p.D;
-  float const *gp = p.d_o + (int64_t)b * p.o_bs + (int64_t)head * p.D;
-  float const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * p.D;
-  float const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * p.D;
+  float const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * p.Dq;
+  float const *gp = p.d_o + (int64_t)b * p.o_bs + (int64_t)head * p.Dv;
+  float const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * p.Dq;
+  float const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * p.Dv;
   float const *lsep = p.lse + ((int64_t)b * p.H + head) * p.Sq;
   float const *delp = p.delta + ((int64_t)b * p.H + head) * p.Sq;
 
-  float kf[DP / 2], vf[DP / 2];
-  load_owned_row<DP>(kp + (int64_t)min(kvrow, p.Skv - 1) * p.k_ss, p.D, h32, kf);
-  load_owned_row<DP>(vp + (int64_t)min(kvrow, p.Skv - 1) * p.v_ss, p.D, h32, vf);
-  f32x16 dk[DP / 32], dv[DP / 32];
+  float kf[DP / 2];
+  float vf[kDK ? DP / 2 : 1];
+  load_owned_row<DP>(kp + (int64_t)min(kvrow, p.Skv - 1) * p.k_ss, p.Dq, h32, kf);
+  if constexpr (kDK) load_owned_row<DP>(vp + (int64_t)min(kvrow, p.Skv - 1) * p.v_ss, p.Dv, h32, vf);
+  f32x16 dk[kDK ? DP / 32 : 1], dv[kDV ? DP / 32 : 1];
 #pragma unroll
-  for (int i = 0; i < DP / 32; i++)
+  for (int i = 0; i < (kDK ? DP / 32 : 1); i++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      dk[i][r] = 0.0f;
-      dv[i][r] = 0.0f;
-    }
+    for (int r = 0; r < 16; r++) dk[i][r] = 0.0f;
+#pragma unroll
+  for (int i = 0; i < (kDV ? DP / 32 : 1); i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dv[i][r] = 0.0f;
 
   int const q_begin = p.causal ? (kv0 / C::kTile) * C::kTile : 0;
   int const ntiles = q_begin < p.Sq ? (p.Sq - q_begin + C::kTile - 1) / C::kTile : 0;
@@ -292,8 +310,8 @@ __global__ __launch_bounds__(256) void attn_f32_bwd_dkdv_kernel(AttnF32Params p)
   f32x4 rq[C::kChunks], rg[C::kChunks];
   float rl = 0.0f, rd = 0.0f;
   auto gload = [&](int qt0) {
-    tile_gload<DP>(qp, p.q_ss, qt0, p.Sq - 1, p.D, t, rq);
-    tile_gload<DP>(gp, p.o_ss, qt0, p.Sq - 1, p.D, t, rg);
+    tile_gload<DP>(qp, p.q_ss, qt0, p.Sq - 1, p.Dq, t, rq);
+    tile_gload<DP>(gp, p.o_ss, qt0, p.Sq - 1, p.Dv, t, rg);
     int const gr = min(qt0 + (t & (C::kTile - 1)), p.Sq - 1);
     rl = lsep[gr] * kLog2eF;
     rd = delp[gr];
@@ -315,7 +333,7 @@ __global__ __launch_bounds__(256) void attn_f32_bwd_dkdv_kernel(AttnF32Params p)
   for (int it = 0; it < ntiles; it++) {
     int const qt0 = q_begin + it * C::kTile;
     bool const more = it + 1 < ntiles;
-    if (more) gload(qt0 + C::kTile);
+    if (C::kPrefetch && more) gload(qt0 + C::kTile);
     // a wave whose keys all lie after this query tile (causal) contributes nothing
     bool const active = !p.causal || kv0 + wave * 32 <= qt0 + C::kTile - 1;
     if (active) {
@@ -327,7 +345,7 @@ __global__ __launch_bounds__(256) void attn_f32_bwd_dkdv_kernel(AttnF32Params p)
         dp[r] = 0.0f;
       }
       contract_d<DP>(Qs[cur] + l32 * C::kStrideB + h32 * (DP / 2), kf, s);
-      contract_d<DP>(Gs[cur] + l32 * C::kStrideB + h32 * (DP / 2), vf, dp);
+      if constexpr (kDK) contract_d<DP>(Gs[cur] + l32 * C::kStrideB + h32 * (DP / 2), vf, dp);
       float pv[16], dsv[16];
 #pragma unroll
       for (int r = 0; r < 16; r++) {
@@ -348,29 +366,40 @@ __global__ __launch_bounds__(256) void attn_f32_bwd_dkdv_kernel(AttnF32Params p)
         int const qr = 8 * (r >> 2) + (r & 3);
 #pragma unroll
         for (int i = 0; i < DP / 32; i++) {
-          dv[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(pv[r], gt[qr * C::kStrideB + i * 32], dv[i], 0, 0, 0);
-          dk[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(dsv[r], qt[qr * C::kStrideB + i * 32], dk[i], 0, 0, 0);
+          if constexpr (kDV) {
+            dv[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(pv[r], gt[qr * C::kStrideB + i * 32], dv[i], 0, 0, 0);
+          }
+          if constexpr (kDK) {
+            dk[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(dsv[r], qt[qr * C::kStrideB + i * 32], dk[i], 0, 0, 0);
+          }
         }
       }
     }
-    if (more) lstore(cur ^ 1);
+    if (more) {
+      if (!C::kPrefetch) gload(qt0 + C::kTile);
+      lstore(cur ^ 1);
+    }
     __syncthreads();
     cur ^= 1;
   }
 
   // accumulator element r: key row 8*(r/4) + 4*h + r%4 of this wave's 32, column d = i*32 + l%32:
   // the 32 lanes of a half write 128 contiguous bytes of one row
-  float *dkp = p.dk + (int64_t)b * p.k_bs + (int64_t)head * p.D;
-  float *dvp = p.dv + (int64_t)b * p.v_bs + (int64_t)head * p.D;
+  float *dkp = p.dk + (int64_t)b * p.k_bs + (int64_t)head * p.Dq;
+  float *dvp = p.dv + (int64_t)b * p.v_bs + (int64_t)head * p.Dv;
 #pragma unroll
   for (int i = 0; i < DP / 32; i++) {
     int const d = i * 32 + l32;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       int const grow = kv0 + wave * 32 + 8 * (r >> 2) + 4 * h32 + (r & 3);
-      if (grow < p.Skv && d < p.D) {
-        dkp[(int64_t)grow * p.k_ss + d] = dk[i][r];
-        dvp[(int64_t)grow * p.v_ss + d] = dv[i][r];
+      if (grow < p.Skv) {
+        if constexpr (kDK) {
+          if (d < p.Dq) dkp[(int64_t)grow * p.k_ss + d] = dk[i][r];
+        }
+        if constexpr (kDV) {
+          if (d < p.Dv) dvp[(int64_t)grow * p.v_ss + d] = dv[i][r];
+        }
       }
     }
   }
@@ -392,15 +421,15 @@ __global__ __launch_bounds__(256) void attn_f32_bwd_dq_kernel(AttnF32Params p) {
   int const head = hb % p.H, b = hb / p.H;
   int const q0 = qb * C::kBlk;
   int const qrow = q0 + wave * 32 + l32;
-  float const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * p.D;
-  float const *gp = p.d_o + (int64_t)b * p.o_bs + (int64_t)head * p.D;
-  float const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * p.D;
-  float const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * p.D;
+  float const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * p.Dq;
+  float const *gp = p.d_o + (int64_t)b * p.o_bs + (int64_t)head * p.Dv;
+  float const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * p.Dq;
+  float const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * p.Dv;
 
   float qf[DP / 2], gf[DP / 2];
   int const rq = min(qrow, p.Sq - 1);
-  load_owned_row<DP>(qp + (int64_t)rq * p.q_ss, p.D, h32, qf);
-  load_owned_row<DP>(gp + (int64_t)rq * p.o_ss, p.D, h32, gf);
+  load_owned_row<DP>(qp + (int64_t)rq * p.q_ss, p.Dq, h32, qf);
+  load_owned_row<DP>(gp + (int64_t)rq * p.o_ss, p.Dv, h32, gf);
   float const lse2 = p.lse[((int64_t)b * p.H + head) * p.Sq + rq] * kLog2eF;
   float const delta_s = p.delta[((int64_t)b * p.H + head) * p.Sq + rq] * p.scale;
   f32x16 dq[DP / 32];
@@ -414,19 +443,22 @@ __global__ __launch_bounds__(256) void attn_f32_bwd_dq_kernel(AttnF32Params p) {
   int const ntiles = (kv_end + C::kTile - 1) / C::kTile;
 
   f32x4 rk[C::kChunks], rv[C::kChunks];
-  tile_gload<DP>(kp, p.k_ss, 0, p.Skv - 1, p.D, t, rk);
-  tile_gload<DP>(vp, p.v_ss, 0, p.Skv - 1, p.D, t, rv);
-  tile_lstore<DP, C::kStrideB>(Ks[0], t, rk);
-  tile_lstore<DP, C::kStrideA>(Vs[0], t, rv);
+  auto fetch = [&](int kt0) {
+    tile_gload<DP>(kp, p.k_ss, kt0, p.Skv - 1, p.Dq, t, rk);
+    tile_gload<DP>(vp, p.v_ss, kt0, p.Skv - 1, p.Dv, t, rv);
+  };
+  auto stash = [&](int buf) {
+    tile_lstore<DP, C::kStrideB>(Ks[buf], t, rk);
+    tile_lstore<DP, C::kStrideA>(Vs[buf], t, rv);
+  };
+  fetch(0);
+  stash(0);
   __syncthreads();
   int cur = 0;
   for (int it = 0; it < ntiles; it++) {
     int const kt0 = it * C::kTile;
     bool const more = it + 1 < ntiles;
-    if (more) {
-      tile_gload<DP>(kp, p.k_ss, kt0 + C::kTile, p.Skv - 1, p.D, t, rk);
-      tile_gload<DP>(vp, p.v_ss, kt0 + C::kTile, p.Skv - 1, p.D, t, rv);
-    }
+    if (C::kPrefetch && more) fetch(kt0 + C::kTile);
     bool const active = !p.causal || kt0 <= q0 + wave * 32 + 31;
     if (active) {
       // S^T = K Q^T, dP^T = V dO^T: rows = keys of the tile, column = this lane's query
@@ -458,21 +490,21 @@ __global__ __launch_bounds__(256) void attn_f32_bwd_dq_kernel(AttnF32Params p) {
       }
     }
     if (more) {
-      tile_lstore<DP, C::kStrideB>(Ks[cur ^ 1], t, rk);
-      tile_lstore<DP, C::kStrideA>(Vs[cur ^ 1], t, rv);
+      if (!C::kPrefetch) fetch(kt0 + C::kTile);
+      stash(cur ^ 1);
     }
     __syncthreads();
     cur ^= 1;
   }
 
   if (qrow < p.Sq) {
-    float *dqp = p.dq + (int64_t)b * p.q_bs + (int64_t)qrow * p.q_ss + (int64_t)head * p.D;
+    float *dqp = p.dq + (int64_t)b * p.q_bs + (int64_t)qrow * p.q_ss + (int64_t)head * p.Dq;
 #pragma unroll
     for (int i = 0; i < DP / 32; i++) {
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         int const d = i * 32 + 8 * g + 4 * h32;
-        if (d < p.D) {
+        if (d < p.Dq) {
           f32x4 w = {dq[i][4 * g], dq[i][4 * g + 1], dq[i][4 * g + 2], dq[i][4 * g + 3]};
           *reinterpret_cast<f32x4 *>(dqp + d) = w;
         }
@@ -482,8 +514,10 @@ __global__ __launch_bounds__(256) void attn_f32_bwd_dq_kernel(AttnF32Params p) {
 }
 
 static int check_desc_f32(char const *who, ffk_attention_desc_t const *d) {
-  FFK_REQUIRE(d->head_dim > 0 && d->head_dim <= 128 && d->head_dim % 4 == 0,
-              "%s: fp32 head_dim %lld not supported (a multiple of 4 up to 128)", who, (long long)d->head_dim);
+  int64_t const dq = d->head_dim, dv = d->v_head_dim > 0 ? d->v_head_dim : d->head_dim;
+  FFK_REQUIRE(dq > 0 && dq <= 256 && dq % 4 == 0 && dv <= 256 && dv % 4 == 0,
+              "%s: fp32 head_dim %lld / v_head_dim %lld not supported (multiples of 4 up to 256)", who,
+              (long long)dq, (long long)dv);
   FFK_REQUIRE(d->batch > 0 && d->heads > 0 && d->seq_q > 0 && d->seq_kv > 0, "%s: bad shape", who);
   FFK_REQUIRE(d->batch * d->heads * ((d->seq_q > d->seq_kv ? d->seq_q : d->seq_kv) / 128 + 1) < (1ll << 31),
               "%s: too many workgroups", who);
@@ -492,8 +526,8 @@ static int check_desc_f32(char const *who, ffk_attention_desc_t const *d) {
                   d->o_seq_stride % 4 == 0 && d->q_batch_stride % 4 == 0 && d->k_batch_stride % 4 == 0 &&
                   d->v_batch_stride % 4 == 0 && d->o_batch_stride % 4 == 0,
               "%s: fp32 strides must be multiples of 4 elements", who);
-  FFK_REQUIRE(d->q_seq_stride >= d->heads * d->head_dim && d->k_seq_stride >= d->heads * d->head_dim &&
-                  d->v_seq_stride >= d->heads * d->head_dim && d->o_seq_stride >= d->heads * d->head_dim,
+  FFK_REQUIRE(d->q_seq_stride >= d->heads * dq && d->k_seq_stride >= d->heads * dq &&
+                  d->v_seq_stride >= d->heads * dv && d->o_seq_stride >= d->heads * dv,
               "%s: sequence stride smaller than heads * head_dim", who);
   return FFK_OK;
 }
@@ -501,7 +535,8 @@ static int check_desc_f32(char const *who, ffk_attention_desc_t const *d) {
 static AttnF32Params make_params(ffk_attention_desc_t const *d) {
   AttnF32Params p = {};
   p.B = (int)d->batch; p.H = (int)d->heads; p.Sq = (int)d->seq_q; p.Skv = (int)d->seq_kv;
-  p.D = (int)d->head_dim;
+  p.Dq = (int)d->head_dim;
+  p.Dv = (int)(d->v_head_dim > 0 ? d->v_head_dim : d->head_dim);
   p.q_bs = d->q_batch_stride; p.q_ss = d->q_seq_stride;
   p.k_bs = d->k_batch_stride; p.k_ss = d->k_seq_stride;
   p.v_bs = d->v_batch_stride; p.v_ss = d->v_seq_stride;
@@ -516,7 +551,8 @@ static AttnF32Params make_params(ffk_attention_desc_t const *d) {
   do {                                                                         \
     if ((D_) <= 32) { CALL(32); }                                              \
     else if ((D_) <= 64) { CALL(64); }                                         \
-    else { CALL(128); }                                                        \
+    else if ((D_) <= 128) { CALL(128); }                                       \
+    else { CALL(256); }                                                        \
   } while (0)
 
 int attention_f32_forward(hipStream_t st, ffk_attention_desc_t const *d, void const *q, void const *k,
@@ -530,11 +566,24 @@ int attention_f32_forward(hipStream_t st, ffk_attention_desc_t const *d, void co
   p.out = static_cast<float *>(o);
   p.lse = lse;
   unsigned const grid = (unsigned)(ceil_div(p.Sq, 128) * p.H * p.B);
+  int const dmax = p.Dq > p.Dv ? p.Dq : p.Dv;
 #define CALL(DP_) attn_f32_fwd_kernel<DP_><<<grid, 256, 0, st>>>(p)
-  FFK_ATTN_F32_DISPATCH(p.D, CALL);
+  FFK_ATTN_F32_DISPATCH(dmax, CALL);
 #undef CALL
   FFK_CHECK_LAUNCH();
   return FFK_OK;
+}
+
+template <int DP>
+static void launch_f32_backward(hipStream_t st, AttnF32Params const &p, int64_t rows, unsigned gkv, unsigned gq) {
+  attn_f32_delta_kernel<DP><<<(unsigned)ceil_div(rows, 4 * (64 / (DP / 4))), 256, 0, st>>>(p);
+  if constexpr (DP <= 128) {
+    attn_f32_bwd_dkdv_kernel<DP, 3><<<gkv, 256, 0, st>>>(p);
+  } else {
+    attn_f32_bwd_dkdv_kernel<DP, 1><<<gkv, 256, 0, st>>>(p);
+    attn_f32_bwd_dkdv_kernel<DP, 2><<<gkv, 256, 0, st>>>(p);
+  }
+  attn_f32_bwd_dq_kernel<DP><<<gq, 256, 0, st>>>(p);
 }
 
 int attention_f32_backward(hipStream_t st, ffk_attention_desc_t const *d, void const *q, void const *k,
@@ -556,13 +605,9 @@ int attention_f32_backward(hipStream_t st, ffk_attention_desc_t const *d, void c
   int64_t const rows = (int64_t)p.B * p.H * p.Sq;
   unsigned const gkv = (unsigned)(ceil_div(p.Skv, 128) * p.H * p.B);
   unsigned const gq = (unsigned)(ceil_div(p.Sq, 128) * p.H * p.B);
-#define CALL(DP_)                                                                                    \
-  do {                                                                                               \
-    attn_f32_delta_kernel<DP_><<<(unsigned)ceil_div(rows, 4 * (64 / (DP_ / 4))), 256, 0, st>>>(p);   \
-    attn_f32_bwd_dkdv_kernel<DP_><<<gkv, 256, 0, st>>>(p);                                           \
-    attn_f32_bwd_dq_kernel<DP_><<<gq, 256, 0, st>>>(p);                                              \
-  } while (0)
-  FFK_ATTN_F32_DISPATCH(p.D, CALL);
+  int const dmax = p.Dq > p.Dv ? p.Dq : p.Dv;
+#define CALL(DP_) launch_f32_backward<DP_>(st, p, rows, gkv, gq)
+  FFK_ATTN_F32_DISPATCH(dmax, CALL);
 #undef CALL
   FFK_CHECK_LAUNCH();
   return FFK_OK;

@@ -5,11 +5,13 @@
 //
 // Weight blob: [ W_Q | W_K | W_V | W_O ] with W_Q = [heads*qProj, qSize]
 // (head-major rows), W_K = [heads*kProj, kSize], W_V = [heads*vProj, vSize],
-// W_O = [oProj, heads*vProj], all row-major.  When query, key and value are
-// the same tensor the three input projections run as one GEMM against the
-// contiguous [3*heads*proj, size] block and the core reads the fused buffer
-// through strides.  FLOAT (the reference's data type) and BF16; the core is
-// attention_f32.hip / attention.hip.
+// W_O = [oProj, heads*vProj], all row-major.  qProj = kProj (the reference
+// asserts it, src/cuda/ops/attention_kernels.cu:61); vProj is free.  When
+// query, key and value are the same tensor the three input projections run as
+// one GEMM against the contiguous [heads*(2*qProj + vProj), size] block and the
+// core reads the fused buffer through strides.  FLOAT (the reference's data
+// type) and BF16; the core is attention_f32.hip / attention.hip /
+// attention_gen.hip.
 //
 // Reserve space layout (bytes, each region 256-byte aligned):
 //   QKV projections | context | lse | delta | d(context) | d(QKV projections)
@@ -56,24 +58,20 @@ static int check_mha(char const *who, int dtype, ffk_mha_desc_t const *d) {
                   d->v_size > 0 && d->o_proj_size > 0 && d->qo_seq_length > 0 && d->kv_seq_length > 0,
               "%s: non-positive size", who);
   FFK_REQUIRE(d->q_proj_size == d->k_proj_size, "%s: qProjSize must equal kProjSize", who);
-  FFK_REQUIRE(d->v_proj_size == d->q_proj_size,
-              "%s: vProjSize != qProjSize is not supported by the fused core", who);
-  if (dtype == FFK_BF16) {
-    FFK_REQUIRE(d->q_proj_size == 64 || d->q_proj_size == 128,
-                "%s: bf16 projection size %lld not supported (64 or 128)", who, (long long)d->q_proj_size);
-  } else {
-    FFK_REQUIRE(d->q_proj_size <= 128 && d->q_proj_size % 4 == 0,
-                "%s: fp32 projection size %lld not supported (a multiple of 4 up to 128)", who,
-                (long long)d->q_proj_size);
-  }
+  FFK_REQUIRE(d->q_proj_size > 0 && d->v_proj_size > 0, "%s: non-positive projection size", who);
+  int64_t const unit = dtype == FFK_BF16 ? 8 : 4;
+  FFK_REQUIRE(d->q_proj_size <= 256 && d->q_proj_size % unit == 0 && d->v_proj_size <= 256 &&
+                  d->v_proj_size % unit == 0,
+              "%s: projection size %lld / %lld not supported (multiples of %lld up to 256)", who,
+              (long long)d->q_proj_size, (long long)d->v_proj_size, (long long)unit);
   return FFK_OK;
 }
 
 // The reserve layout depends on the descriptor alone, so a backward call finds
 // what the forward call wrote whatever the caller's pointers are: with equal
 // input widths and sequence lengths the three projections are the column
-// blocks of ONE [tokens, 3*heads*proj] buffer (the core reads them through
-// strides), otherwise three dense tensors one after the other.
+// blocks of ONE [tokens, heads*(2*qProj + vProj)] buffer (the core reads them
+// through strides), otherwise three dense tensors one after the other.
 static bool is_interleaved(ffk_mha_desc_t const *d) {
   return d->q_size == d->k_size && d->k_size == d->v_size && d->qo_seq_length == d->kv_seq_length;
 }
@@ -83,19 +81,22 @@ static bool is_aliased(ffk_mha_desc_t const *d, void const *q, void const *k, vo
 }
 
 static ffk_attention_desc_t core_desc(ffk_mha_desc_t const *d, bool fused) {
-  int64_t const H = d->num_heads, D = d->q_proj_size;
+  int64_t const H = d->num_heads, Dq = d->q_proj_size, Dv = d->v_proj_size;
   ffk_attention_desc_t a;
   a.batch = d->num_samples;
   a.heads = H;
   a.seq_q = d->qo_seq_length;
   a.seq_kv = d->kv_seq_length;
-  a.head_dim = D;
-  int64_t const row = fused ? 3 * H * D : H * D;
-  a.q_seq_stride = a.k_seq_stride = a.v_seq_stride = row;
-  a.q_batch_stride = d->qo_seq_length * row;
-  a.k_batch_stride = a.v_batch_stride = d->kv_seq_length * row;
-  a.o_seq_stride = H * D;
-  a.o_batch_stride = d->qo_seq_length * H * D;
+  a.head_dim = Dq;
+  a.v_head_dim = Dv;
+  int64_t const row = H * (2 * Dq + Dv);
+  a.q_seq_stride = a.k_seq_stride = fused ? row : H * Dq;
+  a.v_seq_stride = fused ? row : H * Dv;
+  a.q_batch_stride = d->qo_seq_length * a.q_seq_stride;
+  a.k_batch_stride = d->kv_seq_length * a.k_seq_stride;
+  a.v_batch_stride = d->kv_seq_length * a.v_seq_stride;
+  a.o_seq_stride = H * Dv;
+  a.o_batch_stride = d->qo_seq_length * H * Dv;
   a.scale = d->scale;
   a.causal = d->causal;
   return a;
@@ -133,30 +134,30 @@ extern "C" int ffk_mha_forward(ffk_stream_t stream, int dtype,
   hipStream_t st = as_stream(stream);
   uint8_t *rs = static_cast<uint8_t *>(reserve);
   uint8_t const *w = static_cast<uint8_t const *>(weight);
-  int64_t const H = d->num_heads, D = d->q_proj_size, HD = H * D;
+  int64_t const H = d->num_heads, HDq = H * d->q_proj_size, HDv = H * d->v_proj_size;
+  int64_t const row = 2 * HDq + HDv;  // the interleaved buffer's row: [ Q | K | V ]
   bool const fused = is_interleaved(d);
   uint8_t *qkv = rs + L.off_qkv;
   GemmEpilogue ep;
   void const *qp, *kp, *vp;
   if (is_aliased(d, query, key, value)) {
-    // [T, 3HD] = X . [W_Q; W_K; W_V]^T
-    rc = gemm_dispatch(st, dtype, false, true, L.TQ, 3 * HD, d->q_size, query, d->q_size,
-                       w + L.wq * es, d->q_size, qkv, 3 * HD, ep);
+    // [T, row] = X . [W_Q; W_K; W_V]^T
+    rc = gemm_dispatch(st, dtype, false, true, L.TQ, row, d->q_size, query, d->q_size,
+                       w + L.wq * es, d->q_size, qkv, row, ep);
     if (rc != FFK_OK) return rc;
     qp = qkv;
-    kp = qkv + HD * es;
-    vp = qkv + 2 * HD * es;
+    kp = qkv + HDq * es;
+    vp = qkv + 2 * HDq * es;
   } else {
-    uint8_t *Q = qkv, *K = fused ? qkv + HD * es : qkv + L.nQ * es, *V = fused ? qkv + 2 * HD * es : K + L.nK * es;
-    int64_t const ld = fused ? 3 * HD : HD;
-    rc = gemm_dispatch(st, dtype, false, true, L.TQ, HD, d->q_size, query, d->q_size,
-                       w + L.wq * es, d->q_size, Q, ld, ep);
+    uint8_t *Q = qkv, *K = fused ? qkv + HDq * es : qkv + L.nQ * es, *V = fused ? qkv + 2 * HDq * es : K + L.nK * es;
+    rc = gemm_dispatch(st, dtype, false, true, L.TQ, HDq, d->q_size, query, d->q_size,
+                       w + L.wq * es, d->q_size, Q, fused ? row : HDq, ep);
     if (rc != FFK_OK) return rc;
-    rc = gemm_dispatch(st, dtype, false, true, L.TK, HD, d->k_size, key, d->k_size,
-                       w + L.wk * es, d->k_size, K, ld, ep);
+    rc = gemm_dispatch(st, dtype, false, true, L.TK, HDq, d->k_size, key, d->k_size,
+                       w + L.wk * es, d->k_size, K, fused ? row : HDq, ep);
     if (rc != FFK_OK) return rc;
-    rc = gemm_dispatch(st, dtype, false, true, L.TK, HD, d->v_size, value, d->v_size,
-                       w + L.wv * es, d->v_size, V, ld, ep);
+    rc = gemm_dispatch(st, dtype, false, true, L.TK, HDv, d->v_size, value, d->v_size,
+                       w + L.wv * es, d->v_size, V, fused ? row : HDv, ep);
     if (rc != FFK_OK) return rc;
     qp = Q; kp = K; vp = V;
   }
@@ -164,9 +165,9 @@ extern "C" int ffk_mha_forward(ffk_stream_t stream, int dtype,
   rc = ffk_attention_forward(stream, dtype, &a, qp, kp, vp, rs + L.off_ctx,
                              reinterpret_cast<float *>(rs + L.off_lse));
   if (rc != FFK_OK) return rc;
-  // output[T, oProj] = context[T, HD] . W_O[oProj, HD]^T
-  return gemm_dispatch(st, dtype, false, true, L.TQ, d->o_proj_size, HD, rs + L.off_ctx, HD,
-                       w + L.wo * es, HD, output, d->o_proj_size, ep);
+  // output[T, oProj] = context[T, H*vProj] . W_O[oProj, H*vProj]^T
+  return gemm_dispatch(st, dtype, false, true, L.TQ, d->o_proj_size, HDv, rs + L.off_ctx, HDv,
+                       w + L.wo * es, HDv, output, d->o_proj_size, ep);
 }
 
 extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
@@ -190,7 +191,8 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
   uint8_t *rs = static_cast<uint8_t *>(reserve);
   uint8_t const *w = static_cast<uint8_t const *>(weight);
   uint8_t *dw = static_cast<uint8_t *>(weight_grad);
-  int64_t const H = d->num_heads, D = d->q_proj_size, HD = H * D;
+  int64_t const H = d->num_heads, HDq = H * d->q_proj_size, HDv = H * d->v_proj_size;
+  int64_t const row = 2 * HDq + HDv;  // the interleaved buffers' row: [ Q | K | V ]
   bool const fused = is_interleaved(d);
   bool const aliased = is_aliased(d, query, key, value);
   // one tensor, three roles: its gradient is the sum of the three, which needs
@@ -205,17 +207,17 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
   in_ep.accumulate = (accumulate & FFK_MHA_ACC_INPUT_GRADS) != 0;
 
   // d(context) = dOut . W_O ; dW_O += dOut^T . context
-  rc = gemm_dispatch(st, dtype, false, false, L.TQ, HD, d->o_proj_size, output_grad,
-                     d->o_proj_size, w + L.wo * es, HD, dctx, HD, over);
+  rc = gemm_dispatch(st, dtype, false, false, L.TQ, HDv, d->o_proj_size, output_grad,
+                     d->o_proj_size, w + L.wo * es, HDv, dctx, HDv, over);
   if (rc != FFK_OK) return rc;
   // The two weight gradients of a self-attention block (output projection and
   // folded Q/K/V projection) have the same reduction length and each leaves
   // part of the chip idle: where the library can, they run as ONE launch after
   // the core's backward.
   bool const folded = aliased && key_grad == nullptr && value_grad == nullptr;
-  GemmProblem const wo_grad = {d->o_proj_size, HD, output_grad, d->o_proj_size, ctx, HD,
-                               dw != nullptr ? dw + L.wo * es : nullptr, HD};
-  GemmProblem const wqkv_grad = {3 * HD, d->q_size, dqkv, 3 * HD, query, d->q_size,
+  GemmProblem const wo_grad = {d->o_proj_size, HDv, output_grad, d->o_proj_size, ctx, HDv,
+                               dw != nullptr ? dw + L.wo * es : nullptr, HDv};
+  GemmProblem const wqkv_grad = {row, d->q_size, dqkv, row, query, d->q_size,
                                  dw != nullptr ? dw + L.wq * es : nullptr, d->q_size};
   bool const paired = dw != nullptr && folded && gemm_pair_supported(dtype, true, false, L.TQ, wqkv_grad, wo_grad);
   if (dw != nullptr && !paired) {
@@ -224,23 +226,20 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
     GemmEpilogue acc_o = acc;
     acc_o.splitk_ws = dqkv;
     acc_o.splitk_ws_bytes = L.total - L.off_dqkv;
-    rc = gemm_dispatch(st, dtype, true, false, d->o_proj_size, HD, L.TQ, output_grad,
-                       d->o_proj_size, ctx, HD, dw + L.wo * es, HD, acc_o);
+    rc = gemm_dispatch(st, dtype, true, false, d->o_proj_size, HDv, L.TQ, output_grad,
+                       d->o_proj_size, ctx, HDv, dw + L.wo * es, HDv, acc_o);
     if (rc != FFK_OK) return rc;
   }
 
   ffk_attention_desc_t a = core_desc(d, fused);
   void const *qp, *kp, *vp;
   void *dqp, *dkp, *dvp;
-  int64_t ld;
   if (fused) {
-    qp = qkv; kp = qkv + HD * es; vp = qkv + 2 * HD * es;
-    dqp = dqkv; dkp = dqkv + HD * es; dvp = dqkv + 2 * HD * es;
-    ld = 3 * HD;
+    qp = qkv; kp = qkv + HDq * es; vp = qkv + 2 * HDq * es;
+    dqp = dqkv; dkp = dqkv + HDq * es; dvp = dqkv + 2 * HDq * es;
   } else {
     qp = qkv; kp = qkv + L.nQ * es; vp = qkv + (L.nQ + L.nK) * es;
     dqp = dqkv; dkp = dqkv + L.nQ * es; dvp = dqkv + (L.nQ + L.nK) * es;
-    ld = HD;
   }
   // The core writes dQ/dK/dV with the same strides it reads Q/K/V with.
   rc = ffk_attention_backward(stream, dtype, &a, qp, kp, vp, ctx, dctx,
@@ -249,9 +248,9 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
   if (rc != FFK_OK) return rc;
 
   if (folded) {
-    // dX (+)= dQKV[T,3HD] . [W_Q; W_K; W_V]  and  dW_QKV += dQKV^T . X
+    // dX (+)= dQKV[T,row] . [W_Q; W_K; W_V]  and  dW_QKV += dQKV^T . X
     if (query_grad != nullptr) {
-      rc = gemm_dispatch(st, dtype, false, false, L.TQ, d->q_size, 3 * HD, dqkv, 3 * HD,
+      rc = gemm_dispatch(st, dtype, false, false, L.TQ, d->q_size, row, dqkv, row,
                          w + L.wq * es, d->q_size, query_grad, d->q_size, in_ep);
       if (rc != FFK_OK) return rc;
     }
@@ -259,21 +258,22 @@ extern "C" int ffk_mha_backward(ffk_stream_t stream, int dtype,
       return gemm_dispatch_pair(st, dtype, true, false, L.TQ, wqkv_grad, wo_grad, acc.accumulate);
     }
     if (dw != nullptr) {
-      rc = gemm_dispatch(st, dtype, true, false, 3 * HD, d->q_size, L.TQ, dqkv, 3 * HD, query,
+      rc = gemm_dispatch(st, dtype, true, false, row, d->q_size, L.TQ, dqkv, row, query,
                          d->q_size, dw + L.wq * es, d->q_size, acc);
       if (rc != FFK_OK) return rc;
     }
     return FFK_OK;
   }
   struct Part {
-    void const *x; void *dx; void const *dp; int64_t T, size, woff;
+    void const *x; void *dx; void const *dp; int64_t T, size, woff, HD;
   } parts[3] = {
-      {query, query_grad, dqp, L.TQ, d->q_size, L.wq},
-      {key, key_grad, dkp, L.TK, d->k_size, L.wk},
-      {value, value_grad, dvp, L.TK, d->v_size, L.wv},
+      {query, query_grad, dqp, L.TQ, d->q_size, L.wq, HDq},
+      {key, key_grad, dkp, L.TK, d->k_size, L.wk, HDq},
+      {value, value_grad, dvp, L.TK, d->v_size, L.wv, HDv},
   };
   for (int i = 0; i < 3; i++) {
     Part const &pt = parts[i];
+    int64_t const HD = pt.HD, ld = fused ? row : HD;
     if (pt.dx != nullptr) {
       rc = gemm_dispatch(st, dtype, false, false, pt.T, pt.size, HD, pt.dp, ld,
                          w + pt.woff * es, pt.size, pt.dx, pt.size, in_ep);

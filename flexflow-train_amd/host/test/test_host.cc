@@ -1258,6 +1258,90 @@ static void gpu_tests() {
     }
   });
 
+  // The encoder layer of the reference's transformer builder with its default configuration
+  // (lib/models/src/models/transformer/transformer.cc:6-16,32-67): 512 features, 8 heads,
+  // kdim = vdim = dim_feedforward / num_heads = 256, feed-forward 2048 with ReLU, dropout 0.1,
+  // LayerNorm after each residual add.  FLOAT (the reference's data type) and BF16.
+  run("The reference's default transformer encoder layer (512 features, 8 heads x 256, FFN 2048): steps, fused = unfused, loss falls", [&] {
+    int64_t const B = 2, S = 40, E = 512, FF = 2048;
+    int const H = 8, KD = (int)(FF / H);
+    float const rate = 0.1f, eps = 1e-5f;
+    for (DataType type : {DataType::FLOAT, DataType::BF16}) {
+      tensor_guid_t x, out;
+      auto build = [&](ComputationGraphBuilder &cgb) {
+        x = cgb.create_input(shape({B, S, E}, type), CreateGrad::YES);
+        tensor_guid_t attn = cgb.multihead_attention(x, x, x, (int)E, H, KD, KD, rate, false);
+        tensor_guid_t n1 = cgb.layer_norm(cgb.add(attn, x), {-1}, true, eps);
+        tensor_guid_t ff1 = cgb.dropout(cgb.dense(n1, (int)FF, Activation::RELU, true), rate);
+        tensor_guid_t ff2 = cgb.dropout(cgb.dense(ff1, (int)E, std::nullopt, true), rate);
+        tensor_guid_t n2 = cgb.layer_norm(cgb.add(n1, ff2), {-1}, true, eps);
+        out = type == DataType::FLOAT ? n2 : cgb.cast(n2, DataType::FLOAT);
+      };
+      device_id_t dev = make_device_id_t_from_idx(0, DeviceType::GPU);
+      auto label = random_vec(B * S * E, 401);
+      auto LABEL = device_accessor(gpu, shape({B, S, E}, DataType::FLOAT), label);
+      auto loss_of = [&](std::vector<float> const &o) {
+        double l = 0;
+        for (size_t i = 0; i < o.size(); i++) l += ((double)o[i] - label[i]) * ((double)o[i] - label[i]);
+        return l / (double)o.size();
+      };
+      std::vector<std::vector<float>> results[2];
+      std::vector<double> losses;
+      for (int unfused = 0; unfused < 2; unfused++) {
+        ComputationGraphBuilder cgb;
+        build(cgb);
+        // the attention layer's weight has the reference's element count (attention.cc:165-185)
+        if (unfused) ffk_set_option(FFK_OPTION_LAYER_UNFUSED, 1);
+        ComputationGraphInstance inst = create_computation_graph_instance(
+            cgb.computation_graph, OptimizerAttrs{SGDOptimizerAttrs{0.05, 0.9, false, 0.0}},
+            LossConfig{NonconfigurableLossAttrs{LossFunction::MEAN_SQUARED_ERROR_AVG_REDUCE}, LABEL, out}, {}, gpu,
+            ProfilingSettings{0, 0}, handle, dev);
+        if (unfused) ffk_set_option(FFK_OPTION_LAYER_UNFUSED, 0);
+        std::vector<tensor_guid_t> ws;
+        unsigned seed = 500;
+        for (size_t t = 0; t < cgb.computation_graph.tensors.size(); t++) {
+          tensor_guid_t g{(int)t};
+          auto const &src = cgb.computation_graph.layers.at(cgb.computation_graph.tensors[t].source.raw);
+          bool const weight = std::holds_alternative<WeightAttrs>(src.attrs.op_attrs);
+          if (!weight && !(g == x)) continue;
+          if (weight) ws.push_back(g);
+          TensorShape ts = cgb.computation_graph.tensors[t].shape;
+          bool const vec = weight && ts.dims.ff_ordered.size() == 1 && get_num_elements(ts.dims) <= FF;
+          auto host = g == x ? random_vec((size_t)get_num_elements(ts.dims), seed++)
+                             : random_vec((size_t)get_num_elements(ts.dims), seed++, vec ? 0.5f : -0.05f, vec ? 1.5f : 0.05f);
+          copy_accessor_data_to_l_from_r(inst.get_tensor_accessor(g), device_accessor(gpu, ts, host));
+        }
+        if (!unfused) {
+          // 3 * (512 * 256) * 8 + 512 * 256 * 8 elements
+          size_t attn_w = 0;
+          for (tensor_guid_t w : ws) attn_w = std::max(attn_w, (size_t)get_num_elements(cgb.computation_graph.tensors[w.raw].shape.dims));
+          CHECK(attn_w == (size_t)(4 * E * KD * H));
+        }
+        for (int step = 0; step < (unfused ? 3 : 6); step++) {
+          perform_all_passes_for_computation_graph_instance(inst, ProfilingSettings{0, 0}, handle, dev);
+          if (step == 2) {
+            results[unfused].push_back(to_host(inst.get_tensor_accessor(out)));
+            results[unfused].push_back(to_host(*inst.get_gradient_accessor(x)));
+            for (tensor_guid_t w : ws) results[unfused].push_back(to_host(inst.get_tensor_accessor(w)));
+          }
+          if (!unfused) losses.push_back(loss_of(to_host(inst.get_tensor_accessor(out))));
+        }
+      }
+      CHECK(results[0].size() == results[1].size() && results[0].size() == 11);
+      for (size_t i = 0; i < results[0].size(); i++) {
+        CHECK(contains_non_zero(results[0][i]));
+        bool finite = true;
+        for (float v : results[0][i]) finite = finite && std::isfinite(v);
+        CHECK(finite);
+        CHECK(results[0][i] == results[1][i]);
+      }
+      CHECK(losses.size() == 6 && std::isfinite(losses[5]));
+      CHECK(losses[5] < losses[0]);
+      printf("    %s loss per step: %.4f %.4f %.4f %.4f %.4f %.4f\n", type == DataType::FLOAT ? "fp32" : "bf16", losses[0],
+             losses[1], losses[2], losses[3], losses[4], losses[5]);
+    }
+  });
+
   // Token embedding -> encoder layer -> vocabulary projection -> softmax -> sparse cross entropy:
   // the shape of the reference's BERT builder (lib/models/src/models/bert/bert.cc) at toy size.
   // Two instances, one created with one kernel per operator: the planner's fusions must not change

@@ -539,12 +539,16 @@ int ffk_embedding_backward(ffk_stream_t stream, int index_dtype,
 /* Fused (flash-style) scaled-dot-product attention core: the QK^T / softmax /
  * PV contraction that cudnnMultiHeadAttnForward/BackwardData perform inside
  * lib/kernels/src/cuda/ops/attention_kernels.cu:224,261, without the S x S
- * score matrix ever reaching HBM.  dtype FFK_BF16 (head_dim 64 or 128, strides
- * multiples of 8) or FFK_FLOAT (the reference's data type; head_dim any
- * multiple of 4 up to 128, strides multiples of 4).
+ * score matrix ever reaching HBM.  dtype FFK_BF16 (head sizes multiples of 8
+ * up to 256, strides multiples of 8; 64 and 128 with v_head_dim = head_dim run
+ * the tuned kernels) or FFK_FLOAT (the reference's data type; head sizes
+ * multiples of 4 up to 256, strides multiples of 4).  q and k have head_dim
+ * columns per head, v and o have v_head_dim (qProjSize / vProjSize of
+ * lib/kernels/src/cuda/ops/attention_kernels.cu:78-80; the reference's model
+ * builders use 256 for both, lib/models/src/models/transformer/transformer.cc:37-38).
  *   q,k,v,o: element (b, s, h, d) at  b*batch_stride + s*seq_stride +
- *   h*head_dim + d  (strides in elements), so the same kernel reads the
- *   [batch, seq, heads*head_dim] projections and a fused QKV buffer.
+ *   h*(head_dim or v_head_dim) + d  (strides in elements), so the same kernel
+ *   reads the [batch, seq, heads*head_dim] projections and a fused QKV buffer.
  *   lse [batch, heads, seq_q] fp32: log-sum-exp of the scaled scores, written
  *   by forward and read by backward.  scale multiplies QK^T (the reference
  *   uses 1.0, attention_kernels.cu:76); causal != 0 masks key index > query
@@ -559,6 +563,7 @@ typedef struct {
   int64_t o_batch_stride, o_seq_stride;
   float scale;
   int causal;
+  int64_t v_head_dim; /* head size of v, o (and their gradients); 0 = head_dim */
 } ffk_attention_desc_t;
 
 int ffk_attention_forward(ffk_stream_t stream, int dtype,
@@ -576,8 +581,11 @@ int ffk_attention_backward(ffk_stream_t stream, int dtype,
  * lib/kernels/src/cuda/ops/attention_kernels.cu:215-303).
  *   query [B,Sq,qSize], key [B,Skv,kSize], value [B,Skv,vSize],
  *   output [B,Sq,oProjSize].  No bias, no dropout (attention_kernels.cu:73-92).
- *   dtype FFK_FLOAT (the reference's) or FFK_BF16.  q/k/v_proj_size must be
- *   equal: FLOAT any multiple of 4 up to 128, BF16 64 or 128.
+ *   dtype FFK_FLOAT (the reference's) or FFK_BF16.  q_proj_size must equal
+ *   k_proj_size (the reference asserts it, attention_kernels.cu:61);
+ *   v_proj_size is free.  FLOAT: multiples of 4 up to 256; BF16: multiples of
+ *   8 up to 256 (the reference's model builders use 256,
+ *   lib/models/src/models/transformer/transformer.cc:37-38, bert/bert.cc:64-65).
  *   weight blob (defined by this library; the reference never indexes it):
  *     [ W_Q | W_K | W_V | W_O ], W_Q = [heads*qProj, qSize] row-major with
  *     head-major rows (likewise W_K [heads*kProj, kSize], W_V [heads*vProj,

@@ -16,23 +16,33 @@ def say(*a):
     sys.stdout.flush()
 
 
-SHAPES = [  # B, H, Sq, Skv, D
+SHAPES = [  # B, H, Sq, Skv, D (, Dv)
     (1, 1, 8, 8, 64), (2, 3, 11, 11, 64), (1, 2, 100, 100, 128), (2, 2, 129, 129, 64),
     (1, 4, 256, 256, 128), (1, 2, 300, 300, 64), (1, 1, 64, 200, 64), (2, 1, 160, 96, 128),
+    # the head size of the reference's transformer and BERT builders (transformer.cc:37-38, bert.cc:64-65)
+    (1, 2, 70, 70, 256), (2, 2, 129, 200, 256), (1, 1, 300, 300, 256),
+    # a value head size of its own (vdim != kdim), and head sizes that are no power of two
+    (1, 2, 100, 100, 64, 128), (2, 1, 129, 96, 128, 64), (1, 2, 40, 72, 256, 64), (1, 1, 65, 65, 64, 256),
+    (1, 2, 50, 50, 32), (1, 2, 90, 130, 96), (1, 3, 33, 33, 40, 72), (1, 1, 140, 140, 200, 8),
 ]
+
+
+def _dv(shape):
+    return shape[5] if len(shape) > 5 else shape[4]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
 @pytest.mark.parametrize("causal", [False, True])
 def test_attention_core(ffk, oracle, shape, causal):
     # causal with Sq != Skv: key j is visible to query i iff j <= i (the mask is aligned top-left)
-    B, H, Sq, Skv, D = shape
+    B, H, Sq, Skv, D = shape[:5]
+    Dv = _dv(shape)
     say("attention core", shape, "causal", causal)
     g = rng(Sq * 7 + D + int(causal))
     q = bf16_round(g.standard_normal((B, Sq, H, D)))
     k = bf16_round(g.standard_normal((B, Skv, H, D)))
-    v = bf16_round(g.standard_normal((B, Skv, H, D)))
-    do = bf16_round(g.standard_normal((B, Sq, H, D)))
+    v = bf16_round(g.standard_normal((B, Skv, H, Dv)))
+    do = bf16_round(g.standard_normal((B, Sq, H, Dv)))
     scale = 1.0 / np.sqrt(D)
     o_ref, lse_ref = oracle.attention_forward(q, k, v, scale, causal, bf16_mode=True)
     qd, kd, vd, dod = (to_dev(a, torch, BT) for a in (q, k, v, do))
@@ -128,9 +138,11 @@ def test_attention_forward_growing_scores(ffk, oracle, causal):
     assert_close(to_np(lse), lse_ref, 1e-3, "lse")
 
 
-F32_SHAPES = [  # B, H, Sq, Skv, D
+F32_SHAPES = [  # B, H, Sq, Skv, D (, Dv)
     (1, 1, 8, 8, 64), (2, 3, 11, 11, 32), (1, 2, 100, 100, 128), (2, 2, 129, 129, 64), (1, 2, 40, 40, 4),
     (1, 4, 256, 256, 128), (1, 2, 300, 300, 48), (1, 1, 64, 200, 64), (2, 1, 160, 96, 100), (1, 3, 70, 33, 20),
+    (1, 2, 70, 70, 256), (2, 2, 129, 200, 256), (1, 1, 200, 140, 132),
+    (1, 2, 100, 100, 64, 128), (2, 1, 129, 96, 128, 36), (1, 2, 40, 72, 256, 64), (1, 1, 65, 65, 16, 256),
 ]
 
 
@@ -138,11 +150,12 @@ F32_SHAPES = [  # B, H, Sq, Skv, D
 @pytest.mark.parametrize("causal", [False, True])
 def test_attention_core_fp32(ffk, oracle, shape, causal):
     """The fp32 core behind the reference's float MultiHeadAttention signature."""
-    B, H, Sq, Skv, D = shape
+    B, H, Sq, Skv, D = shape[:5]
+    Dv = _dv(shape)
     say("attention core fp32", shape, "causal", causal)
     g = rng(Sq * 5 + D + int(causal))
     q, k, v, do = (g.standard_normal(s).astype(np.float32)
-                   for s in ((B, Sq, H, D), (B, Skv, H, D), (B, Skv, H, D), (B, Sq, H, D)))
+                   for s in ((B, Sq, H, D), (B, Skv, H, D), (B, Skv, H, Dv), (B, Sq, H, Dv)))
     scale = 1.0 / np.sqrt(D)
     o_ref, lse_ref = oracle.attention_forward(q, k, v, scale, causal, bf16_mode=False)
     qd, kd, vd, dod = (to_dev(a, torch) for a in (q, k, v, do))
@@ -206,10 +219,13 @@ def test_attention_strided_views(ffk, oracle):
 
 
 def test_attention_errors(ffk):
-    q = torch.zeros((1, 8, 1, 32), dtype=BT, device="cuda")
+    q = torch.zeros((1, 8, 2, 264), dtype=BT, device="cuda")
     with pytest.raises(ffk.FFKError, match="head_dim"):
         ffk.attention_forward(q, q, q, 1.0, False)
-    q32 = torch.zeros((1, 8, 1, 132), dtype=torch.float32, device="cuda")
+    q = torch.zeros((1, 8, 2, 36), dtype=BT, device="cuda")  # strides of 72 are fine, the head size is no multiple of 8
+    with pytest.raises(ffk.FFKError, match="head_dim"):
+        ffk.attention_forward(q, q, q, 1.0, False)
+    q32 = torch.zeros((1, 8, 1, 260), dtype=torch.float32, device="cuda")
     with pytest.raises(ffk.FFKError, match="head_dim"):
         ffk.attention_forward(q32, q32, q32, 1.0, False)
     q16 = torch.zeros((1, 8, 1, 64), dtype=torch.float16, device="cuda")
@@ -325,15 +341,24 @@ def test_mha_config5_block_causal_prefix(ffk, oracle):
     assert_close(to_np(dw3), to_np(dw2) + to_np(dw), BF16_RTOL, "weight gradient is linear in the upstream gradient")
 
 
-MHA_CASES = [  # B, Sq, Skv, H, E(q), Ek, Ev, Dh, oProj, self-attention?
+MHA_CASES = [  # B, Sq, Skv, H, E(q), Ek, Ev, Dh, oProj, self-attention? (, vProj)
     (2, 20, 20, 4, 64, 64, 64, 64, 64, True),
     (2, 33, 33, 2, 128, 128, 128, 64, 96, True),
     (1, 24, 40, 2, 64, 72, 80, 64, 64, False),
     (2, 64, 64, 2, 256, 256, 256, 128, 256, True),
     (2, 64, 64, 12, 768, 768, 768, 64, 768, True),  # both weight gradients in one two-problem GEMM launch
     (2, 24, 24, 2, 64, 64, 64, 64, 64, False),      # three tensors of one shape: one interleaved projection buffer
+    # the reference's default transformer layer: 512 features, 8 heads, kdim = vdim = 2048 / 8 = 256
+    # (lib/models/src/models/transformer/transformer.cc:37-38)
+    (2, 40, 40, 8, 512, 512, 512, 256, 512, True),
+    (1, 24, 40, 2, 64, 72, 80, 256, 64, False),
+    # vdim != kdim (lib/op-attrs/src/op-attrs/ops/attention.cc:23-37 leaves both free)
+    (2, 33, 33, 2, 128, 128, 128, 64, 96, True, 128),
+    (2, 24, 24, 2, 64, 64, 64, 128, 64, False, 64),
+    (1, 24, 40, 2, 64, 72, 80, 64, 64, False, 256),
+    (2, 20, 20, 3, 96, 96, 96, 40, 96, True, 24),
 ]
-MHA_CASES_FP32 = MHA_CASES[:4] + [
+MHA_CASES_FP32 = MHA_CASES[:4] + MHA_CASES[6:] + [
     (2, 20, 20, 4, 64, 64, 64, 16, 64, True),   # head sizes the bf16 core does not take
     (1, 24, 40, 2, 64, 72, 80, 40, 56, False),
     (2, 24, 24, 2, 64, 64, 64, 32, 64, False),
@@ -341,7 +366,8 @@ MHA_CASES_FP32 = MHA_CASES[:4] + [
 
 
 def _mha_case(ffk, oracle, case, causal, fp32):
-    B, Sq, Skv, H, E, Ek, Ev, Dh, oP, self_attn = case
+    B, Sq, Skv, H, E, Ek, Ev, Dh, oP, self_attn = case[:10]
+    Dv = case[10] if len(case) > 10 else Dh
     say("mha", "fp32" if fp32 else "bf16", case, "causal", causal)
     BT, BF16_RTOL, dtype = (torch.float32, FP32_RTOL, ffk.FLOAT) if fp32 else (torch.bfloat16, 2e-2, ffk.BF16)
     bf16_round = (lambda a: np.asarray(a, dtype=np.float32)) if fp32 else globals()["bf16_round"]
@@ -350,10 +376,10 @@ def _mha_case(ffk, oracle, case, causal, fp32):
     query = bf16_round(g.standard_normal((B, Sq, E)))
     key = query if self_attn else bf16_round(g.standard_normal((B, Skv, Ek)))
     value = query if self_attn else bf16_round(g.standard_normal((B, Skv, Ev)))
-    odesc = oracle.mha_desc(B, H, E, Ek, Ev, Dh, Dh, Dh, oP, Sq, Skv, scale, causal)
-    desc = ffk.mha_desc(B, H, E, Ek, Ev, Dh, Dh, Dh, oP, Sq, Skv, scale, causal)
+    odesc = oracle.mha_desc(B, H, E, Ek, Ev, Dh, Dh, Dv, oP, Sq, Skv, scale, causal)
+    desc = ffk.mha_desc(B, H, E, Ek, Ev, Dh, Dh, Dv, oP, Sq, Skv, scale, causal)
     nw = ffk.lib().ffk_mha_weight_elements(desc)
-    assert nw == H * Dh * (E + Ek + Ev) + oP * H * Dh
+    assert nw == H * Dh * (E + Ek) + H * Dv * Ev + oP * H * Dv
     w = bf16_round(g.standard_normal((nw,)) * (2.0 / np.sqrt(E)))
     dout = bf16_round(g.standard_normal((B, Sq, oP)))
     out_ref = oracle.mha_forward(odesc, query, key, value, w, bf16_mode=not fp32)
@@ -450,10 +476,13 @@ def test_mha_errors(ffk):
     small = torch.zeros((16,), dtype=torch.uint8, device="cuda")
     with pytest.raises(ffk.FFKError, match="reserve"):
         ffk.mha_forward(desc, x, x, x, w, small)
-    bad = ffk.mha_desc(1, 2, 64, 64, 64, 48, 48, 48, 64, 8, 8)
+    bad = ffk.mha_desc(1, 2, 64, 64, 64, 44, 44, 44, 64, 8, 8)
     with pytest.raises(ffk.FFKError, match="projection size"):
         ffk.mha_forward(bad, x, x, x, w, ffk.mha_reserve(desc, ffk.BF16))
-    bad = ffk.mha_desc(1, 2, 64, 64, 64, 256, 256, 256, 64, 8, 8)
+    bad = ffk.mha_desc(1, 2, 64, 64, 64, 64, 128, 64, 64, 8, 8)
+    with pytest.raises(ffk.FFKError, match="qProjSize must equal kProjSize"):
+        ffk.mha_forward(bad, x, x, x, w, ffk.mha_reserve(desc, ffk.BF16))
+    bad = ffk.mha_desc(1, 2, 64, 64, 64, 260, 260, 260, 64, 8, 8)
     x32, w32 = x.float(), torch.zeros((ffk.lib().ffk_mha_weight_elements(bad),), dtype=torch.float32, device="cuda")
     with pytest.raises(ffk.FFKError, match="projection size"):
         ffk.mha_forward(bad, x32, x32, x32, w32, ffk.mha_reserve(bad, ffk.FLOAT))
