@@ -240,8 +240,9 @@ def time_dominant_kernel(ffk, torch, cfg, iters=50, calibration_copy=False):
     return dict(bound="mfma", achieved=flops / sec / 1e12, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
                 frac=flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                 traffic=dominant_kernel_traffic(),
-                kernel="gemm_bf16_pipe_kernel<256,256,128,128,64,2,1,false,true,0,false> "
-                       "(FFN up-projection, M%d N%d K%d, bias)" % (T, F, E),
+                # asked of the library's own dispatch for this shape, not written down here
+                kernel="%s (FFN up-projection, M%d N%d K%d, bias)"
+                       % (ffk.gemm_kernel_name(ffk.BF16, False, True, T, F, E, has_bias=True), T, F, E),
                 us_per_launch=us)
 
 

@@ -106,6 +106,7 @@ SIGNATURES = {
                                     c_i64, c_i64, c_i64, c_p, c_sz, c_int]),
     "ffk_linear_l2_regularizer_grad": (c_int, [c_p, c_int, c_p, c_p, c_i64, c_f]),
     "ffk_gemm": (c_int, [c_p, c_int, c_int, c_int, c_i64, c_i64, c_i64, c_p, c_p, c_p, c_int]),
+    "ffk_gemm_kernel_name": (c_int, [c_int, c_int, c_int, c_i64, c_i64, c_i64, c_int, c_int, ctypes.c_char_p, c_sz]),
     "ffk_element_unary_forward": (c_int, [c_p, c_int, c_int, c_f, c_p, c_p, c_i64]),
     "ffk_element_unary_backward": (c_int, [c_p, c_int, c_int, c_f, c_p, c_p, c_p, c_p, c_i64,
                                            c_int]),
@@ -288,6 +289,13 @@ def linear_backward(y, dy, x, w, dx=None, dw=None, db=None, activation=ACT_NONE,
                                     batch, in_dim, out_dim, ptr(workspace), ws_bytes,
                                     7 if accumulate is True else int(accumulate)))
     return dx, dw, db
+
+
+def gemm_kernel_name(dtype, trans_a, trans_b, M, N, K, has_bias=False, activation=ACT_NONE):
+    """The kernel (template instance) the GEMM dispatch picks for a dense problem; launches nothing."""
+    buf = ctypes.create_string_buffer(256)
+    check(lib().ffk_gemm_kernel_name(dtype, int(trans_a), int(trans_b), M, N, K, int(has_bias), activation, buf, 256))
+    return buf.value.decode()
 
 
 def linear_l2_regularizer_grad(w, dw, lam):

@@ -29,18 +29,9 @@ int fail(int code, char const *fmt, ...) {
   return code;
 }
 
-// Process-wide switches (ffk_set_option).  Each starts from its environment
-// variable, read once when the library is loaded; the dispatch paths read an
-// atomic int, never the environment.
-static int env_int(char const *name) {
-  char const *e = getenv(name);
-  return e != nullptr ? atoi(e) : 0;
-}
-static std::atomic<int> g_option[FFK_OPTION_COUNT] = {
-    {env_int("FFK_GEMM_VARIANT")},
-    {env_int("FFK_LAYER_UNFUSED")},
-    {env_int("FFK_ATTENTION_VARIANT")},
-};
+// Process-wide switches: changed by ffk_set_option only (nothing in the
+// library reads the environment), all 0 = the dispatch's own choices.
+static std::atomic<int> g_option[FFK_OPTION_COUNT] = {{0}, {0}, {0}};
 int option(int which) { return g_option[which].load(std::memory_order_relaxed); }
 
 // Zero fill as a kernel (not hipMemsetAsync) so that callers may capture the

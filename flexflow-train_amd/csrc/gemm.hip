@@ -15,6 +15,7 @@
 #include "lds_dma.h"
 #include "gemm.h"
 #include "colreduce.h"
+#include <stdarg.h>
 #include <stdlib.h>
 #include <type_traits>
 
@@ -60,6 +61,24 @@ __device__ __forceinline__ void tile_coords(int pid, int nbm, int nbn, int &tm,
   tm = first_m + in_group % rows;
   tn = in_group / rows;
 }
+
+// ---------------------------------------------------------------------------
+// Asking instead of launching: while this thread's name sink is set (by
+// ffk_gemm_kernel_name), every launch site below writes the kernel it would
+// have launched into the sink and returns without touching the device.
+// ---------------------------------------------------------------------------
+static thread_local char *tl_name_sink = nullptr;
+static thread_local size_t tl_name_sink_bytes = 0;
+static bool describe_only(char const *fmt, ...) __attribute__((format(printf, 1, 2)));
+static bool describe_only(char const *fmt, ...) {
+  if (tl_name_sink == nullptr) return false;
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(tl_name_sink, tl_name_sink_bytes, fmt, ap);
+  va_end(ap);
+  return true;
+}
+static char const *tf(bool b) { return b ? "true" : "false"; }
 
 // ---------------------------------------------------------------------------
 // bf16 MFMA kernel
@@ -937,6 +956,10 @@ static hipError_t launch_pipe(hipStream_t st, bf16 const *A, bf16 const *B,
                               int splits = 1) {
   using Cfg = PipeCfg<BM, BN, WM, WN, BK, STAGES>;
   constexpr int NT = Cfg::NW * 64;
+  if (describe_only("gemm_bf16_pipe_kernel<%d,%d,%d,%d,%d,%d,%d,%s,%s,%d,false>%s", BM, BN, WM, WN, BK, STAGES, PF,
+                    tf(TA), tf(TB), TAIL, splits > 1 ? " (split-K) + splitk_reduce_kernel" : "")) {
+    return hipSuccess;
+  }
   auto kern = gemm_bf16_pipe_kernel<BM, BN, WM, WN, BK, STAGES, PF, TA, TB, TAIL>;
   GemmTailArgs const tail = {static_cast<bf16 const *>(ep.tail_in), static_cast<bf16 *>(ep.tail_out),
                              ep.tail_dropout, ep.tail_colsum_partials};
@@ -1098,6 +1121,7 @@ static hipError_t launch_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   bool const edge = (M % BM) || (N % BN) || (K % kBK);
   bf16 const *bias = static_cast<bf16 const *>(ep.bias);
+  if (describe_only("gemm_bf16_kernel<%d,%d,%d,%d,%s,%s,%s>", BM, BN, WM, WN, tf(TA), tf(TB), tf(edge))) return hipSuccess;
   if (edge) {
     gemm_bf16_kernel<BM, BN, WM, WN, TA, TB, true><<<blocks, NT, 0, st>>>(
         A, B, C, M, N, K, lda, ldb, ldc, bias, ep.activation, ep.accumulate);
@@ -1488,6 +1512,7 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
   gemm_f32_kernel<TA_, TB_><<<blocks, 256, 0, st>>>(                           \
       a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, bias, ep.activation,     \
       ep.accumulate)
+    if (describe_only("gemm_f32_kernel<%s,%s>", tf(ta), tf(tb))) return FFK_OK;
     if (!ta && !tb) FFK_LAUNCH_F32(false, false);
     else if (!ta && tb) FFK_LAUNCH_F32(false, true);
     else if (ta && !tb) FFK_LAUNCH_F32(true, false);
@@ -1508,6 +1533,7 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
                   (tb || N % 8 == 0) && K > 0;
     if (!vec_ok) {
       int64_t total = M * N;
+      if (describe_only("gemm_bf16_plain_kernel")) return FFK_OK;
       gemm_bf16_plain_kernel<<<(unsigned)ceil_div(total, 256), 256, 0, st>>>(
           a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, ta, tb,
           static_cast<bf16 const *>(ep.bias), ep.activation, ep.accumulate);
@@ -1531,6 +1557,26 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
 }  // namespace ffk
 
 using namespace ffk;
+
+extern "C" int ffk_gemm_kernel_name(int dtype, int trans_a, int trans_b, int64_t M, int64_t N, int64_t K,
+                                    int has_bias, int activation, char *name, size_t name_bytes) {
+  FFK_REQUIRE(name != nullptr && name_bytes > 0, "gemm_kernel_name: no room for the name");
+  FFK_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_kernel_name: non-positive dimension");
+  name[0] = 0;
+  // dense, 16-byte aligned operands: the addresses only have to pass the alignment checks,
+  // nothing is launched while the sink is set
+  void *const somewhere = reinterpret_cast<void *>(uintptr_t(1) << 20);
+  GemmEpilogue ep;
+  ep.bias = has_bias ? somewhere : nullptr;
+  ep.activation = activation;
+  tl_name_sink = name;
+  tl_name_sink_bytes = name_bytes;
+  int const rc = gemm_dispatch(nullptr, dtype, trans_a != 0, trans_b != 0, M, N, K, somewhere, trans_a ? M : K,
+                               somewhere, trans_b ? K : N, somewhere, N, ep);
+  tl_name_sink = nullptr;
+  tl_name_sink_bytes = 0;
+  return rc;
+}
 
 extern "C" int ffk_gemm(ffk_stream_t stream, int dtype, int trans_a,
                         int trans_b, int64_t M, int64_t N, int64_t K,

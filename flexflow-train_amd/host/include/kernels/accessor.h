@@ -20,11 +20,22 @@ struct GenericTensorAccessorR {
   void const *ptr;
   DeviceType device_type;
 
-  float const *get_float_ptr() const { return typed<float>(DataType::FLOAT); }
-  int32_t const *get_int32_ptr() const { return typed<int32_t>(DataType::INT32); }
-  int64_t const *get_int64_ptr() const { return typed<int64_t>(DataType::INT64); }
+  // accessor.h:24-29: the typed pointer, after a check of the data type
+  template <DataType DT>
+  real_type_t<DT> const *get() const { return typed<real_type_t<DT>>(DT); }
+  float const *get_float_ptr() const { return get<DataType::FLOAT>(); }
+  double const *get_double_ptr() const { return get<DataType::DOUBLE>(); }
+  half const *get_half_ptr() const { return get<DataType::HALF>(); }
+  int32_t const *get_int32_ptr() const { return get<DataType::INT32>(); }
+  int64_t const *get_int64_ptr() const { return get<DataType::INT64>(); }
 
-  // Element access on a CPU-resident accessor (asserts residency and dtype).
+  // accessor.h:46-57: element access on a CPU-resident accessor (residency and data type checked)
+  template <DataType DT>
+  real_type_t<DT> const &at(TensorDimsCoord const &coord) const {
+    if (device_type != DeviceType::CPU) throw std::runtime_error("GenericTensorAccessorR::at() requires CPU-allocated tensor");
+    return get<DT>()[calculate_accessor_offset(coord, shape.dims)];
+  }
+  // the same by element type (any type of the data type's size)
   template <typename T>
   T const &at(TensorDimsCoord const &coord) const {
     if (device_type != DeviceType::CPU) throw std::runtime_error("at() requires a CPU accessor");
@@ -35,7 +46,7 @@ struct GenericTensorAccessorR {
  private:
   template <typename T>
   T const *typed(DataType want) const {
-    if (shape.data_type != want) throw std::runtime_error("accessor: invalid data type");
+    if (shape.data_type != want) throw std::runtime_error("accessor: Invalid datatype requested");
     return static_cast<T const *>(ptr);
   }
 };
@@ -46,9 +57,20 @@ struct GenericTensorAccessorW {
   DeviceType device_type;
 
   operator GenericTensorAccessorR() const { return GenericTensorAccessorR{shape, ptr, device_type}; }
-  float *get_float_ptr() const {
-    if (shape.data_type != DataType::FLOAT) throw std::runtime_error("accessor: invalid data type");
-    return static_cast<float *>(ptr);
+  template <DataType DT>
+  real_type_t<DT> *get() const {
+    if (shape.data_type != DT) throw std::runtime_error("accessor: Invalid datatype requested");
+    return static_cast<real_type_t<DT> *>(ptr);
+  }
+  float *get_float_ptr() const { return get<DataType::FLOAT>(); }
+  double *get_double_ptr() const { return get<DataType::DOUBLE>(); }
+  half *get_half_ptr() const { return get<DataType::HALF>(); }
+  int32_t *get_int32_ptr() const { return get<DataType::INT32>(); }
+  int64_t *get_int64_ptr() const { return get<DataType::INT64>(); }
+  template <DataType DT>
+  real_type_t<DT> &at(TensorDimsCoord const &coord) const {
+    if (device_type != DeviceType::CPU) throw std::runtime_error("GenericTensorAccessorW::at() requires CPU-allocated tensor");
+    return get<DT>()[calculate_accessor_offset(coord, shape.dims)];
   }
   template <typename T>
   T &at(TensorDimsCoord const &coord) const {

@@ -1,7 +1,9 @@
 // Allocator / IAllocator and the local CPU / device allocators (reference:
 // lib/kernels/include/kernels/allocation.h:10-42, local_cpu_allocator.h,
-// local_cuda_allocator.h; bodies lib/kernels/src/kernels/local_*_allocator.cc).
-// The device allocator keeps the reference's name so callers compile unchanged.
+// local_cuda_allocator.h, create_local_allocator_for_device_type.h,
+// copy_tensor_accessor.h; bodies lib/kernels/src/kernels/local_*_allocator.cc).
+// Headers under those reference names include this one.  The device allocator
+// keeps the reference's name so callers compile unchanged.
 #pragma once
 #include "kernels/accessor.h"
 #include <cstddef>
@@ -61,7 +63,12 @@ Allocator create_local_cpu_memory_allocator();
 Allocator create_local_cuda_memory_allocator();
 Allocator create_local_allocator_for_device_type(DeviceType);
 
+// copy_tensor_accessor.h:9-25: a fresh tensor from the allocator with the source's contents
+// (whatever side each lives on); the _to_cpu_if_necessary forms return the source itself when
+// it already is host-resident.
 GenericTensorAccessorW copy_tensor_accessor_w(GenericTensorAccessorW const &src, Allocator &allocator);
-GenericTensorAccessorR copy_tensor_accessor_r(GenericTensorAccessorR const &src, Allocator &allocator);
+GenericTensorAccessorW copy_tensor_accessor_r(GenericTensorAccessorR const &src, Allocator &allocator);
+GenericTensorAccessorR copy_tensor_accessor_r_to_cpu_if_necessary(GenericTensorAccessorR const &, Allocator &cpu_allocator);
+GenericTensorAccessorW copy_tensor_accessor_w_to_cpu_if_necessary(GenericTensorAccessorW const &, Allocator &cpu_allocator);
 
 }  // namespace FlexFlow

@@ -1,70 +1,4 @@
-// ElementUnary / ElementBinary entry points (reference:
-// lib/kernels/include/kernels/element_unary_kernels.h:13-39,
-// element_binary_kernels.h:16-51; states element_{unary,binary}_per_device_state.dtg.toml).
+// Both element-wise operator families in one include.
 #pragma once
-#include "kernels/accessor.h"
-#include "kernels/device_stream_t.h"
-#include "op-attrs/attrs.h"
-
-namespace FlexFlow {
-
-struct ElementUnaryPerDeviceState {
-  TensorShape input_shape, output_shape;
-  OperatorType op_type;
-};
-
-struct ElementBinaryPerDeviceState {
-  PerDeviceFFHandle handle;
-  OperatorType op_type;
-  bool should_broadcast_lhs, should_broadcast_rhs;
-  TensorShape lhs_shape, rhs_shape, output_shape;
-};
-
-namespace Kernels::ElementUnary {
-std::optional<ElementUnaryPerDeviceState> init_kernel(DeviceType device_type,
-                                                      TensorShape const &input_shape,
-                                                      TensorShape const &output_shape,
-                                                      ElementUnaryAttrs const &attrs);
-void forward_kernel(device_stream_t const &stream,
-                    std::optional<ElementUnaryPerDeviceState> const &device_state,
-                    ElementUnaryAttrs const &attrs, device_handle_t const &handle,
-                    GenericTensorAccessorR const &input, GenericTensorAccessorW const &output);
-void backward_kernel(device_stream_t const &stream,
-                     std::optional<ElementUnaryPerDeviceState> const &device_state,
-                     ElementUnaryAttrs const &attrs, device_handle_t const &handle,
-                     GenericTensorAccessorR const &output, GenericTensorAccessorR const &output_grad,
-                     GenericTensorAccessorR const &input, GenericTensorAccessorW const &input_grad);
-void cleanup_kernel(DeviceType device_type,
-                    std::optional<ElementUnaryPerDeviceState> &per_device_state);
-}  // namespace Kernels::ElementUnary
-
-namespace Kernels::ElementBinary {
-std::optional<ElementBinaryPerDeviceState> init_kernel(
-    DeviceType device_type, device_handle_t const &handle, OperatorType op_type,
-    bool should_broadcast_lhs, bool should_broadcast_rhs, TensorShape const &lhs_shape,
-    TensorShape const &rhs_shape, TensorShape const &output_shape);
-// fp32 pointers (the reference's signatures); gradients accumulate (beta = 1).
-void forward_kernel(device_stream_t const &stream,
-                    std::optional<ElementBinaryPerDeviceState> const &per_device_state,
-                    float const *lhs_ptr, float const *rhs_ptr, float *out_ptr,
-                    OperatorType op_type, bool broadcast_inputLHS, device_handle_t const &handle);
-void backward_kernel(device_stream_t const &stream,
-                     std::optional<ElementBinaryPerDeviceState> const &per_device_state,
-                     float const *out_grad_ptr, float const *lhs_ptr, float const *rhs_ptr,
-                     float *lhs_grad_ptr, float *rhs_grad_ptr, OperatorType op_type,
-                     bool broadcast_inputLHS, bool broadcast_inputRHS,
-                     device_handle_t const &handle);
-// extension: dtype from the accessors
-void forward_kernel(device_stream_t const &stream,
-                    std::optional<ElementBinaryPerDeviceState> const &per_device_state,
-                    GenericTensorAccessorR const &lhs, GenericTensorAccessorR const &rhs,
-                    GenericTensorAccessorW const &out);
-void backward_kernel(device_stream_t const &stream,
-                     std::optional<ElementBinaryPerDeviceState> const &per_device_state,
-                     GenericTensorAccessorR const &out_grad, GenericTensorAccessorR const &lhs,
-                     GenericTensorAccessorR const &rhs, GenericTensorAccessorW const &lhs_grad,
-                     GenericTensorAccessorW const &rhs_grad);
-void cleanup_kernel(DeviceType device_type,
-                    std::optional<ElementBinaryPerDeviceState> const &per_device_state);
-}  // namespace Kernels::ElementBinary
-}  // namespace FlexFlow
+#include "kernels/element_binary_kernels.h"
+#include "kernels/element_unary_kernels.h"

@@ -4,6 +4,7 @@
 // here f is called once, untimed, so a training loop given {0, 0} still runs.
 #pragma once
 #include "kernels/device_stream_t.h"
+#include "kernels/profiling_settings.dtg.h"
 #include <optional>
 #include <utility>
 
@@ -16,11 +17,6 @@ int ffk_event_elapsed_ms(void *start, void *stop, float *ms);
 }
 
 namespace FlexFlow {
-
-struct ProfilingSettings {
-  int warmup_iters;
-  int measure_iters;
-};
 
 struct milliseconds_t {
   float value;

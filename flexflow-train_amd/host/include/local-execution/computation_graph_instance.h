@@ -29,8 +29,8 @@
 //    GEMM (its own output is never written); one whose input only comes from
 //    such a GELU -> Dropout pair writes the gradient of the GELU's input from
 //    its input-gradient GEMM (the gradient of its own input is never written).
-//    FFK_LAYER_UNFUSED=1 in the environment at creation keeps one kernel per
-//    operator.
+//    ffk_set_option(FFK_OPTION_LAYER_UNFUSED, 1) before creation keeps one
+//    kernel per operator.
 //  * the backward of an element-wise add copies nothing: an operand whose
 //    gradient has no other producer shares the output gradient's memory
 //    (get_gradient_accessor of both returns the same pointer), an operand that

@@ -118,10 +118,26 @@ GenericTensorAccessorW copy_tensor_accessor_w(GenericTensorAccessorW const &src,
   copy_accessor_data_to_l_from_r(dst, read_only_accessor_from_write_accessor(src));
   return dst;
 }
-GenericTensorAccessorR copy_tensor_accessor_r(GenericTensorAccessorR const &src, Allocator &allocator) {
+GenericTensorAccessorW copy_tensor_accessor_r(GenericTensorAccessorR const &src, Allocator &allocator) {
   GenericTensorAccessorW dst = allocator.allocate_tensor(src.shape);
   copy_accessor_data_to_l_from_r(dst, src);
-  return read_only_accessor_from_write_accessor(dst);
+  return dst;
+}
+
+// src/kernels/copy_tensor_accessor.cc: the source itself when it is host-resident already
+GenericTensorAccessorR copy_tensor_accessor_r_to_cpu_if_necessary(GenericTensorAccessorR const &src, Allocator &cpu_allocator) {
+  if (cpu_allocator.get_allocation_device_type() != DeviceType::CPU) {
+    throw std::runtime_error("copy_tensor_accessor_r_to_cpu_if_necessary: a CPU allocator is required");
+  }
+  if (src.device_type == DeviceType::CPU) return src;
+  return read_only_accessor_from_write_accessor(copy_tensor_accessor_r(src, cpu_allocator));
+}
+GenericTensorAccessorW copy_tensor_accessor_w_to_cpu_if_necessary(GenericTensorAccessorW const &src, Allocator &cpu_allocator) {
+  if (cpu_allocator.get_allocation_device_type() != DeviceType::CPU) {
+    throw std::runtime_error("copy_tensor_accessor_w_to_cpu_if_necessary: a CPU allocator is required");
+  }
+  if (src.device_type == DeviceType::CPU) return src;
+  return copy_tensor_accessor_w(src, cpu_allocator);
 }
 
 // ---- streams and handles --------------------------------------------------

@@ -30,6 +30,9 @@
 
 using namespace FlexFlow;
 
+// test_reference_includes.cc: a translation unit that uses only the reference's include lines
+std::string reference_style_translation_unit();
+
 static int g_failed = 0, g_checks = 0;
 #define CHECK(cond)                                                            \
   do {                                                                         \
@@ -233,6 +236,12 @@ static void gpu_tests() {
   device_handle_t handle = device_handle_t_from_managed_ff_handle(managed_handle);
   device_stream_t stream = get_gpu_device_stream();
   Allocator gpu = create_local_cuda_memory_allocator();
+
+  run("A translation unit with the reference's include lines and get<DataType>() / at<DataType>() accessor calls", [&] {
+    std::string const bad = reference_style_translation_unit();
+    if (!bad.empty()) printf("  failed: %s\n", bad.c_str());
+    CHECK(bad.empty());
+  });
 
   run("linear_forward_kernel / linear_backward_kernel (reference KAT, exact)", [&] {
     std::vector<float> x = {3, 3, 6, 2, 1, 5, 1, 2, -2, 8, 0.5, -3}, w = {1, 2, 1.5, 0.5, 4, -1}, b = {3, -1};

@@ -132,15 +132,15 @@ int ffk_probe_mfma_bf16(ffk_stream_t stream, int iterations, uint32_t seed,
                         float *out, size_t out_bytes, double *flops);
 
 /* Process-wide switches for tuning runs and tests; no counterpart in the
- * reference.  Each starts from the environment variable of the same name,
- * read once when the library is loaded.
- *   FFK_OPTION_GEMM_VARIANT (FFK_GEMM_VARIANT): 0 = the dispatch heuristic;
+ * reference.  All start at 0 and change through ffk_set_option only: the
+ * library never reads the environment.
+ *   FFK_OPTION_GEMM_VARIANT: 0 = the dispatch heuristic;
  *     128 / 256 force that pipelined bf16 tile (eight waves), 264 the 256 tile
  *     with one wave per SIMD, 1 the register-staged kernel.
- *   FFK_OPTION_LAYER_UNFUSED (FFK_LAYER_UNFUSED): != 0 makes the encoder-layer
+ *   FFK_OPTION_LAYER_UNFUSED: != 0 makes the encoder-layer
  *     entry points (and a step-driver instance created while it is set) run
  *     one kernel per operator.
- *   FFK_OPTION_ATTENTION_VARIANT (FFK_ATTENTION_VARIANT): 0 = the default bf16
+ *   FFK_OPTION_ATTENTION_VARIANT: 0 = the default bf16
  *     attention kernels (forward: 64 query rows per wavefront from 1024 keys
  *     on, 32 below; dK/dV: 64-row query tiles as two pipelined halves);
  *     1 = the forward kernel with 32 query rows per wavefront and the dK/dV
@@ -214,6 +214,16 @@ int ffk_linear_l2_regularizer_grad(ffk_stream_t stream, int dtype,
 int ffk_gemm(ffk_stream_t stream, int dtype, int trans_a, int trans_b,
              int64_t M, int64_t N, int64_t K, void const *A, void const *B,
              void *C, int accumulate);
+
+/* Which kernel ffk_gemm / ffk_linear_forward would launch for a dense problem of
+ * this data type, kind, shape and epilogue (bias, FFK_ACT_*), as the kernel's
+ * template instance, e.g. "gemm_bf16_pipe_kernel<256,256,128,128,64,2,1,false,
+ * true,0,false>".  Nothing is launched and no device is touched: the dispatch
+ * runs with a name sink in place of the launch.  For reports that must name
+ * the kernel they measured; no counterpart in the reference.                  */
+int ffk_gemm_kernel_name(int dtype, int trans_a, int trans_b, int64_t M,
+                         int64_t N, int64_t K, int has_bias, int activation,
+                         char *name, size_t name_bytes);
 
 /* ------------------------------------------------------------------------ */
 /* ElementUnary -- Kernels::ElementUnary::gpu_forward_kernel/gpu_backward_kernel

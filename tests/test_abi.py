@@ -35,3 +35,20 @@ def test_argument_checks_do_not_need_a_device(ffk):
                                      ffk.AGGR_NONE, 4, 2, 8, 10) == 1
     assert lib.ffk_element_unary_forward(None, ffk.FLOAT, 9999, 0.0, 1, 1, 4) == 3
     assert lib.ffk_gemm(None, ffk.DOUBLE, 0, 0, 4, 4, 4, 1, 1, 1, 0) == 3
+
+
+def test_gemm_kernel_name_needs_no_device(ffk):
+    """The dispatch answers which kernel a shape runs on without launching anything."""
+    big = ffk.gemm_kernel_name(ffk.BF16, False, True, 4096, 4096, 1024, has_bias=True)
+    assert big.startswith("gemm_bf16_pipe_kernel<256,256,") and big.endswith("false,true,0,false>")
+    assert ffk.gemm_kernel_name(ffk.BF16, True, False, 1024, 1024, 4096).startswith("gemm_bf16_pipe_kernel<128,128,")
+    assert ffk.gemm_kernel_name(ffk.FLOAT, False, True, 32, 128, 64, has_bias=True).startswith("gemm_f32_kernel")
+    assert ffk.gemm_kernel_name(ffk.BF16, False, False, 51, 131, 251) == "gemm_bf16_plain_kernel"
+    # an activation changes the instance, and the answer follows the option that forces a tile
+    relu = ffk.gemm_kernel_name(ffk.BF16, False, True, 4096, 4096, 1024, True, ffk.ACT_RELU)
+    assert relu != big
+    ffk.set_option(ffk.OPTION_GEMM_VARIANT, 128)
+    try:
+        assert ffk.gemm_kernel_name(ffk.BF16, False, True, 4096, 4096, 1024, True).startswith("gemm_bf16_pipe_kernel<128,128,")
+    finally:
+        ffk.set_option(ffk.OPTION_GEMM_VARIANT, 0)
