@@ -75,6 +75,183 @@ static hipError_t l2_reg_grad(hipStream_t st, void const *w, void *dw, int64_t n
   return ew_launch<T, 2, 1>(st, a, L2RegGrad{lambda});
 }
 
+// ---------------------------------------------------------------------------
+// The whole backward of a small fp32 Linear in ONE launch.  At sizes like the
+// reference's CPU-runnable case ([32,64] . [128,64]^T) every kernel is a few
+// microseconds of launch latency around almost no work, so the activation
+// gradient, the two products and the bias sums, which are independent given
+// (output, output_grad), run as jobs of one grid: workgroups [0, tiles_dx)
+// compute 64x64 tiles of input_grad, the next tiles_dw ones tiles of
+// weight_grad, the rest 64 columns of bias_grad each.  g = act'(output) *
+// output_grad is applied where an operand element is loaded, never stored.
+// ---------------------------------------------------------------------------
+struct SmallLinearBwd {
+  float const *y, *dy, *x, *w;
+  float *dx, *dw, *db;
+  int batch, in_dim, out_dim;
+  int act, relu_mode, accumulate;  // accumulate: FFK_ACC_* bits
+  int tiles_dx, tiles_dw;
+};
+
+__device__ __forceinline__ float small_act_grad(int act, int mode, float y, float dy) {
+  switch (act) {
+    case FFK_ACT_RELU:
+      return mode == 1 ? (dy > 0.0f ? 1.0f : 0.0f) : (y > 0.0f ? dy : 0.0f);
+    case FFK_ACT_SIGMOID:
+      return dy * y * (1.0f - y);
+    case FFK_ACT_TANH:
+      return dy * (1.0f - y * y);
+    default:
+      return dy;
+  }
+}
+
+// One 64x64 tile of sum_k a(m, k) * b(k, n), handed element by element to store(m, n, value); a
+// and b return 0 outside the problem.  A_KFAST: consecutive lanes walk k of the A operand (it
+// lies [M][K]); otherwise m; B_KFAST likewise for B lying [N][K].  A k-tile is 64 deep and all of a thread's 32 loads are issued
+// before the first is waited for: at these sizes the reduction is one or two such tiles, and
+// the time is the number of round trips to memory, not the arithmetic.
+constexpr int kSmallBK = 64;
+template <bool A_KFAST, bool B_KFAST, typename FA, typename FB, typename FS>
+__device__ __forceinline__ void small_f32_tile(FA a, FB b, int M, int N, int K, int m0, int n0, FS store,
+                                               float (&As)[kSmallBK][68], float (&Bs)[kSmallBK][68]) {
+  int const t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  int const wm0 = (wave >> 1) * 32, wn0 = (wave & 1) * 32;
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+  for (int k0 = 0; k0 < K; k0 += kSmallBK) {
+    float ra[16], rb[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      int const k = A_KFAST ? (t & 63) : (t >> 6) + 4 * i;
+      int const m = A_KFAST ? (t >> 6) + 4 * i : (t & 63);
+      int const kb = B_KFAST ? (t & 63) : (t >> 6) + 4 * i;
+      int const n = B_KFAST ? (t >> 6) + 4 * i : (t & 63);
+      ra[i] = a(m0 + m, k0 + k);
+      rb[i] = b(k0 + kb, n0 + n);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      int const k = A_KFAST ? (t & 63) : (t >> 6) + 4 * i;
+      int const m = A_KFAST ? (t >> 6) + 4 * i : (t & 63);
+      int const kb = B_KFAST ? (t & 63) : (t >> 6) + 4 * i;
+      int const n = B_KFAST ? (t >> 6) + 4 * i : (t & 63);
+      As[k][m] = ra[i];
+      Bs[kb][n] = rb[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < kSmallBK / 2; kk++) {
+      float const av = As[2 * kk + (lane >> 5)][wm0 + (lane & 31)];
+      float const bv = Bs[2 * kk + (lane >> 5)][wn0 + (lane & 31)];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  int const n = n0 + wn0 + (lane & 31);
+  if (n < N) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      int const m = m0 + wm0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+      if (m < M) store(m, n, acc[r]);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void linear_small_bwd_f32_kernel(SmallLinearBwd p) {
+  __shared__ float As[kSmallBK][68], Bs[kSmallBK][68];
+  int const bid = blockIdx.x;
+  auto g = [&](int row, int col) -> float {  // g[batch, out]
+    if (row >= p.batch || col >= p.out_dim) return 0.0f;
+    int64_t const i = (int64_t)row * p.out_dim + col;
+    return small_act_grad(p.act, p.relu_mode, p.act == FFK_ACT_NONE ? 0.0f : p.y[i], p.dy[i]);
+  };
+  if (bid < p.tiles_dx) {
+    // input_grad[batch, in] (+)= g[batch, out] . weight[out, in]
+    int const nbn = (p.in_dim + 63) / 64;
+    auto b = [&](int k, int n) -> float {
+      return k < p.out_dim && n < p.in_dim ? p.w[(int64_t)k * p.in_dim + n] : 0.0f;
+    };
+    bool const add = (p.accumulate & FFK_ACC_INPUT) != 0;
+    auto store = [&](int m, int n, float v) {
+      float *dst = p.dx + (int64_t)m * p.in_dim + n;
+      *dst = add ? *dst + v : v;
+    };
+    small_f32_tile<true, false>(g, b, p.batch, p.in_dim, p.out_dim, (bid / nbn) * 64, (bid % nbn) * 64, store, As, Bs);
+  } else if (bid < p.tiles_dx + p.tiles_dw) {
+    // weight_grad[out, in] (+)= g[batch, out]^T . input[batch, in]
+    int const tb = bid - p.tiles_dx, nbn = (p.in_dim + 63) / 64;
+    auto a = [&](int m, int k) -> float { return g(k, m); };
+    auto b = [&](int k, int n) -> float {
+      return k < p.batch && n < p.in_dim ? p.x[(int64_t)k * p.in_dim + n] : 0.0f;
+    };
+    bool const add = (p.accumulate & FFK_ACC_WEIGHT) != 0;
+    auto store = [&](int m, int n, float v) {
+      float *dst = p.dw + (int64_t)m * p.in_dim + n;
+      *dst = add ? *dst + v : v;
+    };
+    small_f32_tile<false, false>(a, b, p.out_dim, p.in_dim, p.batch, (tb / nbn) * 64, (tb % nbn) * 64, store, As, Bs);
+  } else {
+    // bias_grad[out] (+)= column sums of g: 64 columns, four row lanes that meet in LDS
+    int const col = (bid - p.tiles_dx - p.tiles_dw) * 64 + (threadIdx.x & 63);
+    int const ry = threadIdx.x >> 6;
+    float s = 0.0f;
+    for (int row = ry; row < p.batch; row += 4) s += g(row, col);
+    As[ry][threadIdx.x & 63] = s;
+    __syncthreads();
+    if (ry == 0 && col < p.out_dim) {
+      float const v = (As[0][threadIdx.x] + As[1][threadIdx.x]) + (As[2][threadIdx.x] + As[3][threadIdx.x]);
+      p.db[col] = (p.accumulate & FFK_ACC_BIAS) != 0 ? p.db[col] + v : v;
+    }
+  }
+}
+
+// Forward of a small fp32 Linear: output = act(input . weight^T + bias), one 64x64 tile per
+// workgroup, the same 64-deep reduction tiles.
+struct SmallLinearFwd {
+  float const *x, *w, *bias;
+  float *y;
+  int batch, in_dim, out_dim, act;
+};
+
+__global__ __launch_bounds__(256) void linear_small_fwd_f32_kernel(SmallLinearFwd p) {
+  __shared__ float As[kSmallBK][68], Bs[kSmallBK][68];
+  int const nbn = (p.out_dim + 63) / 64;
+  auto a = [&](int m, int k) -> float {
+    return m < p.batch && k < p.in_dim ? p.x[(int64_t)m * p.in_dim + k] : 0.0f;
+  };
+  // weight is [out, in]: b(k, n) = weight[n][k], k contiguous like the input's
+  auto b = [&](int k, int n) -> float {
+    return k < p.in_dim && n < p.out_dim ? p.w[(int64_t)n * p.in_dim + k] : 0.0f;
+  };
+  auto store = [&](int m, int n, float v) {
+    v += p.bias != nullptr ? p.bias[n] : 0.0f;
+    switch (p.act) {
+      case FFK_ACT_RELU: v = v >= 0.0f ? v : 0.0f; break;  // tensor_accessor_unary_ops.cc:32-38 keeps x >= 0
+      case FFK_ACT_SIGMOID: v = 1.0f / (1.0f + expf(-v)); break;
+      case FFK_ACT_TANH: v = tanhf(v); break;
+      case FFK_ACT_GELU: v = gelu_forward(v); break;
+      default: break;
+    }
+    p.y[(int64_t)m * p.out_dim + n] = v;
+  };
+  small_f32_tile<true, true>(a, b, p.batch, p.out_dim, p.in_dim, (blockIdx.x / nbn) * 64, (blockIdx.x % nbn) * 64, store, As, Bs);
+}
+
+// Small enough that launches, not work, set the time: at most two workgroups per CU in all.
+static bool small_linear_bwd(int dtype, int64_t batch, int64_t in_dim, int64_t out_dim, bool bias, int &tiles_dx,
+                             int &tiles_dw, int &blocks) {
+  if (dtype != FFK_FLOAT || batch > 8192 || in_dim > (1 << 20) || out_dim > (1 << 20)) return false;
+  int64_t const tdx = ceil_div(batch, 64) * ceil_div(in_dim, 64), tdw = ceil_div(out_dim, 64) * ceil_div(in_dim, 64);
+  int64_t const tb = bias ? ceil_div(out_dim, 64) : 0;
+  if (tdx + tdw + tb > 2 * kNumCU) return false;
+  tiles_dx = (int)tdx;
+  tiles_dw = (int)tdw;
+  blocks = (int)(tdx + tdw + tb);
+  return true;
+}
+
 }  // namespace ffk
 
 using namespace ffk;
@@ -105,6 +282,16 @@ extern "C" int ffk_linear_forward(ffk_stream_t stream, int dtype,
   FFK_REQUIRE(batch > 0 && in_dim > 0 && out_dim > 0,
               "linear_forward: non-positive dimension");
   FFK_REQUIRE(input && output && weight, "linear_forward: NULL tensor");
+  if (dtype == FFK_FLOAT && batch <= 8192 && ceil_div(batch, 64) * ceil_div(out_dim, 64) <= 2 * kNumCU &&
+      in_dim <= (1 << 20)) {
+    SmallLinearFwd p = {static_cast<float const *>(input), static_cast<float const *>(weight),
+                        static_cast<float const *>(bias), static_cast<float *>(output),
+                        (int)batch, (int)in_dim, (int)out_dim, activation};
+    unsigned const blocks = (unsigned)(ceil_div(batch, 64) * ceil_div(out_dim, 64));
+    linear_small_fwd_f32_kernel<<<blocks, 256, 0, as_stream(stream)>>>(p);
+    FFK_CHECK_LAUNCH();
+    return FFK_OK;
+  }
   GemmEpilogue ep;
   ep.bias = bias;
   ep.activation = activation;
@@ -131,6 +318,33 @@ static int linear_backward_impl(
               "linear_backward: non-positive dimension");
   FFK_REQUIRE(output_grad && weight && input, "linear_backward: NULL tensor");
   hipStream_t st = as_stream(stream);
+  if (activation != FFK_ACT_NONE) {
+    FFK_REQUIRE(output != nullptr, "linear_backward: output needed for activation");
+  }
+  // a small fp32 problem whose three gradients are all asked for: one launch, no scratch
+  int tiles_dx = 0, tiles_dw = 0, blocks = 0;
+  if (input_tail == nullptr && input_grad != nullptr && weight_grad != nullptr &&
+      small_linear_bwd(dtype, batch, in_dim, out_dim, bias_grad != nullptr, tiles_dx, tiles_dw, blocks)) {
+    SmallLinearBwd p;
+    p.y = static_cast<float const *>(output);
+    p.dy = static_cast<float const *>(output_grad);
+    p.x = static_cast<float const *>(input);
+    p.w = static_cast<float const *>(weight);
+    p.dx = static_cast<float *>(input_grad);
+    p.dw = static_cast<float *>(weight_grad);
+    p.db = static_cast<float *>(bias_grad);
+    p.batch = (int)batch;
+    p.in_dim = (int)in_dim;
+    p.out_dim = (int)out_dim;
+    p.act = activation;
+    p.relu_mode = relu_grad_mode;
+    p.accumulate = accumulate;
+    p.tiles_dx = tiles_dx;
+    p.tiles_dw = tiles_dw;
+    linear_small_bwd_f32_kernel<<<blocks, 256, 0, st>>>(p);
+    FFK_CHECK_LAUNCH();
+    return FFK_OK;
+  }
   size_t need = ffk_linear_backward_workspace_bytes(dtype, activation,
                                                     bias_grad != nullptr, batch, out_dim);
   if (need > 0 && (workspace == nullptr || workspace_bytes < need)) {
@@ -141,7 +355,6 @@ static int linear_backward_impl(
   uint8_t *ws = static_cast<uint8_t *>(workspace);
   void const *g = output_grad;
   if (activation != FFK_ACT_NONE) {
-    FFK_REQUIRE(output != nullptr, "linear_backward: output needed for activation");
     int64_t n = batch * out_dim;
     hipError_t e = dtype == FFK_FLOAT
                        ? act_grad<float>(st, activation, relu_grad_mode, output, output_grad, ws, n)

@@ -121,6 +121,34 @@ def test_linear_backward_with_l2_regularizer(ffk, oracle, dtype, shape):
         assert np.array_equal(to_np(z), oracle.linear_l2_regularizer_grad(w, np.zeros_like(w), lam))
 
 
+@pytest.mark.parametrize("act", [-1, 0, 1, 2])
+@pytest.mark.parametrize("shape", [(32, 64, 128), (70, 17, 65), (1, 1, 1), (300, 200, 130)])
+def test_small_fp32_backward_in_one_launch_equals_the_general_path(ffk, oracle, shape, act):
+    """A small fp32 backward with all three gradients runs as ONE launch (activation gradient,
+    both products and the bias sums as jobs of one grid); asked for one gradient at a time the
+    same entry point takes the general path (one kernel per product).  Same values either way,
+    both against the oracle, with and without accumulation."""
+    batch, in_dim, out_dim = shape
+    say("small fp32 linear backward, one launch vs general", shape, "act", act)
+    x, w, b, dy = _cfg1_inputs(seed=11 + batch, batch=batch, in_dim=in_dim, out_dim=out_dim)
+    w = w * 20
+    y_ref = oracle.linear_forward(x, w, b, activation=act)
+    dx_ref, dw_ref, db_ref = oracle.linear_backward(y_ref, dy, x, w, activation=act)
+    xd, wd, yd, dyd = (to_dev(a, torch) for a in (x, w, y_ref, dy))
+    one = [torch.full_like(xd, 0.5), torch.full_like(wd, 0.25), torch.full((out_dim,), 2.0, device="cuda")]
+    ffk.linear_backward(yd, dyd, xd, wd, *one, activation=act, accumulate=True)
+    sep = [torch.full_like(xd, 0.5), torch.full_like(wd, 0.25), torch.full((out_dim,), 2.0, device="cuda")]
+    ffk.linear_backward(yd, dyd, xd, wd, sep[0], None, None, activation=act, accumulate=True)
+    ffk.linear_backward(yd, dyd, xd, wd, None, sep[1], sep[2], activation=act, accumulate=True)
+    for got, gen, want, base, name in zip(one, sep, (dx_ref, dw_ref, db_ref), (0.5, 0.25, 2.0), ("dx", "dw", "db")):
+        assert_close(to_np(got), want + base, FP32_RTOL, name + " (one launch)")
+        assert_close(to_np(got), to_np(gen), FP32_RTOL, name + " one launch vs general")
+    # storing mode ignores what the tensors held
+    ffk.linear_backward(yd, dyd, xd, wd, *one, activation=act, accumulate=False)
+    for got, want, name in zip(one, (dx_ref, dw_ref, db_ref), ("dx", "dw", "db")):
+        assert_close(to_np(got), want, FP32_RTOL, name + " stored")
+
+
 def test_linear_no_bias_and_skipped_grads(ffk, oracle):
     x, w, b, dy = _cfg1_inputs(seed=5, batch=16, in_dim=24, out_dim=40)
     say("linear fp32 no bias / NULL grads")
@@ -141,8 +169,14 @@ def test_linear_errors(ffk):
     x = torch.zeros((4, 4), device="cuda")
     with pytest.raises(ffk.FFKError, match="Unhandled activation"):
         ffk.linear_forward(x, x, None, activation=9)
+    # (a small fp32 backward with all gradients asked for runs as one launch and needs no scratch;
+    # without the input gradient it takes the general path, which does)
     with pytest.raises(ffk.FFKError, match="workspace"):
         ffk.check(ffk.lib().ffk_linear_backward(0, ffk.FLOAT, ffk.ACT_RELU, 0, x.data_ptr(), x.data_ptr(),
+                                                x.data_ptr(), None, x.data_ptr(), x.data_ptr(), None,
+                                                4, 4, 4, None, 0, 0))
+    with pytest.raises(ffk.FFKError, match="output needed"):
+        ffk.check(ffk.lib().ffk_linear_backward(0, ffk.FLOAT, ffk.ACT_RELU, 0, None, x.data_ptr(),
                                                 x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), None,
                                                 4, 4, 4, None, 0, 0))
 
