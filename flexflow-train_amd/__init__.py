@@ -434,6 +434,10 @@ def layer_norm_forward(x, gamma, beta, eps, out=None, mean=None, rstd=None):
     return out, mean, rstd
 
 
+# bits of ffk_layer_norm_backward's accumulate_input_grad
+LN_ACC_INPUT, LN_ACC_PARAMS = 1, 2
+
+
 def layer_norm_backward(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, accumulate=False,
                         workspace=None):
     torch = _torch()

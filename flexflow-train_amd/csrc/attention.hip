@@ -594,7 +594,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
 // 64 query rows per wavefront (attention_fwd.hip)
 hipError_t attention_bf16_forward_wide(hipStream_t st, AttnParams const &p, int head_dim);
 
-// dK/dV with direct loads, two workgroups per CU (attention_bwd.hip)
+// dK/dV with direct loads, one workgroup per CU: its three Q and three dO tile buffers take
+// 48 KB (head size 64) or 96 KB (128) of LDS, and one wave per SIMD holds the accumulators (attention_bwd.hip)
 hipError_t attention_bf16_dkdv(hipStream_t st, AttnBwdParams const &p, int head_dim);
 bool attention_bf16_bwd_direct_ok(AttnBwdParams const &p);
 

@@ -409,7 +409,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // segment s of row k sits at segment s ^ (k % 4).
   constexpr int ROWS_PER_LOAD_KC = NT / CPRK;     // rows covered by one load of all threads
   static_assert((ROWS_PER_LOAD_KC / RPW) % CPRK == 0, "swizzle must repeat per load");
-  static_assert((NT * 8 / BM) % 4 == 0 && (NT * 8 / BN) % 4 == 0, "swizzle must repeat per load");
+  static_assert((!TA || (NT * 8 % BM == 0 && (NT * 8 / BM) % 4 == 0)) && (!TBL || (NT * 8 % BN == 0 && (NT * 8 / BN) % 4 == 0)),
+                "a panel lying [BK][cols] must divide into whole loads, and the swizzle repeat per load");
   unsigned voff_a, voff_b;
   {
     int c = wave * 64 + lane;
@@ -533,7 +534,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   constexpr int PART = SPREAD ? LPT / KS : LPT;
   // One wave per SIMD and two stages: a refill goes out in two halves, the first behind the
   // barrier that frees its stage, the second in the first k-step of the following tile.
-  constexpr bool WIDE2 = WM == 128 && WN == 128 && STAGES == 2;
+  constexpr bool WIDE2 = WM == 128 && (WN == 128 || WN == 96) && STAGES == 2;
   constexpr int PRO_PART = WIDE2 ? LPT / 2 : PART;  // of the last tile the prologue starts
 #pragma unroll
   for (int s = 0; s < STAGES; s++) {
@@ -585,7 +586,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       // that the compiler keeps them there.  The refill of a stage goes out in two halves: the
       // first behind the barrier that frees the stage (last step of its tile), the second in
       // step 0 of the following tile; the steps in between carry fragment reads only.
-      static_assert(PF == 1 && TM == 4 && TN == 4 && LPT == 16 && KS >= 2, "written for this shape");
+      static_assert(PF == 1 && TM == 4 && (TN == 4 || TN == 3) && LPT % 2 == 0 && KS >= 2, "written for these shapes");
+      // A k-step has NS = TM * TN MFMAs; behind them go the NR = TM + TN fragment reads of the
+      // next step and, in the two steps that carry them, NL = LPT / 2 direct loads, each kind
+      // spread evenly over the slots with the loads half a spacing behind the reads (4 x 4
+      // blocks: reads in the even slots, loads in the odd ones; 4 x 3: twelve slots for seven
+      // reads and seven loads).
+      constexpr int NS = TM * TN, NR = TM + TN, NL = LPT / 2;
 #pragma unroll
       for (int kk = 0; kk < KS; kk++) {
         int const cur = kk % NB, nxt = (kk + PF) % NB;
@@ -605,10 +612,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
         auto aux = [&](int p) __attribute__((always_inline)) {
           // (all reads first, then the loads, measured 2-7% slower: the four waves' reads then
           // meet in the LDS pipeline in bursts)
-          int const r = p / 2;
-          if (p % 2 == 1) {
-            if (loads) issue_some(ltile, lstage, lfirst + r, 1);
-          } else if (reads) {
+#pragma unroll
+          for (int r = 0; r < NR; r++) {
+            if (r * NS / NR != p || !reads) continue;
             if (r == 0 || r > TN) {
               int const i = r == 0 ? 0 : r - TN;
               af[nxt][i] = TA ? frag_tr(ra, BM, tr_tab_a, wm0 + i * 32, rkk) : frag_kc(ra, wm0 + i * 32, rkk);
@@ -616,6 +622,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
               int const j = r - 1;
               bfr[nxt][j] = TBL ? frag_tr(rb, BN, tr_tab_b, wn0 + j * 32, rkk) : frag_kc(rb, wn0 + j * 32, rkk);
             }
+          }
+#pragma unroll
+          for (int l = 0; l < NL; l++) {
+            if ((2 * l + 1) * NS / (2 * NL) != p || !loads) continue;
+            issue_some(ltile, lstage, lfirst + l, 1);
           }
         };
         __builtin_amdgcn_sched_barrier(0);
@@ -705,7 +716,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // epilogue below, whose stores are whole 128-byte lines, is 2-5% ahead.  (The 32-byte pieces
   // cost memory traffic: 49 MB written per 32 MB tile set by the write counter, whatever the
   // order of the stores; going row by row instead of column block by column block is 3% slower.)
-  if constexpr (TAIL == GemmEpilogue::kTailNone && WM == 128 && WN == 128) {
+  if constexpr (TAIL == GemmEpilogue::kTailNone && WIDE2) {
     if (partial == nullptr && accumulate == 0) {  // uniform over the launch
       auto direct = [&](auto actf) __attribute__((always_inline)) {
 #pragma unroll
@@ -762,7 +773,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
     // and those complete in program order: no barrier.  With one wave per SIMD (128x128 wave tiles)
     // the tile goes out in two halves of 64 rows, so that the stores of the first half are under
     // way while the second is converted.
-    constexpr int HALVES = (WM == 128 && WN == 128) ? 2 : 1;
+    constexpr int HALVES = WIDE2 ? 2 : 1;
     constexpr int TMH = TM / HALVES;
 #pragma unroll
     for (int half = 0; half < HALVES; half++) {
@@ -874,8 +885,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // One wave per SIMD with a 128x128 wave tile keeps 256 accumulator registers: only the plain
   // epilogue (bias, no activation, no split-K) is compiled for it, so that nothing outside the
   // loop competes for registers.
-  constexpr bool WIDE = WM == 128 && WN == 128;
-  if constexpr (WIDE) {
+  if constexpr (WIDE2) {
     finish([](float v) { return v; });
     return;
   }
@@ -1156,16 +1166,21 @@ size_t gemm_splitk_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K) {
   return s > 1 ? (size_t)s * (size_t)(M * N) * sizeof(float) : 0;
 }
 
-// Which pipelined tile a bf16 GEMM runs on: 256, 128, or 0 (none of the two:
-// split-K or the register-staged kernels).
-static int pipe_tile_for(bf16 const *C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-                         GemmEpilogue const &ep, int variant) {
+// What every pipelined kernel asks of the operands, whatever its tile.
+static bool pipe_operands_ok(bf16 const *C, int K, int64_t lda, int64_t ldb, int64_t ldc, GemmEpilogue const &ep) {
   bool const c_vec = (ldc % 8 == 0) && aligned16(C);
   // the pipelined kernels fetch the bias in 8-byte pieces
   bool const aux_ok = reinterpret_cast<uintptr_t>(ep.bias) % 8 == 0;
   // the direct loads address an operand panel with 32-bit byte offsets
   bool const panel_ok = 2 * 256 * std::max(lda, ldb) < (int64_t(1) << 31);
-  if (!(c_vec && aux_ok && panel_ok && K % 64 == 0 && variant != 1)) return 0;
+  return c_vec && aux_ok && panel_ok && K % 64 == 0;
+}
+
+// Which pipelined tile a bf16 GEMM runs on: 256, 128, or 0 (none of the two:
+// split-K or the register-staged kernels).
+static int pipe_tile_for(bf16 const *C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                         GemmEpilogue const &ep, int variant) {
+  if (!pipe_operands_ok(C, K, lda, ldb, ldc, ep) || variant == 1) return 0;
   bool const fits256 = M % 256 == 0 && N % 256 == 0;
   bool const fits128 = M % 128 == 0 && N % 128 == 0;
   int64_t const t256 = fits256 ? (int64_t)(M / 256) * (N / 256) : 0;
@@ -1216,6 +1231,20 @@ static hipError_t pick_bf16(hipStream_t st, bf16 const *A, bf16 const *B,
         }
       }
       return hipErrorInvalidValue;
+    }
+    // An output that 256x256 tiles cover in a ragged last round but 256x192 tiles cover in whole
+    // rounds of the chip (the attention block's fused Q/K/V projection: [4096, 3072] is 192 tiles of
+    // the first kind on 256 CUs, 256 of the second): one wave per SIMD on 128x96 wave tiles.  Only
+    // with both operands K-contiguous: a [K][192] panel does not divide into whole direct loads.
+    if constexpr (!TA && TB) {
+      bool const fits192 = M % 256 == 0 && N % 192 == 0;
+      int64_t const t256 = M % 256 == 0 && N % 256 == 0 ? (int64_t)(M / 256) * (N / 256) : 0;
+      int64_t const t192 = fits192 ? (int64_t)(M / 256) * (N / 192) : 0;
+      bool const whole_rounds = t192 > 0 && t192 % kNumCU == 0 && t256 % kNumCU != 0;
+      if (pipe_operands_ok(C, K, lda, ldb, ldc, ep) && variant != 1 && ep.activation == FFK_ACT_NONE && K >= 1024 &&
+          (variant == 192 ? fits192 : (variant == 0 && whole_rounds))) {
+        return launch_pipe<256, 192, 128, 96, 64, 2, 1, TA, TB>(st, A, B, C, M, N, K, lda, ldb, ldc, ep);
+      }
     }
     // Reductions from 1024 on without an activation: one wave per SIMD on 128x128 wave tiles, two
     // 64-deep stages, every instruction of the loop placed by hand.  (Below that the eight-wave

@@ -651,6 +651,9 @@ extern "C" int ffk_layer_norm_backward(
   if (M == 0) return FFK_OK;
   FFK_REQUIRE(M < (1ll << 31), "layer_norm_backward: too many rows");
   FFK_REQUIRE(output_grad && input && mean && rstd, "layer_norm_backward: NULL tensor");
+  FFK_REQUIRE((accumulate_input_grad & ~(FFK_LN_ACC_INPUT | FFK_LN_ACC_PARAMS)) == 0,
+              "layer_norm_backward: accumulate_input_grad %d is not a mask of FFK_LN_ACC_INPUT | FFK_LN_ACC_PARAMS",
+              accumulate_input_grad);
   bool const acc = (accumulate_input_grad & FFK_LN_ACC_INPUT) != 0;
   bool const acc_params = (accumulate_input_grad & FFK_LN_ACC_PARAMS) != 0;
   if (dtype == FFK_FLOAT)
@@ -731,6 +734,9 @@ extern "C" int ffk_layer_norm_backward_static(
   FFK_REQUIRE(M < (1ll << 31), "layer_norm_backward_static: too many rows");
   FFK_REQUIRE(output_grad && input && mean && rstd, "layer_norm_backward_static: NULL tensor");
   FFK_REQUIRE(dtype == FFK_FLOAT || dtype == FFK_BF16, "layer_norm_backward_static: dtype %d not supported", dtype);
+  FFK_REQUIRE((accumulate_input_grad & ~(FFK_LN_ACC_INPUT | FFK_LN_ACC_PARAMS)) == 0,
+              "layer_norm_backward_static: accumulate_input_grad %d is not a mask of FFK_LN_ACC_INPUT | "
+              "FFK_LN_ACC_PARAMS", accumulate_input_grad);
   if (N > FFK_LAYER_NORM_STATIC_MAX_N) {
     return fail(FFK_ERR_WORKSPACE,
                 "layer_norm_backward_static: rows of %lld elements exceed the limit of %d "
@@ -743,7 +749,21 @@ extern "C" int ffk_layer_norm_backward_static(
   // The array is shared by every call on this device, so its column reduction
   // runs here and now: a collected one would read the partial sums after a
   // later call has overwritten them.
+  // A reduction collected earlier on this thread that writes the same
+  // gamma_grad / beta_grad (shared LayerNorm parameters) has to reach them
+  // first, as the calls were made: run what is collected before this one.
   ColreduceBatch *const collecting = tl_colreduce_batch;
+  if (collecting != nullptr) {
+    for (int k = 0; k < collecting->count; k++) {
+      ColreduceJob const &c = collecting->job[k];
+      bool const clash = (gamma_grad != nullptr && (c.out0 == gamma_grad || c.out1 == gamma_grad)) ||
+                         (beta_grad != nullptr && (c.out0 == beta_grad || c.out1 == beta_grad));
+      if (clash) {
+        FFK_HIP(colreduce_flush(as_stream(stream), *collecting));
+        break;
+      }
+    }
+  }
   tl_colreduce_batch = nullptr;
   bool const acc = (accumulate_input_grad & FFK_LN_ACC_INPUT) != 0;
   bool const acc_params = (accumulate_input_grad & FFK_LN_ACC_PARAMS) != 0;

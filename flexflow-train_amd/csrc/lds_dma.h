@@ -41,8 +41,15 @@ __device__ __forceinline__ void lds_dma16(i32x4 rsrc, unsigned lane_byte_off, un
                :
                : "s"(lds_byte_addr), "v"(lane_byte_off), "s"(rsrc), "s"(uniform_byte_off)
                : "memory");  // M0 is not in the clobber list (the compiler rejects
-                             // reserved registers there); nothing else in these
-                             // kernels uses M0 (no GDS, message or relative-move ops)
+                             // reserved registers there).  The invariant every
+                             // kernel that includes this header keeps: no register
+                             // array is indexed by a run-time value (all such loops
+                             // are fully unrolled), so the compiler emits no
+                             // relative-move or GDS/message instruction and holds
+                             // nothing live in M0 across these blocks.  Guarded by
+                             // the bit-equality tests against the kernels without
+                             // direct loads (tests/test_gpu_linear.py: GEMM variants;
+                             // tests/test_gpu_attention.py: the two dK/dV kernels).
 }
 // The same for 4 bytes per lane: lane l's dword lands at lds_base + 4 l.
 __device__ __forceinline__ void lds_dma4(i32x4 rsrc, unsigned lane_byte_off, unsigned uniform_byte_off,

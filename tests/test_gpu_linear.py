@@ -315,6 +315,45 @@ def test_gemm_bf16_one_wave_per_simd(ffk, oracle, trans_a, trans_b, mnk):
     assert_close(to_np(out[264][1])[rows], oracle.gemm_f64(A_rows, B, trans_a, trans_b) + C0[rows], 2.0 ** -7, "C acc")
 
 
+@pytest.mark.parametrize("mnk", [(512, 384, 1024), (256, 384, 2048), (4096, 3072, 1024)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_gemm_bf16_256x192_tile(ffk, oracle, mnk, bias):
+    """The 256x192 tile (one wave per SIMD, 128x96 wave tiles) that the fused Q/K/V projection's
+    [4096, 3072] output takes so that its tiles cover the chip in one whole round: option 192
+    forces it at any fitting size; against the oracle on sampled rows and columns, and bit for
+    bit against the 128x128-tile kernel (every pipelined kernel adds the k-steps in the same
+    order).  At [4096, 3072] the dispatch must pick it by itself."""
+    M, N, K = mnk
+    say("gemm bf16 256x192 tile", mnk, "bias", bias)
+    g = rng(7 * M + N + K)
+    A = bf16_round(g.standard_normal((M, K)))
+    B = bf16_round(g.standard_normal((N, K)) * 0.05)
+    bv = bf16_round(g.standard_normal((N,))) if bias else None
+    Ad, Bd = to_dev(A, torch, torch.bfloat16), to_dev(B, torch, torch.bfloat16)
+    bd = to_dev(bv, torch, torch.bfloat16) if bias else None
+    out = {}
+    try:
+        for variant in (192, 128):
+            ffk.set_option(ffk.OPTION_GEMM_VARIANT, variant)
+            out[variant] = ffk.linear_forward(Ad, Bd, bd)
+            name = ffk.gemm_kernel_name(ffk.BF16, False, True, M, N, K, has_bias=bias)
+            assert name.startswith("gemm_bf16_pipe_kernel<256,192,128,96," if variant == 192 else "gemm_bf16_pipe_kernel<128,128,"), name
+    finally:
+        ffk.set_option(ffk.OPTION_GEMM_VARIANT, 0)
+    assert torch.equal(out[192], out[128])
+    Cn = to_np(out[192])
+    rows = np.sort(g.choice(M, 16, replace=False))
+    cols = np.sort(g.choice(N, 16, replace=False))
+    want_r = oracle.gemm_f64(np.ascontiguousarray(A[rows]), B, False, True) + (bv if bias else 0.0)
+    want_c = oracle.gemm_f64(A, np.ascontiguousarray(B[cols]), False, True) + (bv[cols] if bias else 0.0)
+    assert_close(Cn[rows], want_r, 2.0 ** -8, "C rows")
+    assert_close(Cn[:, cols], want_c, 2.0 ** -8, "C cols")
+    if mnk == (4096, 3072, 1024):
+        assert ffk.gemm_kernel_name(ffk.BF16, False, True, M, N, K, has_bias=bias).startswith(
+            "gemm_bf16_pipe_kernel<256,192,128,96,")
+        assert torch.equal(ffk.linear_forward(Ad, Bd, bd), out[192])
+
+
 @pytest.mark.parametrize("act", [-1, 0])
 def test_linear_bf16_pipelined(ffk, oracle, act):
     """Linear at a size whose three products all take the pipelined kernels

@@ -34,10 +34,13 @@ def _case(ffk, oracle, M, N, dtype, same_grid):
     got = [torch.full_like(xd, -3.0), torch.full_like(gd, -3.0), torch.full_like(gd, -3.0)]
     ffk.layer_norm_backward(dyd, xd, mean, rstd, gd, *want)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # free device memory as the driver reports it (hipMemGetInfo): it also sees an allocation
+    # made inside the library, which torch's own counter would not
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     ffk.layer_norm_backward_static(dyd, xd, mean, rstd, gd, *got)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated during the call"
     # dX never depends on how many workgroups walk the rows
     assert torch.equal(got[0], want[0]), "dx bits differ"
     if same_grid:
@@ -105,6 +108,52 @@ def test_static_scratch_inside_a_collecting_region(ffk, oracle):
         ffk.layer_norm_backward(dyd, xd, mean, rstd, gd, dx2, dg2, db2)
         torch.cuda.synchronize()
         assert torch.equal(dx, dx2) and torch.equal(dg, dg2) and torch.equal(db, db2)
+
+
+def test_static_scratch_in_a_collecting_region_with_shared_parameters(ffk):
+    """Two LayerNorms that share gamma / beta gradients inside one collecting region: the
+    workspace form first (its column sums are collected), the static form after it (its own run
+    at once).  In storing mode the later call's values must be what the tensors hold at the
+    end, as outside a region; in accumulating mode the sum of both."""
+    g = rng(6)
+    tdt = torch.bfloat16
+    N = 1024
+    cases = []
+    for M in (384, 512):
+        x = bf16_round(g.standard_normal((M, N)))
+        dy = bf16_round(g.standard_normal((M, N)))
+        gamma = bf16_round(1 + 0.1 * g.standard_normal((N,)))
+        xd, dyd, gd = (to_dev(a, torch, tdt) for a in (x, dy, gamma))
+        _, mean, rstd = ffk.layer_norm_forward(xd, gd, gd, 1e-5)
+        cases.append((dyd, xd, mean, rstd, gd))
+    alone = []
+    for c in cases:
+        dx, dg, db = torch.empty_like(c[1]), torch.zeros((N,), dtype=tdt, device="cuda"), torch.zeros((N,), dtype=tdt, device="cuda")
+        ffk.layer_norm_backward(*c, dx, dg, db)
+        alone.append((dg, db))
+    for accumulate in (0, ffk.LN_ACC_PARAMS):
+        dg, db = torch.zeros((N,), dtype=tdt, device="cuda"), torch.zeros((N,), dtype=tdt, device="cuda")
+        ffk.check(ffk.lib().ffk_column_reductions_begin())
+        try:
+            ffk.layer_norm_backward(*cases[0], torch.empty_like(cases[0][1]), dg, db, accumulate=accumulate)
+            ffk.layer_norm_backward_static(*cases[1], torch.empty_like(cases[1][1]), dg, db, accumulate=accumulate)
+        finally:
+            ffk.check(ffk.lib().ffk_column_reductions_end(ffk.current_stream()))
+        torch.cuda.synchronize()
+        if accumulate == 0:
+            assert torch.equal(dg, alone[1][0]) and torch.equal(db, alone[1][1]), "the later call must win"
+        else:
+            want_g = (alone[0][0].float() + alone[1][0].float()).to(tdt)
+            want_b = (alone[0][1].float() + alone[1][1].float()).to(tdt)
+            assert torch.equal(dg, want_g) and torch.equal(db, want_b), "both calls must add"
+
+
+def test_static_scratch_rejects_a_flag_that_is_no_mask(ffk):
+    x = torch.zeros((2, 64), dtype=torch.bfloat16, device="cuda")
+    m = torch.zeros((2,), dtype=torch.float32, device="cuda")
+    rc = ffk.lib().ffk_layer_norm_backward_static(0, ffk.BF16, x.data_ptr(), x.data_ptr(), m.data_ptr(), m.data_ptr(),
+                                                  None, x.data_ptr(), None, None, 2, 64, -1)
+    assert rc == 1 and b"not a mask" in ffk.lib().ffk_last_error()
 
 
 def test_static_scratch_rejects_rows_beyond_the_limit(ffk):
