@@ -93,35 +93,45 @@ struct SmallLinearBwd {
   int tiles_dx, tiles_dw;
 };
 
-__device__ __forceinline__ float small_act_grad(int act, int mode, float y, float dy) {
-  switch (act) {
-    case FFK_ACT_RELU:
-      return mode == 1 ? (dy > 0.0f ? 1.0f : 0.0f) : (y > 0.0f ? dy : 0.0f);
-    case FFK_ACT_SIGMOID:
-      return dy * y * (1.0f - y);
-    case FFK_ACT_TANH:
-      return dy * (1.0f - y * y);
-    default:
-      return dy;
+// ACT is a template argument of the kernel: a run-time switch here puts a branch and a wait
+// between every two loads of a thread, and the kernel's time is its round trips to memory.
+template <int ACT>
+__device__ __forceinline__ float small_act_grad(int mode, float y, float dy) {
+  if constexpr (ACT == FFK_ACT_RELU) {
+    return mode == 1 ? (dy > 0.0f ? 1.0f : 0.0f) : (y > 0.0f ? dy : 0.0f);
+  } else if constexpr (ACT == FFK_ACT_SIGMOID) {
+    return dy * y * (1.0f - y);
+  } else if constexpr (ACT == FFK_ACT_TANH) {
+    return dy * (1.0f - y * y);
+  } else {
+    return dy;
   }
 }
 
-// One 64x64 tile of sum_k a(m, k) * b(k, n), handed element by element to store(m, n, value); a
-// and b return 0 outside the problem.  A_KFAST: consecutive lanes walk k of the A operand (it
-// lies [M][K]); otherwise m; B_KFAST likewise for B lying [N][K].  A k-tile is 64 deep and all of a thread's 32 loads are issued
-// before the first is waited for: at these sizes the reduction is one or two such tiles, and
-// the time is the number of round trips to memory, not the arithmetic.
+// One 64x64 tile of sum_k a(m, k) * b(k, n), handed element by element to store(m, n, value).  a
+// and b clamp their coordinates into the problem and return what lies there: rows and columns
+// past the edge give values that are never stored, k past the edge is zeroed here when the tile
+// is written to LDS (a select on a loaded value any earlier is a wait for that load).  A_KFAST: consecutive lanes walk k of the A operand (it
+// lies [M][K]); otherwise m; B_KFAST likewise for B lying [N][K].  A k-tile is 64 deep, all of a thread's 32 loads are issued
+// before the first is waited for, and the next k-tile's are issued before this one is multiplied: at these sizes the
+// time is the number of round trips to memory, not the arithmetic.
 constexpr int kSmallBK = 64;
-template <bool A_KFAST, bool B_KFAST, typename FA, typename FB, typename FS>
-__device__ __forceinline__ void small_f32_tile(FA a, FB b, int M, int N, int K, int m0, int n0, FS store,
-                                               float (&As)[kSmallBK][68], float (&Bs)[kSmallBK][68]) {
+constexpr int kSmallMaxDepth = 1024;  // longest reduction the one-launch kernels take (16 k-tiles)
+// a returns what it loaded (a float, or the pair an activation gradient is made of) and av turns
+// that into the operand's value when the tile is written to LDS, one k-tile later: arithmetic on a
+// loaded value any earlier would make the wave wait for the load it is meant to run under.
+template <bool A_KFAST, bool B_KFAST, typename FA, typename FAV, typename FB, typename FS>
+__device__ __forceinline__ void small_f32_tile(FA a, FAV av, FB b, int M, int N, int K, int m0, int n0, FS store,
+                                               float (&As)[kSmallBK][68], float (&Bs)[kSmallBK][68],
+                                               float const *prior = nullptr, int64_t prior_ld = 0) {
   int const t = threadIdx.x, lane = t & 63, wave = t >> 6;
   int const wm0 = (wave >> 1) * 32, wn0 = (wave & 1) * 32;
   f32x16 acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.0f;
-  for (int k0 = 0; k0 < K; k0 += kSmallBK) {
-    float ra[16], rb[16];
+  decltype(a(0, 0)) ra[16];
+  float rb[16];
+  auto fetch = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       int const k = A_KFAST ? (t & 63) : (t >> 6) + 4 * i;
@@ -131,16 +141,20 @@ __device__ __forceinline__ void small_f32_tile(FA a, FB b, int M, int N, int K, 
       ra[i] = a(m0 + m, k0 + k);
       rb[i] = b(k0 + kb, n0 + n);
     }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += kSmallBK) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       int const k = A_KFAST ? (t & 63) : (t >> 6) + 4 * i;
       int const m = A_KFAST ? (t >> 6) + 4 * i : (t & 63);
       int const kb = B_KFAST ? (t & 63) : (t >> 6) + 4 * i;
       int const n = B_KFAST ? (t >> 6) + 4 * i : (t & 63);
-      As[k][m] = ra[i];
-      Bs[kb][n] = rb[i];
+      As[k][m] = k0 + k < K ? av(ra[i]) : 0.0f;
+      Bs[kb][n] = k0 + kb < K ? rb[i] : 0.0f;
     }
     __syncthreads();
+    if (k0 + kSmallBK < K) fetch(k0 + kSmallBK);  // on its way while this tile is multiplied
 #pragma unroll
     for (int kk = 0; kk < kSmallBK / 2; kk++) {
       float const av = As[2 * kk + (lane >> 5)][wm0 + (lane & 31)];
@@ -151,6 +165,16 @@ __device__ __forceinline__ void small_f32_tile(FA a, FB b, int M, int N, int K, 
   }
   int const n = n0 + wn0 + (lane & 31);
   if (n < N) {
+    if (prior != nullptr) {  // accumulating: what the destination holds, all 16 loads in flight together
+      float old[16];
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        int const m = m0 + wm0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        old[r] = prior[(int64_t)(m < M ? m : M - 1) * prior_ld + n];
+      }
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[r] = old[r] + acc[r];
+    }
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       int const m = m0 + wm0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
@@ -159,45 +183,52 @@ __device__ __forceinline__ void small_f32_tile(FA a, FB b, int M, int N, int K, 
   }
 }
 
+template <int ACT>
 __global__ __launch_bounds__(256) void linear_small_bwd_f32_kernel(SmallLinearBwd p) {
   __shared__ float As[kSmallBK][68], Bs[kSmallBK][68];
   int const bid = blockIdx.x;
-  auto g = [&](int row, int col) -> float {  // g[batch, out]
-    if (row >= p.batch || col >= p.out_dim) return 0.0f;
-    int64_t const i = (int64_t)row * p.out_dim + col;
-    return small_act_grad(p.act, p.relu_mode, p.act == FFK_ACT_NONE ? 0.0f : p.y[i], p.dy[i]);
+  // g[batch, out] = act'(output) * output_grad, as the pair it is made of and as its value
+  auto g_raw = [&](int row, int col) -> float2 {
+    int const r = row < p.batch ? row : p.batch - 1, c = col < p.out_dim ? col : p.out_dim - 1;
+    int64_t const i = (int64_t)r * p.out_dim + c;
+    float yv = 0.0f;
+    if constexpr (ACT == FFK_ACT_RELU || ACT == FFK_ACT_SIGMOID || ACT == FFK_ACT_TANH) yv = p.y[i];
+    return make_float2(yv, p.dy[i]);
   };
+  auto g_val = [&](float2 r) -> float { return small_act_grad<ACT>(p.relu_mode, r.x, r.y); };
   if (bid < p.tiles_dx) {
     // input_grad[batch, in] (+)= g[batch, out] . weight[out, in]
     int const nbn = (p.in_dim + 63) / 64;
     auto b = [&](int k, int n) -> float {
-      return k < p.out_dim && n < p.in_dim ? p.w[(int64_t)k * p.in_dim + n] : 0.0f;
+      return p.w[(int64_t)(k < p.out_dim ? k : p.out_dim - 1) * p.in_dim + (n < p.in_dim ? n : p.in_dim - 1)];
     };
     bool const add = (p.accumulate & FFK_ACC_INPUT) != 0;
-    auto store = [&](int m, int n, float v) {
-      float *dst = p.dx + (int64_t)m * p.in_dim + n;
-      *dst = add ? *dst + v : v;
-    };
-    small_f32_tile<true, false>(g, b, p.batch, p.in_dim, p.out_dim, (bid / nbn) * 64, (bid % nbn) * 64, store, As, Bs);
+    auto store = [&](int m, int n, float v) { p.dx[(int64_t)m * p.in_dim + n] = v; };
+    small_f32_tile<true, false>(g_raw, g_val, b, p.batch, p.in_dim, p.out_dim, (bid / nbn) * 64, (bid % nbn) * 64, store, As, Bs,
+                                add ? p.dx : nullptr, p.in_dim);
   } else if (bid < p.tiles_dx + p.tiles_dw) {
     // weight_grad[out, in] (+)= g[batch, out]^T . input[batch, in]
     int const tb = bid - p.tiles_dx, nbn = (p.in_dim + 63) / 64;
-    auto a = [&](int m, int k) -> float { return g(k, m); };
+    auto a = [&](int m, int k) -> float2 { return g_raw(k, m); };
     auto b = [&](int k, int n) -> float {
-      return k < p.batch && n < p.in_dim ? p.x[(int64_t)k * p.in_dim + n] : 0.0f;
+      return p.x[(int64_t)(k < p.batch ? k : p.batch - 1) * p.in_dim + (n < p.in_dim ? n : p.in_dim - 1)];
     };
     bool const add = (p.accumulate & FFK_ACC_WEIGHT) != 0;
-    auto store = [&](int m, int n, float v) {
-      float *dst = p.dw + (int64_t)m * p.in_dim + n;
-      *dst = add ? *dst + v : v;
-    };
-    small_f32_tile<false, false>(a, b, p.out_dim, p.in_dim, p.batch, (tb / nbn) * 64, (tb % nbn) * 64, store, As, Bs);
+    auto store = [&](int m, int n, float v) { p.dw[(int64_t)m * p.in_dim + n] = v; };
+    small_f32_tile<false, false>(a, g_val, b, p.out_dim, p.in_dim, p.batch, (tb / nbn) * 64, (tb % nbn) * 64, store, As, Bs,
+                                add ? p.dw : nullptr, p.in_dim);
   } else {
     // bias_grad[out] (+)= column sums of g: 64 columns, four row lanes that meet in LDS
     int const col = (bid - p.tiles_dx - p.tiles_dw) * 64 + (threadIdx.x & 63);
     int const ry = threadIdx.x >> 6;
     float s = 0.0f;
-    for (int row = ry; row < p.batch; row += 4) s += g(row, col);
+    for (int row = ry; row < p.batch; row += 32) {  // eight loads in flight, added in row order
+      float2 v[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = g_raw(row + 4 * i, col);
+#pragma unroll
+      for (int i = 0; i < 8; i++) s += row + 4 * i < p.batch ? g_val(v[i]) : 0.0f;
+    }
     As[ry][threadIdx.x & 63] = s;
     __syncthreads();
     if (ry == 0 && col < p.out_dim) {
@@ -219,11 +250,11 @@ __global__ __launch_bounds__(256) void linear_small_fwd_f32_kernel(SmallLinearFw
   __shared__ float As[kSmallBK][68], Bs[kSmallBK][68];
   int const nbn = (p.out_dim + 63) / 64;
   auto a = [&](int m, int k) -> float {
-    return m < p.batch && k < p.in_dim ? p.x[(int64_t)m * p.in_dim + k] : 0.0f;
+    return p.x[(int64_t)(m < p.batch ? m : p.batch - 1) * p.in_dim + (k < p.in_dim ? k : p.in_dim - 1)];
   };
   // weight is [out, in]: b(k, n) = weight[n][k], k contiguous like the input's
   auto b = [&](int k, int n) -> float {
-    return k < p.in_dim && n < p.out_dim ? p.w[(int64_t)n * p.in_dim + k] : 0.0f;
+    return p.w[(int64_t)(n < p.out_dim ? n : p.out_dim - 1) * p.in_dim + (k < p.in_dim ? k : p.in_dim - 1)];
   };
   auto store = [&](int m, int n, float v) {
     v += p.bias != nullptr ? p.bias[n] : 0.0f;
@@ -236,13 +267,14 @@ __global__ __launch_bounds__(256) void linear_small_fwd_f32_kernel(SmallLinearFw
     }
     p.y[(int64_t)m * p.out_dim + n] = v;
   };
-  small_f32_tile<true, true>(a, b, p.batch, p.out_dim, p.in_dim, (blockIdx.x / nbn) * 64, (blockIdx.x % nbn) * 64, store, As, Bs);
+  small_f32_tile<true, true>(a, [](float v) { return v; }, b, p.batch, p.out_dim, p.in_dim, (blockIdx.x / nbn) * 64, (blockIdx.x % nbn) * 64, store, As, Bs);
 }
 
 // Small enough that launches, not work, set the time: at most two workgroups per CU in all.
 static bool small_linear_bwd(int dtype, int64_t batch, int64_t in_dim, int64_t out_dim, bool bias, int &tiles_dx,
                              int &tiles_dw, int &blocks) {
-  if (dtype != FFK_FLOAT || batch > 8192 || in_dim > (1 << 20) || out_dim > (1 << 20)) return false;
+  // a tile's reduction (out_dim for the input gradient, batch for the weight gradient) stays short
+  if (dtype != FFK_FLOAT || batch > kSmallMaxDepth || out_dim > kSmallMaxDepth || in_dim > (1 << 20)) return false;
   int64_t const tdx = ceil_div(batch, 64) * ceil_div(in_dim, 64), tdw = ceil_div(out_dim, 64) * ceil_div(in_dim, 64);
   int64_t const tb = bias ? ceil_div(out_dim, 64) : 0;
   if (tdx + tdw + tb > 2 * kNumCU) return false;
@@ -283,7 +315,7 @@ extern "C" int ffk_linear_forward(ffk_stream_t stream, int dtype,
               "linear_forward: non-positive dimension");
   FFK_REQUIRE(input && output && weight, "linear_forward: NULL tensor");
   if (dtype == FFK_FLOAT && batch <= 8192 && ceil_div(batch, 64) * ceil_div(out_dim, 64) <= 2 * kNumCU &&
-      in_dim <= (1 << 20)) {
+      in_dim <= kSmallMaxDepth) {
     SmallLinearFwd p = {static_cast<float const *>(input), static_cast<float const *>(weight),
                         static_cast<float const *>(bias), static_cast<float *>(output),
                         (int)batch, (int)in_dim, (int)out_dim, activation};
@@ -341,7 +373,12 @@ static int linear_backward_impl(
     p.accumulate = accumulate;
     p.tiles_dx = tiles_dx;
     p.tiles_dw = tiles_dw;
-    linear_small_bwd_f32_kernel<<<blocks, 256, 0, st>>>(p);
+    switch (activation) {
+      case FFK_ACT_RELU: linear_small_bwd_f32_kernel<FFK_ACT_RELU><<<blocks, 256, 0, st>>>(p); break;
+      case FFK_ACT_SIGMOID: linear_small_bwd_f32_kernel<FFK_ACT_SIGMOID><<<blocks, 256, 0, st>>>(p); break;
+      case FFK_ACT_TANH: linear_small_bwd_f32_kernel<FFK_ACT_TANH><<<blocks, 256, 0, st>>>(p); break;
+      default: linear_small_bwd_f32_kernel<FFK_ACT_NONE><<<blocks, 256, 0, st>>>(p); break;
+    }
     FFK_CHECK_LAUNCH();
     return FFK_OK;
   }

@@ -255,6 +255,39 @@ def bench_attention():
             report("  forward, 64 query rows per wavefront", t, flops=f)
         finally:
             ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, 0)
+    # the kernels for every other head size (multiples of 8 up to 256, value heads of their own
+    # size): 32 query rows per wavefront, head size padded to the next of 32 / 64 / 128 / 256
+    for (B, H, S, Dq, Dv, dt) in [(4, 8, 2048, 256, 256, BT), (4, 16, 2048, 96, 64, BT), (4, 16, 2048, 80, 80, BT),
+                                  (2, 8, 1024, 256, 256, torch.float32), (2, 8, 1024, 64, 64, torch.float32)]:
+        q, k = (torch.randn((B, S, H, Dq), device="cuda").to(dt) for _ in range(2))
+        v, do = (torch.randn((B, S, H, Dv), device="cuda").to(dt) for _ in range(2))
+        scale = 1.0 / math.sqrt(Dq)
+        o, lse = ffk.attention_forward(q, k, v, scale, False)
+        f = 2.0 * B * H * S * S * (Dq + Dv)
+        tag = "B%d H%d S%d Dq%d Dv%d %s" % (B, H, S, Dq, Dv, "bf16" if dt == BT else "fp32")
+        t = timeit(lambda: ffk.attention_forward(q, k, v, scale, False), iters=10)
+        report("attention fwd " + tag, t, flops=f)
+        t = timeit(lambda: ffk.attention_backward(q, k, v, o, do, lse, scale, False), iters=10)
+        report("attention bwd " + tag, t, flops=2.5 * f)
+
+
+def bench_small_linear():
+    # fp32 Linear at sizes where a launch costs more than the arithmetic: the forward is one
+    # launch of 64x64 tiles, the whole backward (dX, dW, bias sums) one launch
+    for (batch, in_dim, out_dim, act) in [(32, 64, 128, ffk.ACT_RELU), (256, 256, 256, ffk.ACT_NONE), (1024, 512, 512, ffk.ACT_RELU)]:
+        x = torch.randn((batch, in_dim), device="cuda")
+        w = torch.randn((out_dim, in_dim), device="cuda") * 0.1
+        b = torch.randn((out_dim,), device="cuda")
+        y = torch.empty((batch, out_dim), device="cuda")
+        dy = torch.randn((batch, out_dim), device="cuda")
+        dx, dw, db = torch.empty_like(x), torch.empty_like(w), torch.empty_like(b)
+        ffk.linear_forward(x, w, b, act, out=y)
+        t = timeit(lambda: ffk.linear_forward(x, w, b, act, out=y), iters=50)
+        report("Linear fp32 fwd [%d,%d]x[%d,%d]^T act %d" % (batch, in_dim, out_dim, in_dim, act), t, flops=2.0 * batch * in_dim * out_dim)
+        ws = torch.empty((max(1, ffk.lib().ffk_linear_backward_workspace_bytes(ffk.FLOAT, act, 1, batch, out_dim)),),
+                         dtype=torch.uint8, device="cuda")
+        t = timeit(lambda: ffk.linear_backward(y, dy, x, w, dx, dw, db, act, workspace=ws), iters=50)
+        report("Linear fp32 bwd (one launch)", t, flops=4.0 * batch * in_dim * out_dim)
 
 
 def bench_update():
@@ -338,7 +371,7 @@ def bench_shape():
     report("Gather backward (row sums in LDS) [16384,1024] -> [16384,4096]", t, bytes_=idx2.numel() * (4 + 4 + 8))
 
 
-GROUPS = dict(gemm=bench_gemm, fused_linear=bench_fused_linear, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention,
+GROUPS = dict(gemm=bench_gemm, fused_linear=bench_fused_linear, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention, small_linear=bench_small_linear,
               update=bench_update, shape=bench_shape)
 
 if __name__ == "__main__":

@@ -122,12 +122,13 @@ def test_linear_backward_with_l2_regularizer(ffk, oracle, dtype, shape):
 
 
 @pytest.mark.parametrize("act", [-1, 0, 1, 2])
-@pytest.mark.parametrize("shape", [(32, 64, 128), (70, 17, 65), (1, 1, 1), (300, 200, 130)])
+@pytest.mark.parametrize("shape", [(32, 64, 128), (70, 17, 65), (1, 1, 1), (300, 200, 130), (1024, 96, 80), (1100, 64, 72)])
 def test_small_fp32_backward_in_one_launch_equals_the_general_path(ffk, oracle, shape, act):
     """A small fp32 backward with all three gradients runs as ONE launch (activation gradient,
     both products and the bias sums as jobs of one grid); asked for one gradient at a time the
     same entry point takes the general path (one kernel per product).  Same values either way,
-    both against the oracle, with and without accumulation."""
+    both against the oracle, with and without accumulation.  The last shape's batch is beyond
+    the reduction depth the one-launch kernel takes: both calls go the general way."""
     batch, in_dim, out_dim = shape
     say("small fp32 linear backward, one launch vs general", shape, "act", act)
     x, w, b, dy = _cfg1_inputs(seed=11 + batch, batch=batch, in_dim=in_dim, out_dim=out_dim)
