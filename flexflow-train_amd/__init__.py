@@ -173,6 +173,7 @@ SIGNATURES = {
     "ffk_embedding_backward_workspace_bytes": (c_sz, [c_i64, c_i64]),
     "ffk_embedding_backward": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_int, c_i64, c_i64,
                                        c_i64, c_i64, c_int, c_p, c_sz]),
+    "ffk_embedding_backward_typed": (c_int, [c_p, c_int, c_int, c_p, c_p, c_p, c_int, c_i64, c_i64, c_i64, c_i64]),
     "ffk_attention_forward": (c_int, [c_p, c_int, ctypes.POINTER(AttentionDesc), c_p, c_p, c_p,
                                       c_p, c_p]),
     "ffk_attention_backward": (c_int, [c_p, c_int, ctypes.POINTER(AttentionDesc), c_p, c_p, c_p,
@@ -663,6 +664,20 @@ def embedding_backward(indices, out_grad, weight_grad, aggr=AGGR_NONE, determini
                                        ptr(indices), ptr(out_grad), ptr(weight_grad), aggr,
                                        num_bags, bag, D, V, int(deterministic), ptr(ws),
                                        ws_bytes))
+    return weight_grad
+
+
+def embedding_backward_typed(indices, out_grad, weight_grad, aggr=AGGR_NONE):
+    """HALF / DOUBLE (or FLOAT) tables: weight_grad has out_grad's dtype and is added to in that type."""
+    V, D = weight_grad.shape
+    assert out_grad.dtype == weight_grad.dtype
+    if aggr == AGGR_NONE:
+        num_bags, bag = indices.numel(), 1
+    else:
+        bag = indices.shape[-1]
+        num_bags = indices.numel() // bag
+    check(lib().ffk_embedding_backward_typed(current_stream(), dtype_of(indices), dtype_of(out_grad), ptr(indices),
+                                             ptr(out_grad), ptr(weight_grad), aggr, num_bags, bag, D, V))
     return weight_grad
 
 

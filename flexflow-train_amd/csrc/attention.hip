@@ -230,207 +230,6 @@ struct AttnBwdCfg {
   static_assert(kTile * D / 8 % 256 == 0, "tile chunks");
 };
 
-// (A) dK, dV: workgroup owns 128 key rows (32 per wave), streams query tiles.
-template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
-  using C = AttnBwdCfg<D>;
-  __shared__ __attribute__((aligned(16))) bf16 Qs[2][C::kTile * C::kStride];
-  __shared__ __attribute__((aligned(16))) bf16 Gs[2][C::kTile * C::kStride];  // dO
-  __shared__ __attribute__((aligned(16))) float Ls[2][C::kTile], Ds[2][C::kTile];
-  int const t = threadIdx.x, lane = t & 63, h32 = lane >> 5;
-  // the wave index as a scalar: tile-level decisions taken from it are branches, not lane masks
-  int const wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  // key block 0 sees every query under a causal mask: heaviest first for all heads
-  int const hb = blockIdx.x % (p.H * p.B);
-  int const head = hb % p.H, b = hb / p.H;
-  int const kv0 = (blockIdx.x / (p.H * p.B)) * C::kBlk;
-  int const kvrow = kv0 + wave * 32 + (lane & 31);
-  bf16 const *qp = p.q + (int64_t)b * p.q_bs + (int64_t)head * D;
-  bf16 const *gp = p.d_o + (int64_t)b * p.o_bs + (int64_t)head * D;
-  bf16 const *kp = p.k + (int64_t)b * p.k_bs + (int64_t)head * D;
-  bf16 const *vp = p.v + (int64_t)b * p.v_bs + (int64_t)head * D;
-  float const *lsep = p.lse + ((int64_t)b * p.H + head) * p.Sq;
-  float const *delp = p.delta + ((int64_t)b * p.H + head) * p.Sq;
-
-  // K and V rows of this lane as B operands (column = key row, k = d).
-  bf16x8 kf[D / 16], vf[D / 16];
-  {
-    int const r = min(kvrow, p.Skv - 1);
-#pragma unroll
-    for (int kk = 0; kk < D / 16; kk++) {
-      kf[kk] = *reinterpret_cast<bf16x8 const *>(kp + (int64_t)r * p.k_ss + kk * 16 + h32 * 8);
-      vf[kk] = *reinterpret_cast<bf16x8 const *>(vp + (int64_t)r * p.v_ss + kk * 16 + h32 * 8);
-    }
-  }
-  f32x16 dk[D / 32], dv[D / 32];
-#pragma unroll
-  for (int i = 0; i < D / 32; i++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      dk[i][r] = 0.0f;
-      dv[i][r] = 0.0f;
-    }
-
-  int const q_begin = p.causal ? (kv0 / C::kTile) * C::kTile : 0;
-  int const ntiles = (p.Sq - q_begin + C::kTile - 1) / C::kTile;
-
-  // Tiles travel global -> registers -> LDS.  Two register sets: the loads of
-  // tile it + 2 are issued at the start of step it and stored to LDS at the end
-  // of step it + 1, so a load has two steps to arrive (with one wave per SIMD
-  // nothing else covers the latency; one step was measured not to be enough).
-  // Tile n uses register set n % 2 and LDS buffer n % 2.
-  u32x4 rq[2][C::kChunks], rg[2][C::kChunks];
-  float rl[2] = {0.0f, 0.0f}, rd[2] = {0.0f, 0.0f};
-  auto gload = [&](int qt0, auto set_tag) {
-    constexpr int R = decltype(set_tag)::value;
-#pragma unroll
-    for (int i = 0; i < C::kChunks; i++) {
-      int c = t + i * 256;
-      int row = c / (D / 8), ch = c % (D / 8);
-      int gr = min(qt0 + row, p.Sq - 1);
-      rq[R][i] = *reinterpret_cast<u32x4 const *>(qp + (int64_t)gr * p.q_ss + ch * 8);
-      rg[R][i] = *reinterpret_cast<u32x4 const *>(gp + (int64_t)gr * p.o_ss + ch * 8);
-    }
-    // every lane loads (lanes >= kTile a duplicate): a load under a branch would make the
-    // number of loads in flight path-dependent and force full waits on the older tile
-    {
-      int gr = min(qt0 + (t & (C::kTile - 1)), p.Sq - 1);
-      rl[R] = lsep[gr] * kLog2e;
-      rd[R] = delp[gr];
-    }
-  };
-  auto lstore = [&](auto set_tag) {
-    constexpr int R = decltype(set_tag)::value;
-#pragma unroll
-    for (int i = 0; i < C::kChunks; i++) {
-      int c = t + i * 256;
-      int row = c / (D / 8), ch = c % (D / 8);
-      *reinterpret_cast<u32x4 *>(&Qs[R][row * C::kStride + ch * 8]) = rq[R][i];
-      *reinterpret_cast<u32x4 *>(&Gs[R][row * C::kStride + ch * 8]) = rg[R][i];
-    }
-    if (t < C::kTile) {
-      Ls[R][t] = rl[R];
-      Ds[R][t] = rd[R] * p.scale;  // delta * scale, so dS is one fma and one multiply per element
-    }
-  };
-  using Set0 = std::integral_constant<int, 0>;
-  using Set1 = std::integral_constant<int, 1>;
-
-  int const koff = lane_k_off(C::kStride, lane);
-  int const toff = lane_tr_off(C::kStride, lane);
-  if (ntiles > 0) {
-    gload(q_begin, Set0{});
-    lstore(Set0{});
-  }
-  // Tiles past the end are loaded too (their rows clamp to the last row, nothing is done with
-  // them): with the same loads in flight on every path, a step waits for exactly the tile it
-  // needs and leaves the younger prefetch in flight.
-  gload(q_begin + C::kTile, Set1{});
-  __syncthreads();
-  auto step = [&](int it, auto parity) {
-    constexpr int cur = decltype(parity)::value;  // == it % 2
-    int const qt0 = q_begin + it * C::kTile;
-    gload(qt0 + 2 * C::kTile, parity);
-    // A wave whose keys all lie after this query tile (causal) contributes 0.
-    bool const active = it < ntiles && (!p.causal || kv0 + wave * 32 <= qt0 + C::kTile - 1);
-    if (active) {
-      bf16 const *qk = Qs[cur] + koff, *gk = Gs[cur] + koff;
-      bf16 const *qtr = Qs[cur] + toff, *gtr = Gs[cur] + toff;
-      // S = Q K^T and dP = dO V^T: rows = queries of the tile, column = key.
-      f32x16 s, dp;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        s[r] = 0.0f;
-        dp[r] = 0.0f;
-      }
-#pragma unroll
-      for (int kk = 0; kk < D / 16; kk++) {
-        bf16x8 qa = frag_k(qk, C::kStride, 0, kk * 16);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s, 0, 0, 0);
-        bf16x8 ga = frag_k(gk, C::kStride, 0, kk * 16);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[kk], dp, 0, 0, 0);
-      }
-      float pv[16], dsv[16];
-      // wave-uniform: does any element of this wave's 32 x 32 block need masking?
-      bool const edge = qt0 + C::kTile > p.Sq || kv0 + wave * 32 + 32 > p.Skv || (p.causal && kv0 + wave * 32 + 31 > qt0);
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        // rows 8 g + 4 h + 0..3 of the tile: one 16-byte read each
-        f32x4 const lrow = *reinterpret_cast<f32x4 const *>(&Ls[cur][8 * g + 4 * h32]);
-        f32x4 const drow = *reinterpret_cast<f32x4 const *>(&Ds[cur][8 * g + 4 * h32]);
-#pragma unroll
-        for (int e4 = 0; e4 < 4; e4++) {
-          int const r = 4 * g + e4;
-          float const e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], p.scale_log2, -lrow[e4]));
-          pv[r] = e;
-          // dS = P (dP - delta) scale; Ds holds delta * scale
-          dsv[r] = e * __builtin_fmaf(dp[r], p.scale, -drow[e4]);
-        }
-      }
-      if (edge) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          int const qg = qt0 + 8 * (r >> 2) + 4 * h32 + (r & 3);
-          bool const masked = qg >= p.Sq || kvrow >= p.Skv || (p.causal && kvrow > qg);
-          pv[r] = masked ? 0.0f : pv[r];
-          dsv[r] = masked ? 0.0f : dsv[r];
-        }
-      }
-      // dV += P^T dO ; dK += dS^T Q.  A = accumulator re-used (row = key),
-      // B = dO / Q read with the matching reduction order (k = query).
-#pragma unroll
-      for (int s2 = 0; s2 < 2; s2++) {
-        bf16x8 pa = pack8(pv + 8 * s2);
-        bf16x8 da = pack8(dsv + 8 * s2);
-#pragma unroll
-        for (int i = 0; i < D / 32; i++) {
-          bf16x8 gb = frag_tr_acc(gtr, C::kStride, 0, s2, i * 32);
-          dv[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa, gb, dv[i], 0, 0, 0);
-          bf16x8 qb = frag_tr_acc(qtr, C::kStride, 0, s2, i * 32);
-          dk[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, qb, dk[i], 0, 0, 0);
-        }
-      }
-    }
-    if (it + 1 < ntiles) lstore(std::integral_constant<int, cur ^ 1>{});
-    __syncthreads();
-  };
-  // always in pairs (an odd count runs one idle step): the loop body then issues the same
-  // loads whatever the tile count, which keeps the waits on them exact
-  for (int it = 0; it < ntiles; it += 2) {
-    step(it, Set0{});
-    step(it + 1, Set1{});
-  }
-
-  // dK / dV accumulators: row = key (32 per wave, 8*(r/4)+4*h+r%4), column = d: a lane
-  // holds one column of 16 rows.  Each wave turns its 32 x D block around in LDS (the
-  // streamed tiles are done with) and writes whole 16-byte pieces of rows.
-  __syncthreads();
-  constexpr int kOutStride = D + 8;
-  bf16 *const stage = (wave < 2 ? &Qs[0][0] : &Gs[0][0]) + (wave & 1) * 32 * kOutStride;
-  static_assert(2 * 32 * kOutStride <= 2 * C::kTile * C::kStride, "staging fits the tile buffers");
-  auto write_out = [&](f32x16 const (&acc)[D / 32], bf16 *out, int64_t row_stride) {
-#pragma unroll
-    for (int i = 0; i < D / 32; i++) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        int const row = 8 * (r >> 2) + 4 * h32 + (r & 3);
-        VecIO<bf16>::store1(stage + row * kOutStride + i * 32 + (lane & 31), acc[i][r]);
-      }
-    }
-    // LDS operations of one wave complete in order: the reads below see the writes above
-#pragma unroll
-    for (int k = 0; k < 32 * (D / 8) / 64; k++) {
-      int const c = lane + k * 64;
-      int const row = c / (D / 8), ch = c % (D / 8);
-      u32x4 const v = *reinterpret_cast<u32x4 const *>(stage + row * kOutStride + ch * 8);
-      int const grow = kv0 + wave * 32 + row;
-      if (grow < p.Skv) *reinterpret_cast<u32x4 *>(out + (int64_t)grow * row_stride + ch * 8) = v;
-    }
-  };
-  write_out(dk, p.dk + (int64_t)b * p.k_bs + (int64_t)head * D, p.k_ss);
-  write_out(dv, p.dv + (int64_t)b * p.v_bs + (int64_t)head * D, p.v_ss);
-}
-
 // (B) dQ: workgroup owns 128 query rows (32 per wave), streams key tiles.
 template <int D>
 __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
@@ -597,7 +396,6 @@ hipError_t attention_bf16_forward_wide(hipStream_t st, AttnParams const &p, int 
 // dK/dV with direct loads, one workgroup per CU: its three Q and three dO tile buffers take
 // 48 KB (head size 64) or 96 KB (128) of LDS, and one wave per SIMD holds the accumulators (attention_bwd.hip)
 hipError_t attention_bf16_dkdv(hipStream_t st, AttnBwdParams const &p, int head_dim);
-bool attention_bf16_bwd_direct_ok(AttnBwdParams const &p);
 
 // the fp32 core (attention_f32.hip)
 int attention_f32_forward(hipStream_t st, ffk_attention_desc_t const *d, void const *q, void const *k,
@@ -709,7 +507,11 @@ extern "C" int ffk_attention_backward(ffk_stream_t stream, int dtype,
   }
   int rc = check_desc("attention_backward", dtype, d);
   if (rc != FFK_OK) return rc;
-  if (!tuned_head_size(d)) {
+  // (the tuned dK/dV kernel addresses a batch entry's rows with 32-bit byte offsets)
+  int64_t const lim = int64_t(1) << 32;
+  bool const offsets_fit = d->seq_q * d->q_seq_stride * 2 < lim && d->seq_q * d->o_seq_stride * 2 < lim &&
+                           d->seq_kv * d->k_seq_stride * 2 < lim && d->seq_kv * d->v_seq_stride * 2 < lim;
+  if (!tuned_head_size(d) || !offsets_fit) {
     return attention_bf16_general_backward(as_stream(stream), d, q, k, v, o, d_o, lse, delta, dq, dk, dv);
   }
   AttnBwdParams p;
@@ -732,27 +534,15 @@ extern "C" int ffk_attention_backward(ffk_stream_t stream, int dtype,
   p.scale_log2 = d->scale * kLog2e;
   p.causal = d->causal;
   hipStream_t st = as_stream(stream);
-  bool const direct = option(FFK_OPTION_ATTENTION_VARIANT) != 1 && attention_bf16_bwd_direct_ok(p);
-  dim3 gkv((unsigned)(ceil_div(p.Skv, 128) * p.H * p.B));
-  dim3 gq((unsigned)(ceil_div(p.Sq, 128) * p.H * p.B));
   // dQ first: it computes delta for its rows and leaves it in `delta` for the dK/dV kernel
+  dim3 gq((unsigned)(ceil_div(p.Sq, 128) * p.H * p.B));
   if (d->head_dim == 64) {
     attn_bwd_dq_kernel<64><<<gq, 256, 0, st>>>(p);
-    FFK_CHECK_LAUNCH();
-    if (direct) {
-      FFK_HIP(attention_bf16_dkdv(st, p, 64));
-    } else {
-      attn_bwd_dkdv_kernel<64><<<gkv, 256, 0, st>>>(p);
-    }
   } else {
     attn_bwd_dq_kernel<128><<<gq, 256, 0, st>>>(p);
-    FFK_CHECK_LAUNCH();
-    if (direct) {
-      FFK_HIP(attention_bf16_dkdv(st, p, 128));
-    } else {
-      attn_bwd_dkdv_kernel<128><<<gkv, 256, 0, st>>>(p);
-    }
   }
+  FFK_CHECK_LAUNCH();
+  FFK_HIP(attention_bf16_dkdv(st, p, (int)d->head_dim));
   FFK_CHECK_LAUNCH();
   return FFK_OK;
 }

@@ -362,12 +362,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv2_kernel(AttnBwdParams p) {
 
 // Whether the kernels of this file can address the problem: a tile's byte offset inside a
 // (batch, head)'s rows is a 32-bit scalar.
-bool attention_bf16_bwd_direct_ok(AttnBwdParams const &p) {
-  int64_t const lim = int64_t(1) << 32;
-  return (int64_t)p.Sq * p.q_ss * 2 < lim && (int64_t)p.Sq * p.o_ss * 2 < lim && (int64_t)p.Skv * p.k_ss * 2 < lim &&
-         (int64_t)p.Skv * p.v_ss * 2 < lim;
-}
-
 hipError_t attention_bf16_dkdv(hipStream_t st, AttnBwdParams const &p, int head_dim) {
   dim3 grid((unsigned)(ceil_div(p.Skv, 128) * p.H * p.B));
   if (head_dim == 64) {

@@ -179,6 +179,65 @@ __global__ __launch_bounds__(kEmbThreads) void embedding_fwd_scalar_kernel(
   }
 }
 
+// HALF and DOUBLE tables (embedding_kernels.cu:374-449,491-566 forward, 609-808 backward): table,
+// output and gradients share one type T and all arithmetic is T's own, as in the reference -- a bag
+// is summed in T entry by entry, the backward adds T values atomically.  One thread per (bag,
+// column); no configuration uses these types, so nothing here is tuned.
+template <typename IT, typename T>
+__global__ __launch_bounds__(kEmbThreads) void embedding_fwd_typed_kernel(
+    IT const *__restrict__ idx, T *__restrict__ out, T const *__restrict__ W,
+    int64_t num_bags, int bag, int64_t dim, int64_t num_entries, bool avg) {
+  int64_t const total = num_bags * dim;
+  int64_t const stride = (int64_t)gridDim.x * kEmbThreads;
+  T const scale = (T)(1.0f / (float)bag);  // the reference's `TD scale = 1.0f / in_dim`
+  for (int64_t i = (int64_t)blockIdx.x * kEmbThreads + threadIdx.x; i < total; i += stride) {
+    int64_t const b = i / dim, d = i % dim;
+    T acc = (T)0;
+    for (int j = 0; j < bag; j++) {
+      int64_t const r = (int64_t)idx[b * bag + j];
+      if ((uint64_t)r < (uint64_t)num_entries) acc = acc + W[r * dim + d];
+    }
+    if (avg) acc = acc * scale;
+    out[i] = acc;
+  }
+}
+
+__device__ __forceinline__ void atomic_add_typed(double *p, double v) { atomicAdd(p, v); }
+// no 16-bit atomic: compare-and-swap on the aligned word that holds the half
+__device__ __forceinline__ void atomic_add_typed(_Float16 *p, _Float16 v) {
+  uintptr_t const a = reinterpret_cast<uintptr_t>(p);
+  uint32_t *word = reinterpret_cast<uint32_t *>(a & ~(uintptr_t)3);
+  bool const high = (a & 2) != 0;
+  uint32_t seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (;;) {
+    uint16_t const bits = high ? (uint16_t)(seen >> 16) : (uint16_t)(seen & 0xffffu);
+    _Float16 const sum = __builtin_bit_cast(_Float16, bits) + v;
+    uint32_t const sb = __builtin_bit_cast(uint16_t, sum);
+    uint32_t const want = high ? (seen & 0x0000ffffu) | (sb << 16) : (seen & 0xffff0000u) | sb;
+    uint32_t const prev = atomicCAS(word, seen, want);
+    if (prev == seen) break;
+    seen = prev;
+  }
+}
+
+template <typename IT, typename T>
+__global__ __launch_bounds__(kEmbThreads) void embedding_bwd_typed_kernel(
+    IT const *__restrict__ idx, T const *__restrict__ dY, T *dW,
+    int64_t num_bags, int bag, int64_t dim, int64_t num_entries, bool avg) {
+  int64_t const total = num_bags * dim;
+  int64_t const stride = (int64_t)gridDim.x * kEmbThreads;
+  T const scale = (T)(1.0f / (float)bag);
+  for (int64_t i = (int64_t)blockIdx.x * kEmbThreads + threadIdx.x; i < total; i += stride) {
+    int64_t const b = i / dim, d = i % dim;
+    T g = dY[i];
+    if (avg) g = g * scale;
+    for (int j = 0; j < bag; j++) {
+      int64_t const r = (int64_t)idx[b * bag + j];
+      if ((uint64_t)r < (uint64_t)num_entries) atomic_add_typed(dW + r * dim + d, g);
+    }
+  }
+}
+
 // One wave per (bag, 64-float column segment): every atomic instruction of the
 // wave covers 256 contiguous bytes of one weight-gradient row.
 template <typename IT, typename GT>
@@ -686,6 +745,22 @@ extern "C" int ffk_embedding_forward(ffk_stream_t stream, int index_dtype,
     if (weight_dtype == FFK_BF16 && output_dtype == FFK_FLOAT) FFK_EMB_FWD(int64_t, bf16, float);
   }
 #undef FFK_EMB_FWD
+  if (weight_dtype == output_dtype && (weight_dtype == FFK_HALF || weight_dtype == FFK_DOUBLE) &&
+      (index_dtype == FFK_INT32 || index_dtype == FFK_INT64)) {
+    bool const avg = aggr == FFK_AGGR_AVG;
+    int const grid = emb_grid(num_bags * dim);
+#define FFK_EMB_TYPED(IT, T)                                                   \
+  embedding_fwd_typed_kernel<IT, T><<<grid, kEmbThreads, 0, st>>>(             \
+      static_cast<IT const *>(indices), static_cast<T *>(output), static_cast<T const *>(weight), num_bags, (int)bag, \
+      dim, num_entries, avg)
+    if (index_dtype == FFK_INT32 && weight_dtype == FFK_HALF) FFK_EMB_TYPED(int32_t, _Float16);
+    else if (index_dtype == FFK_INT32) FFK_EMB_TYPED(int32_t, double);
+    else if (weight_dtype == FFK_HALF) FFK_EMB_TYPED(int64_t, _Float16);
+    else FFK_EMB_TYPED(int64_t, double);
+#undef FFK_EMB_TYPED
+    FFK_CHECK_LAUNCH();
+    return FFK_OK;
+  }
   return fail(FFK_ERR_UNSUPPORTED,
               "embedding_forward: dtypes (index %d, weight %d, output %d) not supported",
               index_dtype, weight_dtype, output_dtype);
@@ -727,4 +802,37 @@ extern "C" int ffk_embedding_backward(ffk_stream_t stream, int index_dtype,
   return fail(FFK_ERR_UNSUPPORTED,
               "embedding_backward: dtypes (index %d, grad %d) not supported",
               index_dtype, output_grad_dtype);
+}
+
+extern "C" int ffk_embedding_backward_typed(ffk_stream_t stream, int index_dtype, int dtype,
+                                            void const *indices, void const *output_grad,
+                                            void *weight_grad, int aggr, int64_t num_bags,
+                                            int64_t bag, int64_t dim, int64_t num_entries) {
+  if (dtype == FFK_FLOAT) {
+    return ffk_embedding_backward(stream, index_dtype, FFK_FLOAT, indices, output_grad,
+                                  static_cast<float *>(weight_grad), aggr, num_bags, bag, dim, num_entries, 0,
+                                  nullptr, 0);
+  }
+  int rc = check_common("embedding_backward_typed", aggr, num_bags, bag, dim, num_entries);
+  if (rc != FFK_OK) return rc;
+  FFK_REQUIRE(dtype == FFK_HALF || dtype == FFK_DOUBLE,
+              "embedding_backward_typed: dtype %d not supported (HALF, FLOAT or DOUBLE)", dtype);
+  FFK_REQUIRE(index_dtype == FFK_INT32 || index_dtype == FFK_INT64,
+              "embedding_backward_typed: index dtype %d not supported", index_dtype);
+  if (num_bags == 0) return FFK_OK;
+  FFK_REQUIRE(indices && output_grad && weight_grad, "embedding_backward_typed: NULL tensor");
+  hipStream_t st = as_stream(stream);
+  bool const avg = aggr == FFK_AGGR_AVG;
+  int const grid = emb_grid(num_bags * dim);
+#define FFK_EMB_TYPED(IT, T)                                                   \
+  embedding_bwd_typed_kernel<IT, T><<<grid, kEmbThreads, 0, st>>>(             \
+      static_cast<IT const *>(indices), static_cast<T const *>(output_grad), static_cast<T *>(weight_grad), num_bags, \
+      (int)bag, dim, num_entries, avg)
+  if (index_dtype == FFK_INT32 && dtype == FFK_HALF) FFK_EMB_TYPED(int32_t, _Float16);
+  else if (index_dtype == FFK_INT32) FFK_EMB_TYPED(int32_t, double);
+  else if (dtype == FFK_HALF) FFK_EMB_TYPED(int64_t, _Float16);
+  else FFK_EMB_TYPED(int64_t, double);
+#undef FFK_EMB_TYPED
+  FFK_CHECK_LAUNCH();
+  return FFK_OK;
 }

@@ -500,11 +500,23 @@ void backward_kernel(device_stream_t const &stream, GenericTensorAccessorR const
                      DataType output_data_type, DataType input_data_type, std::optional<AggregateOp> aggr,
                      num_tensor_dims_t, num_tensor_dims_t, int) {
   if (!stream.is_gpu()) no_cpu("Embedding::backward_kernel");
-  if (weight_grad.shape.data_type != DataType::FLOAT) {
-    throw std::runtime_error("Embedding::backward_kernel: weight_grad must be FLOAT (fp32 accumulators)");
-  }
   int64_t num_bags, bag;
   bag_geometry(input, aggr, num_bags, bag);
+  if (weight_grad.shape.data_type == DataType::HALF || weight_grad.shape.data_type == DataType::DOUBLE) {
+    // the reference's half / double instantiations: one type throughout (embedding_kernels.cu:609-808)
+    if (output_data_type != weight_grad.shape.data_type) {
+      throw std::runtime_error("Embedding::backward_kernel: a HALF or DOUBLE weight_grad takes an output gradient of its type");
+    }
+    check_ffk(ffk_embedding_backward_typed(stream.require_gpu(), dt(input_data_type), dt(output_data_type), input.ptr,
+                                           output.ptr, weight_grad.ptr,
+                                           aggr.has_value() ? static_cast<int>(*aggr) : FFK_AGGR_NONE, num_bags, bag,
+                                           dim_at_idx(weight_grad.shape.dims, 1), dim_at_idx(weight_grad.shape.dims, 0)),
+              "Embedding::backward_kernel");
+    return;
+  }
+  if (weight_grad.shape.data_type != DataType::FLOAT) {
+    throw std::runtime_error("Embedding::backward_kernel: weight_grad must be FLOAT (fp32 accumulators), HALF or DOUBLE");
+  }
   check_ffk(ffk_embedding_backward(stream.require_gpu(), dt(input_data_type), dt(output_data_type), input.ptr,
                                    output.ptr, static_cast<float *>(weight_grad.ptr),
                                    aggr.has_value() ? static_cast<int>(*aggr) : FFK_AGGR_NONE, num_bags, bag,

@@ -495,6 +495,30 @@ static void gpu_tests() {
     CHECK(to_host(O) == out);
     Kernels::Embedding::backward_kernel(stream, DYa, I, DW, DataType::FLOAT, DataType::INT32, AggregateOp::SUM, 2, 2, (int)B);
     CHECK(close(to_host(DW), dw, 1e-5));
+    // DOUBLE tables (the reference instantiates HALF, FLOAT and DOUBLE): one type throughout.  The
+    // values are quarters of small integers, so every sum is exact in fp32 as in double and the
+    // fp32 oracle's result, widened, is the expected one to the bit.
+    std::vector<double> wd(V * D), dyd(B * D);
+    std::vector<float> wq(V * D), dyq(B * D), outq(B * D), dwq(V * D, 0.0f);
+    for (size_t i = 0; i < wd.size(); i++) wd[i] = wq[i] = (float)((int)(gen() % 65) - 32) / 4.0f;
+    for (size_t i = 0; i < dyd.size(); i++) dyd[i] = dyq[i] = (float)((int)(gen() % 33) - 16) / 4.0f;
+    orc_embedding_forward(idx.data(), outq.data(), wq.data(), 0, B, bag, D, V);
+    orc_embedding_backward(idx.data(), dyq.data(), dwq.data(), 0, B, bag, D, V);
+    GenericTensorAccessorW hw = cpu.allocate_tensor(shape({V, D}, DataType::DOUBLE)), hdy = cpu.allocate_tensor(shape({B, D}, DataType::DOUBLE));
+    memcpy(hw.ptr, wd.data(), wd.size() * 8);
+    memcpy(hdy.ptr, dyd.data(), dyd.size() * 8);
+    GenericTensorAccessorW Wd = copy_tensor_accessor_w(hw, gpu), DYd = copy_tensor_accessor_w(hdy, gpu);
+    auto Od = gpu.allocate_tensor(shape({B, D}, DataType::DOUBLE)), DWd = gpu.allocate_tensor(Wd.shape);
+    fill_with_zeros(DWd);
+    Kernels::Embedding::forward_kernel(stream, I, Od, Wd, DataType::INT32, DataType::DOUBLE, AggregateOp::SUM, 2, 2, (int)B);
+    Kernels::Embedding::backward_kernel(stream, DYd, I, DWd, DataType::DOUBLE, DataType::INT32, AggregateOp::SUM, 2, 2, (int)B);
+    GenericTensorAccessorW hod = copy_tensor_accessor_w(Od, cpu), hdwd = copy_tensor_accessor_w(DWd, cpu);
+    bool same = true;
+    for (int64_t i = 0; i < B * D; i++) same = same && hod.get<DataType::DOUBLE>()[i] == (double)outq[i];
+    for (int64_t i = 0; i < V * D; i++) same = same && hdwd.get<DataType::DOUBLE>()[i] == (double)dwq[i];
+    CHECK(same);
+    // a FLOAT gradient into a DOUBLE weight_grad is refused
+    CHECK_THROWS(Kernels::Embedding::backward_kernel(stream, DYa, I, DWd, DataType::FLOAT, DataType::INT32, AggregateOp::SUM, 2, 2, (int)B));
   });
 
   run("MultiHeadAttention (bf16 accessors) vs oracle", [&] {

@@ -140,12 +140,9 @@ int ffk_probe_mfma_bf16(ffk_stream_t stream, int iterations, uint32_t seed,
  *   FFK_OPTION_LAYER_UNFUSED: != 0 makes the encoder-layer
  *     entry points (and a step-driver instance created while it is set) run
  *     one kernel per operator.
- *   FFK_OPTION_ATTENTION_VARIANT: 0 = the default bf16
- *     attention kernels (forward: 64 query rows per wavefront from 1024 keys
- *     on, 32 below; dK/dV: 64-row query tiles as two pipelined halves);
- *     1 = the forward kernel with 32 query rows per wavefront and the dK/dV
- *     kernel with 32-row query tiles at every size; 2 = the forward kernel
- *     with 64 query rows per wavefront at every size.                        */
+ *   FFK_OPTION_ATTENTION_VARIANT: which of the two tuned bf16 forward
+ *     kernels runs: 0 = 64 query rows per wavefront from 1024 keys on, 32
+ *     below; 1 = 32 rows at every size; 2 = 64 rows at every size.          */
 enum {
   FFK_OPTION_GEMM_VARIANT = 0,
   FFK_OPTION_LAYER_UNFUSED = 1,
@@ -517,7 +514,9 @@ int ffk_layer_norm_backward_residual(
  * (embedding_kernels_gpu.h:10-28; lib/kernels/src/cuda/embedding_kernels.cu:
  * 48-317,811-853).  indices [num_bags, bag] (bag == 1 with FFK_AGGR_NONE),
  * index_dtype FFK_INT32 or FFK_INT64; weight [num_entries, dim]; output
- * [num_bags, dim].  AVG divides the bag sum by `bag` (not the reference's
+ * [num_bags, dim]; weight / output FFK_FLOAT or FFK_BF16 in any pairing, or both
+ * FFK_HALF or both FFK_DOUBLE (see ffk_embedding_backward_typed).
+ * AVG divides the bag sum by `bag` (not the reference's
  * scale-inside-the-loop, embedding_kernels.cu:85-98).
  * forward:  output[b,:] = sum_j weight[indices[b,j],:]
  * backward: weight_grad[indices[b,j],:] += output_grad[b,:] (* 1/bag for AVG),
@@ -544,6 +543,18 @@ int ffk_embedding_backward(ffk_stream_t stream, int index_dtype,
                            int aggr, int64_t num_bags, int64_t bag, int64_t dim,
                            int64_t num_entries, int deterministic,
                            void *workspace, size_t workspace_bytes);
+/* The reference's HALF and DOUBLE instantiations (embedding_kernels.cu:374-449,
+ * 491-566 forward; 609-808 backward): table, output and both gradients have one
+ * type and all arithmetic is that type's, as there -- ffk_embedding_forward with
+ * weight_dtype == output_dtype == FFK_HALF or FFK_DOUBLE sums a bag in that type
+ * entry by entry; this entry point adds output_grad (* T(1/bag) for AVG) into
+ * weight_grad of the same dtype with atomics (compare-and-swap for HALF).
+ * dtype FFK_FLOAT forwards to ffk_embedding_backward without workspace.
+ * One thread per element: correct, not tuned (no configuration uses them). */
+int ffk_embedding_backward_typed(ffk_stream_t stream, int index_dtype, int dtype,
+                                 void const *indices, void const *output_grad,
+                                 void *weight_grad, int aggr, int64_t num_bags,
+                                 int64_t bag, int64_t dim, int64_t num_entries);
 
 /* ------------------------------------------------------------------------ */
 /* Fused (flash-style) scaled-dot-product attention core: the QK^T / softmax /

@@ -242,14 +242,11 @@ def bench_attention():
         report("attention fwd B%d H%d S%d D%d causal=%d" % (B, H, S, D, causal), t, flops=f)
         t = timeit(lambda: ffk.attention_backward(q, k, v, o, do, lse, scale, causal), iters=10)
         report("attention bwd B%d H%d S%d D%d causal=%d" % (B, H, S, D, causal), t, flops=2.5 * f)
-        # the other kernels: 32 query rows per wavefront forward and 32-row tiles in dK/dV (the
-        # defaults before), then the forward with 64 rows per wavefront whatever the size
+        # the other forward kernel at this size: 32 query rows per wavefront, then 64 whatever the size
         try:
             ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, 1)
             t = timeit(lambda: ffk.attention_forward(q, k, v, scale, causal), iters=10)
             report("  forward, 32 query rows per wavefront", t, flops=f)
-            t = timeit(lambda: ffk.attention_backward(q, k, v, o, do, lse, scale, causal), iters=10)
-            report("  backward with the 32-row-tile dK/dV kernel", t, flops=2.5 * f)
             ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, 2)
             t = timeit(lambda: ffk.attention_forward(q, k, v, scale, causal), iters=10)
             report("  forward, 64 query rows per wavefront", t, flops=f)

@@ -349,6 +349,54 @@ def embedding_backward(indices, out_grad, num_entries, aggr=-1, f64=False, dw_in
     return dw
 
 
+def _bags(indices, aggr):
+    idx = np.ascontiguousarray(indices, dtype=np.int64)
+    if idx.ndim == 1 or aggr < 0:
+        return idx.reshape(-1, 1)
+    return idx.reshape(-1, idx.shape[-1])
+
+
+def embedding_forward_typed(indices, weight, aggr=-1):
+    """The reference's HALF / DOUBLE instantiations (embedding_kernels.cu:48-125 with TD = half or
+    double): the bag is summed entry by entry in the table's own type (numpy's float16 add is the
+    correctly rounded one: two halves add exactly in the float32 it goes through unless one is
+    below an eighth of the other's last place, where no rounding boundary is near); AVG
+    multiplies the sum by TD(1.0f / bag) -- once, the same true average as orc_embedding_forward,
+    not the reference's multiplication inside the loop."""
+    weight = np.asarray(weight)
+    assert weight.dtype in (np.float16, np.float64)
+    idx2 = _bags(indices, aggr)
+    num_bags, bag = idx2.shape
+    if idx2.min() < 0 or idx2.max() >= weight.shape[0]:
+        raise ValueError("embedding_forward_typed: index out of range")
+    acc = np.zeros((num_bags, weight.shape[1]), weight.dtype)
+    for j in range(bag):
+        acc = (acc + weight[idx2[:, j]]).astype(weight.dtype)
+    if aggr == 1:
+        acc = (acc * weight.dtype.type(np.float32(1.0) / np.float32(bag))).astype(weight.dtype)
+    return acc
+
+
+def embedding_backward_typed(indices, out_grad, num_entries, aggr=-1, dw_init=None):
+    """embedding_kernels.cu:128-317 with TD = half or double and the atomics replaced by adds in
+    lookup order: weight_grad[row] += out_grad[bag] (* TD(1.0f / bag) for AVG), every add rounded
+    to TD.  (The device's order is not fixed: tests use sums that are exact in TD.)"""
+    g = np.asarray(out_grad)
+    assert g.dtype in (np.float16, np.float64)
+    idx2 = _bags(indices, aggr)
+    num_bags, bag = idx2.shape
+    dw = np.zeros((num_entries, g.shape[-1]), g.dtype) if dw_init is None else np.array(dw_init, dtype=g.dtype)
+    if aggr == 1:
+        g = (g * g.dtype.type(np.float32(1.0) / np.float32(bag))).astype(g.dtype)
+    for b in range(num_bags):
+        for j in range(bag):
+            row = idx2[b, j]
+            if row < 0 or row >= num_entries:
+                raise ValueError("embedding_backward_typed: index out of range")
+            dw[row] = (dw[row] + g[b]).astype(g.dtype)
+    return dw
+
+
 def attention_forward(q, k, v, scale, causal, bf16_mode=False):
     """q [B,Sq,H,D], k [B,Skv,H,D], v [B,Skv,H,Dv] -> o [B,Sq,H,Dv], lse [B,H,Sq]."""
     q, k, v = _f32(q), _f32(k), _f32(v)

@@ -88,9 +88,8 @@ def test_attention_forward_kernels(ffk, oracle, shape, causal, variant):
 @pytest.mark.parametrize("shape", FWD_SHAPES)
 @pytest.mark.parametrize("causal", [False, True])
 def test_attention_backward_kernels(ffk, oracle, shape, causal):
-    """The dK/dV kernel that streams 64-row query tiles as two pipelined halves (default) against
-    the oracle, and against the kernel it replaced (option 1: 32-row tiles, one at a time): both
-    add up the same products in the same order, so the gradients agree to the bit."""
+    """The tuned backward kernels (dQ; dK/dV streaming 64-row query tiles as two pipelined halves)
+    against the oracle; nothing in them is atomic, so a second run gives the same bits."""
     B, H, Sq, Skv, D = shape
     say("attention backward", shape, "causal", causal)
     g = rng(Sq * 5 + Skv + D + int(causal))
@@ -101,17 +100,12 @@ def test_attention_backward_kernels(ffk, oracle, shape, causal):
     scale = 1.0 / np.sqrt(D)
     qd, kd, vd, dod = (to_dev(a, torch, BT) for a in (q, k, v, do))
     o, lse = ffk.attention_forward(qd, kd, vd, scale, causal)
-    grads = {}
-    try:
-        for variant in (0, 1):
-            ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, variant)
-            grads[variant] = ffk.attention_backward(qd, kd, vd, o, dod, lse, scale, causal)
-    finally:
-        ffk.set_option(ffk.OPTION_ATTENTION_VARIANT, 0)
+    grads = ffk.attention_backward(qd, kd, vd, o, dod, lse, scale, causal)
+    again = ffk.attention_backward(qd, kd, vd, o, dod, lse, scale, causal)
     dq_ref, dk_ref, dv_ref = oracle.attention_backward(q, k, v, do, scale, causal)
-    for name, got, want in zip(("dQ", "dK", "dV"), grads[0], (dq_ref, dk_ref, dv_ref)):
+    for name, got, want in zip(("dQ", "dK", "dV"), grads, (dq_ref, dk_ref, dv_ref)):
         assert_close(to_np(got), want, BF16_RTOL, name)
-    for name, a, b in zip(("dQ", "dK", "dV"), grads[0], grads[1]):
+    for name, a, b in zip(("dQ", "dK", "dV"), grads, again):
         assert torch.equal(a, b), name
 
 

@@ -143,3 +143,57 @@ def test_scatter_add_modes(ffk, oracle, mode, idt, gdt, V, D, B, bag):
         dw2 = torch.zeros((V, D), device="cuda")
         ffk.embedding_backward(to_dev(ids_dev, torch, idt), to_dev(dy, torch, gdt), dw2, aggr=aggr, **kw)
         assert torch.equal(dw, dw2)
+
+
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+@pytest.mark.parametrize("dt,ndt", [(torch.float16, np.float16), (torch.float64, np.float64)])
+@pytest.mark.parametrize("aggr,V,D,B,bag", [(-1, 97, 33, 50, 1), (0, 1000, 128, 64, 32), (1, 100, 17, 9, 5),
+                                            (1, 40, 8, 700, 4)])
+def test_half_and_double_tables(ffk, oracle, idt, dt, ndt, aggr, V, D, B, bag):
+    """The reference's HALF and DOUBLE instantiations: table, output and gradients of one type, all
+    arithmetic in that type.  Forward: the bag is summed entry by entry, so the oracle's order
+    is the device's and random data must match to the bit.  Backward: the atomics' order is
+    free, so the gradients are eighths of small integers, whose sums are exact in half whatever
+    the order (|sum| <= 700 * 4 * 2 / 8 < 2048 / 8 steps) -- bit-exact again."""
+    say("embedding HALF/DOUBLE tables", idt, dt, (aggr, V, D, B, bag))
+    g = rng(V + B + bag)
+    w = g.standard_normal((V, D)).astype(ndt)
+    ids = zipf_ids(g, B * bag, V).reshape(B, bag) if aggr >= 0 else zipf_ids(g, B, V)
+    want = oracle.embedding_forward_typed(ids, w, aggr=aggr)
+    wd, idd = torch.from_numpy(w).cuda(), to_dev(ids, torch, idt)
+    out = ffk.embedding_forward(idd, wd, aggr=aggr)
+    assert out.dtype == dt
+    assert np.array_equal(out.cpu().numpy(), want)
+    # backward: exact sums; AVG's factor half(1/bag) is exact for bag 4 and rounds for bag 5, and is
+    # applied to the gradient once per bag, before the adds, in the oracle as on the device
+    dy = (g.integers(-2, 3, (ids.shape[0], D)) * (bag if aggr == 1 and bag == 4 else 1) / 8.0).astype(ndt)
+    init = (g.integers(-4, 5, (V, D)) / 4.0).astype(ndt)
+    if aggr == 1 and bag == 5:
+        # half(1/5) times an eighth is not a short binary fraction: keep every row's lookups few
+        # enough that order cannot matter by giving each lookup its own row
+        ids = g.permutation(V)[:B * bag].reshape(B, bag) if B * bag <= V else ids
+        idd = to_dev(ids, torch, idt)
+    want_dw = oracle.embedding_backward_typed(ids, dy, V, aggr=aggr, dw_init=init)
+    dw = torch.from_numpy(init).cuda()
+    ffk.embedding_backward_typed(idd, torch.from_numpy(dy).cuda(), dw, aggr=aggr)
+    assert dw.dtype == dt
+    assert np.array_equal(dw.cpu().numpy(), want_dw)
+
+
+def test_half_and_double_tables_errors(ffk):
+    w = torch.ones((10, 8), device="cuda", dtype=torch.float16)
+    ids = torch.tensor([1, 10, -1, 3], dtype=torch.int64, device="cuda")
+    out = ffk.embedding_forward(ids, w)  # ids outside the table are skipped, as for the other types
+    assert out[0].sum() == 8 and out[1].sum() == 0 and out[2].sum() == 0
+    dw = torch.zeros((10, 8), device="cuda", dtype=torch.float16)
+    ffk.embedding_backward_typed(ids, torch.ones((4, 8), device="cuda", dtype=torch.float16), dw)
+    assert dw.sum() == 16
+    # FLOAT goes to the fp32 entry point; bf16 has no typed form (its gradients accumulate in fp32)
+    dwf = torch.zeros((10, 8), device="cuda")
+    ffk.embedding_backward_typed(ids, torch.ones((4, 8), device="cuda"), dwf)
+    assert dwf.sum() == 16
+    with pytest.raises(ffk.FFKError, match="not supported"):
+        ffk.embedding_backward_typed(ids, torch.ones((4, 8), device="cuda", dtype=torch.bfloat16),
+                                     torch.zeros((10, 8), device="cuda", dtype=torch.bfloat16))
+    with pytest.raises(ffk.FFKError, match="not supported"):  # table and output types must agree
+        ffk.embedding_forward(ids, w, out_dtype=torch.float32)

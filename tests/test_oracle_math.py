@@ -261,6 +261,48 @@ def test_embedding_against_torch(oracle):
         oracle.embedding_forward(np.array([V]), w)
 
 
+@pytest.mark.parametrize("dt", [np.float16, np.float64])
+def test_typed_embedding_against_torch_and_the_fp32_restatement(oracle, dt):
+    """The HALF / DOUBLE restatements (numpy) against torch's embedding_bag in float64 and against
+    the C fp32 restatement on data whose sums are exact in every type (eighths of small integers),
+    where the three must agree to the bit; then what only arithmetic in the table's own type gives."""
+    g = rng(81)
+    V, D, B, bag = 40, 6, 13, 4
+    w = (g.integers(-32, 33, (V, D)) / 8.0).astype(dt)
+    bags = g.integers(0, V, (B, bag))
+    dy = (g.integers(-16, 17, (B, D)) / 4.0).astype(dt)
+    for aggr, mode in ((0, "sum"), (1, "mean")):  # bag = 4: the average is exact too
+        want = F.embedding_bag(torch.from_numpy(bags), t64(w.astype(np.float64)), mode=mode).numpy()
+        got = oracle.embedding_forward_typed(bags, w, aggr=aggr)
+        assert got.dtype == dt and np.array_equal(got.astype(np.float64), want)
+        assert np.array_equal(got.astype(np.float32), oracle.embedding_forward(bags, w.astype(np.float32), aggr=aggr))
+        wt = t64(w.astype(np.float64)).requires_grad_()
+        F.embedding_bag(torch.from_numpy(bags), wt, mode=mode).backward(t64(dy.astype(np.float64)))
+        dw = oracle.embedding_backward_typed(bags, dy, V, aggr=aggr)
+        assert dw.dtype == dt and np.array_equal(dw.astype(np.float64), wt.grad.numpy())
+        assert np.array_equal(dw.astype(np.float32), oracle.embedding_backward(bags, dy.astype(np.float32), V, aggr=aggr))
+    idx = g.integers(0, V, (B,))
+    assert np.array_equal(oracle.embedding_forward_typed(idx, w), w[idx])
+    # accumulation into what weight_grad held
+    init = np.full((V, D), 0.5, dt)
+    assert np.array_equal(oracle.embedding_backward_typed(idx, dy, V, dw_init=init),
+                          oracle.embedding_backward_typed(idx, dy, V) + dt(0.5))
+    with pytest.raises(ValueError):
+        oracle.embedding_forward_typed(np.array([V]), w)
+    if dt == np.float16:
+        # a bag summed in half: 2048 + 1 is a tie that rounds back to 2048 each time; in fp32 it is 2050
+        w2 = np.array([[2048.0], [1.0]], np.float16)
+        assert oracle.embedding_forward_typed(np.array([[0, 1, 1]]), w2, aggr=0)[0, 0] == 2048.0
+        assert oracle.embedding_forward(np.array([[0, 1, 1]]), w2.astype(np.float32), aggr=0)[0, 0] == 2050.0
+        # AVG's factor is half(1/3) = 0.333251953125, not a division
+        assert oracle.embedding_forward_typed(np.array([[0, 0, 0]]), np.array([[1.0]], np.float16), aggr=1)[0, 0] \
+            == np.float16(np.float16(3.0) * np.float16(np.float32(1.0) / np.float32(3.0)))
+    else:
+        # double keeps what fp32 loses
+        w2 = np.array([[2.0 ** 30], [2.0 ** -30]], np.float64)
+        assert oracle.embedding_forward_typed(np.array([[0, 1]]), w2, aggr=0)[0, 0] == 2.0 ** 30 + 2.0 ** -30
+
+
 @pytest.mark.parametrize("Dv", [8, 5, 12])
 @pytest.mark.parametrize("causal", [False, True])
 def test_attention_against_torch_sdpa(oracle, causal, Dv):
