@@ -48,8 +48,8 @@ __device__ __forceinline__ void lds_dma16(i32x4 rsrc, unsigned lane_byte_off, un
                              // relative-move or GDS/message instruction and holds
                              // nothing live in M0 across these blocks.  Guarded by
                              // the bit-equality tests against the kernels without
-                             // direct loads (tests/test_gpu_linear.py: GEMM variants;
-                             // tests/test_gpu_attention.py: the two dK/dV kernels).
+                             // direct loads (tests/test_gpu_linear.py: GEMM variants)
+                             // and by the attention kernels' tests against the oracle.
 }
 // The same for 4 bytes per lane: lane l's dword lands at lds_base + 4 l.
 __device__ __forceinline__ void lds_dma4(i32x4 rsrc, unsigned lane_byte_off, unsigned uniform_byte_off,
