@@ -1101,6 +1101,186 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// fp32 MFMA kernel for operands that can be read 16 bytes at a time: 128 x BN
+// block tile (BN = 128 or 64), 2 x 2 waves of 64 x BN/2, reduction tiles of 32.
+// The next tile travels global -> registers while this one is multiplied and
+// goes to the other LDS buffer afterwards: one barrier per tile.  The fp32
+// MFMA (32x32x2, 64 cycles) is so slow next to its two one-register operands
+// that LDS and issue bandwidth are never short; what the kernel has to do is
+// keep loads in flight and the matrix pipe fed, which two workgroups per CU and
+// fragments read one step ahead take care of.
+//   An operand whose reduction index is contiguous in memory (A[M,K], B[N,K])
+// lies in LDS as [k / 2][row][k % 2], row stride 2 * rows + 4: a lane's four
+// consecutive k go out as two 8-byte writes, and the MFMA read -- lanes 0-31
+// one k, lanes 32-63 the next -- touches 64 consecutive floats.  An operand
+// whose rows are contiguous (A[K,M], B[K,N]) lies as [k][row] with the two
+// 32-float halves of every odd k swapped, which does the same for the read
+// without padding.  Every element's products are added in ascending k, two per
+// MFMA, as in gemm_f32_kernel: the two kernels give the same bits.
+// Rows and columns past the edge are read from the last valid ones and never
+// stored; k past the end is zeroed when the tile is written to LDS.
+// ---------------------------------------------------------------------------
+template <bool TA, bool TB, int BN>
+__global__ __launch_bounds__(256, 2) void gemm_f32_tiled_kernel(
+    float const *__restrict__ A, float const *__restrict__ B, float *C, int M, int N, int K, int64_t lda,
+    int64_t ldb, int64_t ldc, float const *__restrict__ bias, int act, int accumulate) {
+  constexpr int BM = 128, BKT = 32;
+  constexpr int TNW = BN / 64;              // 32-column blocks per wave
+  constexpr bool A_KC = !TA, B_KC = TB;     // reduction index contiguous in memory
+  constexpr int A_CH = BM * BKT / 4 / 256, B_CH = BN * BKT / 4 / 256;  // 16-byte chunks per thread and tile
+  constexpr int A_SP = 2 * BM + 4, B_SP = 2 * BN + 4;                  // pair-layout row strides
+  constexpr int A_FLOATS = A_KC ? (BKT / 2) * A_SP : BKT * BM;
+  constexpr int B_FLOATS = B_KC ? (BKT / 2) * B_SP : BKT * BN;
+  __shared__ __attribute__((aligned(16))) float As[2][A_FLOATS];
+  __shared__ __attribute__((aligned(16))) float Bs[2][B_FLOATS];
+  int const t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  int const h = lane >> 5, l32 = lane & 31;
+  int const wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * (BN / 2);
+  int tm, tn;
+  tile_coords(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+  int const m0 = tm * BM, n0 = tn * BN;
+
+  // chunk i of this thread: (row, k quad) of a k-contiguous operand, (k row, row quad) otherwise
+  f32x4 ra[A_CH], rb[B_CH];
+  auto gload = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < A_CH; i++) {
+      int const c = t + i * 256;
+      if (A_KC) {
+        int const row = min(m0 + c / 8, M - 1), k = min(k0 + 4 * (c % 8), K - 4);
+        ra[i] = *reinterpret_cast<f32x4 const *>(A + (int64_t)row * lda + k);
+      } else {
+        int const k = min(k0 + c / (BM / 4), K - 1), row = min(m0 + 4 * (c % (BM / 4)), M - 4);
+        ra[i] = *reinterpret_cast<f32x4 const *>(A + (int64_t)k * lda + row);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < B_CH; i++) {
+      int const c = t + i * 256;
+      if (B_KC) {
+        int const row = min(n0 + c / 8, N - 1), k = min(k0 + 4 * (c % 8), K - 4);
+        rb[i] = *reinterpret_cast<f32x4 const *>(B + (int64_t)row * ldb + k);
+      } else {
+        int const k = min(k0 + c / (BN / 4), K - 1), row = min(n0 + 4 * (c % (BN / 4)), N - 4);
+        rb[i] = *reinterpret_cast<f32x4 const *>(B + (int64_t)k * ldb + row);
+      }
+    }
+  };
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  auto lstore = [&](int buf, int k0) {
+    f32x4 const zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < A_CH; i++) {
+      int const c = t + i * 256;
+      if (A_KC) {
+        int const row = c / 8, kq = c % 8;
+        f32x4 const v = k0 + 4 * kq < K ? ra[i] : zero;
+        *reinterpret_cast<f32x2 *>(&As[buf][(2 * kq) * A_SP + 2 * row]) = f32x2{v[0], v[1]};
+        *reinterpret_cast<f32x2 *>(&As[buf][(2 * kq + 1) * A_SP + 2 * row]) = f32x2{v[2], v[3]};
+      } else {
+        int const k = c / (BM / 4), rq = c % (BM / 4);
+        f32x4 const v = k0 + k < K ? ra[i] : zero;
+        *reinterpret_cast<f32x4 *>(&As[buf][k * BM + ((4 * rq) ^ ((k & 1) * 32))]) = v;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < B_CH; i++) {
+      int const c = t + i * 256;
+      if (B_KC) {
+        int const row = c / 8, kq = c % 8;
+        f32x4 const v = k0 + 4 * kq < K ? rb[i] : zero;
+        *reinterpret_cast<f32x2 *>(&Bs[buf][(2 * kq) * B_SP + 2 * row]) = f32x2{v[0], v[1]};
+        *reinterpret_cast<f32x2 *>(&Bs[buf][(2 * kq + 1) * B_SP + 2 * row]) = f32x2{v[2], v[3]};
+      } else {
+        int const k = c / (BN / 4), rq = c % (BN / 4);
+        f32x4 const v = k0 + k < K ? rb[i] : zero;
+        *reinterpret_cast<f32x4 *>(&Bs[buf][k * BN + ((4 * rq) ^ ((k & 1) * 32))]) = v;
+      }
+    }
+  };
+  // operand value of this lane for MFMA step kk (k = 2 kk + h) and its row
+  auto frag_a = [&](int buf, int kk, int row) -> float {
+    return A_KC ? As[buf][kk * A_SP + 2 * row + h] : As[buf][(2 * kk + h) * BM + (row ^ (h * 32))];
+  };
+  auto frag_b = [&](int buf, int kk, int row) -> float {
+    return B_KC ? Bs[buf][kk * B_SP + 2 * row + h] : Bs[buf][(2 * kk + h) * BN + (row ^ (h * 32))];
+  };
+
+  f32x16 acc[2][TNW];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < TNW; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  int const KT = (K + BKT - 1) / BKT;
+  gload(0);
+  lstore(0, 0);
+  __syncthreads();
+  int cur = 0;
+  for (int kt = 0; kt < KT; kt++) {
+    bool const more = kt + 1 < KT;
+    if (more) gload((kt + 1) * BKT);
+    float af[2][2], bfv[2][TNW];
+#pragma unroll
+    for (int i = 0; i < 2; i++) af[0][i] = frag_a(cur, 0, wm0 + i * 32 + l32);
+#pragma unroll
+    for (int j = 0; j < TNW; j++) bfv[0][j] = frag_b(cur, 0, wn0 + j * 32 + l32);
+#pragma unroll
+    for (int kk = 0; kk < BKT / 2; kk++) {
+      int const c = kk & 1, nx = c ^ 1;
+      // the next step's fragments are asked for before this step's MFMAs are issued (a wave
+      // sits at each MFMA until the pipe takes it; reads issued behind them would start their
+      // round trip only then).  The fences keep the compiler from moving them back.
+      if (kk + 1 < BKT / 2) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) af[nx][i] = frag_a(cur, kk + 1, wm0 + i * 32 + l32);
+#pragma unroll
+        for (int j = 0; j < TNW; j++) bfv[nx][j] = frag_b(cur, kk + 1, wn0 + j * 32 + l32);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < TNW; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c][i], bfv[c][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (more) lstore(cur ^ 1, (kt + 1) * BKT);
+    __syncthreads();
+    cur ^= 1;
+  }
+
+  // accumulator element r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of its block
+#pragma unroll
+  for (int j = 0; j < TNW; j++) {
+    int const n = n0 + wn0 + j * 32 + l32;
+    if (n >= N) continue;
+    float const bv = bias != nullptr ? bias[n] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      int const mb = m0 + wm0 + i * 32 + 4 * h;
+      float old[16];
+      if (accumulate) {  // what C holds, all loads in flight together
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          int const m = min(mb + 8 * (r >> 2) + (r & 3), M - 1);
+          old[r] = C[(int64_t)m * ldc + n];
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        int const m = mb + 8 * (r >> 2) + (r & 3);
+        float v = apply_activation(acc[i][j][r] + bv, act);
+        if (accumulate) v += old[r];
+        if (m < M) C[(int64_t)m * ldc + n] = v;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Plain kernel for bf16 shapes the tiled kernel cannot take.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void gemm_bf16_plain_kernel(
@@ -1536,6 +1716,32 @@ int gemm_dispatch(hipStream_t st, int dtype, bool ta, bool tb, int64_t M,
     float const *b = static_cast<float const *>(B);
     float *c = static_cast<float *>(C);
     float const *bias = static_cast<float const *>(ep.bias);
+    // 16-byte reads: aligned rows, and whole quads along whichever index is contiguous
+    bool const tiled = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0 && K >= 4 &&
+                       (ta ? M % 4 == 0 && M >= 4 : K % 4 == 0) && (tb ? K % 4 == 0 : N % 4 == 0 && N >= 4) &&
+                       M * N >= 128 * 128;
+    if (tiled) {
+      // 128 x 128 tiles when they give every CU two workgroups, 128 x 64 otherwise
+      bool const wide = ceil_div(M, 128) * ceil_div(N, 128) >= 2 * kNumCU;
+      int const tblocks = (int)(ceil_div(M, 128) * ceil_div(N, wide ? 128 : 64));
+      if (describe_only("gemm_f32_tiled_kernel<%s,%s,%d>", tf(ta), tf(tb), wide ? 128 : 64)) return FFK_OK;
+#define FFK_LAUNCH_F32T(TA_, TB_)                                              \
+  do {                                                                         \
+    if (wide)                                                                  \
+      gemm_f32_tiled_kernel<TA_, TB_, 128><<<tblocks, 256, 0, st>>>(           \
+          a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, bias, ep.activation, ep.accumulate); \
+    else                                                                       \
+      gemm_f32_tiled_kernel<TA_, TB_, 64><<<tblocks, 256, 0, st>>>(            \
+          a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, bias, ep.activation, ep.accumulate); \
+  } while (0)
+      if (!ta && !tb) FFK_LAUNCH_F32T(false, false);
+      else if (!ta && tb) FFK_LAUNCH_F32T(false, true);
+      else if (ta && !tb) FFK_LAUNCH_F32T(true, false);
+      else FFK_LAUNCH_F32T(true, true);
+#undef FFK_LAUNCH_F32T
+      FFK_CHECK_LAUNCH();
+      return FFK_OK;
+    }
     int const blocks = (int)(ceil_div(M, 64) * ceil_div(N, 64));
 #define FFK_LAUNCH_F32(TA_, TB_)                                               \
   gemm_f32_kernel<TA_, TB_><<<blocks, 256, 0, st>>>(                           \

@@ -203,6 +203,83 @@ def test_gemm_bf16(ffk, oracle, trans_a, trans_b, mnk):
     assert_close(to_np(Cd), want + C0, 2.0 ** -7, "C accumulate")
 
 
+F32_GEMM_SHAPES = [  # M, N, K: whole tiles, ragged edges in every direction, one k quad, both tile widths
+    (128, 128, 32), (300, 260, 100), (128, 132, 4), (1000, 192, 36), (256, 64, 68), (1152, 2048, 64), (4096, 8192, 40),
+]
+
+
+@pytest.mark.parametrize("trans_a", [False, True])
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("mnk", F32_GEMM_SHAPES)
+def test_gemm_fp32_tiled(ffk, oracle, trans_a, trans_b, mnk):
+    """The fp32 kernel with 128-row tiles (operands read 16 bytes at a time) against the fp64
+    product, and against the bounds-checked 64x64 kernel, which adds every element's products in
+    the same order: equal bits.  The general kernel is reached through a view whose rows start
+    4 bytes off 16-byte alignment."""
+    M, N, K = mnk
+    if M * N > 2 ** 24 and (trans_a or not trans_b):
+        pytest.skip("the largest shape once")
+    say("gemm fp32 tiled", mnk, "ta", trans_a, "tb", trans_b)
+    name = ffk.gemm_kernel_name(ffk.FLOAT, trans_a, trans_b, M, N, K)
+    assert name.startswith("gemm_f32_tiled_kernel"), name
+    g = rng(3 * M + 5 * N + K)
+    A = g.standard_normal((K, M) if trans_a else (M, K)).astype(np.float32)
+    B = g.standard_normal((N, K) if trans_b else (K, N)).astype(np.float32)
+    Ad, Bd = to_dev(A, torch), to_dev(B, torch)
+    C = torch.full((M, N), 7.0, device="cuda")
+    ffk.gemm(Ad, Bd, C, trans_a, trans_b)
+    if M * N <= 2 ** 22:
+        want = oracle.gemm_f64(A, B, trans_a, trans_b)
+        assert_close(to_np(C), want, FP32_RTOL, "C")
+    else:
+        rows = np.sort(g.choice(M, 24, replace=False))
+        A_rows = np.ascontiguousarray(A[:, rows] if trans_a else A[rows])
+        assert_close(to_np(C[torch.from_numpy(rows).cuda()]), oracle.gemm_f64(A_rows, B, trans_a, trans_b), FP32_RTOL, "C rows")
+    # the same product by the general kernel: operands shifted one float off alignment
+    def shifted(t):
+        flat = torch.empty((t.numel() + 1,), device="cuda")
+        v = flat[1:].view(t.shape)
+        v.copy_(t)
+        return v
+    A1, B1 = shifted(Ad), shifted(Bd)
+    C1 = torch.full((M, N), 7.0, device="cuda")
+    ffk.check(ffk.lib().ffk_gemm(ffk.current_stream(), ffk.FLOAT, int(trans_a), int(trans_b), M, N, K,
+                                 A1.data_ptr(), B1.data_ptr(), C1.data_ptr(), 0))
+    assert torch.equal(C, C1)
+    # accumulate: C += product, old contents read once
+    C0 = g.standard_normal((M, N)).astype(np.float32)
+    Cd, Cd1 = to_dev(C0, torch), to_dev(C0, torch)
+    ffk.gemm(Ad, Bd, Cd, trans_a, trans_b, accumulate=True)
+    ffk.check(ffk.lib().ffk_gemm(ffk.current_stream(), ffk.FLOAT, int(trans_a), int(trans_b), M, N, K,
+                                 A1.data_ptr(), B1.data_ptr(), Cd1.data_ptr(), 1))
+    assert torch.equal(Cd, Cd1)
+    assert torch.equal(Cd, C + to_dev(C0, torch))
+
+
+@pytest.mark.parametrize("act", [-1, 0, 1, 2, 3])
+def test_linear_fp32_tiled_bias_and_activation(ffk, oracle, act):
+    """A fp32 Linear large enough for the tiled kernel: bias and every activation on its store."""
+    batch, in_dim, out_dim = 520, 136, 384
+    say("linear fp32 tiled", (batch, in_dim, out_dim), "act", act)
+    assert ffk.gemm_kernel_name(ffk.FLOAT, False, True, batch, out_dim, in_dim, True, act).startswith("gemm_f32_tiled_kernel")
+    x, w, b, dy = _cfg1_inputs(seed=31, batch=batch, in_dim=in_dim, out_dim=out_dim)
+    w = w * 10
+    if act == 3:  # the reference's Linear has no GELU; this one is Linear -> ElementUnary GELU
+        y_ref = oracle.element_unary_forward(ffk.OP["GELU"], oracle.linear_forward(x, w, b, activation=-1))
+    else:
+        y_ref = oracle.linear_forward(x, w, b, activation=act)
+    xd, wd, bd, dyd = (to_dev(a, torch) for a in (x, w, b, dy))
+    y = ffk.linear_forward(xd, wd, bd, activation=act)
+    assert_close(to_np(y), y_ref, FP32_RTOL, "y")
+    if act != 3:  # GELU has no backward on the Linear
+        dx_ref, dw_ref, db_ref = oracle.linear_backward(y_ref, dy, x, w, activation=act)
+        dx, dw, db = torch.zeros_like(xd), torch.zeros_like(wd), torch.zeros_like(bd)
+        ffk.linear_backward(to_dev(y_ref, torch), dyd, xd, wd, dx, dw, db, activation=act)
+        assert_close(to_np(dx), dx_ref, FP32_RTOL, "dx")
+        assert_close(to_np(dw), dw_ref, FP32_RTOL, "dw")
+        assert_close(to_np(db), db_ref, FP32_RTOL, "db")
+
+
 @pytest.mark.parametrize("mnk", [(7, 5, 3), (33, 9, 12), (16, 24, 20)])
 def test_gemm_bf16_unaligned_shapes_take_the_plain_kernel(ffk, oracle, mnk):
     M, N, K = mnk
