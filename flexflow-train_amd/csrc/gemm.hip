@@ -1112,7 +1112,12 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 //   An operand whose reduction index is contiguous in memory (A[M,K], B[N,K])
 // lies in LDS as [k / 2][row][k % 2], row stride 2 * rows + 4: a lane's four
 // consecutive k go out as two 8-byte writes, and the MFMA read -- lanes 0-31
-// one k, lanes 32-63 the next -- touches 64 consecutive floats.  An operand
+// one k, lanes 32-63 the next -- touches 64 consecutive floats.  The compiler
+// pairs a lane's reads for two 32-row blocks into one two-dword read, which is
+// served 32 lanes at a time: the pairs of odd blocks are stored swapped, so
+// that those 32 lanes take even banks for one block and odd banks for the
+// other (unswapped they met in the same banks: 2.6 conflict cycles per cycle
+// of LDS work, the matrix pipe 80% busy).  An operand
 // whose rows are contiguous (A[K,M], B[K,N]) lies as [k][row] with the two
 // 32-float halves of every odd k swapped, which does the same for the read
 // without padding.  Every element's products are added in ascending k, two per
@@ -1140,70 +1145,88 @@ __global__ __launch_bounds__(256, 2) void gemm_f32_tiled_kernel(
   tile_coords(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
   int const m0 = tm * BM, n0 = tn * BN;
 
-  // chunk i of this thread: (row, k quad) of a k-contiguous operand, (k row, row quad) otherwise
-  f32x4 ra[A_CH], rb[B_CH];
-  auto gload = [&](int k0) {
+  // Chunk i of this thread: (row, k quad) of a k-contiguous operand, (k row, row quad) otherwise.
+  // Its address for k-tile 0 is kept and moved on by a constant per tile; only a tile that
+  // reaches past K (the last one of a ragged reduction) computes clamped addresses afresh.
+  constexpr int NCH = A_CH + B_CH;
+  f32x4 rgs[2][NCH];  // k-tile kt travels in set kt % 2, two tiles ahead of its use
+  float const *pg[NCH];
 #pragma unroll
-    for (int i = 0; i < A_CH; i++) {
-      int const c = t + i * 256;
-      if (A_KC) {
-        int const row = min(m0 + c / 8, M - 1), k = min(k0 + 4 * (c % 8), K - 4);
-        ra[i] = *reinterpret_cast<f32x4 const *>(A + (int64_t)row * lda + k);
+  for (int i = 0; i < A_CH; i++) {
+    int const c = t + i * 256;
+    pg[i] = A_KC ? A + (int64_t)min(m0 + c / 8, M - 1) * lda + 4 * (c % 8)
+                 : A + (int64_t)(c / (BM / 4)) * lda + min(m0 + 4 * (c % (BM / 4)), M - 4);
+  }
+#pragma unroll
+  for (int i = 0; i < B_CH; i++) {
+    int const c = t + i * 256;
+    pg[A_CH + i] = B_KC ? B + (int64_t)min(n0 + c / 8, N - 1) * ldb + 4 * (c % 8)
+                        : B + (int64_t)(c / (BN / 4)) * ldb + min(n0 + 4 * (c % (BN / 4)), N - 4);
+  }
+  int64_t const step_a = A_KC ? BKT : (int64_t)BKT * lda, step_b = B_KC ? BKT : (int64_t)BKT * ldb;
+  // load of chunk i of k-tile kt; pg[i] points at k-tile kt on entry and at kt + 1 on return
+  auto gload_chunk = [&](int kt, int i, f32x4 (&rg)[NCH]) __attribute__((always_inline)) {
+    int const k0 = kt * BKT;
+    bool const is_a = i < A_CH;
+    if (k0 + BKT <= K) {
+      rg[i] = *reinterpret_cast<f32x4 const *>(pg[i]);
+    } else {
+      int const c = t + (is_a ? i : i - A_CH) * 256;
+      // how far this chunk's k lies past the last one it may read
+      if (is_a ? A_KC : B_KC) {
+        int const over = max(k0 + 4 * (c % 8) - (K - 4), 0);
+        rg[i] = *reinterpret_cast<f32x4 const *>(pg[i] - over);
       } else {
-        int const k = min(k0 + c / (BM / 4), K - 1), row = min(m0 + 4 * (c % (BM / 4)), M - 4);
-        ra[i] = *reinterpret_cast<f32x4 const *>(A + (int64_t)k * lda + row);
+        int const over = max(k0 + c / ((is_a ? BM : BN) / 4) - (K - 1), 0);
+        rg[i] = *reinterpret_cast<f32x4 const *>(pg[i] - (int64_t)over * (is_a ? lda : ldb));
       }
     }
+    pg[i] += is_a ? step_a : step_b;
+  };
+  auto gload = [&](int kt, f32x4 (&rg)[NCH]) {
 #pragma unroll
-    for (int i = 0; i < B_CH; i++) {
-      int const c = t + i * 256;
-      if (B_KC) {
-        int const row = min(n0 + c / 8, N - 1), k = min(k0 + 4 * (c % 8), K - 4);
-        rb[i] = *reinterpret_cast<f32x4 const *>(B + (int64_t)row * ldb + k);
-      } else {
-        int const k = min(k0 + c / (BN / 4), K - 1), row = min(n0 + 4 * (c % (BN / 4)), N - 4);
-        rb[i] = *reinterpret_cast<f32x4 const *>(B + (int64_t)k * ldb + row);
-      }
-    }
+    for (int i = 0; i < NCH; i++) gload_chunk(kt, i, rg);
   };
   typedef float f32x2 __attribute__((ext_vector_type(2)));
-  auto lstore = [&](int buf, int k0) {
+  // chunk i of k-tile kt from its registers into buffer buf, k past the end zeroed
+  auto lstore_chunk = [&](int buf, int kt, int i, f32x4 const (&rg)[NCH]) __attribute__((always_inline)) {
     f32x4 const zero = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int i = 0; i < A_CH; i++) {
-      int const c = t + i * 256;
-      if (A_KC) {
-        int const row = c / 8, kq = c % 8;
-        f32x4 const v = k0 + 4 * kq < K ? ra[i] : zero;
-        *reinterpret_cast<f32x2 *>(&As[buf][(2 * kq) * A_SP + 2 * row]) = f32x2{v[0], v[1]};
-        *reinterpret_cast<f32x2 *>(&As[buf][(2 * kq + 1) * A_SP + 2 * row]) = f32x2{v[2], v[3]};
-      } else {
-        int const k = c / (BM / 4), rq = c % (BM / 4);
-        f32x4 const v = k0 + k < K ? ra[i] : zero;
-        *reinterpret_cast<f32x4 *>(&As[buf][k * BM + ((4 * rq) ^ ((k & 1) * 32))]) = v;
+    int const k0 = kt * BKT;
+    bool const is_a = i < A_CH;
+    int const c = t + (is_a ? i : i - A_CH) * 256;
+    float *dst = is_a ? As[buf] : Bs[buf];
+    int const SP = is_a ? A_SP : B_SP, R = is_a ? BM : BN;
+    // (vector instructions between the MFMAs are not free: with two waves on a SIMD the masks
+    // and selects of this function, applied to every tile, cost 5-10% of the matrix pipe's time.
+    // The mask is for the one tile that reaches past K; which blocks are swapped is known per chunk.)
+    bool const whole = k0 + BKT <= K;  // uniform
+    if (is_a ? A_KC : B_KC) {
+      int const row = c / 8, kq = c % 8;
+      f32x4 v = rg[i];
+      if (!whole) {
+        asm volatile("" ::: "memory");  // a branch, not four selects on every tile
+        v = k0 + 4 * kq < K ? v : zero;
       }
-    }
-#pragma unroll
-    for (int i = 0; i < B_CH; i++) {
-      int const c = t + i * 256;
-      if (B_KC) {
-        int const row = c / 8, kq = c % 8;
-        f32x4 const v = k0 + 4 * kq < K ? rb[i] : zero;
-        *reinterpret_cast<f32x2 *>(&Bs[buf][(2 * kq) * B_SP + 2 * row]) = f32x2{v[0], v[1]};
-        *reinterpret_cast<f32x2 *>(&Bs[buf][(2 * kq + 1) * B_SP + 2 * row]) = f32x2{v[2], v[3]};
-      } else {
-        int const k = c / (BN / 4), rq = c % (BN / 4);
-        f32x4 const v = k0 + k < K ? rb[i] : zero;
-        *reinterpret_cast<f32x4 *>(&Bs[buf][k * BN + ((4 * rq) ^ ((k & 1) * 32))]) = v;
+      // odd 32-row blocks hold their k pairs swapped; row / 32 = chunk number (t / 8 < 32)
+      bool const odd = (((is_a ? i : i - A_CH) & 1) != 0);
+      *reinterpret_cast<f32x2 *>(&dst[(2 * kq) * SP + 2 * row]) = odd ? f32x2{v[1], v[0]} : f32x2{v[0], v[1]};
+      *reinterpret_cast<f32x2 *>(&dst[(2 * kq + 1) * SP + 2 * row]) = odd ? f32x2{v[3], v[2]} : f32x2{v[2], v[3]};
+    } else {
+      int const k = c / (R / 4), rq = c % (R / 4);
+      f32x4 v = rg[i];
+      if (!whole) {
+        asm volatile("" ::: "memory");
+        v = k0 + k < K ? v : zero;
       }
+      *reinterpret_cast<f32x4 *>(&dst[k * R + ((4 * rq) ^ ((k & 1) * 32))]) = v;
     }
   };
   // operand value of this lane for MFMA step kk (k = 2 kk + h) and its row
   auto frag_a = [&](int buf, int kk, int row) -> float {
-    return A_KC ? As[buf][kk * A_SP + 2 * row + h] : As[buf][(2 * kk + h) * BM + (row ^ (h * 32))];
+    return A_KC ? As[buf][kk * A_SP + 2 * row + (h ^ ((row >> 5) & 1))] : As[buf][(2 * kk + h) * BM + (row ^ (h * 32))];
   };
   auto frag_b = [&](int buf, int kk, int row) -> float {
-    return B_KC ? Bs[buf][kk * B_SP + 2 * row + h] : Bs[buf][(2 * kk + h) * BN + (row ^ (h * 32))];
+    return B_KC ? Bs[buf][kk * B_SP + 2 * row + (h ^ ((row >> 5) & 1))] : Bs[buf][(2 * kk + h) * BN + (row ^ (h * 32))];
   };
 
   f32x16 acc[2][TNW];
@@ -1215,41 +1238,72 @@ __global__ __launch_bounds__(256, 2) void gemm_f32_tiled_kernel(
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
   int const KT = (K + BKT - 1) / BKT;
-  gload(0);
-  lstore(0, 0);
+  gload(0, rgs[0]);
+  if (KT > 1) gload(1, rgs[1]);
+#pragma unroll
+  for (int i = 0; i < NCH; i++) lstore_chunk(0, 0, i, rgs[0]);
   __syncthreads();
-  int cur = 0;
-  for (int kt = 0; kt < KT; kt++) {
-    bool const more = kt + 1 < KT;
-    if (more) gload((kt + 1) * BKT);
+  // One k-tile, kt, from buffer kt % 2.  AHEAD2: k-tile kt + 2 exists; its loads go out one per
+  // step in the first NCH steps (a burst of them holds the wave, and with it its MFMAs, for as
+  // long as the memory pipeline takes to accept them), into the register set that tile kt
+  // travelled in.  AHEAD1: k-tile kt + 1
+  // exists; it was asked for a tile ago and is written to the other buffer (which nobody reads
+  // during this tile) one chunk per step in the last NCH steps, under the MFMAs.  A wave sits
+  // at each MFMA until the pipe takes it, so whatever is placed between two of them costs
+  // nothing as long as it is short; the fences keep it there.
+  constexpr int KS = BKT / 2;
+  static_assert(NCH <= KS, "one chunk per step");
+  auto tile = [&](int kt, auto set_tag, auto ahead1_tag, auto ahead2_tag) {
+    constexpr int SET = decltype(set_tag)::value;  // = kt % 2
+    constexpr bool AHEAD1 = decltype(ahead1_tag)::value, AHEAD2 = decltype(ahead2_tag)::value;
     float af[2][2], bfv[2][TNW];
 #pragma unroll
-    for (int i = 0; i < 2; i++) af[0][i] = frag_a(cur, 0, wm0 + i * 32 + l32);
+    for (int i = 0; i < 2; i++) af[0][i] = frag_a(SET, 0, wm0 + i * 32 + l32);
 #pragma unroll
-    for (int j = 0; j < TNW; j++) bfv[0][j] = frag_b(cur, 0, wn0 + j * 32 + l32);
+    for (int j = 0; j < TNW; j++) bfv[0][j] = frag_b(SET, 0, wn0 + j * 32 + l32);
 #pragma unroll
-    for (int kk = 0; kk < BKT / 2; kk++) {
+    for (int kk = 0; kk < KS; kk++) {
       int const c = kk & 1, nx = c ^ 1;
-      // the next step's fragments are asked for before this step's MFMAs are issued (a wave
-      // sits at each MFMA until the pipe takes it; reads issued behind them would start their
-      // round trip only then).  The fences keep the compiler from moving them back.
-      if (kk + 1 < BKT / 2) {
+      // the next step's fragments are asked for before this step's MFMAs are issued: reads
+      // issued behind them would start their round trip only when the last one has gone
+      if (kk + 1 < KS) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) af[nx][i] = frag_a(cur, kk + 1, wm0 + i * 32 + l32);
+        for (int i = 0; i < 2; i++) af[nx][i] = frag_a(SET, kk + 1, wm0 + i * 32 + l32);
 #pragma unroll
-        for (int j = 0; j < TNW; j++) bfv[nx][j] = frag_b(cur, kk + 1, wn0 + j * 32 + l32);
+        for (int j = 0; j < TNW; j++) bfv[nx][j] = frag_b(SET, kk + 1, wn0 + j * 32 + l32);
       }
+      __builtin_amdgcn_sched_barrier(0);
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c][0], bfv[c][0], acc[0][0], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (AHEAD2 && kk < NCH) gload_chunk(kt + 2, kk, rgs[SET]);
+      if (AHEAD1 && kk >= KS - NCH) lstore_chunk(SET ^ 1, kt + 1, kk - (KS - NCH), rgs[SET ^ 1]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 2; i++)
 #pragma unroll
         for (int j = 0; j < TNW; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c][i], bfv[c][j], acc[i][j], 0, 0, 0);
+          if (i + j > 0) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c][i], bfv[c][j], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (more) lstore(cur ^ 1, (kt + 1) * BKT);
     __syncthreads();
-    cur ^= 1;
+  };
+  using T0 = std::integral_constant<int, 0>;
+  using T1 = std::integral_constant<int, 1>;
+  int kt = 0;
+  for (; kt + 3 < KT; kt += 2) {  // both tiles of the pair have two successors
+    tile(kt, T0{}, std::true_type{}, std::true_type{});
+    tile(kt + 1, T1{}, std::true_type{}, std::true_type{});
+  }
+  // the last one to three tiles (kt is even)
+  if (kt + 2 < KT) {
+    tile(kt, T0{}, std::true_type{}, std::true_type{});
+    tile(kt + 1, T1{}, std::true_type{}, std::false_type{});
+    tile(kt + 2, T0{}, std::false_type{}, std::false_type{});
+  } else if (kt + 1 < KT) {
+    tile(kt, T0{}, std::true_type{}, std::false_type{});
+    tile(kt + 1, T1{}, std::false_type{}, std::false_type{});
+  } else {
+    tile(kt, T0{}, std::false_type{}, std::false_type{});
   }
 
   // accumulator element r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of its block

@@ -100,6 +100,26 @@ def bench_gemm():
         report("  vendor library (torch.matmul)", t, flops=2.0 * M * N * K)
 
 
+def bench_gemm_fp32():
+    # the reference's own data type: Linear shapes of the config 2 layer in fp32 (v_mfma_f32_32x32x2f32,
+    # 157.3 TFLOP/s dense peak), and a large square
+    for (M, N, K, ta, tb) in [(4096, 4096, 1024, 0, 1), (4096, 1024, 4096, 0, 1), (4096, 1024, 4096, 0, 0),
+                              (1024, 4096, 4096, 1, 0), (8192, 8192, 8192, 0, 1)]:
+        A = torch.randn((K, M) if ta else (M, K), device="cuda")
+        B = torch.randn((N, K) if tb else (K, N), device="cuda")
+        C = torch.empty((M, N), device="cuda")
+        iters = 5 if M * N * K > 2 ** 36 else 20
+        t = timeit(lambda: ffk.gemm(A, B, C, bool(ta), bool(tb)), iters=iters)
+        print("%-46s %9.1f us  %8.1f TFLOP/s (%5.1f%% of 157.3 TFLOP/s)  %s" % (
+            "gemm fp32 M%d N%d K%d %s%s" % (M, N, K, "T" if ta else "N", "T" if tb else "N"), t * 1e6,
+            2.0 * M * N * K / t / 1e12, 2.0 * M * N * K / t / 157.3e12 * 100,
+            ffk.gemm_kernel_name(ffk.FLOAT, bool(ta), bool(tb), M, N, K)), flush=True)
+        At, Bt = (A.t() if ta else A), (B.t() if tb else B)
+        t = timeit(lambda: torch.matmul(At, Bt, out=C), iters=iters)
+        print("%-46s %9.1f us  %8.1f TFLOP/s (%5.1f%% of 157.3 TFLOP/s)" % (
+            "  vendor library (torch.matmul)", t * 1e6, 2.0 * M * N * K / t / 1e12, 2.0 * M * N * K / t / 157.3e12 * 100), flush=True)
+
+
 def bench_fused_linear():
     # Config 2's feed-forward block (4096 tokens, 1024 -> 4096 -> 1024): each Linear with the
     # element-wise operators around it as separate launches and on the GEMM's tile store
@@ -368,7 +388,7 @@ def bench_shape():
     report("Gather backward (row sums in LDS) [16384,1024] -> [16384,4096]", t, bytes_=idx2.numel() * (4 + 4 + 8))
 
 
-GROUPS = dict(gemm=bench_gemm, fused_linear=bench_fused_linear, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention, small_linear=bench_small_linear,
+GROUPS = dict(gemm=bench_gemm, gemm_fp32=bench_gemm_fp32, fused_linear=bench_fused_linear, bandwidth=bench_bandwidth, embedding=bench_embedding, attention=bench_attention, small_linear=bench_small_linear,
               update=bench_update, shape=bench_shape)
 
 if __name__ == "__main__":
