@@ -576,9 +576,15 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
   // One k-tile.  STEADY: every condition of the generic body is known true
   // (next tile exists, a refill is due, STAGES-2 younger tiles in flight), so
   // the steady-state loop is branch-free.
-  auto tile_step = [&](int kt, auto steady_tag) {
+  // SST: the tile's stage when the caller knows it (the steady loop, unrolled by STAGES), -1
+  // otherwise.  With the stage a constant every LDS address of the tile is a loop-invariant
+  // register plus an immediate; computed from kt it costs three vector instructions per k-step,
+  // which two waves on a SIMD do not get for free.
+  auto tile_step = [&](int kt, auto steady_tag, auto stage_tag) {
     constexpr bool STEADY = decltype(steady_tag)::value;
-    int const stage = kt % STAGES;
+    constexpr int SST = decltype(stage_tag)::value;
+    auto stage_at = [&](int d) { return SST >= 0 ? (SST + d) % STAGES : (kt + d) % STAGES; };
+    int const stage = stage_at(0);
     if constexpr (WIDE2) {
       // One wave per SIMD: nothing but this wave's own instruction order hides a latency, so
       // the order is written out.  A k-step is 16 MFMAs.  Behind each of them sits one of the 8
@@ -598,13 +604,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
         int const cur = kk % NB, nxt = (kk + PF) % NB;
         bool const within = kk + PF < KS;            // the next step lies in this tile
         bool const reads = within || STEADY || kt + 1 < KT;
-        int const rstage = within ? stage : (kt + 1) % STAGES;
+        int const rstage = within ? stage : stage_at(1);
         int const rkk = within ? kk + PF : kk + PF - KS;
         bf16 const *ra = smem + rstage * STAGE_ELEMS;
         bf16 const *rb = ra + A_ELEMS;
         bool const loads = kk == 0 ? (STEADY || kt + 1 < KT) : !within ? (STEADY || kt + 2 < KT) : false;
         int const ltile = kk == 0 ? kt + 1 : kt + 2;
-        int const lstage = kk == 0 ? (kt + 1) % STAGES : stage;
+        int const lstage = kk == 0 ? stage_at(1) : stage;
         int const lfirst = kk == 0 ? LPT / 2 : 0;
         // slot p follows MFMA p.  Even slots: a fragment read, in the order in which the next
         // step's MFMAs (row block by row block) first use the fragments: A0, B0..B3, A1, A2, A3.
@@ -663,7 +669,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       if (SPREAD && kk + 1 < KS) {
         // part kk+1 of the tile that goes into the stage freed one tile ago
         if (STEADY || kt + STAGES - 1 < KT) {
-          issue_some(kt + STAGES - 1, (kt + STAGES - 1) % STAGES, (kk + 1) * PART, PART);
+          issue_some(kt + STAGES - 1, stage_at(STAGES - 1), (kk + 1) * PART, PART);
         }
       }
       if (kk + PF < KS) {
@@ -684,7 +690,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
             issue_some(kt + STAGES, stage, 0, PART);
           }
         }
-        read_frags(nxt, (kt + 1) % STAGES, kk + PF - KS);
+        read_frags(nxt, stage_at(1), kk + PF - KS);
       }
       __builtin_amdgcn_sched_barrier(0);
       // Transposed accumulation: rows of the MFMA result = output columns.
@@ -697,12 +703,23 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_pipe_ker
       __builtin_amdgcn_sched_barrier(0);
     }
   };
+  using Dyn = std::integral_constant<int, -1>;
   int kt = 0;
+  if constexpr (!WIDE2 && (STAGES == 4 || STAGES == 2)) {
+    for (; kt + 2 * STAGES - 1 < KT; kt += STAGES) {  // kt % STAGES == 0, all STAGES tiles steady
+      tile_step(kt, std::true_type{}, std::integral_constant<int, 0>{});
+      tile_step(kt + 1, std::true_type{}, std::integral_constant<int, 1>{});
+      if constexpr (STAGES == 4) {
+        tile_step(kt + 2, std::true_type{}, std::integral_constant<int, 2>{});
+        tile_step(kt + 3, std::true_type{}, std::integral_constant<int, 3>{});
+      }
+    }
+  }
   for (; kt + STAGES < KT; kt++) {
-    tile_step(kt, std::true_type{});
+    tile_step(kt, std::true_type{}, Dyn{});
   }
   for (; kt < KT; kt++) {
-    tile_step(kt, std::false_type{});
+    tile_step(kt, std::false_type{}, Dyn{});
   }
   // acc[i][j][r]: output row m = wm0 + 32 i + lane % 32,
   //               column n = wn0 + 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4.
